@@ -1,0 +1,37 @@
+/* Function-pointer types of the hooks returned by gpuarray_get_extension()
+ * on the "hip" backend.  Counterpart of the reference's CUDA hook list
+ * (src/gpuarray/ext_cuda.h:1-46); only what a caller of the elementwise and
+ * reduction path needs is published. */
+#ifndef GPUARRAY_EXT_HIP_H
+#define GPUARRAY_EXT_HIP_H
+
+#include <gpuarray/buffer.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* "hip_get_stream": the context's single stream as a hipStream_t. */
+typedef void *(*ga_hip_get_stream_fn)(gpucontext *ctx);
+/* "hip_get_ptr": raw device address of a buffer. */
+typedef void *(*ga_hip_get_ptr_fn)(gpudata *b);
+/* "hip_get_sz": byte size of a buffer. */
+typedef size_t (*ga_hip_get_sz_fn)(gpudata *b);
+/* "hip_make_buf": wrap caller-owned device memory (not freed on release). */
+typedef gpudata *(*ga_hip_make_buf_fn)(gpucontext *ctx, void *devptr,
+                                       size_t sz);
+/* "hip_compile_only": compile kernel source for gfx950 without a device and
+ * return GA_NO_ERROR or GA_IMPL_ERROR; *log (if not NULL) gets a malloc'd
+ * compiler log.  Lets host-only checks see that generated kernels build. */
+typedef int (*ga_hip_compile_only_fn)(unsigned int count, const char **strs,
+                                      const size_t *lens, char **log);
+/* "hip_time_begin"/"hip_time_end": bracket queued work with events on the
+ * context's stream; end waits and returns elapsed milliseconds (< 0 on
+ * error). */
+typedef int (*ga_hip_time_begin_fn)(gpucontext *ctx);
+typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,80 @@
+/* GpuReduction: reductions over any subset of the axes of a strided array.
+ *
+ * The reference snapshot has no such header: its only C reduction is
+ * GpuArray_maxandargmax (src/gpuarray/array.h:607-644,
+ * src/gpuarray_reduction.c:100-124) and sum/prod/any/all exist only in its
+ * Python layer (pygpu/reduction.py:137-319, pygpu/_array.py:238-294).  This
+ * header gives those semantics, plus min, max, arg-min/max and bitwise, one C entry
+ * point.  GpuArray_maxandargmax is a wrapper around GA_REDUCE_MAXANDARGMAX.
+ */
+#ifndef GPUARRAY_REDUCTION_H
+#define GPUARRAY_REDUCTION_H
+
+#include <gpuarray/array.h>
+#include <gpuarray/buffer.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum _ga_reduce_op {
+  /*                               d0 (value)        d1 (index)          */
+  GA_REDUCE_SUM = 0,            /* sum                 -                  */
+  GA_REDUCE_PROD,               /* product             -                  */
+  GA_REDUCE_PRODNZ,             /* product of non-zero elements           */
+  GA_REDUCE_MIN,                /* minimum             -                  */
+  GA_REDUCE_MAX,                /* maximum             -                  */
+  GA_REDUCE_ARGMIN,             /* -                   index of minimum   */
+  GA_REDUCE_ARGMAX,             /* -                   index of maximum   */
+  GA_REDUCE_MINANDARGMIN,       /* minimum             index of minimum   */
+  GA_REDUCE_MAXANDARGMAX,       /* maximum             index of maximum   */
+  GA_REDUCE_AND,                /* bitwise and         -                  */
+  GA_REDUCE_OR,                 /* bitwise or          -                  */
+  GA_REDUCE_XOR,                /* bitwise xor         -                  */
+  GA_REDUCE_ALL,                /* 1 if all non-zero   -                  */
+  GA_REDUCE_ANY,                /* 1 if any non-zero   -                  */
+  GA_REDUCE_ENDSUPPORTED
+} ga_reduce_op;
+
+typedef struct _GpuReduction GpuReduction;
+
+/* Create a reduction operator.
+ *   ndf, ndr    expected numbers of free and reduced axes; hints only, any
+ *               rank is accepted by GpuReduction_call.
+ *   s0Typecode  element type of the source.
+ * Returns GA_NO_ERROR and *gr, or an error code with *gr == NULL. */
+GPUARRAY_PUBLIC int GpuReduction_new(GpuReduction **gr, gpucontext *ctx,
+                                     ga_reduce_op op, unsigned ndf,
+                                     unsigned ndr, int s0Typecode, int flags);
+GPUARRAY_PUBLIC void GpuReduction_free(GpuReduction *gr);
+
+/* Reduce s0 over the axes in reduxList.
+ *
+ *   d0  value result (NULL for ARGMIN/ARGMAX), d1 index result (NULL unless
+ *       the op has one).  Each has the shape of s0 with the reduced axes
+ *       removed, in ascending axis order, and is written through its own
+ *       strides; GA_VALUE_ERROR on a shape mismatch.
+ *   accumulation type = d0's element type: SUM/PROD of int32 into an int64
+ *       d0 accumulates in 64 bits (the rule of pygpu/_array.py:250-293);
+ *       half sources are widened to float and accumulated in float whatever
+ *       d0 is (float or half).  Integer sums wrap modulo 2^bits, so they are
+ *       exact and order-independent.  Floating sums use a fixed tree order:
+ *       the same call gives the same bits every time.
+ *   ALL/ANY test `element != 0` and write 0/1 (pygpu/_array.py:238-248).
+ *   MIN/MAX/ARG*: d0 must have s0's type, d1 a 64-bit integer type
+ *       (GA_LONG, GA_ULONG).  The index is flattened over the reduced axes
+ *       in reduxList order (see GpuArray_maxandargmax); ties resolve to the
+ *       lowest index; NaN is ignored unless it is element 0 of the scan.
+ *   empty reduction (a reduced axis of length 0): d0 gets the neutral
+ *       element (0, 1, all-ones, ...); MIN/MAX/ARG* give GA_VALUE_ERROR.
+ *   reduxLen == 0 is GA_INVALID_ERROR, as are repeated or out-of-range axes.
+ */
+GPUARRAY_PUBLIC int GpuReduction_call(const GpuReduction *gr, GpuArray *d0,
+                                      GpuArray *d1, const GpuArray *s0,
+                                      unsigned reduxLen, const int *reduxList,
+                                      int flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

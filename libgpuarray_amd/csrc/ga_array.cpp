@@ -1,0 +1,651 @@
+// GpuArray: views, slicing, reshaping and data movement.
+// Semantics follow the reference's src/gpuarray_array.c (cited per function);
+// strided and type-converting copies run through GpuElemwise("dst = src").
+#include "private.hpp"
+
+#include <map>
+#include <utility>
+#include <vector>
+
+// ---- strided / converting copy ------------------------------------------------
+// One GpuElemwise per (source type, destination type), kept for the life of
+// the context (reference ga_extcopy, src/gpuarray_array.c:42-86, which keeps
+// them in a small 2Q cache; there are at most a few hundred type pairs, so a
+// map that never evicts is simpler and never recompiles).
+typedef std::map<std::pair<int, int>, GpuElemwise *> extcopy_map;
+
+void ga_extcopy_cache_free(gpucontext *ctx) {
+  extcopy_map *m = (extcopy_map *)ctx->extcopy_cache;
+  if (m == nullptr) return;
+  ctx->extcopy_cache = nullptr;
+  for (auto &kv : *m) GpuElemwise_free(kv.second);
+  delete m;
+}
+
+static int ga_extcopy(GpuArray *dst, const GpuArray *src) {
+  gpucontext *ctx = GpuArray_context(dst);
+  if (ctx != GpuArray_context(src))
+    return ga_err_set(ctx->err, GA_INVALID_ERROR, "src and dst context differ");
+  if (ctx->extcopy_cache == nullptr) ctx->extcopy_cache = new extcopy_map();
+  extcopy_map &m = *(extcopy_map *)ctx->extcopy_cache;
+  auto key = std::make_pair(src->typecode, dst->typecode);
+  GpuElemwise *ge = nullptr;
+  auto it = m.find(key);
+  if (it != m.end()) {
+    ge = it->second;
+  } else {
+    gpuelemwise_arg gargs[2];
+    gargs[0].name = "src";
+    gargs[0].typecode = src->typecode;
+    gargs[0].flags = GE_READ;
+    gargs[1].name = "dst";
+    gargs[1].typecode = dst->typecode;
+    gargs[1].flags = GE_WRITE;
+    ge = GpuElemwise_new(ctx, "", "dst = src", 2, gargs, 0, GE_CONVERT_F16);
+    if (ge == nullptr) return ctx->err->code;
+    m[key] = ge;
+  }
+  void *args[2] = {(void *)src, (void *)dst};
+  return GpuElemwise_call(ge, args, GE_BROADCAST);
+}
+
+// ---- flags ----------------------------------------------------------------------
+// A dim of extent 1 never breaks contiguity (reference :1159-1194).
+
+extern "C" int GpuArray_is_c_contiguous(const GpuArray *a) {
+  size_t run = GpuArray_ITEMSIZE(a);
+  for (unsigned int i = a->nd; i > 0; i--) {
+    if (a->dimensions[i - 1] != 1 && a->strides[i - 1] != (ssize_t)run) return 0;
+    run *= a->dimensions[i - 1];
+  }
+  return 1;
+}
+
+extern "C" int GpuArray_is_f_contiguous(const GpuArray *a) {
+  size_t run = GpuArray_ITEMSIZE(a);
+  for (unsigned int i = 0; i < a->nd; i++) {
+    if (a->dimensions[i] != 1 && a->strides[i] != (ssize_t)run) return 0;
+    run *= a->dimensions[i];
+  }
+  return 1;
+}
+
+extern "C" int GpuArray_is_aligned(const GpuArray *a) {
+  size_t al = gpuarray_get_type(a->typecode)->align;
+  if (al == 0) al = 1;
+  if (a->offset % al != 0) return 0;
+  for (unsigned int i = 0; i < a->nd; i++)
+    if (a->strides[i] % (ssize_t)al != 0) return 0;
+  return 1;
+}
+
+static bool mul_overflows(size_t a, size_t b) {
+  return b != 0 && a > SIZE_MAX / b;
+}
+
+static void contiguous_strides(ssize_t *str, const size_t *dims, unsigned int nd,
+                               size_t elsize, ga_order ord) {
+  size_t run = elsize;
+  if (ord == GA_F_ORDER) {
+    for (unsigned int i = 0; i < nd; i++) { str[i] = (ssize_t)run; run *= dims[i]; }
+  } else {
+    for (unsigned int i = nd; i > 0; i--) { str[i - 1] = (ssize_t)run; run *= dims[i - 1]; }
+  }
+}
+
+extern "C" {
+
+void GpuArray_fix_flags(GpuArray *a) {
+  a->flags &= GA_WRITEABLE;
+  if (GpuArray_is_c_contiguous(a)) a->flags |= GA_C_CONTIGUOUS;
+  if (GpuArray_is_f_contiguous(a)) a->flags |= GA_F_CONTIGUOUS;
+  if (GpuArray_is_aligned(a)) a->flags |= GA_ALIGNED;
+}
+
+// reference :100-178
+int GpuArray_empty(GpuArray *a, gpucontext *ctx, int typecode, unsigned int nd,
+                   const size_t *dims, ga_order ord) {
+  if (typecode == GA_SIZE || typecode == GA_SSIZE)
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Cannot create array with size type");
+  size_t elsize = gpuarray_get_elsize(typecode);
+  if (elsize == 0)
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Unknown typecode %d", typecode);
+  if (ord == GA_ANY_ORDER) ord = GA_C_ORDER;
+  if (ord != GA_C_ORDER && ord != GA_F_ORDER)
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Invalid order");
+
+  size_t bytes = elsize;
+  for (unsigned int i = 0; i < nd; i++) {
+    if (mul_overflows(bytes, dims[i]))
+      return ga_err_set(ctx->err, GA_XLARGE_ERROR,
+                        "Total array size greater than addressable space");
+    bytes *= dims[i];
+  }
+  memset(a, 0, sizeof(*a));
+  int res = GA_NO_ERROR;
+  a->data = gpudata_alloc(ctx, bytes, nullptr, 0, &res);
+  if (a->data == nullptr) return ctx->err->code;
+  a->nd = nd;
+  a->offset = 0;
+  a->typecode = typecode;
+  a->dimensions = (size_t *)calloc(nd ? nd : 1, sizeof(size_t));
+  a->strides = (ssize_t *)calloc(nd ? nd : 1, sizeof(ssize_t));
+  if (a->dimensions == nullptr || a->strides == nullptr) {
+    GpuArray_clear(a);
+    return ga_err_sys(ctx->err, "calloc");
+  }
+  if (nd) memcpy(a->dimensions, dims, nd * sizeof(size_t));
+  contiguous_strides(a->strides, a->dimensions, nd, elsize, ord);
+  a->flags = GA_BEHAVED | (ord == GA_F_ORDER ? GA_F_CONTIGUOUS : GA_C_CONTIGUOUS);
+  if (nd <= 1) a->flags |= GA_C_CONTIGUOUS | GA_F_CONTIGUOUS;
+  return GA_NO_ERROR;
+}
+
+int GpuArray_zeros(GpuArray *a, gpucontext *ctx, int typecode, unsigned int nd,
+                   const size_t *dims, ga_order ord) {
+  int err = GpuArray_empty(a, ctx, typecode, nd, dims, ord);
+  if (err != GA_NO_ERROR) return err;
+  err = gpudata_memset(a->data, a->offset, 0);
+  if (err != GA_NO_ERROR) GpuArray_clear(a);
+  return err;
+}
+
+// reference :196-222
+int GpuArray_fromdata(GpuArray *a, gpudata *data, size_t offset, int typecode,
+                      unsigned int nd, const size_t *dims, const ssize_t *strides,
+                      int writeable) {
+  gpucontext *ctx = gpudata_context(data);
+  if (typecode == GA_SIZE || typecode == GA_SSIZE)
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Cannot create array with size type");
+  memset(a, 0, sizeof(*a));
+  a->data = data;
+  gpudata_retain(data);
+  a->nd = nd;
+  a->offset = offset;
+  a->typecode = typecode;
+  a->flags = writeable ? GA_WRITEABLE : 0;
+  a->dimensions = (size_t *)calloc(nd ? nd : 1, sizeof(size_t));
+  a->strides = (ssize_t *)calloc(nd ? nd : 1, sizeof(ssize_t));
+  if (a->dimensions == nullptr || a->strides == nullptr) {
+    GpuArray_clear(a);
+    return ga_err_set(ctx->err, GA_MEMORY_ERROR, "Out of memory");
+  }
+  if (nd) {
+    memcpy(a->dimensions, dims, nd * sizeof(size_t));
+    memcpy(a->strides, strides, nd * sizeof(ssize_t));
+  }
+  GpuArray_fix_flags(a);
+  return GA_NO_ERROR;
+}
+
+// reference :224-241
+int GpuArray_view(GpuArray *v, const GpuArray *a) {
+  gpucontext *ctx = GpuArray_context(a);
+  v->data = a->data;
+  gpudata_retain(a->data);
+  v->nd = a->nd;
+  v->offset = a->offset;
+  v->typecode = a->typecode;
+  v->flags = a->flags;
+  v->dimensions = (size_t *)calloc(a->nd ? a->nd : 1, sizeof(size_t));
+  v->strides = (ssize_t *)calloc(a->nd ? a->nd : 1, sizeof(ssize_t));
+  if (v->dimensions == nullptr || v->strides == nullptr) {
+    GpuArray_clear(v);
+    return ga_err_set(ctx->err, GA_MEMORY_ERROR, "Out of memory");
+  }
+  if (a->nd) {
+    memcpy(v->dimensions, a->dimensions, a->nd * sizeof(size_t));
+    memcpy(v->strides, a->strides, a->nd * sizeof(ssize_t));
+  }
+  return GA_NO_ERROR;
+}
+
+int GpuArray_sync(GpuArray *a) { return gpudata_sync(a->data); }
+
+// reference :243-313.  Per dim: start in [-1, len]; with step 0 the start
+// must be a valid index; otherwise stop in [-1, len] and the span must run in
+// the step's direction.  New extent = (stop-start+step-sign(step))/step.
+int GpuArray_index_inplace(GpuArray *a, const ssize_t *starts, const ssize_t *stops,
+                           const ssize_t *steps) {
+  gpucontext *ctx = GpuArray_context(a);
+  if (starts == nullptr || stops == nullptr || steps == nullptr)
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Invalid slice (contains NULL)");
+
+  std::vector<size_t> nd_dims;
+  std::vector<ssize_t> nd_strs;
+  size_t off = a->offset;
+  for (unsigned int i = 0; i < a->nd; i++) {
+    const ssize_t st = starts[i], sp = stops[i], step = steps[i];
+    const size_t len = a->dimensions[i];
+    bool bad = st < -1 || (st > 0 && (size_t)st > len);
+    if (!bad && step == 0) bad = st == -1 || (size_t)st >= len;
+    if (!bad && step != 0)
+      bad = sp < -1 || (sp > 0 && (size_t)sp > len) || (sp - st) / step < 0;
+    if (bad)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                        "Invalid slice value: slice(%lld, %lld, %lld) when indexing array on "
+                        "dimension %u of length %lld",
+                        (long long)st, (long long)sp, (long long)step, i, (long long)len);
+    off += (size_t)(st * a->strides[i]);
+    if (step != 0) {
+      nd_strs.push_back(step * a->strides[i]);
+      nd_dims.push_back((size_t)((sp - st + step - (step < 0 ? -1 : 1)) / step));
+    }
+  }
+  unsigned int nnd = (unsigned int)nd_dims.size();
+  size_t *newdims = (size_t *)calloc(nnd ? nnd : 1, sizeof(size_t));
+  ssize_t *newstrs = (ssize_t *)calloc(nnd ? nnd : 1, sizeof(ssize_t));
+  if (newdims == nullptr || newstrs == nullptr) {
+    free(newdims);
+    free(newstrs);
+    return ga_err_sys(ctx->err, "calloc");
+  }
+  for (unsigned int i = 0; i < nnd; i++) {
+    newdims[i] = nd_dims[i];
+    newstrs[i] = nd_strs[i];
+  }
+  free(a->dimensions);
+  free(a->strides);
+  a->dimensions = newdims;
+  a->strides = newstrs;
+  a->nd = nnd;
+  a->offset = off;
+  GpuArray_fix_flags(a);
+  return GA_NO_ERROR;
+}
+
+int GpuArray_index(GpuArray *r, const GpuArray *a, const ssize_t *starts,
+                   const ssize_t *stops, const ssize_t *steps) {
+  int err = GpuArray_view(r, a);
+  if (err != GA_NO_ERROR) return err;
+  err = GpuArray_index_inplace(r, starts, stops, steps);
+  if (err != GA_NO_ERROR) GpuArray_clear(r);
+  return err;
+}
+
+// reference :550-609
+int GpuArray_setarray(GpuArray *a, const GpuArray *v) {
+  gpucontext *ctx = GpuArray_context(a);
+  if (a->nd < v->nd)
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Dimension error. a->nd = %u, v->nd = %u", a->nd,
+                      v->nd);
+  if (!GpuArray_ISWRITEABLE(a))
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array not writable");
+  if (!GpuArray_ISALIGNED(v) || !GpuArray_ISALIGNED(a))
+    return ga_err_set(ctx->err, GA_UNALIGNED_ERROR, "One of the inputs is unaligned");
+
+  const unsigned int off = a->nd - v->nd;
+  bool same_shape = true;
+  for (unsigned int i = 0; i < v->nd; i++) {
+    if (v->dimensions[i] == a->dimensions[i + off]) continue;
+    if (v->dimensions[i] != 1)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                        "Shape error. v->dimensions[%u] = %zu, a->dimensions[%u + %u] = %zu", i,
+                        v->dimensions[i], i, off, a->dimensions[i + off]);
+    same_shape = false;
+  }
+  if (same_shape && a->nd == v->nd && a->typecode == v->typecode &&
+      GpuArray_ISONESEGMENT(a) && GpuArray_ISONESEGMENT(v) &&
+      GpuArray_ISFORTRAN(a) == GpuArray_ISFORTRAN(v)) {
+    size_t sz = gpuarray_get_elsize(a->typecode);
+    for (unsigned int i = 0; i < a->nd; i++) sz *= a->dimensions[i];
+    return gpudata_move(a->data, a->offset, v->data, v->offset, sz);
+  }
+  // View v with a's shape: broadcast dims get stride 0.
+  std::vector<ssize_t> strs(a->nd ? a->nd : 1, 0);
+  for (unsigned int i = off; i < a->nd; i++)
+    if (v->dimensions[i - off] == a->dimensions[i]) strs[i] = v->strides[i - off];
+  GpuArray tv = *v;
+  tv.nd = a->nd;
+  tv.dimensions = a->dimensions;
+  tv.strides = strs.data();
+  if (tv.nd != 0) GpuArray_fix_flags(&tv);
+  return ga_extcopy(a, &tv);
+}
+
+// No-copy reshape (reference :625-772).  The old and new shapes are cut into
+// groups of equal element count; a group of old dims can be re-split iff the
+// array walks it as one evenly strided run in the requested order.  Old dims
+// of extent 1 carry no layout information and are dropped first.
+int GpuArray_reshape_inplace(GpuArray *a, unsigned int nd, const size_t *newdims,
+                             ga_order ord) {
+  gpucontext *ctx = GpuArray_context(a);
+  if (ord == GA_ANY_ORDER) ord = (GpuArray_ISFORTRAN(a) && a->nd > 1) ? GA_F_ORDER : GA_C_ORDER;
+
+  size_t oldsize = 1, newsize = 1;
+  for (unsigned int i = 0; i < a->nd; i++) oldsize *= a->dimensions[i];
+  for (unsigned int i = 0; i < nd; i++) {
+    if (mul_overflows(newsize, newdims[i]))
+      return ga_err_set(ctx->err, GA_XLARGE_ERROR,
+                        "Output array size greater than addressable space");
+    newsize *= newdims[i];
+  }
+  if (newsize != oldsize)
+    return ga_err_set(ctx->err, GA_INVALID_ERROR, "New shape differs in total size");
+
+  const size_t elsize = gpuarray_get_elsize(a->typecode);
+  std::vector<ssize_t> ns(nd ? nd : 1, 0);
+
+  const bool already = (ord == GA_C_ORDER && GpuArray_CHKFLAGS(a, GA_C_CONTIGUOUS)) ||
+                       (ord == GA_F_ORDER && GpuArray_CHKFLAGS(a, GA_F_CONTIGUOUS));
+  if (already || newsize == 0) {
+    contiguous_strides(ns.data(), newdims, nd, elsize, ord);
+  } else {
+    // Work in "slowest first" order; F order is the mirror image.
+    std::vector<size_t> od, nw(nd);
+    std::vector<ssize_t> os;
+    for (unsigned int i = 0; i < a->nd; i++) {
+      unsigned int k = ord == GA_F_ORDER ? a->nd - 1 - i : i;
+      if (a->dimensions[k] == 1) continue;
+      od.push_back(a->dimensions[k]);
+      os.push_back(a->strides[k]);
+    }
+    for (unsigned int i = 0; i < nd; i++) nw[i] = newdims[ord == GA_F_ORDER ? nd - 1 - i : i];
+    std::vector<ssize_t> res(nd ? nd : 1, (ssize_t)elsize);
+    size_t oi = 0, ni = 0;
+    while (ni < nd && oi < od.size()) {
+      size_t np = nw[ni], op = od[oi], nj = ni + 1, oj = oi + 1;
+      while (np != op) {
+        if (np < op) np *= nw[nj++];
+        else op *= od[oj++];
+      }
+      for (size_t k = oi; k + 1 < oj; k++)
+        if (os[k] != (ssize_t)od[k + 1] * os[k + 1])
+          return ga_err_set(ctx->err, GA_COPY_ERROR,
+                            "Copy is needed but disallowed by parameters");
+      res[nj - 1] = os[oj - 1];
+      for (size_t k = nj - 1; k > ni; k--) res[k - 1] = res[k] * (ssize_t)nw[k];
+      ni = nj;
+      oi = oj;
+    }
+    // what is left on the new side are extents of 1: any stride does, use
+    // the element size
+    for (unsigned int i = 0; i < nd; i++) ns[ord == GA_F_ORDER ? nd - 1 - i : i] = res[i];
+  }
+
+  size_t *dcopy = (size_t *)calloc(nd ? nd : 1, sizeof(size_t));
+  ssize_t *scopy = (ssize_t *)calloc(nd ? nd : 1, sizeof(ssize_t));
+  if (dcopy == nullptr || scopy == nullptr) {
+    free(dcopy);
+    free(scopy);
+    return ga_err_sys(ctx->err, "calloc");
+  }
+  for (unsigned int i = 0; i < nd; i++) {
+    dcopy[i] = newdims[i];
+    scopy[i] = ns[i];
+  }
+  free(a->dimensions);
+  free(a->strides);
+  a->dimensions = dcopy;
+  a->strides = scopy;
+  a->nd = nd;
+  GpuArray_fix_flags(a);
+  return GA_NO_ERROR;
+}
+
+// reference :611-623
+int GpuArray_reshape(GpuArray *res, const GpuArray *a, unsigned int nd, const size_t *newdims,
+                     ga_order ord, int nocopy) {
+  int err = GpuArray_view(res, a);
+  if (err != GA_NO_ERROR) return err;
+  err = GpuArray_reshape_inplace(res, nd, newdims, ord);
+  if (err == GA_COPY_ERROR && !nocopy) {
+    GpuArray_clear(res);
+    err = GpuArray_copy(res, a, ord);
+    if (err != GA_NO_ERROR) return err;
+    err = GpuArray_reshape_inplace(res, nd, newdims, ord);
+  }
+  if (err != GA_NO_ERROR) GpuArray_clear(res);
+  return err;
+}
+
+// reference :785-828: NULL reverses the axes; a repeated axis is an error.
+int GpuArray_transpose_inplace(GpuArray *a, const unsigned int *new_axes) {
+  gpucontext *ctx = GpuArray_context(a);
+  const unsigned int nd = a->nd;
+  std::vector<size_t> d(nd ? nd : 1);
+  std::vector<ssize_t> s(nd ? nd : 1);
+  std::vector<char> seen(nd ? nd : 1, 0);
+  for (unsigned int i = 0; i < nd; i++) {
+    unsigned int j = new_axes == nullptr ? nd - 1 - i : new_axes[i];
+    if (j >= nd)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Axis %u out of range in transpose (nd = %u)", j,
+                        nd);
+    if (seen[j])
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Repeated axes in transpose: axis %u", j);
+    seen[j] = 1;
+    d[i] = a->dimensions[j];
+    s[i] = a->strides[j];
+  }
+  for (unsigned int i = 0; i < nd; i++) {
+    a->dimensions[i] = d[i];
+    a->strides[i] = s[i];
+  }
+  GpuArray_fix_flags(a);
+  return GA_NO_ERROR;
+}
+
+int GpuArray_transpose(GpuArray *res, const GpuArray *a, const unsigned int *new_axes) {
+  int err = GpuArray_view(res, a);
+  if (err != GA_NO_ERROR) return err;
+  err = GpuArray_transpose_inplace(res, new_axes);
+  if (err != GA_NO_ERROR) GpuArray_clear(res);
+  return err;
+}
+
+void GpuArray_clear(GpuArray *a) {
+  if (a->data) gpudata_release(a->data);
+  free(a->dimensions);
+  free(a->strides);
+  memset(a, 0, sizeof(*a));
+}
+
+int GpuArray_share(const GpuArray *a, const GpuArray *b) {
+  if (a->data != b->data) return 0;
+  return gpudata_share(a->data, b->data, nullptr);
+}
+
+gpucontext *GpuArray_context(const GpuArray *a) { return gpudata_context(a->data); }
+
+// reference :849-877
+int GpuArray_move(GpuArray *dst, const GpuArray *src) {
+  gpucontext *ctx = GpuArray_context(dst);
+  if (!GpuArray_ISWRITEABLE(dst))
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array (dst) not writeable");
+  if (!GpuArray_ISALIGNED(src))
+    return ga_err_set(ctx->err, GA_UNALIGNED_ERROR, "Source array (src) not aligned");
+  if (!GpuArray_ISALIGNED(dst))
+    return ga_err_set(ctx->err, GA_UNALIGNED_ERROR, "Destination array (dst) not aligned");
+  if (src->nd != dst->nd)
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Dimension mismatch. src->nd = %u, dst->nd = %u",
+                      src->nd, dst->nd);
+  for (unsigned int i = 0; i < src->nd; i++)
+    if (src->dimensions[i] != dst->dimensions[i])
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                        "Dimension mismatch. src->dimensions[%u] = %zu, dst->dimensions[%u] = %zu",
+                        i, src->dimensions[i], i, dst->dimensions[i]);
+  if (!GpuArray_ISONESEGMENT(dst) || !GpuArray_ISONESEGMENT(src) ||
+      GpuArray_ISFORTRAN(dst) != GpuArray_ISFORTRAN(src) || dst->typecode != src->typecode)
+    return ga_extcopy(dst, src);
+  size_t sz = gpuarray_get_elsize(dst->typecode);
+  for (unsigned int i = 0; i < dst->nd; i++) sz *= dst->dimensions[i];
+  return gpudata_move(dst->data, dst->offset, src->data, src->offset, sz);
+}
+
+// reference :879-900
+int GpuArray_write(GpuArray *dst, const void *src, size_t src_sz) {
+  gpucontext *ctx = GpuArray_context(dst);
+  if (!GpuArray_ISWRITEABLE(dst))
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array (dst) not writeable");
+  if (!GpuArray_ISONESEGMENT(dst))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Destination array (dst) not one segment");
+  return gpudata_write(dst->data, dst->offset, src, src_sz);
+}
+
+int GpuArray_read(void *dst, size_t dst_sz, const GpuArray *src) {
+  gpucontext *ctx = GpuArray_context(src);
+  if (!GpuArray_ISONESEGMENT(src))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (src) not one segment");
+  return gpudata_read(dst, src->data, src->offset, dst_sz);
+}
+
+int GpuArray_memset(GpuArray *a, int data) {
+  gpucontext *ctx = GpuArray_context(a);
+  if (!GpuArray_ISONESEGMENT(a))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (a) not one segment");
+  return gpudata_memset(a->data, a->offset, data);
+}
+
+int GpuArray_copy(GpuArray *res, const GpuArray *a, ga_order order) {
+  int err = GpuArray_empty(res, GpuArray_context(a), a->typecode, a->nd, a->dimensions, order);
+  if (err != GA_NO_ERROR) return err;
+  err = GpuArray_move(res, a);
+  if (err != GA_NO_ERROR) GpuArray_clear(res);
+  return err;
+}
+
+// reference :913-932
+int GpuArray_transfer(GpuArray *res, const GpuArray *a) {
+  gpucontext *ctx = GpuArray_context(res);
+  if (!GpuArray_ISONESEGMENT(res))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (res) not one segment");
+  if (!GpuArray_ISONESEGMENT(a))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (a) not one segment");
+  if (res->typecode != a->typecode)
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "typecode mismatch");
+  size_t sz = gpuarray_get_elsize(a->typecode);
+  for (unsigned int i = 0; i < a->nd; i++) sz *= a->dimensions[i];
+  return gpudata_transfer(res->data, res->offset, a->data, a->offset, sz);
+}
+
+// reference :934-980: n cut points give n+1 views along `axis`.
+int GpuArray_split(GpuArray **rs, const GpuArray *a, size_t n, size_t *p, unsigned int axis) {
+  gpucontext *ctx = GpuArray_context(a);
+  if (axis >= a->nd)
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Invalid axis %u for an array of %u dimensions",
+                      axis, a->nd);
+  std::vector<ssize_t> starts(a->nd, 0), stops(a->nd), steps(a->nd, 1);
+  for (unsigned int i = 0; i < a->nd; i++) stops[i] = (ssize_t)a->dimensions[i];
+  int err = GA_NO_ERROR;
+  size_t i;
+  for (i = 0; i <= n; i++) {
+    starts[axis] = i > 0 ? (ssize_t)p[i - 1] : 0;
+    stops[axis] = i < n ? (ssize_t)p[i] : (ssize_t)a->dimensions[axis];
+    err = GpuArray_index(rs[i], a, starts.data(), stops.data(), steps.data());
+    if (err != GA_NO_ERROR) break;
+  }
+  if (err != GA_NO_ERROR)
+    for (size_t k = 0; k < i; k++) GpuArray_clear(rs[k]);
+  return err;
+}
+
+// reference :982-1065: all inputs share every extent but `axis`; the result
+// is filled piece by piece through a window of the result array.
+int GpuArray_concatenate(GpuArray *r, const GpuArray **as, size_t n, unsigned int axis,
+                         int restype) {
+  gpucontext *ctx = GpuArray_context(as[0]);
+  const unsigned int nd = as[0]->nd;
+  if (axis >= nd)
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Invalid axis. axis = %u, as[0]->nd = %u", axis, nd);
+  std::vector<size_t> dims(as[0]->dimensions, as[0]->dimensions + nd);
+  for (size_t i = 0; i < n; i++) {
+    if (!GpuArray_ISALIGNED(as[i]))
+      return ga_err_fmt(ctx->err, GA_UNALIGNED_ERROR, "Unaligned array (as[%zu]).", i);
+    if (i == 0) continue;
+    if (as[i]->nd != nd)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                        "Shape mismatch. as[%zu]->nd = %u, as[0]->nd = %u", i, as[i]->nd, nd);
+    for (unsigned int d = 0; d < nd; d++) {
+      if (d == axis) {
+        dims[d] += as[i]->dimensions[d];
+      } else if (dims[d] != as[i]->dimensions[d]) {
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                          "Dimension mismatch. as[%zu]->dimensions[%u] = %zu, "
+                          "as[0]->dimensions[%u] = %zu",
+                          i, d, as[i]->dimensions[d], d, dims[d]);
+      }
+    }
+  }
+  int err = GpuArray_empty(r, ctx, restype, nd, dims.data(), GA_ANY_ORDER);
+  if (err != GA_NO_ERROR) return err;
+
+  GpuArray win = *r;   // borrowed window over r's storage
+  std::vector<size_t> wdims(nd);
+  win.dimensions = wdims.data();
+  for (size_t i = 0; i < n; i++) {
+    for (unsigned int d = 0; d < nd; d++) wdims[d] = as[i]->dimensions[d];
+    GpuArray_fix_flags(&win);
+    err = ga_extcopy(&win, as[i]);
+    if (err != GA_NO_ERROR) {
+      GpuArray_clear(r);
+      return err;
+    }
+    win.offset += (size_t)(r->strides[axis] * (ssize_t)as[i]->dimensions[axis]);
+  }
+  return GA_NO_ERROR;
+}
+
+const char *GpuArray_error(const GpuArray *a, int err) {
+  return gpucontext_error(gpudata_context(a->data), err);
+}
+
+void GpuArray_fprintf(FILE *fd, const GpuArray *a) {
+  fprintf(fd, "GpuArray <%p, data: %p (%p)> nd=%u\n", (const void *)a, (void *)a->data,
+          a->data ? a->data->devptr : nullptr, a->nd);
+  fprintf(fd, "\tITEMSIZE: %zu\n\tTYPECODE: %d\n\tOFFSET: %zu\n\tHOST_DIMS:      ",
+          GpuArray_ITEMSIZE(a), a->typecode, a->offset);
+  for (unsigned int i = 0; i < a->nd; i++) fprintf(fd, "%zu\t", a->dimensions[i]);
+  fprintf(fd, "\n\tHOST_STRIDES: ");
+  for (unsigned int i = 0; i < a->nd; i++) fprintf(fd, "%zd\t", a->strides[i]);
+  fprintf(fd, "\nFLAGS:");
+  const struct { int bit; const char *name; } names[] = {
+      {GA_C_CONTIGUOUS, "GA_C_CONTIGUOUS"}, {GA_F_CONTIGUOUS, "GA_F_CONTIGUOUS"},
+      {GA_ALIGNED, "GA_ALIGNED"},           {GA_WRITEABLE, "GA_WRITEABLE"}};
+  bool first = true;
+  for (const auto &nm : names) {
+    if (!(a->flags & nm.bit)) continue;
+    fprintf(fd, "%s %s", first ? "" : ",", nm.name);
+    first = false;
+  }
+  fputc('\n', fd);
+}
+
+// reference :1113-1157: one "[k] = value" line per element, four types only.
+int GpuArray_fdump(FILE *fd, const GpuArray *a) {
+  gpucontext *ctx = GpuArray_context(a);
+  const size_t el = GpuArray_ITEMSIZE(a);
+  size_t count = 1;
+  for (unsigned int i = 0; i < a->nd; i++) count *= a->dimensions[i];
+  if (a->typecode != GA_UINT && a->typecode != GA_LONG && a->typecode != GA_FLOAT &&
+      a->typecode != GA_SSIZE) {
+    fprintf(fd, "<unsupported data type %d>\n", a->typecode);
+    return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Unsupported data type for dump: %d",
+                      a->typecode);
+  }
+  std::vector<char> buf(count * el ? count * el : 1);
+  int err = GpuArray_read(buf.data(), count * el, a);
+  if (err != GA_NO_ERROR) return err;
+  for (size_t k = 0; k < count; k++) {
+    const char *p = buf.data() + k * el;
+    fprintf(fd, "[%zu] = ", k);
+    switch (a->typecode) {
+    case GA_UINT: { uint32_t v; memcpy(&v, p, 4); fprintf(fd, "%u", v); break; }
+    case GA_LONG: { int64_t v; memcpy(&v, p, 8); fprintf(fd, "%lld", (long long)v); break; }
+    case GA_FLOAT: { float v; memcpy(&v, p, 4); fprintf(fd, "%f", v); break; }
+    default: { ssize_t v; memcpy(&v, p, sizeof(v)); fprintf(fd, "%zd", v); break; }
+    }
+    fputc('\n', fd);
+  }
+  return GA_NO_ERROR;
+}
+
+// Gather along the first axis.  Listed after the elementwise and reduction
+// path in the build order; until it lands the call reports that plainly
+// instead of computing something else.
+int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_error) {
+  (void)v; (void)i; (void)check_error;
+  gpucontext *ctx = GpuArray_context(a);
+  return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "GpuArray_take1 is not implemented by the hip backend yet");
+}
+
+}  // extern "C"

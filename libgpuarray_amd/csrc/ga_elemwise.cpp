@@ -1,0 +1,814 @@
+// GpuElemwise: argument checking, iteration-space planning and kernel
+// generation for one C-like expression over broadcastable strided arrays.
+//
+// The contract is the reference's (src/gpuarray_elemwise.c):
+//   - GpuElemwise_new copies the descriptors and compiles the flat kernel at
+//     once, so a bad expression fails here (:604-737);
+//   - GpuElemwise_call first tries the flat path: every array has the first
+//     array's exact shape and all are C- or all F-contiguous (:547-602);
+//   - otherwise shapes are left-padded (GE_PADSHAPE), size-1 input dims are
+//     stretched (GE_BROADCAST), outputs never stretch, the first GE_WRITE
+//     array fixes the iteration space, and every mismatch is GA_VALUE_ERROR
+//     (:272-383);
+//   - n == 0 succeeds without a launch (:778,783).
+//
+// What is different is everything after the checks.  The reference unravels
+// the flat index with one `%` and one `/` per dimension per ELEMENT
+// (:198-209) and moves 4 bytes per lane.  Here:
+//   - the order of an elementwise iteration space is free, so dims are sorted
+//     by the output's stride before collapsing: an all-Fortran call, or a
+//     transposed output, becomes a plain run;
+//   - flat kernel: 256-lane groups, 16-byte loads and stores per lane, four
+//     independent tiles of loads in flight before the first use;
+//   - strided kernel: group index -> (row block, column block) with one
+//     division per GROUP; a lane owns one row and walks the inner dim, so the
+//     row is unravelled once per lane, never per element;
+//   - an operand whose unit stride lies on another dim than the output's
+//     (a transposed view) is staged through a padded 64x65 LDS tile so that
+//     both its global access and the output's are coalesced.
+#include "private.hpp"
+
+#include <algorithm>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace {
+
+struct ge_arg {
+  std::string name;
+  int typecode;
+  int flags;
+  bool is_array() const { return !(flags & GE_SCALAR); }
+  bool reads() const { return flags & GE_READ; }
+  bool writes() const { return flags & GE_WRITE; }
+};
+
+// Flat kernel geometry: 256 lanes, each moving GE_U chunks of up to 16 bytes
+// per array and tile.
+constexpr unsigned GE_LANES = 256;
+
+unsigned long env_ul(const char *name, unsigned long dflt) {
+  const char *v = getenv(name);
+  if (v == nullptr || *v == 0) return dflt;
+  char *end = nullptr;
+  unsigned long r = strtoul(v, &end, 10);
+  return end == v ? dflt : r;
+}
+
+void appendf(std::string &s, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void appendf(std::string &s, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  int n = vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  if (n < 0) return;
+  if ((size_t)n < sizeof(buf)) {
+    s.append(buf, (size_t)n);
+    return;
+  }
+  std::vector<char> big((size_t)n + 1);
+  va_start(ap, fmt);
+  vsnprintf(big.data(), big.size(), fmt, ap);
+  va_end(ap);
+  s.append(big.data(), (size_t)n);
+}
+
+const char *ctype(int typecode) { return gpuarray_get_type(typecode)->cluda_name; }
+
+const char *chunk_type(size_t bytes) {
+  switch (bytes) {
+  case 1: return "ga_ubyte";
+  case 2: return "ga_ushort";
+  case 4: return "ga_uint";
+  case 8: return "ga_chunk8";
+  default: return "ga_chunk16";
+  }
+}
+
+}  // namespace
+
+struct _GpuElemwise {
+  gpucontext *ctx = nullptr;
+  std::string expr, preamble;
+  std::vector<ge_arg> args;
+  unsigned int narray = 0;
+  int flags = 0;
+  int kflags = 0;           // GA_USE_* for the compiler
+  unsigned int vec = 1;     // elements per chunk in the flat kernel
+  unsigned int unroll = 1;  // chunks per lane and tile in the flat kernel
+  GpuKernel k_flat = {nullptr, nullptr};
+  // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
+  std::map<std::string, GpuKernel> k_strided;
+  // planning scratch
+  std::vector<size_t> dims;
+  std::vector<std::vector<ssize_t>> strs;
+  std::vector<ssize_t *> strp;
+};
+
+namespace {
+
+bool local_is_float(const GpuElemwise *ge, const ge_arg &a) {
+  return (ge->flags & GE_CONVERT_F16) && a.typecode == GA_HALF;
+}
+
+// "T name;" plus the load, given an lvalue expression for the element.
+void emit_load(const GpuElemwise *ge, std::string &s, const ge_arg &a, const std::string &src) {
+  const bool cvt = local_is_float(ge, a);
+  appendf(s, "%s %s;", cvt ? "ga_float" : ctype(a.typecode), a.name.c_str());
+  if (a.reads()) {
+    if (cvt) appendf(s, " %s = ga_half2float(%s);", a.name.c_str(), src.c_str());
+    else appendf(s, " %s = %s;", a.name.c_str(), src.c_str());
+  }
+  s += "\n";
+}
+
+void emit_store(const GpuElemwise *ge, std::string &s, const ge_arg &a, const std::string &dst) {
+  if (!a.writes()) return;
+  if (local_is_float(ge, a)) appendf(s, "%s = ga_float2half(%s);\n", dst.c_str(), a.name.c_str());
+  else appendf(s, "%s = %s;\n", dst.c_str(), a.name.c_str());
+}
+
+void emit_header(const GpuElemwise *ge, std::string &s) {
+  s += "#include \"cluda.h\"\n";
+  s += "typedef ga_uint __attribute__((ext_vector_type(2))) ga_chunk8;\n"
+       "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n";
+  s += ge->preamble;
+  s += "\n";
+}
+
+// ---- flat kernel --------------------------------------------------------------
+// elem(n, {data, byte offset | scalar}..., ga_vec)
+//   ga_vec != 0: every array base is aligned to a whole chunk of V elements
+//   (16 bytes of the widest type).  Chunk c belongs to lane c % 256 of group
+//   (c / 256) % G; a lane issues the loads of its next U chunks (G*256 chunks
+//   apart, so every load instruction of a wavefront covers one contiguous
+//   kilobyte) before the first use.  The last n % V elements, and the whole
+//   range when ga_vec == 0, run one element per lane.
+std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
+  std::string s;
+  const unsigned V = ge->vec, U = ge->unroll;
+  emit_header(ge, s);
+  s += "KERNEL void __launch_bounds__(256) elem(const ga_size n";
+  ktypes.push_back(GA_SIZE);
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_p, const ga_size %s_offset", ctype(a.typecode),
+              a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_vec) {\n";
+  ktypes.push_back(GA_UINT);
+  for (const ge_arg &a : ge->args)
+    if (a.is_array())
+      appendf(s, "%s_p = (GLOBAL_MEM %s *)((GLOBAL_MEM char *)%s_p + %s_offset);\n",
+              a.name.c_str(), ctype(a.typecode), a.name.c_str(), a.name.c_str());
+  s += "const ga_size ga_gtid = (ga_size)GID_0 * LDIM_0 + LID_0;\n"
+       "const ga_size ga_nthr = (ga_size)GDIM_0 * LDIM_0;\n"
+       "ga_size ga_done = 0;\n";
+  if (V > 1 || U > 1) {
+    appendf(s, "if (ga_vec) {\nconst ga_size ga_nchunks = n / %uu;\n", V);
+    appendf(s, "for (ga_size ga_c0 = ga_gtid; ga_c0 < ga_nchunks; ga_c0 += ga_nthr * %uu) {\n", U);
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array()) continue;
+      size_t cb = gpuarray_get_elsize(a.typecode) * V;
+      appendf(s, "union { %s c; %s e[%u]; } %s_u[%u];\n", chunk_type(cb), ctype(a.typecode), V,
+              a.name.c_str(), U);
+    }
+    appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
+    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_nthr;\nif (ga_c < ga_nchunks) {\n";
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array() || !a.reads()) continue;
+      size_t cb = gpuarray_get_elsize(a.typecode) * V;
+      appendf(s, "%s_u[ga_u].c = __builtin_nontemporal_load((const %s *)%s_p + ga_c);\n",
+              a.name.c_str(), chunk_type(cb), a.name.c_str());
+    }
+    s += "}\n}\n";
+    appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
+    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_nthr;\nif (ga_c < ga_nchunks) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
+    appendf(s, "const ga_size i = ga_c * %uu + ga_v; (void)i;\n{\n", V);
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_load(ge, s, a, a.name + "_u[ga_u].e[ga_v]");
+    s += ge->expr;
+    s += ";\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_store(ge, s, a, a.name + "_u[ga_u].e[ga_v]");
+    s += "}\n}\n";
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array() || !a.writes()) continue;
+      size_t cb = gpuarray_get_elsize(a.typecode) * V;
+      appendf(s, "__builtin_nontemporal_store(%s_u[ga_u].c, (%s *)%s_p + ga_c);\n",
+              a.name.c_str(), chunk_type(cb), a.name.c_str());
+    }
+    s += "}\n}\n";
+    appendf(s, "}\nga_done = ga_nchunks * %uu;\n}\n", V);
+  }
+  s += "for (ga_size i = ga_done + ga_gtid; i < n; i += ga_nthr) {\n";
+  for (const ge_arg &a : ge->args)
+    if (a.is_array()) emit_load(ge, s, a, a.name + "_p[i]");
+  s += ge->expr;
+  s += ";\n";
+  for (const ge_arg &a : ge->args)
+    if (a.is_array()) emit_store(ge, s, a, a.name + "_p[i]");
+  s += "}\n}\n";
+  return s;
+}
+
+// ---- strided kernel -------------------------------------------------------------
+// elem(dim0..dim{nd-1}, {data, byte offset, str_0..str_{nd-1} | scalar}...,
+//      ga_gx, ga_ltx)
+//
+// Dims arrive sorted and collapsed; x = dim nd-1 is the output's fastest dim.
+//
+// Plain variant (no transposed operand): a group is TX x TY lanes (TX =
+// 1 << ga_ltx, 256 lanes in all).  Lane (tx, ty) of group (bx, by) owns row
+// by*TY + ty of the nd-1 outer dims and the columns (bx*4 + e)*TX + tx,
+// e = 0..3.  The group id is split with one division; the row is unravelled
+// once.
+//
+// Transposed variant: y = dim nd-2 is where the transposed operands have
+// their small stride.  A group handles a 64 (y) x 64 (x) tile with 64 x 4
+// lanes; transposed reads enter through LDS (lanes along y), the expression
+// runs with lanes along x, transposed writes leave through LDS.
+std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
+                        std::vector<int> &ktypes) {
+  std::string s;
+  const char *I = idx64 ? "ga_ssize" : "ga_int";     // byte offsets
+  const char *N = idx64 ? "ga_size" : "ga_uint";     // counts
+  emit_header(ge, s);
+  s += "KERNEL void __launch_bounds__(256) elem(";
+  for (unsigned d = 0; d < nd; d++) {
+    appendf(s, "%sconst ga_size dim%u", d ? ", " : "", d);
+    ktypes.push_back(GA_SIZE);
+  }
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset", ctype(a.typecode),
+              a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+      for (unsigned d = 0; d < nd; d++) {
+        appendf(s, ", const ga_ssize %s_str_%u", a.name.c_str(), d);
+        ktypes.push_back(GA_SSIZE);
+      }
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n";
+  ktypes.push_back(GA_UINT);
+  ktypes.push_back(GA_UINT);
+
+  // array index among arrays, for the transposed mask
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto is_t = [&](size_t j) { return aidx[j] >= 0 && ((tmask >> aidx[j]) & 1u); };
+
+  for (const ge_arg &a : ge->args)
+    if (a.is_array())
+      appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n",
+              a.name.c_str(), a.name.c_str(), a.name.c_str());
+
+  if (tmask == 0) {
+    appendf(s, "const %s ga_tx = LID_0 & ((1u << ga_ltx) - 1u);\n", N);
+    appendf(s, "const %s ga_ty = LID_0 >> ga_ltx;\n", N);
+    appendf(s, "const %s ga_bx = GID_0 %% ga_gx;\n", N);
+    appendf(s, "const %s ga_by = GID_0 / ga_gx;\n", N);
+    appendf(s, "%s ga_rows = 1;\n", N);
+    for (unsigned d = 0; d + 1 < nd; d++) appendf(s, "ga_rows *= (%s)dim%u;\n", N, d);
+    appendf(s, "const %s ga_row = ga_by * (256u >> ga_ltx) + ga_ty;\n", N);
+    s += "if (ga_row >= ga_rows) return;\n";
+    // unravel the row over dims nd-2 .. 0
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
+    if (nd >= 2) {
+      appendf(s, "{ %s ga_r = ga_row; %s ga_c;\n", N, N);
+      for (unsigned d = nd - 1; d-- > 0;) {
+        if (d > 0) appendf(s, "ga_c = ga_r %% (%s)dim%u; ga_r = ga_r / (%s)dim%u;\n", N, d, N, d);
+        else s += "ga_c = ga_r;\n";
+        for (const ge_arg &a : ge->args)
+          if (a.is_array())
+            appendf(s, "%s_o += (%s)ga_c * (%s)%s_str_%u;\n", a.name.c_str(), I, I,
+                    a.name.c_str(), d);
+      }
+      s += "}\n";
+    }
+    const unsigned xd = nd - 1;
+    appendf(s, "const %s ga_x0 = (ga_bx * 4u << ga_ltx) + ga_tx;\n", N);
+    s += "#pragma unroll\nfor (int ga_e = 0; ga_e < 4; ga_e++) {\n";
+    appendf(s, "const %s ga_x = ga_x0 + ((%s)ga_e << ga_ltx);\n", N, N);
+    appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array()) continue;
+      std::string at;
+      appendf(at, "*(GLOBAL_MEM %s *)(%s_b + (%s_o + (%s)ga_x * (%s)%s_str_%u))", ctype(a.typecode),
+              a.name.c_str(), a.name.c_str(), I, I, a.name.c_str(), xd);
+      emit_load(ge, s, a, at);
+    }
+    s += ge->expr;
+    s += ";\n";
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array()) continue;
+      std::string at;
+      appendf(at, "*(GLOBAL_MEM %s *)(%s_b + (%s_o + (%s)ga_x * (%s)%s_str_%u))", ctype(a.typecode),
+              a.name.c_str(), a.name.c_str(), I, I, a.name.c_str(), xd);
+      emit_store(ge, s, a, at);
+    }
+    s += "}\n}\n}\n";
+    return s;
+  }
+
+  // transposed variant, nd >= 2
+  const unsigned xd = nd - 1, yd = nd - 2;
+  for (size_t j = 0; j < ge->args.size(); j++)
+    if (is_t(j))
+      appendf(s, "LOCAL_MEM %s %s_t[64 * 65];\n", ctype(ge->args[j].typecode),
+              ge->args[j].name.c_str());
+  appendf(s, "const %s ga_tx = LID_0 & 63u;\nconst %s ga_ty = LID_0 >> 6;\n", N, N);
+  appendf(s, "const %s ga_gy = ((%s)dim%u + 63u) / 64u;\n", N, N, yd);
+  appendf(s, "const %s ga_bx = GID_0 %% ga_gx;\n", N);
+  appendf(s, "%s ga_r = GID_0 / ga_gx;\n", N);
+  appendf(s, "const %s ga_by = ga_r %% ga_gy;\nga_r = ga_r / ga_gy;\n", N);
+  for (const ge_arg &a : ge->args)
+    if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
+  if (nd >= 3) {
+    appendf(s, "{ %s ga_c;\n", N);
+    for (unsigned d = nd - 2; d-- > 0;) {
+      if (d > 0) appendf(s, "ga_c = ga_r %% (%s)dim%u; ga_r = ga_r / (%s)dim%u;\n", N, d, N, d);
+      else s += "ga_c = ga_r;\n";
+      for (const ge_arg &a : ge->args)
+        if (a.is_array())
+          appendf(s, "%s_o += (%s)ga_c * (%s)%s_str_%u;\n", a.name.c_str(), I, I, a.name.c_str(),
+                  d);
+    }
+    s += "}\n";
+  }
+  appendf(s, "const %s ga_x0 = ga_bx * 64u;\nconst %s ga_y0 = ga_by * 64u;\n", N, N);
+  auto gaddr = [&](const ge_arg &a, const char *y, const char *x) {
+    std::string at;
+    appendf(at, "*(GLOBAL_MEM %s *)(%s_b + (%s_o + (%s)(%s) * (%s)%s_str_%u + (%s)(%s) * (%s)%s_str_%u))",
+            ctype(a.typecode), a.name.c_str(), a.name.c_str(), I, y, I, a.name.c_str(), yd, I, x,
+            I, a.name.c_str(), xd);
+    return at;
+  };
+  // phase 1: transposed reads, lanes along y
+  bool any_tr = false, any_tw = false;
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    if (!is_t(j)) continue;
+    if (ge->args[j].reads()) any_tr = true;
+    if (ge->args[j].writes()) any_tw = true;
+  }
+  if (any_tr) {
+    s += "#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = ga_tx, ga_lx = ga_ty + 4u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.reads()) continue;
+      appendf(s, "%s_t[ga_lx * 65u + ga_ly] = %s;\n", a.name.c_str(),
+              gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+    }
+    s += "}\n}\nlocal_barrier();\n";
+  }
+  // phase 2: expression, lanes along x
+  s += "#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+  appendf(s, "const %s ga_lx = ga_tx, ga_ly = ga_ty + 4u * (%s)ga_k;\n", N, N);
+  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_lx * 65u + ga_ly]");
+    else emit_load(ge, s, a, gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx"));
+  }
+  s += ge->expr;
+  s += ";\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_lx * 65u + ga_ly]");
+    else emit_store(ge, s, a, gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx"));
+  }
+  s += "}\n}\n";
+  // phase 3: transposed writes, lanes along y
+  if (any_tw) {
+    s += "local_barrier();\n#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = ga_tx, ga_lx = ga_ty + 4u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.writes()) continue;
+      appendf(s, "%s = %s_t[ga_lx * 65u + ga_ly];\n",
+              gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str(), a.name.c_str());
+    }
+    s += "}\n}\n";
+  }
+  s += "}\n";
+  return s;
+}
+
+int build_kernel(GpuElemwise *ge, GpuKernel *k, const std::string &src,
+                 const std::vector<int> &ktypes) {
+  const char *strs[1] = {src.c_str()};
+  size_t lens[1] = {src.size()};
+  return GpuKernel_init(k, ge->ctx, 1, strs, lens, "elem", (unsigned)ktypes.size(), ktypes.data(),
+                        ge->kflags, nullptr);
+}
+
+// ---- flat path ------------------------------------------------------------------
+
+// reference check_contig (:547-576): returns -1 when shapes differ.
+int check_flat(GpuElemwise *ge, void **args, size_t *n_out, bool *flat) {
+  const GpuArray *first = nullptr;
+  size_t n = 1;
+  bool c_all = true, f_all = true;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (!ge->args[i].is_array()) continue;
+    const GpuArray *v = (const GpuArray *)args[i];
+    if (first == nullptr) {
+      first = v;
+      for (unsigned j = 0; j < v->nd; j++) n *= v->dimensions[j];
+    } else {
+      if (v->nd != first->nd) return -1;
+      for (unsigned j = 0; j < v->nd; j++)
+        if (v->dimensions[j] != first->dimensions[j]) return -1;
+    }
+    c_all = c_all && GpuArray_IS_C_CONTIGUOUS(v);
+    f_all = f_all && GpuArray_IS_F_CONTIGUOUS(v);
+  }
+  *flat = c_all || f_all;
+  *n_out = n;
+  return GA_NO_ERROR;
+}
+
+// Launch the flat kernel over n elements; offs[k] is the byte offset of
+// array k's first element in its buffer.
+int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
+  GpuKernel *k = &ge->k_flat;
+  unsigned p = 0, l = 0;
+  int err;
+  unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u;
+  if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (ge->args[i].is_array()) {
+      GpuArray *a = (GpuArray *)args[i];
+      size_t off = offs[l++];
+      size_t chunk = gpuarray_get_elsize(a->typecode) * ge->vec;
+      if (((uintptr_t)a->data->devptr + off) % chunk != 0) vec_ok = 0;
+      if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
+      if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
+    } else {
+      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
+    }
+  }
+  if (n < ge->vec) vec_ok = 0;
+  if ((err = GpuKernel_setarg(k, p++, &vec_ok)) != GA_NO_ERROR) return err;
+
+  // Grid: one lane per chunk (or per element) up to a fixed number of groups
+  // per compute unit; beyond that the lanes stride over the range.
+  const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 8);
+  size_t cap = (size_t)ga_hip_numprocs(ge->ctx) * (per_cu ? per_cu : 8);
+  size_t units = vec_ok ? n / ge->vec : n;
+  size_t want = (units + GE_LANES - 1) / GE_LANES;
+  size_t gs = want < 1 ? 1 : (want > cap ? cap : want);
+  size_t ls = GE_LANES;
+  return GpuKernel_call(k, 1, &gs, &ls, 0, nullptr);
+}
+
+// ---- general path ---------------------------------------------------------------
+
+// Reference check_basic (:272-383) up to, not including, the collapse:
+// fills ge->dims / ge->strs with the padded, broadcast-adjusted view of
+// every array and returns nd and n.
+int check_general(GpuElemwise *ge, void **args, int flags, size_t *n_out, unsigned *nd_out) {
+  gpucontext *ctx = ge->ctx;
+  const GpuArray *out = nullptr;
+  unsigned nd = 0, seen = 0;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (!ge->args[i].is_array()) continue;
+    const GpuArray *v = (const GpuArray *)args[i];
+    if (seen == 0) {
+      nd = v->nd;
+    } else if (v->nd != nd) {
+      if (!(flags & GE_PADSHAPE))
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Arg %zu has differing nd = %u", i, v->nd);
+      nd = std::max(nd, v->nd);
+    }
+    seen++;
+    if (out == nullptr && ge->args[i].writes()) out = v;
+  }
+  if (out == nullptr) return ga_err_set(ctx->err, GA_VALUE_ERROR, "No output arrays");
+  if (out->nd != nd)
+    // the output fixes the iteration space, so it cannot be the padded one
+    return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                      "Output has nd = %u but an input has nd = %u: outputs do not broadcast",
+                      out->nd, nd);
+
+  ge->dims.assign(out->dimensions, out->dimensions + nd);
+  ge->strs.assign(ge->narray, std::vector<ssize_t>(nd ? nd : 1, 0));
+  unsigned p = 0;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (!ge->args[i].is_array()) continue;
+    const GpuArray *v = (const GpuArray *)args[i];
+    const unsigned pad = nd - v->nd;
+    for (unsigned j = 0; j < nd; j++) {
+      const size_t vd = j < pad ? 1 : v->dimensions[j - pad];
+      if (vd != ge->dims[j]) {
+        if (!(flags & GE_BROADCAST) || ge->args[i].writes() || vd != 1)
+          return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                            "Mismatched dimension %u for input %zu (expected %zu got %zu)", j, i,
+                            ge->dims[j], vd);
+      }
+      // a dim of extent 1 never moves: stride 0 whether or not it broadcasts
+      ge->strs[p][j] = (j < pad || vd == 1) ? 0 : v->strides[j - pad];
+    }
+    p++;
+  }
+  size_t n = 1;
+  for (unsigned j = 0; j < nd; j++) n *= ge->dims[j];
+  *n_out = n;
+  *nd_out = nd;
+  return GA_NO_ERROR;
+}
+
+inline size_t sabs(ssize_t v) { return v < 0 ? (size_t)(-v) : (size_t)v; }
+
+int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
+  gpucontext *ctx = ge->ctx;
+  const unsigned na = ge->narray;
+  std::vector<size_t> &dims = ge->dims;
+  std::vector<std::vector<ssize_t>> &strs = ge->strs;
+
+  // which array is the (first) output, and per-array element sizes / offsets
+  std::vector<size_t> elsz(na), offs(na);
+  int outk = -1;
+  {
+    unsigned k = 0;
+    for (size_t i = 0; i < ge->args.size(); i++) {
+      if (!ge->args[i].is_array()) continue;
+      const GpuArray *v = (const GpuArray *)args[i];
+      elsz[k] = gpuarray_get_elsize(v->typecode);
+      offs[k] = v->offset;
+      if (outk < 0 && ge->args[i].writes()) outk = (int)k;
+      k++;
+    }
+  }
+
+  if (nd == 0) {  // 0-d arrays: one element
+    nd = 1;
+    dims.assign(1, 1);
+    for (auto &s : strs) s.assign(1, 0);
+  }
+
+  // Sort dims so the output's stride shrinks towards the last dim (stable),
+  // then drop size-1 dims and fuse runs.
+  {
+    std::vector<unsigned> order(nd);
+    for (unsigned j = 0; j < nd; j++) order[j] = j;
+    std::stable_sort(order.begin(), order.end(), [&](unsigned a, unsigned b) {
+      return sabs(strs[outk][a]) > sabs(strs[outk][b]);
+    });
+    std::vector<size_t> d2(nd);
+    for (unsigned j = 0; j < nd; j++) d2[j] = dims[order[j]];
+    dims = d2;
+    for (unsigned k = 0; k < na; k++) {
+      std::vector<ssize_t> s2(nd);
+      for (unsigned j = 0; j < nd; j++) s2[j] = strs[k][order[j]];
+      strs[k] = s2;
+    }
+  }
+  ge->strp.resize(na);
+  for (unsigned k = 0; k < na; k++) ge->strp[k] = strs[k].data();
+  gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
+
+  // One evenly strided run with every array stepping by its own element
+  // size is the flat case again (all-Fortran inputs, sliced-then-dense...).
+  if (nd == 1) {
+    bool unit = true;
+    for (unsigned k = 0; k < na && unit; k++)
+      unit = dims[0] == 1 || strs[k][0] == (ssize_t)elsz[k];
+    if (unit) return call_flat(ge, args, n, offs.data());
+  }
+
+  // Transposed operands: small stride on some outer dim, large on x.
+  unsigned tmask = 0;
+  if (nd >= 2 && dims[nd - 1] >= 16) {
+    // candidate y axis: the outer dim on which most arrays have their
+    // smallest non-zero stride
+    std::vector<unsigned> votes(nd, 0);
+    std::vector<int> best(na, -1);
+    for (unsigned k = 0; k < na; k++) {
+      size_t sx = sabs(strs[k][nd - 1]);
+      if (sx == 0) continue;
+      int b = -1;
+      size_t bs = sx;
+      for (unsigned j = 0; j + 1 < nd; j++) {
+        size_t sj = sabs(strs[k][j]);
+        if (sj != 0 && sj < bs && sj <= 4 * elsz[k] && dims[j] >= 16) { bs = sj; b = (int)j; }
+      }
+      best[k] = b;
+      if (b >= 0) votes[b]++;
+    }
+    int y = -1;
+    for (unsigned j = 0; j + 1 < nd; j++)
+      if (votes[j] > 0 && (y < 0 || votes[j] > votes[y])) y = (int)j;
+    if (y >= 0) {
+      size_t lds = 0;
+      for (unsigned k = 0; k < na; k++)
+        if (best[k] == y) { tmask |= 1u << k; lds += 64 * 65 * elsz[k]; }
+      if (lds > 64 * 1024 || na > 31) tmask = 0;
+      if (tmask && (unsigned)y != nd - 2) {
+        // rotate y into position nd-2
+        size_t dy = dims[y];
+        dims.erase(dims.begin() + y);
+        dims.insert(dims.begin() + (nd - 2), dy);
+        for (unsigned k = 0; k < na; k++) {
+          ssize_t sy = strs[k][y];
+          strs[k].erase(strs[k].begin() + y);
+          strs[k].insert(strs[k].begin() + (nd - 2), sy);
+        }
+      }
+    }
+  }
+
+  // 32-bit offsets when every reachable byte offset fits
+  bool idx64 = n >= (size_t)GA_SADDR32_MAX;
+  for (unsigned k = 0; k < na && !idx64; k++) {
+    size_t reach = elsz[k];
+    for (unsigned j = 0; j < nd; j++) reach += (dims[j] - 1) * sabs(strs[k][j]);
+    if (reach >= (size_t)GA_SADDR32_MAX) idx64 = true;
+  }
+
+  // launch geometry
+  size_t gx, groups;
+  unsigned ltx = 0;
+  if (tmask == 0) {
+    size_t inner = dims[nd - 1];
+    ltx = 4;
+    while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
+    size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
+    size_t rows = n / inner;
+    gx = (inner + 4 * tx - 1) / (4 * tx);
+    groups = gx * ((rows + ty - 1) / ty);
+  } else {
+    gx = (dims[nd - 1] + 63) / 64;
+    size_t gy = (dims[nd - 2] + 63) / 64;
+    size_t outer = n / dims[nd - 1] / dims[nd - 2];
+    groups = gx * gy * outer;
+  }
+  if (!idx64 && (groups >= (size_t)GA_SADDR32_MAX || gx >= (size_t)GA_SADDR32_MAX)) idx64 = true;
+  if (groups > 0x7fffffffull || gx > 0xffffffffull)
+    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
+
+  char key[64];
+  snprintf(key, sizeof(key), "%u:%d:%x", nd, idx64 ? 1 : 0, tmask);
+  GpuKernel *k;
+  auto it = ge->k_strided.find(key);
+  if (it != ge->k_strided.end()) {
+    k = &it->second;
+  } else {
+    std::vector<int> ktypes;
+    std::string src = gen_strided(ge, nd, idx64, tmask, ktypes);
+    GpuKernel nk = {nullptr, nullptr};
+    int err = build_kernel(ge, &nk, src, ktypes);
+    if (err != GA_NO_ERROR) return err;
+    k = &ge->k_strided.emplace(key, nk).first->second;
+  }
+
+  unsigned p = 0, l = 0;
+  int err;
+  for (unsigned j = 0; j < nd; j++)
+    if ((err = GpuKernel_setarg(k, p++, &dims[j])) != GA_NO_ERROR) return err;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (ge->args[i].is_array()) {
+      GpuArray *v = (GpuArray *)args[i];
+      if ((err = GpuKernel_setarg(k, p++, v->data)) != GA_NO_ERROR) return err;
+      if ((err = GpuKernel_setarg(k, p++, &v->offset)) != GA_NO_ERROR) return err;
+      for (unsigned j = 0; j < nd; j++)
+        if ((err = GpuKernel_setarg(k, p++, &strs[l][j])) != GA_NO_ERROR) return err;
+      l++;
+    } else {
+      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
+    }
+  }
+  unsigned int gx32 = (unsigned int)gx;
+  if ((err = GpuKernel_setarg(k, p++, &gx32)) != GA_NO_ERROR) return err;
+  if ((err = GpuKernel_setarg(k, p++, &ltx)) != GA_NO_ERROR) return err;
+  size_t ls = 256;
+  return GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
+}
+
+}  // namespace
+
+// Fill the descriptor part of an operator (no context, no kernels).
+static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, unsigned int n,
+                       gpuelemwise_arg *args, int flags, ga_errrec *err) {
+  ge->expr = expr;
+  ge->preamble = preamble ? preamble : "";
+  ge->flags = flags;
+  size_t maxel = 1;
+  for (unsigned int i = 0; i < n; i++) {
+    ge_arg a;
+    a.name = args[i].name ? args[i].name : "";
+    a.typecode = args[i].typecode;
+    a.flags = args[i].flags;
+    if (a.name.empty() || gpuarray_get_type(a.typecode)->cluda_name == nullptr)
+      return ga_err_fmt(err, GA_VALUE_ERROR, "Argument %u has no name or an unknown type (%d)", i,
+                        a.typecode);
+    if (a.is_array()) {
+      ge->narray++;
+      maxel = std::max(maxel, gpuarray_get_elsize(a.typecode));
+    }
+    ge->args.push_back(a);
+  }
+  ge->kflags = gpuarray_type_flagsa(n, args);
+  // chunk = 16 bytes of the widest element type; fewer chunks in flight when
+  // many arrays are live at once
+  ge->vec = maxel >= 16 ? 1 : (unsigned)(16 / maxel);
+  ge->unroll = ge->narray <= 4 ? 4 : (ge->narray <= 8 ? 2 : 1);
+  ge->unroll = (unsigned)env_ul("GPUARRAY_ELEMWISE_UNROLL", ge->unroll);
+  if (ge->unroll < 1) ge->unroll = 1;
+  return GA_NO_ERROR;
+}
+
+extern "C" {
+
+// Kernel text for one variant, for checks that have no device: strided == 0
+// gives the flat kernel, otherwise the strided kernel for (nd, idx64, tmask).
+// The caller frees the result.
+GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *expr,
+                                             unsigned int n, gpuelemwise_arg *args, int flags,
+                                             int strided, unsigned int nd, int idx64,
+                                             unsigned int tmask) {
+  GpuElemwise ge;
+  if (expr == nullptr || ge_describe(&ge, preamble, expr, n, args, flags, ga_global_err) != GA_NO_ERROR)
+    return nullptr;
+  std::vector<int> ktypes;
+  std::string src = strided ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes) : gen_flat(&ge, ktypes);
+  return strdup(src.c_str());
+}
+
+GpuElemwise *GpuElemwise_new(gpucontext *ctx, const char *preamble, const char *expr,
+                             unsigned int n, gpuelemwise_arg *args, unsigned int nd, int flags) {
+  (void)nd;  // strided kernels are specialised on the call's layout and built on first use
+  if (expr == nullptr || (n > 0 && args == nullptr)) {
+    ga_err_set(ctx->err, GA_VALUE_ERROR, "GpuElemwise_new: NULL expression or arguments");
+    return nullptr;
+  }
+  GpuElemwise *ge = new (std::nothrow) GpuElemwise();
+  if (ge == nullptr) {
+    ga_err_set(ctx->err, GA_MEMORY_ERROR, "Out of memory");
+    return nullptr;
+  }
+  ge->ctx = ctx;
+  if (ge_describe(ge, preamble, expr, n, args, flags, ctx->err) != GA_NO_ERROR) {
+    delete ge;
+    return nullptr;
+  }
+
+  std::vector<int> ktypes;
+  std::string src = gen_flat(ge, ktypes);
+  if (build_kernel(ge, &ge->k_flat, src, ktypes) != GA_NO_ERROR) {
+    GpuElemwise_free(ge);
+    return nullptr;
+  }
+  return ge;
+}
+
+void GpuElemwise_free(GpuElemwise *ge) {
+  if (ge == nullptr) return;
+  if (ge->k_flat.k != nullptr || ge->k_flat.args != nullptr) GpuKernel_clear(&ge->k_flat);
+  for (auto &kv : ge->k_strided) GpuKernel_clear(&kv.second);
+  delete ge;
+}
+
+int GpuElemwise_call(GpuElemwise *ge, void **args, int flags) {
+  size_t n = 0;
+  bool flat = false;
+  if (check_flat(ge, args, &n, &flat) == GA_NO_ERROR && flat) {
+    if (n == 0) return GA_NO_ERROR;
+    std::vector<size_t> offs;
+    for (size_t i = 0; i < ge->args.size(); i++)
+      if (ge->args[i].is_array()) offs.push_back(((GpuArray *)args[i])->offset);
+    if (offs.empty()) return ga_err_set(ge->ctx->err, GA_VALUE_ERROR, "No output arrays");
+    return call_flat(ge, args, n, offs.data());
+  }
+  unsigned nd = 0;
+  int err = check_general(ge, args, flags, &n, &nd);
+  if (err != GA_NO_ERROR) return err;
+  if (n == 0) return GA_NO_ERROR;
+  return call_general(ge, args, n, nd);
+}
+
+}  // extern "C"

@@ -1,0 +1,487 @@
+/* Reduction kernels for gfx950, written for 64-lane wavefronts.
+ *
+ * This text is compiled at run time behind a short list of #defines that the
+ * host planner emits (element types, operation, lane geometry):
+ *
+ *   RD_SRC_T    source element type        RD_SRC_HALF  source is ga_half
+ *   RD_ACC_T    accumulator type           RD_KIND      operation, RD_K_* below
+ *   RD_DST_T    value result type          RD_DST_HALF  value result is ga_half
+ *   RD_IDX_T    index result type          RD_ARG       carry (value, index)
+ *   RD_HAS_D0 / RD_HAS_D1                  which results are written
+ *   RD_NEUTRAL  neutral element of the operation, of type RD_ACC_T
+ *   RD_FLT      source is a floating type (NaN rules apply)
+ *   RD_G        lanes that share one output in redux_row: 64 or 256
+ *   RD_VEC      elements per load in redux_row (inner reduced stride is the
+ *               element size and everything is aligned when > 1)
+ *   RD_U        loads in flight per lane
+ *
+ * Semantics (reference src/gpuarray_reduction.c:545-607 for max/argmax,
+ * pygpu/reduction.py:33-134 for sum/prod/any/all):
+ *   - the accumulator has the result's type; each element is converted to it
+ *     before the operation;
+ *   - arg-reductions return the flattened index over the reduced axes in the
+ *     caller's axis order; ties keep the lowest index.  The reference scans
+ *     sequentially with a strict compare, which is the same thing; here the
+ *     (value, index) pair is combined with "better value, or equal value and
+ *     lower index", so the result does not depend on the shape of the tree;
+ *   - NaN never wins a strict compare, so the reference ignores a NaN unless
+ *     it is the first element scanned, in which case it stays.  Elements
+ *     other than the first are therefore mapped to -inf (max) / +inf (min),
+ *     and the result is overwritten when element 0 is NaN;
+ *   - sums use a fixed order (per lane sequential over its units, pairwise
+ *     inside a unit, then the cross-lane network below), so results are
+ *     reproducible run to run.
+ *
+ * Three kernels:
+ *   redux_row    lanes run along the fastest REDUCED dim; RD_G lanes
+ *                cooperate on one output; a row can be cut in `nsplit` pieces
+ *                that each leave a partial.
+ *   redux_col    lanes run along the fastest FREE dim (coalesced), each lane
+ *                owns one output and walks the reduced range; 4 lane rows
+ *                share the range and meet in LDS.
+ *   redux_final  second pass: combines the partials of one output.
+ */
+#include "cluda.h"
+
+#define RD_K_SUM 0
+#define RD_K_PROD 1
+#define RD_K_PRODNZ 2
+#define RD_K_MIN 3
+#define RD_K_MAX 4
+#define RD_K_AND 5
+#define RD_K_OR 6
+#define RD_K_XOR 7
+#define RD_K_ALL 8
+#define RD_K_ANY 9
+
+#define RD_MAXD 8
+
+/* Iteration space, by value.  Dims are sorted slowest first and collapsed.
+ * Strides are in bytes.  `rmul` is what one step along a reduced dim adds to
+ * the flattened index. */
+struct rd_plan {
+  ga_long fdim[RD_MAXD], fsstr[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
+  ga_long rdim[RD_MAXD], rsstr[RD_MAXD], rmul[RD_MAXD];
+  ga_long nrows;   /* number of outputs */
+  ga_long rtotal;  /* elements reduced per output */
+  ga_long nseg;    /* redux_row: segments per pass over the inner reduced dim */
+  ga_long units;   /* redux_row: (outer reduced count) * nseg */
+  ga_long upb;     /* work per split: units (row) or elements (col) */
+  ga_long gx;      /* redux_col: groups along the inner free dim */
+  ga_int nf, nr, nsplit, pad;
+};
+
+struct rd_acc {
+  RD_ACC_T v;
+#if RD_ARG
+  ga_long i;
+#endif
+};
+
+#define RD_IDX_NONE 0x7fffffffffffffffLL
+
+static __device__ inline rd_acc rd_neutral() {
+  rd_acc a;
+  a.v = RD_NEUTRAL;
+#if RD_ARG
+  a.i = RD_IDX_NONE;
+#endif
+  return a;
+}
+
+static __device__ inline rd_acc rd_combine(rd_acc a, rd_acc b) {
+#if RD_KIND == RD_K_SUM
+  a.v = a.v + b.v;
+#elif RD_KIND == RD_K_PROD || RD_KIND == RD_K_PRODNZ
+  a.v = a.v * b.v;
+#elif RD_KIND == RD_K_AND
+  a.v = a.v & b.v;
+#elif RD_KIND == RD_K_OR
+  a.v = a.v | b.v;
+#elif RD_KIND == RD_K_XOR
+  a.v = a.v ^ b.v;
+#elif RD_KIND == RD_K_ALL
+  a.v = (a.v && b.v) ? 1 : 0;
+#elif RD_KIND == RD_K_ANY
+  a.v = (a.v || b.v) ? 1 : 0;
+#elif RD_KIND == RD_K_MAX
+#if RD_ARG
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) a = b;
+#else
+  if (b.v > a.v) a = b;
+#endif
+#elif RD_KIND == RD_K_MIN
+#if RD_ARG
+  if (b.v < a.v || (b.v == a.v && b.i < a.i)) a = b;
+#else
+  if (b.v < a.v) a = b;
+#endif
+#endif
+  return a;
+}
+
+/* A half source is loaded as its 16 raw bits (RD_SRC_T is ga_ushort then) and
+ * widened to float here; every other type is used as it is. */
+#if RD_SRC_HALF
+static __device__ inline float rd_src_val(const RD_SRC_T raw) {
+  ga_half h;
+  h.data = raw;
+  return ga_half2float(h);
+}
+#else
+static __device__ inline RD_SRC_T rd_src_val(const RD_SRC_T raw) { return raw; }
+#endif
+
+/* One source element, converted for the operation. */
+static __device__ inline rd_acc rd_elem(const RD_SRC_T x_in, ga_long idx) {
+  rd_acc a;
+  const auto x = rd_src_val(x_in);
+#if RD_KIND == RD_K_ALL || RD_KIND == RD_K_ANY
+  a.v = (x != 0) ? 1 : 0;
+#elif RD_KIND == RD_K_PRODNZ
+  a.v = (x == 0) ? (RD_ACC_T)1 : (RD_ACC_T)x;
+#elif RD_KIND == RD_K_MAX && RD_FLT
+  a.v = (x != x) ? (RD_ACC_T)(-INFINITY) : (RD_ACC_T)x;
+#elif RD_KIND == RD_K_MIN && RD_FLT
+  a.v = (x != x) ? (RD_ACC_T)(INFINITY) : (RD_ACC_T)x;
+#else
+  a.v = (RD_ACC_T)x;
+#endif
+#if RD_ARG
+  a.i = idx;
+#else
+  (void)idx;
+#endif
+  return a;
+}
+
+/* ---- cross-lane network --------------------------------------------------
+ * Data-parallel-primitive moves on 32-bit words; an accumulator is moved
+ * word by word.  Steps: swap with the neighbour (quad_perm 1,0,3,2), with the
+ * other pair (quad_perm 2,3,0,1), mirror within 8, mirror within 16 - after
+ * which all 16 lanes of a row agree - then row 0 -> row 1 and row 2 -> row 3
+ * (row_bcast:15), rows 0-1 -> rows 2-3 (row_bcast:31).  Lane 63 ends up with
+ * the combination of all 64 lanes and is broadcast by a lane read. */
+#define RD_DPP_XOR1 0xB1
+#define RD_DPP_XOR2 0x4E
+#define RD_DPP_HALF_MIRROR 0x141
+#define RD_DPP_MIRROR 0x140
+#define RD_DPP_BCAST15 0x142
+#define RD_DPP_BCAST31 0x143
+
+#define RD_ACC_WORDS ((sizeof(rd_acc) + 3) / 4)
+
+template <int CTRL, int ROWMASK>
+static __device__ inline rd_acc rd_dpp(rd_acc x, rd_acc fallback) {
+  union { rd_acc a; ga_int w[RD_ACC_WORDS]; } in, old, out;
+  in.a = x;
+  old.a = fallback;
+#pragma unroll
+  for (unsigned k = 0; k < RD_ACC_WORDS; k++)
+    out.w[k] = __builtin_amdgcn_update_dpp(old.w[k], in.w[k], CTRL, ROWMASK, 0xf, false);
+  return out.a;
+}
+
+static __device__ inline rd_acc rd_readlane63(rd_acc x) {
+  union { rd_acc a; ga_int w[RD_ACC_WORDS]; } in, out;
+  in.a = x;
+#pragma unroll
+  for (unsigned k = 0; k < RD_ACC_WORDS; k++) out.w[k] = __builtin_amdgcn_readlane(in.w[k], 63);
+  return out.a;
+}
+
+/* Every lane returns the combination of the 64 lanes. */
+static __device__ inline rd_acc rd_wave_reduce(rd_acc a) {
+  const rd_acc nt = rd_neutral();
+  a = rd_combine(a, rd_dpp<RD_DPP_XOR1, 0xf>(a, nt));
+  a = rd_combine(a, rd_dpp<RD_DPP_XOR2, 0xf>(a, nt));
+  a = rd_combine(a, rd_dpp<RD_DPP_HALF_MIRROR, 0xf>(a, nt));
+  a = rd_combine(a, rd_dpp<RD_DPP_MIRROR, 0xf>(a, nt));
+  a = rd_combine(a, rd_dpp<RD_DPP_BCAST15, 0xa>(a, nt));
+  a = rd_combine(a, rd_dpp<RD_DPP_BCAST31, 0xc>(a, nt));
+  return rd_readlane63(a);
+}
+
+/* Combination over the 4 wavefronts of a 256-lane group, through LDS. */
+static __device__ inline rd_acc rd_block_reduce(rd_acc a, rd_acc *lds) {
+  a = rd_wave_reduce(a);
+  const unsigned wave = LID_0 >> 6, lane = LID_0 & 63u;
+  if (lane == 0) lds[wave] = a;
+  local_barrier();
+  rd_acc r = lds[0];
+  r = rd_combine(r, lds[1]);
+  r = rd_combine(r, lds[2]);
+  r = rd_combine(r, lds[3]);
+  return r;
+}
+
+/* ---- addressing ------------------------------------------------------------ */
+
+/* Offsets of output `row` (flat index over the free dims, slowest first). */
+static __device__ inline void rd_row_offsets(const rd_plan &p, ga_long row, ga_long *so,
+                                             ga_long *d0o, ga_long *d1o) {
+  ga_long s = 0, a = 0, b = 0;
+  for (int d = p.nf - 1; d >= 0; d--) {
+    ga_long c;
+    if (d > 0) { c = row % p.fdim[d]; row = row / p.fdim[d]; } else { c = row; }
+    s += c * p.fsstr[d];
+    a += c * p.fd0str[d];
+    b += c * p.fd1str[d];
+  }
+  *so = s; *d0o = a; *d1o = b;
+}
+
+/* Byte offset and index base of outer reduced coordinate `ro` (flat over the
+ * reduced dims 0..ri-1). */
+static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long ro, ga_long *rb,
+                                               ga_long *ib) {
+  ga_long b = 0, x = 0;
+  for (int d = ri - 1; d >= 0; d--) {
+    ga_long c;
+    if (d > 0) { c = ro % p.rdim[d]; ro = ro / p.rdim[d]; } else { c = ro; }
+    b += c * p.rsstr[d];
+    x += c * p.rmul[d];
+  }
+  *rb = b; *ib = x;
+}
+
+/* Write the finished value(s) of one output. */
+static __device__ inline void rd_store(rd_acc a, const char *srow, char *d0, ga_long d0o, char *d1,
+                                       ga_long d1o, ga_long rtotal) {
+#if RD_FLT && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN)
+  /* a NaN in the first position of the scan stays (see the header) */
+  if (rtotal > 0) {
+    const auto first = rd_src_val(*(const RD_SRC_T *)srow);
+    if (first != first) {
+      a.v = (RD_ACC_T)first;
+#if RD_ARG
+      a.i = 0;
+#endif
+    }
+  }
+#else
+  (void)srow; (void)rtotal;
+#endif
+#if RD_HAS_D0
+#if RD_DST_HALF
+  *(ga_half *)(d0 + d0o) = ga_float2half((float)a.v);
+#else
+  *(RD_DST_T *)(d0 + d0o) = (RD_DST_T)a.v;
+#endif
+#else
+  (void)d0; (void)d0o;
+#endif
+#if RD_HAS_D1
+  *(RD_IDX_T *)(d1 + d1o) = (RD_IDX_T)a.i;
+#else
+  (void)d1; (void)d1o;
+#endif
+}
+
+static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *pi, ga_long slot) {
+  pv[slot] = a.v;
+#if RD_ARG
+  pi[slot] = a.i;
+#else
+  (void)pi;
+#endif
+}
+
+/* ---- redux_row ------------------------------------------------------------- */
+
+#if RD_VEC > 1
+typedef RD_SRC_T rd_vec_t __attribute__((ext_vector_type(RD_VEC)));
+#endif
+
+KERNEL void __launch_bounds__(256)
+redux_row(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
+          const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+  const unsigned rows_per_group = 256u / RD_G;
+  const unsigned lane = LID_0 % RD_G;
+  const ga_long split = GID_0 % (unsigned)p.nsplit;
+  const ga_long row = (ga_long)(GID_0 / (unsigned)p.nsplit) * rows_per_group + LID_0 / RD_G;
+#if RD_G == 256
+  __shared__ rd_acc lds[4];
+#endif
+  if (row >= p.nrows) return;   /* uniform per wavefront; per group when RD_G == 256 */
+
+  ga_long so, d0o, d1o;
+  rd_row_offsets(p, row, &so, &d0o, &d1o);
+  const char *srow = src + src_off + so;
+
+  const int ri = p.nr - 1;                 /* inner reduced dim */
+  const ga_long rin = p.nr > 0 ? p.rdim[ri] : 1;
+  const ga_long rstr = p.nr > 0 ? p.rsstr[ri] : 0;
+  const ga_long rml = p.nr > 0 ? p.rmul[ri] : 0;
+  const ga_long seg = (ga_long)RD_G * RD_VEC * RD_U;
+
+  ga_long u0 = split * p.upb, u1 = u0 + p.upb;
+  if (u1 > p.units) u1 = p.units;
+
+  /* unit -> (outer reduced coordinate ro, segment k of the inner dim): one
+   * division for the first unit, then counted up */
+  ga_long ro = 0, k = u0;
+  if (p.nr > 1) { ro = u0 / p.nseg; k = u0 - ro * p.nseg; }
+  ga_long rb = 0, ib = 0;
+  rd_outer_offsets(p, ri, ro, &rb, &ib);
+
+  rd_acc acc = rd_neutral();
+  for (ga_long u = u0; u < u1; u++) {
+    const ga_long e0 = k * seg + (ga_long)lane * RD_VEC;
+#if RD_VEC > 1
+    rd_vec_t x[RD_U];
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
+      if (e < rin) x[j] = *(const rd_vec_t *)(srow + rb + e * rstr);
+    }
+    rd_acc t[RD_U];
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
+      t[j] = rd_neutral();
+      if (e < rin) {
+#pragma unroll
+        for (int v = 0; v < RD_VEC; v++)
+          t[j] = rd_combine(t[j], rd_elem(x[j][v], ib + (e + v) * rml));
+      }
+    }
+#else
+    RD_SRC_T x[RD_U];
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      const ga_long e = e0 + (ga_long)j * RD_G;
+      if (e < rin) x[j] = *(const RD_SRC_T *)(srow + rb + e * rstr);
+    }
+    rd_acc t[RD_U];
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      const ga_long e = e0 + (ga_long)j * RD_G;
+      t[j] = (e < rin) ? rd_elem(x[j], ib + e * rml) : rd_neutral();
+    }
+#endif
+    /* pairwise over the unit, then onto the running value */
+#pragma unroll
+    for (int w = 1; w < RD_U; w *= 2)
+#pragma unroll
+      for (int j = 0; j + w < RD_U; j += 2 * w) t[j] = rd_combine(t[j], t[j + w]);
+    acc = rd_combine(acc, t[0]);
+    if (++k == p.nseg) {
+      k = 0;
+      ro++;
+      rd_outer_offsets(p, ri, ro, &rb, &ib);
+    }
+  }
+
+#if RD_G == 256
+  acc = rd_block_reduce(acc, lds);
+#else
+  acc = rd_wave_reduce(acc);
+#endif
+  if (lane == 0) {
+    if (p.nsplit == 1) rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+    else rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
+  }
+}
+
+/* ---- redux_col ------------------------------------------------------------- */
+
+KERNEL void __launch_bounds__(256)
+redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
+          const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+  __shared__ rd_acc lds[4][64];
+  const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
+  const ga_long split = GID_0 % (unsigned)p.nsplit;
+  ga_long t = GID_0 / (unsigned)p.nsplit;
+  const ga_long bx = t % p.gx;
+  const ga_long fo = t / p.gx;   /* flat index over the outer free dims */
+  const int fi_d = p.nf - 1;
+  const ga_long fin = p.fdim[fi_d];
+  const ga_long fi = bx * 64 + tx;
+  const bool live = fi < fin;
+
+  /* offsets of this lane's output */
+  ga_long so = 0, d0o = 0, d1o = 0;
+  {
+    ga_long r = fo;
+    for (int d = fi_d - 1; d >= 0; d--) {
+      ga_long c;
+      if (d > 0) { c = r % p.fdim[d]; r = r / p.fdim[d]; } else { c = r; }
+      so += c * p.fsstr[d];
+      d0o += c * p.fd0str[d];
+      d1o += c * p.fd1str[d];
+    }
+    so += fi * p.fsstr[fi_d];
+    d0o += fi * p.fd0str[fi_d];
+    d1o += fi * p.fd1str[fi_d];
+  }
+  const char *srow = src + src_off + so;
+
+  ga_long r0 = split * p.upb, r1 = r0 + p.upb;
+  if (r1 > p.rtotal) r1 = p.rtotal;
+
+  rd_acc acc = rd_neutral();
+  if (live) {
+    for (ga_long j0 = r0 + ty; j0 < r1; j0 += 4 * RD_U) {
+      RD_SRC_T x[RD_U];
+      ga_long idx[RD_U];
+#pragma unroll
+      for (int q = 0; q < RD_U; q++) {
+        const ga_long j = j0 + 4 * q;
+        if (j < r1) {
+          ga_long off = 0, ix = 0, r = j;
+          for (int d = p.nr - 1; d >= 0; d--) {
+            ga_long c;
+            if (d > 0) { c = r % p.rdim[d]; r = r / p.rdim[d]; } else { c = r; }
+            off += c * p.rsstr[d];
+            ix += c * p.rmul[d];
+          }
+          x[q] = *(const RD_SRC_T *)(srow + off);
+          idx[q] = ix;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + 4 * q < r1) acc = rd_combine(acc, rd_elem(x[q], idx[q]));
+    }
+  }
+  lds[ty][tx] = acc;
+  local_barrier();
+  if (ty == 0 && live) {
+    acc = rd_combine(acc, lds[1][tx]);
+    acc = rd_combine(acc, lds[2][tx]);
+    acc = rd_combine(acc, lds[3][tx]);
+    const ga_long row = fo * fin + fi;
+    if (p.nsplit == 1) {
+      /* element 0 of the scan is at the start of the lane's reduced range */
+      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+    } else {
+      rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
+    }
+  }
+}
+
+/* ---- redux_final ------------------------------------------------------------
+ * One wavefront per output: combine its nsplit partials and write the result. */
+KERNEL void __launch_bounds__(256)
+redux_final(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
+            const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+  const unsigned lane = LID_0 & 63u;
+  const ga_long row = (ga_long)GID_0 * 4 + (LID_0 >> 6);
+  if (row >= p.nrows) return;
+  rd_acc acc = rd_neutral();
+  for (ga_long s = lane; s < p.nsplit; s += 64) {
+    rd_acc t;
+    t.v = part_v[row * p.nsplit + s];
+#if RD_ARG
+    t.i = part_i[row * p.nsplit + s];
+#endif
+    acc = rd_combine(acc, t);
+  }
+  acc = rd_wave_reduce(acc);
+  if (lane == 0) {
+    ga_long so, d0o, d1o;
+    rd_row_offsets(p, row, &so, &d0o, &d1o);
+    rd_store(acc, src + src_off + so, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+  }
+}

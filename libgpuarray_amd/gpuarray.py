@@ -1,0 +1,404 @@
+"""Contexts and arrays over the C ABI, with the names and behaviour of the
+reference's Python layer for this path (pygpu/gpuarray.pyx: GpuContext :1027,
+GpuArray :1482, `array`/`empty`/`zeros` :700-930) and its numpy-like array
+class (pygpu/_array.py: ndgpuarray).
+
+All device work happens inside libgpuarray.so; this file only marshals
+shapes, strides and pointers.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import lib, check, GpuArrayException, GpuArrayStruct, c_ssize_t
+
+# numpy dtype.num equals the typecode on LP64 Linux
+# (reference pygpu/gpuarray.pyx:101-116).
+_TYPECODES = {
+    np.dtype("bool"): _lib.GA_BOOL, np.dtype("int8"): _lib.GA_BYTE,
+    np.dtype("uint8"): _lib.GA_UBYTE, np.dtype("int16"): _lib.GA_SHORT,
+    np.dtype("uint16"): _lib.GA_USHORT, np.dtype("int32"): _lib.GA_INT,
+    np.dtype("uint32"): _lib.GA_UINT, np.dtype("int64"): _lib.GA_LONG,
+    np.dtype("uint64"): _lib.GA_ULONG, np.dtype("float32"): _lib.GA_FLOAT,
+    np.dtype("float64"): _lib.GA_DOUBLE, np.dtype("float16"): _lib.GA_HALF,
+    np.dtype("complex64"): _lib.GA_CFLOAT, np.dtype("complex128"): _lib.GA_CDOUBLE,
+}
+_DTYPES = {v: k for k, v in _TYPECODES.items()}
+
+
+def dtype_to_typecode(dtype):
+    try:
+        return _TYPECODES[np.dtype(dtype)]
+    except KeyError:
+        raise ValueError("don't know how to convert to dtype: %s" % (dtype,))
+
+
+def typecode_to_dtype(typecode):
+    try:
+        return _DTYPES[typecode]
+    except KeyError:
+        raise NotImplementedError("TODO: support for typecode %d" % typecode)
+
+
+def count_devices(kind="hip", platform=0):
+    n = C.c_uint(0)
+    check(lib.gpu_get_device_count(kind.encode(), platform, C.byref(n)))
+    return n.value
+
+
+class GpuContext(object):
+    """One device, one stream (reference pygpu/gpuarray.pyx:1027-1168)."""
+
+    def __init__(self, kind="hip", devno=0, single_stream=True):
+        props = C.c_void_p()
+        check(lib.gpucontext_props_new(C.byref(props)))
+        lib.gpucontext_props_hip_dev(props, devno)
+        if single_stream:
+            lib.gpucontext_props_set_single_stream(props)
+        self.ctx = C.c_void_p()
+        self.kind = kind
+        # init consumes props
+        check(lib.gpucontext_init(C.byref(self.ctx), kind.encode(), props))
+
+    def __del__(self):
+        ctx = getattr(self, "ctx", None)
+        if ctx:
+            lib.gpucontext_deref(ctx)
+            self.ctx = None
+
+    def _prop(self, prop_id, ctype):
+        v = ctype()
+        check(lib.gpucontext_property(self.ctx, prop_id, C.byref(v)), self.ctx)
+        return v.value
+
+    @property
+    def devname(self):
+        buf = C.create_string_buffer(256)
+        check(lib.gpucontext_property(self.ctx, _lib.GA_CTX_PROP_DEVNAME, buf), self.ctx)
+        return buf.value.decode()
+
+    @property
+    def bin_id(self):
+        return self._prop(_lib.GA_CTX_PROP_BIN_ID, C.c_char_p).decode()
+
+    numprocs = property(lambda s: s._prop(_lib.GA_CTX_PROP_NUMPROCS, C.c_uint))
+    lmemsize = property(lambda s: s._prop(_lib.GA_CTX_PROP_LMEMSIZE, C.c_size_t))
+    maxlsize0 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXLSIZE0, C.c_size_t))
+    maxgsize0 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXGSIZE0, C.c_size_t))
+    total_gmem = property(lambda s: s._prop(_lib.GA_CTX_PROP_TOTAL_GMEM, C.c_size_t))
+    free_gmem = property(lambda s: s._prop(_lib.GA_CTX_PROP_FREE_GMEM, C.c_size_t))
+
+    def error(self):
+        return lib.gpucontext_error(self.ctx, 0).decode(errors="replace")
+
+    # timing on the context's own stream (HIP events), in milliseconds
+    def time_begin(self):
+        fn = _lib.extension("hip_time_begin", C.c_int, [C.c_void_p])
+        check(fn(self.ctx), self.ctx)
+
+    def time_end(self):
+        fn = _lib.extension("hip_time_end", C.c_float, [C.c_void_p])
+        ms = fn(self.ctx)
+        if ms < 0:
+            raise GpuArrayException("event timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
+        return ms
+
+    def sync(self):
+        # any buffer of the context syncs the one stream; use the error buffer
+        eb = C.c_void_p()
+        check(lib.gpucontext_property(self.ctx, _lib.GA_CTX_PROP_ERRBUF, C.byref(eb)), self.ctx)
+        check(lib.gpudata_sync(eb), self.ctx)
+
+
+_default_context = None
+
+
+def set_default_context(ctx):
+    global _default_context
+    _default_context = ctx
+
+
+def get_default_context():
+    return _default_context
+
+
+def init(dev="hip0"):
+    """`init("hipN")`: reference pygpu.gpuarray.init("cudaN"/"openclP:D")."""
+    if not dev.startswith("hip"):
+        raise ValueError("only \"hipN\" devices exist on this backend, got %r" % (dev,))
+    devno = int(dev[3:] or 0)
+    return GpuContext("hip", devno)
+
+
+def _ensure_context(context):
+    ctx = context if context is not None else _default_context
+    if ctx is None:
+        raise TypeError("No context specified.")
+    return ctx
+
+
+class flags(object):
+    """numpy-style flag view (reference pygpu/gpuarray.pyx:1390-1480)."""
+
+    def __init__(self, fl):
+        self.fl = fl
+
+    c_contiguous = property(lambda s: bool(s.fl & _lib.GA_C_CONTIGUOUS))
+    f_contiguous = property(lambda s: bool(s.fl & _lib.GA_F_CONTIGUOUS))
+    aligned = property(lambda s: bool(s.fl & _lib.GA_ALIGNED))
+    writeable = property(lambda s: bool(s.fl & _lib.GA_WRITEABLE))
+    contiguous = c_contiguous
+    fortran = property(lambda s: s.f_contiguous and not s.c_contiguous)
+    forc = property(lambda s: s.c_contiguous or s.f_contiguous)
+
+    def __getitem__(self, name):
+        return getattr(self, name.lower())
+
+    def __repr__(self):
+        return "  C_CONTIGUOUS : %s\n  F_CONTIGUOUS : %s\n  WRITEABLE : %s\n  ALIGNED : %s" % (
+            self.c_contiguous, self.f_contiguous, self.writeable, self.aligned)
+
+
+class GpuArray(object):
+    """A strided view over a device buffer (reference pygpu/gpuarray.pyx:1482-2160
+    and pygpu/_array.py)."""
+
+    def __init__(self, context):
+        self.context = context
+        self.ga = GpuArrayStruct()
+        self.base = None
+
+    def __del__(self):
+        ga = getattr(self, "ga", None)
+        if ga is not None and ga.data:
+            lib.GpuArray_clear(C.byref(ga))
+
+    # -- metadata ---------------------------------------------------------------
+    shape = property(lambda s: tuple(s.ga.dimensions[i] for i in range(s.ga.nd)))
+    strides = property(lambda s: tuple(s.ga.strides[i] for i in range(s.ga.nd)))
+    ndim = property(lambda s: s.ga.nd)
+    offset = property(lambda s: s.ga.offset)
+    typecode = property(lambda s: s.ga.typecode)
+    dtype = property(lambda s: typecode_to_dtype(s.ga.typecode))
+    itemsize = property(lambda s: s.dtype.itemsize)
+    flags = property(lambda s: flags(s.ga.flags))
+
+    @property
+    def size(self):
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+    def __len__(self):
+        if self.ga.nd == 0:
+            raise TypeError("len() of unsized object")
+        return self.ga.dimensions[0]
+
+    def _ptr(self):
+        return C.byref(self.ga)
+
+    def _check(self, err):
+        check(err, self.context.ctx)
+
+    def _new(self):
+        return type(self)(self.context)
+
+    # -- data movement ------------------------------------------------------------
+    def sync(self):
+        self._check(lib.GpuArray_sync(self._ptr()))
+
+    def write(self, src):
+        """Copy a numpy array of the same shape and dtype in (one-segment arrays)."""
+        src = np.asarray(src)
+        if src.dtype != self.dtype or src.shape != self.shape:
+            raise ValueError("shape or dtype mismatch")
+        if self.flags.c_contiguous:
+            src = np.ascontiguousarray(src)
+        elif self.flags.f_contiguous:
+            src = np.asfortranarray(src)
+        self._check(lib.GpuArray_write(self._ptr(), src.ctypes.data_as(C.c_void_p), src.nbytes))
+
+    def __array__(self, dtype=None, copy=None):
+        a = self
+        if not (self.flags.c_contiguous or self.flags.f_contiguous):
+            a = self.copy("C")
+        order = "C" if a.flags.c_contiguous else "F"
+        out = np.empty(a.shape, dtype=a.dtype, order=order)
+        if out.nbytes:
+            a._check(lib.GpuArray_read(out.ctypes.data_as(C.c_void_p), out.nbytes, a._ptr()))
+        if dtype is not None and np.dtype(dtype) != out.dtype:
+            out = out.astype(dtype)
+        return out
+
+    def copy(self, order="C"):
+        res = self._new()
+        o = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER}[order.upper()]
+        if o == _lib.GA_ANY_ORDER:
+            o = _lib.GA_F_ORDER if (self.flags.f_contiguous and not self.flags.c_contiguous) \
+                else _lib.GA_C_ORDER
+        self._check(lib.GpuArray_copy(res._ptr(), self._ptr(), o))
+        return res
+
+    def astype(self, dtype, order="A"):
+        res = empty(self.shape, dtype=dtype, order="C" if order in "AC" else "F",
+                    context=self.context, cls=type(self))
+        self._check(lib.GpuArray_move(res._ptr(), self._ptr()))
+        return res
+
+    def view(self):
+        res = self._new()
+        self._check(lib.GpuArray_view(res._ptr(), self._ptr()))
+        res.base = self
+        return res
+
+    def memset(self, byte):
+        self._check(lib.GpuArray_memset(self._ptr(), byte))
+
+    # -- shape manipulation ---------------------------------------------------------
+    def transpose(self, *axes):
+        if len(axes) == 1 and isinstance(axes[0], (tuple, list)):
+            axes = tuple(axes[0])
+        res = self._new()
+        if len(axes) == 0 or axes == (None,):
+            arg = None
+        else:
+            if len(axes) != self.ndim:
+                raise ValueError("axes don't match array")
+            arg = (C.c_uint * len(axes))(*[a % self.ndim if self.ndim else a for a in axes])
+        self._check(lib.GpuArray_transpose(res._ptr(), self._ptr(), arg))
+        res.base = self
+        return res
+
+    T = property(lambda s: s.transpose())
+
+    def reshape(self, shape, order="C"):
+        if isinstance(shape, int):
+            shape = (shape,)
+        shape = list(shape)
+        if shape.count(-1) == 1:
+            known = 1
+            for d in shape:
+                if d != -1:
+                    known *= d
+            shape[shape.index(-1)] = self.size // known if known else 0
+        dims = (C.c_size_t * max(len(shape), 1))(*shape)
+        o = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER}[order.upper()]
+        res = self._new()
+        self._check(lib.GpuArray_reshape(res._ptr(), self._ptr(), len(shape), dims, o, 0))
+        return res
+
+    def __getitem__(self, key):
+        """Basic indexing only: ints, slices, Ellipsis (reference
+        pygpu/gpuarray.pyx:1928-2069 lowers these to start/stop/step triples)."""
+        if not isinstance(key, tuple):
+            key = (key,)
+        nd = self.ndim
+        if key.count(Ellipsis) > 1:
+            raise IndexError("an index can only have a single ellipsis")
+        n_explicit = len([k for k in key if k is not Ellipsis])
+        if n_explicit > nd:
+            raise IndexError("too many indices for array")
+        full = []
+        for k in key:
+            if k is Ellipsis:
+                full.extend([slice(None)] * (nd - n_explicit))
+            else:
+                full.append(k)
+        full.extend([slice(None)] * (nd - len(full)))
+        starts = (c_ssize_t * max(nd, 1))()
+        stops = (c_ssize_t * max(nd, 1))()
+        steps = (c_ssize_t * max(nd, 1))()
+        for i, k in enumerate(full):
+            dim = self.shape[i]
+            if isinstance(k, slice):
+                st, sp, stp = k.indices(dim)
+                if stp < 0 and sp < 0:
+                    sp = -1
+                if (stp > 0 and sp < st) or (stp < 0 and sp > st):
+                    sp = st
+                starts[i], stops[i], steps[i] = st, sp, stp
+            else:
+                k = int(k)
+                if k < 0:
+                    k += dim
+                if k < 0 or k >= dim:
+                    raise IndexError("index %d out of bounds" % k)
+                starts[i], stops[i], steps[i] = k, k + 1, 0
+        res = self._new()
+        self._check(lib.GpuArray_index(res._ptr(), self._ptr(), starts, stops, steps))
+        res.base = self
+        return res
+
+    def __setitem__(self, key, value):
+        """a[key] = value through GpuArray_setarray (reference gpuarray.pyx:2071-2096)."""
+        target = self if key is Ellipsis or key == slice(None) else self.__getitem__(key)
+        if not isinstance(value, GpuArray):
+            value = array(np.asarray(value, dtype=self.dtype), context=self.context)
+        target._check(lib.GpuArray_setarray(target._ptr(), value._ptr()))
+
+    def __repr__(self):
+        return "gpuarray." + repr(np.asarray(self))
+
+
+def _make(cls, context):
+    return (cls or GpuArray)(context)
+
+
+def empty(shape, dtype="float32", order="C", context=None, cls=None):
+    ctx = _ensure_context(context)
+    if isinstance(shape, (int, np.integer)):
+        shape = (int(shape),)
+    shape = tuple(int(d) for d in shape)
+    res = _make(cls, ctx)
+    dims = (C.c_size_t * max(len(shape), 1))(*shape)
+    o = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER}[order.upper()]
+    check(lib.GpuArray_empty(res._ptr(), ctx.ctx, dtype_to_typecode(dtype), len(shape), dims, o),
+          ctx.ctx)
+    return res
+
+
+def zeros(shape, dtype="float32", order="C", context=None, cls=None):
+    res = empty(shape, dtype, order, context, cls)
+    res.memset(0)
+    return res
+
+
+def array(obj, dtype=None, order="A", context=None, cls=None):
+    """Device copy of anything numpy can turn into an array."""
+    if isinstance(obj, GpuArray):
+        return obj.copy("C" if order == "A" else order)
+    a = np.array(obj, dtype=dtype, copy=True)
+    if order.upper() == "F" or (order.upper() == "A" and a.flags.f_contiguous
+                                and not a.flags.c_contiguous):
+        a = np.asfortranarray(a)
+        o = "F"
+    else:
+        a = np.ascontiguousarray(a)
+        o = "C"
+    res = empty(a.shape, a.dtype, o, context, cls)
+    if a.nbytes:
+        check(lib.GpuArray_write(res._ptr(), a.ctypes.data_as(C.c_void_p), a.nbytes),
+              res.context.ctx)
+    return res
+
+
+def asarray(obj, dtype=None, order="A", context=None, cls=None):
+    if isinstance(obj, GpuArray) and (dtype is None or np.dtype(dtype) == obj.dtype):
+        return obj
+    return array(obj, dtype, order, context, cls)
+
+
+def from_strided(base, offset, shape, strides, dtype=None, writeable=True):
+    """View `base`'s buffer with explicit byte offset and strides
+    (GpuArray_fromdata; reference gpuarray.pyx `from_gpudata` :760-815)."""
+    res = type(base)(base.context)
+    nd = len(shape)
+    dims = (C.c_size_t * max(nd, 1))(*shape)
+    strs = (c_ssize_t * max(nd, 1))(*strides)
+    tc = base.typecode if dtype is None else dtype_to_typecode(dtype)
+    check(lib.GpuArray_fromdata(res._ptr(), base.ga.data, offset, tc, nd, dims, strs,
+                                1 if writeable else 0), base.context.ctx)
+    res.base = base
+    return res
