@@ -31,6 +31,23 @@ typedef int (*ga_hip_compile_only_fn)(unsigned int count, const char **strs,
 typedef int (*ga_hip_time_begin_fn)(gpucontext *ctx);
 typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
 
+/* "hip_event_record": put timing mark number `slot` on the context's stream
+ * (marks are created on first use and reused); does not wait.
+ * "hip_event_elapsed": milliseconds from mark a to mark b; waits for b;
+ * < 0 on error. */
+typedef int (*ga_hip_event_record_fn)(gpucontext *ctx, unsigned int slot);
+typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsigned int b);
+/* "hip_elemwise_source" / "hip_reduction_source": the kernel text the
+ * generators would compile for a given variant, as a malloc'd string the
+ * caller frees.  For host-side checks of the generated code. */
+typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
+                                           unsigned int n, void *args, int flags,
+                                           int strided, unsigned int nd, int idx64,
+                                           unsigned int tmask);
+typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
+                                            int d1_typecode, unsigned int lanes_per_output,
+                                            unsigned int vec, unsigned int unroll);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,70 @@
+"""Compile every device-side text for gfx950, without a device.
+
+The library compiles kernels at run time with hipRTC; this script asks the
+freshly built library for representative kernel texts (flat and strided
+elementwise variants, every reduction operation) and runs each through the
+same hipRTC invocation the library uses.  It is the "does the device code
+build" check of the build step.
+"""
+import ctypes as C
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB = os.path.join(os.path.dirname(HERE), "libgpuarray.so")
+
+
+class ElemwiseArg(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("typecode", C.c_int), ("flags", C.c_int)]
+
+
+def main():
+    lib = C.CDLL(LIB)
+    lib.gpuarray_get_extension.restype = C.c_void_p
+    lib.gpuarray_get_extension.argtypes = [C.c_char_p]
+
+    def ext(name, res, args):
+        return C.CFUNCTYPE(res, *args)(lib.gpuarray_get_extension(name))
+
+    gen_e = ext(b"hip_elemwise_source", C.c_void_p,
+                [C.c_char_p, C.c_char_p, C.c_uint, C.POINTER(ElemwiseArg), C.c_int, C.c_int,
+                 C.c_uint, C.c_int, C.c_uint])
+    gen_r = ext(b"hip_reduction_source", C.c_void_p,
+                [C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_uint])
+    comp = ext(b"hip_compile_only", C.c_int,
+               [C.c_uint, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t), C.POINTER(C.c_char_p)])
+
+    def check(label, ptr):
+        if not ptr:
+            raise SystemExit("%s: generator failed" % label)
+        arr = (C.c_char_p * 1)(C.string_at(ptr))
+        log = C.c_char_p()
+        if comp(1, arr, None, C.byref(log)) != 0:
+            raise SystemExit("%s: does not compile for gfx950:\n%s" % (label, (log.value or b"").decode()))
+
+    GA_FLOAT, GA_HALF, GA_INT, GA_LONG, GA_UBYTE, GA_BOOL, GA_DOUBLE = 11, 23, 5, 7, 2, 0, 12
+    args = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_FLOAT, 2),
+                             ElemwiseArg(b"c", GA_FLOAT, 4))
+    check("elemwise flat", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 0, 0, 0, 0))
+    for nd, idx64, tmask in [(1, 0, 0), (2, 0, 0), (3, 1, 0), (2, 0, 1), (3, 1, 3)]:
+        check("elemwise strided nd=%d idx64=%d tmask=%x" % (nd, idx64, tmask),
+              gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 1, nd, idx64, tmask))
+    hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
+    check("elemwise half->double copy", gen_e(b"", b"dst = src", 2, hargs, 2, 0, 0, 0, 0))
+    n = 0
+    for op in range(14):
+        for src, d0 in [(GA_FLOAT, GA_FLOAT), (GA_INT, GA_LONG if op < 3 else GA_INT),
+                        (GA_HALF, GA_FLOAT if op < 3 else GA_HALF)]:
+            if op in (9, 10, 11) and src != GA_INT:
+                continue          # bitwise ops: integers only
+            if op in (12, 13):
+                d0 = GA_BOOL
+            check("reduction op=%d src=%d" % (op, src), gen_r(op, src, d0, GA_LONG, 256, 4, 4))
+            n += 1
+    check("reduction wave-per-row", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4))
+    check("reduction bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1))
+    print("device sources compile for gfx950 (%d reduction variants, 7 elementwise)" % (n + 2))
+
+
+if __name__ == "__main__":
+    sys.exit(main())

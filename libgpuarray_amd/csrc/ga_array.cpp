@@ -41,7 +41,12 @@ static int ga_extcopy(GpuArray *dst, const GpuArray *src) {
     gargs[1].name = "dst";
     gargs[1].typecode = dst->typecode;
     gargs[1].flags = GE_WRITE;
-    ge = GpuElemwise_new(ctx, "", "dst = src", 2, gargs, 0, GE_CONVERT_F16);
+    // Into a boolean the value is its truth, not its low byte: the reference
+    // assigns straight through ("dst = src" into an unsigned char,
+    // src/gpuarray_array.c:64), which stores 62 for 62.5 and 0 for 256.
+    const char *expr = dst->typecode == GA_BOOL && src->typecode != GA_BOOL ? "dst = (src != 0)"
+                                                                            : "dst = src";
+    ge = GpuElemwise_new(ctx, "", expr, 2, gargs, 0, GE_CONVERT_F16);
     if (ge == nullptr) return ctx->err->code;
     m[key] = ge;
   }
@@ -136,8 +141,11 @@ int GpuArray_empty(GpuArray *a, gpucontext *ctx, int typecode, unsigned int nd,
   }
   if (nd) memcpy(a->dimensions, dims, nd * sizeof(size_t));
   contiguous_strides(a->strides, a->dimensions, nd, elsize, ord);
-  a->flags = GA_BEHAVED | (ord == GA_F_ORDER ? GA_F_CONTIGUOUS : GA_C_CONTIGUOUS);
-  if (nd <= 1) a->flags |= GA_C_CONTIGUOUS | GA_F_CONTIGUOUS;
+  // The reference sets the flag of the requested order only, plus both for
+  // nd <= 1 (:160-175).  Computing them also marks shapes like (1, n) or
+  // (n, 1) as contiguous both ways, which they are, as NumPy does.
+  a->flags = GA_WRITEABLE;
+  GpuArray_fix_flags(a);
   return GA_NO_ERROR;
 }
 

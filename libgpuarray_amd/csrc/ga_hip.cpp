@@ -40,6 +40,7 @@ struct hip_context : _gpucontext {
   gpudata *scratch = nullptr;
   size_t scratch_sz = 0;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
   void *redux_cache = nullptr;
   ga_errrec errstore;
 };
@@ -122,6 +123,7 @@ void ctx_destroy(hip_context *ctx) {
     delete kv.second;
   }
   ctx->modcache.clear();
+  for (hipEvent_t e : ctx->evpool) (void)hipEventDestroy(e);
   if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
   if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -765,6 +767,32 @@ extern "C" char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int d1_t
                                          unsigned int V, unsigned int U);
 namespace {
 
+// Numbered timing marks on the context's stream: record as many as wanted
+// without waiting, read the spans afterwards.
+int ext_event_record(gpucontext *c, unsigned int slot) {
+  hip_context *ctx = HC(c);
+  int err;
+  if ((err = enter(ctx)) != GA_NO_ERROR) return err;
+  while (ctx->evpool.size() <= slot) {
+    hipEvent_t e = nullptr;
+    HIP_TRY(ctx, hipEventCreate(&e));
+    ctx->evpool.push_back(e);
+  }
+  HIP_TRY(ctx, hipEventRecord(ctx->evpool[slot], ctx->stream));
+  return GA_NO_ERROR;
+}
+
+// Milliseconds between marks a and b; waits for b.  < 0 on error.
+float ext_event_elapsed(gpucontext *c, unsigned int a, unsigned int b) {
+  hip_context *ctx = HC(c);
+  float ms = -1.0f;
+  if (a >= ctx->evpool.size() || b >= ctx->evpool.size()) return -1.0f;
+  if (enter(ctx) != GA_NO_ERROR) return -1.0f;
+  if (hipEventSynchronize(ctx->evpool[b]) != hipSuccess) return -1.0f;
+  if (hipEventElapsedTime(&ms, ctx->evpool[a], ctx->evpool[b]) != hipSuccess) return -1.0f;
+  return ms;
+}
+
 struct ext_entry { const char *name; void *fn; };
 const ext_entry k_exts[] = {
     {"hip_get_stream", (void *)ext_get_stream},
@@ -774,6 +802,8 @@ const ext_entry k_exts[] = {
     {"hip_compile_only", (void *)ext_compile_only},
     {"hip_time_begin", (void *)ext_time_begin},
     {"hip_time_end", (void *)ext_time_end},
+    {"hip_event_record", (void *)ext_event_record},
+    {"hip_event_elapsed", (void *)ext_event_elapsed},
     {"hip_elemwise_source", (void *)ga_elemwise_gen_source},
     {"hip_reduction_source", (void *)ga_reduction_gen_source},
 };

@@ -104,6 +104,19 @@ class GpuContext(object):
             raise GpuArrayException("event timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
         return ms
 
+    def mark(self, slot):
+        """Timing mark `slot` on the stream (no wait)."""
+        fn = _lib.extension("hip_event_record", C.c_int, [C.c_void_p, C.c_uint])
+        check(fn(self.ctx, slot), self.ctx)
+
+    def elapsed(self, a, b):
+        """Milliseconds between marks a and b (waits for b)."""
+        fn = _lib.extension("hip_event_elapsed", C.c_float, [C.c_void_p, C.c_uint, C.c_uint])
+        ms = fn(self.ctx, a, b)
+        if ms < 0:
+            raise GpuArrayException("event timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
+        return ms
+
     def sync(self):
         # any buffer of the context syncs the one stream; use the error buffer
         eb = C.c_void_p()
@@ -370,12 +383,13 @@ def array(obj, dtype=None, order="A", context=None, cls=None):
     if isinstance(obj, GpuArray):
         return obj.copy("C" if order == "A" else order)
     a = np.array(obj, dtype=dtype, copy=True)
+    # (np.ascontiguousarray would turn a 0-d array into a 1-d one)
     if order.upper() == "F" or (order.upper() == "A" and a.flags.f_contiguous
                                 and not a.flags.c_contiguous):
-        a = np.asfortranarray(a)
+        a = np.array(a, order="F", copy=None)
         o = "F"
     else:
-        a = np.ascontiguousarray(a)
+        a = np.array(a, order="C", copy=None)
         o = "C"
     res = empty(a.shape, a.dtype, o, context, cls)
     if a.nbytes:

@@ -1,0 +1,140 @@
+"""Generated kernel text compiles for gfx950 (hipRTC needs no device), and the
+device prelude offers the vocabulary kernels written for the reference use.
+No kernel is launched here."""
+import ctypes as C
+
+import pytest
+
+from libgpuarray_amd import _lib
+
+gen_elemwise = _lib.extension("hip_elemwise_source", C.c_void_p,
+                              [C.c_char_p, C.c_char_p, C.c_uint, C.POINTER(_lib.ElemwiseArg),
+                               C.c_int, C.c_int, C.c_uint, C.c_int, C.c_uint])
+gen_reduction = _lib.extension("hip_reduction_source", C.c_void_p,
+                               [C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_uint])
+compile_only = _lib.extension("hip_compile_only", C.c_int,
+                              [C.c_uint, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t),
+                               C.POINTER(C.c_char_p)])
+libc = C.CDLL(None)
+libc.free.argtypes = [C.c_void_p]
+
+
+def take_string(p):
+    assert p, "generator returned NULL"
+    s = C.string_at(p)
+    libc.free(p)
+    return s
+
+
+def compile_src(src):
+    arr = (C.c_char_p * 1)(src)
+    log = C.c_char_p()
+    err = compile_only(1, arr, None, C.byref(log))
+    return err, (log.value or b"").decode(errors="replace")
+
+
+def args_of(spec):
+    arr = (_lib.ElemwiseArg * len(spec))()
+    keep = []
+    for i, (name, tc, fl) in enumerate(spec):
+        keep.append(name.encode())
+        arr[i].name, arr[i].typecode, arr[i].flags = keep[-1], tc, fl
+    arr._keep = keep
+    return arr
+
+
+R, W, S = _lib.GE_READ, _lib.GE_WRITE, _lib.GE_SCALAR | _lib.GE_READ
+F32 = [("a", _lib.GA_FLOAT, R), ("b", _lib.GA_FLOAT, R), ("c", _lib.GA_FLOAT, W)]
+
+
+def test_flat_kernel_text_shape():
+    src = take_string(gen_elemwise(b"", b"c = a*b + 0.5f", 3, args_of(F32), 0, 0, 0, 0, 0)).decode()
+    # same argument order as the reference's flat kernel
+    # (src/gpuarray_elemwise.c:472-488): n, then data+offset per array
+    assert "elem(const ga_size n, GLOBAL_MEM ga_float *a_p, const ga_size a_offset" in src
+    assert "ga_chunk16" in src and "__builtin_nontemporal_load" in src
+    assert "c = a*b + 0.5f;" in src
+    err, log = compile_src(src.encode())
+    assert err == 0, log
+
+
+@pytest.mark.parametrize("nd,idx64,tmask", [(1, 0, 0), (2, 0, 0), (4, 1, 0), (2, 0, 1), (3, 1, 5)])
+def test_strided_variants_compile(nd, idx64, tmask):
+    src = take_string(gen_elemwise(b"", b"c = a*b + 0.5f", 3, args_of(F32), 0, 1, nd, idx64, tmask))
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
+def test_mixed_types_scalars_and_half_compile():
+    spec = [("x", _lib.GA_HALF, R), ("k", _lib.GA_DOUBLE, S), ("m", _lib.GA_UBYTE, R),
+            ("y", _lib.GA_HALF, R | W), ("z", _lib.GA_LONG, W)]
+    expr = b"y = x * (ga_float)k + y; z = (ga_long)m + (ga_long)y"
+    for strided, nd, tm in [(0, 0, 0), (1, 2, 0), (1, 2, 0b1001)]:
+        src = take_string(gen_elemwise(b"", expr, 5, args_of(spec), _lib.GE_CONVERT_F16, strided,
+                                       nd, 0, tm))
+        err, log = compile_src(src)
+        assert err == 0, log
+
+
+def test_preamble_and_prelude_vocabulary():
+    # pygpu/tests/test_elemwise.py:310-346 uses INFINITY from a preamble
+    pre = (b"WITHIN_KERNEL ga_float clampinf(ga_float v) { return v > 1e30f ? INFINITY : v; }\n"
+           b"#define TWO_PI (2 * M_PI)\n")
+    expr = b"c = clampinf(a) + (ga_float)TWO_PI * b + (isnan(a) ? NAN : 0.0f)"
+    src = take_string(gen_elemwise(pre, expr, 3, args_of(F32), 0, 0, 0, 0, 0))
+    err, log = compile_src(src)
+    assert err == 0, log
+    # a hand-written kernel in the reference's dialect
+    user = b"""#include "cluda.h"
+KERNEL void k(GLOBAL_MEM ga_float *x, ga_size n, GLOBAL_MEM ga_half *h, GLOBAL_MEM ga_int *cnt,
+              GLOBAL_MEM ga_long *lc, GLOBAL_MEM ga_double *dc) {
+  GA_DECL_SHARED_BODY(ga_float, tile)
+  LOCAL_MEM ga_uint hits[GA_WARP_SIZE];
+  ga_size i = GID_0 * LDIM_0 + LID_0;
+  tile[LID_0] = i < n ? x[i] : 0;
+  hits[LID_0 % GA_WARP_SIZE] = 0;
+  local_barrier();
+  if (i < n) {
+    h[i] = ga_float2half(ga_half2float(h[i]) + tile[LID_0]);
+    atom_add_ig(cnt, 1); atom_add_lg(lc, 1); atom_add_dg(dc, 1.0); atom_add_fg(x, 1.0f);
+    atom_add_Il(&hits[0], 1u); atom_xchg_ig(cnt, 2); atom_add_eg(h, h[i]); atom_xchg_eg(h, h[i]);
+  }
+  if (GDIM_0 > 1 && LID_1 + LID_2 + GID_1 + GID_2 + LDIM_1 + LDIM_2 + GDIM_1 + GDIM_2 > 1000) x[0] = MAXFLOAT;
+}
+"""
+    err, log = compile_src(user)
+    assert err == 0, log
+
+
+def test_bad_expression_is_a_compile_error_with_a_log():
+    src = take_string(gen_elemwise(b"", b"c = a +* undefined_name", 3, args_of(F32), 0, 0, 0, 0, 0))
+    err, log = compile_src(src)
+    assert err == _lib.GA_IMPL_ERROR
+    assert "undefined_name" in log or "error" in log
+
+
+@pytest.mark.parametrize("cfg", [
+    # op, src, d0, d1, G, V, U
+    (_lib.GA_REDUCE_SUM, _lib.GA_FLOAT, _lib.GA_FLOAT, _lib.GA_LONG, 256, 4, 4),
+    (_lib.GA_REDUCE_SUM, _lib.GA_HALF, _lib.GA_FLOAT, _lib.GA_LONG, 256, 1, 2),
+    (_lib.GA_REDUCE_SUM, _lib.GA_INT, _lib.GA_LONG, _lib.GA_LONG, 256, 1, 4),
+    (_lib.GA_REDUCE_MAXANDARGMAX, _lib.GA_FLOAT, _lib.GA_FLOAT, _lib.GA_ULONG, 64, 4, 4),
+    (_lib.GA_REDUCE_ARGMIN, _lib.GA_DOUBLE, _lib.GA_DOUBLE, _lib.GA_LONG, 64, 2, 4),
+    (_lib.GA_REDUCE_ANY, _lib.GA_UBYTE, _lib.GA_BOOL, _lib.GA_LONG, 64, 1, 4),
+    (_lib.GA_REDUCE_ALL, _lib.GA_HALF, _lib.GA_BOOL, _lib.GA_LONG, 64, 8, 1),
+    (_lib.GA_REDUCE_XOR, _lib.GA_USHORT, _lib.GA_USHORT, _lib.GA_LONG, 256, 8, 2),
+    (_lib.GA_REDUCE_PRODNZ, _lib.GA_BYTE, _lib.GA_HALF, _lib.GA_LONG, 64, 16, 1),
+])
+def test_reduction_variants_compile(cfg):
+    src = take_string(gen_reduction(*cfg))
+    assert b"redux_row" in src and b"redux_col" in src and b"redux_final" in src
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
+def test_reduction_plan_struct_matches_the_kernel_side():
+    # 7 arrays of 8 x int64 + 6 x int64 + 4 x int32
+    import re
+    src = take_string(gen_reduction(0, _lib.GA_FLOAT, _lib.GA_FLOAT, _lib.GA_LONG, 64, 1, 1)).decode()
+    body = re.search(r"struct rd_plan \{(.*?)\};", src, re.S).group(1)
+    assert body.count("[RD_MAXD]") == 7 and "#define RD_MAXD 8" in src

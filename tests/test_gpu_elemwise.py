@@ -1,0 +1,400 @@
+"""GpuElemwise on the device, through the C ABI, against
+  - the literal results of the reference's tests (tests/check_elemwise.c:39-880),
+  - the CPU checker (oracle/) on seeded random layouts, bit for bit,
+  - NumPy at the BASELINE shapes.
+Float expressions are compiled without contraction, so a*b+c is two roundings
+and results are bit-identical to the checker and to NumPy."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import libgpuarray_amd as ga
+from libgpuarray_amd import _lib, gpuarray
+from support import to_gpu_view, read_root, root_of, arg
+
+pytestmark = pytest.mark.gpu
+lib = _lib.lib
+F16 = np.array([0x0000, 0x3c00, 0x4000, 0x4200, 0x4400, 0x4500, 0x4600, 0x4700, 0x4800, 0x4880],
+               dtype=np.uint16).view(np.float16)
+BCAST, NOCOLLAPSE, PAD = _lib.GE_BROADCAST, _lib.GE_NOCOLLAPSE, _lib.GE_PADSHAPE
+
+
+def raw_call(ge, arrays_and_scalars, flags):
+    """GpuElemwise_call with explicit flags; returns the error code."""
+    keep = []
+    ptrs = (C.c_void_p * len(arrays_and_scalars))()
+    for i, v in enumerate(arrays_and_scalars):
+        if isinstance(v, ga.GpuArray):
+            ptrs[i] = C.addressof(v.ga)
+        else:
+            keep.append(np.ascontiguousarray(v))
+            ptrs[i] = keep[-1].ctypes.data
+    return lib.GpuElemwise_call(ge.ge, ptrs, flags)
+
+
+def dev(values, shape, order="C", dtype=np.uint32, ctx=None):
+    """Device array whose MEMORY holds `values` in order (GpuArray_write into a
+    C- or F-ordered array, as the reference tests do)."""
+    g = gpuarray.empty(shape, dtype, order, context=ctx)
+    flat = np.array(values, dtype=dtype)
+    assert lib.GpuArray_write(g._ptr(), flat.ctypes.data, flat.nbytes) == 0
+    return g
+
+
+def mem(g, count, dtype=np.uint32):
+    out = np.zeros(count, dtype)
+    assert lib.GpuArray_read(out.ctypes.data, out.nbytes, g._ptr()) == 0
+    return out
+
+
+def add_u32(ctx, nd=0, flags=0, expr="c = a + b", dt="uint32"):
+    return ga.GpuElemwise(ctx, expr, [arg("a", dt, read=True), arg("b", dt, read=True),
+                                      arg("c", dt, write=True)], nd=nd,
+                          convert_f16=bool(flags & _lib.GE_CONVERT_F16))
+
+
+# ---- the reference's scenarios ---------------------------------------------------
+
+def test_contig_simple(ctx):
+    a, b = dev([1, 2, 3], (3,), ctx=ctx), dev([4, 5, 6], (3,), ctx=ctx)
+    c = gpuarray.empty((3,), "uint32", context=ctx)
+    assert raw_call(add_u32(ctx, 1), [a, b, c], NOCOLLAPSE) == 0
+    assert mem(c, 3).tolist() == [5, 7, 9]
+
+
+def test_contig_and_basic_f16(ctx):
+    ge = add_u32(ctx, 1, _lib.GE_CONVERT_F16, dt="float16")
+    a = dev(F16[[1, 2, 3]], (3,), dtype=np.float16, ctx=ctx)
+    b = dev(F16[[4, 5, 6]], (3,), dtype=np.float16, ctx=ctx)
+    c = gpuarray.empty((3,), "float16", context=ctx)
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE) == 0
+    assert np.array_equal(mem(c, 3, np.float16).view(np.uint16), F16[[5, 7, 9]].view(np.uint16))
+    a = dev(F16[[1, 2, 3]], (1, 3), dtype=np.float16, ctx=ctx)
+    b = dev(F16[[4, 5, 6]], (1, 3), "F", dtype=np.float16, ctx=ctx)
+    c = gpuarray.empty((1, 3), "float16", context=ctx)
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE) == 0
+    assert np.array_equal(mem(c, 3, np.float16).view(np.uint16), F16[[5, 7, 9]].view(np.uint16))
+
+
+def test_zero_sized(ctx):
+    ge = add_u32(ctx, 1)
+    z = [gpuarray.empty((0,), "uint32", context=ctx) for _ in range(3)]
+    assert raw_call(ge, z, NOCOLLAPSE) == 0
+    a = gpuarray.empty((0, 3), "uint32", "C", context=ctx)
+    b = gpuarray.empty((0, 3), "uint32", "F", context=ctx)
+    c = gpuarray.empty((0, 3), "uint32", "C", context=ctx)
+    assert raw_call(ge, [a, b, c], 0) == 0
+
+
+def test_basic_simple_and_offset(ctx):
+    ge = add_u32(ctx, 2)
+    a = dev([1, 2, 3], (1, 3), ctx=ctx)
+    b = dev([4, 5, 6], (1, 3), "F", ctx=ctx)
+    c = gpuarray.empty((1, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE) == 0
+    assert mem(c, 3).tolist() == [5, 7, 9]
+    # "simulate indexing": offset 12 bytes into a 6-element row (check_elemwise.c:339-345)
+    a = gpuarray.empty((1, 6), "uint32", context=ctx)
+    a.ga.offset = 12
+    a.ga.dimensions[1] = 3
+    lib.GpuArray_fix_flags(a._ptr())
+    data = np.array([1, 2, 3], np.uint32)
+    assert lib.GpuArray_write(a._ptr(), data.ctypes.data, 12) == 0
+    c = gpuarray.empty((1, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE) == 0
+    assert mem(c, 3).tolist() == [5, 7, 9]
+    a.ga.offset = 0   # restore before the array is released
+
+
+def test_basic_scalar(ctx):
+    ge = ga.GpuElemwise(ctx, "c = a + x * b",
+                        [arg("a", "uint32", read=True), arg("x", "uint32", scalar=True),
+                         arg("b", "uint32", read=True), arg("c", "uint32", write=True)], nd=2)
+    a = dev([1, 2, 3], (1, 3), ctx=ctx)
+    b = dev([4, 5], (2, 1), "F", ctx=ctx)
+    c = gpuarray.empty((2, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a, np.uint32(2), b, c], BCAST) == 0
+    assert mem(c, 6).tolist() == [9, 10, 11, 11, 12, 13]
+
+
+def test_basic_scalar_dtype(ctx):
+    ge = ga.GpuElemwise(ctx, "y = a * x + y",
+                        [arg("a", "float32", scalar=True), arg("x", "int32", read=True),
+                         arg("y", "float32", read=True, write=True)], nd=2)
+    x = dev([0, 1, 2, 3], (2, 2), dtype=np.int32, ctx=ctx)
+    y = dev([2.0, 2.0, 2.0, 2.0], (2, 2), "F", dtype=np.float32, ctx=ctx)
+    assert raw_call(ge, [np.float32(1.1), x, y], 0) == 0
+    assert np.array_equal(mem(y, 4, np.float32), np.array([2.0, 4.2, 3.1, 5.3], np.float32))
+
+
+def test_basic_remove1_and_collapse(ctx):
+    ge = add_u32(ctx, 0)
+    a = dev([1, 2, 3, 4, 5, 6], (1, 3, 2, 1), ctx=ctx)
+    b = dev([7, 8, 9, 10, 11, 12], (1, 3, 2, 1), "F", ctx=ctx)
+    c = gpuarray.empty((1, 3, 2, 1), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], 0) == 0
+    assert mem(c, 6).tolist() == [8, 12, 11, 15, 14, 18]
+    a = dev([1, 2, 3, 4, 5, 6], (2, 3), ctx=ctx)
+    b = dev([7, 8, 9, 10, 11, 12], (2, 3), ctx=ctx)
+    c = gpuarray.empty((2, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], 0) == 0
+    assert mem(c, 6).tolist() == [8, 10, 12, 14, 16, 18]
+
+
+def test_basic_broadcast_and_padshape(ctx):
+    ge = add_u32(ctx, 2)
+    a = dev([1, 2, 3], (1, 3), ctx=ctx)
+    b = dev([4, 5], (2, 1), "F", ctx=ctx)
+    c = gpuarray.empty((2, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE) == _lib.GA_VALUE_ERROR
+    assert "Mismatched dimension" in ctx.error()
+    assert raw_call(ge, [a, b, c], NOCOLLAPSE | BCAST) == 0
+    assert mem(c, 6).tolist() == [5, 6, 7, 6, 7, 8]
+    a1 = dev([1, 2, 3], (3,), ctx=ctx)
+    c = gpuarray.empty((2, 3), "uint32", context=ctx)
+    assert raw_call(ge, [a1, b, c], NOCOLLAPSE) == _lib.GA_VALUE_ERROR
+    assert raw_call(ge, [a1, b, c], NOCOLLAPSE | BCAST | PAD) == 0
+    assert mem(c, 6).tolist() == [5, 6, 7, 6, 7, 8]
+    # outputs never broadcast (src/gpuarray_elemwise.c:348-354)
+    c1 = gpuarray.empty((1, 3), "uint32", context=ctx)
+    big = gpuarray.empty((2, 3), "uint32", context=ctx)
+    assert raw_call(ge, [big, a, c1], BCAST) == _lib.GA_VALUE_ERROR
+
+
+def test_basic_neg_strides(ctx):
+    ge = add_u32(ctx, 1)
+    a = dev([1, 2, 3, 4, 5, 6], (6,), ctx=ctx)
+    b = dev([7, 8, 9, 10, 11, 12], (6,), ctx=ctx)
+    st, sp, se = (_lib.c_ssize_t * 1)(5), (_lib.c_ssize_t * 1)(-1), (_lib.c_ssize_t * 1)(-1)
+    assert lib.GpuArray_index_inplace(b._ptr(), st, sp, se) == 0
+    c = gpuarray.empty((6,), "uint32", context=ctx)
+    assert raw_call(ge, [a, b, c], 0) == 0
+    assert mem(c, 6).tolist() == [13] * 6
+
+
+def test_new_reports_compile_errors(ctx):
+    with pytest.raises(ga.GpuArrayException) as e:
+        add_u32(ctx, expr="c = a + not_a_name")
+    assert "not_a_name" in str(e.value)
+    # no output array at all (src/gpuarray_elemwise.c:301-302)
+    ge = ga.GpuElemwise(ctx, "a + b", [arg("a", "uint32", read=True), arg("b", "uint32", read=True)])
+    a = dev([1, 2, 3], (1, 3), ctx=ctx)
+    b = dev([4, 5], (2, 1), "F", ctx=ctx)
+    assert raw_call(ge, [a, b], BCAST) == _lib.GA_VALUE_ERROR
+
+
+# ---- parity with the CPU checker on random layouts ---------------------------------
+
+def random_view(rng, shape, dtype):
+    """A view of `shape` with random memory order, steps, reversals and offset."""
+    nd = len(shape)
+    perm = rng.permutation(nd)
+    steps = [int(rng.choice([1, 1, 2, 3])) for _ in range(nd)]
+    pad = [int(rng.integers(0, 3)) for _ in range(nd)]
+    big = [shape[perm[i]] * steps[i] + pad[i] for i in range(nd)]
+    base = rng.normal(0, 1, big).astype(dtype)
+    idx = tuple(slice(pad[i], pad[i] + shape[perm[i]] * steps[i], steps[i]) for i in range(nd))
+    v = base[idx].transpose(np.argsort(perm))
+    for ax in range(nd):
+        if rng.random() < 0.25:
+            v = np.flip(v, ax)
+    assert v.shape == tuple(shape)
+    return v
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_layouts_bit_exact_vs_checker(seed, ctx, oracle):
+    rng = np.random.default_rng(100 + seed)
+    ge = ga.GpuElemwise(ctx, "out = a + b*c",
+                        [arg("a", "float32", read=True), arg("b", "float32", read=True),
+                         arg("c", "float32", read=True), arg("out", "float32", write=True)])
+    for _ in range(12):
+        nd = int(rng.integers(1, 5))
+        shape = [int(x) for x in rng.integers(1, [40, 20, 9, 5][:nd])]
+        rng.shuffle(shape)
+        ins = []
+        for _k in range(3):
+            shp = [d if rng.random() < 0.7 else 1 for d in shape]
+            ins.append(random_view(rng, shp, np.float32))
+        out = random_view(rng, shape, np.float32)
+        g_in = [to_gpu_view(v, ctx)[0] for v in ins]
+        g_out, g_root = to_gpu_view(out, ctx)
+        # the checker runs on a host copy of the output's whole buffer, viewed
+        # with the same offset and strides
+        want_root = np.ascontiguousarray(root_of(out).reshape(-1, order="A")).copy()
+        off = out.__array_interface__["data"][0] - root_of(out).__array_interface__["data"][0]
+        host_out = np.ndarray(shape=out.shape, dtype=np.float32, buffer=want_root.data,
+                              offset=off, strides=out.strides)
+        assert oracle.elemwise(oracle.A_PLUS_BC_F32, ins + [host_out], [0, 0, 0, 1],
+                               flags=BCAST) == 0
+        assert raw_call(ge, g_in + [g_out], BCAST) == 0
+        got_root = np.asarray(g_root)[:want_root.nbytes].view(np.float32)
+        assert np.array_equal(got_root, want_root), (shape, [v.strides for v in ins], out.strides)
+        assert np.array_equal(host_out, np.broadcast_to(ins[0] + ins[1] * ins[2], out.shape))
+
+
+def test_dtype_matrix_copy_cast_vs_numpy(ctx):
+    rng = np.random.default_rng(7)
+    dts = ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64",
+           "float16", "float32", "float64"]
+    src = rng.uniform(0, 100, (33, 17))
+    for sd in dts:
+        n = src.astype(sd)
+        g = gpuarray.array(n, context=ctx)
+        for dd in dts:
+            got = np.asarray(g.T.astype(dd))       # transposed source -> tiled kernel
+            assert np.array_equal(got, n.T.astype(dd)), (sd, dd)
+
+
+def test_all_fortran_inputs_take_the_flat_path(ctx):
+    rng = np.random.default_rng(8)
+    a = np.asfortranarray(rng.normal(size=(130, 70)).astype(np.float32))
+    b = np.asfortranarray(rng.normal(size=(130, 70)).astype(np.float32))
+    ga_, gb = gpuarray.array(a, order="F", context=ctx), gpuarray.array(b, order="F", context=ctx)
+    gc = gpuarray.empty((130, 70), "float32", "F", context=ctx)
+    ge = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [arg("a", "float32", read=True),
+                                                arg("b", "float32", read=True),
+                                                arg("c", "float32", write=True)])
+    ge(ga_, gb, gc)
+    assert np.array_equal(np.asarray(gc), a * b + np.float32(0.5))
+    # C output, F inputs: general path, dims sorted by the output's strides
+    gc2 = gpuarray.empty((130, 70), "float32", "C", context=ctx)
+    ge(ga_, gb, gc2)
+    assert np.array_equal(np.asarray(gc2), a * b + np.float32(0.5))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 65, 255, 256, 257, 1023, 4095, 4096, 4097,
+                               65535, 1 << 20, (1 << 20) + 1, (1 << 22) + 3])
+def test_flat_sizes_tails_and_misalignment(n, ctx, oracle):
+    rng = np.random.default_rng(n)
+    a = rng.uniform(-1, 1, n + 3).astype(np.float32)
+    b = rng.uniform(-1, 1, n + 3).astype(np.float32)
+    ge = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [arg("a", "float32", read=True),
+                                                arg("b", "float32", read=True),
+                                                arg("c", "float32", write=True)])
+    want = np.empty(n, np.float32)
+    for off in (0, 1, 3):          # element offsets: 0 keeps 16-byte alignment, 1 and 3 break it
+        av, bv = a[off:off + n], b[off:off + n]
+        oracle.elemwise_contig_muladd(np.ascontiguousarray(av), np.ascontiguousarray(bv), want)
+        gav, gbv = to_gpu_view(av, ctx)[0], to_gpu_view(bv, ctx)[0]
+        gc = gpuarray.zeros((n + 3,), "float32", context=ctx)
+        ge(gav, gbv, gc[off:off + n])
+        got = np.asarray(gc)
+        assert np.array_equal(got[off:off + n], want)
+        assert np.all(got[:off] == 0) and np.all(got[off + n:] == 0)   # nothing outside the view
+
+
+def test_small_types_vectorised_flat_path(ctx):
+    rng = np.random.default_rng(9)
+    for dt in ("uint8", "int16", "float16", "float64", "int64"):
+        n = 100003
+        a = rng.integers(0, 50, n).astype(dt)
+        b = rng.integers(0, 50, n).astype(dt)
+        ge = ga.GpuElemwise(ctx, "c = a + b", [arg("a", dt, read=True), arg("b", dt, read=True),
+                                               arg("c", dt, write=True)], convert_f16=True)
+        gc = gpuarray.empty((n,), dt, context=ctx)
+        ge(gpuarray.array(a, context=ctx), gpuarray.array(b, context=ctx), gc)
+        assert np.array_equal(np.asarray(gc), (a + b).astype(dt)), dt
+
+
+def test_inplace_and_multiple_outputs(ctx):
+    rng = np.random.default_rng(10)
+    x = rng.normal(size=(257, 33)).astype(np.float32)
+    g = gpuarray.array(x, context=ctx)
+    s = gpuarray.empty(x.shape, "float32", context=ctx)
+    d = gpuarray.empty(x.shape, "float64", "F", context=ctx)
+    ge = ga.GpuElemwise(ctx, "s = x * 2.0f; d = (ga_double)x - 1.0; x = -x",
+                        [arg("x", "float32", read=True, write=True), arg("s", "float32", write=True),
+                         arg("d", "float64", write=True)])
+    ge(g, s, d)
+    assert np.array_equal(np.asarray(g), -x)
+    assert np.array_equal(np.asarray(s), x * np.float32(2))
+    assert np.array_equal(np.asarray(d), x.astype(np.float64) - 1.0)
+
+
+def test_zero_dimensional_and_size_one(ctx):
+    ge = add_u32(ctx, dt="float32")
+    a = gpuarray.array(np.float32(2.5), context=ctx)
+    b = gpuarray.array(np.float32(4.0), context=ctx)
+    c = gpuarray.empty((), "float32", context=ctx)
+    ge(a, b, c)
+    assert np.asarray(c) == np.float32(6.5)
+    c3 = gpuarray.empty((1, 1, 1), "float32", context=ctx)
+    ge(a, b, c3)                                      # padshape + broadcast defaults
+    assert np.asarray(c3).ravel()[0] == np.float32(6.5)
+
+
+# ---- BASELINE shapes -----------------------------------------------------------------
+
+def test_config1_contiguous_2p24(ctx, oracle):
+    rng = np.random.default_rng(0)
+    n = 1 << 24
+    a = rng.uniform(-1, 1, n).astype(np.float32)
+    b = rng.uniform(-1, 1, n).astype(np.float32)
+    ge = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [arg("a", "float32", read=True),
+                                                arg("b", "float32", read=True),
+                                                arg("c", "float32", write=True)])
+    gc = gpuarray.empty((n,), "float32", context=ctx)
+    ge(gpuarray.array(a, context=ctx), gpuarray.array(b, context=ctx), gc)
+    got = np.asarray(gc)
+    want = np.empty(n, np.float32)
+    oracle.elemwise_contig_muladd(a, b, want)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, a * b + np.float32(0.5))
+
+
+def test_config2_transposed_broadcast_4096(ctx, oracle):
+    rng = np.random.default_rng(1)
+    a = rng.normal(0, 1, (4096, 4096)).astype(np.float32)
+    b = rng.normal(0, 1, (1, 4096)).astype(np.float32)
+    c = rng.normal(0, 1, (4096, 1)).astype(np.float32)
+    ge = ga.GpuElemwise(ctx, "out = a + b*c",
+                        [arg("a", "float32", read=True), arg("b", "float32", read=True),
+                         arg("c", "float32", read=True), arg("out", "float32", write=True)])
+    g_a = gpuarray.array(a, context=ctx).T
+    assert g_a.strides == (4, 16384) and g_a.flags.f_contiguous and not g_a.flags.c_contiguous
+    out = gpuarray.empty((4096, 4096), "float32", context=ctx)
+    # without GE_BROADCAST the call is refused, as in the reference
+    assert raw_call(ge, [g_a, gpuarray.array(b, context=ctx), gpuarray.array(c, context=ctx), out],
+                    0) == _lib.GA_VALUE_ERROR
+    ge(g_a, gpuarray.array(b, context=ctx), gpuarray.array(c, context=ctx), out)
+    got = np.asarray(out)
+    assert np.array_equal(got, a.T + b * c)
+    # the checker, on a corner that it finishes quickly
+    sub = np.zeros((256, 256), np.float32)
+    assert oracle.elemwise(oracle.A_PLUS_BC_F32, [a.T[:256, :256], b[:, :256], c[:256], sub],
+                           [0, 0, 0, 1], flags=BCAST) == 0
+    assert np.array_equal(got[:256, :256], sub)
+
+
+def test_config5_strided_copy_of_the_view(ctx):
+    rng = np.random.default_rng(6)
+    base = rng.integers(-1000, 1001, (64, 128, 1024), dtype=np.int32)
+    g = gpuarray.array(base, context=ctx)[:, :, ::2]
+    assert g.strides == (128 * 1024 * 4, 4096, 8)
+    c = g.copy()
+    assert c.flags.c_contiguous and np.array_equal(np.asarray(c), base[:, :, ::2])
+
+
+def test_linearity_at_full_size(ctx):
+    # size-independent property at the 2^28 target shape: (a*b + 0.5) with
+    # b == 1 is a + 0.5 exactly, and with a == 0 is 0.5 everywhere
+    n = 1 << 28
+    ge = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [arg("a", "float32", read=True),
+                                                arg("b", "float32", read=True),
+                                                arg("c", "float32", write=True)])
+    a = gpuarray.zeros((n,), "float32", context=ctx)
+    b = gpuarray.empty((n,), "float32", context=ctx)
+    c = gpuarray.empty((n,), "float32", context=ctx)
+    ge(a, b, c)                                   # a == 0 but b is garbage: NaN/inf can appear
+    fill = ga.GpuElemwise(ctx, "b = 1.0f", [arg("b", "float32", write=True)])
+    fill(b)
+    iota = ga.GpuElemwise(ctx, "a = (ga_float)(i & 1023)", [arg("a", "float32", write=True)])
+    iota(a)
+    ge(a, b, c)
+    # sample three windows, including the very end
+    for lo in (0, n // 2 - 5000, n - 10000):
+        got = np.asarray(c[lo:lo + 10000])
+        want = (np.arange(lo, lo + 10000) & 1023).astype(np.float32) + np.float32(0.5)
+        assert np.array_equal(got, want)

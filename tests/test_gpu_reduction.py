@@ -1,0 +1,464 @@
+"""Reductions on the device, through the C ABI, against
+  - the reference's own four maxandargmax tests (tests/check_reduction.c) on
+    its PCG32 data, bit for bit, with the CPU checker as the expected value,
+  - the checker / NumPy on seeded random layouts, every op and dtype,
+  - the Python layer's rules for sum/prod/all/any (pygpu/tests/test_reduction.py).
+Integer, boolean and index results must be identical; float sums are held to
+1e-5 of the float64 sum (relative to the sum of magnitudes when the result
+itself is tiny), fp16 inputs to 1e-2."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import libgpuarray_amd as ga
+from libgpuarray_amd import _lib, gpuarray, reduction as R
+from support import to_gpu_view, gen_gpuarray
+
+pytestmark = pytest.mark.gpu
+lib = _lib.lib
+
+
+def np_maxandargmax(x, redux, op="max"):
+    free = [i for i in range(x.ndim) if i not in redux]
+    y = x.transpose(free + list(redux)).reshape([x.shape[i] for i in free] + [-1])
+    return (y.max(-1), y.argmax(-1)) if op == "max" else (y.min(-1), y.argmin(-1))
+
+
+def assert_sum_close(got, x64sum, abs64sum, rtol=1e-5):
+    got = np.asarray(got, dtype=np.float64)
+    err = np.abs(got - x64sum)
+    # 1e-5 of the result; when cancellation makes the result tiny, of the
+    # sum of magnitudes times the float32 epsilon (what any order can promise)
+    bound = np.maximum(rtol * np.abs(x64sum), abs64sum * 6e-8 * 8)
+    assert np.all(err <= bound), (err.max(), bound.min())
+
+
+# ---- the reference's four tests ------------------------------------------------------
+
+@pytest.mark.parametrize("shape,redux", [
+    ((32, 50, 79), [0, 2]),                       # test_reduction
+    ((32, 50, 79), [2, 0]),                       # test_idxtranspose
+    ((1171, 373, 2, 1, 2, 1, 2, 1), [2, 4, 7, 5]),  # test_veryhighrank
+    ((32, 50, 79), [0, 1, 2]),                    # test_alldimsreduced
+])
+def test_reference_maxandargmax_tests(shape, redux, ctx, oracle):
+    x = oracle.pcg_fill_f32(int(np.prod(shape)), seed=1).reshape(shape)
+    g = gpuarray.array(x, context=ctx)
+    oshape = tuple(d for i, d in enumerate(shape) if i not in redux)
+    gmax = gpuarray.empty(oshape, "float32", context=ctx)
+    garg = gpuarray.empty(oshape, "uint64", context=ctx)    # the tests allocate GA_ULONG
+    gmax.memset(0xff)
+    garg.memset(0xff)
+    arr = (C.c_uint * len(redux))(*redux)
+    assert lib.GpuArray_maxandargmax(gmax._ptr(), garg._ptr(), g._ptr(), len(redux), arr) == 0
+    wm, wa = oracle.maxandargmax(x, redux)
+    assert np.array_equal(np.asarray(gmax), wm)
+    assert np.array_equal(np.asarray(garg).astype(np.int64), wa)
+    nm, na = np_maxandargmax(x, redux)
+    assert np.array_equal(wm, nm) and np.array_equal(wa, na)
+
+
+def test_maxandargmax_argument_errors(ctx):         # src/gpuarray_reduction.c:198-261
+    g = gpuarray.zeros((4, 5), "float32", context=ctx)
+    m = gpuarray.empty((4,), "float32", context=ctx)
+    a = gpuarray.empty((4,), "uint64", context=ctx)
+    def call(n, axes, src=g, dm=m, da=a):
+        arr = (C.c_uint * max(len(axes), 1))(*axes)
+        return lib.GpuArray_maxandargmax(dm._ptr() if dm is not None else None,
+                                         da._ptr() if da is not None else None,
+                                         src._ptr() if src is not None else None, n, arr)
+    assert call(1, [1]) == 0
+    assert call(0, []) == _lib.GA_INVALID_ERROR
+    assert call(3, [0, 1, 1]) == _lib.GA_INVALID_ERROR
+    assert call(2, [1, 1]) == _lib.GA_INVALID_ERROR
+    assert call(1, [2]) == _lib.GA_INVALID_ERROR
+    assert call(1, [1], dm=None) == _lib.GA_INVALID_ERROR
+    assert call(1, [1], src=None) == _lib.GA_INVALID_ERROR
+    z = gpuarray.zeros((), "float32", context=ctx)
+    assert call(1, [0], src=z) == _lib.GA_INVALID_ERROR
+    # destination shape is checked here (the reference does not, and would
+    # write out of bounds)
+    wrong = gpuarray.empty((5,), "float32", context=ctx)
+    assert call(1, [1], dm=wrong) == _lib.GA_VALUE_ERROR
+
+
+def test_ties_nan_and_signed_zero(ctx, oracle):
+    x = np.zeros((6, 300), np.float32)
+    x[0, [250, 17, 123]] = 4.0                    # ties -> first index
+    x[1, :] = 2.0                                 # constant row -> 0
+    x[2, :] = np.arange(300)                      # increasing -> last
+    x[3, 5] = np.nan; x[3, 9] = 1.0               # NaN not first: ignored
+    x[4, 0] = np.nan; x[4, 9] = 1.0               # NaN first: stays
+    x[5, :] = -0.0; x[5, 100] = 0.0               # equal zeros: first one scanned
+    g = gpuarray.array(x, context=ctx)
+    v, i = R.maxandargmax(g, axis=1)
+    wm, wa = oracle.maxandargmax(x, [1])
+    got_v, got_i = np.asarray(v), np.asarray(i)
+    assert np.array_equal(got_i, wa) and got_i.tolist() == [17, 0, 299, 9, 0, 0]
+    assert np.array_equal(got_v.view(np.uint32), wm.view(np.uint32))     # bits, incl. NaN and -0
+    # plain max gives the same values as maxandargmax
+    assert np.array_equal(np.asarray(R.max(g, axis=1)).view(np.uint32), wm.view(np.uint32))
+    # ties across a split full reduction and across wavefronts
+    big = np.zeros(1 << 20, np.float32)
+    big[[900000, 70000, 1 << 19]] = 1.0
+    v, i = R.maxandargmax(gpuarray.array(big, context=ctx))
+    assert np.asarray(v) == 1.0 and np.asarray(i) == 70000
+    v, i = R.minandargmin(gpuarray.array(-big, context=ctx))
+    assert np.asarray(v) == -1.0 and np.asarray(i) == 70000
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_layouts_arg_reductions_vs_checker(seed, ctx, oracle):
+    rng = np.random.default_rng(200 + seed)
+    for _ in range(10):
+        nd = int(rng.integers(1, 5))
+        shape = [int(x) for x in rng.integers(1, [70, 12, 7, 4][:nd])]
+        rng.shuffle(shape)
+        dt = rng.choice(["float32", "float64", "int32", "float16"])
+        base = (rng.integers(-20, 20, [2 * d + 1 for d in shape])).astype(dt)  # many ties
+        idx = tuple(slice(int(rng.integers(0, 2)), None, 2) for _ in shape)
+        v = base[idx][tuple(slice(0, d) for d in shape)]
+        v = v.transpose(rng.permutation(nd))
+        nr = int(rng.integers(1, nd + 1))
+        redux = [int(a) for a in rng.permutation(nd)[:nr]]
+        g, _ = to_gpu_view(v, ctx)
+        gv, gi = R._arg_reduce(g, "maxandargmax", redux, True)
+        wm, wa = oracle.maxandargmax(v, redux)
+        assert np.array_equal(np.asarray(gi), wa), (v.shape, v.strides, redux, dt)
+        assert np.array_equal(np.asarray(gv), wm)
+
+
+def test_destination_strides_are_honoured(ctx, oracle):
+    rng = np.random.default_rng(31)
+    x = rng.normal(size=(9, 40, 11)).astype(np.float32)
+    g = gpuarray.array(x, context=ctx)
+    # results go into every other column of a Fortran-ordered block
+    bigm = gpuarray.zeros((9, 22), "float32", "F", context=ctx)
+    biga = gpuarray.zeros((9, 22), "int64", "F", context=ctx)
+    dm, da = bigm[:, ::2], biga[:, ::2]
+    op = ga.GpuReduction(ctx, "maxandargmax", "float32")
+    op(g, [1], d0=dm, d1=da)
+    wm, wa = oracle.maxandargmax(x, [1])
+    assert np.array_equal(np.asarray(bigm)[:, ::2], wm) and np.all(np.asarray(bigm)[:, 1::2] == 0)
+    assert np.array_equal(np.asarray(biga)[:, ::2], wa)
+
+
+# ---- sum / prod / all / any: the Python layer's rules ---------------------------------
+
+DTYPES = ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64",
+          "float32", "float64"]
+
+
+@pytest.mark.parametrize("shape,redux", [
+    ((10,), [True]), ((20, 30), [True, True]), ((20, 30), [True, False]), ((20, 30), [False, True]),
+    ((8, 5, 10), [True, True, True]), ((8, 5, 10), [True, True, False]),
+    ((8, 5, 10), [True, False, True]), ((8, 5, 10), [False, True, True]),
+    ((8, 5, 10), [True, False, False]), ((8, 5, 10), [False, True, False]),
+    ((8, 5, 10), [False, False, True]),
+])
+def test_red_array_basic(shape, redux, ctx, oracle):   # pygpu/tests/test_reduction.py:12-53
+    rng = np.random.default_rng(1)
+    axes = tuple(i for i, r in enumerate(redux) if r)
+    for dt in ["int8", "uint8", "int16", "uint16", "int32", "uint32", "float32", "float64"]:
+        c, g = gen_gpuarray(shape, dt, ctx=ctx, rng=rng)
+        out = R.reduce1(g, "sum", dt, axis=axes)          # same dtype in and out, as the test
+        want = c.sum(axis=axes, dtype=dt)
+        assert out.shape == want.shape and out.dtype == np.dtype(dt)
+        if np.dtype(dt).kind in "iu":
+            assert np.array_equal(np.asarray(out), want)
+        else:
+            assert np.allclose(np.asarray(out), want, rtol=2e-5)
+            chk = oracle.reduk("sum", c, list(axes), dt, ls=64)
+            assert np.allclose(np.asarray(out), chk, rtol=2e-5)
+
+
+@pytest.mark.parametrize("redux", [[True, False, False], [True, False, True],
+                                   [False, True, True], [False, True, False]])
+def test_red_big_array(redux, ctx):                    # pygpu/tests/test_reduction.py:41-46
+    rng = np.random.default_rng(2)
+    axes = tuple(i for i, r in enumerate(redux) if r)
+    c, g = gen_gpuarray((2000, 30, 100), "float32", ctx=ctx, rng=rng)
+    out = np.asarray(R.sum(g, axis=axes))
+    want = c.astype(np.float64).sum(axis=axes)
+    assert np.allclose(out, want, rtol=2e-5)
+    assert_sum_close(out, want, np.abs(c.astype(np.float64)).sum(axis=axes))
+
+
+@pytest.mark.parametrize("axis", [None, 0, 1, -1, (0, 1)])
+def test_reduction_ops_meta_and_content(axis, ctx):    # pygpu/tests/test_reduction.py:86-110
+    rng = np.random.default_rng(3)
+    for op in ("all", "any"):
+        c, g = gen_gpuarray((2, 3), "bool", ctx=ctx, rng=rng, high=1.6)
+        rc, rg = getattr(c, op)(axis=axis), getattr(R, op)(g, axis=axis)
+        assert rg.shape == np.shape(rc) and rg.dtype == np.dtype("bool")
+        assert np.array_equal(np.asarray(rg), rc)
+    for op in ("prod", "sum", "min", "max"):
+        for dt in DTYPES:
+            c, g = gen_gpuarray((2, 3), dt, ctx=ctx, rng=rng, high=5)
+            rc, rg = getattr(c, op)(axis=axis), getattr(R, op)(g, axis=axis)
+            assert rg.shape == np.shape(rc), (op, dt)
+            assert rg.dtype == np.asarray(rc).dtype, (op, dt, rg.dtype, np.asarray(rc).dtype)
+            if np.dtype(dt).kind == "f":
+                assert np.allclose(np.asarray(rg), rc, rtol=1e-6)
+            else:
+                assert np.array_equal(np.asarray(rg), rc), (op, dt)
+            # and again into a caller-provided output
+            outg = gpuarray.empty(rg.shape, rg.dtype, context=ctx)
+            getattr(R, op)(g, axis=axis, out=outg)
+            assert np.array_equal(np.asarray(outg), np.asarray(rg))
+
+
+def test_reduction_wrong_out_and_axis(ctx):            # pygpu/tests/test_reduction.py:113-128
+    c, g = gen_gpuarray((2, 3), "float32", ctx=ctx)
+    with pytest.raises(TypeError):
+        R.sum(g, out=gpuarray.empty((2, 3), "int32", context=ctx))
+    with pytest.raises(TypeError):
+        R.sum(g, axis=0, out=gpuarray.empty((2,), "float32", context=ctx))
+    with pytest.raises(ValueError):
+        R.sum(g, axis=2)
+    with pytest.raises(ValueError):
+        R.sum(g, axis=-3)
+    # the C entry point checks shapes itself
+    op = ga.GpuReduction(ctx, "sum", "float32")
+    with pytest.raises(ValueError):
+        op(g, [0], d0=gpuarray.empty((2,), "float32", context=ctx))
+    with pytest.raises(ga.GpuArrayException):
+        op(g, [0, 0], d0=gpuarray.empty((), "float32", context=ctx))
+    with pytest.raises(ga.GpuArrayException):
+        op(g, [], d0=gpuarray.empty((2, 3), "float32", context=ctx))
+    with pytest.raises(ga.GpuArrayException):   # source dtype differs from the operator's
+        op(g.astype("float64"), [0], d0=gpuarray.empty((3,), "float64", context=ctx))
+
+
+def test_reduction_0d_and_empty(ctx):                  # pygpu/tests/test_reduction.py:131-142
+    for val in (True, False):
+        g = gpuarray.array(np.array(val), context=ctx)
+        assert bool(np.asarray(R.any(g))) == val and bool(np.asarray(R.all(g))) == val
+    # reducing an empty axis gives the neutral element; nothing to write when
+    # the result itself is empty
+    e = gpuarray.zeros((4, 0), "float32", context=ctx)
+    assert np.array_equal(np.asarray(R.sum(e, axis=1)), np.zeros(4, np.float32))
+    assert np.array_equal(np.asarray(R.prod(e, axis=1)), np.ones(4, np.float32))
+    assert np.array_equal(np.asarray(R.all(e, axis=1)), np.ones(4, bool))
+    assert np.array_equal(np.asarray(R.any(e, axis=1)), np.zeros(4, bool))
+    assert R.sum(e, axis=0).shape == (0,)
+    with pytest.raises(ValueError):
+        R.max(e, axis=1)
+
+
+def test_float16_is_accepted_with_float32_accumulation(ctx):
+    # the reference refuses float16 here (pygpu/tests/test_reduction.py:145-148);
+    # this engine widens to float32.  NumPy is the only expected value.
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-4, 4, (37, 513)).astype(np.float16)
+    g = gpuarray.array(x, context=ctx)
+    want = x.astype(np.float64).sum(axis=1)
+    got32 = np.asarray(R.sum(g, axis=1, dtype="float32"))
+    assert np.allclose(got32, want, rtol=1e-2) and np.allclose(got32, want, rtol=1e-5, atol=1e-4)
+    got16 = np.asarray(R.sum(g, axis=1))                # float16 result, float32 accumulator
+    assert got16.dtype == np.float16
+    assert np.array_equal(got16, got32.astype(np.float16))
+
+
+# ---- every op, strided layouts, both kernel families, split and unsplit ---------------
+
+def np_reduce(op, x, axes, out_dtype=None):
+    axes = tuple(axes)
+    if op == "sum":
+        return x.sum(axis=axes, dtype=out_dtype)
+    if op == "prod":
+        return x.prod(axis=axes, dtype=out_dtype)
+    if op == "prodnz":
+        return np.where(x == 0, 1, x).prod(axis=axes, dtype=out_dtype)
+    if op == "and":
+        return np.bitwise_and.reduce(x, axis=axes)
+    if op == "or":
+        return np.bitwise_or.reduce(x, axis=axes)
+    if op == "xor":
+        return np.bitwise_xor.reduce(x, axis=axes)
+    if op == "all":
+        return x.all(axis=axes)
+    if op == "any":
+        return x.any(axis=axes)
+    raise KeyError(op)
+
+
+LAYOUTS = [
+    # (base shape, view maker, axes): chosen to hit row/col kernels, vector and
+    # scalar loads, multi-dim reduced and free sets, and split rows
+    ((64, 1000), lambda b: b, [1]),
+    ((64, 1000), lambda b: b, [0]),
+    ((300, 257), lambda b: b[:, 1:], [1]),
+    ((300, 257), lambda b: b.T, [1]),
+    ((3, 70000), lambda b: b, [1]),                 # few long rows: split + second pass
+    ((70000, 3), lambda b: b, [0]),                 # few long columns: split + second pass
+    ((70000, 3), lambda b: b, [1]),                 # many tiny rows
+    ((16, 64, 256), lambda b: b[:, :, ::2], [0, 2]),
+    ((16, 64, 256), lambda b: b[:, :, ::2], [1]),
+    ((16, 64, 256), lambda b: b[:, :, ::2], [2]),
+    ((16, 64, 256), lambda b: b[::-1, :, ::-3], [2, 0]),
+    ((5, 6, 7, 8), lambda b: b.transpose(3, 1, 0, 2), [0, 2]),
+    ((5, 6, 7, 8), lambda b: b, [0, 1, 2, 3]),
+    ((1 << 21,), lambda b: b, [0]),
+]
+
+
+@pytest.mark.parametrize("layout", range(len(LAYOUTS)))
+def test_all_value_ops_on_layouts(layout, ctx):
+    shape, view, axes = LAYOUTS[layout]
+    rng = np.random.default_rng(300 + layout)
+    others = ["uint8", "int64", "float64", "int16", "uint32", "int8"]
+    for dt in ("int32", "float32", others[layout % len(others)]):
+        if np.dtype(dt).kind == "f":
+            base = rng.normal(0, 1, shape).astype(dt)
+        else:
+            base = rng.integers(-3 if np.dtype(dt).kind == "i" else 0, 4, shape).astype(dt)
+        v = view(base)
+        g, _ = to_gpu_view(v, ctx)
+        ops = ["sum", "prod", "prodnz", "all", "any"]
+        if np.dtype(dt).kind in "iu":
+            ops += ["and", "or", "xor"]
+        for op in ops:
+            if op in ("sum", "prod", "prodnz"):
+                odt = R._upcast(dt)
+            elif op in ("all", "any"):
+                odt = np.dtype("bool")
+            else:
+                odt = np.dtype(dt)
+            want = np_reduce(op, v, axes, odt if op in ("sum", "prod", "prodnz") else None)
+            out = R.reduce1(g, op, odt, axis=tuple(axes))
+            got = np.asarray(out)
+            assert got.shape == want.shape, (op, dt)
+            if np.dtype(dt).kind == "f" and op in ("sum",):
+                x64 = v.astype(np.float64)
+                assert_sum_close(got, x64.sum(axis=tuple(axes)), np.abs(x64).sum(axis=tuple(axes)))
+            elif np.dtype(dt).kind == "f" and op in ("prod", "prodnz"):
+                with np.errstate(all="ignore"):
+                    w64 = np_reduce(op, v.astype(np.float64), axes)
+                ok = np.isclose(got, w64, rtol=1e-3) | ~np.isfinite(w64) | (np.abs(w64) < 1e-30)
+                assert np.all(ok), (op, dt)
+            else:
+                assert np.array_equal(got, want), (op, dt, layout)
+        for op in ("max", "min"):
+            want = v.max(axis=tuple(axes)) if op == "max" else v.min(axis=tuple(axes))
+            assert np.array_equal(np.asarray(getattr(R, op)(g, axis=tuple(axes))), want), (op, dt)
+        wm, wa = np_maxandargmax(v, axes, "min")
+        gv, gi = R._arg_reduce(g, "minandargmin", axes, True)
+        assert np.array_equal(np.asarray(gv), wm) and np.array_equal(np.asarray(gi), wa), dt
+        gi = R._arg_reduce(g, "argmax", axes, False)
+        assert np.array_equal(np.asarray(gi), np_maxandargmax(v, axes)[1]), dt
+
+
+def test_integer_invariants(ctx):
+    # exact in any order: permuting the data or reducing axis by axis gives
+    # the same integers
+    rng = np.random.default_rng(41)
+    x = rng.integers(-1000, 1001, (40, 50, 60), dtype=np.int32)
+    g = gpuarray.array(x, context=ctx)
+    both = np.asarray(R.sum(g, axis=(0, 2)))
+    step = np.asarray(R.sum(R.sum(g, axis=2), axis=0))
+    assert np.array_equal(both, step) and np.array_equal(both, x.sum(axis=(0, 2)))
+    perm = rng.permutation(x.reshape(-1))
+    assert np.asarray(R.sum(gpuarray.array(perm, context=ctx))) == x.sum()
+    # wrap-around modulo 2^32 when the result type is the input type
+    big = np.full(100000, 2 ** 30, np.int32)
+    got = np.asarray(R.reduce1(gpuarray.array(big, context=ctx), "sum", "int32"))
+    assert got == np.int32(np.int64(100000 * 2 ** 30).astype(np.int32))
+
+
+def test_sum_is_reproducible_run_to_run(ctx):
+    rng = np.random.default_rng(42)
+    g = gpuarray.array(rng.normal(0, 1, 1 << 22).astype(np.float32), context=ctx)
+    first = np.asarray(R.sum(g)).tobytes()
+    for _ in range(5):
+        assert np.asarray(R.sum(g)).tobytes() == first
+
+
+# ---- BASELINE shapes at full size -----------------------------------------------------
+
+def test_config3a_sum_axis1_8192(ctx, oracle):
+    rng = np.random.default_rng(2)
+    x = rng.normal(0, 1, (8192, 8192)).astype(np.float32)
+    g = gpuarray.array(x, context=ctx)
+    got = np.asarray(R.sum(g, axis=1))
+    x64 = x.astype(np.float64)
+    assert_sum_close(got, x64.sum(axis=1), np.abs(x64).sum(axis=1))
+    # the reference's own order (one group per row, pygpu/reduction.py:85-132)
+    # on the first rows, at its tolerance
+    chk = oracle.reduk("sum", x[:64], [1], "float32", ls=256)
+    assert np.allclose(got[:64], chk, rtol=2e-5, atol=1e-3)
+    # and the other axis (column kernel)
+    got0 = np.asarray(R.sum(g, axis=0))
+    assert_sum_close(got0, x64.sum(axis=0), np.abs(x64).sum(axis=0))
+
+
+def test_config3b_full_sum_2p28(ctx):
+    rng = np.random.default_rng(3)
+    n = 1 << 28
+    x = rng.standard_normal(n, dtype=np.float32)
+    g = gpuarray.array(x, context=ctx)
+    got = float(np.asarray(R.sum(g)))
+    want = float(x.sum(dtype=np.float64))
+    assert abs(got - want) <= 1e-5 * abs(want), (got, want)
+    # size-independent properties: the halves add up, and a shifted copy adds n*shift
+    h = float(np.asarray(R.sum(g[:n // 2]))) + float(np.asarray(R.sum(g[n // 2:])))
+    assert abs(h - want) <= 1e-5 * abs(want)
+    ones = gpuarray.empty((n,), "float32", context=ctx)
+    ga.GpuElemwise(ctx, "o = 1.0f", [ga.arg("o", "float32", write=True)])(ones)
+    assert float(np.asarray(R.sum(ones))) == float(n)          # exact: all partials are integers
+    v, i = R.maxandargmax(g)
+    assert float(np.asarray(v)) == float(x.max()) and int(np.asarray(i)) == int(x.argmax())
+
+
+def test_config4_maxandargmax_logits(ctx, oracle):
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 2, (65536, 1000)).astype(np.float32)
+    rows = rng.choice(65536, 3277, replace=False)              # 5 % of the rows get duplicated maxima
+    for r in rows:
+        cols = rng.choice(1000, int(rng.integers(1, 4)), replace=False)
+        x[r, cols] = x[r].max()
+    g = gpuarray.array(x, context=ctx)
+    gmax = gpuarray.empty((65536,), "float32", context=ctx)
+    garg = gpuarray.empty((65536,), "uint64", context=ctx)
+    arr = (C.c_uint * 1)(1)
+    assert lib.GpuArray_maxandargmax(gmax._ptr(), garg._ptr(), g._ptr(), 1, arr) == 0
+    got_m, got_a = np.asarray(gmax), np.asarray(garg).astype(np.int64)
+    assert np.array_equal(got_m, x.max(axis=1))
+    assert np.array_equal(got_a, x.argmax(axis=1))             # NumPy: first index on ties
+    wm, wa = oracle.maxandargmax(x[rows[:512]], [1])           # the reference's scan on tied rows
+    assert np.array_equal(got_m[rows[:512]], wm) and np.array_equal(got_a[rows[:512]], wa)
+
+
+def test_config5_mixed_dtypes_strided(ctx, oracle):
+    shape = (256, 512, 1024)
+    rng = np.random.default_rng(5)
+    h = rng.uniform(-4, 4, shape).astype(np.float16)
+    gh = gpuarray.array(h, context=ctx)[:, :, ::2]
+    assert gh.shape == (256, 512, 512) and gh.strides == (1048576, 2048, 4)
+    got = np.asarray(R.sum(gh, axis=(0, 2), dtype="float32"))
+    want = h[:, :, ::2].astype(np.float64).sum(axis=(0, 2))
+    assert got.dtype == np.float32 and np.allclose(got, want, rtol=1e-2)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-2)
+    del gh, h
+
+    rng = np.random.default_rng(6)
+    i32 = rng.integers(-1000, 1001, shape, dtype=np.int32)
+    gi = gpuarray.array(i32, context=ctx)[:, :, ::2]
+    got = np.asarray(R.sum(gi, axis=1))
+    assert got.dtype == np.int64 and np.array_equal(got, i32[:, :, ::2].sum(axis=1))
+    got32 = np.asarray(R.sum(gi, axis=1, dtype="int32"))
+    assert np.array_equal(got32, i32[:, :, ::2].sum(axis=1, dtype=np.int32))
+    chk = oracle.reduk("sum", i32[:4, :, ::2], [1], "int64", ls=64)
+    assert np.array_equal(got[:4], chk)
+    del gi, i32
+
+    rng = np.random.default_rng(7)
+    u8 = (rng.random(shape) < 1e-4).astype(np.uint8)
+    gu = gpuarray.array(u8, context=ctx)[:, :, ::2]
+    any_, all_ = np.asarray(R.any(gu, axis=2)), np.asarray(R.all(gu, axis=2))
+    assert any_.dtype == np.bool_ and np.array_equal(any_, u8[:, :, ::2].any(axis=2))
+    assert np.array_equal(all_, u8[:, :, ::2].all(axis=2)) and not all_.any()
+    assert 0 < any_.sum() < any_.size                          # the test data exercises both answers
+    ones = gpuarray.array(np.ones((8, 16, 64), np.uint8), context=ctx)[:, :, ::2]
+    assert np.asarray(R.all(ones, axis=2)).all()
