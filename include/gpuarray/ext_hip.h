@@ -44,6 +44,8 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
                                            unsigned int n, void *args, int flags,
                                            int strided, unsigned int nd, int idx64,
                                            unsigned int tmask);
+/* vec: elements used per load in bits 0..7, element step of the inner
+ * reduced dim (1, 2 or 4; 0 means 1) in bits 8 and up. */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

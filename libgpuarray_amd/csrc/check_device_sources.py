@@ -63,6 +63,10 @@ def main():
             n += 1
     check("reduction wave-per-row", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4))
     check("reduction bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1))
+    # element step 2 inside a load (a [::2] view): 8 used of 16 fetched bytes
+    check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1))
+    check("reduction stepped halves", gen_r(0, GA_HALF, GA_FLOAT, GA_LONG, 256, 4 | (2 << 8), 1))
+    check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     print("device sources compile for gfx950 (%d reduction variants, 7 elementwise)" % (n + 2))
 
 

@@ -98,6 +98,8 @@ struct _GpuElemwise {
   int kflags = 0;           // GA_USE_* for the compiler
   unsigned int vec = 1;     // elements per chunk in the flat kernel
   unsigned int unroll = 1;  // chunks per lane and tile in the flat kernel
+  bool tile = false;        // a group's chunks are adjacent (tile) or a grid apart
+  bool nontemporal = true;  // streaming hint on the flat kernel's loads and stores
   GpuKernel k_flat = {nullptr, nullptr};
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
@@ -174,7 +176,14 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
        "ga_size ga_done = 0;\n";
   if (V > 1 || U > 1) {
     appendf(s, "if (ga_vec) {\nconst ga_size ga_nchunks = n / %uu;\n", V);
-    appendf(s, "for (ga_size ga_c0 = ga_gtid; ga_c0 < ga_nchunks; ga_c0 += ga_nthr * %uu) {\n", U);
+    if (ge->tile) {
+      appendf(s, "const ga_size ga_ustep = 256;\n"
+                 "for (ga_size ga_c0 = (ga_size)GID_0 * %uu + LID_0; ga_c0 - LID_0 < ga_nchunks; "
+                 "ga_c0 += (ga_size)GDIM_0 * %uu) {\n", 256 * U, 256 * U);
+    } else {
+      s += "const ga_size ga_ustep = ga_nthr;\n";
+      appendf(s, "for (ga_size ga_c0 = ga_gtid; ga_c0 < ga_nchunks; ga_c0 += ga_nthr * %uu) {\n", U);
+    }
     for (const ge_arg &a : ge->args) {
       if (!a.is_array()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
@@ -182,16 +191,20 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
               a.name.c_str(), U);
     }
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
-    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_nthr;\nif (ga_c < ga_nchunks) {\n";
+    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
     for (const ge_arg &a : ge->args) {
       if (!a.is_array() || !a.reads()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
-      appendf(s, "%s_u[ga_u].c = __builtin_nontemporal_load((const %s *)%s_p + ga_c);\n",
-              a.name.c_str(), chunk_type(cb), a.name.c_str());
+      if (ge->nontemporal)
+        appendf(s, "%s_u[ga_u].c = __builtin_nontemporal_load((const %s *)%s_p + ga_c);\n",
+                a.name.c_str(), chunk_type(cb), a.name.c_str());
+      else
+        appendf(s, "%s_u[ga_u].c = ((const %s *)%s_p)[ga_c];\n", a.name.c_str(), chunk_type(cb),
+                a.name.c_str());
     }
     s += "}\n}\n";
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
-    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_nthr;\nif (ga_c < ga_nchunks) {\n";
+    s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
     appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
     appendf(s, "const ga_size i = ga_c * %uu + ga_v; (void)i;\n{\n", V);
     for (const ge_arg &a : ge->args)
@@ -204,8 +217,12 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
     for (const ge_arg &a : ge->args) {
       if (!a.is_array() || !a.writes()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
-      appendf(s, "__builtin_nontemporal_store(%s_u[ga_u].c, (%s *)%s_p + ga_c);\n",
-              a.name.c_str(), chunk_type(cb), a.name.c_str());
+      if (ge->nontemporal)
+        appendf(s, "__builtin_nontemporal_store(%s_u[ga_u].c, (%s *)%s_p + ga_c);\n",
+                a.name.c_str(), chunk_type(cb), a.name.c_str());
+      else
+        appendf(s, "((%s *)%s_p)[ga_c] = %s_u[ga_u].c;\n", chunk_type(cb), a.name.c_str(),
+                a.name.c_str());
     }
     s += "}\n}\n";
     appendf(s, "}\nga_done = ga_nchunks * %uu;\n}\n", V);
@@ -477,10 +494,15 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
 
   // Grid: one lane per chunk (or per element) up to a fixed number of groups
   // per compute unit; beyond that the lanes stride over the range.
-  const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 8);
-  size_t cap = (size_t)ga_hip_numprocs(ge->ctx) * (per_cu ? per_cu : 8);
+  // Measured on MI355X at 2^28 fp32 elements (3 GiB of traffic): one chunk per
+  // lane over the whole range sustains 6.5 TB/s, a grid capped at 8..64 groups
+  // per compute unit that strides over the range 4.2..5.2 TB/s.  So the cap
+  // only matters far beyond that size.
+  const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 2048);
+  size_t cap = (size_t)ga_hip_numprocs(ge->ctx) * (per_cu ? per_cu : 2048);
   size_t units = vec_ok ? n / ge->vec : n;
-  size_t want = (units + GE_LANES - 1) / GE_LANES;
+  size_t per_group = GE_LANES * (size_t)((vec_ok && ge->tile) ? ge->unroll : 1);
+  size_t want = (units + per_group - 1) / per_group;
   size_t gs = want < 1 ? 1 : (want > cap ? cap : want);
   size_t ls = GE_LANES;
   return GpuKernel_call(k, 1, &gs, &ls, 0, nullptr);
@@ -736,9 +758,11 @@ static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, 
   // chunk = 16 bytes of the widest element type; fewer chunks in flight when
   // many arrays are live at once
   ge->vec = maxel >= 16 ? 1 : (unsigned)(16 / maxel);
-  ge->unroll = ge->narray <= 4 ? 4 : (ge->narray <= 8 ? 2 : 1);
+  ge->unroll = ge->narray <= 8 ? 2 : 1;
   ge->unroll = (unsigned)env_ul("GPUARRAY_ELEMWISE_UNROLL", ge->unroll);
   if (ge->unroll < 1) ge->unroll = 1;
+  ge->tile = env_ul("GPUARRAY_ELEMWISE_TILE", 0) != 0;
+  ge->nontemporal = env_ul("GPUARRAY_ELEMWISE_NT", 1) != 0;
   return GA_NO_ERROR;
 }
 

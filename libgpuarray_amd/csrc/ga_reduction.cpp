@@ -119,7 +119,8 @@ std::string neutral_for(rd_kind kind, int acc_tc) {
 }
 
 struct variant {
-  GpuKernel row = {nullptr, nullptr}, col = {nullptr, nullptr}, fin = {nullptr, nullptr};
+  GpuKernel row = {nullptr, nullptr}, col = {nullptr, nullptr}, fin = {nullptr, nullptr},
+            wrows = {nullptr, nullptr};   // wrows only exists in 64-lane variants
 };
 
 struct dimrec {
@@ -154,7 +155,8 @@ namespace {
 
 // The #define block that specialises reduce_kernels.h.
 int gen_defines(const op_info &info, int src_tc, int d0_tc, int d1_tc, unsigned G, unsigned V,
-                unsigned U, std::string &s, ga_errrec *errrec) {
+                unsigned U, std::string &s, ga_errrec *errrec, unsigned opts = 3,
+                unsigned ES = 1) {
   const rd_kind kind = info.kind;
   const bool minmax = kind == K_MIN || kind == K_MAX;
   // min/max compare in the source's type; everything else in the result's
@@ -181,22 +183,24 @@ int gen_defines(const op_info &info, int src_tc, int d0_tc, int d1_tc, unsigned 
   DEF("#define RD_NEUTRAL ((RD_ACC_T)%s)\n",
       neutral_for(kind, kind == K_ALL || kind == K_ANY ? GA_UINT : acc_tc).c_str());
   DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", G, V, U);
+  DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n", opts & 1u,
+      (opts >> 1) & 1u, ES);
 #undef DEF
   return GA_NO_ERROR;
 }
 
 int get_variant(GpuReduction *gr, int d0_tc, int d1_tc, unsigned G, unsigned V, unsigned U,
-                variant **out) {
+                unsigned opts, unsigned ES, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[96];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u", d0_tc, d1_tc, G, V, U);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u", d0_tc, d1_tc, G, V, U, opts, ES);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
     return GA_NO_ERROR;
   }
   std::string s;
-  int herr = gen_defines(gr->info, gr->src_tc, d0_tc, d1_tc, G, V, U, s, ctx->err);
+  int herr = gen_defines(gr->info, gr->src_tc, d0_tc, d1_tc, G, V, U, s, ctx->err, opts, ES);
   if (herr != GA_NO_ERROR) return herr;
   const char *strs[2] = {s.c_str(), ga_reduce_kernels_src};
   size_t lens[2] = {s.size(), strlen(ga_reduce_kernels_src)};
@@ -215,6 +219,13 @@ int get_variant(GpuReduction *gr, int d0_tc, int d1_tc, unsigned G, unsigned V, 
   if ((err = GpuKernel_init(&v.fin, ctx, 2, strs, lens, "redux_final", 9, types, kflags, nullptr)) != GA_NO_ERROR) {
     GpuKernel_clear(&v.row);
     GpuKernel_clear(&v.col);
+    return err;
+  }
+  if (G == 64 &&
+      (err = GpuKernel_init(&v.wrows, ctx, 2, strs, lens, "redux_wrows", 9, types, kflags, nullptr)) != GA_NO_ERROR) {
+    GpuKernel_clear(&v.row);
+    GpuKernel_clear(&v.col);
+    GpuKernel_clear(&v.fin);
     return err;
   }
   *out = &gr->variants.emplace(key, v).first->second;
@@ -249,8 +260,12 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
                                               unsigned int G, unsigned int V, unsigned int U) {
   op_info info;
   if (!op_lookup((ga_reduce_op)op, &info)) return nullptr;
+  // bits 8.. of V carry the element step of strided loads (0 means 1)
+  const unsigned ES = (V >> 8) ? (V >> 8) : 1;
+  V &= 0xffu;
   std::string s;
-  if (gen_defines(info, src_tc, d0_tc, d1_tc, G, V, U, s, ga_global_err) != GA_NO_ERROR) return nullptr;
+  if (gen_defines(info, src_tc, d0_tc, d1_tc, G, V, U, s, ga_global_err, 3, ES) != GA_NO_ERROR)
+    return nullptr;
   s += ga_reduce_kernels_src;
   return strdup(s.c_str());
 }
@@ -285,6 +300,7 @@ void GpuReduction_free(GpuReduction *gr) {
     GpuKernel_clear(&kv.second.row);
     GpuKernel_clear(&kv.second.col);
     GpuKernel_clear(&kv.second.fin);
+    if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
   }
   delete gr;
 }
@@ -418,28 +434,44 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4;
+  unsigned G = 256, V = 1, U = 4, ES = 1;
+  bool wrows = false;
   size_t groups;
   if (use_row) {
-    // widest aligned vector load the layout allows
-    if (p.nr && p.rsstr[p.nr - 1] == elsz && rtotal > 0) {
-      unsigned v = (unsigned)(16 / elsz);
-      const uintptr_t base = (uintptr_t)s0->data->devptr + s0->offset;
-      while (v > 1) {
-        const int64_t bytes = (int64_t)v * elsz;
-        bool ok = rin % v == 0 && base % (uintptr_t)bytes == 0;
-        for (int i = 0; ok && i < p.nf; i++) ok = p.fsstr[i] % bytes == 0;
-        for (int i = 0; ok && i + 1 < p.nr; i++) ok = p.rsstr[i] % bytes == 0;
-        if (ok) break;
-        v /= 2;
+    // Widest aligned load the layout allows.  The inner reduced dim may step
+    // by ES = 1, 2 or 4 elements (a [::2] / [::4] view): a load then fetches
+    // V*ES contiguous elements and uses every ES-th one.  Such a load reads up
+    // to ES-1 elements past the last one used, so it must stay inside the
+    // buffer.
+    if (p.nr && rtotal > 0 && p.rsstr[p.nr - 1] > 0 && p.rsstr[p.nr - 1] % elsz == 0) {
+      const int64_t es = p.rsstr[p.nr - 1] / elsz;
+      if (es == 1 || es == 2 || es == 4) {
+        unsigned v = (unsigned)(16 / (elsz * es));
+        const uintptr_t base = (uintptr_t)s0->data->devptr + s0->offset;
+        size_t bufsz = 0;
+        gpudata_property(s0->data, GA_BUFFER_PROP_SIZE, &bufsz);
+        int64_t last = (int64_t)s0->offset;   // byte offset of the farthest element
+        for (int i = 0; i < p.nf; i++) if (p.fsstr[i] > 0) last += (p.fdim[i] - 1) * p.fsstr[i];
+        for (int i = 0; i < p.nr; i++) if (p.rsstr[i] > 0) last += (p.rdim[i] - 1) * p.rsstr[i];
+        const bool overread_ok = es == 1 || (size_t)(last + es * elsz) <= bufsz;
+        while (v > 1) {
+          const int64_t bytes = (int64_t)v * es * elsz;
+          bool ok = overread_ok && rin % v == 0 && base % (uintptr_t)bytes == 0;
+          for (int i = 0; ok && i < p.nf; i++) ok = p.fsstr[i] % bytes == 0;
+          for (int i = 0; ok && i + 1 < p.nr; i++) ok = p.rsstr[i] % bytes == 0;
+          if (ok) break;
+          v /= 2;
+        }
+        V = v;
+        if (V > 1) ES = (unsigned)es;
       }
-      V = v;
     }
     // one wavefront per output while rows are short and plentiful
     if (rtotal <= 8192 && nrows >= 2 * ncu) G = 64;
     G = (unsigned)env_ul("GPUARRAY_REDUX_G", G) == 64 ? 64 : 256;
     int64_t per_pass = (int64_t)G * V;
-    U = 4;
+    U = (unsigned)env_ul("GPUARRAY_REDUX_U", 8);
+    if (U != 1 && U != 2 && U != 4 && U != 8) U = 8;
     while (U > 1 && per_pass * (U / 2) >= rin) U /= 2;
     const int64_t seg = per_pass * U;
     p.nseg = rin > 0 ? (rin + seg - 1) / seg : 1;
@@ -451,17 +483,42 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     const int64_t rowgroups = (nrows + rows_per_group - 1) / rows_per_group;
     // too few groups to fill the chip: cut the rows
     int64_t nsplit = 1;
-    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 8);
+    // How many groups a compute unit needs depends on how many bytes each one
+    // keeps in flight.  Measured on MI355X (full fp32 sum of 2^28 elements):
+    // 2 groups of 256 lanes per unit, each lane with eight 16-byte streaming
+    // loads outstanding (64 KB per unit), read at 6.9-7.1 TB/s; 16 such
+    // groups per unit at 6.3, 64 at 5.8.  Narrow or strided loads carry fewer
+    // bytes per lane, so they get proportionally more groups, up to 32.
+    int64_t per_cu = (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 0);
+    if (per_cu == 0) {
+      const int64_t inflight = (int64_t)G * U * V * ES * elsz;   // bytes per group
+      per_cu = (65536 + inflight - 1) / inflight;
+      if (per_cu < 2) per_cu = 2;
+      if (per_cu > 32) per_cu = 32;
+    }
+    const int64_t target = ncu * per_cu;
     if (rowgroups < target && p.units >= 8) {
       nsplit = (target + rowgroups - 1) / rowgroups;
       if (nsplit > p.units / 4) nsplit = p.units / 4;
-      if (nsplit > 4096) nsplit = 4096;
+      if (nsplit > 65536) nsplit = 65536;
       if (nsplit < 1) nsplit = 1;
     }
     p.upb = p.units > 0 ? (p.units + nsplit - 1) / nsplit : 0;
     if (p.upb > 0) nsplit = (p.units + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;
     groups = (size_t)(rowgroups * nsplit);
+    // short rows, one wavefront each: let a wavefront walk several rows with
+    // the next row's loads in flight (about 8 wavefronts per SIMD in all)
+    if (G == 64 && nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
+      wrows = true;
+      int64_t rpw = (nrows + ncu * 32 - 1) / (ncu * 32);
+      rpw = rpw < 1 ? 1 : (rpw > 16 ? 16 : rpw);
+      rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", (unsigned long)rpw);
+      if (rpw < 1) rpw = 1;
+      p.upb = rpw;
+      const int64_t waves = (nrows + rpw - 1) / rpw;
+      groups = (size_t)((waves + 3) / 4);
+    }
   } else {
     const int64_t fin = p.fdim[p.nf - 1];
     p.gx = (fin + 63) / 64;
@@ -484,8 +541,12 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
   if (groups == 0 || groups > 0x7fffffffull)
     return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Reduction needs more groups than one launch has");
 
+  // bit 0: streaming loads; bit 1: interleaved splits (single reduced dim only)
+  unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
+  if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
   variant *var = nullptr;
-  int err = get_variant(gr, d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, &var);
+  int err = get_variant(gr, d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts,
+                        use_row ? ES : 1, &var);
   if (err != GA_NO_ERROR) return err;
 
   // partials of a split reduction live in the context's scratch buffer:
@@ -511,7 +572,7 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
   struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + pi_off, ctx};
   void *args[9] = {s0->data, &s_off, d0b, &d0_off, d1b, &d1_off, scratch, &pi_view, &p};
   size_t ls = 256;
-  GpuKernel *k1 = use_row ? &var->row : &var->col;
+  GpuKernel *k1 = use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
   if ((err = GpuKernel_call(k1, 1, &groups, &ls, 0, args)) != GA_NO_ERROR) return err;
   if (p.nsplit > 1) {
     size_t fg = (size_t)((nrows + 3) / 4);

@@ -13,7 +13,14 @@
  *   RD_G        lanes that share one output in redux_row: 64 or 256
  *   RD_VEC      elements per load in redux_row (inner reduced stride is the
  *               element size and everything is aligned when > 1)
+ *   RD_ES       element step of the inner reduced dim inside a load: the dim
+ *               advances by RD_ES elements per index (a [::2] or [::4] view), a
+ *               load fetches RD_VEC*RD_ES contiguous elements and every
+ *               RD_ES-th one is used
  *   RD_U        loads in flight per lane
+ *   RD_NT       streaming (non-temporal) loads in redux_row
+ *   RD_INTERLEAVE  redux_row with one reduced dim: splits take every
+ *               nsplit-th unit instead of a contiguous range
  *
  * Semantics (reference src/gpuarray_reduction.c:545-607 for max/argmax,
  * pygpu/reduction.py:33-134 for sum/prod/any/all):
@@ -32,10 +39,13 @@
  *     inside a unit, then the cross-lane network below), so results are
  *     reproducible run to run.
  *
- * Three kernels:
+ * Four kernels:
  *   redux_row    lanes run along the fastest REDUCED dim; RD_G lanes
  *                cooperate on one output; a row can be cut in `nsplit` pieces
  *                that each leave a partial.
+ *   redux_wrows  the same for short rows (one pass of a wavefront covers a
+ *                row): a wavefront walks several rows and has the next row's
+ *                loads in flight while it combines the current one.
  *   redux_col    lanes run along the fastest FREE dim (coalesced), each lane
  *                owns one output and walks the reduced range; 4 lane rows
  *                share the range and meet in LDS.
@@ -289,13 +299,89 @@ static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *
 
 /* ---- redux_row ------------------------------------------------------------- */
 
-#if RD_VEC > 1
-typedef RD_SRC_T rd_vec_t __attribute__((ext_vector_type(RD_VEC)));
+#define RD_PV (RD_VEC * RD_ES)   /* elements fetched per load */
+typedef RD_SRC_T rd_pvec_t __attribute__((ext_vector_type(RD_PV)));
+/* every source element is read once: stream it past the caches */
+#if RD_NT
+#define RD_LOAD(p) __builtin_nontemporal_load(p)
+#else
+#define RD_LOAD(p) (*(p))
 #endif
 
+/* One "unit" = RD_U loads per lane over RD_G lanes: elements
+ * e0 + j*RD_G*RD_VEC + v of the inner reduced dim, j < RD_U, v < RD_VEC, where
+ * e0 = (first element of the unit) + lane*RD_VEC. */
+static __device__ inline void rd_unit_load(rd_pvec_t *x, const char *base, ga_long e0, ga_long rin,
+                                           ga_long rstr) {
+#pragma unroll
+  for (int j = 0; j < RD_U; j++) {
+    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
+    if (e < rin) x[j] = RD_LOAD((const rd_pvec_t *)(base + e * rstr));
+  }
+}
+
+/* Combination of the lane's elements of one unit.  ib, rml: index of element
+ * 0 of the inner dim and index step per element. */
+static __device__ inline rd_acc rd_unit_combine(const rd_pvec_t *x, ga_long e0, ga_long rin,
+                                                ga_long ib, ga_long rml) {
+#if RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN
+  /* The lane's elements are visited in rising index order, so a strict
+   * compare keeps the first of equals by itself; only the position inside
+   * the unit (a small int) is tracked. */
+  rd_acc r = rd_neutral();
+  if (e0 < rin) {
+    RD_ACC_T bv = rd_elem(x[0][0], 0).v;
+    ga_int bp = 0;
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      if (e0 + (ga_long)j * RD_G * RD_VEC < rin) {
+#pragma unroll
+        for (int v = 0; v < RD_VEC; v++) {
+          if (j == 0 && v == 0) continue;
+          const RD_ACC_T val = rd_elem(x[j][v * RD_ES], 0).v;
+#if RD_KIND == RD_K_MAX
+          const bool better = val > bv;
+#else
+          const bool better = val < bv;
+#endif
+          bv = better ? val : bv;
+          bp = better ? (j * RD_G * RD_VEC + v) : bp;
+        }
+      }
+    }
+    r.v = bv;
+#if RD_ARG
+    r.i = ib + (e0 + bp) * rml;
+#else
+    (void)bp; (void)ib; (void)rml;
+#endif
+  }
+  return r;
+#else
+  rd_acc t[RD_U];
+#pragma unroll
+  for (int j = 0; j < RD_U; j++) {
+    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
+    t[j] = rd_neutral();
+    if (e < rin) {
+#pragma unroll
+      for (int v = 0; v < RD_VEC; v++)
+        t[j] = rd_combine(t[j], rd_elem(x[j][v * RD_ES], ib + (e + v) * rml));
+    }
+  }
+  /* pairwise over the unit */
+#pragma unroll
+  for (int w = 1; w < RD_U; w *= 2)
+#pragma unroll
+    for (int j = 0; j + w < RD_U; j += 2 * w) t[j] = rd_combine(t[j], t[j + w]);
+  return t[0];
+#endif
+}
+
 KERNEL void __launch_bounds__(256)
-redux_row(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
-          const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict__ d0,
+          const ga_size d0_off, char *__restrict__ d1, const ga_size d1_off,
+          RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, const rd_plan p) {
   const unsigned rows_per_group = 256u / RD_G;
   const unsigned lane = LID_0 % RD_G;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
@@ -315,8 +401,17 @@ redux_row(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
   const ga_long rml = p.nr > 0 ? p.rmul[ri] : 0;
   const ga_long seg = (ga_long)RD_G * RD_VEC * RD_U;
 
+  /* A split owns a contiguous range of units, or - for a single reduced dim
+   * (RD_INTERLEAVE) - every nsplit-th unit, so that at any moment the splits
+   * of a row read one moving window of memory. */
+#if RD_INTERLEAVE
+  ga_long u0 = split, u1 = p.units;
+  const ga_long ustep = p.nsplit;
+#else
   ga_long u0 = split * p.upb, u1 = u0 + p.upb;
   if (u1 > p.units) u1 = p.units;
+  const ga_long ustep = 1;
+#endif
 
   /* unit -> (outer reduced coordinate ro, segment k of the inner dim): one
    * division for the first unit, then counted up */
@@ -326,51 +421,20 @@ redux_row(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
   rd_outer_offsets(p, ri, ro, &rb, &ib);
 
   rd_acc acc = rd_neutral();
-  for (ga_long u = u0; u < u1; u++) {
+  for (ga_long u = u0; u < u1; u += ustep) {
     const ga_long e0 = k * seg + (ga_long)lane * RD_VEC;
-#if RD_VEC > 1
-    rd_vec_t x[RD_U];
-#pragma unroll
-    for (int j = 0; j < RD_U; j++) {
-      const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
-      if (e < rin) x[j] = *(const rd_vec_t *)(srow + rb + e * rstr);
-    }
-    rd_acc t[RD_U];
-#pragma unroll
-    for (int j = 0; j < RD_U; j++) {
-      const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
-      t[j] = rd_neutral();
-      if (e < rin) {
-#pragma unroll
-        for (int v = 0; v < RD_VEC; v++)
-          t[j] = rd_combine(t[j], rd_elem(x[j][v], ib + (e + v) * rml));
-      }
-    }
+    rd_pvec_t x[RD_U];
+    rd_unit_load(x, srow + rb, e0, rin, rstr);
+    acc = rd_combine(acc, rd_unit_combine(x, e0, rin, ib, rml));
+#if RD_INTERLEAVE
+    k += ustep;   /* single reduced dim: the unit is the segment */
 #else
-    RD_SRC_T x[RD_U];
-#pragma unroll
-    for (int j = 0; j < RD_U; j++) {
-      const ga_long e = e0 + (ga_long)j * RD_G;
-      if (e < rin) x[j] = *(const RD_SRC_T *)(srow + rb + e * rstr);
-    }
-    rd_acc t[RD_U];
-#pragma unroll
-    for (int j = 0; j < RD_U; j++) {
-      const ga_long e = e0 + (ga_long)j * RD_G;
-      t[j] = (e < rin) ? rd_elem(x[j], ib + e * rml) : rd_neutral();
-    }
-#endif
-    /* pairwise over the unit, then onto the running value */
-#pragma unroll
-    for (int w = 1; w < RD_U; w *= 2)
-#pragma unroll
-      for (int j = 0; j + w < RD_U; j += 2 * w) t[j] = rd_combine(t[j], t[j + w]);
-    acc = rd_combine(acc, t[0]);
     if (++k == p.nseg) {
       k = 0;
       ro++;
       rd_outer_offsets(p, ri, ro, &rb, &ib);
     }
+#endif
   }
 
 #if RD_G == 256
@@ -383,6 +447,49 @@ redux_row(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
     else rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
   }
 }
+
+/* ---- redux_wrows -----------------------------------------------------------
+ * Rows that one pass of a wavefront covers (at most one reduced dim, one
+ * unit per row, no split).  Wavefront w owns rows [w*upb, (w+1)*upb); the
+ * loads of row r+1 are issued before row r is combined, so memory latency
+ * overlaps the cross-lane work.  Only built for RD_G == 64. */
+#if RD_G == 64
+KERNEL void __launch_bounds__(256)
+redux_wrows(const char *__restrict__ src, const ga_size src_off, char *__restrict__ d0,
+            const ga_size d0_off, char *__restrict__ d1, const ga_size d1_off,
+            RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, const rd_plan p) {
+  (void)part_v; (void)part_i;
+  const unsigned lane = LID_0 & 63u;
+  const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
+  ga_long row = wave * p.upb;
+  ga_long row_end = row + p.upb;
+  if (row_end > p.nrows) row_end = p.nrows;
+  if (row >= row_end) return;
+
+  const ga_long rin = p.nr > 0 ? p.rdim[0] : 1;
+  const ga_long rstr = p.nr > 0 ? p.rsstr[0] : 0;
+  const ga_long rml = p.nr > 0 ? p.rmul[0] : 0;
+  const ga_long e0 = (ga_long)lane * RD_VEC;
+
+  ga_long so, d0o, d1o;
+  rd_row_offsets(p, row, &so, &d0o, &d1o);
+  rd_pvec_t cur[RD_U];
+  rd_unit_load(cur, src + src_off + so, e0, rin, rstr);
+  for (; row < row_end; row++) {
+    ga_long nso = 0, nd0o = 0, nd1o = 0;
+    rd_pvec_t nxt[RD_U];
+    if (row + 1 < row_end) {
+      rd_row_offsets(p, row + 1, &nso, &nd0o, &nd1o);
+      rd_unit_load(nxt, src + src_off + nso, e0, rin, rstr);
+    }
+    rd_acc acc = rd_wave_reduce(rd_unit_combine(cur, e0, rin, 0, rml));
+    if (lane == 0) rd_store(acc, src + src_off + so, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) cur[j] = nxt[j];
+    so = nso; d0o = nd0o; d1o = nd1o;
+  }
+}
+#endif
 
 /* ---- redux_col ------------------------------------------------------------- */
 
@@ -436,7 +543,7 @@ redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
             off += c * p.rsstr[d];
             ix += c * p.rmul[d];
           }
-          x[q] = *(const RD_SRC_T *)(srow + off);
+          x[q] = RD_LOAD((const RD_SRC_T *)(srow + off));
           idx[q] = ix;
         }
       }
