@@ -30,6 +30,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
+# HBM bytes per launch of the flat elementwise kernel at 2^28 elements, from
+# two counter runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known
+# size; the runs and the arithmetic are in
+# profiles/elem_flat_fp32_2p28_hbm_traffic.md.  Counters cannot be read from
+# inside this process, so the figure is carried here for the shape it was
+# measured on.
+MEASURED_TRAFFIC = {28: 3219778560}
 
 
 def main():
@@ -39,6 +46,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip the per-config table")
     ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count")
+    ap.add_argument("--only", choices=["step", "elem", "sum", "copy"], default="step",
+                    help="launch only one kernel per step (for profiler runs): the elementwise "
+                         "kernel, the sum, or a plain copy dst = src of the same size whose "
+                         "traffic is known (4*n read + 4*n written) to scale byte counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -64,13 +75,21 @@ def main():
                            ga.arg("c", "float32", write=True)])
     summ = ga.GpuReduction(ctx, "sum", "float32")
 
+    copy = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", "float32", read=True),
+                                             ga.arg("dst", "float32", write=True)])
+    only = args.only
+
     def step(i=None):
         if i is not None:
             ctx.mark(3 * i)
-        elem(a, b, c)
+        if only in ("step", "elem"):
+            elem(a, b, c)
+        elif only == "copy":
+            copy(a, c)
         if i is not None:
             ctx.mark(3 * i + 1)
-        summ(x, [0], d0=s)
+        if only in ("step", "sum"):
+            summ(x, [0], d0=s)
         if i is not None:
             ctx.mark(3 * i + 2)
 
@@ -91,6 +110,15 @@ def main():
     step_bytes = elem_bytes + sum_bytes
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    if only != "step":
+        # profiler run: report the one kernel that was launched and stop
+        ms = elem_ms if only in ("elem", "copy") else sum_ms
+        nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
+        print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
+                          "bytes_per_launch": nbytes,
+                          "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1)}))
+        return
+
     # parity spot-check of what was just timed
     got = np.asarray(c[:4096])
     assert np.array_equal(got, a_h[:4096] * b_h[:4096] + np.float32(0.5)), "elementwise result wrong"
@@ -101,7 +129,8 @@ def main():
     achieved = elem_bytes / (elem_avg * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "elem (flat GpuElemwise kernel, c = a*b + 0.5f)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC.get(args.log2n),
                 "avg_launch_us": round(elem_avg * 1e3, 2),
                 "median_launch_us": round(float(np.median(elem_ms)) * 1e3, 2),
                 "algorithmic_bytes_per_launch": elem_bytes}
