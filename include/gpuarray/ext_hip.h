@@ -40,6 +40,9 @@ typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsign
 /* "hip_elemwise_source" / "hip_reduction_source": the kernel text the
  * generators would compile for a given variant, as a malloc'd string the
  * caller frees.  For host-side checks of the generated code. */
+/* strided: 0 flat kernel, 1 strided kernel with one element per lane,
+ * 2 strided kernel with four elements per lane (tmask bits 0..15: arrays
+ * staged through LDS; bits 16..: arrays with unit stride along x). */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
                                            unsigned int n, void *args, int flags,
                                            int strided, unsigned int nd, int idx64,

@@ -49,6 +49,9 @@ def main():
     for nd, idx64, tmask in [(1, 0, 0), (2, 0, 0), (3, 1, 0), (2, 0, 1), (3, 1, 3)]:
         check("elemwise strided nd=%d idx64=%d tmask=%x" % (nd, idx64, tmask),
               gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 1, nd, idx64, tmask))
+    # four elements per lane: plain (umask in bits 16..) and transposed
+    check("elemwise strided vec4 plain", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 2, 2, 0, 0b101 << 16))
+    check("elemwise strided vec4 transposed", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 2, 3, 1, 0b001 | (0b110 << 16)))
     hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
     check("elemwise half->double copy", gen_e(b"", b"dst = src", 2, hargs, 2, 0, 0, 0, 0))
     n = 0
@@ -67,7 +70,7 @@ def main():
     check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1))
     check("reduction stepped halves", gen_r(0, GA_HALF, GA_FLOAT, GA_LONG, 256, 4 | (2 << 8), 1))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
-    print("device sources compile for gfx950 (%d reduction variants, 7 elementwise)" % (n + 2))
+    print("device sources compile for gfx950 (%d reduction variants, 9 elementwise)" % (n + 5))
 
 
 if __name__ == "__main__":

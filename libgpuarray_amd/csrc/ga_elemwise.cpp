@@ -83,6 +83,7 @@ const char *chunk_type(size_t bytes) {
   case 2: return "ga_ushort";
   case 4: return "ga_uint";
   case 8: return "ga_chunk8";
+  case 32: return "ga_chunk32";
   default: return "ga_chunk16";
   }
 }
@@ -135,7 +136,8 @@ void emit_store(const GpuElemwise *ge, std::string &s, const ge_arg &a, const st
 void emit_header(const GpuElemwise *ge, std::string &s) {
   s += "#include \"cluda.h\"\n";
   s += "typedef ga_uint __attribute__((ext_vector_type(2))) ga_chunk8;\n"
-       "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n";
+       "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n"
+       "typedef ga_uint __attribute__((ext_vector_type(8))) ga_chunk32;\n";
   s += ge->preamble;
   s += "\n";
 }
@@ -435,6 +437,306 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
   return s;
 }
 
+
+// ---- strided kernel, four elements per lane -------------------------------------
+// Same arguments as the scalar strided kernel.  Preconditions checked by the
+// caller: the x extent (and the y extent when operands are transposed) is a
+// multiple of 4, element sizes are at most 8 bytes, and every array marked in
+// `umask` (unit stride along x) or `tmask` (unit stride along y) has its base
+// and all its other strides aligned to 4 elements, so that a lane can move 4
+// consecutive elements with one access.  Arrays in neither mask (broadcast or
+// oddly strided along x) are accessed element by element.
+//
+// Plain variant: a lane owns one row and 4 quads TX quads apart; all loads
+// of the 16 elements are issued before the first use.
+// Transposed variant: 64 x 64 tile.  Transposed reads: a lane loads 4
+// consecutive y of one x column and scatters them into the padded tile;
+// the expression runs on 4 consecutive x of one y row; transposed writes
+// gather 4 consecutive y from the tile and store them with one access.
+std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
+                            unsigned umask, std::vector<int> &ktypes) {
+  std::string s;
+  const char *I = idx64 ? "ga_ssize" : "ga_int";
+  const char *N = idx64 ? "ga_size" : "ga_uint";
+  emit_header(ge, s);
+  s += "KERNEL void __launch_bounds__(256) elem(";
+  for (unsigned d = 0; d < nd; d++) {
+    appendf(s, "%sconst ga_size dim%u", d ? ", " : "", d);
+    ktypes.push_back(GA_SIZE);
+  }
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset", ctype(a.typecode),
+              a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+      for (unsigned d = 0; d < nd; d++) {
+        appendf(s, ", const ga_ssize %s_str_%u", a.name.c_str(), d);
+        ktypes.push_back(GA_SSIZE);
+      }
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n";
+  ktypes.push_back(GA_UINT);
+  ktypes.push_back(GA_UINT);
+
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto is_t = [&](size_t j) { return aidx[j] >= 0 && ((tmask >> aidx[j]) & 1u); };
+  auto is_u = [&](size_t j) { return aidx[j] >= 0 && ((umask >> aidx[j]) & 1u); };
+  auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * 4); };
+
+  for (const ge_arg &a : ge->args)
+    if (a.is_array())
+      appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n",
+              a.name.c_str(), a.name.c_str(), a.name.c_str());
+  const unsigned xd = nd - 1;
+
+  // element (q, i) of array a, given the row offset expression `rowoff`
+  auto elem_at = [&](const ge_arg &a, const std::string &rowoff, const std::string &x) {
+    std::string at;
+    appendf(at, "*(GLOBAL_MEM %s *)(%s_b + (%s + (%s)(%s) * (%s)%s_str_%u))", ctype(a.typecode),
+            a.name.c_str(), rowoff.c_str(), I, x.c_str(), I, a.name.c_str(), xd);
+    return at;
+  };
+  auto quad_at = [&](const ge_arg &a, const std::string &rowoff, const std::string &x) {
+    std::string at;
+    appendf(at, "*(GLOBAL_MEM %s *)(%s_b + (%s + (%s)(%s) * (%s)%s_str_%u))", quad_t(a),
+            a.name.c_str(), rowoff.c_str(), I, x.c_str(), I, a.name.c_str(), xd);
+    return at;
+  };
+
+  if (tmask == 0) {
+    appendf(s, "const %s ga_tx = LID_0 & ((1u << ga_ltx) - 1u);\n", N);
+    appendf(s, "const %s ga_ty = LID_0 >> ga_ltx;\n", N);
+    appendf(s, "const %s ga_bx = GID_0 %% ga_gx;\nconst %s ga_by = GID_0 / ga_gx;\n", N, N);
+    appendf(s, "%s ga_rows = 1;\n", N);
+    for (unsigned d = 0; d + 1 < nd; d++) appendf(s, "ga_rows *= (%s)dim%u;\n", N, d);
+    appendf(s, "const %s ga_row = ga_by * (256u >> ga_ltx) + ga_ty;\n", N);
+    s += "if (ga_row >= ga_rows) return;\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
+    if (nd >= 2) {
+      appendf(s, "{ %s ga_r = ga_row; %s ga_c;\n", N, N);
+      for (unsigned d = nd - 1; d-- > 0;) {
+        if (d > 0) appendf(s, "ga_c = ga_r %% (%s)dim%u; ga_r = ga_r / (%s)dim%u;\n", N, d, N, d);
+        else s += "ga_c = ga_r;\n";
+        for (const ge_arg &a : ge->args)
+          if (a.is_array())
+            appendf(s, "%s_o += (%s)ga_c * (%s)%s_str_%u;\n", a.name.c_str(), I, I,
+                    a.name.c_str(), d);
+      }
+      s += "}\n";
+    }
+    // quad index q = (bx*4 + e) * TX + tx, x = 4q
+    appendf(s, "const %s ga_q0 = (ga_bx * 4u << ga_ltx) + ga_tx;\n", N);
+    appendf(s, "const %s ga_nq = (%s)dim%u / 4u;\n", N, N, xd);
+    for (const ge_arg &a : ge->args)
+      if (a.is_array())
+        appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode),
+                a.name.c_str());
+    s += "#pragma unroll\nfor (int ga_e = 0; ga_e < 4; ga_e++) {\n";
+    appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
+    appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!a.is_array() || !a.reads()) continue;
+      if (is_u(j)) {
+        appendf(s, "%s_u[ga_e].c = %s;\n", a.name.c_str(), quad_at(a, a.name + "_o", "ga_x").c_str());
+      } else {
+        for (int i = 0; i < 4; i++) {
+          char xi[32];
+          snprintf(xi, sizeof(xi), "ga_x + %du", i);
+          appendf(s, "%s_u[ga_e].e[%d] = %s;\n", a.name.c_str(), i,
+                  elem_at(a, a.name + "_o", xi).c_str());
+        }
+      }
+    }
+    s += "}\n}\n";
+    s += "#pragma unroll\nfor (int ga_e = 0; ga_e < 4; ga_e++) {\n";
+    appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
+    appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
+    s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_load(ge, s, a, a.name + "_u[ga_e].e[ga_v]");
+    s += ge->expr;
+    s += ";\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_store(ge, s, a, a.name + "_u[ga_e].e[ga_v]");
+    s += "}\n";
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!a.is_array() || !a.writes()) continue;
+      if (is_u(j)) {
+        appendf(s, "%s = %s_u[ga_e].c;\n", quad_at(a, a.name + "_o", "ga_x").c_str(), a.name.c_str());
+      } else {
+        for (int i = 0; i < 4; i++) {
+          char xi[32];
+          snprintf(xi, sizeof(xi), "ga_x + %du", i);
+          appendf(s, "%s = %s_u[ga_e].e[%d];\n", elem_at(a, a.name + "_o", xi).c_str(),
+                  a.name.c_str(), i);
+        }
+      }
+    }
+    s += "}\n}\n}\n";
+    return s;
+  }
+
+  // ---- transposed, nd >= 2 ----
+  const unsigned yd = nd - 2;
+  for (size_t j = 0; j < ge->args.size(); j++)
+    if (is_t(j))
+      appendf(s, "LOCAL_MEM %s %s_t[64 * 65];\n", ctype(ge->args[j].typecode),
+              ge->args[j].name.c_str());
+  appendf(s, "const %s ga_lo = LID_0 & 15u;\nconst %s ga_hi = LID_0 >> 4;\n", N, N);
+  appendf(s, "const %s ga_gy = ((%s)dim%u + 63u) / 64u;\n", N, N, yd);
+  appendf(s, "const %s ga_bx = GID_0 %% ga_gx;\n", N);
+  appendf(s, "%s ga_r = GID_0 / ga_gx;\n", N);
+  appendf(s, "const %s ga_by = ga_r %% ga_gy;\nga_r = ga_r / ga_gy;\n", N);
+  for (const ge_arg &a : ge->args)
+    if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
+  if (nd >= 3) {
+    appendf(s, "{ %s ga_c;\n", N);
+    for (unsigned d = nd - 2; d-- > 0;) {
+      if (d > 0) appendf(s, "ga_c = ga_r %% (%s)dim%u; ga_r = ga_r / (%s)dim%u;\n", N, d, N, d);
+      else s += "ga_c = ga_r;\n";
+      for (const ge_arg &a : ge->args)
+        if (a.is_array())
+          appendf(s, "%s_o += (%s)ga_c * (%s)%s_str_%u;\n", a.name.c_str(), I, I, a.name.c_str(), d);
+    }
+    s += "}\n";
+  }
+  appendf(s, "const %s ga_x0 = ga_bx * 64u;\nconst %s ga_y0 = ga_by * 64u;\n", N, N);
+  // byte offset of (y, x) for array a
+  auto off_yx = [&](const ge_arg &a, const char *y, const char *x) {
+    std::string o;
+    appendf(o, "(%s_o + (%s)(%s) * (%s)%s_str_%u + (%s)(%s) * (%s)%s_str_%u)", a.name.c_str(), I,
+            y, I, a.name.c_str(), yd, I, x, I, a.name.c_str(), xd);
+    return o;
+  };
+  bool any_tr = false, any_tw = false;
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    if (!is_t(j)) continue;
+    if (ge->args[j].reads()) any_tr = true;
+    if (ge->args[j].writes()) any_tw = true;
+  }
+  // phase 1: transposed reads.  lane: y quad ga_lo (y = 4*ga_lo..+3), x column ga_hi + 16k
+  if (any_tr) {
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (is_t(j) && a.reads())
+        appendf(s, "union { %s c; %s e[4]; } %s_in[4];\n", quad_t(a), ctype(a.typecode),
+                a.name.c_str());
+    }
+    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.reads()) continue;
+      appendf(s, "%s_in[ga_k].c = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), quad_t(a),
+              a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+    }
+    s += "}\n}\n";
+    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.reads()) continue;
+      appendf(s, "#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
+                 "%s_t[(ga_ly + ga_i) * 65u + ga_lx] = %s_in[ga_k].e[ga_i];\n",
+              a.name.c_str(), a.name.c_str());
+    }
+    s += "}\n}\nlocal_barrier();\n";
+  }
+  // phase 2: the expression.  lane: x quad ga_lo (x = 4*ga_lo..+3), y row ga_hi + 16k
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (a.is_array() && !is_t(j))
+      appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), a.name.c_str());
+  }
+  s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + 16u * (%s)ga_k;\n", N, N);
+  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array() || is_t(j) || !a.reads()) continue;
+    if (is_u(j)) {
+      appendf(s, "%s_u[ga_k].c = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), quad_t(a),
+              a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+    } else {
+      for (int i = 0; i < 4; i++) {
+        char xi[48];
+        snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
+        appendf(s, "%s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), i,
+                ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
+      }
+    }
+  }
+  s += "}\n}\n";
+  s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + 16u * (%s)ga_k;\n", N, N);
+  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+  s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * 65u + ga_lx + ga_v]");
+    else emit_load(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
+  }
+  s += ge->expr;
+  s += ";\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * 65u + ga_lx + ga_v]");
+    else emit_store(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
+  }
+  s += "}\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array() || is_t(j) || !a.writes()) continue;
+    if (is_u(j)) {
+      appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].c;\n", quad_t(a), a.name.c_str(),
+              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str(), a.name.c_str());
+    } else {
+      for (int i = 0; i < 4; i++) {
+        char xi[48];
+        snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
+        appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].e[%d];\n", ctype(a.typecode),
+                a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str(), a.name.c_str(), i);
+      }
+    }
+  }
+  s += "}\n}\n";
+  // phase 3: transposed writes, mirror of phase 1
+  if (any_tw) {
+    s += "local_barrier();\n#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.writes()) continue;
+      appendf(s, "{ union { %s c; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
+                 "ga_o.e[ga_i] = %s_t[(ga_ly + ga_i) * 65u + ga_lx];\n",
+              quad_t(a), ctype(a.typecode), a.name.c_str());
+      appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = ga_o.c; }\n", quad_t(a), a.name.c_str(),
+              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+    }
+    s += "}\n}\n";
+  }
+  s += "}\n";
+  return s;
+}
+
 int build_kernel(GpuElemwise *ge, GpuKernel *k, const std::string &src,
                  const std::vector<int> &ktypes) {
   const char *strs[1] = {src.c_str()};
@@ -672,15 +974,41 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     if (reach >= (size_t)GA_SADDR32_MAX) idx64 = true;
   }
 
+  // Four elements per lane when the layout allows it (see gen_strided_vec).
+  bool vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % 4 == 0 &&
+              dims[nd - 1] >= 16 && strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
+  unsigned umask = 0;
+  if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
+  for (unsigned k = 0; k < na && vec4; k++) {
+    if (elsz[k] > 8) { vec4 = false; break; }
+    const size_t q = 4 * elsz[k];
+    unsigned l2 = 0;
+    const GpuArray *v = nullptr;
+    for (size_t i = 0; i < ge->args.size(); i++)
+      if (ge->args[i].is_array() && l2++ == k) { v = (const GpuArray *)args[i]; break; }
+    const bool base_ok = ((uintptr_t)v->data->devptr + v->offset) % q == 0;
+    const bool tr = (tmask >> k) & 1u;
+    const unsigned unit_dim = tr ? nd - 2 : nd - 1;
+    bool aligned = base_ok && strs[k][unit_dim] == (ssize_t)elsz[k];
+    for (unsigned j = 0; j < nd && aligned; j++)
+      if (j != unit_dim && strs[k][j] % (ssize_t)q != 0) aligned = false;
+    if (tr) {
+      if (!aligned) vec4 = false;          // a transposed operand must be vector-accessible
+    } else if (aligned) {
+      umask |= 1u << k;
+    }
+  }
+  if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
+
   // launch geometry
   size_t gx, groups;
   unsigned ltx = 0;
   if (tmask == 0) {
-    size_t inner = dims[nd - 1];
-    ltx = 4;
+    size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
+    ltx = vec4 ? 0 : 4;
     while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
     size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
-    size_t rows = n / inner;
+    size_t rows = n / dims[nd - 1];
     gx = (inner + 4 * tx - 1) / (4 * tx);
     groups = gx * ((rows + ty - 1) / ty);
   } else {
@@ -694,14 +1022,16 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
 
   char key[64];
-  snprintf(key, sizeof(key), "%u:%d:%x", nd, idx64 ? 1 : 0, tmask);
+  snprintf(key, sizeof(key), "%s%u:%d:%x:%x", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+           vec4 ? umask : 0u);
   GpuKernel *k;
   auto it = ge->k_strided.find(key);
   if (it != ge->k_strided.end()) {
     k = &it->second;
   } else {
     std::vector<int> ktypes;
-    std::string src = gen_strided(ge, nd, idx64, tmask, ktypes);
+    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes)
+                           : gen_strided(ge, nd, idx64, tmask, ktypes);
     GpuKernel nk = {nullptr, nullptr};
     int err = build_kernel(ge, &nk, src, ktypes);
     if (err != GA_NO_ERROR) return err;
@@ -779,7 +1109,11 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   if (expr == nullptr || ge_describe(&ge, preamble, expr, n, args, flags, ga_global_err) != GA_NO_ERROR)
     return nullptr;
   std::vector<int> ktypes;
-  std::string src = strided ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes) : gen_flat(&ge, ktypes);
+  // strided: 0 flat, 1 strided one element per lane, 2 strided four elements per
+  // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride)
+  std::string src = strided == 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes)
+                    : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
+                               : gen_flat(&ge, ktypes);
   return strdup(src.c_str());
 }
 

@@ -466,9 +466,15 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
         if (V > 1) ES = (unsigned)es;
       }
     }
-    // one wavefront per output while rows are short and plentiful
-    if (rtotal <= 8192 && nrows >= 2 * ncu) G = 64;
-    G = (unsigned)env_ul("GPUARRAY_REDUX_G", G) == 64 ? 64 : 256;
+    // One wavefront per output when eight loads per lane cover the inner
+    // reduced dim, four wavefronts otherwise.  Measured on MI355X: rows of
+    // 8192 floats run at 6.7 TB/s with 256 lanes per row and 6.0 with 64;
+    // rows of 512 stepped halves at 3.1 TB/s (useful) with 64 and 2.0 with 256.
+    G = (rin <= (int64_t)64 * V * 8) ? 64 : 256;
+    {
+      const unsigned long force = env_ul("GPUARRAY_REDUX_G", 0);
+      if (force == 64 || force == 256) G = (unsigned)force;
+    }
     int64_t per_pass = (int64_t)G * V;
     U = (unsigned)env_ul("GPUARRAY_REDUX_U", 8);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 8;
@@ -507,13 +513,14 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     if (p.upb > 0) nsplit = (p.units + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;
     groups = (size_t)(rowgroups * nsplit);
-    // short rows, one wavefront each: let a wavefront walk several rows with
-    // the next row's loads in flight (about 8 wavefronts per SIMD in all)
+    // Short rows, one wavefront each, take the kernel without the unit loop.
+    // It can walk several rows per wavefront with the next row's loads in
+    // flight, but on MI355X one row per wavefront measured best (65536 rows
+    // of 1000 floats: 43 us with 1 row, 45 / 47 / 52 us with 2 / 4 / 8), so
+    // that is the default.
     if (G == 64 && nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
       wrows = true;
-      int64_t rpw = (nrows + ncu * 32 - 1) / (ncu * 32);
-      rpw = rpw < 1 ? 1 : (rpw > 16 ? 16 : rpw);
-      rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", (unsigned long)rpw);
+      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", 1);
       if (rpw < 1) rpw = 1;
       p.upb = rpw;
       const int64_t waves = (nrows + rpw - 1) / rpw;

@@ -65,6 +65,16 @@ def test_strided_variants_compile(nd, idx64, tmask):
     assert err == 0, log
 
 
+@pytest.mark.parametrize("nd,idx64,tmask,umask", [(1, 0, 0, 0b101), (2, 0, 0b001, 0b110),
+                                                  (3, 1, 0b100, 0b011), (2, 0, 0, 0b100)])
+def test_four_elements_per_lane_variants_compile(nd, idx64, tmask, umask):
+    src = take_string(gen_elemwise(b"", b"c = a*b + 0.5f", 3, args_of(F32), 0, 2, nd, idx64,
+                                   tmask | (umask << 16)))
+    assert b"ga_chunk16" in src
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
 def test_mixed_types_scalars_and_half_compile():
     spec = [("x", _lib.GA_HALF, R), ("k", _lib.GA_DOUBLE, S), ("m", _lib.GA_UBYTE, R),
             ("y", _lib.GA_HALF, R | W), ("z", _lib.GA_LONG, W)]
