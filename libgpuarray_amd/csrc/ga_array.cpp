@@ -4,6 +4,7 @@
 #include "private.hpp"
 
 #include <map>
+#include <string>
 #include <utility>
 #include <vector>
 
@@ -52,6 +53,16 @@ static int ga_extcopy(GpuArray *dst, const GpuArray *src) {
   }
   void *args[2] = {(void *)src, (void *)dst};
   return GpuElemwise_call(ge, args, GE_BROADCAST);
+}
+
+void ga_take1_cache_free(gpucontext *ctx) {
+  typedef std::map<std::string, GpuKernel> cache_t;
+  void **slot = ga_hip_take1_cache_slot(ctx);
+  if (*slot == nullptr) return;
+  cache_t *cache = (cache_t *)*slot;
+  *slot = nullptr;
+  for (auto &kv : *cache) GpuKernel_clear(&kv.second);
+  delete cache;
 }
 
 // ---- flags ----------------------------------------------------------------------
@@ -647,13 +658,168 @@ int GpuArray_fdump(FILE *fd, const GpuArray *a) {
   return GA_NO_ERROR;
 }
 
-// Gather along the first axis.  Listed after the elementwise and reduction
-// path in the build order; until it lands the call reports that plainly
-// instead of computing something else.
+// a[k, ...] = v[i[k], ...]  (reference :325-548).  Rules kept: a and i are
+// C-contiguous, i is 1-D with a's leading extent, trailing extents of a and v
+// agree, every array is aligned; a negative index counts from the end; an
+// index out of range leaves its row untouched and sets the context's error
+// word, which `check_error` reads back (blocking), resets, and reports as
+// GA_VALUE_ERROR "Index out of bounds".
+// The kernel is a row copy: the trailing dims of v are collapsed on the host
+// (one dim when v's rows are dense), a group owns one output row and a chunk
+// of its columns, lanes run along the columns so both sides are coalesced, and
+// the index is read once per group instead of once per element.  Kernels are
+// kept per context by (types, collapsed rank), so repeated calls compile
+// nothing; the reference rebuilds its kernel on every call (:469-477).
 int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_error) {
-  (void)v; (void)i; (void)check_error;
   gpucontext *ctx = GpuArray_context(a);
-  return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "GpuArray_take1 is not implemented by the hip backend yet");
+  if (!GpuArray_ISWRITEABLE(a))
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array not writeable");
+  if (!GpuArray_ISALIGNED(a) || !GpuArray_ISALIGNED(v) || !GpuArray_ISALIGNED(i))
+    return ga_err_fmt(ctx->err, GA_UNALIGNED_ERROR,
+                      "Not all arrays are aligned: a (%d), b (%d), i (%d)", GpuArray_ISALIGNED(a),
+                      GpuArray_ISALIGNED(v), GpuArray_ISALIGNED(i));
+  if (!GpuArray_IS_C_CONTIGUOUS(a))
+    return ga_err_set(ctx->err, GA_INVALID_ERROR, "Destination array (a) not C-contiguous");
+  if (!GpuArray_IS_C_CONTIGUOUS(i))
+    return ga_err_set(ctx->err, GA_INVALID_ERROR, "Index array (i) not C-contiguous");
+  if (v->nd == 0 || a->nd == 0 || i->nd != 1 || a->nd != v->nd)
+    return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
+                      "Dimension mismatch. v->nd = %u, a->nd = %u, i->nd = %u", v->nd, a->nd, i->nd);
+  if (a->dimensions[0] != i->dimensions[0])
+    return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
+                      "Dimension mismatch. a->dimensions[0] = %zu, i->dimensions[0] = %zu",
+                      a->dimensions[0], i->dimensions[0]);
+  size_t n0 = i->dimensions[0], n1 = 1;
+  for (unsigned int j = 1; j < v->nd; j++) {
+    if (a->dimensions[j] != v->dimensions[j])
+      return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
+                        "Dimension mismatch. a->dimensions[%u] = %zu, v->dimensions[%u] = %zu", j,
+                        a->dimensions[j], j, v->dimensions[j]);
+    n1 *= v->dimensions[j];
+  }
+  const gpuarray_type *ta = gpuarray_get_type(a->typecode), *tv = gpuarray_get_type(v->typecode),
+                      *ti = gpuarray_get_type(i->typecode);
+  if (i->typecode < GA_BYTE || i->typecode > GA_ULONG)
+    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Index array must have an integer type");
+  if (n0 == 0 || n1 == 0) return GA_NO_ERROR;
+
+  // collapse v's trailing dims into as few strided runs as possible
+  unsigned int tnd = v->nd - 1;
+  std::vector<size_t> tdims(v->dimensions + 1, v->dimensions + v->nd);
+  std::vector<ssize_t> tstr(v->strides + 1, v->strides + v->nd);
+  if (tnd == 0) {
+    tnd = 1;
+    tdims.assign(1, 1);
+    tstr.assign(1, 0);
+  } else {
+    ssize_t *row = tstr.data();
+    gpuarray_elemwise_collapse(1, &tnd, tdims.data(), &row);
+  }
+
+  typedef std::map<std::string, GpuKernel> cache_t;
+  void **slot = ga_hip_take1_cache_slot(ctx);
+  if (*slot == nullptr) *slot = new cache_t();
+  cache_t &cache = *(cache_t *)*slot;
+  char key[64];
+  snprintf(key, sizeof(key), "%d:%d:%d:%u", a->typecode, v->typecode, i->typecode, tnd);
+  GpuKernel *k;
+  auto it = cache.find(key);
+  if (it != cache.end()) {
+    k = &it->second;
+  } else {
+    std::string s = "#include \"cluda.h\"\nKERNEL void __launch_bounds__(256) take1(GLOBAL_MEM ";
+    s += ta->cluda_name;
+    s += " *r, const ga_size r_off, GLOBAL_MEM const char *v, const ga_size v_off, "
+         "const ga_ssize s0, const ga_size d0";
+    std::vector<int> types = {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_SSIZE, GA_SIZE};
+    for (unsigned int d = 0; d < tnd; d++) {
+      char b[96];
+      snprintf(b, sizeof(b), ", const ga_ssize s%u, const ga_size d%u", d + 1, d + 1);
+      s += b;
+      types.push_back(GA_SSIZE);
+      types.push_back(GA_SIZE);
+    }
+    s += ", GLOBAL_MEM const ";
+    s += ti->cluda_name;
+    s += " *ind, const ga_size i_off, const ga_size n1, const ga_uint gx, GLOBAL_MEM ga_int *err) {\n"
+         "  const ga_size row = GID_0 / gx;\n"
+         "  const ga_size x0 = (ga_size)(GID_0 % gx) * 1024u + LID_0;\n"
+         "  ind = (GLOBAL_MEM const ";
+    s += ti->cluda_name;
+    s += " *)((GLOBAL_MEM const char *)ind + i_off);\n"
+         "  ga_long ii = (ga_long)ind[row];\n"
+         "  if (ii < 0) ii += (ga_long)d0;\n"
+         "  if (ii < 0 || ii >= (ga_long)d0) { if (LID_0 == 0) *err = -1; return; }\n"
+         "  v += v_off + ii * s0;\n"
+         "  r = (GLOBAL_MEM ";
+    s += ta->cluda_name;
+    s += " *)((GLOBAL_MEM char *)r + r_off) + row * n1;\n"
+         "#pragma unroll\n"
+         "  for (int e = 0; e < 4; e++) {\n"
+         "    const ga_size x = x0 + (ga_size)e * 256u;\n"
+         "    if (x < n1) {\n"
+         "      ga_ssize p = 0; ga_size c = x;\n";
+    for (unsigned int d = tnd; d > 1; d--) {
+      char b[128];
+      snprintf(b, sizeof(b), "      p += (ga_ssize)(c %% d%u) * s%u; c /= d%u;\n", d, d, d);
+      s += b;
+    }
+    s += "      p += (ga_ssize)c * s1;\n      r[x] = *(GLOBAL_MEM const ";
+    s += tv->cluda_name;
+    s += " *)(v + p);\n    }\n  }\n}\n";
+    types.push_back(GA_BUFFER);
+    types.push_back(GA_SIZE);
+    types.push_back(GA_SIZE);
+    types.push_back(GA_UINT);
+    types.push_back(GA_BUFFER);
+    const char *strs[1] = {s.c_str()};
+    size_t lens[1] = {s.size()};
+    GpuKernel nk = {nullptr, nullptr};
+    int flags = gpuarray_type_flags(a->typecode, v->typecode, i->typecode, -1);
+    if (a->typecode == GA_HALF || v->typecode == GA_HALF) {
+      if (a->typecode != v->typecode)
+        return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "take1 between half and another type");
+    }
+    int err = GpuKernel_init(&nk, ctx, 1, strs, lens, "take1", (unsigned)types.size(), types.data(),
+                             flags, nullptr);
+    if (err != GA_NO_ERROR) return err;
+    k = &cache.emplace(key, nk).first->second;
+  }
+
+  gpudata *errbuf = nullptr;
+  int err = gpudata_property(v->data, GA_CTX_PROP_ERRBUF, &errbuf);
+  if (err != GA_NO_ERROR) return err;
+  const size_t gx = (n1 + 1023) / 1024;
+  if (gx > 0xffffffffull || n0 > 0x7fffffffull / gx)
+    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "take1 needs more groups than one launch has");
+  unsigned int gx32 = (unsigned int)gx, p = 0;
+  GpuKernel_setarg(k, p++, a->data);
+  GpuKernel_setarg(k, p++, (void *)&a->offset);
+  GpuKernel_setarg(k, p++, v->data);
+  GpuKernel_setarg(k, p++, (void *)&v->offset);
+  GpuKernel_setarg(k, p++, &v->strides[0]);
+  GpuKernel_setarg(k, p++, &v->dimensions[0]);
+  for (unsigned int d = 0; d < tnd; d++) {
+    GpuKernel_setarg(k, p++, &tstr[d]);
+    GpuKernel_setarg(k, p++, &tdims[d]);
+  }
+  GpuKernel_setarg(k, p++, i->data);
+  GpuKernel_setarg(k, p++, (void *)&i->offset);
+  GpuKernel_setarg(k, p++, &n1);
+  GpuKernel_setarg(k, p++, &gx32);
+  GpuKernel_setarg(k, p++, errbuf);
+  size_t groups = gx * n0, ls = 256;
+  err = GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
+  if (check_error && err == GA_NO_ERROR) {
+    int kerr = 0;
+    err = gpudata_read(&kerr, errbuf, 0, sizeof(int));
+    if (err == GA_NO_ERROR && kerr != 0) {
+      err = ga_err_set(ctx->err, GA_VALUE_ERROR, "Index out of bounds");
+      kerr = 0;
+      gpudata_write(errbuf, 0, &kerr, sizeof(int));
+    }
+  }
+  return err;
 }
 
 }  // extern "C"

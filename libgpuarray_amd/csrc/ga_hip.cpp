@@ -13,6 +13,12 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <fcntl.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <iterator>
+#include <map>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -24,6 +30,168 @@ struct hip_module {
   hipModule_t mod = nullptr;
   unsigned refcnt = 0;
   std::string key;
+};
+
+// ---- device memory cache ------------------------------------------------------
+// hipMalloc and hipFree cost tens to hundreds of microseconds and hipFree
+// waits for the device, so temporaries (results, copies) would dominate the
+// time per call.  Freed buffers therefore go back to a per-context cache
+// instead of to the driver.  The policy is the reference CUDA backend's
+// (src/gpuarray_buffer_cuda.c:607-889): memory comes from the driver in
+// segments of at least 4 MiB, requests are rounded up to a fragment size and
+// served best-fit from the free blocks, a block is split when it is larger
+// than needed and merged with free neighbours of the same segment when it
+// comes back; `max` bounds what is taken from the driver (0 turns the cache
+// off).  Unlike there, no events guard reuse: one in-order stream means work
+// queued on a block before it was freed completes before anything queued
+// after it is handed out again.  Fragments are 256 bytes, so every buffer is
+// aligned for 16-byte vector access.  Lookups are O(log n): free blocks are
+// indexed by size, all blocks by address.
+struct mem_segment {
+  char *base;
+  size_t size;
+};
+
+struct mem_block {
+  char *ptr;
+  size_t size;
+  bool is_free;
+  mem_segment *seg;
+};
+
+struct mem_cache {
+  static constexpr size_t FRAG = 256;
+  static constexpr size_t SEG_MIN = (size_t)4 << 20;
+  static constexpr size_t SEG_ROUND = (size_t)2 << 20;
+  std::map<char *, mem_block *> by_addr;
+  std::multimap<size_t, mem_block *> free_by_size;
+  std::vector<mem_segment *> segs;
+  size_t from_driver = 0;          // bytes currently held from hipMalloc
+  size_t max = (size_t)-1;         // cap on from_driver; 0 = cache disabled
+
+  void index_free(mem_block *b) { b->is_free = true; free_by_size.emplace(b->size, b); }
+  void unindex_free(mem_block *b) {
+    auto r = free_by_size.equal_range(b->size);
+    for (auto it = r.first; it != r.second; ++it)
+      if (it->second == b) { free_by_size.erase(it); break; }
+    b->is_free = false;
+  }
+
+  // Give fully free segments back to the driver (when the device runs out).
+  size_t trim() {
+    size_t released = 0;
+    for (size_t i = 0; i < segs.size();) {
+      mem_segment *sg = segs[i];
+      auto it = by_addr.find(sg->base);
+      if (it != by_addr.end() && it->second->is_free && it->second->size == sg->size) {
+        mem_block *b = it->second;
+        unindex_free(b);
+        by_addr.erase(it);
+        delete b;
+        (void)hipFree(sg->base);
+        from_driver -= sg->size;
+        released += sg->size;
+        delete sg;
+        segs.erase(segs.begin() + (long)i);
+      } else {
+        i++;
+      }
+    }
+    return released;
+  }
+
+  // 0 ok, 1 cap reached, 2 device out of memory, 3 other driver error (*herr)
+  int grow(size_t asize, hipError_t *herr) {
+    size_t want = asize < SEG_MIN ? SEG_MIN : ((asize + SEG_ROUND - 1) / SEG_ROUND) * SEG_ROUND;
+    if (want < asize) return 2;   // overflow
+    if (max != (size_t)-1 && (from_driver > max || want > max - from_driver)) {
+      // try again with exactly what is needed before giving up
+      want = asize;
+      if (from_driver > max || want > max - from_driver) {
+        trim();
+        if (from_driver > max || want > max - from_driver) return 1;
+      }
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      if (trim() > 0) e = hipMalloc(&p, want);
+      if (e != hipSuccess && want != asize) { (void)hipGetLastError(); want = asize; e = hipMalloc(&p, want); }
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      *herr = e;
+      return (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) ? 2 : 3;
+    }
+    mem_segment *sg = new mem_segment{(char *)p, want};
+    segs.push_back(sg);
+    from_driver += want;
+    mem_block *b = new mem_block{(char *)p, want, false, sg};
+    by_addr.emplace(b->ptr, b);
+    index_free(b);
+    return 0;
+  }
+
+  mem_block *take(size_t size, int *why, hipError_t *herr) {
+    size_t asize = ((size ? size : 1) + FRAG - 1) / FRAG * FRAG;
+    if (asize < size) { *why = 2; return nullptr; }
+    auto it = free_by_size.lower_bound(asize);
+    if (it == free_by_size.end()) {
+      if ((*why = grow(asize, herr)) != 0) return nullptr;
+      it = free_by_size.lower_bound(asize);
+    }
+    mem_block *b = it->second;
+    free_by_size.erase(it);
+    b->is_free = false;
+    if (b->size - asize >= FRAG) {
+      mem_block *rest = new mem_block{b->ptr + asize, b->size - asize, false, b->seg};
+      b->size = asize;
+      by_addr.emplace(rest->ptr, rest);
+      index_free(rest);
+    }
+    return b;
+  }
+
+  void give_back(mem_block *b) {
+    auto it = by_addr.find(b->ptr);
+    // merge with the next block of the same segment
+    auto nx = std::next(it);
+    if (nx != by_addr.end() && nx->second->is_free && nx->second->seg == b->seg &&
+        b->ptr + b->size == nx->second->ptr) {
+      mem_block *n = nx->second;
+      unindex_free(n);
+      b->size += n->size;
+      by_addr.erase(nx);
+      delete n;
+    }
+    // and with the previous one
+    if (it != by_addr.begin()) {
+      auto pv = std::prev(it);
+      mem_block *p = pv->second;
+      if (p->is_free && p->seg == b->seg && p->ptr + p->size == b->ptr) {
+        unindex_free(p);
+        p->size += b->size;
+        by_addr.erase(it);
+        delete b;
+        b = p;
+      }
+    }
+    index_free(b);
+  }
+
+  void destroy() {
+    for (auto &kv : by_addr) delete kv.second;
+    by_addr.clear();
+    free_by_size.clear();
+    for (mem_segment *sg : segs) { (void)hipFree(sg->base); delete sg; }
+    segs.clear();
+    from_driver = 0;
+  }
+
+  size_t largest_free() const {
+    return free_by_size.empty() ? 0 : free_by_size.rbegin()->first;
+  }
 };
 
 struct hip_context : _gpucontext {
@@ -42,6 +210,9 @@ struct hip_context : _gpucontext {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
   void *redux_cache = nullptr;
+  void *take1_cache = nullptr;
+  mem_cache mem;
+  std::string disk_cache;   // directory of the on-disk kernel cache, empty = off
   ga_errrec errstore;
 };
 
@@ -52,6 +223,7 @@ struct hip_data : _gpudata {
   size_t sz;
   unsigned int refcnt;
   int flags;
+  mem_block *block;   // cache block behind devptr; NULL when taken straight from the driver
 };
 
 struct hip_kernel : _gpukernel {
@@ -118,6 +290,7 @@ void ctx_destroy(hip_context *ctx) {
   // internal buffers do not count as owners, so they are still here
   if (ctx->errbuf) { hip_release(ctx->errbuf); ctx->errbuf = nullptr; }
   if (ctx->scratch) { hip_release(ctx->scratch); ctx->scratch = nullptr; }
+  ctx->mem.destroy();
   for (auto &kv : ctx->modcache) {
     if (kv.second->mod) (void)hipModuleUnload(kv.second->mod);
     delete kv.second;
@@ -206,6 +379,22 @@ gpucontext *hip_init(gpucontext_props *p) {
   snprintf(ctx->bin_id, sizeof(ctx->bin_id), "%.*s", (int)alen, arch);
 #undef INIT_TRY
 
+  {
+    const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
+    if (dc != nullptr && *dc != 0) ctx->disk_cache = dc;
+  }
+  ctx->mem.max = p->max_cache_size;
+  if (p->initial_cache_size != 0 && ctx->mem.max != 0) {
+    // reserve the first segment now (reference src/gpuarray_buffer_cuda.c:349-356)
+    gpudata *warm = hip_alloc(ctx, p->initial_cache_size, nullptr, BUF_INTERNAL);
+    if (warm == nullptr) {
+      ga_err_set(ga_global_err, ctx->err->code, ctx->err->msg);
+      ctx_destroy(ctx);
+      return nullptr;
+    }
+    hip_release(warm);
+  }
+
   // 8 zeroed bytes kernels can use to report a fault
   // (reference GA_CTX_PROP_ERRBUF, src/gpuarray/buffer.h:646-658).
   uint64_t zero = 0;
@@ -223,6 +412,7 @@ void hip_deinit(gpucontext *c) {
   // Cached operators hold kernels, which hold the context: drop them first.
   ga_extcopy_cache_free(c);
   ga_redux_cache_free(c);
+  ga_take1_cache_free(c);
   ctx_unref(ctx);
 }
 
@@ -250,25 +440,45 @@ gpudata *hip_alloc(gpucontext *c, size_t sz, void *data, int flags) {
     return nullptr;
   }
   size_t asz = sz ? sz : 1;   // a zero-byte request still yields a valid buffer
-  hipError_t e = hipMalloc(&b->devptr, asz);
-  if (e != hipSuccess) {
-    free(b);
-    if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation)
-      ga_err_fmt(ctx->err, GA_MEMORY_ERROR, "hipMalloc(%zu): out of device memory", asz);
-    else
-      hip_fail(ctx->err, "hipMalloc", e);
-    return nullptr;
+  if (ctx->mem.max != 0) {
+    int why = 0;
+    hipError_t herr = hipSuccess;
+    mem_block *blk = ctx->mem.take(asz, &why, &herr);
+    if (blk == nullptr) {
+      free(b);
+      if (why == 1)
+        ga_err_set(ctx->err, GA_VALUE_ERROR, "Maximum cache size reached");
+      else if (why == 2)
+        ga_err_fmt(ctx->err, GA_MEMORY_ERROR, "hipMalloc(%zu): out of device memory", asz);
+      else
+        hip_fail(ctx->err, "hipMalloc", herr);
+      return nullptr;
+    }
+    b->devptr = blk->ptr;
+    b->block = blk;   // the block may be larger; sz stays the size asked for
+  } else {
+    hipError_t e = hipMalloc(&b->devptr, asz);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      free(b);
+      if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation)
+        ga_err_fmt(ctx->err, GA_MEMORY_ERROR, "hipMalloc(%zu): out of device memory", asz);
+      else
+        hip_fail(ctx->err, "hipMalloc", e);
+      return nullptr;
+    }
   }
   b->ctx = ctx;
   b->sz = asz;
   b->refcnt = 1;
   b->flags = (flags & (GA_BUFFER_MASK | BUF_INTERNAL)) | BUF_OWNED;
   if (flags & GA_BUFFER_INIT) {
-    e = hipMemcpyHtoDAsync(b->devptr, data, sz, ctx->stream);
+    hipError_t e = hipMemcpyHtoDAsync(b->devptr, data, sz, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
       hip_fail(ctx->err, "hipMemcpyHtoDAsync", e);
-      (void)hipFree(b->devptr);
+      if (b->block) ctx->mem.give_back(b->block);
+      else (void)hipFree(b->devptr);
       free(b);
       return nullptr;
     }
@@ -283,7 +493,10 @@ void hip_release(gpudata *bb) {
   hip_data *b = HD(bb);
   if (--b->refcnt != 0) return;
   hip_context *ctx = HC(b->ctx);
-  if (b->flags & BUF_OWNED) {
+  if (b->block != nullptr) {
+    // back to the cache; stream order protects work still queued on it
+    ctx->mem.give_back(b->block);
+  } else if (b->flags & BUF_OWNED) {
     (void)hipSetDevice(ctx->dev);
     // hipFree waits for the device, so queued work that still uses the
     // memory completes first.
@@ -444,6 +657,110 @@ int rtc_compile(const std::string &src, std::vector<char> &code, std::string &lo
   return GA_NO_ERROR;
 }
 
+// ---- on-disk cache of compiled kernels ------------------------------------------
+// A compile costs 0.3-0.5 s; a process that builds a few hundred operators
+// spends minutes in the compiler.  With a cache directory (property
+// kernel_cache_path or environment GPUARRAY_CACHE_PATH, the reference's
+// names: src/gpuarray_buffer_cuda.c:301-331) code objects are kept across
+// processes.  Layout follows the reference's disk cache (src/cache/disk.c:
+// 214-289): the key is {format tag, compiler version, ISA, options, source},
+// the file name is the hex of a hash of the key under a two-level directory,
+// the file holds 8-byte big-endian key and value lengths, then key, then
+// value, and is written under a temporary name and renamed.  The stored key
+// is compared in full on load, so a hash collision is a miss, not a wrong
+// kernel; a checksum of the value follows it, so a damaged file is a miss too
+// and is never handed to the loader.
+std::string disk_key(const std::string &src, const char *isa) {
+  std::string k = "ga-hip-kcache-1|";
+  int maj = 0, min = 0;
+  if (hiprtcVersion(&maj, &min) == HIPRTC_SUCCESS) k += std::to_string(maj) + "." + std::to_string(min);
+  k += "|";
+  k += isa;
+  for (const char *o : k_rtc_opts) { k += "|"; k += o; }
+  k += "|";
+  k += ga_cluda_hip_src;
+  k += "|";
+  k += src;
+  return k;
+}
+
+void hash128(const std::string &k, uint64_t out[2]) {
+  // two independent FNV-1a style streams; only used to name files
+  uint64_t a = 0xcbf29ce484222325ull, b = 0x84222325cbf29ce4ull;
+  for (unsigned char c : k) {
+    a = (a ^ c) * 0x100000001b3ull;
+    b = (b ^ (c + 0x9e)) * 0x100000001b5ull;
+    b ^= b >> 29;
+  }
+  out[0] = a;
+  out[1] = b;
+}
+
+std::string disk_path(const std::string &dir, const std::string &key, bool mkdirs) {
+  uint64_t h[2];
+  hash128(key, h);
+  char name[64];
+  snprintf(name, sizeof(name), "%016llx%016llx", (unsigned long long)h[0], (unsigned long long)h[1]);
+  std::string sub = dir + "/" + std::string(name, 4);
+  if (mkdirs) {
+    (void)mkdir(dir.c_str(), 0777);
+    (void)mkdir(sub.c_str(), 0777);
+  }
+  return sub + "/" + (name + 4);
+}
+
+void put_be64(unsigned char *p, uint64_t v) {
+  for (int i = 7; i >= 0; i--) { p[i] = (unsigned char)(v & 0xff); v >>= 8; }
+}
+uint64_t get_be64(const unsigned char *p) {
+  uint64_t v = 0;
+  for (int i = 0; i < 8; i++) v = (v << 8) | p[i];
+  return v;
+}
+
+uint64_t checksum64(const std::vector<char> &v) {
+  uint64_t a = 0xcbf29ce484222325ull;
+  for (char c : v) a = (a ^ (unsigned char)c) * 0x100000001b3ull;
+  return a;
+}
+
+bool disk_load(const std::string &dir, const std::string &key, std::vector<char> &code) {
+  FILE *f = fopen(disk_path(dir, key, false).c_str(), "rb");
+  if (f == nullptr) return false;
+  unsigned char hdr[16];
+  bool ok = fread(hdr, 1, 16, f) == 16;
+  uint64_t kl = ok ? get_be64(hdr) : 0, vl = ok ? get_be64(hdr + 8) : 0;
+  ok = ok && kl == key.size() && vl > 0 && vl < ((uint64_t)1 << 31);
+  if (ok) {
+    std::string stored(kl, '\0');
+    ok = fread(&stored[0], 1, kl, f) == kl && stored == key;
+  }
+  if (ok) {
+    code.resize(vl);
+    ok = fread(code.data(), 1, vl, f) == vl;
+  }
+  unsigned char sum[8];
+  ok = ok && fread(sum, 1, 8, f) == 8 && get_be64(sum) == checksum64(code);
+  fclose(f);
+  return ok;
+}
+
+void disk_store(const std::string &dir, const std::string &key, const std::vector<char> &code) {
+  std::string path = disk_path(dir, key, true);
+  std::string tmp = path + ".tmp." + std::to_string((long)getpid());
+  FILE *f = fopen(tmp.c_str(), "wb");
+  if (f == nullptr) return;   // a cache that cannot be written is only slower
+  unsigned char hdr[16];
+  put_be64(hdr, key.size());
+  put_be64(hdr + 8, code.size());
+  unsigned char sum[8];
+  put_be64(sum, checksum64(code));
+  bool ok = fwrite(hdr, 1, 16, f) == 16 && fwrite(key.data(), 1, key.size(), f) == key.size() &&
+            fwrite(code.data(), 1, code.size(), f) == code.size() && fwrite(sum, 1, 8, f) == 8;
+  ok = fclose(f) == 0 && ok;
+  if (!ok || rename(tmp.c_str(), path.c_str()) != 0) (void)unlink(tmp.c_str());
+}
+
 void mod_unref(hip_context *ctx, hip_module *m) {
   // Modules stay cached for the life of the context: recompiling costs
   // hundreds of milliseconds, keeping one costs a few kilobytes.
@@ -479,14 +796,34 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
     m = it->second;
   } else {
     std::vector<char> code;
-    std::string log;
-    err = rtc_compile(src, code, log);
-    if (err != GA_NO_ERROR) {
-      if (err_str) *err_str = strdup(log.c_str());
-      return ga_err_fmt(ctx->err, GA_IMPL_ERROR, "Kernel compilation failed: %.900s", log.c_str());
+    std::string log, dkey;
+    bool from_disk = false;
+    if (!ctx->disk_cache.empty()) {
+      dkey = disk_key(src, ctx->bin_id);
+      from_disk = disk_load(ctx->disk_cache, dkey, code);
+    }
+    if (!from_disk) {
+      err = rtc_compile(src, code, log);
+      if (err != GA_NO_ERROR) {
+        if (err_str) *err_str = strdup(log.c_str());
+        return ga_err_fmt(ctx->err, GA_IMPL_ERROR, "Kernel compilation failed: %.900s", log.c_str());
+      }
+      if (!ctx->disk_cache.empty()) disk_store(ctx->disk_cache, dkey, code);
     }
     m = new hip_module();
     hipError_t e = hipModuleLoadData(&m->mod, code.data());
+    if (e != hipSuccess && from_disk) {
+      // a damaged cache entry: compile afresh and replace it
+      (void)hipGetLastError();
+      err = rtc_compile(src, code, log);
+      if (err != GA_NO_ERROR) {
+        delete m;
+        if (err_str) *err_str = strdup(log.c_str());
+        return ga_err_fmt(ctx->err, GA_IMPL_ERROR, "Kernel compilation failed: %.900s", log.c_str());
+      }
+      disk_store(ctx->disk_cache, dkey, code);
+      e = hipModuleLoadData(&m->mod, code.data());
+    }
     if (e != hipSuccess) {
       delete m;
       return hip_fail(ctx->err, "hipModuleLoadData", e);
@@ -661,7 +998,19 @@ int hip_property(gpucontext *c, gpudata *buf, gpukernel *k, int prop_id, void *r
     int e;
     if ((e = enter(ctx)) != GA_NO_ERROR) return e;
     HIP_TRY(ctx, hipMemGetInfo(&fr, &tot));
-    *(size_t *)res = prop_id == GA_CTX_PROP_TOTAL_GMEM ? tot : fr;
+    if (prop_id == GA_CTX_PROP_TOTAL_GMEM) {
+      *(size_t *)res = tot;
+    } else if (prop_id == GA_CTX_PROP_FREE_GMEM) {
+      // what the driver still has plus what the cache can hand out again
+      size_t cached = 0;
+      for (const auto &kv : ctx->mem.free_by_size) cached += kv.first;
+      *(size_t *)res = fr + cached;
+    } else {
+      // the reference guesses a quarter of the driver's free memory, or the
+      // largest cached block if that is bigger (src/gpuarray_buffer_cuda.c:621-635)
+      size_t guess = fr / 4, big = ctx->mem.largest_free();
+      *(size_t *)res = big > guess ? big : guess;
+    }
     return GA_NO_ERROR;
   }
   case GA_CTX_PROP_NATIVE_FLOAT16:
@@ -833,6 +1182,7 @@ gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
 
 unsigned int ga_hip_numprocs(gpucontext *c) { return HC(c)->numprocs; }
 void **ga_hip_redux_cache_slot(gpucontext *c) { return &HC(c)->redux_cache; }
+void **ga_hip_take1_cache_slot(gpucontext *c) { return &HC(c)->take1_cache; }
 
 const ga_buffer_ops ga_hip_ops = {
     hip_get_platform_count, hip_get_device_count, hip_init,        hip_deinit,

@@ -142,6 +142,9 @@ void ga_extcopy_cache_free(gpucontext *ctx);
 // Frees the per-context cache behind GpuArray_maxandargmax (reduction.cpp).
 void ga_redux_cache_free(gpucontext *ctx);
 void **ga_hip_redux_cache_slot(gpucontext *ctx);
+// Frees the per-context kernels of GpuArray_take1 (array.cpp).
+void ga_take1_cache_free(gpucontext *ctx);
+void **ga_hip_take1_cache_slot(gpucontext *ctx);
 
 // Typecode of the opaque by-value "plan" kernel argument of `bytes` bytes
 // (registered on first use through gpuarray_register_type).

@@ -7,6 +7,7 @@ All device work happens inside libgpuarray.so; this file only marshals
 shapes, strides and pointers.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -50,12 +51,25 @@ def count_devices(kind="hip", platform=0):
 class GpuContext(object):
     """One device, one stream (reference pygpu/gpuarray.pyx:1027-1168)."""
 
-    def __init__(self, kind="hip", devno=0, single_stream=True):
+    def __init__(self, kind="hip", devno=0, single_stream=True, initial_cache_size=None,
+                 max_cache_size=None, kernel_cache_path=None):
         props = C.c_void_p()
         check(lib.gpucontext_props_new(C.byref(props)))
         lib.gpucontext_props_hip_dev(props, devno)
         if single_stream:
             lib.gpucontext_props_set_single_stream(props)
+        if kernel_cache_path is not None:
+            # the props object keeps the pointer, not a copy: hold the bytes
+            self._kcache = os.fsencode(kernel_cache_path)
+            lib.gpucontext_props_kernel_cache(props, self._kcache)
+        if initial_cache_size is not None or max_cache_size is not None:
+            # max_cache_size == 0 turns the device memory cache off
+            err = lib.gpucontext_props_alloc_cache(
+                props, initial_cache_size or 0,
+                (1 << 64) - 1 if max_cache_size is None else max_cache_size)
+            if err:
+                lib.gpucontext_props_del(props)
+                check(err)
         self.ctx = C.c_void_p()
         self.kind = kind
         # init consumes props
@@ -252,6 +266,22 @@ class GpuArray(object):
             o = _lib.GA_F_ORDER if (self.flags.f_contiguous and not self.flags.c_contiguous) \
                 else _lib.GA_C_ORDER
         self._check(lib.GpuArray_copy(res._ptr(), self._ptr(), o))
+        return res
+
+    def take1(self, idx):
+        """Rows of `self` picked by the 1-D integer array `idx`
+        (reference pygpu/gpuarray.pyx:2098-2113): negative entries count from
+        the end, an entry out of range raises IndexError."""
+        if idx.ndim != 1:
+            raise ValueError("Expected index with nd=1")
+        if self.ndim == 0:
+            raise _lib.GpuArrayException("take1 of a 0-d array", _lib.GA_INVALID_ERROR)
+        res = empty((idx.shape[0],) + self.shape[1:], self.dtype, context=self.context)
+        err = lib.GpuArray_take1(res._ptr(), self._ptr(), idx._ptr(), 1)
+        if err == _lib.GA_VALUE_ERROR:
+            msg = lib.gpucontext_error(self.context.ctx, err)
+            raise IndexError(msg.decode(errors="replace") if msg else "Index out of bounds")
+        self._check(err)
         return res
 
     def astype(self, dtype, order="A"):

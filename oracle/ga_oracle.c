@@ -472,3 +472,44 @@ int orc_reduk(int op, const char *src, int in_t, unsigned nd, const size_t *dims
   free(li);
   return 0;
 }
+
+/* ---- take1, src/gpuarray_array.c:325-383 (kernel text) and :385-548 -------
+ * r is C-contiguous [n0, n1]; for every (i0, i1): the index ind[i0] is
+ * wrapped once when negative, an index still outside [0, d0) sets *err = -1
+ * and leaves the element alone; i1 is unravelled over v's trailing dims,
+ * last dim fastest (:352-361), into a byte position through v's strides.
+ * Elements are moved as `elsz` bytes (same type on both sides).
+ * ind_kind: size in bytes of an index, negative when the type is signed. */
+int orc_take1(char *r, const char *v, size_t elsz, unsigned nd, const size_t *vdims,
+              const ssize_t *vstr, const void *ind, int ind_kind, size_t n0, int *err) {
+  size_t n1 = 1;
+  for (unsigned j = 1; j < nd; j++) n1 *= vdims[j];
+  for (size_t i0 = 0; i0 < n0; i0++) {
+    for (size_t i1 = 0; i1 < n1; i1++) {
+      long long ii0;
+      switch (ind_kind) {
+      case -1: ii0 = ((const int8_t *)ind)[i0]; break;
+      case 1: ii0 = ((const uint8_t *)ind)[i0]; break;
+      case -2: ii0 = ((const int16_t *)ind)[i0]; break;
+      case 2: ii0 = ((const uint16_t *)ind)[i0]; break;
+      case -4: ii0 = ((const int32_t *)ind)[i0]; break;
+      case 4: ii0 = ((const uint32_t *)ind)[i0]; break;
+      case -8: ii0 = ((const int64_t *)ind)[i0]; break;
+      case 8: ii0 = (long long)((const uint64_t *)ind)[i0]; break;
+      default: return 4;
+      }
+      ssize_t pos = 0;
+      size_t idx = i1;
+      if (ii0 < 0) ii0 += (long long)vdims[0];
+      if (ii0 < 0 || ii0 >= (long long)vdims[0]) { *err = -1; continue; }
+      pos += ii0 * vstr[0];
+      for (unsigned j = nd - 1; j >= 1; j--) {
+        size_t ij = idx % vdims[j];
+        idx /= vdims[j];
+        pos += (ssize_t)ij * vstr[j];
+      }
+      memcpy(r + (i0 * n1 + i1) * elsz, v + pos, elsz);
+    }
+  }
+  return 0;
+}

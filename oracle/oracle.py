@@ -45,6 +45,8 @@ def _load():
                                    C.POINTER(C.c_uint), C.c_void_p, PSS, C.c_void_p, PSS]
     L.orc_reduk.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_uint, PS, PSS, C.POINTER(C.c_int),
                             C.c_void_p, C.c_int, C.c_size_t]
+    L.orc_take1.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint, PS, PSS, C.c_void_p,
+                            C.c_int, C.c_size_t, C.POINTER(C.c_int)]
     return L
 
 
@@ -266,3 +268,24 @@ def check_args(shapes, strides, collapse=False, broadcast=False):
                         del st[i]
                 nd -= 1
     return n, nd, tuple(dims), tuple(None if st is None else tuple(st) for st in strs)
+
+
+def take1(v, ind, out=None):
+    """GpuArray_take1 (src/gpuarray_array.c:325-548) on host arrays: returns
+    (rows, err) where err is -1 when some index was out of range (those rows
+    keep the content of `out`, or zeros)."""
+    ind = np.ascontiguousarray(ind)
+    n0 = ind.shape[0]
+    if out is None:
+        out = np.zeros((n0,) + v.shape[1:], dtype=v.dtype)
+    assert out.flags.c_contiguous and out.dtype == v.dtype
+    nd = v.ndim
+    dims = (C.c_size_t * nd)(*v.shape)
+    strs = (C.c_ssize_t * nd)(*v.strides)
+    kind = ind.dtype.itemsize * (-1 if ind.dtype.kind == "i" else 1)
+    err = C.c_int(0)
+    rc = _L.orc_take1(C.c_void_p(out.ctypes.data), C.c_void_p(v.ctypes.data), v.dtype.itemsize, nd,
+                      dims, strs, C.c_void_p(ind.ctypes.data), kind, n0, C.byref(err))
+    if rc:
+        raise ValueError("orc_take1: error %d" % rc)
+    return out, err.value

@@ -279,3 +279,105 @@ def test_split_and_concatenate(ctx):
     lib.GpuArray_clear(C.byref(r))
     for o in outs:
         lib.GpuArray_clear(C.byref(o))
+
+
+def test_memory_cache_reuses_and_never_overlaps(ctx):
+    # freed blocks come back without a trip to the driver, live blocks never
+    # overlap, and their contents survive neighbours being split and merged
+    rng = np.random.default_rng(12)
+    ptr_of = _lib.extension("hip_get_ptr", C.c_void_p, [C.c_void_p])
+    size_of = _lib.extension("hip_get_sz", C.c_size_t, [C.c_void_p])
+    d = lib.gpudata_alloc(ctx.ctx, 1 << 20, None, 0, None)
+    p0 = ptr_of(d)
+    lib.gpudata_release(d)
+    d = lib.gpudata_alloc(ctx.ctx, 1 << 20, None, 0, None)
+    assert ptr_of(d) == p0                       # best fit finds the block just freed
+    assert size_of(d) == 1 << 20 and ptr_of(d) % 256 == 0
+    lib.gpudata_release(d)
+    live = {}
+    for step in range(400):
+        if live and rng.random() < 0.45:
+            key = list(live)[int(rng.integers(len(live)))]
+            buf, pattern = live.pop(key)
+            back = np.empty_like(pattern)
+            assert lib.gpudata_read(back.ctypes.data, buf, 0, back.nbytes) == 0
+            assert np.array_equal(back, pattern)
+            lib.gpudata_release(buf)
+        else:
+            n = int(rng.choice([1, 7, 255, 256, 257, 4096, 70000, 1 << 20, (1 << 22) + 5]))
+            buf = lib.gpudata_alloc(ctx.ctx, n, None, 0, None)
+            assert buf and ptr_of(buf) % 256 == 0
+            pattern = rng.integers(0, 256, n, dtype=np.uint8)
+            assert lib.gpudata_write(buf, 0, pattern.ctypes.data, n) == 0
+            live[step] = (buf, pattern)
+        spans = sorted((ptr_of(b), ptr_of(b) + size_of(b)) for b, _ in live.values())
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+    for buf, pattern in live.values():
+        back = np.empty_like(pattern)
+        assert lib.gpudata_read(back.ctypes.data, buf, 0, back.nbytes) == 0
+        assert np.array_equal(back, pattern)
+        lib.gpudata_release(buf)
+
+
+def test_memory_cache_limits():
+    # reference rules: max bounds what is taken from the device and the error
+    # is "Maximum cache size reached" (src/gpuarray_buffer_cuda.c:649-653);
+    # max == 0 turns the cache off; initial must not exceed max
+    c = ga.GpuContext("hip", 0, initial_cache_size=1 << 20, max_cache_size=16 << 20)
+    e = C.c_int(0)
+    bufs = []
+    while True:
+        b = lib.gpudata_alloc(c.ctx, 4 << 20, None, 0, C.byref(e))
+        if not b:
+            break
+        bufs.append(b)
+        assert len(bufs) <= 4                    # 16 MiB cap, 4 MiB each
+    assert len(bufs) >= 3                        # the context's own 8-byte buffer sits in one segment
+    assert e.value == _lib.GA_VALUE_ERROR and "Maximum cache size reached" in c.error()
+    lib.gpudata_release(bufs.pop())
+    again = lib.gpudata_alloc(c.ctx, 3 << 20, None, 0, None)      # fits in what was freed
+    assert again
+    for b in bufs + [again]:
+        lib.gpudata_release(b)
+    nocache = ga.GpuContext("hip", 0, max_cache_size=0)
+    a = gpuarray.array(np.arange(1000, dtype=np.float32), context=nocache)
+    assert np.array_equal(np.asarray(a), np.arange(1000, dtype=np.float32))
+    with pytest.raises(ga.GpuArrayException):
+        ga.GpuContext("hip", 0, initial_cache_size=2, max_cache_size=1)
+
+
+def test_disk_kernel_cache(tmp_path):
+    import glob, os, time
+    d = str(tmp_path / "kcache")
+    expr = "c = a*b + 0.25f /* disk cache test */"
+    spec = [ga.arg("a", "float32", read=True), ga.arg("b", "float32", read=True),
+            ga.arg("c", "float32", write=True)]
+
+    def run(c):
+        t0 = time.perf_counter()
+        k = ga.GpuElemwise(c, expr, spec)
+        dt = time.perf_counter() - t0
+        a = gpuarray.array(np.arange(1000, dtype=np.float32), context=c)
+        out = gpuarray.empty((1000,), "float32", context=c)
+        k(a, a, out)
+        want = np.arange(1000, dtype=np.float32) ** 2 + np.float32(0.25)
+        assert np.array_equal(np.asarray(out), want)
+        return dt
+
+    cold = run(ga.GpuContext("hip", 0, kernel_cache_path=d))
+    files = [f for f in glob.glob(os.path.join(d, "*", "*")) if ".tmp." not in f]
+    assert len(files) == 1
+    # entry layout: 8-byte big-endian key and value lengths, key, value, checksum
+    raw = open(files[0], "rb").read()
+    kl, vl = int.from_bytes(raw[:8], "big"), int.from_bytes(raw[8:16], "big")
+    assert len(raw) == 16 + kl + vl + 8 and expr.encode() in raw[16:16 + kl]
+    assert raw[16 + kl:16 + kl + 4] == b"\x7fELF"
+    warm = run(ga.GpuContext("hip", 0, kernel_cache_path=d))     # new context: module comes from disk
+    assert warm < cold / 3, (cold, warm)
+    # a damaged entry fails its checksum: it is recompiled and replaced, and
+    # the damaged code never reaches the loader
+    with open(files[0], "r+b") as f:
+        f.seek(16 + kl + 64)
+        f.write(b"\0" * 256)
+    run(ga.GpuContext("hip", 0, kernel_cache_path=d))
+    assert open(files[0], "rb").read()[16 + kl:] == raw[16 + kl:]

@@ -326,3 +326,41 @@ def test_contig_muladd_two_roundings(oracle):
     # a fused multiply-add would differ somewhere on this input
     fused = (a.astype(np.float64) * b.astype(np.float64) + 0.5).astype(np.float32)
     assert not np.array_equal(c, fused)
+
+
+# ---- take1: tests/check_array.c:17-250 and pygpu/tests/test_gpu_ndarray.py:740-754 ----
+
+@pytest.mark.parametrize("case", KATS["take1"]["cases"], ids=lambda c: "x".join(map(str, c["v_shape"])))
+def test_take1_reference_vectors(oracle, case):
+    v = np.arange(case["v_elems"], dtype=np.uint32).reshape(case["v_shape"])
+    got, err = oracle.take1(v, np.array(case["index"], dtype=np.int64))
+    assert err == 0
+    assert got.ravel().tolist() == case["expect"]
+
+
+@pytest.mark.parametrize("case", KATS["take1"]["pygpu_cases"]["cases"],
+                         ids=lambda c: "x".join(map(str, c["shape"])))
+def test_take1_is_numpy_take(oracle, case):
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal(case["shape"]).astype(np.float32)
+    idx = np.array(case["index"])
+    got, err = oracle.take1(v, idx)
+    assert err == 0 and np.array_equal(got, v.take(idx, axis=0))
+
+
+def test_take1_strided_source_wrap_and_bounds(oracle):
+    rng = np.random.default_rng(6)
+    base = rng.integers(0, 1 << 30, size=(9, 6, 10), dtype=np.int32)
+    v = base[::2, ::-1, 1::3]                       # (5, 6, 3), mixed-sign strides
+    for dt in (np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64):
+        idx = np.array([4, 0, 3, 3, 1], dtype=dt)
+        got, err = oracle.take1(v, idx)
+        assert err == 0 and np.array_equal(got, v[idx.astype(np.int64)])
+    idx = np.array([-1, -5, 2], dtype=np.int32)
+    got, err = oracle.take1(v, idx)
+    assert err == 0 and np.array_equal(got, v[[4, 0, 2]])
+    # one wrap only: -6 and 5 are outside [0, 5); those rows are left alone
+    out = np.full((4, 6, 3), -7, dtype=np.int32)
+    got, err = oracle.take1(v, np.array([1, -6, 5, 2], dtype=np.int64), out=out)
+    assert err == -1
+    assert np.array_equal(got[[0, 3]], v[[1, 2]]) and np.all(got[[1, 2]] == -7)
