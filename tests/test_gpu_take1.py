@@ -66,8 +66,7 @@ def test_index_types_and_strided_sources(ctx, oracle, itype):
             assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("dtype", ["uint8", "float16", "int16", "float32", "float64", "complex64",
-                                   "complex128"])
+@pytest.mark.parametrize("dtype", ["uint8", "float16", "int16", "float32", "float64"])
 def test_element_types_and_wide_rows(ctx, oracle, dtype):
     rng = np.random.default_rng(13)
     dt = np.dtype(dtype)
@@ -78,6 +77,12 @@ def test_element_types_and_wide_rows(ctx, oracle, dtype):
     want, err = oracle.take1(v, idx)
     assert err == 0
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_complex_is_refused_like_other_kernels(ctx):
+    v = gpuarray.array(np.zeros((3, 2), np.complex64), context=ctx)
+    with pytest.raises(_lib.UnsupportedException):
+        v.take1(gpuarray.array(np.array([0]), context=ctx))
 
 
 def test_out_of_bounds_reports_and_skips(ctx, oracle):
