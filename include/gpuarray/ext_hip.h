@@ -52,6 +52,15 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);
+/* "hip_mapreduce_source": the same for an operator of GpuReduction_new_map
+ * (same leading arguments); vecmask bit k: array argument k is fetched with
+ * vector loads, the others element by element. */
+typedef char *(*ga_hip_mapreduce_source_fn)(int op, const char *reduce_expr, const char *neutral,
+                                            int acc_typecode, const char *preamble,
+                                            const char *map_expr, unsigned int n, const void *args,
+                                            int d0_typecode, unsigned int lanes_per_output,
+                                            unsigned int vec, unsigned int unroll,
+                                            unsigned int vecmask);
 
 #ifdef __cplusplus
 }

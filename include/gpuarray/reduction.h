@@ -12,6 +12,7 @@
 
 #include <gpuarray/array.h>
 #include <gpuarray/buffer.h>
+#include <gpuarray/elemwise.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -33,6 +34,7 @@ typedef enum _ga_reduce_op {
   GA_REDUCE_XOR,                /* bitwise xor         -                  */
   GA_REDUCE_ALL,                /* 1 if all non-zero   -                  */
   GA_REDUCE_ANY,                /* 1 if any non-zero   -                  */
+  GA_REDUCE_CUSTOM,             /* caller's expression (GpuReduction_new_map only) */
   GA_REDUCE_ENDSUPPORTED
 } ga_reduce_op;
 
@@ -73,6 +75,51 @@ GPUARRAY_PUBLIC int GpuReduction_call(const GpuReduction *gr, GpuArray *d0,
                                       GpuArray *d1, const GpuArray *s0,
                                       unsigned reduxLen, const int *reduxList,
                                       int flags);
+
+/* A reduction fed by an elementwise expression over several arguments, in one
+ * pass over memory: the C counterpart of the reference's
+ * ReductionKernel(map_expr=..., arguments=...) (pygpu/reduction.py:137-291,
+ * used as in pygpu/tests/test_reduction.py:57-84), which exists there only in
+ * Python.
+ *
+ *   op           any ga_reduce_op.  GA_REDUCE_CUSTOM combines with the caller's
+ *                `reduce_expr`, an expression in `a` and `b` (the reference's
+ *                REDUCE(a, b) macro, pygpu/reduction.py:38), starting from
+ *                `neutral`; the expression must be associative and
+ *                commutative and `neutral` its identity.  Both are NULL for
+ *                the other operations.
+ *   accTypecode  type the expression's value is converted to, the operation
+ *                runs in, and the value result d0 has (ALL/ANY: any integer
+ *                d0).  GA_HALF accumulates in float and stores a half.
+ *   preamble     device code placed before the expression (may be NULL).
+ *   map_expr     expression over the argument names, e.g. "a*b"; an array
+ *                argument's name stands for its element (half elements are
+ *                seen as float), a scalar's for its value.
+ *   args         n descriptors as for GpuElemwise_new; GE_SCALAR marks
+ *                scalars, GE_WRITE is refused.  At least one array, at most 8.
+ */
+GPUARRAY_PUBLIC int GpuReduction_new_map(GpuReduction **gr, gpucontext *ctx,
+                                         ga_reduce_op op,
+                                         const char *reduce_expr,
+                                         const char *neutral, int accTypecode,
+                                         const char *preamble,
+                                         const char *map_expr, unsigned int n,
+                                         const gpuelemwise_arg *args,
+                                         int flags);
+
+/* Run an operator made by GpuReduction_new_map.
+ *   args   n pointers in descriptor order: GpuArray* for arrays, pointer to a
+ *          host value of the declared type for scalars (the convention of
+ *          GpuElemwise_call).
+ *   flags  GE_BROADCAST: an extent of 1 stretches to the other arrays' extent.
+ *          All arrays must have the same number of dimensions.
+ * d0, d1, reduxLen, reduxList and every rule on values, indices, ties, NaN and
+ * empty axes are those of GpuReduction_call, applied to the expression's
+ * values over the common (broadcast) shape. */
+GPUARRAY_PUBLIC int GpuReduction_call_map(const GpuReduction *gr, GpuArray *d0,
+                                          GpuArray *d1, void **args,
+                                          unsigned reduxLen,
+                                          const int *reduxList, int flags);
 
 #ifdef __cplusplus
 }

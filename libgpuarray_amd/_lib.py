@@ -71,7 +71,8 @@ GA_KERNEL_PROP_NUMARGS = 1027
 
 (GA_REDUCE_SUM, GA_REDUCE_PROD, GA_REDUCE_PRODNZ, GA_REDUCE_MIN, GA_REDUCE_MAX,
  GA_REDUCE_ARGMIN, GA_REDUCE_ARGMAX, GA_REDUCE_MINANDARGMIN, GA_REDUCE_MAXANDARGMAX,
- GA_REDUCE_AND, GA_REDUCE_OR, GA_REDUCE_XOR, GA_REDUCE_ALL, GA_REDUCE_ANY) = range(14)
+ GA_REDUCE_AND, GA_REDUCE_OR, GA_REDUCE_XOR, GA_REDUCE_ALL, GA_REDUCE_ANY,
+ GA_REDUCE_CUSTOM) = range(15)
 
 
 # ---- structs -----------------------------------------------------------------
@@ -211,6 +212,11 @@ SIGNATURES = {
     # reduction.h
     "GpuReduction_new": (C.c_int, [C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_uint,
                                    C.c_uint, C.c_int, C.c_int]),
+    "GpuReduction_new_map": (C.c_int, [C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_char_p,
+                                       C.c_char_p, C.c_int, C.c_char_p, C.c_char_p, C.c_uint,
+                                       C.c_void_p, C.c_int]),
+    "GpuReduction_call_map": (C.c_int, [C.c_void_p, PA, PA, C.POINTER(C.c_void_p), C.c_uint,
+                                        C.POINTER(C.c_int), C.c_int]),
     "GpuReduction_free": (None, [C.c_void_p]),
     "GpuReduction_call": (C.c_int, [C.c_void_p, PA, PA, PA, C.c_uint, C.POINTER(C.c_int),
                                     C.c_int]),

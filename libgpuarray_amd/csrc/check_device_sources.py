@@ -31,6 +31,9 @@ def main():
                  C.c_uint, C.c_int, C.c_uint])
     gen_r = ext(b"hip_reduction_source", C.c_void_p,
                 [C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_uint])
+    gen_m = ext(b"hip_mapreduce_source", C.c_void_p,
+                [C.c_int, C.c_char_p, C.c_char_p, C.c_int, C.c_char_p, C.c_char_p, C.c_uint,
+                 C.POINTER(ElemwiseArg), C.c_int, C.c_uint, C.c_uint, C.c_uint, C.c_uint])
     comp = ext(b"hip_compile_only", C.c_int,
                [C.c_uint, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t), C.POINTER(C.c_char_p)])
 
@@ -70,7 +73,20 @@ def main():
     check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1))
     check("reduction stepped halves", gen_r(0, GA_HALF, GA_FLOAT, GA_LONG, 256, 4 | (2 << 8), 1))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
-    print("device sources compile for gfx950 (%d reduction variants, 9 elementwise)" % (n + 5))
+    # an expression over several arrays and a scalar feeding the reduction
+    margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),
+                              ElemwiseArg(b"s", GA_FLOAT, 1 | 2))
+    m = 0
+    for op, red, neu, acc in [(0, None, None, GA_FLOAT), (8, None, None, GA_FLOAT),
+                              (14, b"a + b", b"0", GA_DOUBLE), (13, None, None, GA_FLOAT),
+                              (14, b"max(a, b)", b"-INFINITY", GA_HALF)]:
+        d0 = GA_BOOL if op == 13 else acc
+        for G, V, U, mask in [(256, 4, 4, 0b11), (64, 4, 2, 0b01), (256, 1, 4, 0b11)]:
+            check("map-reduce op=%d G=%d V=%d mask=%x" % (op, G, V, mask),
+                  gen_m(op, red, neu, acc, b"", b"s*a*b", 3, margs, d0, G, V, U, mask))
+            m += 1
+    print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, 9 elementwise)"
+          % (n + 5, m))
 
 
 if __name__ == "__main__":

@@ -1114,6 +1114,11 @@ extern "C" char *ga_elemwise_gen_source(const char *preamble, const char *expr, 
                                         unsigned int nd, int idx64, unsigned int tmask);
 extern "C" char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int d1_tc, unsigned int G,
                                          unsigned int V, unsigned int U);
+extern "C" char *ga_mapreduce_gen_source(int op, const char *reduce_expr, const char *neutral,
+                                         int acc_tc, const char *preamble, const char *map_expr,
+                                         unsigned int n, const gpuelemwise_arg *args, int d0_tc,
+                                         unsigned int G, unsigned int V, unsigned int U,
+                                         unsigned int vecmask);
 namespace {
 
 // Numbered timing marks on the context's stream: record as many as wanted
@@ -1155,6 +1160,7 @@ const ext_entry k_exts[] = {
     {"hip_event_elapsed", (void *)ext_event_elapsed},
     {"hip_elemwise_source", (void *)ga_elemwise_gen_source},
     {"hip_reduction_source", (void *)ga_reduction_gen_source},
+    {"hip_mapreduce_source", (void *)ga_mapreduce_gen_source},
 };
 
 }  // namespace

@@ -22,6 +22,7 @@
 #include "private.hpp"
 
 #include <algorithm>
+#include <cctype>
 #include <map>
 #include <mutex>
 #include <string>
@@ -31,15 +32,18 @@ namespace {
 
 constexpr int RD_MAXD = 8;
 
-// Must match `struct rd_plan` in reduce_kernels.h.
+constexpr unsigned RD_MAXSRC = 8;
+
+// Must match `struct rd_plan` in reduce_kernels.h: this fixed part, then the
+// sources' free strides [nsrc][RD_MAXD] and reduced strides [nsrc][RD_MAXD].
 struct rd_plan {
-  int64_t fdim[RD_MAXD], fsstr[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
-  int64_t rdim[RD_MAXD], rsstr[RD_MAXD], rmul[RD_MAXD];
+  int64_t fdim[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
+  int64_t rdim[RD_MAXD], rmul[RD_MAXD];
   int64_t nrows, rtotal, nseg, units, upb, gx;
   int32_t nf, nr, nsplit, pad;
 };
 
-enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL, K_ANY };
+enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL, K_ANY, K_CUSTOM };
 
 bool is_float_type(int tc) { return tc == GA_FLOAT || tc == GA_DOUBLE || tc == GA_HALF; }
 bool is_int_type(int tc) { return tc >= GA_BOOL && tc <= GA_ULONG; }
@@ -73,6 +77,7 @@ bool op_lookup(ga_reduce_op op, op_info *o) {
   case GA_REDUCE_XOR: *o = {K_XOR, true, false}; return true;
   case GA_REDUCE_ALL: *o = {K_ALL, true, false}; return true;
   case GA_REDUCE_ANY: *o = {K_ANY, true, false}; return true;
+  case GA_REDUCE_CUSTOM: *o = {K_CUSTOM, true, false}; return true;
   default: return false;
   }
 }
@@ -114,6 +119,7 @@ std::string neutral_for(rd_kind kind, int acc_tc) {
     case GA_ULONG: return "18446744073709551615ULL";
     default: return "4294967295u";
     }
+  case K_CUSTOM: break;
   }
   return "0";
 }
@@ -124,7 +130,14 @@ struct variant {
 };
 
 struct dimrec {
-  int64_t dim, s, a, b;   // extent, source stride, (d0 stride | index multiplier), d1 stride
+  int64_t dim, s[RD_MAXSRC], a, b;   // extent, source strides, (d0 stride | index multiplier), d1 stride
+  int64_t smax;                      // largest |source stride|: the sort key
+};
+
+struct rd_arg {
+  std::string name;
+  int tc;
+  bool scalar;
 };
 
 inline int64_t iabs(int64_t v) { return v < 0 ? -v : v; }
@@ -135,8 +148,16 @@ struct _GpuReduction {
   gpucontext *ctx;
   ga_reduce_op op;
   op_info info;
-  int src_tc;
+  // Arguments in the caller's order.  A plain reduction has one array
+  // argument and the identity as its expression.
+  std::vector<rd_arg> args;
+  std::vector<unsigned> arrays, scalars;   // positions in args
+  bool mapped = false;        // an expression feeds the reduction
+  int acc_tc = -1;            // mapped: accumulator (= value result) type
+  std::string map_expr, preamble, reduce_expr, neutral;
   std::map<std::string, variant> variants;
+  int src_tc() const { return args[arrays[0]].tc; }
+  unsigned nsrc() const { return (unsigned)arrays.size(); }
 };
 
 int ga_plan_typecode(size_t bytes) {
@@ -153,80 +174,208 @@ int ga_plan_typecode(size_t bytes) {
 
 namespace {
 
-// The #define block that specialises reduce_kernels.h.
-int gen_defines(const op_info &info, int src_tc, int d0_tc, int d1_tc, unsigned G, unsigned V,
-                unsigned U, std::string &s, ga_errrec *errrec, unsigned opts = 3,
-                unsigned ES = 1) {
+// What a variant of the kernels is specialised on besides the operator.
+struct variant_spec {
+  int d0_tc, d1_tc;
+  unsigned G, V, U, opts, ES;
+  unsigned vecmask;   // bit k: array source k is fetched with vector loads
+};
+
+const char *load_type_name(int tc) {
+  return tc == GA_HALF ? "ga_ushort" : gpuarray_get_type(tc)->cluda_name;
+}
+const char *value_type_name(int tc) {
+  return tc == GA_HALF ? "ga_float" : gpuarray_get_type(tc)->cluda_name;
+}
+
+// Accumulator type of the operator for a value result of type d0_tc.
+int acc_typecode(const GpuReduction *gr, int d0_tc) {
+  const rd_kind kind = gr->info.kind;
+  if (gr->mapped) return gr->acc_tc;
+  // min/max compare in the source's type; everything else in the result's
+  return (kind == K_MIN || kind == K_MAX) ? gr->src_tc() : d0_tc;
+}
+
+// The text that specialises reduce_kernels.h: `defs` goes in front of it,
+// `gen` replaces its @RD_GENERATED@ mark.
+int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string &defs,
+                     std::string &gen, ga_errrec *errrec) {
+  const op_info &info = gr->info;
   const rd_kind kind = info.kind;
   const bool minmax = kind == K_MIN || kind == K_MAX;
-  // min/max compare in the source's type; everything else in the result's
-  const int acc_tc = minmax ? src_tc : d0_tc;
-  const char *acc_t = kind == K_ALL || kind == K_ANY ? "ga_uint" : acc_type_for(acc_tc, kind);
+  const int acc_tc = acc_typecode(gr, vs.d0_tc);
+  const char *acc_t;
+  if (kind == K_ALL || kind == K_ANY) acc_t = "ga_uint";
+  else if (kind == K_CUSTOM) acc_t = value_type_name(acc_tc);
+  else acc_t = acc_type_for(acc_tc, kind);
   if (acc_t == nullptr)
     return ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "No accumulator for typecode %d", acc_tc);
-  const bool srcf = is_float_type(src_tc);
+  const bool valf = is_float_type(acc_tc);
   // floating min/max track the index even when it is not returned: the
   // lowest-index rule is what makes -0.0 / +0.0 come out as in a sequential scan
-  const bool arg = info.has_d1 || (minmax && srcf);
-  char line[256];
-#define DEF(...) do { snprintf(line, sizeof(line), __VA_ARGS__); s += line; } while (0)
-  DEF("#define RD_SRC_T %s\n", src_tc == GA_HALF ? "ga_ushort" : gpuarray_get_type(src_tc)->cluda_name);
-  DEF("#define RD_SRC_HALF %d\n", src_tc == GA_HALF ? 1 : 0);
+  const bool arg = info.has_d1 || (minmax && valf);
+  const unsigned K = gr->nsrc();
+  char line[512];
+#define DEF(...) do { snprintf(line, sizeof(line), __VA_ARGS__); defs += line; } while (0)
+  DEF("#define RD_NSRC %u\n", K);
   DEF("#define RD_ACC_T %s\n", acc_t);
-  DEF("#define RD_DST_T %s\n", info.has_d0 ? gpuarray_get_type(d0_tc)->cluda_name : "ga_int");
-  DEF("#define RD_DST_HALF %d\n", info.has_d0 && d0_tc == GA_HALF ? 1 : 0);
-  DEF("#define RD_IDX_T %s\n", info.has_d1 ? gpuarray_get_type(d1_tc)->cluda_name : "ga_long");
+  DEF("#define RD_DST_T %s\n", info.has_d0 ? gpuarray_get_type(vs.d0_tc)->cluda_name : "ga_int");
+  DEF("#define RD_DST_HALF %d\n", info.has_d0 && vs.d0_tc == GA_HALF ? 1 : 0);
+  DEF("#define RD_IDX_T %s\n", info.has_d1 ? gpuarray_get_type(vs.d1_tc)->cluda_name : "ga_long");
   DEF("#define RD_KIND %d\n", (int)kind);
   DEF("#define RD_ARG %d\n", arg ? 1 : 0);
   DEF("#define RD_HAS_D0 %d\n#define RD_HAS_D1 %d\n", info.has_d0 ? 1 : 0, info.has_d1 ? 1 : 0);
-  DEF("#define RD_FLT %d\n", srcf ? 1 : 0);
-  DEF("#define RD_NEUTRAL ((RD_ACC_T)%s)\n",
-      neutral_for(kind, kind == K_ALL || kind == K_ANY ? GA_UINT : acc_tc).c_str());
-  DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", G, V, U);
-  DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n", opts & 1u,
-      (opts >> 1) & 1u, ES);
+  DEF("#define RD_FLT %d\n", valf ? 1 : 0);
+  if (kind == K_CUSTOM) {
+    defs += "#define RD_NEUTRAL ((RD_ACC_T)(" + gr->neutral + "))\n";
+    defs += "#define RD_CUSTOM_OP(a, b) (" + gr->reduce_expr + ")\n";
+  } else {
+    DEF("#define RD_NEUTRAL ((RD_ACC_T)%s)\n",
+        neutral_for(kind, kind == K_ALL || kind == K_ANY ? GA_UINT : acc_tc).c_str());
+  }
+  DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", vs.G, vs.V, vs.U);
+  DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n", vs.opts & 1u,
+      (vs.opts >> 1) & 1u, vs.ES);
 #undef DEF
+
+#define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
+  // kernel parameters and base pointers of the sources
+  gen += "#define RD_SRC_PARAMS ";
+  for (unsigned k = 0; k < K; k++)
+    GEN("%sconst char *__restrict__ rd_s%u, const ga_size rd_s%u_off", k ? ", " : "", k, k);
+  gen += "\n#define RD_SRC_BASES(b) do {";
+  for (unsigned k = 0; k < K; k++) GEN(" (b)[%u] = rd_s%u + rd_s%u_off;", k, k, k);
+  gen += " } while (0)\n";
+  // scalars of the expression
+  std::string sp, sa;
+  for (unsigned i : gr->scalars) {
+    sp += std::string(", const ") + gpuarray_get_type(gr->args[i].tc)->cluda_name + " " + gr->args[i].name;
+    sa += ", " + gr->args[i].name;
+  }
+  gen += "#define RD_SCALAR_PARAMS " + sp + "\n#define RD_SCALAR_FPARAMS " + sp +
+         "\n#define RD_SCALAR_ARGS " + sa + "\n";
+  // registers of one unit / one element
+  std::string unit = "struct rd_unit {", one = "struct rd_one {";
+  for (unsigned k = 0; k < K; k++) {
+    const int tc = gr->args[gr->arrays[k]].tc;
+    const char *lt = load_type_name(tc);
+    if ((vs.vecmask >> k) & 1u) {
+      GEN("typedef %s rd_pvec%u_t __attribute__((ext_vector_type(RD_PV)));\n", lt, k);
+      snprintf(line, sizeof(line), " rd_pvec%u_t x%u[RD_U];", k, k);
+    } else {
+      snprintf(line, sizeof(line), " %s x%u[RD_U][RD_VEC];", lt, k);
+    }
+    unit += line;
+    snprintf(line, sizeof(line), " %s x%u;", lt, k);
+    one += line;
+    // raw loaded bits -> the value the expression sees (half widens to float)
+    if (tc == GA_HALF)
+      GEN("static __device__ inline ga_float rd_w%u(const ga_ushort r) { ga_half h; h.data = r; "
+          "return ga_half2float(h); }\n", k);
+    else
+      GEN("static __device__ inline %s rd_w%u(const %s r) { return r; }\n", lt, k, lt);
+  }
+  gen += unit + " };\n" + one + " };\n";
+  // the expression
+  if (!gr->preamble.empty()) gen += gr->preamble + "\n";
+  gen += "static __device__ inline auto rd_map(";
+  for (unsigned k = 0; k < K; k++) {
+    const rd_arg &a = gr->args[gr->arrays[k]];
+    GEN("%sconst %s %s", k ? ", " : "", value_type_name(a.tc), a.name.c_str());
+  }
+  gen += " RD_SCALAR_FPARAMS) { return (" + gr->map_expr + "); }\n";
+  // loads
+  gen += "static __device__ inline void rd_unit_load(rd_unit &u, const char *const *base, "
+         "ga_long e0, ga_long rin, const ga_long *rstr) {\n"
+         "_Pragma(\"unroll\")\n"
+         "  for (int j = 0; j < RD_U; j++) {\n"
+         "    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;\n"
+         "    if (e < rin) {\n";
+  for (unsigned k = 0; k < K; k++) {
+    const char *lt = load_type_name(gr->args[gr->arrays[k]].tc);
+    if ((vs.vecmask >> k) & 1u)
+      GEN("      u.x%u[j] = RD_LOAD((const rd_pvec%u_t *)(base[%u] + e * rstr[%u]));\n", k, k, k, k);
+    else
+      GEN("_Pragma(\"unroll\")\n      for (int v = 0; v < RD_VEC; v++) u.x%u[j][v] = "
+          "RD_LOAD((const %s *)(base[%u] + (e + v) * rstr[%u]));\n", k, lt, k, k);
+  }
+  gen += "    }\n  }\n}\n#define RD_UNIT_VAL(u, j, v) rd_map(";
+  for (unsigned k = 0; k < K; k++) {
+    if ((vs.vecmask >> k) & 1u) GEN("%srd_w%u((u).x%u[j][(v) * RD_ES])", k ? ", " : "", k, k);
+    else GEN("%srd_w%u((u).x%u[j][v])", k ? ", " : "", k, k);
+  }
+  gen += " RD_SCALAR_ARGS)\n"
+         "static __device__ inline void rd_one_load(rd_one &o, const char *const *p) {\n";
+  for (unsigned k = 0; k < K; k++)
+    GEN("  o.x%u = RD_LOAD((const %s *)p[%u]);\n", k, load_type_name(gr->args[gr->arrays[k]].tc), k);
+  gen += "}\n#define RD_ONE_VAL(o) rd_map(";
+  for (unsigned k = 0; k < K; k++) GEN("%srd_w%u((o).x%u)", k ? ", " : "", k, k);
+  gen += " RD_SCALAR_ARGS)\n";
+#undef GEN
   return GA_NO_ERROR;
 }
 
-int get_variant(GpuReduction *gr, int d0_tc, int d1_tc, unsigned G, unsigned V, unsigned U,
-                unsigned opts, unsigned ES, variant **out) {
+// Whole kernel text of a variant.
+int variant_source(const GpuReduction *gr, const variant_spec &vs, std::string &out,
+                   ga_errrec *errrec) {
+  std::string defs, gen;
+  int err = gen_variant_text(gr, vs, defs, gen, errrec);
+  if (err != GA_NO_ERROR) return err;
+  static const char mark[] = "/*@RD_GENERATED@*/";
+  const char *at = strstr(ga_reduce_kernels_src, mark);
+  if (at == nullptr) return ga_err_set(errrec, GA_IMPL_ERROR, "reduction kernel text has no insertion mark");
+  out = defs;
+  out.append(ga_reduce_kernels_src, (size_t)(at - ga_reduce_kernels_src));
+  out += gen;
+  out += at + sizeof(mark) - 1;
+  return GA_NO_ERROR;
+}
+
+size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * RD_MAXD * sizeof(int64_t); }
+
+int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
-  char key[96];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u", d0_tc, d1_tc, G, V, U, opts, ES);
+  char key[128];
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
+           vs.opts, vs.ES, vs.vecmask);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
     return GA_NO_ERROR;
   }
   std::string s;
-  int herr = gen_defines(gr->info, gr->src_tc, d0_tc, d1_tc, G, V, U, s, ctx->err, opts, ES);
-  if (herr != GA_NO_ERROR) return herr;
-  const char *strs[2] = {s.c_str(), ga_reduce_kernels_src};
-  size_t lens[2] = {s.size(), strlen(ga_reduce_kernels_src)};
-  const int plan_tc = ga_plan_typecode(sizeof(rd_plan));
-  const int types[9] = {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_BUFFER,
-                        GA_SIZE,   GA_BUFFER, GA_BUFFER, plan_tc};
-  const int kflags = gpuarray_type_flags(gr->src_tc, d0_tc, -1);
+  int err = variant_source(gr, vs, s, ctx->err);
+  if (err != GA_NO_ERROR) return err;
+  const char *strs[1] = {s.c_str()};
+  size_t lens[1] = {s.size()};
+  // sources (buffer, offset) ..., d0, d0_off, d1, d1_off, part_v, part_i, plan, scalars ...
+  std::vector<int> types;
+  std::vector<int> flag_types;
+  for (unsigned k = 0; k < gr->nsrc(); k++) {
+    types.push_back(GA_BUFFER);
+    types.push_back(GA_SIZE);
+    flag_types.push_back(gr->args[gr->arrays[k]].tc);
+  }
+  for (int t : {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_BUFFER, GA_BUFFER}) types.push_back(t);
+  types.push_back(ga_plan_typecode(plan_bytes(gr->nsrc())));
+  for (unsigned i : gr->scalars) {
+    types.push_back(gr->args[i].tc);
+    flag_types.push_back(gr->args[i].tc);
+  }
+  flag_types.push_back(vs.d0_tc);
+  if (gr->mapped) flag_types.push_back(gr->acc_tc);
+  int kflags = 0;
+  for (int t : flag_types) kflags |= gpuarray_type_flags(t, -1);
+  const unsigned na = (unsigned)types.size();
   variant v;
-  int err;
-  if ((err = GpuKernel_init(&v.row, ctx, 2, strs, lens, "redux_row", 9, types, kflags, nullptr)) != GA_NO_ERROR)
-    return err;
-  if ((err = GpuKernel_init(&v.col, ctx, 2, strs, lens, "redux_col", 9, types, kflags, nullptr)) != GA_NO_ERROR) {
-    GpuKernel_clear(&v.row);
-    return err;
-  }
-  if ((err = GpuKernel_init(&v.fin, ctx, 2, strs, lens, "redux_final", 9, types, kflags, nullptr)) != GA_NO_ERROR) {
-    GpuKernel_clear(&v.row);
-    GpuKernel_clear(&v.col);
-    return err;
-  }
-  if (G == 64 &&
-      (err = GpuKernel_init(&v.wrows, ctx, 2, strs, lens, "redux_wrows", 9, types, kflags, nullptr)) != GA_NO_ERROR) {
-    GpuKernel_clear(&v.row);
-    GpuKernel_clear(&v.col);
-    GpuKernel_clear(&v.fin);
-    return err;
+  const char *names[4] = {"redux_row", "redux_col", "redux_final", "redux_wrows"};
+  GpuKernel *ks[4] = {&v.row, &v.col, &v.fin, &v.wrows};
+  for (int i = 0; i < (vs.G == 64 ? 4 : 3); i++) {
+    err = GpuKernel_init(ks[i], ctx, 1, strs, lens, names[i], na, types.data(), kflags, nullptr);
+    if (err != GA_NO_ERROR) {
+      for (int j = 0; j < i; j++) GpuKernel_clear(ks[j]);
+      return err;
+    }
   }
   *out = &gr->variants.emplace(key, v).first->second;
   return GA_NO_ERROR;
@@ -234,92 +383,136 @@ int get_variant(GpuReduction *gr, int d0_tc, int d1_tc, unsigned G, unsigned V, 
 
 // Sort slowest-stride first, then fuse neighbours that every listed stride
 // walks as one run.
-void sort_and_fuse(std::vector<dimrec> &v, bool use_b) {
-  std::stable_sort(v.begin(), v.end(),
-                   [](const dimrec &x, const dimrec &y) { return iabs(x.s) > iabs(y.s); });
+void sort_and_fuse(std::vector<dimrec> &v, unsigned nsrc, bool use_b) {
+  for (dimrec &d : v) {
+    d.smax = 0;
+    for (unsigned k = 0; k < nsrc; k++) d.smax = std::max(d.smax, iabs(d.s[k]));
+  }
+  std::stable_sort(v.begin(), v.end(), [](const dimrec &x, const dimrec &y) { return x.smax > y.smax; });
   for (size_t i = v.size(); i-- > 1;) {
     const dimrec &in = v[i];
     dimrec &out = v[i - 1];
-    if (out.s == in.dim * in.s && out.a == in.dim * in.a && (!use_b || out.b == in.dim * in.b)) {
+    bool ok = out.a == in.dim * in.a && (!use_b || out.b == in.dim * in.b);
+    for (unsigned k = 0; ok && k < nsrc; k++) ok = out.s[k] == in.dim * in.s[k];
+    if (ok) {
       out.dim *= in.dim;
-      out.s = in.s;
+      for (unsigned k = 0; k < nsrc; k++) out.s[k] = in.s[k];
       out.a = in.a;
       out.b = in.b;
+      out.smax = in.smax;
       v.erase(v.begin() + (long)i);
     }
   }
 }
 
-}  // namespace
-
-extern "C" {
-
-// Full kernel text of one variant, for checks that have no device.  The
-// caller frees the result.
-GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int d1_tc,
-                                              unsigned int G, unsigned int V, unsigned int U) {
-  op_info info;
-  if (!op_lookup((ga_reduce_op)op, &info)) return nullptr;
-  // bits 8.. of V carry the element step of strided loads (0 means 1)
-  const unsigned ES = (V >> 8) ? (V >> 8) : 1;
-  V &= 0xffu;
-  std::string s;
-  if (gen_defines(info, src_tc, d0_tc, d1_tc, G, V, U, s, ga_global_err, 3, ES) != GA_NO_ERROR)
-    return nullptr;
-  s += ga_reduce_kernels_src;
-  return strdup(s.c_str());
+bool valid_identifier(const char *s) {
+  if (s == nullptr || !(isalpha((unsigned char)*s) || *s == '_')) return false;
+  for (const char *c = s; *c; c++)
+    if (!(isalnum((unsigned char)*c) || *c == '_')) return false;
+  return true;
 }
 
-int GpuReduction_new(GpuReduction **grp, gpucontext *ctx, ga_reduce_op op, unsigned ndf,
-                     unsigned ndr, int s0Typecode, int flags) {
-  (void)ndf; (void)ndr; (void)flags;
-  if (grp == nullptr) return GA_INVALID_ERROR;
-  *grp = nullptr;
-  if (ctx == nullptr) return ga_err_set(ga_global_err, GA_INVALID_ERROR, "GpuReduction_new: no context");
+// Builds an operator without touching a device (shared by the constructors and
+// by the source generators used for build-time checks).
+int make_operator(GpuReduction **grp, gpucontext *ctx, ga_errrec *errrec, ga_reduce_op op,
+                  const char *reduce_expr, const char *neutral, int acc_tc, const char *preamble,
+                  const char *map_expr, unsigned n, const gpuelemwise_arg *args) {
   op_info info;
   if (!op_lookup(op, &info))
-    return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Unknown reduction operation %d", (int)op);
-  if (!is_int_type(s0Typecode) && !is_float_type(s0Typecode))
-    return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Reductions over typecode %d are not supported",
-                      s0Typecode);
-  if ((info.kind == K_AND || info.kind == K_OR || info.kind == K_XOR) && !is_int_type(s0Typecode))
-    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Bitwise reductions need an integer source");
+    return ga_err_fmt(errrec, GA_INVALID_ERROR, "Unknown reduction operation %d", (int)op);
+  if (info.kind == K_CUSTOM && (reduce_expr == nullptr || neutral == nullptr || *reduce_expr == 0 || *neutral == 0))
+    return ga_err_set(errrec, GA_INVALID_ERROR, "A custom reduction needs a combining expression and a neutral element");
+  if (map_expr == nullptr || *map_expr == 0 || n == 0 || args == nullptr)
+    return ga_err_set(errrec, GA_INVALID_ERROR, "A mapped reduction needs an expression and arguments");
+  if (!is_int_type(acc_tc) && !is_float_type(acc_tc))
+    return ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "Accumulator typecode %d is not supported", acc_tc);
+  if ((info.kind == K_AND || info.kind == K_OR || info.kind == K_XOR) && !is_int_type(acc_tc))
+    return ga_err_set(errrec, GA_UNSUPPORTED_ERROR, "Bitwise reductions need an integer accumulator");
   GpuReduction *gr = new (std::nothrow) GpuReduction();
-  if (gr == nullptr) return ga_err_set(ctx->err, GA_MEMORY_ERROR, "Out of memory");
+  if (gr == nullptr) return ga_err_set(errrec, GA_MEMORY_ERROR, "Out of memory");
   gr->ctx = ctx;
   gr->op = op;
   gr->info = info;
-  gr->src_tc = s0Typecode;
+  gr->mapped = true;
+  gr->acc_tc = acc_tc;
+  gr->map_expr = map_expr;
+  gr->preamble = preamble ? preamble : "";
+  gr->reduce_expr = reduce_expr ? reduce_expr : "";
+  gr->neutral = neutral ? neutral : "";
+  int err = GA_NO_ERROR;
+  for (unsigned i = 0; i < n && err == GA_NO_ERROR; i++) {
+    const gpuelemwise_arg &a = args[i];
+    const bool scalar = (a.flags & GE_SCALAR) != 0;
+    if (!valid_identifier(a.name))
+      err = ga_err_fmt(errrec, GA_VALUE_ERROR, "Argument %u has no valid name", i);
+    else if (a.flags & GE_WRITE)
+      err = ga_err_fmt(errrec, GA_VALUE_ERROR, "Argument %s: a reduction only reads its arguments", a.name);
+    else if (!is_int_type(a.typecode) && !is_float_type(a.typecode))
+      err = ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "Argument %s: typecode %d is not supported", a.name, a.typecode);
+    else if (scalar && a.typecode == GA_HALF)
+      err = ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "Argument %s: half scalars are not supported", a.name);
+    for (unsigned j = 0; j < i && err == GA_NO_ERROR; j++)
+      if (gr->args[j].name == a.name)
+        err = ga_err_fmt(errrec, GA_VALUE_ERROR, "Argument name %s is used twice", a.name);
+    if (err != GA_NO_ERROR) break;
+    gr->args.push_back({a.name, a.typecode, scalar});
+    (scalar ? gr->scalars : gr->arrays).push_back(i);
+  }
+  if (err == GA_NO_ERROR && gr->arrays.empty())
+    err = ga_err_set(errrec, GA_VALUE_ERROR, "A reduction needs at least one array argument");
+  if (err == GA_NO_ERROR && gr->arrays.size() > RD_MAXSRC)
+    err = ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "More than %u array arguments", RD_MAXSRC);
+  if (err != GA_NO_ERROR) {
+    delete gr;
+    return err;
+  }
   *grp = gr;
   return GA_NO_ERROR;
 }
 
-void GpuReduction_free(GpuReduction *gr) {
-  if (gr == nullptr) return;
-  for (auto &kv : gr->variants) {
-    GpuKernel_clear(&kv.second.row);
-    GpuKernel_clear(&kv.second.col);
-    GpuKernel_clear(&kv.second.fin);
-    if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
-  }
-  delete gr;
+int make_plain_operator(GpuReduction **grp, gpucontext *ctx, ga_errrec *errrec, ga_reduce_op op,
+                        int s0Typecode) {
+  op_info info;
+  if (!op_lookup(op, &info) || info.kind == K_CUSTOM)
+    return ga_err_fmt(errrec, GA_INVALID_ERROR, "Unknown reduction operation %d", (int)op);
+  if (!is_int_type(s0Typecode) && !is_float_type(s0Typecode))
+    return ga_err_fmt(errrec, GA_UNSUPPORTED_ERROR, "Reductions over typecode %d are not supported",
+                      s0Typecode);
+  if ((info.kind == K_AND || info.kind == K_OR || info.kind == K_XOR) && !is_int_type(s0Typecode))
+    return ga_err_set(errrec, GA_UNSUPPORTED_ERROR, "Bitwise reductions need an integer source");
+  GpuReduction *gr = new (std::nothrow) GpuReduction();
+  if (gr == nullptr) return ga_err_set(errrec, GA_MEMORY_ERROR, "Out of memory");
+  gr->ctx = ctx;
+  gr->op = op;
+  gr->info = info;
+  gr->args.push_back({"x", s0Typecode, false});
+  gr->arrays.push_back(0);
+  gr->map_expr = "x";
+  *grp = gr;
+  return GA_NO_ERROR;
 }
 
-int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const GpuArray *s0,
-                      unsigned reduxLen, const int *reduxList, int flags) {
-  (void)flags;
-  GpuReduction *gr = const_cast<GpuReduction *>(cgr);
-  if (gr == nullptr || s0 == nullptr) return GA_INVALID_ERROR;
+// The launch: checks, plan, kernels.  `srcs` are the array arguments with the
+// strides to use (broadcast dims already have stride 0) over the common
+// extents `dims`; `scalars` point at host values of the declared types.
+struct src_view {
+  const GpuArray *a;
+  std::vector<int64_t> strides;
+};
+
+int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
+                  const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
+                  unsigned reduxLen, const int *reduxList) {
   gpucontext *ctx = gr->ctx;
   const op_info &info = gr->info;
+  const unsigned K = gr->nsrc();
   if ((info.has_d0 && d0 == nullptr) || (info.has_d1 && d1 == nullptr))
     return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array required by the operation is NULL");
   if (!info.has_d0) d0 = nullptr;
   if (!info.has_d1) d1 = nullptr;
-  if (s0->nd == 0 || reduxLen == 0 || reduxLen > s0->nd || reduxList == nullptr)
+  if (nd == 0 || reduxLen == 0 || reduxLen > nd || reduxList == nullptr)
     return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
-                      "Invalid reduction: source nd = %u, %u axes to reduce", s0->nd, reduxLen);
-  const unsigned nd = s0->nd;
+                      "Invalid reduction: source nd = %u, %u axes to reduce", nd, reduxLen);
   std::vector<char> reduced(nd, 0);
   for (unsigned i = 0; i < reduxLen; i++) {
     const int ax = reduxList[i];
@@ -327,23 +520,32 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
       return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Reduction axis %d is out of range or repeated", ax);
     reduced[ax] = 1;
   }
-  if (s0->typecode != gr->src_tc)
-    return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Source has typecode %d, operator was made for %d",
-                      s0->typecode, gr->src_tc);
-  if (GpuArray_context(s0) != ctx || (d0 && GpuArray_context(d0) != ctx) ||
-      (d1 && GpuArray_context(d1) != ctx))
+  for (unsigned k = 0; k < K; k++) {
+    const GpuArray *s = srcs[k].a;
+    const int want = gr->args[gr->arrays[k]].tc;
+    if (s->typecode != want)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Source has typecode %d, operator was made for %d",
+                        s->typecode, want);
+    if (GpuArray_context(s) != ctx)
+      return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
+  }
+  if ((d0 && GpuArray_context(d0) != ctx) || (d1 && GpuArray_context(d1) != ctx))
     return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
 
   // result types
   const rd_kind kind = info.kind;
   const bool minmax = kind == K_MIN || kind == K_MAX;
-  int d0_tc = d0 ? d0->typecode : gr->src_tc, d1_tc = d1 ? d1->typecode : GA_LONG;
+  const bool logical = kind == K_ALL || kind == K_ANY;
+  int d0_tc = d0 ? d0->typecode : (gr->mapped ? gr->acc_tc : gr->src_tc());
+  const int d1_tc = d1 ? d1->typecode : GA_LONG;
   if (d0) {
     if (!GpuArray_ISWRITEABLE(d0)) return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination not writeable");
-    if (minmax && d0_tc != gr->src_tc)
+    if (gr->mapped && !logical && d0_tc != gr->acc_tc)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                        "Result has typecode %d, the operator accumulates in %d", d0_tc, gr->acc_tc);
+    if (!gr->mapped && minmax && d0_tc != gr->src_tc())
       return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max results must have the source's type");
-    if ((kind == K_AND || kind == K_OR || kind == K_XOR || kind == K_ALL || kind == K_ANY) &&
-        !is_int_type(d0_tc))
+    if ((kind == K_AND || kind == K_OR || kind == K_XOR || logical) && !is_int_type(d0_tc))
       return ga_err_set(ctx->err, GA_VALUE_ERROR, "Result of a logical/bitwise reduction must be an integer type");
     if (!is_int_type(d0_tc) && !is_float_type(d0_tc))
       return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Result typecode %d is not supported", d0_tc);
@@ -363,10 +565,10 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     unsigned k = 0;
     for (unsigned ax = 0; ax < nd; ax++) {
       if (reduced[ax]) continue;
-      if (d->dimensions[k] != s0->dimensions[ax])
+      if (d->dimensions[k] != dims[ax])
         return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
                           "Destination dimension %u is %zu, source axis %u is %zu", k,
-                          d->dimensions[k], ax, s0->dimensions[ax]);
+                          d->dimensions[k], ax, dims[ax]);
       k++;
     }
   }
@@ -378,19 +580,32 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     unsigned k = 0;
     for (unsigned ax = 0; ax < nd; ax++) {
       if (reduced[ax]) continue;
-      const int64_t dim = (int64_t)s0->dimensions[ax];
+      const int64_t dim = (int64_t)dims[ax];
       nrows *= dim;
-      if (dim != 1)
-        fr.push_back({dim, (int64_t)s0->strides[ax], d0 ? (int64_t)d0->strides[k] : 0,
-                      d1 ? (int64_t)d1->strides[k] : 0});
+      if (dim != 1) {
+        dimrec r;
+        memset(&r, 0, sizeof(r));
+        r.dim = dim;
+        for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
+        r.a = d0 ? (int64_t)d0->strides[k] : 0;
+        r.b = d1 ? (int64_t)d1->strides[k] : 0;
+        fr.push_back(r);
+      }
       k++;
     }
     int64_t mul = 1;
     for (unsigned i = reduxLen; i-- > 0;) {
       const int ax = reduxList[i];
-      const int64_t dim = (int64_t)s0->dimensions[ax];
+      const int64_t dim = (int64_t)dims[ax];
       rtotal *= dim;
-      if (dim != 1) rd.insert(rd.begin(), {dim, (int64_t)s0->strides[ax], mul, 0});
+      if (dim != 1) {
+        dimrec r;
+        memset(&r, 0, sizeof(r));
+        r.dim = dim;
+        for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
+        r.a = mul;
+        rd.insert(rd.begin(), r);
+      }
       mul *= dim;
     }
   }
@@ -398,35 +613,46 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
   if (rtotal == 0 && minmax)
     return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max over an empty axis has no value");
   if (rtotal == 0) rd.clear();
-  sort_and_fuse(fr, true);
-  sort_and_fuse(rd, false);
+  sort_and_fuse(fr, K, true);
+  sort_and_fuse(rd, K, false);
   if (fr.size() > (size_t)RD_MAXD || rd.size() > (size_t)RD_MAXD)
     return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR,
                       "More than %d non-mergeable free or reduced dimensions", RD_MAXD);
 
-  rd_plan p;
-  memset(&p, 0, sizeof(p));
+  // plan = fixed part + per-source stride tables
+  std::vector<int64_t> planbuf(plan_bytes(K) / sizeof(int64_t), 0);
+  rd_plan &p = *reinterpret_cast<rd_plan *>(planbuf.data());
+  int64_t *fsstr = planbuf.data() + sizeof(rd_plan) / sizeof(int64_t);   // [K][RD_MAXD]
+  int64_t *rsstr = fsstr + (size_t)K * RD_MAXD;                           // [K][RD_MAXD]
   p.nf = (int)fr.size();
   p.nr = (int)rd.size();
   for (int i = 0; i < p.nf; i++) {
-    p.fdim[i] = fr[i].dim; p.fsstr[i] = fr[i].s; p.fd0str[i] = fr[i].a; p.fd1str[i] = fr[i].b;
+    p.fdim[i] = fr[i].dim; p.fd0str[i] = fr[i].a; p.fd1str[i] = fr[i].b;
+    for (unsigned q = 0; q < K; q++) fsstr[q * RD_MAXD + i] = fr[i].s[q];
   }
   for (int i = 0; i < p.nr; i++) {
-    p.rdim[i] = rd[i].dim; p.rsstr[i] = rd[i].s; p.rmul[i] = rd[i].a;
+    p.rdim[i] = rd[i].dim; p.rmul[i] = rd[i].a;
+    for (unsigned q = 0; q < K; q++) rsstr[q * RD_MAXD + i] = rd[i].s[q];
   }
   p.nrows = nrows;
   p.rtotal = rtotal;
   p.nsplit = 1;
 
-  const int64_t elsz = (int64_t)gpuarray_get_elsize(gr->src_tc);
+  int64_t elsz_max = 0, elsz_sum = 0;
+  std::vector<int64_t> elsz(K);
+  for (unsigned q = 0; q < K; q++) {
+    elsz[q] = (int64_t)gpuarray_get_elsize(gr->args[gr->arrays[q]].tc);
+    elsz_max = std::max(elsz_max, elsz[q]);
+    elsz_sum += elsz[q];
+  }
   const int64_t ncu = (int64_t)ga_hip_numprocs(ctx);
   const int64_t rin = p.nr ? p.rdim[p.nr - 1] : 1;
-  const int64_t rstr = p.nr ? iabs(p.rsstr[p.nr - 1]) : 0;
-  const int64_t fstr = p.nf ? iabs(p.fsstr[p.nf - 1]) : INT64_MAX;
+  const int64_t rstr = p.nr ? rd[p.nr - 1].smax : 0;
+  const int64_t fstr = p.nf ? fr[p.nf - 1].smax : INT64_MAX;
 
   // Lanes along the reduced run unless the free run is the one that is
   // contiguous in memory (or the reduced run is too short to feed a wavefront).
-  bool use_row = p.nf == 0 || (rstr <= fstr && rin >= 32) || (rin >= 4096 && rstr <= 4 * elsz);
+  bool use_row = p.nf == 0 || (rstr <= fstr && rin >= 32) || (rin >= 4096 && rstr <= 4 * elsz_max);
   if (rtotal == 0) use_row = true;
   {
     const char *force = getenv("GPUARRAY_REDUX_FAMILY");
@@ -434,36 +660,54 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1;
   bool wrows = false;
   size_t groups;
   if (use_row) {
-    // Widest aligned load the layout allows.  The inner reduced dim may step
-    // by ES = 1, 2 or 4 elements (a [::2] / [::4] view): a load then fetches
-    // V*ES contiguous elements and uses every ES-th one.  Such a load reads up
-    // to ES-1 elements past the last one used, so it must stay inside the
-    // buffer.
-    if (p.nr && rtotal > 0 && p.rsstr[p.nr - 1] > 0 && p.rsstr[p.nr - 1] % elsz == 0) {
-      const int64_t es = p.rsstr[p.nr - 1] / elsz;
+    // Widest aligned load the layout allows, for a source whose inner reduced
+    // stride is its element size: v elements, v*elsz bytes, everything the
+    // lane's address is built from a multiple of that.
+    auto fits = [&](unsigned q, unsigned v, int64_t es) {
+      const GpuArray *s0 = srcs[q].a;
+      const int64_t bytes = (int64_t)v * es * elsz[q];
+      const uintptr_t base = (uintptr_t)s0->data->devptr + s0->offset;
+      bool ok = rin % v == 0 && base % (uintptr_t)bytes == 0;
+      for (int i = 0; ok && i < p.nf; i++) ok = fsstr[q * RD_MAXD + i] % bytes == 0;
+      for (int i = 0; ok && i + 1 < p.nr; i++) ok = rsstr[q * RD_MAXD + i] % bytes == 0;
+      return ok;
+    };
+    if (K == 1 && p.nr && rtotal > 0 && rsstr[p.nr - 1] > 0 && rsstr[p.nr - 1] % elsz[0] == 0) {
+      // One source: its inner reduced dim may also step by ES = 2 or 4
+      // elements (a [::2] / [::4] view): a load then fetches V*ES contiguous
+      // elements and uses every ES-th one.  Such a load reads up to ES-1
+      // elements past the last one used, so it must stay inside the buffer.
+      const GpuArray *s0 = srcs[0].a;
+      const int64_t es = rsstr[p.nr - 1] / elsz[0];
       if (es == 1 || es == 2 || es == 4) {
-        unsigned v = (unsigned)(16 / (elsz * es));
-        const uintptr_t base = (uintptr_t)s0->data->devptr + s0->offset;
+        unsigned v = (unsigned)(16 / (elsz[0] * es));
         size_t bufsz = 0;
         gpudata_property(s0->data, GA_BUFFER_PROP_SIZE, &bufsz);
         int64_t last = (int64_t)s0->offset;   // byte offset of the farthest element
-        for (int i = 0; i < p.nf; i++) if (p.fsstr[i] > 0) last += (p.fdim[i] - 1) * p.fsstr[i];
-        for (int i = 0; i < p.nr; i++) if (p.rsstr[i] > 0) last += (p.rdim[i] - 1) * p.rsstr[i];
-        const bool overread_ok = es == 1 || (size_t)(last + es * elsz) <= bufsz;
-        while (v > 1) {
-          const int64_t bytes = (int64_t)v * es * elsz;
-          bool ok = overread_ok && rin % v == 0 && base % (uintptr_t)bytes == 0;
-          for (int i = 0; ok && i < p.nf; i++) ok = p.fsstr[i] % bytes == 0;
-          for (int i = 0; ok && i + 1 < p.nr; i++) ok = p.rsstr[i] % bytes == 0;
-          if (ok) break;
-          v /= 2;
-        }
+        for (int i = 0; i < p.nf; i++) if (fsstr[i] > 0) last += (p.fdim[i] - 1) * fsstr[i];
+        for (int i = 0; i < p.nr; i++) if (rsstr[i] > 0) last += (p.rdim[i] - 1) * rsstr[i];
+        const bool overread_ok = es == 1 || (size_t)(last + es * elsz[0]) <= bufsz;
+        while (v > 1 && !(overread_ok && fits(0, v, es))) v /= 2;
         V = v;
         if (V > 1) ES = (unsigned)es;
+      }
+    } else if (K > 1 && p.nr && rtotal > 0) {
+      // Several sources: the widest type gets 16-byte loads when every source
+      // that is contiguous along the inner reduced dim is aligned for its
+      // share; sources with another stride there (0 for a broadcast one) are
+      // fetched element by element.
+      unsigned v = (unsigned)(16 / elsz_max), unit_mask = 0;
+      for (unsigned q = 0; q < K; q++)
+        if (rsstr[q * RD_MAXD + p.nr - 1] == elsz[q]) unit_mask |= 1u << q;
+      if (unit_mask != 0) {
+        for (unsigned q = 0; q < K; q++)
+          while (v > 1 && ((unit_mask >> q) & 1u) && !fits(q, v, 1)) v /= 2;
+        V = v;
+        if (V > 1) vecmask = unit_mask;
       }
     }
     // One wavefront per output when eight loads per lane cover the inner
@@ -478,6 +722,8 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     int64_t per_pass = (int64_t)G * V;
     U = (unsigned)env_ul("GPUARRAY_REDUX_U", 8);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 8;
+    // several sources share the lane's registers
+    while (U > 1 && (int64_t)U * V * ES * elsz_sum > 128) U /= 2;
     while (U > 1 && per_pass * (U / 2) >= rin) U /= 2;
     const int64_t seg = per_pass * U;
     p.nseg = rin > 0 ? (rin + seg - 1) / seg : 1;
@@ -497,7 +743,7 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     // bytes per lane, so they get proportionally more groups, up to 32.
     int64_t per_cu = (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 0);
     if (per_cu == 0) {
-      const int64_t inflight = (int64_t)G * U * V * ES * elsz;   // bytes per group
+      const int64_t inflight = (int64_t)G * U * V * ES * elsz_sum;   // bytes per group
       per_cu = (65536 + inflight - 1) / inflight;
       if (per_cu < 2) per_cu = 2;
       if (per_cu > 32) per_cu = 32;
@@ -551,41 +797,188 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
   // bit 0: streaming loads; bit 1: interleaved splits (single reduced dim only)
   unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
   if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
+  variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
+                     use_row ? vecmask : (1u << K) - 1};
   variant *var = nullptr;
-  int err = get_variant(gr, d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts,
-                        use_row ? ES : 1, &var);
+  int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
 
   // partials of a split reduction live in the context's scratch buffer:
   // values first, indices after, both 8-byte aligned
-  const size_t accsz = (kind == K_ALL || kind == K_ANY) ? 4 : acc_size_for(minmax ? gr->src_tc : d0_tc);
+  const int acc_tc = acc_typecode(gr, d0_tc);
+  const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
   gpudata *scratch = ga_hip_scratch(ctx, 16);
-  size_t pv_off = 0, pi_off = 0;
+  size_t pi_off = 0;
   if (p.nsplit > 1) {
     const size_t slots = (size_t)nrows * (size_t)p.nsplit;
     pi_off = (slots * accsz + 255) & ~(size_t)255;
     scratch = ga_hip_scratch(ctx, pi_off + slots * 8);
   }
   if (scratch == nullptr) return ctx->err->code;
-  (void)pv_off;
 
   // A destination the operation does not write still needs a valid pointer.
   gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
-  size_t s_off = s0->offset, d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
+  size_t d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
+  std::vector<size_t> s_off(K);
 
   // The two scratch views are passed as (buffer) arguments; the index part
   // starts pi_off bytes in, which the kernels receive through a second
   // gpudata wrapping the same memory.
   struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + pi_off, ctx};
-  void *args[9] = {s0->data, &s_off, d0b, &d0_off, d1b, &d1_off, scratch, &pi_view, &p};
+  std::vector<void *> args;
+  for (unsigned q = 0; q < K; q++) {
+    s_off[q] = srcs[q].a->offset;
+    args.push_back(srcs[q].a->data);
+    args.push_back(&s_off[q]);
+  }
+  args.push_back(d0b);
+  args.push_back(&d0_off);
+  args.push_back(d1b);
+  args.push_back(&d1_off);
+  args.push_back(scratch);
+  args.push_back(&pi_view);
+  args.push_back(planbuf.data());
+  for (void *sc : scalars) args.push_back(sc);
   size_t ls = 256;
   GpuKernel *k1 = use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
-  if ((err = GpuKernel_call(k1, 1, &groups, &ls, 0, args)) != GA_NO_ERROR) return err;
+  if ((err = GpuKernel_call(k1, 1, &groups, &ls, 0, args.data())) != GA_NO_ERROR) return err;
   if (p.nsplit > 1) {
     size_t fg = (size_t)((nrows + 3) / 4);
-    if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args)) != GA_NO_ERROR) return err;
+    if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args.data())) != GA_NO_ERROR) return err;
   }
   return GA_NO_ERROR;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Full kernel text of one variant, for checks that have no device.  The
+// caller frees the result.
+GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int d1_tc,
+                                              unsigned int G, unsigned int V, unsigned int U) {
+  GpuReduction *gr = nullptr;
+  if (make_plain_operator(&gr, nullptr, ga_global_err, (ga_reduce_op)op, src_tc) != GA_NO_ERROR)
+    return nullptr;
+  // bits 8.. of V carry the element step of strided loads (0 means 1)
+  const unsigned ES = (V >> 8) ? (V >> 8) : 1;
+  V &= 0xffu;
+  std::string s;
+  variant_spec vs = {d0_tc, d1_tc, G, V, U, 3, ES, 1};
+  const int err = variant_source(gr, vs, s, ga_global_err);
+  delete gr;
+  return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
+}
+
+// The same for an operator with an expression; vecmask as in variant_spec.
+GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, const char *neutral,
+                                              int acc_tc, const char *preamble, const char *map_expr,
+                                              unsigned int n, const gpuelemwise_arg *args, int d0_tc,
+                                              unsigned int G, unsigned int V, unsigned int U,
+                                              unsigned int vecmask) {
+  GpuReduction *gr = nullptr;
+  if (make_operator(&gr, nullptr, ga_global_err, (ga_reduce_op)op, reduce_expr, neutral, acc_tc,
+                    preamble, map_expr, n, args) != GA_NO_ERROR)
+    return nullptr;
+  std::string s;
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask};
+  const int err = variant_source(gr, vs, s, ga_global_err);
+  delete gr;
+  return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
+}
+
+int GpuReduction_new(GpuReduction **grp, gpucontext *ctx, ga_reduce_op op, unsigned ndf,
+                     unsigned ndr, int s0Typecode, int flags) {
+  (void)ndf; (void)ndr; (void)flags;
+  if (grp == nullptr) return GA_INVALID_ERROR;
+  *grp = nullptr;
+  if (ctx == nullptr) return ga_err_set(ga_global_err, GA_INVALID_ERROR, "GpuReduction_new: no context");
+  return make_plain_operator(grp, ctx, ctx->err, op, s0Typecode);
+}
+
+int GpuReduction_new_map(GpuReduction **grp, gpucontext *ctx, ga_reduce_op op,
+                         const char *reduce_expr, const char *neutral, int accTypecode,
+                         const char *preamble, const char *map_expr, unsigned int n,
+                         const gpuelemwise_arg *args, int flags) {
+  (void)flags;
+  if (grp == nullptr) return GA_INVALID_ERROR;
+  *grp = nullptr;
+  if (ctx == nullptr)
+    return ga_err_set(ga_global_err, GA_INVALID_ERROR, "GpuReduction_new_map: no context");
+  return make_operator(grp, ctx, ctx->err, op, reduce_expr, neutral, accTypecode, preamble,
+                       map_expr, n, args);
+}
+
+void GpuReduction_free(GpuReduction *gr) {
+  if (gr == nullptr) return;
+  for (auto &kv : gr->variants) {
+    GpuKernel_clear(&kv.second.row);
+    GpuKernel_clear(&kv.second.col);
+    GpuKernel_clear(&kv.second.fin);
+    if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
+  }
+  delete gr;
+}
+
+int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const GpuArray *s0,
+                      unsigned reduxLen, const int *reduxList, int flags) {
+  (void)flags;
+  GpuReduction *gr = const_cast<GpuReduction *>(cgr);
+  if (gr == nullptr || s0 == nullptr) return GA_INVALID_ERROR;
+  if (gr->nsrc() != 1 || !gr->scalars.empty())
+    return ga_err_set(gr->ctx->err, GA_INVALID_ERROR,
+                      "This operator takes several arguments: use GpuReduction_call_map");
+  std::vector<src_view> srcs(1);
+  srcs[0].a = s0;
+  srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);
+  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, srcs, {}, reduxLen, reduxList);
+}
+
+int GpuReduction_call_map(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, void **args,
+                          unsigned reduxLen, const int *reduxList, int flags) {
+  GpuReduction *gr = const_cast<GpuReduction *>(cgr);
+  if (gr == nullptr || args == nullptr) return GA_INVALID_ERROR;
+  gpucontext *ctx = gr->ctx;
+  const unsigned K = gr->nsrc();
+  std::vector<src_view> srcs(K);
+  std::vector<void *> scalars;
+  for (unsigned i : gr->scalars) {
+    if (args[i] == nullptr) return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Argument %u is NULL", i);
+    scalars.push_back(args[i]);
+  }
+  unsigned nd = 0;
+  for (unsigned q = 0; q < K; q++) {
+    const GpuArray *a = (const GpuArray *)args[gr->arrays[q]];
+    if (a == nullptr) return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Argument %u is NULL", gr->arrays[q]);
+    if (q == 0) nd = a->nd;
+    else if (a->nd != nd)
+      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Argument %u has nd = %u, the first array %u",
+                        gr->arrays[q], a->nd, nd);
+    srcs[q].a = a;
+  }
+  // common extents; an extent of 1 stretches when broadcasting is allowed
+  // (the rule of GpuElemwise_call, reference src/gpuarray_elemwise.c:272-383)
+  std::vector<size_t> dims(nd ? nd : 1, 1);
+  for (unsigned ax = 0; ax < nd; ax++) {
+    size_t d = srcs[0].a->dimensions[ax];
+    for (unsigned q = 1; q < K; q++) {
+      const size_t dq = srcs[q].a->dimensions[ax];
+      if (dq == d) continue;
+      if ((flags & GE_BROADCAST) && d == 1) d = dq;
+      else if (!((flags & GE_BROADCAST) && dq == 1))
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                          "Mismatched dimension %u: argument %u has %zu, expected %zu", ax,
+                          gr->arrays[q], dq, d);
+    }
+    dims[ax] = d;
+  }
+  for (unsigned q = 0; q < K; q++) {
+    const GpuArray *a = srcs[q].a;
+    srcs[q].strides.resize(nd);
+    for (unsigned ax = 0; ax < nd; ax++)
+      srcs[q].strides[ax] = a->dimensions[ax] == dims[ax] ? (int64_t)a->strides[ax] : 0;
+  }
+  return reduce_launch(gr, d0, d1, nd, dims.data(), srcs, scalars, reduxLen, reduxList);
 }
 
 // Reference entry point (src/gpuarray_reduction.c:100-124).  The operator is

@@ -3,13 +3,17 @@
  * This text is compiled at run time behind a short list of #defines that the
  * host planner emits (element types, operation, lane geometry):
  *
- *   RD_SRC_T    source element type        RD_SRC_HALF  source is ga_half
+ *   RD_NSRC     number of source arrays (1 for a plain reduction; more when
+ *               an elementwise expression over several arrays feeds the
+ *               reduction)
  *   RD_ACC_T    accumulator type           RD_KIND      operation, RD_K_* below
  *   RD_DST_T    value result type          RD_DST_HALF  value result is ga_half
  *   RD_IDX_T    index result type          RD_ARG       carry (value, index)
  *   RD_HAS_D0 / RD_HAS_D1                  which results are written
  *   RD_NEUTRAL  neutral element of the operation, of type RD_ACC_T
- *   RD_FLT      source is a floating type (NaN rules apply)
+ *   RD_FLT      the reduced values are floating (NaN rules apply)
+ *   RD_CUSTOM_OP(a, b) / RD_NEUTRAL  the caller's combination and its neutral
+ *               element when RD_KIND is RD_K_CUSTOM
  *   RD_G        lanes that share one output in redux_row: 64 or 256
  *   RD_VEC      elements per load in redux_row (inner reduced stride is the
  *               element size and everything is aligned when > 1)
@@ -21,6 +25,12 @@
  *   RD_NT       streaming (non-temporal) loads in redux_row
  *   RD_INTERLEAVE  redux_row with one reduced dim: splits take every
  *               nsplit-th unit instead of a contiguous range
+ *
+ * and, also emitted by the planner, the part that depends on the number and
+ * types of the sources (inserted at the @RD_GENERATED@ mark below): the kernels' source
+ * parameters, the registers of one lane's loads (rd_unit, rd_one), how they
+ * are filled, and the value computed from them (the source element itself, or
+ * the caller's expression over the elements of all sources).
  *
  * Semantics (reference src/gpuarray_reduction.c:545-607 for max/argmax,
  * pygpu/reduction.py:33-134 for sum/prod/any/all):
@@ -63,6 +73,7 @@
 #define RD_K_XOR 7
 #define RD_K_ALL 8
 #define RD_K_ANY 9
+#define RD_K_CUSTOM 10
 
 #define RD_MAXD 8
 
@@ -70,8 +81,8 @@
  * Strides are in bytes.  `rmul` is what one step along a reduced dim adds to
  * the flattened index. */
 struct rd_plan {
-  ga_long fdim[RD_MAXD], fsstr[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
-  ga_long rdim[RD_MAXD], rsstr[RD_MAXD], rmul[RD_MAXD];
+  ga_long fdim[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
+  ga_long rdim[RD_MAXD], rmul[RD_MAXD];
   ga_long nrows;   /* number of outputs */
   ga_long rtotal;  /* elements reduced per output */
   ga_long nseg;    /* redux_row: segments per pass over the inner reduced dim */
@@ -79,6 +90,7 @@ struct rd_plan {
   ga_long upb;     /* work per split: units (row) or elements (col) */
   ga_long gx;      /* redux_col: groups along the inner free dim */
   ga_int nf, nr, nsplit, pad;
+  ga_long fsstr[RD_NSRC][RD_MAXD], rsstr[RD_NSRC][RD_MAXD];   /* per source */
 };
 
 struct rd_acc {
@@ -114,6 +126,8 @@ static __device__ inline rd_acc rd_combine(rd_acc a, rd_acc b) {
   a.v = (a.v && b.v) ? 1 : 0;
 #elif RD_KIND == RD_K_ANY
   a.v = (a.v || b.v) ? 1 : 0;
+#elif RD_KIND == RD_K_CUSTOM
+  a.v = (RD_ACC_T)RD_CUSTOM_OP(a.v, b.v);
 #elif RD_KIND == RD_K_MAX
 #if RD_ARG
   if (b.v > a.v || (b.v == a.v && b.i < a.i)) a = b;
@@ -130,22 +144,11 @@ static __device__ inline rd_acc rd_combine(rd_acc a, rd_acc b) {
   return a;
 }
 
-/* A half source is loaded as its 16 raw bits (RD_SRC_T is ga_ushort then) and
- * widened to float here; every other type is used as it is. */
-#if RD_SRC_HALF
-static __device__ inline float rd_src_val(const RD_SRC_T raw) {
-  ga_half h;
-  h.data = raw;
-  return ga_half2float(h);
-}
-#else
-static __device__ inline RD_SRC_T rd_src_val(const RD_SRC_T raw) { return raw; }
-#endif
-
-/* One source element, converted for the operation. */
-static __device__ inline rd_acc rd_elem(const RD_SRC_T x_in, ga_long idx) {
+/* One reduced value (a source element, or the caller's expression over the
+ * sources' elements), converted for the operation. */
+template <typename T>
+static __device__ inline rd_acc rd_elem(const T x, ga_long idx) {
   rd_acc a;
-  const auto x = rd_src_val(x_in);
 #if RD_KIND == RD_K_ALL || RD_KIND == RD_K_ANY
   a.v = (x != 0) ? 1 : 0;
 #elif RD_KIND == RD_K_PRODNZ
@@ -227,43 +230,80 @@ static __device__ inline rd_acc rd_block_reduce(rd_acc a, rd_acc *lds) {
 
 /* ---- addressing ------------------------------------------------------------ */
 
-/* Offsets of output `row` (flat index over the free dims, slowest first). */
+/* Offsets of output `row` (flat index over the free dims, slowest first):
+ * one per source, and the two destinations'. */
 static __device__ inline void rd_row_offsets(const rd_plan &p, ga_long row, ga_long *so,
                                              ga_long *d0o, ga_long *d1o) {
-  ga_long s = 0, a = 0, b = 0;
+  ga_long a = 0, b = 0;
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) so[k] = 0;
   for (int d = p.nf - 1; d >= 0; d--) {
     ga_long c;
     if (d > 0) { c = row % p.fdim[d]; row = row / p.fdim[d]; } else { c = row; }
-    s += c * p.fsstr[d];
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) so[k] += c * p.fsstr[k][d];
     a += c * p.fd0str[d];
     b += c * p.fd1str[d];
   }
-  *so = s; *d0o = a; *d1o = b;
+  *d0o = a; *d1o = b;
 }
 
-/* Byte offset and index base of outer reduced coordinate `ro` (flat over the
- * reduced dims 0..ri-1). */
+/* Byte offsets (per source) and index base of outer reduced coordinate `ro`
+ * (flat over the reduced dims 0..ri-1). */
 static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long ro, ga_long *rb,
                                                ga_long *ib) {
-  ga_long b = 0, x = 0;
+  ga_long x = 0;
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) rb[k] = 0;
   for (int d = ri - 1; d >= 0; d--) {
     ga_long c;
     if (d > 0) { c = ro % p.rdim[d]; ro = ro / p.rdim[d]; } else { c = ro; }
-    b += c * p.rsstr[d];
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) rb[k] += c * p.rsstr[k][d];
     x += c * p.rmul[d];
   }
-  *rb = b; *ib = x;
+  *ib = x;
 }
 
+/* ---- the part that depends on the sources ------------------------------------
+ * Emitted by the planner:
+ *   RD_SRC_PARAMS            kernel parameters: (pointer, byte offset) per source
+ *   RD_SRC_BASES(b)          b[k] = pointer + offset, for every source
+ *   RD_SCALAR_PARAMS / RD_SCALAR_FPARAMS / RD_SCALAR_ARGS
+ *                            scalar arguments of the caller's expression as
+ *                            trailing kernel parameters, function parameters
+ *                            and call arguments (all empty when there are none)
+ *   struct rd_unit           what one lane fetches for one unit: per source
+ *                            RD_U vector loads, or RD_U x RD_VEC scalar loads
+ *                            when its inner reduced stride is not its element
+ *                            size
+ *   rd_unit_load(u, base, e0, rin, rstr)   fill it (loads past `rin` skipped)
+ *   RD_UNIT_VAL(u, j, v)     the reduced value of element v of load j
+ *   struct rd_one, rd_one_load(o, ptrs), RD_ONE_VAL(o)   the same for one
+ *                            element addressed by one pointer per source
+ * RD_PV (elements per vector load) and RD_LOAD are defined first because the
+ * emitted text uses them. */
+#define RD_PV (RD_VEC * RD_ES)
+/* every source element is read once: stream it past the caches */
+#if RD_NT
+#define RD_LOAD(p) __builtin_nontemporal_load(p)
+#else
+#define RD_LOAD(p) (*(p))
+#endif
+
+/*@RD_GENERATED@*/
+
 /* Write the finished value(s) of one output. */
-static __device__ inline void rd_store(rd_acc a, const char *srow, char *d0, ga_long d0o, char *d1,
-                                       ga_long d1o, ga_long rtotal) {
+static __device__ inline void rd_store(rd_acc a, const char *const *srow, char *d0, ga_long d0o,
+                                       char *d1, ga_long d1o, ga_long rtotal RD_SCALAR_FPARAMS) {
 #if RD_FLT && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN)
   /* a NaN in the first position of the scan stays (see the header) */
   if (rtotal > 0) {
-    const auto first = rd_src_val(*(const RD_SRC_T *)srow);
+    rd_one o;
+    rd_one_load(o, srow);
+    const RD_ACC_T first = (RD_ACC_T)RD_ONE_VAL(o);
     if (first != first) {
-      a.v = (RD_ACC_T)first;
+      a.v = first;
 #if RD_ARG
       a.i = 0;
 #endif
@@ -299,38 +339,21 @@ static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *
 
 /* ---- redux_row ------------------------------------------------------------- */
 
-#define RD_PV (RD_VEC * RD_ES)   /* elements fetched per load */
-typedef RD_SRC_T rd_pvec_t __attribute__((ext_vector_type(RD_PV)));
-/* every source element is read once: stream it past the caches */
-#if RD_NT
-#define RD_LOAD(p) __builtin_nontemporal_load(p)
-#else
-#define RD_LOAD(p) (*(p))
-#endif
-
 /* One "unit" = RD_U loads per lane over RD_G lanes: elements
  * e0 + j*RD_G*RD_VEC + v of the inner reduced dim, j < RD_U, v < RD_VEC, where
- * e0 = (first element of the unit) + lane*RD_VEC. */
-static __device__ inline void rd_unit_load(rd_pvec_t *x, const char *base, ga_long e0, ga_long rin,
-                                           ga_long rstr) {
-#pragma unroll
-  for (int j = 0; j < RD_U; j++) {
-    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
-    if (e < rin) x[j] = RD_LOAD((const rd_pvec_t *)(base + e * rstr));
-  }
-}
-
-/* Combination of the lane's elements of one unit.  ib, rml: index of element
+ * e0 = (first element of the unit) + lane*RD_VEC.
+ *
+ * Combination of the lane's elements of one unit.  ib, rml: index of element
  * 0 of the inner dim and index step per element. */
-static __device__ inline rd_acc rd_unit_combine(const rd_pvec_t *x, ga_long e0, ga_long rin,
-                                                ga_long ib, ga_long rml) {
+static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga_long rin,
+                                                ga_long ib, ga_long rml RD_SCALAR_FPARAMS) {
 #if RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN
   /* The lane's elements are visited in rising index order, so a strict
    * compare keeps the first of equals by itself; only the position inside
    * the unit (a small int) is tracked. */
   rd_acc r = rd_neutral();
   if (e0 < rin) {
-    RD_ACC_T bv = rd_elem(x[0][0], 0).v;
+    RD_ACC_T bv = rd_elem(RD_UNIT_VAL(x, 0, 0), 0).v;
     ga_int bp = 0;
 #pragma unroll
     for (int j = 0; j < RD_U; j++) {
@@ -338,7 +361,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_pvec_t *x, ga_long e0, 
 #pragma unroll
         for (int v = 0; v < RD_VEC; v++) {
           if (j == 0 && v == 0) continue;
-          const RD_ACC_T val = rd_elem(x[j][v * RD_ES], 0).v;
+          const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
 #if RD_KIND == RD_K_MAX
           const bool better = val > bv;
 #else
@@ -366,7 +389,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_pvec_t *x, ga_long e0, 
     if (e < rin) {
 #pragma unroll
       for (int v = 0; v < RD_VEC; v++)
-        t[j] = rd_combine(t[j], rd_elem(x[j][v * RD_ES], ib + (e + v) * rml));
+        t[j] = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v) * rml));
     }
   }
   /* pairwise over the unit */
@@ -379,9 +402,9 @@ static __device__ inline rd_acc rd_unit_combine(const rd_pvec_t *x, ga_long e0, 
 }
 
 KERNEL void __launch_bounds__(256)
-redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict__ d0,
-          const ga_size d0_off, char *__restrict__ d1, const ga_size d1_off,
-          RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, const rd_plan p) {
+redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+          const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+          const rd_plan p RD_SCALAR_PARAMS) {
   const unsigned rows_per_group = 256u / RD_G;
   const unsigned lane = LID_0 % RD_G;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
@@ -391,15 +414,20 @@ redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict_
 #endif
   if (row >= p.nrows) return;   /* uniform per wavefront; per group when RD_G == 256 */
 
-  ga_long so, d0o, d1o;
-  rd_row_offsets(p, row, &so, &d0o, &d1o);
-  const char *srow = src + src_off + so;
-
   const int ri = p.nr - 1;                 /* inner reduced dim */
   const ga_long rin = p.nr > 0 ? p.rdim[ri] : 1;
-  const ga_long rstr = p.nr > 0 ? p.rsstr[ri] : 0;
   const ga_long rml = p.nr > 0 ? p.rmul[ri] : 0;
   const ga_long seg = (ga_long)RD_G * RD_VEC * RD_U;
+
+  ga_long so[RD_NSRC], d0o, d1o, rstr[RD_NSRC];
+  rd_row_offsets(p, row, so, &d0o, &d1o);
+  const char *srow[RD_NSRC];
+  RD_SRC_BASES(srow);
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) {
+    srow[k] += so[k];
+    rstr[k] = p.nr > 0 ? p.rsstr[k][ri] : 0;
+  }
 
   /* A split owns a contiguous range of units, or - for a single reduced dim
    * (RD_INTERLEAVE) - every nsplit-th unit, so that at any moment the splits
@@ -417,22 +445,25 @@ redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict_
    * division for the first unit, then counted up */
   ga_long ro = 0, k = u0;
   if (p.nr > 1) { ro = u0 / p.nseg; k = u0 - ro * p.nseg; }
-  ga_long rb = 0, ib = 0;
-  rd_outer_offsets(p, ri, ro, &rb, &ib);
+  ga_long rb[RD_NSRC], ib = 0;
+  rd_outer_offsets(p, ri, ro, rb, &ib);
 
   rd_acc acc = rd_neutral();
   for (ga_long u = u0; u < u1; u += ustep) {
     const ga_long e0 = k * seg + (ga_long)lane * RD_VEC;
-    rd_pvec_t x[RD_U];
-    rd_unit_load(x, srow + rb, e0, rin, rstr);
-    acc = rd_combine(acc, rd_unit_combine(x, e0, rin, ib, rml));
+    rd_unit x;
+    const char *ub[RD_NSRC];
+#pragma unroll
+    for (int s = 0; s < RD_NSRC; s++) ub[s] = srow[s] + rb[s];
+    rd_unit_load(x, ub, e0, rin, rstr);
+    acc = rd_combine(acc, rd_unit_combine(x, e0, rin, ib, rml RD_SCALAR_ARGS));
 #if RD_INTERLEAVE
     k += ustep;   /* single reduced dim: the unit is the segment */
 #else
     if (++k == p.nseg) {
       k = 0;
       ro++;
-      rd_outer_offsets(p, ri, ro, &rb, &ib);
+      rd_outer_offsets(p, ri, ro, rb, &ib);
     }
 #endif
   }
@@ -443,8 +474,10 @@ redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict_
   acc = rd_wave_reduce(acc);
 #endif
   if (lane == 0) {
-    if (p.nsplit == 1) rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
-    else rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
+    if (p.nsplit == 1)
+      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
+    else
+      rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
   }
 }
 
@@ -455,9 +488,9 @@ redux_row(const char *__restrict__ src, const ga_size src_off, char *__restrict_
  * overlaps the cross-lane work.  Only built for RD_G == 64. */
 #if RD_G == 64
 KERNEL void __launch_bounds__(256)
-redux_wrows(const char *__restrict__ src, const ga_size src_off, char *__restrict__ d0,
-            const ga_size d0_off, char *__restrict__ d1, const ga_size d1_off,
-            RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, const rd_plan p) {
+redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const rd_plan p RD_SCALAR_PARAMS) {
   (void)part_v; (void)part_i;
   const unsigned lane = LID_0 & 63u;
   const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
@@ -467,26 +500,38 @@ redux_wrows(const char *__restrict__ src, const ga_size src_off, char *__restric
   if (row >= row_end) return;
 
   const ga_long rin = p.nr > 0 ? p.rdim[0] : 1;
-  const ga_long rstr = p.nr > 0 ? p.rsstr[0] : 0;
   const ga_long rml = p.nr > 0 ? p.rmul[0] : 0;
   const ga_long e0 = (ga_long)lane * RD_VEC;
-
-  ga_long so, d0o, d1o;
-  rd_row_offsets(p, row, &so, &d0o, &d1o);
-  rd_pvec_t cur[RD_U];
-  rd_unit_load(cur, src + src_off + so, e0, rin, rstr);
-  for (; row < row_end; row++) {
-    ga_long nso = 0, nd0o = 0, nd1o = 0;
-    rd_pvec_t nxt[RD_U];
-    if (row + 1 < row_end) {
-      rd_row_offsets(p, row + 1, &nso, &nd0o, &nd1o);
-      rd_unit_load(nxt, src + src_off + nso, e0, rin, rstr);
-    }
-    rd_acc acc = rd_wave_reduce(rd_unit_combine(cur, e0, rin, 0, rml));
-    if (lane == 0) rd_store(acc, src + src_off + so, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+  ga_long rstr[RD_NSRC];
+  const char *base[RD_NSRC];
+  RD_SRC_BASES(base);
 #pragma unroll
-    for (int j = 0; j < RD_U; j++) cur[j] = nxt[j];
-    so = nso; d0o = nd0o; d1o = nd1o;
+  for (int k = 0; k < RD_NSRC; k++) rstr[k] = p.nr > 0 ? p.rsstr[k][0] : 0;
+
+  ga_long so[RD_NSRC], d0o, d1o;
+  const char *srow[RD_NSRC];
+  rd_row_offsets(p, row, so, &d0o, &d1o);
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) srow[k] = base[k] + so[k];
+  rd_unit cur;
+  rd_unit_load(cur, srow, e0, rin, rstr);
+  for (; row < row_end; row++) {
+    ga_long nso[RD_NSRC], nd0o = 0, nd1o = 0;
+    const char *nrow[RD_NSRC];
+    rd_unit nxt;
+    if (row + 1 < row_end) {
+      rd_row_offsets(p, row + 1, nso, &nd0o, &nd1o);
+#pragma unroll
+      for (int k = 0; k < RD_NSRC; k++) nrow[k] = base[k] + nso[k];
+      rd_unit_load(nxt, nrow, e0, rin, rstr);
+    }
+    rd_acc acc = rd_wave_reduce(rd_unit_combine(cur, e0, rin, 0, rml RD_SCALAR_ARGS));
+    if (lane == 0)
+      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
+    cur = nxt;
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) srow[k] = nrow[k];
+    d0o = nd0o; d1o = nd1o;
   }
 }
 #endif
@@ -494,8 +539,8 @@ redux_wrows(const char *__restrict__ src, const ga_size src_off, char *__restric
 /* ---- redux_col ------------------------------------------------------------- */
 
 KERNEL void __launch_bounds__(256)
-redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
-          const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
+          RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
   __shared__ rd_acc lds[4][64];
   const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
@@ -508,21 +553,28 @@ redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
   const bool live = fi < fin;
 
   /* offsets of this lane's output */
-  ga_long so = 0, d0o = 0, d1o = 0;
+  ga_long so[RD_NSRC], d0o = 0, d1o = 0;
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) so[k] = 0;
   {
     ga_long r = fo;
     for (int d = fi_d - 1; d >= 0; d--) {
       ga_long c;
       if (d > 0) { c = r % p.fdim[d]; r = r / p.fdim[d]; } else { c = r; }
-      so += c * p.fsstr[d];
+#pragma unroll
+      for (int k = 0; k < RD_NSRC; k++) so[k] += c * p.fsstr[k][d];
       d0o += c * p.fd0str[d];
       d1o += c * p.fd1str[d];
     }
-    so += fi * p.fsstr[fi_d];
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) so[k] += fi * p.fsstr[k][fi_d];
     d0o += fi * p.fd0str[fi_d];
     d1o += fi * p.fd1str[fi_d];
   }
-  const char *srow = src + src_off + so;
+  const char *srow[RD_NSRC];
+  RD_SRC_BASES(srow);
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) srow[k] += so[k];
 
   ga_long r0 = split * p.upb, r1 = r0 + p.upb;
   if (r1 > p.rtotal) r1 = p.rtotal;
@@ -530,26 +582,32 @@ redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
   rd_acc acc = rd_neutral();
   if (live) {
     for (ga_long j0 = r0 + ty; j0 < r1; j0 += 4 * RD_U) {
-      RD_SRC_T x[RD_U];
+      rd_one x[RD_U];
       ga_long idx[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
         const ga_long j = j0 + 4 * q;
         if (j < r1) {
-          ga_long off = 0, ix = 0, r = j;
+          ga_long off[RD_NSRC], ix = 0, r = j;
+#pragma unroll
+          for (int k = 0; k < RD_NSRC; k++) off[k] = 0;
           for (int d = p.nr - 1; d >= 0; d--) {
             ga_long c;
             if (d > 0) { c = r % p.rdim[d]; r = r / p.rdim[d]; } else { c = r; }
-            off += c * p.rsstr[d];
+#pragma unroll
+            for (int k = 0; k < RD_NSRC; k++) off[k] += c * p.rsstr[k][d];
             ix += c * p.rmul[d];
           }
-          x[q] = RD_LOAD((const RD_SRC_T *)(srow + off));
+          const char *ep[RD_NSRC];
+#pragma unroll
+          for (int k = 0; k < RD_NSRC; k++) ep[k] = srow[k] + off[k];
+          rd_one_load(x[q], ep);
           idx[q] = ix;
         }
       }
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
-        if (j0 + 4 * q < r1) acc = rd_combine(acc, rd_elem(x[q], idx[q]));
+        if (j0 + 4 * q < r1) acc = rd_combine(acc, rd_elem(RD_ONE_VAL(x[q]), idx[q]));
     }
   }
   lds[ty][tx] = acc;
@@ -561,7 +619,7 @@ redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
     const ga_long row = fo * fin + fi;
     if (p.nsplit == 1) {
       /* element 0 of the scan is at the start of the lane's reduced range */
-      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
     } else {
       rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
     }
@@ -571,8 +629,8 @@ redux_col(const char *src, const ga_size src_off, char *d0, const ga_size d0_off
 /* ---- redux_final ------------------------------------------------------------
  * One wavefront per output: combine its nsplit partials and write the result. */
 KERNEL void __launch_bounds__(256)
-redux_final(const char *src, const ga_size src_off, char *d0, const ga_size d0_off, char *d1,
-            const ga_size d1_off, RD_ACC_T *part_v, ga_long *part_i, const rd_plan p) {
+redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
+            RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
   const unsigned lane = LID_0 & 63u;
   const ga_long row = (ga_long)GID_0 * 4 + (LID_0 >> 6);
   if (row >= p.nrows) return;
@@ -587,8 +645,12 @@ redux_final(const char *src, const ga_size src_off, char *d0, const ga_size d0_o
   }
   acc = rd_wave_reduce(acc);
   if (lane == 0) {
-    ga_long so, d0o, d1o;
-    rd_row_offsets(p, row, &so, &d0o, &d1o);
-    rd_store(acc, src + src_off + so, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal);
+    ga_long so[RD_NSRC], d0o, d1o;
+    rd_row_offsets(p, row, so, &d0o, &d1o);
+    const char *srow[RD_NSRC];
+    RD_SRC_BASES(srow);
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) srow[k] += so[k];
+    rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
   }
 }

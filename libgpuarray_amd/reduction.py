@@ -14,6 +14,7 @@ exist in the reference only as GpuArray_maxandargmax
 """
 import builtins as _b
 import ctypes as C
+import re
 
 import numpy as np
 
@@ -55,6 +56,209 @@ class GpuReduction(object):
         check(lib.GpuReduction_call(self.gr, d0._ptr() if d0 is not None else None,
                                     d1._ptr() if d1 is not None else None, src._ptr(),
                                     len(axes), arr, 0), self.context.ctx)
+
+
+class Argument(object):
+    """reference pygpu/tools.py:22-37"""
+
+    def __init__(self, dtype, name):
+        self.dtype = np.dtype(dtype)
+        self.name = name
+
+    def __hash__(self):
+        return hash(type(self)) ^ hash(self.dtype) ^ hash(self.name)
+
+    def __eq__(self, other):
+        return type(self) == type(other) and self.dtype == other.dtype and self.name == other.name
+
+
+class ArrayArg(Argument):
+    def isarray(self):
+        return True
+
+    def expr(self):
+        return "%s[i]" % (self.name,)
+
+
+class ScalarArg(Argument):
+    def isarray(self):
+        return False
+
+    def expr(self):
+        return self.name
+
+
+def as_argument(obj, name):
+    """reference pygpu/tools.py:15-19"""
+    if isinstance(obj, GpuArray):
+        return ArrayArg(obj.dtype, name)
+    return ScalarArg(np.asarray(obj).dtype, name)
+
+
+_C_TYPES = {
+    "bool": "bool", "char": "int8", "signed char": "int8", "unsigned char": "uint8",
+    "short": "int16", "unsigned short": "uint16", "int": "int32", "unsigned": "uint32",
+    "unsigned int": "uint32", "long": "int64", "unsigned long": "uint64",
+    "long long": "int64", "unsigned long long": "uint64", "float": "float32",
+    "double": "float64", "half": "float16", "ga_half": "float16", "ga_bool": "bool",
+    "ga_byte": "int8", "ga_ubyte": "uint8", "ga_short": "int16", "ga_ushort": "uint16",
+    "ga_int": "int32", "ga_uint": "uint32", "ga_long": "int64", "ga_ulong": "uint64",
+    "ga_float": "float32", "ga_double": "float64",
+}
+_DECL_RE = re.compile(r"(\**)\s*([_a-zA-Z0-9]+)(\s*\[[ 0-9]*\])*\s*$")
+_INDEX_RE = re.compile(r"([a-zA-Z_][a-zA-Z0-9_]*)\[i\]")
+
+
+def parse_c_args(arguments):
+    """"float *a, float *b, float s" -> (ArrayArg, ArrayArg, ScalarArg)
+    (reference pygpu/reduction.py:13-15, pygpu/dtypes.py:121-147)."""
+    res = []
+    for c_arg in arguments.split(","):
+        c_arg = c_arg.replace("const", "").replace("volatile", "").replace("GLOBAL_MEM", "")
+        m = _DECL_RE.search(c_arg)
+        if m is None:
+            raise ValueError("couldn't parse C declarator '%s'" % c_arg)
+        tp = " ".join(c_arg[:m.start()].split())
+        if tp not in _C_TYPES:
+            raise ValueError("unknown type '%s'" % tp)
+        cls = ArrayArg if (m.group(1) or m.group(3) is not None) else ScalarArg
+        res.append(cls(np.dtype(_C_TYPES[tp]), m.group(2)))
+    return tuple(res)
+
+
+class ReductionKernel(object):
+    """reference pygpu/reduction.py:137-291: `reduce_expr` (in a and b) folds
+    the values of `map_expr` (arrays written `name[i]`) over the axes flagged
+    in `redux`, starting from `neutral`, accumulating in `dtype_out`.  One
+    pass over the inputs: the expression is evaluated inside the reduction
+    kernel.  Differences: float16 is accepted (accumulated in float32; the
+    reference raises NotImplementedError, :156-160) and nothing limits the
+    number of outputs (:256-258)."""
+
+    def __init__(self, context, dtype_out, neutral, reduce_expr, redux, map_expr=None,
+                 arguments=None, preamble="", init_nd=None):
+        self.context = context
+        self.neutral = neutral
+        self.redux = tuple(redux)
+        if not _b.any(self.redux):
+            raise ValueError("Reduction is along no axes")
+        self.dtype_out = np.dtype(dtype_out)
+        if isinstance(arguments, str):
+            self.arguments = parse_c_args(arguments)
+        elif arguments is None:
+            self.arguments = [ArrayArg(self.dtype_out, "_reduce_input")]
+        else:
+            self.arguments = list(arguments)
+        self.reduce_expr = reduce_expr
+        if map_expr is None:
+            if len(self.arguments) != 1:
+                raise ValueError("Don't know what to do with more than one argument. "
+                                 "Specify map_expr to explicitly state what you want.")
+            self.operation = "%s[i]" % (self.arguments[0].name,)
+        else:
+            self.operation = map_expr
+        if not _b.any(a.isarray() for a in self.arguments):
+            raise ValueError("ReductionKernel can only be used with functions that have at "
+                             "least one vector argument.")
+        self.preamble = preamble
+        # arrays are named by their element in the C interface
+        expr = _INDEX_RE.sub(r"\g<1>", self.operation)
+        self._op = MapReduction(context, "custom", self.dtype_out, expr, self.arguments,
+                                preamble=preamble, reduce_expr=str(reduce_expr),
+                                neutral=str(neutral))
+
+    def __call__(self, *args, **kwargs):
+        broadcast = kwargs.pop("broadcast", None)
+        out = kwargs.pop("out", None)
+        if len(kwargs) != 0:
+            raise TypeError("Unexpected keyword argument: %s" % list(kwargs.keys())[0])
+        if len(args) != len(self.arguments):
+            raise TypeError("Expected %d arguments, got %d" % (len(self.arguments), len(args)))
+        arrays = [a for a, d in zip(args, self.arguments) if d.isarray()]
+        for a in arrays:
+            if not isinstance(a, GpuArray):
+                raise TypeError("array argument expected, got %r" % (type(a),))
+            if a.ndim != len(self.redux):
+                raise ValueError("Array has %d dimensions, the kernel reduces over %d" % (
+                    a.ndim, len(self.redux)))
+        dims = _common_shape(arrays, broadcast)
+        out_shape = tuple(d for i, d in enumerate(dims) if not self.redux[i])
+        if out is None:
+            out = gpuarray.empty(out_shape, dtype=self.dtype_out, context=self.context)
+        elif out.shape != out_shape or out.dtype != self.dtype_out:
+            raise TypeError("Out array is not of expected type (expected %s %s, got %s %s)" % (
+                out_shape, self.dtype_out, out.shape, out.dtype))
+        axes = [i for i, r in enumerate(self.redux) if r]
+        self._op(args, axes, d0=out, broadcast=bool(broadcast))
+        return out
+
+
+def _common_shape(arrays, broadcast):
+    """reference pygpu/tools.py check_args with collapse=False"""
+    dims = list(arrays[0].shape)
+    for a in arrays[1:]:
+        if a.ndim != len(dims):
+            raise ValueError("Arrays have %d and %d dimensions" % (len(dims), a.ndim))
+        for i, d in enumerate(a.shape):
+            if d != dims[i]:
+                if broadcast and dims[i] == 1:
+                    dims[i] = d
+                elif not (broadcast and d == 1):
+                    raise ValueError("Array shape mismatch on dimension %d: %d vs %d" % (
+                        i, d, dims[i]))
+    return dims
+
+
+class MapReduction(object):
+    """GpuReduction_new_map / GpuReduction_call_map: operation `op` (a name of
+    the table above, or "custom" with `reduce_expr` in a and b and its
+    `neutral`) over the values of `map_expr`, an expression in the names of
+    `arguments` (ArrayArg / ScalarArg), evaluated in the reduction kernel and
+    accumulated in `acc_dtype`."""
+
+    def __init__(self, context, op, acc_dtype, map_expr, arguments, preamble="",
+                 reduce_expr=None, neutral=None):
+        self.context = context
+        self.arguments = list(arguments)
+        self.acc_dtype = np.dtype(acc_dtype)
+        n = len(self.arguments)
+        self._names = [a.name.encode() for a in self.arguments]
+        self._descr = (_lib.ElemwiseArg * _b.max(n, 1))()
+        for i, a in enumerate(self.arguments):
+            self._descr[i].name = self._names[i]
+            self._descr[i].typecode = dtype_to_typecode(a.dtype)
+            self._descr[i].flags = _lib.GE_READ | (0 if a.isarray() else _lib.GE_SCALAR)
+        opid = _lib.GA_REDUCE_CUSTOM if op == "custom" else _OPS[op]
+        self.gr = C.c_void_p()
+        check(lib.GpuReduction_new_map(
+            C.byref(self.gr), context.ctx, opid,
+            reduce_expr.encode() if reduce_expr is not None else None,
+            neutral.encode() if neutral is not None else None,
+            dtype_to_typecode(self.acc_dtype), preamble.encode(), map_expr.encode(), n,
+            C.cast(self._descr, C.c_void_p), 0), context.ctx)
+
+    def __del__(self):
+        gr = getattr(self, "gr", None)
+        if gr:
+            lib.GpuReduction_free(gr)
+            self.gr = None
+
+    def __call__(self, args, axes, d0=None, d1=None, broadcast=False):
+        keep = []
+        ptrs = (C.c_void_p * _b.max(len(args), 1))()
+        for i, (a, d) in enumerate(zip(args, self.arguments)):
+            if d.isarray():
+                ptrs[i] = C.cast(a._ptr(), C.c_void_p)
+            else:
+                v = np.asarray(a, dtype=d.dtype).reshape(1).copy()
+                keep.append(v)
+                ptrs[i] = v.ctypes.data
+        axes = list(axes)
+        arr = (C.c_int * _b.max(len(axes), 1))(*axes)
+        check(lib.GpuReduction_call_map(self.gr, d0._ptr() if d0 is not None else None,
+                                        d1._ptr() if d1 is not None else None, ptrs, len(axes),
+                                        arr, _lib.GE_BROADCAST if broadcast else 0),
+              self.context.ctx)
 
 
 _cache = {}
@@ -102,8 +306,35 @@ def _upcast(dtype):
     return dtype
 
 
-def reduce1(ary, op, out_type, axis=None, out=None):
-    """Value reduction `op` of `ary` over `axis` into dtype `out_type`."""
+# (C operator, neutral) pairs of the reference's reduce1 callers
+# (pygpu/_array.py:238-294) and the built-in operation each one is
+_BUILTIN = {("+", "0"): "sum", ("*", "1"): "prod", ("&&", "1"): "all", ("||", "0"): "any",
+            ("&", "-1"): "and", ("|", "0"): "or", ("^", "0"): "xor"}
+
+
+def reduce1(ary, op, neutral, out_type, axis=None, out=None, oper=None):
+    """reference pygpu/reduction.py:294-319: reduce `ary` over `axis` with the
+    C binary operator `op` (or the expression `oper` in a and b) from
+    `neutral`, accumulating in `out_type`.  The operator/neutral pairs the
+    reference's own callers use run the built-in operations; anything else
+    goes through ReductionKernel."""
+    name = _BUILTIN.get((op, str(neutral).strip())) if oper is None else None
+    if name in ("all", "any") and np.dtype(out_type) != np.dtype("bool"):
+        name = None
+    if name is not None:
+        return _reduce_named(ary, name, out_type, axis, out)
+    if ary.ndim == 0:
+        return ary.astype(out_type) if np.dtype(out_type) != ary.dtype else ary.copy()
+    axes = _normalize_axes(ary.ndim, axis)
+    redux = [i in axes for i in range(ary.ndim)]
+    r = ReductionKernel(ary.context, dtype_out=out_type, neutral=neutral,
+                        reduce_expr=oper if oper is not None else "a %s b" % (op,), redux=redux,
+                        arguments=[ArrayArg(ary.dtype, "a")])
+    return r(ary, out=out)
+
+
+def _reduce_named(ary, op, out_type, axis=None, out=None):
+    """Built-in value reduction `op` of `ary` over `axis` into dtype `out_type`."""
     out_type = np.dtype(out_type)
     if ary.ndim == 0:
         res = ary.astype(out_type) if out_type != ary.dtype else ary.copy()
@@ -120,27 +351,27 @@ def reduce1(ary, op, out_type, axis=None, out=None):
 
 
 def sum(ary, axis=None, dtype=None, out=None):
-    return reduce1(ary, "sum", _upcast(ary.dtype) if dtype is None else dtype, axis, out)
+    return _reduce_named(ary, "sum", _upcast(ary.dtype) if dtype is None else dtype, axis, out)
 
 
 def prod(ary, axis=None, dtype=None, out=None):
-    return reduce1(ary, "prod", _upcast(ary.dtype) if dtype is None else dtype, axis, out)
+    return _reduce_named(ary, "prod", _upcast(ary.dtype) if dtype is None else dtype, axis, out)
 
 
 def all(ary, axis=None, out=None):
-    return reduce1(ary, "all", np.dtype("bool"), axis, out)
+    return _reduce_named(ary, "all", np.dtype("bool"), axis, out)
 
 
 def any(ary, axis=None, out=None):
-    return reduce1(ary, "any", np.dtype("bool"), axis, out)
+    return _reduce_named(ary, "any", np.dtype("bool"), axis, out)
 
 
 def max(ary, axis=None, out=None):
-    return reduce1(ary, "max", ary.dtype, axis, out)
+    return _reduce_named(ary, "max", ary.dtype, axis, out)
 
 
 def min(ary, axis=None, out=None):
-    return reduce1(ary, "min", ary.dtype, axis, out)
+    return _reduce_named(ary, "min", ary.dtype, axis, out)
 
 
 def _arg_reduce(ary, op, axis, want_value):

@@ -513,3 +513,82 @@ int orc_take1(char *r, const char *v, size_t elsz, unsigned nd, const size_t *vd
   }
   return 0;
 }
+
+/* ---- the same kernel with a map expression over two arrays and a scalar ------
+ * pygpu/reduction.py:33-134 with `arguments` = (a, b, s) and `map_expr` set
+ * (the use of pygpu/tests/test_reduction.py:57-84): each array has its own
+ * strides over the common dims (0 on a broadcast dim, pygpu/tools.py
+ * check_args); element i of the flattened reduced index contributes
+ * REDUCE(acc, map(a[i], b[i], s)); accumulator and output have type `t`
+ * (0 float, 1 double).
+ *   map: 0 a*b   1 fabs(a-b)   2 s*a+b   3 a*a
+ *   red: 0 a+b from 0          1 max(a,b) from -inf */
+static double map2(int map, double a, double b, double s, int t) {
+  if (t == 0) {
+    volatile float r;
+    float fa = (float)a, fb = (float)b, fs = (float)s;
+    switch (map) {
+    case 0: r = fa * fb; break;
+    case 1: r = fabsf(fa - fb); break;
+    case 2: { volatile float m = fs * fa; r = m + fb; break; }
+    default: r = fa * fa; break;
+    }
+    return r;
+  }
+  switch (map) {
+  case 0: return a * b;
+  case 1: return fabs(a - b);
+  case 2: { volatile double m = s * a; return m + b; }
+  default: return a * a;
+  }
+}
+static double red2(int red, double x, double y, int t) {
+  if (red == 1) return (y > x) ? y : x;
+  if (t == 0) { volatile float r = (float)x + (float)y; return r; }
+  return x + y;
+}
+int orc_reduk_map2(int map, int red, int t, unsigned nd, const size_t *dims, const char *a,
+                   const ssize_t *astr, const char *b, const ssize_t *bstr, double s,
+                   const int *redux, char *out, size_t ls) {
+  size_t gs = 1, n = 1;
+  for (unsigned d = 0; d < nd; d++) {
+    if (redux[d]) n *= dims[d]; else gs *= dims[d];
+  }
+  double *ld = (double *)malloc(ls * sizeof(double));
+  if (!ld) return 1;
+  for (size_t g = 0; g < gs; g++) {
+    size_t tt = g;
+    ssize_t fa = 0, fb = 0;
+    for (unsigned d = nd; d > 0; d--) {
+      if (redux[d - 1]) continue;
+      size_t c = tt % dims[d - 1];
+      tt /= dims[d - 1];
+      fa += (ssize_t)c * astr[d - 1];
+      fb += (ssize_t)c * bstr[d - 1];
+    }
+    for (size_t lid = 0; lid < ls; lid++) {
+      double acc = red == 1 ? -INFINITY : 0.0;
+      for (size_t i = lid; i < n; i += ls) {
+        size_t u = i;
+        ssize_t ra = 0, rb = 0;
+        for (unsigned d = nd; d > 0; d--) {
+          if (!redux[d - 1]) continue;
+          size_t c = u % dims[d - 1];
+          u /= dims[d - 1];
+          ra += (ssize_t)c * astr[d - 1];
+          rb += (ssize_t)c * bstr[d - 1];
+        }
+        double xa = t == 0 ? *(const float *)(a + fa + ra) : *(const double *)(a + fa + ra);
+        double xb = t == 0 ? *(const float *)(b + fb + rb) : *(const double *)(b + fb + rb);
+        acc = red2(red, acc, map2(map, xa, xb, s, t), t);
+      }
+      ld[lid] = acc;
+    }
+    for (size_t cur = ls / 2; cur >= 1; cur /= 2)
+      for (size_t lid = 0; lid < cur; lid++) ld[lid] = red2(red, ld[lid], ld[lid + cur], t);
+    if (t == 0) ((float *)out)[g] = (float)ld[0];
+    else ((double *)out)[g] = ld[0];
+  }
+  free(ld);
+  return 0;
+}

@@ -45,6 +45,8 @@ def _load():
                                    C.POINTER(C.c_uint), C.c_void_p, PSS, C.c_void_p, PSS]
     L.orc_reduk.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_uint, PS, PSS, C.POINTER(C.c_int),
                             C.c_void_p, C.c_int, C.c_size_t]
+    L.orc_reduk_map2.argtypes = [C.c_int, C.c_int, C.c_int, C.c_uint, PS, C.c_void_p, PSS, C.c_void_p,
+                                 PSS, C.c_double, C.POINTER(C.c_int), C.c_void_p, C.c_size_t]
     L.orc_take1.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint, PS, PSS, C.c_void_p,
                             C.c_int, C.c_size_t, C.POINTER(C.c_int)]
     return L
@@ -289,3 +291,30 @@ def take1(v, ind, out=None):
     if rc:
         raise ValueError("orc_take1: error %d" % rc)
     return out, err.value
+
+
+MAP_MUL, MAP_ABSDIFF, MAP_SAXPY, MAP_SQUARE = range(4)
+RED_ADD, RED_MAX = range(2)
+
+
+def reduk_map2(map_id, red_id, a, b, s, axes, ls=256):
+    """pygpu/reduction.py:33-134 with map_expr over arrays a, b (broadcast
+    against each other, pygpu/tools.py check_args) and scalar s; float32 or
+    float64 throughout."""
+    assert a.dtype == b.dtype and a.dtype in (np.float32, np.float64) and a.ndim == b.ndim
+    nd = a.ndim
+    shape = tuple(max(x, y) for x, y in zip(a.shape, b.shape))
+    astr = [st if d == full else 0 for st, d, full in zip(a.strides, a.shape, shape)]
+    bstr = [st if d == full else 0 for st, d, full in zip(b.strides, b.shape, shape)]
+    axes = [x % nd for x in axes]
+    redux = (C.c_int * nd)(*[1 if i in axes else 0 for i in range(nd)])
+    oshape = tuple(d for i, d in enumerate(shape) if i not in axes)
+    out = np.empty(oshape, dtype=a.dtype)
+    rc = _L.orc_reduk_map2(map_id, red_id, 0 if a.dtype == np.float32 else 1, nd,
+                           (C.c_size_t * nd)(*shape), C.c_void_p(a.ctypes.data),
+                           (C.c_ssize_t * nd)(*astr), C.c_void_p(b.ctypes.data),
+                           (C.c_ssize_t * nd)(*bstr), float(s), redux,
+                           C.c_void_p(out.ctypes.data), ls)
+    if rc:
+        raise ValueError("orc_reduk_map2: error %d" % rc)
+    return out

@@ -162,7 +162,7 @@ def test_red_array_basic(shape, redux, ctx, oracle):   # pygpu/tests/test_reduct
     axes = tuple(i for i, r in enumerate(redux) if r)
     for dt in ["int8", "uint8", "int16", "uint16", "int32", "uint32", "float32", "float64"]:
         c, g = gen_gpuarray(shape, dt, ctx=ctx, rng=rng)
-        out = R.reduce1(g, "sum", dt, axis=axes)          # same dtype in and out, as the test
+        out = R.reduce1(g, "+", "0", dt, axis=axes)          # same dtype in and out, as the test
         want = c.sum(axis=axes, dtype=dt)
         assert out.shape == want.shape and out.dtype == np.dtype(dt)
         if np.dtype(dt).kind in "iu":
@@ -327,7 +327,7 @@ def test_all_value_ops_on_layouts(layout, ctx):
             else:
                 odt = np.dtype(dt)
             want = np_reduce(op, v, axes, odt if op in ("sum", "prod", "prodnz") else None)
-            out = R.reduce1(g, op, odt, axis=tuple(axes))
+            out = R._reduce_named(g, op, odt, axis=tuple(axes))
             got = np.asarray(out)
             assert got.shape == want.shape, (op, dt)
             if np.dtype(dt).kind == "f" and op in ("sum",):
@@ -363,7 +363,7 @@ def test_integer_invariants(ctx):
     assert np.asarray(R.sum(gpuarray.array(perm, context=ctx))) == x.sum()
     # wrap-around modulo 2^32 when the result type is the input type
     big = np.full(100000, 2 ** 30, np.int32)
-    got = np.asarray(R.reduce1(gpuarray.array(big, context=ctx), "sum", "int32"))
+    got = np.asarray(R.reduce1(gpuarray.array(big, context=ctx), "+", "0", "int32"))
     assert got == np.int32(np.int64(100000 * 2 ** 30).astype(np.int32))
 
 

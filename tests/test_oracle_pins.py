@@ -364,3 +364,40 @@ def test_take1_strided_source_wrap_and_bounds(oracle):
     got, err = oracle.take1(v, np.array([1, -6, 5, 2], dtype=np.int64), out=out)
     assert err == -1
     assert np.array_equal(got[[0, 3]], v[[1, 2]]) and np.all(got[[1, 2]] == -7)
+
+
+# ---- map + reduce in one kernel: pygpu/reduction.py:33-134 with map_expr -------
+
+def test_reduk_map_is_numpy_on_exact_data(oracle):
+    """Small integers in float: every product and partial sum is exact, so the
+    template's order does not matter and NumPy is the answer bit for bit.  The
+    shapes are the reference's own broadcast case
+    (pygpu/tests/test_reduction.py:57-84: (5,10,15) * (1,10,15), axis 1)."""
+    rng = np.random.default_rng(21)
+    for dt in (np.float32, np.float64):
+        x = rng.integers(-8, 9, size=(5, 10, 15)).astype(dt)
+        y = rng.integers(-8, 9, size=(1, 10, 15)).astype(dt)
+        for axes in ([1], [0], [2], [0, 2], [0, 1, 2]):
+            got = oracle.reduk_map2(oracle.MAP_MUL, oracle.RED_ADD, x, y, 0.0, axes, ls=16)
+            assert np.array_equal(got, (x * y).sum(axis=tuple(axes)))
+            got = oracle.reduk_map2(oracle.MAP_ABSDIFF, oracle.RED_MAX, x, y, 0.0, axes, ls=8)
+            assert np.array_equal(got, np.abs(x - y).max(axis=tuple(axes)))
+            got = oracle.reduk_map2(oracle.MAP_SAXPY, oracle.RED_ADD, x, y, 3.0, axes, ls=4)
+            assert np.array_equal(got, (dt(3) * x + y).sum(axis=tuple(axes)))
+            got = oracle.reduk_map2(oracle.MAP_SQUARE, oracle.RED_ADD, x, y, 0.0, axes, ls=1)
+            assert np.array_equal(got, np.broadcast_to(x * x, (5, 10, 15)).sum(axis=tuple(axes)))
+
+
+def test_reduk_map_strided_views_and_tolerance(oracle):
+    rng = np.random.default_rng(22)
+    xb = rng.standard_normal((12, 9, 14))
+    yb = rng.standard_normal((14, 9, 12))
+    x, y = xb[::2, ::-1, 1::3], yb.T[::2, :, 1::3]          # both (6, 9, 5)
+    got = oracle.reduk_map2(oracle.MAP_MUL, oracle.RED_ADD, x, y, 0.0, [0, 2], ls=32)
+    np.testing.assert_allclose(got, (x * y).sum(axis=(0, 2)), rtol=1e-12, atol=1e-12)
+    # one lane per group is the plain left-to-right loop
+    got1 = oracle.reduk_map2(oracle.MAP_MUL, oracle.RED_ADD, x, y, 0.0, [1], ls=1)
+    want = np.zeros((6, 5))
+    for j in range(9):
+        want = want + x[:, j, :] * y[:, j, :]
+    assert np.array_equal(got1, want)
