@@ -307,6 +307,37 @@ def per_config(ctx, ga, R):
               host_time(lambda: getattr(U[:, :, ::2], nm)(axis=2), reps=1), "useful bytes; stride-2 view")
     del gu, U
 
+    # Beyond the BASELINE shapes: an expression feeding a reduction in one pass
+    # (dot product of two 2^27 vectors; the two-pass alternative writes and
+    # re-reads a 512 MiB temporary) and a row gather.
+    n = 1 << 27
+    rng = np.random.default_rng(8)
+    p_h, q_h = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
+    gp, gq = ga.array(p_h, context=ctx), ga.array(q_h, context=ctx)
+    dot = R.MapReduction(ctx, "sum", f32, "p*q", [R.ArrayArg(f32, "p"), R.ArrayArg(f32, "q")])
+    od = ga.empty((), f32, context=ctx)
+    us = time_calls(ctx, lambda i: dot([gp, gq], [0], d0=od))
+    tmp = ga.empty((n,), f32, context=ctx)
+    mul = ga.GpuElemwise(ctx, "t = p*q", [ga.arg("p", f32, read=True), ga.arg("q", f32, read=True),
+                                          ga.arg("t", f32, write=True)])
+    opsum = ga.GpuReduction(ctx, "sum", f32)
+
+    def two_pass(i):
+        mul(gp, gq, tmp)
+        opsum(tmp, [0], d0=od)
+    us2 = time_calls(ctx, two_pass)
+    entry("F4_dot_2x2^27_fused", 8 * n + 4, us, us, host_time(lambda: np.dot(p_h, q_h)),
+          "one kernel pass; elementwise-then-sum takes %.1f us for the same result" % us2)
+    del gp, gq, tmp, p_h, q_h
+    rows, width = 65536, 1024
+    V = np.random.default_rng(9).standard_normal((rows, width), dtype=np.float32)
+    idx = np.random.default_rng(10).permutation(rows)
+    gv, gidx = ga.array(V, context=ctx), ga.array(idx, context=ctx)
+    us = time_calls(ctx, lambda i: gv.take1(gidx))
+    entry("F2_take1_65536x1024_rows", 2 * rows * width * 4 + rows * 8, us, us,
+          host_time(lambda: V.take(idx, axis=0)), "includes the result's allocation and the bounds-flag read-back")
+    del gv, gidx, V
+
     # launch-latency floor: small shapes, host-side wall time per call included
     lat = {}
     for m in (1, 1 << 10, 1 << 16):

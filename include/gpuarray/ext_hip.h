@@ -37,6 +37,10 @@ typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
  * < 0 on error. */
 typedef int (*ga_hip_event_record_fn)(gpucontext *ctx, unsigned int slot);
 typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsigned int b);
+/* "hip_module_cache_stats": out[0..2] = entries in the hot, warm and cold
+ * lists of the context's loaded-module cache (the reference's 2Q policy,
+ * src/cache/twoq.c), out[3] = code objects currently loaded. */
+typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
 /* "hip_elemwise_source" / "hip_reduction_source": the kernel text the
  * generators would compile for a given variant, as a malloc'd string the
  * caller frees.  For host-side checks of the generated code. */

@@ -18,6 +18,7 @@
 #include <unistd.h>
 
 #include <iterator>
+#include <list>
 #include <map>
 #include <mutex>
 #include <string>
@@ -28,8 +29,86 @@ namespace {
 
 struct hip_module {
   hipModule_t mod = nullptr;
-  unsigned refcnt = 0;
+  unsigned refcnt = 0;     // kernels made from this module
+  bool cached = false;     // the module cache still lists it
   std::string key;
+};
+
+// ---- loaded-module cache ------------------------------------------------------
+// Source text -> loaded code object, bounded by the reference's 2Q policy
+// (src/cache/twoq.c:232-316, sized 64/128/64/8 by its CUDA backend,
+// src/gpuarray_buffer_cuda.c:291): a new entry enters `hot`; when hot
+// overflows its oldest entry moves to `cold`; a hit in cold promotes the entry
+// to `warm`, whose overflow goes back to cold; cold is cut back to its size
+// once it exceeds size + elasticity.  An entry that leaves the cache is
+// unloaded when the last kernel made from it is gone.
+class module_cache {
+ public:
+  typedef std::list<hip_module *> list_t;
+  size_t hot_size = 64, warm_size = 128, cold_size = 64, elasticity = 8;
+
+  hip_module *get(const std::string &key) {
+    auto it = index_.find(key);
+    if (it == index_.end()) return nullptr;
+    slot &s = it->second;
+    hip_module *m = *s.pos;
+    switch (s.temp) {
+    case HOT: hot_.splice(hot_.end(), hot_, s.pos); break;
+    case WARM: warm_.splice(warm_.end(), warm_, s.pos); break;
+    case COLD:
+      warm_.splice(warm_.end(), cold_, s.pos);
+      s.temp = WARM;
+      if (warm_.size() > warm_size) {
+        index_[warm_.front()->key].temp = COLD;
+        cold_.splice(cold_.end(), warm_, warm_.begin());
+      }
+      break;
+    }
+    return m;
+  }
+
+  // Adds m (its key must not be listed); `evicted` receives what fell out.
+  void add(hip_module *m, std::vector<hip_module *> &evicted) {
+    hot_.push_back(m);
+    index_[m->key] = {HOT, std::prev(hot_.end())};
+    m->cached = true;
+    while (hot_.size() > hot_size) {
+      index_[hot_.front()->key].temp = COLD;
+      cold_.splice(cold_.end(), hot_, hot_.begin());
+    }
+    if (cold_.size() > cold_size + elasticity) {
+      while (cold_.size() > cold_size) {
+        hip_module *old = cold_.front();
+        cold_.pop_front();
+        index_.erase(old->key);
+        old->cached = false;
+        evicted.push_back(old);
+      }
+    }
+  }
+
+  void counts(size_t out[3]) const { out[0] = hot_.size(); out[1] = warm_.size(); out[2] = cold_.size(); }
+
+  // Empties the cache; every listed module is handed to `evicted`.
+  void clear(std::vector<hip_module *> &evicted) {
+    for (list_t *l : {&hot_, &warm_, &cold_}) {
+      for (hip_module *m : *l) {
+        m->cached = false;
+        evicted.push_back(m);
+      }
+      l->clear();
+    }
+    index_.clear();
+  }
+
+ private:
+  enum temp_t { HOT, WARM, COLD };
+  struct slot {
+    temp_t temp;
+    list_t::iterator pos;
+  };
+  list_t hot_, warm_, cold_;
+  std::unordered_map<std::string, slot> index_;
 };
 
 // ---- device memory cache ------------------------------------------------------
@@ -204,7 +283,8 @@ struct hip_context : _gpucontext {
   size_t maxthreads = 0;
   char devname[256] = {0};
   char pciid[16] = {0};
-  std::unordered_map<std::string, hip_module *> modcache;
+  module_cache modcache;
+  size_t live_modules = 0;   // loaded code objects, cached or still referenced
   gpudata *scratch = nullptr;
   size_t scratch_sz = 0;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -291,11 +371,15 @@ void ctx_destroy(hip_context *ctx) {
   if (ctx->errbuf) { hip_release(ctx->errbuf); ctx->errbuf = nullptr; }
   if (ctx->scratch) { hip_release(ctx->scratch); ctx->scratch = nullptr; }
   ctx->mem.destroy();
-  for (auto &kv : ctx->modcache) {
-    if (kv.second->mod) (void)hipModuleUnload(kv.second->mod);
-    delete kv.second;
+  {
+    // every kernel is gone by now (each one holds a reference to the context)
+    std::vector<hip_module *> gone;
+    ctx->modcache.clear(gone);
+    for (hip_module *m : gone) {
+      if (m->mod) (void)hipModuleUnload(m->mod);
+      delete m;
+    }
   }
-  ctx->modcache.clear();
   for (hipEvent_t e : ctx->evpool) (void)hipEventDestroy(e);
   if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
   if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
@@ -382,6 +466,17 @@ gpucontext *hip_init(gpucontext_props *p) {
   {
     const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
     if (dc != nullptr && *dc != 0) ctx->disk_cache = dc;
+  }
+  {
+    // "hot,warm,cold,elasticity" overrides the module cache's sizes
+    const char *mc = getenv("GPUARRAY_MODULE_CACHE");
+    unsigned long h, w, c, el;
+    if (mc != nullptr && sscanf(mc, "%lu,%lu,%lu,%lu", &h, &w, &c, &el) == 4 && h >= 1) {
+      ctx->modcache.hot_size = h;
+      ctx->modcache.warm_size = w;
+      ctx->modcache.cold_size = c;
+      ctx->modcache.elasticity = el;
+    }
   }
   ctx->mem.max = p->max_cache_size;
   if (p->initial_cache_size != 0 && ctx->mem.max != 0) {
@@ -761,11 +856,17 @@ void disk_store(const std::string &dir, const std::string &key, const std::vecto
   if (!ok || rename(tmp.c_str(), path.c_str()) != 0) (void)unlink(tmp.c_str());
 }
 
+// A module is unloaded when the cache has dropped it and no kernel uses it.
+void mod_reap(hip_context *ctx, hip_module *m) {
+  if (m->cached || m->refcnt != 0) return;
+  if (m->mod) (void)hipModuleUnload(m->mod);
+  if (ctx->live_modules > 0) ctx->live_modules--;
+  delete m;
+}
+
 void mod_unref(hip_context *ctx, hip_module *m) {
-  // Modules stay cached for the life of the context: recompiling costs
-  // hundreds of milliseconds, keeping one costs a few kilobytes.
-  (void)ctx;
   if (m->refcnt > 0) m->refcnt--;
+  mod_reap(ctx, m);
 }
 
 int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char **strings,
@@ -790,11 +891,8 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
   if ((err = enter(ctx)) != GA_NO_ERROR) return err;
 
   std::string src = join_sources(count, strings, lengths);
-  hip_module *m = nullptr;
-  auto it = ctx->modcache.find(src);
-  if (it != ctx->modcache.end()) {
-    m = it->second;
-  } else {
+  hip_module *m = ctx->modcache.get(src);
+  if (m == nullptr) {
     std::vector<char> code;
     std::string log, dkey;
     bool from_disk = false;
@@ -829,14 +927,21 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
       return hip_fail(ctx->err, "hipModuleLoadData", e);
     }
     m->key = src;
-    ctx->modcache.emplace(m->key, m);
+    ctx->live_modules++;
+    m->refcnt++;   // keeps it alive across the eviction pass below
+    std::vector<hip_module *> evicted;
+    ctx->modcache.add(m, evicted);
+    m->refcnt--;
+    for (hip_module *old : evicted) mod_reap(ctx, old);
   }
 
   hipFunction_t fn = nullptr;
   hipError_t e = hipModuleGetFunction(&fn, m->mod, fname);
-  if (e != hipSuccess)
+  if (e != hipSuccess) {
+    mod_reap(ctx, m);
     return ga_err_fmt(ctx->err, GA_IMPL_ERROR, "Kernel entry point \"%s\" not found: %s", fname,
                       hipGetErrorString(e));
+  }
 
   hip_kernel *k = (hip_kernel *)calloc(1, sizeof(hip_kernel));
   if (k == nullptr) return ga_err_sys(ctx->err, "calloc");
@@ -1147,6 +1252,15 @@ float ext_event_elapsed(gpucontext *c, unsigned int a, unsigned int b) {
   return ms;
 }
 
+// Entries in the hot, warm and cold lists of the module cache, and the number
+// of code objects currently loaded (cached or kept alive by a kernel).
+int ext_module_cache_stats(gpucontext *c, size_t out[4]) {
+  hip_context *ctx = HC(c);
+  ctx->modcache.counts(out);
+  out[3] = ctx->live_modules;
+  return GA_NO_ERROR;
+}
+
 struct ext_entry { const char *name; void *fn; };
 const ext_entry k_exts[] = {
     {"hip_get_stream", (void *)ext_get_stream},
@@ -1161,6 +1275,7 @@ const ext_entry k_exts[] = {
     {"hip_elemwise_source", (void *)ga_elemwise_gen_source},
     {"hip_reduction_source", (void *)ga_reduction_gen_source},
     {"hip_mapreduce_source", (void *)ga_mapreduce_gen_source},
+    {"hip_module_cache_stats", (void *)ext_module_cache_stats},
 };
 
 }  // namespace

@@ -381,3 +381,88 @@ def test_disk_kernel_cache(tmp_path):
         f.write(b"\0" * 256)
     run(ga.GpuContext("hip", 0, kernel_cache_path=d))
     assert open(files[0], "rb").read()[16 + kl:] == raw[16 + kl:]
+
+
+class _TwoQ(object):
+    """The reference's policy restated from src/cache/twoq.c:232-316, to
+    predict what the module cache holds."""
+
+    def __init__(self, hot, warm, cold, elasticity):
+        self.sizes = (hot, warm, cold, elasticity)
+        self.hot, self.warm, self.cold = [], [], []
+
+    def add(self, k):
+        hot, _, cold, el = self.sizes
+        self.hot.append(k)
+        while len(self.hot) > hot:
+            self.cold.append(self.hot.pop(0))
+        if len(self.cold) > cold + el:
+            while len(self.cold) > cold:
+                self.cold.pop(0)
+
+    def get(self, k):
+        if k in self.hot:
+            self.hot.remove(k); self.hot.append(k)
+        elif k in self.warm:
+            self.warm.remove(k); self.warm.append(k)
+        elif k in self.cold:
+            self.cold.remove(k); self.warm.append(k)
+            if len(self.warm) > self.sizes[1]:
+                self.cold.append(self.warm.pop(0))
+        else:
+            return False
+        return True
+
+    def cached(self):
+        return set(self.hot) | set(self.warm) | set(self.cold)
+
+
+def test_module_cache_follows_the_2q_policy(monkeypatch, tmp_path):
+    monkeypatch.setenv("GPUARRAY_MODULE_CACHE", "2,2,1,1")
+    c = ga.GpuContext("hip", 0, kernel_cache_path=str(tmp_path / "k"))
+    stats_fn = _lib.extension("hip_module_cache_stats", C.c_int, [C.c_void_p, C.POINTER(C.c_size_t)])
+
+    def stats():
+        out = (C.c_size_t * 4)()
+        assert stats_fn(c.ctx, out) == 0
+        return list(out)
+
+    base = stats()                       # whatever the context itself has built
+    assert base[3] == sum(base[:3])
+    model = _TwoQ(2, 2, 1, 1)
+    spec = [ga.arg("a", "float32", read=True), ga.arg("c", "float32", write=True)]
+    a = gpuarray.array(np.arange(100, dtype=np.float32), context=c)
+    out = gpuarray.empty((100,), "float32", context=c)
+    held = {}
+
+    def make(i):
+        k = ga.GpuElemwise(c, "c = a + %d.0f /* 2q test */" % i, spec)
+        if not model.get(i):
+            model.add(i)
+        return k
+
+    def check_counts(nheld_uncached):
+        s = stats()
+        assert s[:3] == [len(model.hot), len(model.warm), len(model.cold)], (s, model.__dict__)
+        assert s[3] == len(model.cached()) + nheld_uncached
+
+    assert base[:3] == [0, 0, 0]
+    for i in range(6):
+        held[i] = make(i)
+        uncached = [j for j in held if j not in model.cached()]
+        check_counts(len(uncached))
+    # entries that fell out stay loaded while an operator uses them, and run
+    uncached = [j for j in held if j not in model.cached()]
+    assert uncached, "the sizes above must have evicted something"
+    for j in held:
+        held[j](a, out)
+        assert np.array_equal(np.asarray(out), np.arange(100, dtype=np.float32) + j)
+    # dropping the operator of an evicted module unloads it
+    del held[uncached[0]]
+    check_counts(len(uncached) - 1)
+    # a hit in cold promotes to warm; making the same operator again compiles nothing new
+    cold_key = model.cold[0]
+    again = make(cold_key)
+    check_counts(len(uncached) - 1)
+    again(a, out)
+    assert np.array_equal(np.asarray(out), np.arange(100, dtype=np.float32) + cold_key)
