@@ -37,6 +37,11 @@ typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
  * < 0 on error. */
 typedef int (*ga_hip_event_record_fn)(gpucontext *ctx, unsigned int slot);
 typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsigned int b);
+/* "hip_take1_source": kernel text of GpuArray_take1 for result/source/index
+ * typecodes and `tnd` collapsed trailing dims; chunks != 0: the variant that
+ * moves dense aligned rows as 16-byte chunks. */
+typedef char *(*ga_hip_take1_source_fn)(int chunks, int a_typecode, int v_typecode,
+                                        int i_typecode, unsigned int tnd);
 /* "hip_module_cache_stats": out[0..2] = entries in the hot, warm and cold
  * lists of the context's loaded-module cache (the reference's 2Q policy,
  * src/cache/twoq.c), out[3] = code objects currently loaded. */

@@ -85,8 +85,16 @@ def main():
             check("map-reduce op=%d G=%d V=%d mask=%x" % (op, G, V, mask),
                   gen_m(op, red, neu, acc, b"", b"s*a*b", 3, margs, d0, G, V, U, mask))
             m += 1
-    print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, 9 elementwise)"
-          % (n + 5, m))
+    gen_t = ext(b"hip_take1_source", C.c_void_p, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint])
+    t = 0
+    for chunks, a_tc, v_tc, i_tc, tnd in [(1, GA_FLOAT, GA_FLOAT, GA_LONG, 1), (0, GA_FLOAT, GA_FLOAT, GA_INT, 1),
+                                          (0, GA_DOUBLE, GA_FLOAT, GA_UBYTE, 3), (0, GA_HALF, GA_HALF, GA_LONG, 2),
+                                          (0, GA_BOOL, GA_BOOL, GA_LONG, 1)]:
+        check("take1 chunks=%d types=%d,%d,%d nd=%d" % (chunks, a_tc, v_tc, i_tc, tnd),
+              gen_t(chunks, a_tc, v_tc, i_tc, tnd))
+        t += 1
+    print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
+          "9 elementwise)" % (n + 5, m, t))
 
 
 if __name__ == "__main__":

@@ -658,6 +658,77 @@ int GpuArray_fdump(FILE *fd, const GpuArray *a) {
   return GA_NO_ERROR;
 }
 
+}  // extern "C"
+
+// Kernel text of GpuArray_take1 for one combination of types and collapsed
+// trailing rank; `types` receives the argument typecodes.
+static std::string take1_source(bool chunks, int a_tc, int v_tc, int i_tc, unsigned int tnd,
+                                std::vector<int> &types) {
+    const gpuarray_type *ta = gpuarray_get_type(a_tc), *tv = gpuarray_get_type(v_tc),
+                      *ti = gpuarray_get_type(i_tc);
+    // halves move as their 16 bits (both sides are half then)
+    const std::string rt = chunks ? "t1_chunk" : (a_tc == GA_HALF ? "ga_ushort" : ta->cluda_name),
+                      vt = chunks ? "t1_chunk" : (v_tc == GA_HALF ? "ga_ushort" : tv->cluda_name);
+    std::string s = "#include \"cluda.h\"\n"
+                    "typedef ga_uint t1_chunk __attribute__((ext_vector_type(4)));\n"
+                    "KERNEL void __launch_bounds__(256) take1(GLOBAL_MEM " + rt +
+                    " *r, const ga_size r_off, GLOBAL_MEM const char *v, const ga_size v_off, "
+                    "const ga_ssize s0, const ga_size d0";
+    types = {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_SSIZE, GA_SIZE};
+    for (unsigned int d = 0; d < tnd; d++) {
+      char b[96];
+      snprintf(b, sizeof(b), ", const ga_ssize s%u, const ga_size d%u", d + 1, d + 1);
+      s += b;
+      types.push_back(GA_SSIZE);
+      types.push_back(GA_SIZE);
+    }
+    s += std::string(", GLOBAL_MEM const ") + ti->cluda_name +
+         " *ind, const ga_size i_off, const ga_size n0, const ga_size n1, const ga_uint gx, "
+         "const ga_uint lsh, GLOBAL_MEM ga_int *err) {\n"
+         "  const ga_uint lane = LID_0 & ((1u << lsh) - 1u);\n"
+         "  const ga_size row = (ga_size)(GID_0 / gx) * (256u >> lsh) + (LID_0 >> lsh);\n"
+         "  if (row >= n0) return;\n"
+         "  const ga_size x0 = (ga_size)(GID_0 % gx) * (4u << lsh) + lane;\n"
+         "  ind = (GLOBAL_MEM const " + ti->cluda_name + " *)((GLOBAL_MEM const char *)ind + i_off);\n"
+         "  ga_long ii = (ga_long)ind[row];\n"
+         "  if (ii < 0) ii += (ga_long)d0;\n"
+         "  if (ii < 0 || ii >= (ga_long)d0) { if (lane == 0) *err = -1; return; }\n"
+         "  v += v_off + ii * s0;\n"
+         "  r = (GLOBAL_MEM " + rt + " *)((GLOBAL_MEM char *)r + r_off) + row * n1;\n"
+         "  " + vt + " t[4];\n"
+         "#pragma unroll\n"
+         "  for (int e = 0; e < 4; e++) {\n"
+         "    const ga_size x = x0 + ((ga_size)e << lsh);\n"
+         "    if (x < n1) {\n"
+         "      ga_ssize p = 0; ga_size c = x;\n";
+    for (unsigned int d = tnd; d > 1; d--) {
+      char b[128];
+      snprintf(b, sizeof(b), "      p += (ga_ssize)(c %% d%u) * s%u; c /= d%u;\n", d, d, d);
+      s += b;
+    }
+    s += "      p += (ga_ssize)c * s1;\n"
+         "      t[e] = __builtin_nontemporal_load((GLOBAL_MEM const " + vt + " *)(v + p));\n"
+         "    }\n  }\n"
+         "#pragma unroll\n"
+         "  for (int e = 0; e < 4; e++) {\n"
+         "    const ga_size x = x0 + ((ga_size)e << lsh);\n";
+    if (chunks || a_tc == v_tc)
+      s += "    if (x < n1) __builtin_nontemporal_store(t[e], r + x);\n";
+    else
+      s += "    if (x < n1) r[x] = t[e];\n";
+    s += "  }\n}\n";
+    for (int t : {GA_BUFFER, GA_SIZE, GA_SIZE, GA_SIZE, GA_UINT, GA_UINT, GA_BUFFER}) types.push_back(t);
+    return s;
+}
+
+extern "C" GPUARRAY_PUBLIC char *ga_take1_gen_source(int chunks, int a_tc, int v_tc, int i_tc,
+                                                     unsigned int tnd) {
+  std::vector<int> types;
+  return strdup(take1_source(chunks != 0, a_tc, v_tc, i_tc, tnd, types).c_str());
+}
+
+extern "C" {
+
 // a[k, ...] = v[i[k], ...]  (reference :325-548).  Rules kept: a and i are
 // C-contiguous, i is 1-D with a's leading extent, trailing extents of a and v
 // agree, every array is aligned; a negative index counts from the end; an
@@ -665,9 +736,12 @@ int GpuArray_fdump(FILE *fd, const GpuArray *a) {
 // word, which `check_error` reads back (blocking), resets, and reports as
 // GA_VALUE_ERROR "Index out of bounds".
 // The kernel is a row copy: the trailing dims of v are collapsed on the host
-// (one dim when v's rows are dense), a group owns one output row and a chunk
-// of its columns, lanes run along the columns so both sides are coalesced, and
-// the index is read once per group instead of once per element.  Kernels are
+// (one dim when v's rows are dense); a power-of-two number of lanes shares an
+// output row (a group of 256 lanes holds 256/lanes rows, so short rows still
+// fill it), lanes run along the columns so both sides are coalesced, every
+// lane has up to four streaming loads in flight before it stores, and the
+// index is read once per lane instead of once per element.  Dense aligned
+// rows of one type on both sides move as 16-byte chunks.  Kernels are
 // kept per context by (types, collapsed rank), so repeated calls compile
 // nothing; the reference rebuilds its kernel on every call (:469-477).
 int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_error) {
@@ -697,10 +771,11 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
                         a->dimensions[j], j, v->dimensions[j]);
     n1 *= v->dimensions[j];
   }
-  const gpuarray_type *ta = gpuarray_get_type(a->typecode), *tv = gpuarray_get_type(v->typecode),
-                      *ti = gpuarray_get_type(i->typecode);
+  const gpuarray_type *tv = gpuarray_get_type(v->typecode);
   if (i->typecode < GA_BYTE || i->typecode > GA_ULONG)
     return ga_err_set(ctx->err, GA_VALUE_ERROR, "Index array must have an integer type");
+  if (gpuarray_type_flags(a->typecode, v->typecode, -1) & GA_USE_COMPLEX)
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Complex types are not supported");
   if (n0 == 0 || n1 == 0) return GA_NO_ERROR;
 
   // collapse v's trailing dims into as few strided runs as possible
@@ -716,70 +791,49 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
     gpuarray_elemwise_collapse(1, &tnd, tdims.data(), &row);
   }
 
+  if ((a->typecode == GA_HALF) != (v->typecode == GA_HALF))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "take1 between half and another type");
+
+  // Rows that are dense, of the same type on both sides and 16-byte aligned
+  // move as 16-byte chunks whatever the element type.
+  const size_t elsz = tv->size;
+  bool chunks = a->typecode == v->typecode && tnd == 1 && (tstr[0] == (ssize_t)elsz || n1 == 1) &&
+                (n1 * elsz) % 16 == 0 && v->strides[0] % 16 == 0 &&
+                ((uintptr_t)v->data->devptr + v->offset) % 16 == 0 &&
+                ((uintptr_t)a->data->devptr + a->offset) % 16 == 0;
+  size_t n1e = n1;               // elements (or chunks) per row
+  if (chunks) {
+    n1e = n1 * elsz / 16;
+    tdims[0] = n1e;
+    tstr[0] = 16;
+  }
+  // lanes per row: a power of two, each lane moves up to four elements
+  unsigned int lsh = 0;
+  while (lsh < 8 && ((size_t)4 << lsh) < n1e) lsh++;
+  const size_t rpg = (size_t)256 >> lsh;                     // rows per group
+  const size_t gx = (n1e + ((size_t)4 << lsh) - 1) / ((size_t)4 << lsh);
+  const size_t gy = (n0 + rpg - 1) / rpg;
+  if (gx > 0xffffffffull || gy > 0x7fffffffull / gx)
+    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "take1 needs more groups than one launch has");
+
   typedef std::map<std::string, GpuKernel> cache_t;
   void **slot = ga_hip_take1_cache_slot(ctx);
   if (*slot == nullptr) *slot = new cache_t();
   cache_t &cache = *(cache_t *)*slot;
   char key[64];
-  snprintf(key, sizeof(key), "%d:%d:%d:%u", a->typecode, v->typecode, i->typecode, tnd);
+  if (chunks) snprintf(key, sizeof(key), "c:%d", i->typecode);
+  else snprintf(key, sizeof(key), "%d:%d:%d:%u", a->typecode, v->typecode, i->typecode, tnd);
   GpuKernel *k;
   auto it = cache.find(key);
   if (it != cache.end()) {
     k = &it->second;
   } else {
-    std::string s = "#include \"cluda.h\"\nKERNEL void __launch_bounds__(256) take1(GLOBAL_MEM ";
-    s += ta->cluda_name;
-    s += " *r, const ga_size r_off, GLOBAL_MEM const char *v, const ga_size v_off, "
-         "const ga_ssize s0, const ga_size d0";
-    std::vector<int> types = {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_SSIZE, GA_SIZE};
-    for (unsigned int d = 0; d < tnd; d++) {
-      char b[96];
-      snprintf(b, sizeof(b), ", const ga_ssize s%u, const ga_size d%u", d + 1, d + 1);
-      s += b;
-      types.push_back(GA_SSIZE);
-      types.push_back(GA_SIZE);
-    }
-    s += ", GLOBAL_MEM const ";
-    s += ti->cluda_name;
-    s += " *ind, const ga_size i_off, const ga_size n1, const ga_uint gx, GLOBAL_MEM ga_int *err) {\n"
-         "  const ga_size row = GID_0 / gx;\n"
-         "  const ga_size x0 = (ga_size)(GID_0 % gx) * 1024u + LID_0;\n"
-         "  ind = (GLOBAL_MEM const ";
-    s += ti->cluda_name;
-    s += " *)((GLOBAL_MEM const char *)ind + i_off);\n"
-         "  ga_long ii = (ga_long)ind[row];\n"
-         "  if (ii < 0) ii += (ga_long)d0;\n"
-         "  if (ii < 0 || ii >= (ga_long)d0) { if (LID_0 == 0) *err = -1; return; }\n"
-         "  v += v_off + ii * s0;\n"
-         "  r = (GLOBAL_MEM ";
-    s += ta->cluda_name;
-    s += " *)((GLOBAL_MEM char *)r + r_off) + row * n1;\n"
-         "#pragma unroll\n"
-         "  for (int e = 0; e < 4; e++) {\n"
-         "    const ga_size x = x0 + (ga_size)e * 256u;\n"
-         "    if (x < n1) {\n"
-         "      ga_ssize p = 0; ga_size c = x;\n";
-    for (unsigned int d = tnd; d > 1; d--) {
-      char b[128];
-      snprintf(b, sizeof(b), "      p += (ga_ssize)(c %% d%u) * s%u; c /= d%u;\n", d, d, d);
-      s += b;
-    }
-    s += "      p += (ga_ssize)c * s1;\n      r[x] = *(GLOBAL_MEM const ";
-    s += tv->cluda_name;
-    s += " *)(v + p);\n    }\n  }\n}\n";
-    types.push_back(GA_BUFFER);
-    types.push_back(GA_SIZE);
-    types.push_back(GA_SIZE);
-    types.push_back(GA_UINT);
-    types.push_back(GA_BUFFER);
+    std::vector<int> types;
+    std::string s = take1_source(chunks, a->typecode, v->typecode, i->typecode, tnd, types);
     const char *strs[1] = {s.c_str()};
     size_t lens[1] = {s.size()};
     GpuKernel nk = {nullptr, nullptr};
     int flags = gpuarray_type_flags(a->typecode, v->typecode, i->typecode, -1);
-    if (a->typecode == GA_HALF || v->typecode == GA_HALF) {
-      if (a->typecode != v->typecode)
-        return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "take1 between half and another type");
-    }
     int err = GpuKernel_init(&nk, ctx, 1, strs, lens, "take1", (unsigned)types.size(), types.data(),
                              flags, nullptr);
     if (err != GA_NO_ERROR) return err;
@@ -789,9 +843,6 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
   gpudata *errbuf = nullptr;
   int err = gpudata_property(v->data, GA_CTX_PROP_ERRBUF, &errbuf);
   if (err != GA_NO_ERROR) return err;
-  const size_t gx = (n1 + 1023) / 1024;
-  if (gx > 0xffffffffull || n0 > 0x7fffffffull / gx)
-    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "take1 needs more groups than one launch has");
   unsigned int gx32 = (unsigned int)gx, p = 0;
   GpuKernel_setarg(k, p++, a->data);
   GpuKernel_setarg(k, p++, (void *)&a->offset);
@@ -805,10 +856,12 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
   }
   GpuKernel_setarg(k, p++, i->data);
   GpuKernel_setarg(k, p++, (void *)&i->offset);
-  GpuKernel_setarg(k, p++, &n1);
+  GpuKernel_setarg(k, p++, &n0);
+  GpuKernel_setarg(k, p++, &n1e);
   GpuKernel_setarg(k, p++, &gx32);
+  GpuKernel_setarg(k, p++, &lsh);
   GpuKernel_setarg(k, p++, errbuf);
-  size_t groups = gx * n0, ls = 256;
+  size_t groups = gx * gy, ls = 256;
   err = GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
   if (check_error && err == GA_NO_ERROR) {
     int kerr = 0;

@@ -1219,6 +1219,7 @@ extern "C" char *ga_elemwise_gen_source(const char *preamble, const char *expr, 
                                         unsigned int nd, int idx64, unsigned int tmask);
 extern "C" char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int d1_tc, unsigned int G,
                                          unsigned int V, unsigned int U);
+extern "C" char *ga_take1_gen_source(int chunks, int a_tc, int v_tc, int i_tc, unsigned int tnd);
 extern "C" char *ga_mapreduce_gen_source(int op, const char *reduce_expr, const char *neutral,
                                          int acc_tc, const char *preamble, const char *map_expr,
                                          unsigned int n, const gpuelemwise_arg *args, int d0_tc,
@@ -1276,6 +1277,7 @@ const ext_entry k_exts[] = {
     {"hip_reduction_source", (void *)ga_reduction_gen_source},
     {"hip_mapreduce_source", (void *)ga_mapreduce_gen_source},
     {"hip_module_cache_stats", (void *)ext_module_cache_stats},
+    {"hip_take1_source", (void *)ga_take1_gen_source},
 };
 
 }  // namespace

@@ -722,8 +722,12 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     int64_t per_pass = (int64_t)G * V;
     U = (unsigned)env_ul("GPUARRAY_REDUX_U", 8);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 8;
-    // several sources share the lane's registers
-    while (U > 1 && (int64_t)U * V * ES * elsz_sum > 128) U /= 2;
+    // Bytes a lane keeps in flight over all sources.  Measured on MI355X
+    // (dot product of two 2^27-float vectors): 64 bytes per lane with 4 groups
+    // per compute unit 162 us, 128 bytes with 2 groups 179 us; one source
+    // keeps the 128 bytes its sweep found best.
+    const int64_t lane_bytes = (int64_t)env_ul("GPUARRAY_REDUX_LANE_BYTES", K > 1 ? 64 : 128);
+    while (U > 1 && (int64_t)U * V * ES * elsz_sum > lane_bytes) U /= 2;
     while (U > 1 && per_pass * (U / 2) >= rin) U /= 2;
     const int64_t seg = per_pass * U;
     p.nseg = rin > 0 ? (rin + seg - 1) / seg : 1;
