@@ -454,7 +454,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // the expression runs on 4 consecutive x of one y row; transposed writes
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
-                            unsigned umask, std::vector<int> &ktypes) {
+                            unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
@@ -492,6 +492,22 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   auto is_t = [&](size_t j) { return aidx[j] >= 0 && ((tmask >> aidx[j]) & 1u); };
   auto is_u = [&](size_t j) { return aidx[j] >= 0 && ((umask >> aidx[j]) & 1u); };
   auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * 4); };
+  // 16-byte accesses of arrays whose every element is touched once carry the
+  // streaming hint (ntmask); broadcast operands stay cacheable
+  auto is_nt = [&](size_t j) { return aidx[j] >= 0 && ((ntmask >> aidx[j]) & 1u); };
+  auto quad_load = [&](size_t j, const std::string &dst, const std::string &ptr_expr) {
+    // ptr_expr is "*(T *)(addr)": strip the leading '*' to get the pointer
+    std::string o;
+    if (is_nt(j)) appendf(o, "%s = __builtin_nontemporal_load(%s);\n", dst.c_str(), ptr_expr.c_str() + 1);
+    else appendf(o, "%s = %s;\n", dst.c_str(), ptr_expr.c_str());
+    return o;
+  };
+  auto quad_store = [&](size_t j, const std::string &ptr_expr, const std::string &val) {
+    std::string o;
+    if (is_nt(j)) appendf(o, "__builtin_nontemporal_store(%s, %s);\n", val.c_str(), ptr_expr.c_str() + 1);
+    else appendf(o, "%s = %s;\n", ptr_expr.c_str(), val.c_str());
+    return o;
+  };
 
   for (const ge_arg &a : ge->args)
     if (a.is_array())
@@ -549,7 +565,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || !a.reads()) continue;
       if (is_u(j)) {
-        appendf(s, "%s_u[ga_e].c = %s;\n", a.name.c_str(), quad_at(a, a.name + "_o", "ga_x").c_str());
+        s += quad_load(j, a.name + "_u[ga_e].c", quad_at(a, a.name + "_o", "ga_x"));
       } else {
         for (int i = 0; i < 4; i++) {
           char xi[32];
@@ -575,7 +591,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || !a.writes()) continue;
       if (is_u(j)) {
-        appendf(s, "%s = %s_u[ga_e].c;\n", quad_at(a, a.name + "_o", "ga_x").c_str(), a.name.c_str());
+        s += quad_store(j, quad_at(a, a.name + "_o", "ga_x"), a.name + "_u[ga_e].c");
       } else {
         for (int i = 0; i < 4; i++) {
           char xi[32];
@@ -641,8 +657,12 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
-      appendf(s, "%s_in[ga_k].c = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), quad_t(a),
-              a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+      {
+        std::string pe;
+        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
+                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+        s += quad_load(j, a.name + "_in[ga_k].c", pe);
+      }
     }
     s += "}\n}\n";
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
@@ -670,8 +690,10 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     const ge_arg &a = ge->args[j];
     if (!a.is_array() || is_t(j) || !a.reads()) continue;
     if (is_u(j)) {
-      appendf(s, "%s_u[ga_k].c = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), quad_t(a),
-              a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+      std::string pe;
+      appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
+              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+      s += quad_load(j, a.name + "_u[ga_k].c", pe);
     } else {
       for (int i = 0; i < 4; i++) {
         char xi[48];
@@ -705,8 +727,10 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     const ge_arg &a = ge->args[j];
     if (!a.is_array() || is_t(j) || !a.writes()) continue;
     if (is_u(j)) {
-      appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].c;\n", quad_t(a), a.name.c_str(),
-              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str(), a.name.c_str());
+      std::string pe;
+      appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
+              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+      s += quad_store(j, pe, a.name + "_u[ga_k].c");
     } else {
       for (int i = 0; i < 4; i++) {
         char xi[48];
@@ -728,8 +752,13 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       appendf(s, "{ union { %s c; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
                  "ga_o.e[ga_i] = %s_t[(ga_ly + ga_i) * 65u + ga_lx];\n",
               quad_t(a), ctype(a.typecode), a.name.c_str());
-      appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = ga_o.c; }\n", quad_t(a), a.name.c_str(),
-              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+      {
+        std::string pe;
+        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
+                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+        s += quad_store(j, pe, "ga_o.c");
+        s += "}\n";
+      }
     }
     s += "}\n}\n";
   }
@@ -999,6 +1028,17 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     }
   }
   if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
+  // arrays read or written exactly once per element stream past the caches
+  unsigned ntmask = 0;
+  if (vec4 && ge->nontemporal) {
+    for (unsigned k = 0; k < na; k++) {
+      bool once = true;
+      for (unsigned j = 0; j < nd && once; j++)
+        if (dims[j] > 1 && strs[k][j] == 0) once = false;
+      if (once) ntmask |= 1u << k;
+    }
+    ntmask &= (unsigned)env_ul("GPUARRAY_ELEMWISE_NT_MASK", 0xffffffffu);
+  }
 
   // launch geometry
   size_t gx, groups;
@@ -1022,15 +1062,15 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
 
   char key[64];
-  snprintf(key, sizeof(key), "%s%u:%d:%x:%x", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-           vec4 ? umask : 0u);
+  snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+           vec4 ? umask : 0u, ntmask);
   GpuKernel *k;
   auto it = ge->k_strided.find(key);
   if (it != ge->k_strided.end()) {
     k = &it->second;
   } else {
     std::vector<int> ktypes;
-    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes)
+    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask)
                            : gen_strided(ge, nd, idx64, tmask, ktypes);
     GpuKernel nk = {nullptr, nullptr};
     int err = build_kernel(ge, &nk, src, ktypes);
@@ -1110,8 +1150,10 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
     return nullptr;
   std::vector<int> ktypes;
   // strided: 0 flat, 1 strided one element per lane, 2 strided four elements per
-  // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride)
-  std::string src = strided == 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes)
+  // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride),
+  // 3 the same with streaming 16-byte accesses on every array
+  std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
+                                                   strided == 3 ? 0xffffffffu : 0u)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());
