@@ -454,12 +454,13 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // the expression runs on 4 consecutive x of one y row; transposed writes
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
-                            unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0) {
+                            unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
+                            unsigned tile = 64) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
   emit_header(ge, s);
-  s += "KERNEL void __launch_bounds__(256) elem(";
+  appendf(s, "KERNEL void __launch_bounds__(%u) elem(", tmask ? tile * tile / 16 : 256u);
   for (unsigned d = 0; d < nd; d++) {
     appendf(s, "%sconst ga_size dim%u", d ? ", " : "", d);
     ktypes.push_back(GA_SIZE);
@@ -607,15 +608,29 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
 
   // ---- transposed, nd >= 2 ----
   const unsigned yd = nd - 2;
+  const unsigned T = tile, Q = tile / 4;
+  const std::string TP = std::to_string(T + 1) + "u";
   for (size_t j = 0; j < ge->args.size(); j++)
     if (is_t(j))
-      appendf(s, "LOCAL_MEM %s %s_t[64 * 65];\n", ctype(ge->args[j].typecode),
-              ge->args[j].name.c_str());
-  appendf(s, "const %s ga_lo = LID_0 & 15u;\nconst %s ga_hi = LID_0 >> 4;\n", N, N);
-  appendf(s, "const %s ga_gy = ((%s)dim%u + 63u) / 64u;\n", N, N, yd);
-  appendf(s, "const %s ga_bx = GID_0 %% ga_gx;\n", N);
-  appendf(s, "%s ga_r = GID_0 / ga_gx;\n", N);
-  appendf(s, "const %s ga_by = ga_r %% ga_gy;\nga_r = ga_r / ga_gy;\n", N);
+      appendf(s, "LOCAL_MEM %s %s_t[%u * %u];\n", ctype(ge->args[j].typecode),
+              ge->args[j].name.c_str(), T, T + 1);
+  // T x T tile, T*T/16 lanes: ga_lo picks a quad along one axis, ga_hi a line
+  // along the other; four passes of T/4 lines cover the tile
+  appendf(s, "const %s ga_lo = LID_0 & %uu;\nconst %s ga_hi = LID_0 / %uu;\n", N, Q - 1, N, Q);
+  appendf(s, "const %s ga_gy = ((%s)dim%u + %uu) / %uu;\n", N, N, yd, T - 1, T);
+  // Tiles of one plane are handed out in bands of ga_ltx tile rows, walking
+  // down a band's rows first: groups that run together then read runs that
+  // are adjacent in the transposed operand's memory and write runs that are
+  // adjacent in the output's (ga_ltx = 1: plain row-major order).
+  appendf(s, "const %s ga_pl = ga_gx * ga_gy;\n", N);
+  appendf(s, "%s ga_r = GID_0 / ga_pl;\n", N);
+  appendf(s, "const %s ga_g = GID_0 - ga_r * ga_pl;\n", N);
+  appendf(s, "const %s ga_band = ga_g / (ga_ltx * ga_gx);\n", N);
+  appendf(s, "const %s ga_in = ga_g - ga_band * ga_ltx * ga_gx;\n", N);
+  appendf(s, "const %s ga_left = ga_gy - ga_band * ga_ltx;\n", N);
+  appendf(s, "const %s ga_bh = ga_left < (%s)ga_ltx ? ga_left : (%s)ga_ltx;\n", N, N, N);
+  appendf(s, "const %s ga_bx = ga_in / ga_bh;\n", N);
+  appendf(s, "const %s ga_by = ga_band * ga_ltx + (ga_in - ga_bx * ga_bh);\n", N);
   for (const ge_arg &a : ge->args)
     if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
   if (nd >= 3) {
@@ -629,7 +644,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     }
     s += "}\n";
   }
-  appendf(s, "const %s ga_x0 = ga_bx * 64u;\nconst %s ga_y0 = ga_by * 64u;\n", N, N);
+  appendf(s, "const %s ga_x0 = ga_bx * %uu;\nconst %s ga_y0 = ga_by * %uu;\n", N, T, N, T);
   // byte offset of (y, x) for array a
   auto off_yx = [&](const ge_arg &a, const char *y, const char *x) {
     std::string o;
@@ -652,7 +667,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
                 a.name.c_str());
     }
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
@@ -666,14 +681,14 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     }
     s += "}\n}\n";
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
       appendf(s, "#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
-                 "%s_t[(ga_ly + ga_i) * 65u + ga_lx] = %s_in[ga_k].e[ga_i];\n",
-              a.name.c_str(), a.name.c_str());
+                 "%s_t[(ga_ly + ga_i) * %uu + ga_lx] = %s_in[ga_k].e[ga_i];\n",
+              a.name.c_str(), T + 1, a.name.c_str());
     }
     s += "}\n}\nlocal_barrier();\n";
   }
@@ -684,7 +699,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), a.name.c_str());
   }
   s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + 16u * (%s)ga_k;\n", N, N);
+  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
   appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
@@ -705,13 +720,13 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   }
   s += "}\n}\n";
   s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + 16u * (%s)ga_k;\n", N, N);
+  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
   appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
   s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * 65u + ga_lx + ga_v]");
+    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * " + TP + " + ga_lx + ga_v]");
     else emit_load(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += ge->expr;
@@ -719,7 +734,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * 65u + ga_lx + ga_v]");
+    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * " + TP + " + ga_lx + ga_v]");
     else emit_store(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += "}\n";
@@ -744,14 +759,14 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // phase 3: transposed writes, mirror of phase 1
   if (any_tw) {
     s += "local_barrier();\n#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + 16u * (%s)ga_k;\n", N, N);
+    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.writes()) continue;
       appendf(s, "{ union { %s c; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
-                 "ga_o.e[ga_i] = %s_t[(ga_ly + ga_i) * 65u + ga_lx];\n",
-              quad_t(a), ctype(a.typecode), a.name.c_str());
+                 "ga_o.e[ga_i] = %s_t[(ga_ly + ga_i) * %uu + ga_lx];\n",
+              quad_t(a), ctype(a.typecode), a.name.c_str(), T + 1);
       {
         std::string pe;
         appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
@@ -1042,7 +1057,7 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
 
   // launch geometry
   size_t gx, groups;
-  unsigned ltx = 0;
+  unsigned ltx = 0, tile = 64;
   if (tmask == 0) {
     size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
     ltx = vec4 ? 0 : 4;
@@ -1052,8 +1067,30 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     gx = (inner + 4 * tx - 1) / (4 * tx);
     groups = gx * ((rows + ty - 1) / ty);
   } else {
-    gx = (dims[nd - 1] + 63) / 64;
-    size_t gy = (dims[nd - 2] + 63) / 64;
+    // Transposed tiles.  A group takes a 64 x 64 tile (256 lanes) or a
+    // 128 x 128 tile (1024 lanes); the tiles of a plane are handed out in bands
+    // of `ltx` tile rows, down a band's rows first.  Measured on MI355X for
+    // out = in.T of n x n floats: n = 4096 (4096 small tiles) 26.8 us with
+    // small tiles in row-major order, 27.6-28.8 with large ones; n = 8192
+    // 112.6 us small row-major, 106.2 small in bands of 8, 91.3 / 93.3 / 89.8
+    // large in bands of 1 / 2 / 4.  So the large tile is used when it still
+    // gives every compute unit eight groups and its staging copies leave room
+    // for two groups per unit.
+    if (vec4) {
+      size_t lds128 = 0;
+      for (unsigned k = 0; k < na; k++)
+        if ((tmask >> k) & 1u) lds128 += (size_t)128 * 129 * elsz[k];
+      const size_t tiles128 = ((dims[nd - 1] + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
+                              (n / dims[nd - 1] / dims[nd - 2]);
+      tile = (tiles128 >= (size_t)8 * ga_hip_numprocs(ctx) && lds128 <= 80 * 1024) ? 128 : 64;
+      const unsigned long ft = env_ul("GPUARRAY_ELEMWISE_TTILE", 0);
+      if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
+      const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
+      ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", tile == 128 ? 4 : (tiles >= 8192 ? 8 : 1));
+      if (ltx < 1) ltx = 1;
+    }
+    gx = (dims[nd - 1] + tile - 1) / tile;
+    size_t gy = (dims[nd - 2] + tile - 1) / tile;
     size_t outer = n / dims[nd - 1] / dims[nd - 2];
     groups = gx * gy * outer;
   }
@@ -1062,15 +1099,15 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
     return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
 
   char key[64];
-  snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-           vec4 ? umask : 0u, ntmask);
+  snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+           vec4 ? umask : 0u, ntmask, tile);
   GpuKernel *k;
   auto it = ge->k_strided.find(key);
   if (it != ge->k_strided.end()) {
     k = &it->second;
   } else {
     std::vector<int> ktypes;
-    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask)
+    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile)
                            : gen_strided(ge, nd, idx64, tmask, ktypes);
     GpuKernel nk = {nullptr, nullptr};
     int err = build_kernel(ge, &nk, src, ktypes);
@@ -1097,7 +1134,7 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
   unsigned int gx32 = (unsigned int)gx;
   if ((err = GpuKernel_setarg(k, p++, &gx32)) != GA_NO_ERROR) return err;
   if ((err = GpuKernel_setarg(k, p++, &ltx)) != GA_NO_ERROR) return err;
-  size_t ls = 256;
+  size_t ls = (vec4 && tmask) ? (size_t)tile * tile / 16 : 256;
   return GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
 }
 
@@ -1151,9 +1188,10 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   std::vector<int> ktypes;
   // strided: 0 flat, 1 strided one element per lane, 2 strided four elements per
   // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride),
-  // 3 the same with streaming 16-byte accesses on every array
+  // 3 the same with streaming 16-byte accesses on every array, 4 as 3 with
+  // 128 x 128 transposed tiles
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
-                                                   strided == 3 ? 0xffffffffu : 0u)
+                                                   strided >= 3 ? 0xffffffffu : 0u, strided == 4 ? 128 : 64)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

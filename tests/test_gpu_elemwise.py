@@ -398,3 +398,42 @@ def test_linearity_at_full_size(ctx):
         got = np.asarray(c[lo:lo + 10000])
         want = (np.arange(lo, lo + 10000) & 1023).astype(np.float32) + np.float32(0.5)
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("tile,band", [(64, 1), (64, 3), (64, 8), (128, 1), (128, 2), (128, 5)])
+def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band):
+    """Every tile size and band height of the transposed kernels, on extents
+    that leave ragged tiles and a partial last band, with one and with two
+    transposed operands, a transposed result, several planes and 8-byte
+    elements: bit-exact against NumPy."""
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_TTILE", str(tile))
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_BAND", str(band))
+    rng = np.random.default_rng(40 + tile + band)
+    f32 = "float32"
+    k2 = ga.GpuElemwise(ctx, "out = a + b*c", [arg("a", f32, read=True), arg("b", f32, read=True),
+                                               arg("c", f32, read=True), arg("out", f32, write=True)])
+    for ny, nx in ((516, 260), (128, 128), (1100, 68), (68, 1100), (644, 388)):
+        a = rng.standard_normal((nx, ny)).astype(np.float32)        # used as a.T: (ny, nx)
+        b = rng.standard_normal((1, nx)).astype(np.float32)
+        c = rng.standard_normal((ny, 1)).astype(np.float32)
+        out = gpuarray.empty((ny, nx), f32, context=ctx)
+        k2(gpuarray.array(a, context=ctx).T, gpuarray.array(b, context=ctx),
+           gpuarray.array(c, context=ctx), out)
+        assert np.array_equal(np.asarray(out), a.T + b * c), (ny, nx)
+        # two transposed inputs
+        a2 = rng.standard_normal((nx, ny)).astype(np.float32)
+        k2(gpuarray.array(a, context=ctx).T, gpuarray.array(a2, context=ctx).T,
+           gpuarray.array(c, context=ctx), out)
+        assert np.array_equal(np.asarray(out), a.T + a2.T * c), (ny, nx)
+        # transposed result: out.T written from C-ordered inputs
+        outT = gpuarray.empty((nx, ny), f32, context=ctx)
+        x = rng.standard_normal((ny, nx)).astype(np.float32)
+        k2(gpuarray.array(x, context=ctx), gpuarray.array(b, context=ctx),
+           gpuarray.array(c, context=ctx), outT.T)
+        assert np.array_equal(np.asarray(outT), (x + b * c).T), (ny, nx)
+    # planes (nd = 3) and 8-byte elements
+    kd = ga.GpuElemwise(ctx, "o = p * 2.0", [arg("p", "float64", read=True), arg("o", "float64", write=True)])
+    p = rng.standard_normal((3, 264, 392))
+    o = gpuarray.empty((3, 392, 264), "float64", context=ctx)
+    kd(gpuarray.array(p, context=ctx).transpose(0, 2, 1), o)
+    assert np.array_equal(np.asarray(o), p.transpose(0, 2, 1) * 2.0)
