@@ -179,6 +179,7 @@ struct variant_spec {
   int d0_tc, d1_tc;
   unsigned G, V, U, opts, ES;
   unsigned vecmask;   // bit k: array source k is fetched with vector loads
+  unsigned RB;        // redux_wrows: rows per batch of loads
 };
 
 const char *load_type_name(int tc) {
@@ -234,8 +235,8 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
         neutral_for(kind, kind == K_ALL || kind == K_ANY ? GA_UINT : acc_tc).c_str());
   }
   DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", vs.G, vs.V, vs.U);
-  DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n", vs.opts & 1u,
-      (vs.opts >> 1) & 1u, vs.ES);
+  DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n#define RD_RB %u\n",
+      vs.opts & 1u, (vs.opts >> 1) & 1u, vs.ES, vs.RB ? vs.RB : 1u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -336,8 +337,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
-           vs.opts, vs.ES, vs.vecmask);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
+           vs.opts, vs.ES, vs.vecmask, vs.RB);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -660,7 +661,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1;
   bool wrows = false;
   size_t groups;
   if (use_row) {
@@ -764,13 +765,18 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     p.nsplit = (int)nsplit;
     groups = (size_t)(rowgroups * nsplit);
     // Short rows, one wavefront each, take the kernel without the unit loop.
-    // It can walk several rows per wavefront with the next row's loads in
-    // flight, but on MI355X one row per wavefront measured best (65536 rows
-    // of 1000 floats: 43 us with 1 row, 45 / 47 / 52 us with 2 / 4 / 8), so
-    // that is the default.
+    // A wavefront takes RB rows at a time and issues their loads together:
+    // a row that is a single load per lane would otherwise leave the
+    // wavefront with one load in flight.
     if (G == 64 && nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
       wrows = true;
-      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", 1);
+      // Measured on MI355X: any() over 131072 rows of 512 stepped bytes 29.8 us
+      // one row at a time, 24.8 us with batches of 4 and 8 rows per wavefront;
+      // rows of 1000 floats (four loads per lane already) 45 us one at a time,
+      // 66 / 92 us in batches of 2 / 4.
+      RB = (unsigned)env_ul("GPUARRAY_REDUX_RB", U == 1 ? 4 : 1);
+      if (RB != 1 && RB != 2 && RB != 4 && RB != 8) RB = 1;
+      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", RB == 1 ? 1 : 2 * RB);
       if (rpw < 1) rpw = 1;
       p.upb = rpw;
       const int64_t waves = (nrows + rpw - 1) / rpw;
@@ -802,7 +808,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
   if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
-                     use_row ? vecmask : (1u << K) - 1};
+                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1};
   variant *var = nullptr;
   int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
@@ -864,11 +870,12 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   GpuReduction *gr = nullptr;
   if (make_plain_operator(&gr, nullptr, ga_global_err, (ga_reduce_op)op, src_tc) != GA_NO_ERROR)
     return nullptr;
-  // bits 8.. of V carry the element step of strided loads (0 means 1)
+  // bits 8.. of V carry the element step of strided loads (0 means 1), bits
+  // 8.. of U the rows per batch of redux_wrows (0 means 1)
   const unsigned ES = (V >> 8) ? (V >> 8) : 1;
   V &= 0xffu;
   std::string s;
-  variant_spec vs = {d0_tc, d1_tc, G, V, U, 3, ES, 1};
+  variant_spec vs = {d0_tc, d1_tc, G, V, U & 0xffu, 3, ES, 1, (U >> 8) ? (U >> 8) : 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
@@ -885,7 +892,7 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask};
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

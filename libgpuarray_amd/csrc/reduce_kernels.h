@@ -22,6 +22,7 @@
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
  *   RD_U        loads in flight per lane
+ *   RD_RB       redux_wrows: rows whose loads a wavefront issues together
  *   RD_NT       streaming (non-temporal) loads in redux_row
  *   RD_INTERLEAVE  redux_row with one reduced dim: splits take every
  *               nsplit-th unit instead of a contiguous range
@@ -54,8 +55,8 @@
  *                cooperate on one output; a row can be cut in `nsplit` pieces
  *                that each leave a partial.
  *   redux_wrows  the same for short rows (one pass of a wavefront covers a
- *                row): a wavefront walks several rows and has the next row's
- *                loads in flight while it combines the current one.
+ *                row): a wavefront takes several rows at a time and issues all
+ *                their loads before it combines the first.
  *   redux_col    lanes run along the fastest FREE dim (coalesced), each lane
  *                owns one output and walks the reduced range; 4 lane rows
  *                share the range and meet in LDS.
@@ -483,10 +484,14 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
 
 /* ---- redux_wrows -----------------------------------------------------------
  * Rows that one pass of a wavefront covers (at most one reduced dim, one
- * unit per row, no split).  Wavefront w owns rows [w*upb, (w+1)*upb); the
- * loads of row r+1 are issued before row r is combined, so memory latency
- * overlaps the cross-lane work.  Only built for RD_G == 64. */
+ * unit per row, no split).  Wavefront w owns rows [w*upb, (w+1)*upb) and takes
+ * them RD_RB at a time: the loads of the whole batch are issued before the
+ * first row is combined, so a wavefront whose row is a single load per lane
+ * still has RD_RB loads in flight.  Only built for RD_G == 64. */
 #if RD_G == 64
+#if RD_RB == 1
+/* one row at a time; with upb > 1 the next row's loads are issued before the
+ * current row is combined */
 KERNEL void __launch_bounds__(256)
 redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
             const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
@@ -534,6 +539,53 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
     d0o = nd0o; d1o = nd1o;
   }
 }
+#else
+KERNEL void __launch_bounds__(256)
+redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const rd_plan p RD_SCALAR_PARAMS) {
+  (void)part_v; (void)part_i;
+  const unsigned lane = LID_0 & 63u;
+  const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
+  ga_long row = wave * p.upb;
+  ga_long row_end = row + p.upb;
+  if (row_end > p.nrows) row_end = p.nrows;
+  if (row >= row_end) return;
+
+  const ga_long rin = p.nr > 0 ? p.rdim[0] : 1;
+  const ga_long rml = p.nr > 0 ? p.rmul[0] : 0;
+  const ga_long e0 = (ga_long)lane * RD_VEC;
+  ga_long rstr[RD_NSRC];
+  const char *base[RD_NSRC];
+  RD_SRC_BASES(base);
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) rstr[k] = p.nr > 0 ? p.rsstr[k][0] : 0;
+
+  for (; row < row_end; row += RD_RB) {
+    rd_unit x[RD_RB];
+    ga_long d0o[RD_RB], d1o[RD_RB];
+    const char *srow[RD_RB][RD_NSRC];
+#pragma unroll
+    for (int b = 0; b < RD_RB; b++) {
+      if (row + b < row_end) {
+        ga_long so[RD_NSRC];
+        rd_row_offsets(p, row + b, so, &d0o[b], &d1o[b]);
+#pragma unroll
+        for (int k = 0; k < RD_NSRC; k++) srow[b][k] = base[k] + so[k];
+        rd_unit_load(x[b], srow[b], e0, rin, rstr);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < RD_RB; b++) {
+      if (row + b < row_end) {
+        rd_acc acc = rd_wave_reduce(rd_unit_combine(x[b], e0, rin, 0, rml RD_SCALAR_ARGS));
+        if (lane == 0)
+          rd_store(acc, srow[b], d0 + d0_off, d0o[b], d1 + d1_off, d1o[b], p.rtotal RD_SCALAR_ARGS);
+      }
+    }
+  }
+}
+#endif
 #endif
 
 /* ---- redux_col ------------------------------------------------------------- */
