@@ -11,6 +11,7 @@ from . import _lib
 from ._lib import lib, check, ElemwiseArg
 from . import gpuarray
 from .gpuarray import GpuArray, dtype_to_typecode
+from .dtypes import dtype_to_ctype, get_common_dtype
 
 
 class arg(object):
@@ -95,47 +96,84 @@ class GpuElemwise(object):
         check(lib.GpuElemwise_call(self.ge, ptrs, flags), self.context.ctx)
 
 
-def _broadcast_shape(*shapes):
-    return np.broadcast_shapes(*shapes)
+def _dtype(o):
+    if hasattr(o, "dtype"):
+        return o.dtype
+    return np.asarray(o).dtype
+
+
+def as_argument(o, name, read=False, write=False):
+    """reference pygpu/elemwise.py:17-21"""
+    if (not read) and (not write):
+        raise ValueError("argument is neither read not write")
+    return arg(name, _dtype(o), scalar=not isinstance(o, GpuArray), read=read, write=write)
 
 
 def elemwise1(a, op, oper=None, op_tmpl="res = %(op)sa", out=None, convert_f16=True):
     """Unary op into a new (or given) array (reference pygpu/elemwise.py:24-39)."""
-    args = (arg("res", a.dtype if out is None else out.dtype, write=True),
-            arg("a", a.dtype, read=True))
-    if out is None:
-        out = gpuarray.empty(a.shape, dtype=a.dtype, context=a.context, cls=type(a))
+    args = (as_argument(a, "res", write=True), as_argument(a, "a", read=True))
+    res = a._empty_like_me() if out is None else out
     if oper is None:
         oper = op_tmpl % {"op": op}
     k = GpuElemwise(a.context, oper, args, convert_f16=convert_f16)
-    k(out, a)
-    return out
+    k(res, a)
+    return res
 
 
-def elemwise2(a, op, b, ary, odtype=None, oper=None, op_tmpl="res = (%(out_t)s)a %(op)s (%(out_t)s)b",
-              broadcast=False, convert_f16=True):
-    """Binary op with numpy result-type rules (reference pygpu/elemwise.py:42-88)."""
-    ctx = ary.context
+def elemwise2(a, op, b, ary, odtype=None, oper=None,
+              op_tmpl="res = (%(out_t)s)a %(op)s (%(out_t)s)b", broadcast=False,
+              convert_f16=True):
+    """Binary op with NumPy's result type (reference pygpu/elemwise.py:42-80)."""
+    ndim_extend = True
     if not isinstance(a, GpuArray):
+        a_np, ndim_extend = a, False
         a = np.asarray(a)
+    else:
+        a_np = a
+    if not isinstance(b, GpuArray):
+        b_np, ndim_extend = b, False
+        b = np.asarray(b)
+    else:
+        b_np = b
+    if odtype is None:
+        odtype = get_common_dtype(a_np, b_np, True)
+    odtype = np.dtype(odtype)
+    args = [arg("res", odtype, write=True), as_argument(a, "a", read=True),
+            as_argument(b, "b", read=True)]
+    if ndim_extend:
+        if a.ndim != b.ndim:
+            nd = max(a.ndim, b.ndim)
+            if a.ndim < nd:
+                a = a.reshape(((1,) * (nd - a.ndim)) + a.shape)
+            if b.ndim < nd:
+                b = b.reshape(((1,) * (nd - b.ndim)) + b.shape)
+        out_shape = tuple(max(sa, sb) for sa, sb in zip(a.shape, b.shape))
+        res = gpuarray.empty(out_shape, dtype=odtype, context=ary.context, cls=ary.__class__)
+    else:
+        res = ary._empty_like_me(dtype=odtype)
+    if oper is None:
+        ot = odtype
+        if convert_f16 and ot == np.dtype("float16"):
+            ot = np.dtype("float32")
+        oper = op_tmpl % {"op": op, "out_t": dtype_to_ctype(ot)}
+    k = GpuElemwise(ary.context, oper, args, convert_f16=convert_f16)
+    k(res, a, b, broadcast=broadcast)
+    return res
+
+
+def ielemwise2(a, op, b, oper=None, op_tmpl="a = a %(op)s b", broadcast=False, convert_f16=True):
+    """In-place binary op (reference pygpu/elemwise.py:83-97)."""
     if not isinstance(b, GpuArray):
         b = np.asarray(b)
-    if odtype is None:
-        odtype = np.result_type(a.dtype, b.dtype)
-    a_scalar = not isinstance(a, GpuArray)
-    b_scalar = not isinstance(b, GpuArray)
-    shapes = [x.shape for x in (a, b) if isinstance(x, GpuArray)]
-    oshape = _broadcast_shape(*shapes) if broadcast else shapes[0]
-    out = gpuarray.empty(oshape, dtype=odtype, context=ctx, cls=type(ary))
-    ctypes_names = {"float16": "ga_float", "float32": "ga_float", "float64": "ga_double",
-                    "bool": "ga_bool", "int8": "ga_byte", "uint8": "ga_ubyte",
-                    "int16": "ga_short", "uint16": "ga_ushort", "int32": "ga_int",
-                    "uint32": "ga_uint", "int64": "ga_long", "uint64": "ga_ulong"}
+    args = [as_argument(a, "a", read=True, write=True), as_argument(b, "b", read=True)]
     if oper is None:
-        oper = op_tmpl % {"op": op, "out_t": ctypes_names[np.dtype(odtype).name]}
-    args = (arg("res", out.dtype, write=True),
-            arg("a", a.dtype, read=True, scalar=a_scalar),
-            arg("b", b.dtype, read=True, scalar=b_scalar))
-    k = GpuElemwise(ctx, oper, args, convert_f16=convert_f16)
-    k(out, a, b, broadcast=broadcast)
-    return out
+        oper = op_tmpl % {"op": op}
+    k = GpuElemwise(a.context, oper, args, convert_f16=convert_f16)
+    k(a, b, broadcast=broadcast)
+    return a
+
+
+def compare(a, op, b, broadcast=False, convert_f16=True):
+    """reference pygpu/elemwise.py:99-102"""
+    return elemwise2(a, op, b, a, odtype=np.dtype("bool"), op_tmpl="res = (a %(op)s b)",
+                     broadcast=broadcast, convert_f16=convert_f16)

@@ -223,6 +223,24 @@ class GpuArray(object):
             raise TypeError("len() of unsized object")
         return self.ga.dimensions[0]
 
+    def __bool__(self):
+        """reference pygpu/gpuarray.pyx:2118-2125"""
+        if self.size == 0:
+            return False
+        if self.size == 1:
+            return bool(np.asarray(self))
+        raise ValueError("Truth value of array with more than one element is ambiguous")
+
+    __hash__ = None
+
+    def _empty_like_me(self, dtype=None, order="C"):
+        """A new array of this one's shape, class and context
+        (reference pygpu/gpuarray.pyx:1714-1735)."""
+        if order.upper() == "A":
+            order = "F" if (self.flags.f_contiguous and not self.flags.c_contiguous) else "C"
+        return empty(self.shape, self.dtype if dtype is None else dtype, order, self.context,
+                     cls=type(self))
+
     def _ptr(self):
         return C.byref(self.ga)
 
@@ -434,10 +452,10 @@ def asarray(obj, dtype=None, order="A", context=None, cls=None):
     return array(obj, dtype, order, context, cls)
 
 
-def from_strided(base, offset, shape, strides, dtype=None, writeable=True):
+def from_strided(base, offset, shape, strides, dtype=None, writeable=True, cls=None):
     """View `base`'s buffer with explicit byte offset and strides
     (GpuArray_fromdata; reference gpuarray.pyx `from_gpudata` :760-815)."""
-    res = type(base)(base.context)
+    res = (cls or type(base))(base.context)
     nd = len(shape)
     dims = (C.c_size_t * max(nd, 1))(*shape)
     strs = (c_ssize_t * max(nd, 1))(*strides)

@@ -16,7 +16,7 @@ def root_of(view):
     return r
 
 
-def to_gpu_view(view, ctx, base_gpu=None):
+def to_gpu_view(view, ctx, base_gpu=None, cls=None):
     """Device array aliasing a device copy of `view`'s whole root buffer, with
     `view`'s exact byte strides and offset (negative and zero strides included).
     Returns (device_view, device_root)."""
@@ -29,7 +29,8 @@ def to_gpu_view(view, ctx, base_gpu=None):
                                   context=ctx)
     offset = view.__array_interface__["data"][0] - root.__array_interface__["data"][0] \
         if view.size or view.ndim else 0
-    dv = gpuarray.from_strided(base_gpu, max(offset, 0), view.shape, view.strides, dtype=view.dtype)
+    dv = gpuarray.from_strided(base_gpu, max(offset, 0), view.shape, view.strides, dtype=view.dtype,
+                               cls=cls)
     return dv, base_gpu
 
 
@@ -42,9 +43,12 @@ def read_root(base_gpu, root):
 
 
 def gen_gpuarray(shape_orig, dtype="float32", offseted_outer=False, offseted_inner=False,
-                 sliced=1, order="c", ctx=None, rng=None, low=0.0, high=10.0):
+                 sliced=1, order="c", ctx=None, rng=None, low=0.0, high=10.0, nozeros=False,
+                 incr=0, cls=None):
     """Same knobs as the reference helper: returns (numpy view, device view)."""
     rng = rng or np.random.default_rng(0)
+    if nozeros:
+        low = 1.0
     shape = np.asarray(shape_orig).copy()
     if sliced != 1 and len(shape) > 0:
         shape[0] *= abs(sliced)
@@ -55,7 +59,7 @@ def gen_gpuarray(shape_orig, dtype="float32", offseted_outer=False, offseted_inn
     if np.dtype(dtype) == np.dtype("bool"):
         a = rng.random(tuple(shape)) < 0.5
     else:
-        a = np.asarray(rng.uniform(low, high, shape), dtype=dtype)
+        a = np.asarray(rng.uniform(low, high, shape) + incr, dtype=dtype)
     if order == "f":
         a = np.asfortranarray(a)
     v = a
@@ -66,7 +70,7 @@ def gen_gpuarray(shape_orig, dtype="float32", offseted_outer=False, offseted_inn
     if sliced != 1 and len(shape) > 0:
         v = v[::sliced]
     assert v.shape == tuple(shape_orig)
-    dv, _ = to_gpu_view(v, ctx)
+    dv, _ = to_gpu_view(v, ctx, cls=cls)
     return v, dv
 
 
