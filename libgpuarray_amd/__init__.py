@@ -12,7 +12,8 @@ the part of the reference's Python layer that drives this path:
 from . import _lib
 from ._lib import GpuArrayException, UnsupportedException, LIB_PATH
 from . import gpuarray, elemwise, reduction
-from .gpuarray import (GpuContext, GpuArray, init, array, asarray, empty, zeros,
+from .gpuarray import (GpuContext, GpuArray, init, array, asarray, empty, zeros, zeros_like,
+                       empty_like, ascontiguousarray, asfortranarray, may_share_memory,
                        set_default_context, get_default_context, count_devices)
 from .elemwise import GpuElemwise, arg, as_argument, elemwise1, elemwise2, ielemwise2, compare
 from .reduction import GpuReduction, ReductionKernel

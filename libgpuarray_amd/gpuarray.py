@@ -202,8 +202,75 @@ class GpuArray(object):
             lib.GpuArray_clear(C.byref(ga))
 
     # -- metadata ---------------------------------------------------------------
-    shape = property(lambda s: tuple(s.ga.dimensions[i] for i in range(s.ga.nd)))
-    strides = property(lambda s: tuple(s.ga.strides[i] for i in range(s.ga.nd)))
+    def _get_shape(self):
+        return tuple(self.ga.dimensions[i] for i in range(self.ga.nd))
+
+    def _set_shape(self, newshape):
+        """In-place reshape; refuses what would need a copy
+        (reference pygpu/gpuarray.pyx:2136-2166)."""
+        if isinstance(newshape, (int, np.integer)):
+            newshape = (newshape,)
+        newshape = self._fill_unknown(list(newshape))
+        dims = (C.c_size_t * max(len(newshape), 1))(*newshape)
+        err = lib.GpuArray_reshape_inplace(self._ptr(), len(newshape), dims, _lib.GA_C_ORDER)
+        if err == _lib.GA_COPY_ERROR:
+            raise AttributeError("Incompatible shape for in-place modification")
+        self._check(err)
+
+    shape = property(_get_shape, _set_shape)
+
+    def _get_strides(self):
+        return tuple(self.ga.strides[i] for i in range(self.ga.nd))
+
+    def _set_strides(self, newstrides):
+        """reference pygpu/gpuarray.pyx:241-267,2177-2185: the new strides must
+        keep every element inside the buffer."""
+        newstrides = tuple(int(v) for v in newstrides)
+        if len(newstrides) != self.ga.nd:
+            raise ValueError("new strides are the wrong length")
+        size = C.c_size_t()
+        self._check(lib.gpudata_property(self.ga.data, _lib.GA_BUFFER_PROP_SIZE, C.byref(size)))
+        lower = upper = self.ga.offset
+        ok = True
+        for i in range(self.ga.nd):
+            if self.ga.dimensions[i] == 0:
+                break
+            off = newstrides[i] * (self.ga.dimensions[i] - 1)
+            if off > 0:
+                if upper + off > size.value:
+                    ok = False
+                    break
+                upper += off
+            else:
+                if lower < -off:
+                    ok = False
+                    break
+                lower += off
+        else:
+            ok = upper + self.itemsize <= size.value
+        if not ok:
+            raise ValueError("new strides go outside of allocated memory")
+        for i in range(self.ga.nd):
+            self.ga.strides[i] = newstrides[i]
+        lib.GpuArray_fix_flags(self._ptr())
+
+    strides = property(_get_strides, _set_strides)
+
+    def _fill_unknown(self, shape):
+        shape = [int(d) for d in shape]
+        if shape.count(-1) > 1:
+            raise ValueError("can only specify one unknown dimension")
+        if shape.count(-1) == 1:
+            known = 1
+            for d in shape:
+                if d != -1:
+                    known *= d
+            if known == 0 or self.size % known:
+                raise ValueError("total size of new array must be unchanged")
+            shape[shape.index(-1)] = self.size // known
+        return shape
+
+    gpudata = property(lambda s: s.ga.data)
     ndim = property(lambda s: s.ga.nd)
     offset = property(lambda s: s.ga.offset)
     typecode = property(lambda s: s.ga.typecode)
@@ -264,6 +331,29 @@ class GpuArray(object):
         elif self.flags.f_contiguous:
             src = np.asfortranarray(src)
         self._check(lib.GpuArray_write(self._ptr(), src.ctypes.data_as(C.c_void_p), src.nbytes))
+
+    def read(self, dst):
+        """Copy into a writeable NumPy array of the same shape, dtype and
+        contiguity (reference pygpu/gpuarray.pyx:1756-1786)."""
+        if not isinstance(dst, np.ndarray) or not dst.flags.writeable:
+            raise ValueError("Destination is not a writeable ndarray")
+        if dst.dtype != self.dtype or dst.shape != self.shape:
+            raise ValueError("shape or dtype mismatch")
+        if self.flags.c_contiguous and dst.flags.c_contiguous:
+            pass
+        elif self.flags.f_contiguous and dst.flags.f_contiguous:
+            pass
+        else:
+            raise ValueError("source and destination must be contiguous in the same order")
+        self._check(lib.GpuArray_read(dst.ctypes.data_as(C.c_void_p), dst.nbytes, self._ptr()))
+
+    def __copy__(self):
+        return self.copy("C")          # reference pygpu/gpuarray.pyx:1793-1800
+
+    def __deepcopy__(self, memo):
+        if id(self) in memo:
+            return memo[id(self)]
+        return self.copy("C")
 
     def __array__(self, dtype=None, copy=None):
         a = self
@@ -337,13 +427,7 @@ class GpuArray(object):
     def reshape(self, shape, order="C"):
         if isinstance(shape, int):
             shape = (shape,)
-        shape = list(shape)
-        if shape.count(-1) == 1:
-            known = 1
-            for d in shape:
-                if d != -1:
-                    known *= d
-            shape[shape.index(-1)] = self.size // known if known else 0
+        shape = self._fill_unknown(list(shape))
         dims = (C.c_size_t * max(len(shape), 1))(*shape)
         o = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER}[order.upper()]
         res = self._new()
@@ -353,10 +437,43 @@ class GpuArray(object):
     def __getitem__(self, key):
         """Basic indexing only: ints, slices, Ellipsis (reference
         pygpu/gpuarray.pyx:1928-2069 lowers these to start/stop/step triples)."""
+        if isinstance(key, list):
+            if any(isinstance(k, slice) or k is Ellipsis for k in key):
+                key = tuple(key)
+            else:
+                raise NotImplementedError("fancy indexing not supported")
         if not isinstance(key, tuple):
             key = (key,)
+        if any(isinstance(k, (list, np.ndarray, GpuArray)) and getattr(k, "ndim", 1) > 0 for k in key):
+            raise NotImplementedError("fancy indexing not supported")
+        if any(k is None for k in key):
+            # index without the None entries, then put the unit dims back
+            # (reference pygpu/gpuarray.pyx:1974-2008)
+            sliced = self.__getitem__(tuple(k for k in key if k is not None))
+            n_real = len([k for k in key if k is not None and k is not Ellipsis])
+            expanded = []
+            for k in key:
+                if k is Ellipsis:
+                    expanded.extend([slice(None)] * (self.ndim - n_real))
+                else:
+                    expanded.append(k)
+            if Ellipsis not in key:
+                expanded.extend([slice(None)] * (self.ndim - n_real))
+            new_shape, new_strides, i = [], [], 0
+            for k in expanded:
+                if k is None:
+                    new_shape.append(1)
+                    new_strides.append(0)
+                elif isinstance(k, slice):
+                    new_shape.append(sliced.shape[i])
+                    new_strides.append(sliced.strides[i])
+                    i += 1
+            res = from_strided(sliced, sliced.offset, new_shape, new_strides,
+                               writeable=sliced.flags.writeable)
+            res.base = self
+            return res
         nd = self.ndim
-        if key.count(Ellipsis) > 1:
+        if len([k for k in key if k is Ellipsis]) > 1:
             raise IndexError("an index can only have a single ellipsis")
         n_explicit = len([k for k in key if k is not Ellipsis])
         if n_explicit > nd:
@@ -381,6 +498,9 @@ class GpuArray(object):
                     sp = st
                 starts[i], stops[i], steps[i] = st, sp, stp
             else:
+                if not isinstance(k, (int, np.integer)) and not (
+                        isinstance(k, np.ndarray) and k.ndim == 0 and k.dtype.kind in "iu"):
+                    raise IndexError("only integers, slices, None and Ellipsis are valid indices")
                 k = int(k)
                 if k < 0:
                     k += dim
@@ -464,3 +584,43 @@ def from_strided(base, offset, shape, strides, dtype=None, writeable=True, cls=N
                                 1 if writeable else 0), base.context.ctx)
     res.base = base
     return res
+
+
+def zeros_like(a, dtype=None, order="C"):
+    return zeros(a.shape, a.dtype if dtype is None else dtype, order, a.context, cls=type(a))
+
+
+def empty_like(a, dtype=None, order="C"):
+    return a._empty_like_me(dtype=dtype, order=order)
+
+
+def ascontiguousarray(a, dtype=None, context=None):
+    """C-ordered device array; `a` itself when it already is one of the right
+    type (reference pygpu/gpuarray.pyx:797-817; 0-d input gives a 1-d result,
+    as NumPy's function does)."""
+    if isinstance(a, GpuArray):
+        if (dtype is None or np.dtype(dtype) == a.dtype) and a.flags.c_contiguous and a.ndim >= 1:
+            return a
+        res = a.astype(a.dtype if dtype is None else dtype, order="C") \
+            if (dtype is not None and np.dtype(dtype) != a.dtype) else a.copy("C")
+        return res.reshape((1,)) if res.ndim == 0 else res
+    res = array(a, dtype=dtype, order="C", context=context)
+    return res.reshape((1,)) if res.ndim == 0 else res
+
+
+def asfortranarray(a, dtype=None, context=None):
+    """Fortran-ordered device array (reference pygpu/gpuarray.pyx:819-839)."""
+    if isinstance(a, GpuArray):
+        if (dtype is None or np.dtype(dtype) == a.dtype) and a.flags.f_contiguous and a.ndim >= 1:
+            return a
+        if dtype is not None and np.dtype(dtype) != a.dtype:
+            a = a.astype(dtype)
+        res = a.copy("F")
+        return res.reshape((1,)) if res.ndim == 0 else res
+    res = array(a, dtype=dtype, order="F", context=context)
+    return res.reshape((1,)) if res.ndim == 0 else res
+
+
+def may_share_memory(a, b):
+    """reference pygpu/gpuarray.pyx:841-847 (GpuArray_share)"""
+    return bool(lib.GpuArray_share(a._ptr(), b._ptr()))

@@ -60,7 +60,7 @@ def gen_gpuarray(shape_orig, dtype="float32", offseted_outer=False, offseted_inn
         a = rng.random(tuple(shape)) < 0.5
     else:
         a = np.asarray(rng.uniform(low, high, shape) + incr, dtype=dtype)
-    if order == "f":
+    if order == "f" and len(shape) > 0:
         a = np.asfortranarray(a)
     v = a
     if offseted_outer and len(shape) > 0:
