@@ -624,3 +624,146 @@ def asfortranarray(a, dtype=None, context=None):
 def may_share_memory(a, b):
     """reference pygpu/gpuarray.pyx:841-847 (GpuArray_share)"""
     return bool(lib.GpuArray_share(a._ptr(), b._ptr()))
+
+
+class GpuKernel(object):
+    """A kernel from source text (reference pygpu/gpuarray.pyx:2269-2500):
+    `types` lists the argument types, GpuArray for buffers and dtypes for
+    by-value arguments; the call takes `n` (a problem size the library turns
+    into a launch shape) or explicit `gs`/`ls` of up to three dims."""
+
+    def __init__(self, source, name, types, context=None, have_double=False, have_small=False,
+                 have_complex=False, have_half=False, cuda=False, opencl=False):
+        self.context = _ensure_context(context)
+        flags = 0
+        if have_double:
+            flags |= _lib.GA_USE_DOUBLE
+        if have_small:
+            flags |= _lib.GA_USE_SMALL
+        if have_complex:
+            flags |= _lib.GA_USE_COMPLEX
+        if have_half:
+            flags |= _lib.GA_USE_HALF
+        if cuda:
+            flags |= _lib.GA_USE_CUDA
+        if opencl:
+            flags |= _lib.GA_USE_OPENCL
+        self._types = [_lib.GA_BUFFER if t is GpuArray else dtype_to_typecode(t) for t in types]
+        self._dtypes = [None if t is GpuArray else np.dtype(t) for t in types]
+        src = source.encode() if isinstance(source, str) else source
+        srcs = (C.c_char_p * 1)(src)
+        lens = (C.c_size_t * 1)(len(src))
+        tarr = (C.c_int * max(len(self._types), 1))(*self._types)
+        self.k = _lib.GpuKernelStruct()
+        err_str = C.c_char_p()
+        err = lib.GpuKernel_init(C.byref(self.k), self.context.ctx, 1, srcs, lens,
+                                 name.encode() if isinstance(name, str) else name,
+                                 len(self._types), tarr, flags, C.byref(err_str))
+        if err != _lib.GA_NO_ERROR:
+            self.k = None
+            log = err_str.value.decode(errors="replace") if err_str.value else ""
+            try:
+                check(err, self.context.ctx)
+            except GpuArrayException as e:
+                raise type(e)("%s\n%s" % (e.args[0], log), err)
+
+    def __del__(self):
+        k = getattr(self, "k", None)
+        if k is not None:
+            lib.GpuKernel_clear(C.byref(k))
+            self.k = None
+
+    def __reduce__(self):
+        raise RuntimeError("Cannot pickle GpuKernel object")
+
+    def _prop(self, prop_id, ctype):
+        v = ctype()
+        check(lib.gpukernel_property(self.k.k, prop_id, C.byref(v)), self.context.ctx)
+        return v.value
+
+    maxlsize = property(lambda s: s._prop(_lib.GA_KERNEL_PROP_MAXLSIZE, C.c_size_t))
+    preflsize = property(lambda s: s._prop(_lib.GA_KERNEL_PROP_PREFLSIZE, C.c_size_t))
+    numargs = property(lambda s: s._prop(_lib.GA_KERNEL_PROP_NUMARGS, C.c_uint))
+
+    def __call__(self, *args, **kwargs):
+        n, gs, ls = kwargs.pop("n", None), kwargs.pop("gs", None), kwargs.pop("ls", None)
+        shared = kwargs.pop("shared", 0)
+        if kwargs:
+            raise TypeError("unexpected keyword arguments: %s" % (sorted(kwargs),))
+        if n is None and (ls is None or gs is None):
+            raise ValueError("Must specify size (n) or both gs and ls")
+        lsz, gsz = (C.c_size_t * 3)(0, 1, 1), (C.c_size_t * 3)(0, 1, 1)
+        if ls is None:
+            nd = 1
+        elif isinstance(ls, (int, np.integer)):
+            lsz[0], nd = int(ls), 1
+        elif isinstance(ls, (list, tuple)):
+            if len(ls) > 3:
+                raise ValueError("ls is not of length 3 or less")
+            nd = len(ls)
+            for i in range(nd):
+                lsz[i] = int(ls[i])
+        else:
+            raise TypeError("ls is not int or list")
+        if gs is None:
+            if nd != 1:
+                raise ValueError("nd mismatch for gs (None)")
+        elif isinstance(gs, (int, np.integer)):
+            if nd != 1:
+                raise ValueError("nd mismatch for gs (int)")
+            gsz[0] = int(gs)
+        elif isinstance(gs, (list, tuple)):
+            if len(gs) > 3:
+                raise ValueError("gs is not of length 3 or less")
+            if len(gs) != nd:
+                raise ValueError("nd mismatch for gs (tuple)")
+            for i in range(nd):
+                gsz[i] = int(gs[i])
+        else:
+            raise TypeError("gs is not int or list")
+        if len(args) != len(self._types):
+            raise TypeError("Expected %d arguments, got %d," % (len(self._types), len(args)))
+        keep = []
+        ptrs = (C.c_void_p * max(len(args), 1))()
+        for i, (t, dt, a) in enumerate(zip(self._types, self._dtypes, args)):
+            if t == _lib.GA_BUFFER:
+                if not isinstance(a, GpuArray):
+                    raise TypeError("expected a GpuArray")
+                ptrs[i] = a.ga.data
+            else:
+                v = np.asarray(a, dtype=dt).reshape(1).copy()
+                keep.append(v)
+                ptrs[i] = v.ctypes.data
+        if n is not None:
+            if nd != 1:
+                raise ValueError("n is specified and nd != 1")
+            check(lib.GpuKernel_sched(C.byref(self.k), int(n), gsz, lsz), self.context.ctx)
+        check(lib.GpuKernel_call(C.byref(self.k), nd, gsz, lsz, int(shared), ptrs), self.context.ctx)
+
+
+def _split(a, ind, axis):
+    """reference pygpu/gpuarray.pyx:1467-1496: views of `a` cut along `axis`
+    at the positions `ind` (capped at the extent)."""
+    if not 0 <= axis < a.ndim:
+        raise ValueError("split on non-existant axis")
+    m = a.shape[axis]
+    cuts = [min(int(v), m) for v in ind]
+    res = [type(a)(a.context) for _ in range(len(cuts) + 1)]
+    ptrs = (_lib.PA * len(res))(*[C.pointer(r.ga) for r in res])
+    p = (C.c_size_t * max(len(cuts), 1))(*cuts)
+    check(lib.GpuArray_split(ptrs, a._ptr(), len(cuts), p, axis), a.context.ctx)
+    for r in res:
+        r.base = a
+    return res
+
+
+def _concatenate(al, axis, restype, cls, context):
+    """reference pygpu/gpuarray.pyx:1505-1522"""
+    context = _ensure_context(context)
+    for a in al:
+        if not isinstance(a, GpuArray):
+            raise TypeError("expected GpuArrays to concatenate")
+    res = _make(cls, context)
+    ptrs = (_lib.PA * len(al))(*[C.pointer(a.ga) for a in al])
+    check(lib.GpuArray_concatenate(res._ptr(), ptrs, len(al), axis, restype), context.ctx)
+    return res
