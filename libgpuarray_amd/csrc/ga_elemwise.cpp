@@ -389,27 +389,56 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
     if (ge->args[j].reads()) any_tr = true;
     if (ge->args[j].writes()) any_tw = true;
   }
+  // Every global load of a phase is issued into registers before its first
+  // use, so a lane has 16 loads in flight instead of one.
   if (any_tr) {
-    s += "#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (is_t(j) && ge->args[j].reads())
+        appendf(s, "%s %s_r[16];\n", ctype(ge->args[j].typecode), ge->args[j].name.c_str());
+    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
     appendf(s, "const %s ga_ly = ga_tx, ga_lx = ga_ty + 4u * (%s)ga_k;\n", N, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
-      appendf(s, "%s_t[ga_lx * 65u + ga_ly] = %s;\n", a.name.c_str(),
+      appendf(s, "%s_r[ga_k] = %s;\n", a.name.c_str(),
               gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+    }
+    s += "}\n}\n";
+    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+    appendf(s, "const %s ga_ly = ga_tx, ga_lx = ga_ty + 4u * (%s)ga_k;\n", N, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!is_t(j) || !a.reads()) continue;
+      appendf(s, "%s_t[ga_lx * 65u + ga_ly] = %s_r[ga_k];\n", a.name.c_str(), a.name.c_str());
     }
     s += "}\n}\nlocal_barrier();\n";
   }
   // phase 2: expression, lanes along x
-  s += "#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (a.is_array() && !is_t(j) && a.reads())
+      appendf(s, "%s %s_g[16];\n", ctype(a.typecode), a.name.c_str());
+  }
+  s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+  appendf(s, "const %s ga_lx = ga_tx, ga_ly = ga_ty + 4u * (%s)ga_k;\n", N, N);
+  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (a.is_array() && !is_t(j) && a.reads())
+      appendf(s, "%s_g[ga_k] = %s;\n", a.name.c_str(),
+              gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+  }
+  s += "}\n}\n";
+  s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
   appendf(s, "const %s ga_lx = ga_tx, ga_ly = ga_ty + 4u * (%s)ga_k;\n", N, N);
   appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
     if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_lx * 65u + ga_ly]");
-    else emit_load(ge, s, a, gaddr(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx"));
+    else emit_load(ge, s, a, a.name + "_g[ga_k]");
   }
   s += ge->expr;
   s += ";\n";
@@ -422,7 +451,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
   s += "}\n}\n";
   // phase 3: transposed writes, lanes along y
   if (any_tw) {
-    s += "local_barrier();\n#pragma unroll 4\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
+    s += "local_barrier();\n#pragma unroll\nfor (int ga_k = 0; ga_k < 16; ga_k++) {\n";
     appendf(s, "const %s ga_ly = ga_tx, ga_lx = ga_ty + 4u * (%s)ga_k;\n", N, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
@@ -1020,7 +1049,7 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
 
   // Four elements per lane when the layout allows it (see gen_strided_vec).
   bool vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % 4 == 0 &&
-              dims[nd - 1] >= 16 && strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
+              strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
   unsigned umask = 0;
   if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
   for (unsigned k = 0; k < na && vec4; k++) {
@@ -1060,7 +1089,10 @@ int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
   unsigned ltx = 0, tile = 64;
   if (tmask == 0) {
     size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
-    ltx = vec4 ? 0 : 4;
+    // as many lanes along x as the inner extent needs (a power of two), the
+    // rest of the 256 along the rows: 2^24 floats in rows of 3 took 191 us
+    // with a floor of 16 lanes along x, 61 us without
+    ltx = 0;
     while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
     size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
     size_t rows = n / dims[nd - 1];
