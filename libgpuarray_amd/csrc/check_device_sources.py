@@ -76,6 +76,9 @@ def main():
     check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1))
     check("reduction stepped halves", gen_r(0, GA_HALF, GA_FLOAT, GA_LONG, 256, 4 | (2 << 8), 1))
     check("reduction short rows in batches of 4", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1 | (4 << 8)))
+    for lanes in (1, 2, 8, 16, 32):
+        check("reduction %d lanes per row" % lanes,
+              gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64 | (lanes << 16), 4, 2 | (2 << 8)))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),
@@ -98,7 +101,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "12 elementwise)" % (n + 6, m, t))
+          "12 elementwise)" % (n + 11, m, t))
 
 
 if __name__ == "__main__":

@@ -180,6 +180,7 @@ struct variant_spec {
   unsigned G, V, U, opts, ES;
   unsigned vecmask;   // bit k: array source k is fetched with vector loads
   unsigned RB;        // redux_wrows: rows per batch of loads
+  unsigned L;         // redux_wrows: lanes per row
 };
 
 const char *load_type_name(int tc) {
@@ -237,6 +238,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", vs.G, vs.V, vs.U);
   DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n#define RD_RB %u\n",
       vs.opts & 1u, (vs.opts >> 1) & 1u, vs.ES, vs.RB ? vs.RB : 1u);
+  DEF("#define RD_L %u\n", vs.L ? vs.L : 64u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -286,11 +288,11 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   }
   gen += " RD_SCALAR_FPARAMS) { return (" + gr->map_expr + "); }\n";
   // loads
-  gen += "static __device__ inline void rd_unit_load(rd_unit &u, const char *const *base, "
+  gen += "template <int LN>\nstatic __device__ inline void rd_unit_load(rd_unit &u, const char *const *base, "
          "ga_long e0, ga_long rin, const ga_long *rstr) {\n"
          "_Pragma(\"unroll\")\n"
          "  for (int j = 0; j < RD_U; j++) {\n"
-         "    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;\n"
+         "    const ga_long e = e0 + (ga_long)j * LN * RD_VEC;\n"
          "    if (e < rin) {\n";
   for (unsigned k = 0; k < K; k++) {
     const char *lt = load_type_name(gr->args[gr->arrays[k]].tc);
@@ -337,8 +339,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
-           vs.opts, vs.ES, vs.vecmask, vs.RB);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
+           vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -653,7 +655,10 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
 
   // Lanes along the reduced run unless the free run is the one that is
   // contiguous in memory (or the reduced run is too short to feed a wavefront).
-  bool use_row = p.nf == 0 || (rstr <= fstr && rin >= 32) || (rin >= 4096 && rstr <= 4 * elsz_max);
+  // Short reduced runs are fine when they are the only reduced dim: several
+  // rows then share a wavefront (redux_wrows).
+  bool use_row = p.nf == 0 || (rstr <= fstr && (rin >= 32 || p.nr <= 1)) ||
+                 (rin >= 4096 && rstr <= 4 * elsz_max);
   if (rtotal == 0) use_row = true;
   {
     const char *force = getenv("GPUARRAY_REDUX_FAMILY");
@@ -661,7 +666,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64;
   bool wrows = false;
   size_t groups;
   if (use_row) {
@@ -774,9 +779,26 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
       // one row at a time, 24.8 us with batches of 4 and 8 rows per wavefront;
       // rows of 1000 floats (four loads per lane already) 45 us one at a time,
       // 66 / 92 us in batches of 2 / 4.
-      RB = (unsigned)env_ul("GPUARRAY_REDUX_RB", U == 1 ? 4 : 1);
+      // A row much shorter than a wavefront's reach gets L < 64 lanes and
+      // 64 / L rows share the wavefront: L is the smallest power of two that
+      // covers the row with four loads per lane.
+      {
+        const int64_t need = (rin + (int64_t)V * 4 - 1) / ((int64_t)V * 4);
+        L = 1;
+        while (L < 64 && (int64_t)L < need) L *= 2;
+        const unsigned long force = env_ul("GPUARRAY_REDUX_L", 0);
+        if (force >= 1 && force <= 64 && (force & (force - 1)) == 0 &&
+            (int64_t)force * V * 8 >= rin)
+          L = (unsigned)force;
+        if (L < 64) {
+          U = 1;
+          while (U < 8 && (int64_t)L * V * U < rin) U *= 2;
+        }
+      }
+      RB = (unsigned)env_ul("GPUARRAY_REDUX_RB", L < 64 ? (U >= 4 ? 1 : 4 / U) : (U == 1 ? 4 : 1));
       if (RB != 1 && RB != 2 && RB != 4 && RB != 8) RB = 1;
-      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", RB == 1 ? 1 : 2 * RB);
+      const int64_t per_batch = (int64_t)(64 / L) * RB;
+      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", (RB == 1 && L == 64) ? 1 : 2 * per_batch);
       if (rpw < 1) rpw = 1;
       p.upb = rpw;
       const int64_t waves = (nrows + rpw - 1) / rpw;
@@ -808,7 +830,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
   if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
-                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1};
+                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64};
   variant *var = nullptr;
   int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
@@ -871,11 +893,13 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   if (make_plain_operator(&gr, nullptr, ga_global_err, (ga_reduce_op)op, src_tc) != GA_NO_ERROR)
     return nullptr;
   // bits 8.. of V carry the element step of strided loads (0 means 1), bits
-  // 8.. of U the rows per batch of redux_wrows (0 means 1)
+  // 8.. of U the rows per batch of redux_wrows (0 means 1), bits 16.. of G its
+  // lanes per row (0 means 64)
   const unsigned ES = (V >> 8) ? (V >> 8) : 1;
   V &= 0xffu;
   std::string s;
-  variant_spec vs = {d0_tc, d1_tc, G, V, U & 0xffu, 3, ES, 1, (U >> 8) ? (U >> 8) : 1};
+  variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu, 3, ES, 1, (U >> 8) ? (U >> 8) : 1,
+                     (G >> 16) ? (G >> 16) : 64};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
@@ -892,7 +916,7 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1};
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

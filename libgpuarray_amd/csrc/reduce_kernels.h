@@ -22,7 +22,9 @@
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
  *   RD_U        loads in flight per lane
- *   RD_RB       redux_wrows: rows whose loads a wavefront issues together
+ *   RD_L        redux_wrows: lanes that share a row (power of two, <= 64);
+ *               64 / RD_L rows sit side by side in a wavefront
+ *   RD_RB       redux_wrows: sets of rows whose loads a wavefront issues together
  *   RD_NT       streaming (non-temporal) loads in redux_row
  *   RD_INTERLEAVE  redux_row with one reduced dim: splits take every
  *               nsplit-th unit instead of a contiguous range
@@ -216,6 +218,25 @@ static __device__ inline rd_acc rd_wave_reduce(rd_acc a) {
   return rd_readlane63(a);
 }
 
+/* The same over aligned segments of L lanes (a power of two): the first
+ * log2(L) steps of the network.  Up to 16 lanes every lane of a segment ends
+ * with the result; for 32 the upper 16 lanes do; for 64 all do.  Lane L-1 of
+ * a segment holds it in every case. */
+template <int L>
+static __device__ inline rd_acc rd_seg_reduce(rd_acc a) {
+  const rd_acc nt = rd_neutral();
+  if (L >= 2) a = rd_combine(a, rd_dpp<RD_DPP_XOR1, 0xf>(a, nt));
+  if (L >= 4) a = rd_combine(a, rd_dpp<RD_DPP_XOR2, 0xf>(a, nt));
+  if (L >= 8) a = rd_combine(a, rd_dpp<RD_DPP_HALF_MIRROR, 0xf>(a, nt));
+  if (L >= 16) a = rd_combine(a, rd_dpp<RD_DPP_MIRROR, 0xf>(a, nt));
+  if (L >= 32) a = rd_combine(a, rd_dpp<RD_DPP_BCAST15, 0xa>(a, nt));
+  if (L >= 64) {
+    a = rd_combine(a, rd_dpp<RD_DPP_BCAST31, 0xc>(a, nt));
+    a = rd_readlane63(a);
+  }
+  return a;
+}
+
 /* Combination over the 4 wavefronts of a 256-lane group, through LDS. */
 static __device__ inline rd_acc rd_block_reduce(rd_acc a, rd_acc *lds) {
   a = rd_wave_reduce(a);
@@ -340,12 +361,14 @@ static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *
 
 /* ---- redux_row ------------------------------------------------------------- */
 
-/* One "unit" = RD_U loads per lane over RD_G lanes: elements
- * e0 + j*RD_G*RD_VEC + v of the inner reduced dim, j < RD_U, v < RD_VEC, where
+/* One "unit" = RD_U loads per lane over LN lanes (RD_G in redux_row, RD_L
+ * in redux_wrows): elements
+ * e0 + j*LN*RD_VEC + v of the inner reduced dim, j < RD_U, v < RD_VEC, where
  * e0 = (first element of the unit) + lane*RD_VEC.
  *
  * Combination of the lane's elements of one unit.  ib, rml: index of element
  * 0 of the inner dim and index step per element. */
+template <int LN>
 static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga_long rin,
                                                 ga_long ib, ga_long rml RD_SCALAR_FPARAMS) {
 #if RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN
@@ -358,7 +381,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
     ga_int bp = 0;
 #pragma unroll
     for (int j = 0; j < RD_U; j++) {
-      if (e0 + (ga_long)j * RD_G * RD_VEC < rin) {
+      if (e0 + (ga_long)j * LN * RD_VEC < rin) {
 #pragma unroll
         for (int v = 0; v < RD_VEC; v++) {
           if (j == 0 && v == 0) continue;
@@ -369,7 +392,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
           const bool better = val < bv;
 #endif
           bv = better ? val : bv;
-          bp = better ? (j * RD_G * RD_VEC + v) : bp;
+          bp = better ? (j * LN * RD_VEC + v) : bp;
         }
       }
     }
@@ -385,7 +408,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
   rd_acc t[RD_U];
 #pragma unroll
   for (int j = 0; j < RD_U; j++) {
-    const ga_long e = e0 + (ga_long)j * RD_G * RD_VEC;
+    const ga_long e = e0 + (ga_long)j * LN * RD_VEC;
     t[j] = rd_neutral();
     if (e < rin) {
 #pragma unroll
@@ -456,8 +479,8 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
     const char *ub[RD_NSRC];
 #pragma unroll
     for (int s = 0; s < RD_NSRC; s++) ub[s] = srow[s] + rb[s];
-    rd_unit_load(x, ub, e0, rin, rstr);
-    acc = rd_combine(acc, rd_unit_combine(x, e0, rin, ib, rml RD_SCALAR_ARGS));
+    rd_unit_load<RD_G>(x, ub, e0, rin, rstr);
+    acc = rd_combine(acc, rd_unit_combine<RD_G>(x, e0, rin, ib, rml RD_SCALAR_ARGS));
 #if RD_INTERLEAVE
     k += ustep;   /* single reduced dim: the unit is the segment */
 #else
@@ -489,7 +512,7 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
  * first row is combined, so a wavefront whose row is a single load per lane
  * still has RD_RB loads in flight.  Only built for RD_G == 64. */
 #if RD_G == 64
-#if RD_RB == 1
+#if RD_RB == 1 && RD_L == 64
 /* one row at a time; with upb > 1 the next row's loads are issued before the
  * current row is combined */
 KERNEL void __launch_bounds__(256)
@@ -519,7 +542,7 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 #pragma unroll
   for (int k = 0; k < RD_NSRC; k++) srow[k] = base[k] + so[k];
   rd_unit cur;
-  rd_unit_load(cur, srow, e0, rin, rstr);
+  rd_unit_load<64>(cur, srow, e0, rin, rstr);
   for (; row < row_end; row++) {
     ga_long nso[RD_NSRC], nd0o = 0, nd1o = 0;
     const char *nrow[RD_NSRC];
@@ -528,9 +551,9 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       rd_row_offsets(p, row + 1, nso, &nd0o, &nd1o);
 #pragma unroll
       for (int k = 0; k < RD_NSRC; k++) nrow[k] = base[k] + nso[k];
-      rd_unit_load(nxt, nrow, e0, rin, rstr);
+      rd_unit_load<64>(nxt, nrow, e0, rin, rstr);
     }
-    rd_acc acc = rd_wave_reduce(rd_unit_combine(cur, e0, rin, 0, rml RD_SCALAR_ARGS));
+    rd_acc acc = rd_wave_reduce(rd_unit_combine<64>(cur, e0, rin, 0, rml RD_SCALAR_ARGS));
     if (lane == 0)
       rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
     cur = nxt;
@@ -540,48 +563,52 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
   }
 }
 #else
+/* RD_L lanes per row, 64 / RD_L rows side by side in a wavefront, RD_RB such
+ * sets per batch.  Every lane computes (a lane whose row is past the end
+ * works on the last row and does not store), so the cross-lane steps never
+ * see a disabled lane. */
 KERNEL void __launch_bounds__(256)
 redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
             const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
             const rd_plan p RD_SCALAR_PARAMS) {
   (void)part_v; (void)part_i;
   const unsigned lane = LID_0 & 63u;
+  const unsigned sub = lane / RD_L, l = lane % RD_L;
   const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
-  ga_long row = wave * p.upb;
-  ga_long row_end = row + p.upb;
+  ga_long row0 = wave * p.upb;
+  ga_long row_end = row0 + p.upb;
   if (row_end > p.nrows) row_end = p.nrows;
-  if (row >= row_end) return;
+  if (row0 >= row_end) return;
 
   const ga_long rin = p.nr > 0 ? p.rdim[0] : 1;
   const ga_long rml = p.nr > 0 ? p.rmul[0] : 0;
-  const ga_long e0 = (ga_long)lane * RD_VEC;
+  const ga_long e0 = (ga_long)l * RD_VEC;
   ga_long rstr[RD_NSRC];
   const char *base[RD_NSRC];
   RD_SRC_BASES(base);
 #pragma unroll
   for (int k = 0; k < RD_NSRC; k++) rstr[k] = p.nr > 0 ? p.rsstr[k][0] : 0;
 
-  for (; row < row_end; row += RD_RB) {
+  for (; row0 < row_end; row0 += (64 / RD_L) * RD_RB) {
     rd_unit x[RD_RB];
     ga_long d0o[RD_RB], d1o[RD_RB];
     const char *srow[RD_RB][RD_NSRC];
 #pragma unroll
     for (int b = 0; b < RD_RB; b++) {
-      if (row + b < row_end) {
-        ga_long so[RD_NSRC];
-        rd_row_offsets(p, row + b, so, &d0o[b], &d1o[b]);
+      ga_long row = row0 + b * (64 / RD_L) + sub;
+      if (row >= row_end) row = row_end - 1;
+      ga_long so[RD_NSRC];
+      rd_row_offsets(p, row, so, &d0o[b], &d1o[b]);
 #pragma unroll
-        for (int k = 0; k < RD_NSRC; k++) srow[b][k] = base[k] + so[k];
-        rd_unit_load(x[b], srow[b], e0, rin, rstr);
-      }
+      for (int k = 0; k < RD_NSRC; k++) srow[b][k] = base[k] + so[k];
+      rd_unit_load<RD_L>(x[b], srow[b], e0, rin, rstr);
     }
 #pragma unroll
     for (int b = 0; b < RD_RB; b++) {
-      if (row + b < row_end) {
-        rd_acc acc = rd_wave_reduce(rd_unit_combine(x[b], e0, rin, 0, rml RD_SCALAR_ARGS));
-        if (lane == 0)
-          rd_store(acc, srow[b], d0 + d0_off, d0o[b], d1 + d1_off, d1o[b], p.rtotal RD_SCALAR_ARGS);
-      }
+      const ga_long row = row0 + b * (64 / RD_L) + sub;
+      rd_acc acc = rd_seg_reduce<RD_L>(rd_unit_combine<RD_L>(x[b], e0, rin, 0, rml RD_SCALAR_ARGS));
+      if (l == RD_L - 1 && row < row_end)
+        rd_store(acc, srow[b], d0 + d0_off, d0o[b], d1 + d1_off, d1o[b], p.rtotal RD_SCALAR_ARGS);
     }
   }
 }
