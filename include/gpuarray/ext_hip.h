@@ -59,7 +59,12 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
                                            int strided, unsigned int nd, int idx64,
                                            unsigned int tmask);
 /* vec: elements used per load in bits 0..7, element step of the inner
- * reduced dim (1, 2 or 4; 0 means 1) in bits 8 and up. */
+ * reduced dim (1, 2 or 4; 0 means 1) in bits 8..15, adjacent outputs per lane
+ * of the column kernel in bits 16 and up (0 means 1).
+ * lanes_per_output: 64 or 256 in bits 0..15; lanes per row of the short-row
+ * kernel in bits 16 and up (0 means 64).
+ * unroll: loads in flight per lane in bits 0..7; rows per batch of the
+ * short-row kernel in bits 8 and up (0 means 1). */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

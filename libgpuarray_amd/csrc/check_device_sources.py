@@ -79,6 +79,10 @@ def main():
     for lanes in (1, 2, 8, 16, 32):
         check("reduction %d lanes per row" % lanes,
               gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64 | (lanes << 16), 4, 2 | (2 << 8)))
+    for cv, src in ((4, GA_FLOAT), (2, GA_DOUBLE), (8, GA_UBYTE)):
+        check("reduction %d outputs per lane" % cv,
+              gen_r(8 if src != GA_UBYTE else 0, src, src if src != GA_UBYTE else GA_LONG, GA_LONG,
+                    256, 1 | (cv << 16), 4))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),
@@ -101,7 +105,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "12 elementwise)" % (n + 11, m, t))
+          "12 elementwise)" % (n + 14, m, t))
 
 
 if __name__ == "__main__":

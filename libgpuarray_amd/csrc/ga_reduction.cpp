@@ -181,6 +181,7 @@ struct variant_spec {
   unsigned vecmask;   // bit k: array source k is fetched with vector loads
   unsigned RB;        // redux_wrows: rows per batch of loads
   unsigned L;         // redux_wrows: lanes per row
+  unsigned CV;        // redux_col: adjacent outputs per lane
 };
 
 const char *load_type_name(int tc) {
@@ -238,7 +239,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", vs.G, vs.V, vs.U);
   DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n#define RD_RB %u\n",
       vs.opts & 1u, (vs.opts >> 1) & 1u, vs.ES, vs.RB ? vs.RB : 1u);
-  DEF("#define RD_L %u\n", vs.L ? vs.L : 64u);
+  DEF("#define RD_L %u\n#define RD_CV %u\n", vs.L ? vs.L : 64u, vs.CV ? vs.CV : 1u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -314,6 +315,18 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   gen += "}\n#define RD_ONE_VAL(o) rd_map(";
   for (unsigned k = 0; k < K; k++) GEN("%srd_w%u((o).x%u)", k ? ", " : "", k, k);
   gen += " RD_SCALAR_ARGS)\n";
+  // RD_CV adjacent elements per source (redux_col)
+  for (unsigned k = 0; k < K; k++)
+    GEN("typedef %s rd_cv%u_t __attribute__((ext_vector_type(RD_CV)));\n",
+        load_type_name(gr->args[gr->arrays[k]].tc), k);
+  gen += "struct rd_cvec {";
+  for (unsigned k = 0; k < K; k++) GEN(" rd_cv%u_t x%u;", k, k);
+  gen += " };\nstatic __device__ inline void rd_cvec_load(rd_cvec &o, const char *const *p) {\n";
+  for (unsigned k = 0; k < K; k++)
+    GEN("  o.x%u = RD_LOAD((const rd_cv%u_t *)p[%u]);\n", k, k, k);
+  gen += "}\n#define RD_CVEC_VAL(o, c) rd_map(";
+  for (unsigned k = 0; k < K; k++) GEN("%srd_w%u((o).x%u[c])", k ? ", " : "", k, k);
+  gen += " RD_SCALAR_ARGS)\n";
 #undef GEN
   return GA_NO_ERROR;
 }
@@ -339,8 +352,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V, vs.U,
-           vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
+           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -666,7 +679,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1;
   bool wrows = false;
   size_t groups;
   if (use_row) {
@@ -806,11 +819,51 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     }
   } else {
     const int64_t fin = p.fdim[p.nf - 1];
-    p.gx = (fin + 63) / 64;
+    // Adjacent outputs per lane: as many as one 16-byte load of the widest
+    // source holds, when the inner free dim is contiguous in every source and
+    // every address a lane forms is a multiple of its load.
+    {
+      unsigned cv = (unsigned)(16 / elsz_max);
+      if (info.has_d1 && cv > 4) cv = 4;
+      if (cv > 8) cv = 8;
+      for (unsigned q = 0; q < K; q++)
+        if (fsstr[q * RD_MAXD + p.nf - 1] != elsz[q]) cv = 1;
+      while (cv > 1) {
+        bool ok = fin % cv == 0;
+        for (unsigned q = 0; ok && q < K; q++) {
+          const int64_t bytes = (int64_t)cv * elsz[q];
+          const uintptr_t base = (uintptr_t)srcs[q].a->data->devptr + srcs[q].a->offset;
+          ok = base % (uintptr_t)bytes == 0;
+          for (int i = 0; ok && i + 1 < p.nf; i++) ok = fsstr[q * RD_MAXD + i] % bytes == 0;
+          for (int i = 0; ok && i < p.nr; i++) ok = rsstr[q * RD_MAXD + i] % bytes == 0;
+        }
+        if (ok) break;
+        cv /= 2;
+      }
+      if (!env_ul("GPUARRAY_REDUX_COLVEC", 1)) cv = 1;
+      // Splitting the reduced range costs a second pass (sum over the middle
+      // axis of 256x512x512 floats: 54 us unsplit with one output per lane,
+      // 64 us split in two with four), so when the widest load leaves too
+      // few groups, take the widest one that still fills the chip unsplit.
+      {
+        const int64_t want = ncu * 4, outer_f = nrows / fin;
+        auto groups_at = [&](unsigned c) { return ((fin + 64 * c - 1) / (64 * c)) * outer_f; };
+        if (groups_at(cv) < want)
+          for (unsigned c = cv / 2; c >= 1; c /= 2)
+            if (groups_at(c) >= want) { cv = c; break; }
+      }
+      CV = cv;
+    }
+    p.gx = (fin + 64 * CV - 1) / (64 * CV);
     const int64_t outer = nrows / fin;
     const int64_t base_groups = p.gx * outer;
     int64_t nsplit = 1;
-    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 8);
+    // Measured on MI355X (sums over axis 0 of 8192x8192, 256x262144, 65536x1000
+    // and 8x2^23 floats): one output per lane 63.6 / 55.2 / 58.5 / 134 us with
+    // 8 groups per compute unit; four outputs per lane 50.1 / 45.8 / 50.5 /
+    // 49.6 us with 3-4 groups, and 60 / 84 / 61 / 51 us with 8 (the second
+    // shape then splits its 256 rows for nothing).
+    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? 4 : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
       if (nsplit > rtotal / 64) nsplit = rtotal / 64;
@@ -821,7 +874,8 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (p.upb > 0) nsplit = (rtotal + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;
     groups = (size_t)(base_groups * nsplit);
-    U = 4;
+    U = (unsigned)env_ul("GPUARRAY_REDUX_COL_U", 4);
+    if (U != 1 && U != 2 && U != 4 && U != 8) U = 4;
   }
   if (groups == 0 || groups > 0x7fffffffull)
     return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Reduction needs more groups than one launch has");
@@ -830,7 +884,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
   if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
-                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64};
+                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV};
   variant *var = nullptr;
   int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
@@ -894,12 +948,13 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
     return nullptr;
   // bits 8.. of V carry the element step of strided loads (0 means 1), bits
   // 8.. of U the rows per batch of redux_wrows (0 means 1), bits 16.. of G its
-  // lanes per row (0 means 64)
-  const unsigned ES = (V >> 8) ? (V >> 8) : 1;
+  // lanes per row (0 means 64), bits 16.. of V the outputs per lane of redux_col
+  const unsigned ES = ((V >> 8) & 0xffu) ? ((V >> 8) & 0xffu) : 1;
+  const unsigned cv_bits = V >> 16;
   V &= 0xffu;
   std::string s;
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu, 3, ES, 1, (U >> 8) ? (U >> 8) : 1,
-                     (G >> 16) ? (G >> 16) : 64};
+                     (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
@@ -916,7 +971,7 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64};
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64, 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

@@ -22,6 +22,7 @@
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
  *   RD_U        loads in flight per lane
+ *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
  *   RD_L        redux_wrows: lanes that share a row (power of two, <= 64);
  *               64 / RD_L rows sit side by side in a wavefront
  *   RD_RB       redux_wrows: sets of rows whose loads a wavefront issues together
@@ -303,6 +304,8 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
  *   RD_UNIT_VAL(u, j, v)     the reduced value of element v of load j
  *   struct rd_one, rd_one_load(o, ptrs), RD_ONE_VAL(o)   the same for one
  *                            element addressed by one pointer per source
+ *   struct rd_cvec, rd_cvec_load(o, ptrs), RD_CVEC_VAL(o, c)   the same for
+ *                            RD_CV adjacent elements (redux_col)
  * RD_PV (elements per vector load) and RD_LOAD are defined first because the
  * emitted text uses them. */
 #define RD_PV (RD_VEC * RD_ES)
@@ -615,12 +618,15 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 #endif
 #endif
 
-/* ---- redux_col ------------------------------------------------------------- */
+/* ---- redux_col -------------------------------------------------------------
+ * Lanes along the fastest free dim; a lane owns RD_CV adjacent outputs and
+ * fetches them with one load (RD_CV > 1 needs that dim to be contiguous in
+ * every source and everything aligned to the load). */
 
 KERNEL void __launch_bounds__(256)
 redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
           RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
-  __shared__ rd_acc lds[4][64];
+  __shared__ rd_acc lds[4][RD_CV][64];
   const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
   ga_long t = GID_0 / (unsigned)p.nsplit;
@@ -628,10 +634,10 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   const ga_long fo = t / p.gx;   /* flat index over the outer free dims */
   const int fi_d = p.nf - 1;
   const ga_long fin = p.fdim[fi_d];
-  const ga_long fi = bx * 64 + tx;
+  const ga_long fi = (bx * 64 + tx) * RD_CV;   /* first of the lane's outputs */
   const bool live = fi < fin;
 
-  /* offsets of this lane's output */
+  /* offsets of this lane's first output */
   ga_long so[RD_NSRC], d0o = 0, d1o = 0;
 #pragma unroll
   for (int k = 0; k < RD_NSRC; k++) so[k] = 0;
@@ -658,10 +664,12 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   ga_long r0 = split * p.upb, r1 = r0 + p.upb;
   if (r1 > p.rtotal) r1 = p.rtotal;
 
-  rd_acc acc = rd_neutral();
+  rd_acc acc[RD_CV];
+#pragma unroll
+  for (int c = 0; c < RD_CV; c++) acc[c] = rd_neutral();
   if (live) {
     for (ga_long j0 = r0 + ty; j0 < r1; j0 += 4 * RD_U) {
-      rd_one x[RD_U];
+      rd_cvec x[RD_U];
       ga_long idx[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
@@ -680,27 +688,40 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
           const char *ep[RD_NSRC];
 #pragma unroll
           for (int k = 0; k < RD_NSRC; k++) ep[k] = srow[k] + off[k];
-          rd_one_load(x[q], ep);
+          rd_cvec_load(x[q], ep);
           idx[q] = ix;
         }
       }
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
-        if (j0 + 4 * q < r1) acc = rd_combine(acc, rd_elem(RD_ONE_VAL(x[q]), idx[q]));
+        if (j0 + 4 * q < r1) {
+#pragma unroll
+          for (int c = 0; c < RD_CV; c++)
+            acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
+        }
     }
   }
-  lds[ty][tx] = acc;
+#pragma unroll
+  for (int c = 0; c < RD_CV; c++) lds[ty][c][tx] = acc[c];
   local_barrier();
   if (ty == 0 && live) {
-    acc = rd_combine(acc, lds[1][tx]);
-    acc = rd_combine(acc, lds[2][tx]);
-    acc = rd_combine(acc, lds[3][tx]);
-    const ga_long row = fo * fin + fi;
-    if (p.nsplit == 1) {
-      /* element 0 of the scan is at the start of the lane's reduced range */
-      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
-    } else {
-      rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
+#pragma unroll
+    for (int c = 0; c < RD_CV; c++) {
+      rd_acc a = acc[c];
+      a = rd_combine(a, lds[1][c][tx]);
+      a = rd_combine(a, lds[2][c][tx]);
+      a = rd_combine(a, lds[3][c][tx]);
+      const ga_long row = fo * fin + fi + c;
+      if (p.nsplit == 1) {
+        /* element 0 of the scan is at the start of the output's reduced range */
+        const char *sc[RD_NSRC];
+#pragma unroll
+        for (int k = 0; k < RD_NSRC; k++) sc[k] = srow[k] + c * p.fsstr[k][fi_d];
+        rd_store(a, sc, d0 + d0_off, d0o + c * p.fd0str[fi_d], d1 + d1_off,
+                 d1o + c * p.fd1str[fi_d], p.rtotal RD_SCALAR_ARGS);
+      } else {
+        rd_store_partial(a, part_v, part_i, row * p.nsplit + split);
+      }
     }
   }
 }
