@@ -83,6 +83,9 @@ def main():
         check("reduction %d outputs per lane" % cv,
               gen_r(8 if src != GA_UBYTE else 0, src, src if src != GA_UBYTE else GA_LONG, GA_LONG,
                     256, 1 | (cv << 16), 4))
+    for lo in (4, 16):
+        check("reduction %d outer coordinates side by side" % lo,
+              gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | (lo << 16)))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),
@@ -105,7 +108,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "12 elementwise)" % (n + 14, m, t))
+          "12 elementwise)" % (n + 16, m, t))
 
 
 if __name__ == "__main__":

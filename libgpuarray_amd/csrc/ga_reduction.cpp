@@ -39,7 +39,7 @@ constexpr unsigned RD_MAXSRC = 8;
 struct rd_plan {
   int64_t fdim[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
   int64_t rdim[RD_MAXD], rmul[RD_MAXD];
-  int64_t nrows, rtotal, nseg, units, upb, gx;
+  int64_t nrows, rtotal, nseg, units, upb, gx, router;
   int32_t nf, nr, nsplit, pad;
 };
 
@@ -182,6 +182,7 @@ struct variant_spec {
   unsigned RB;        // redux_wrows: rows per batch of loads
   unsigned L;         // redux_wrows: lanes per row
   unsigned CV;        // redux_col: adjacent outputs per lane
+  unsigned LO;        // redux_row: outer reduced coordinates side by side
 };
 
 const char *load_type_name(int tc) {
@@ -239,7 +240,8 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_G %u\n#define RD_VEC %u\n#define RD_U %u\n", vs.G, vs.V, vs.U);
   DEF("#define RD_NT %u\n#define RD_INTERLEAVE %u\n#define RD_ES %u\n#define RD_RB %u\n",
       vs.opts & 1u, (vs.opts >> 1) & 1u, vs.ES, vs.RB ? vs.RB : 1u);
-  DEF("#define RD_L %u\n#define RD_CV %u\n", vs.L ? vs.L : 64u, vs.CV ? vs.CV : 1u);
+  DEF("#define RD_L %u\n#define RD_CV %u\n#define RD_LO %u\n", vs.L ? vs.L : 64u,
+      vs.CV ? vs.CV : 1u, vs.LO ? vs.LO : 1u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -352,8 +354,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
-           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
+           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -679,7 +681,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1, LO = 1;
   bool wrows = false;
   size_t groups;
   if (use_row) {
@@ -748,12 +750,28 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     const int64_t lane_bytes = (int64_t)env_ul("GPUARRAY_REDUX_LANE_BYTES", K > 1 ? 64 : 128);
     while (U > 1 && (int64_t)U * V * ES * elsz_sum > lane_bytes) U /= 2;
     while (U > 1 && per_pass * (U / 2) >= rin) U /= 2;
+    int64_t outer = 1;
+    for (int i = 0; i + 1 < p.nr; i++) outer *= p.rdim[i];
+    // Several reduced dims with a short inner one (statistics over the batch
+    // and a small spatial extent, say): the lanes a row does not need take
+    // further outer reduced coordinates.  LI lanes cover the inner dim with up
+    // to four loads each, LO = G / LI outer coordinates sit side by side.
+    if (p.nr >= 2 && rtotal > 0 && G == 64 && env_ul("GPUARRAY_REDUX_LO", 1)) {
+      const int64_t need = (rin + (int64_t)V * 4 - 1) / ((int64_t)V * 4);
+      unsigned LI = 1;
+      while (LI < 64 && (int64_t)LI < need) LI *= 2;
+      if (LI < 64) {
+        LO = 64 / LI;
+        U = 1;
+        while (U < 8 && (int64_t)LI * V * U < rin) U *= 2;
+        per_pass = (int64_t)LI * V;
+      }
+    }
     const int64_t seg = per_pass * U;
     p.nseg = rin > 0 ? (rin + seg - 1) / seg : 1;
     if (p.nseg < 1) p.nseg = 1;
-    int64_t outer = 1;
-    for (int i = 0; i + 1 < p.nr; i++) outer *= p.rdim[i];
-    p.units = rtotal > 0 ? outer * p.nseg : 0;
+    p.router = outer;
+    p.units = rtotal > 0 ? (LO > 1 ? (outer + LO - 1) / LO : outer * p.nseg) : 0;
     const int64_t rows_per_group = 256 / G;
     const int64_t rowgroups = (nrows + rows_per_group - 1) / rows_per_group;
     // too few groups to fill the chip: cut the rows
@@ -884,7 +902,8 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
   if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
-                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV};
+                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
+                     (use_row && !wrows) ? LO : 1};
   variant *var = nullptr;
   int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
@@ -953,8 +972,9 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   const unsigned cv_bits = V >> 16;
   V &= 0xffu;
   std::string s;
-  variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu, 3, ES, 1, (U >> 8) ? (U >> 8) : 1,
-                     (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1};
+  variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu, (U >> 16) ? 1u : 3u, ES, 1,
+                     ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
+                     (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1, (U >> 16) ? (U >> 16) : 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
@@ -971,7 +991,7 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64, 1};
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64, 1, 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

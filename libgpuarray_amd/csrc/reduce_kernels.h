@@ -22,6 +22,8 @@
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
  *   RD_U        loads in flight per lane
+ *   RD_LO       redux_row: outer reduced coordinates handled side by side by
+ *               the RD_G lanes when the inner reduced dim is short (1: none)
  *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
  *   RD_L        redux_wrows: lanes that share a row (power of two, <= 64);
  *               64 / RD_L rows sit side by side in a wavefront
@@ -93,6 +95,7 @@ struct rd_plan {
   ga_long units;   /* redux_row: (outer reduced count) * nseg */
   ga_long upb;     /* work per split: units (row) or elements (col) */
   ga_long gx;      /* redux_col: groups along the inner free dim */
+  ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates */
   ga_int nf, nr, nsplit, pad;
   ga_long fsstr[RD_NSRC][RD_MAXD], rsstr[RD_NSRC][RD_MAXD];   /* per source */
 };
@@ -468,6 +471,28 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
   const ga_long ustep = 1;
 #endif
 
+#if RD_LO > 1
+  /* The inner reduced dim is short: RD_G / RD_LO lanes cover it and RD_LO
+   * outer reduced coordinates sit side by side; unit u holds the outer
+   * coordinates u*RD_LO .. u*RD_LO + RD_LO - 1. */
+  const unsigned li = lane % (RD_G / RD_LO), lo = lane / (RD_G / RD_LO);
+  const ga_long e0 = (ga_long)li * RD_VEC;
+  rd_acc acc = rd_neutral();
+  for (ga_long u = u0; u < u1; u += ustep) {
+    const ga_long ro = u * RD_LO + lo;
+    if (ro < p.router) {
+      ga_long rb[RD_NSRC], ib = 0;
+      rd_outer_offsets(p, ri, ro, rb, &ib);
+      rd_unit x;
+      const char *ub[RD_NSRC];
+#pragma unroll
+      for (int s = 0; s < RD_NSRC; s++) ub[s] = srow[s] + rb[s];
+      rd_unit_load<RD_G / RD_LO>(x, ub, e0, rin, rstr);
+      acc = rd_combine(acc, rd_unit_combine<RD_G / RD_LO>(x, e0, rin, ib, rml RD_SCALAR_ARGS));
+    }
+  }
+  (void)seg;
+#else
   /* unit -> (outer reduced coordinate ro, segment k of the inner dim): one
    * division for the first unit, then counted up */
   ga_long ro = 0, k = u0;
@@ -494,6 +519,8 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
     }
 #endif
   }
+
+#endif
 
 #if RD_G == 256
   acc = rd_block_reduce(acc, lds);

@@ -462,3 +462,72 @@ def test_config5_mixed_dtypes_strided(ctx, oracle):
     assert 0 < any_.sum() < any_.size                          # the test data exercises both answers
     ones = gpuarray.array(np.ones((8, 16, 64), np.uint8), context=ctx)[:, :, ::2]
     assert np.asarray(R.all(ones, axis=2)).all()
+
+
+# ---- lane geometries of the planner: short rows sharing a wavefront, short inner
+# ---- reduced dims with outer ones side by side, several outputs per lane ----------
+
+def _check_ops(ctx, host, axes):
+    """sum (exact for ints, 1e-5 for floats), maxandargmax and minandargmin
+    (bit-exact, first index on ties) of `host` over `axes`."""
+    g, _ = to_gpu_view(host, ctx)
+    axes = tuple(axes)
+    if host.dtype.kind in "iu":
+        got = np.asarray(R.sum(g, axis=axes, dtype="int64"))
+        assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64))
+    else:
+        got = np.asarray(R.sum(g, axis=axes))
+        want = host.sum(axis=axes, dtype=np.float64)
+        scale = np.abs(host).sum(axis=axes, dtype=np.float64)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(scale, 1e-30))
+    # flattened index over the reduced axes in ascending order = NumPy's on the moved array
+    moved = np.moveaxis(host, axes, range(host.ndim - len(axes), host.ndim))
+    flat = moved.reshape(moved.shape[:host.ndim - len(axes)] + (-1,))
+    for name, fn, afn in (("maxandargmax", np.max, np.argmax), ("minandargmin", np.min, np.argmin)):
+        val, idx = getattr(R, name)(g, axis=axes)
+        assert np.array_equal(np.asarray(val), fn(flat, axis=-1)), name
+        assert np.array_equal(np.asarray(idx), afn(flat, axis=-1)), name
+
+
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float64"])
+def test_short_rows_share_a_wavefront(ctx, dtype):
+    rng = np.random.default_rng(50)
+    for shape in ((1000, 1), (1000, 2), (1000, 3), (1003, 4), (517, 8), (777, 33), (513, 100),
+                  (129, 250), (65, 511), (70000, 5)):
+        host = rng.integers(0, 50, size=shape).astype(dtype)          # many ties
+        _check_ops(ctx, host, [1])
+    # rows that are not contiguous in the free direction, and a stepped inner dim
+    base = rng.integers(0, 50, size=(301, 40)).astype(dtype)
+    _check_ops(ctx, base[::3, :12], [1])
+    _check_ops(ctx, base[::-1, ::2], [1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "int32", "float64"])
+def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
+    rng = np.random.default_rng(51)
+    for shape, axes in (((32, 16, 7, 7), (0, 2, 3)), ((16, 24, 16, 20), (1, 3)), ((9, 5, 3), (0, 2)),
+                        ((40, 3, 50, 4), (0, 3)), ((6, 7, 1030, 2), (0, 1, 3)), ((300, 2, 16), (0, 2))):
+        host = rng.integers(0, 30, size=shape).astype(dtype)
+        _check_ops(ctx, host, axes)
+    # enough outer coordinates for the range to be split into partials
+    host = rng.integers(0, 30, size=(4096, 3, 12)).astype(dtype)
+    _check_ops(ctx, host, (0, 2))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float64", "float16"])
+def test_several_outputs_per_lane(ctx, dtype):
+    rng = np.random.default_rng(52)
+    for shape in ((300, 1000), (8, 4096), (1000, 256), (37, 20), (513, 772), (4, 64, 260)):
+        host = rng.integers(0, 40, size=shape).astype(dtype)
+        if dtype == "float16":
+            g, _ = to_gpu_view(host, ctx)
+            val, idx = R.maxandargmax(g, axis=0)
+            assert np.array_equal(np.asarray(val), host.max(axis=0))
+            assert np.array_equal(np.asarray(idx), host.argmax(axis=0))
+            continue
+        _check_ops(ctx, host, [0])
+    # misaligned bases and strides fall back to narrower loads
+    base = rng.integers(0, 40, size=(300, 1001)).astype(dtype if dtype != "float16" else "float32")
+    _check_ops(ctx, base[:, 1:], [0])
+    _check_ops(ctx, base[:, :1000], [0])
+    _check_ops(ctx, base[::2, 2:998:2], [0])
