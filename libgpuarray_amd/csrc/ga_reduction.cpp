@@ -756,7 +756,11 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     // and a small spatial extent, say): the lanes a row does not need take
     // further outer reduced coordinates.  LI lanes cover the inner dim with up
     // to four loads each, LO = G / LI outer coordinates sit side by side.
-    if (p.nr >= 2 && rtotal > 0 && G == 64 && env_ul("GPUARRAY_REDUX_LO", 1)) {
+    // Only when one load per lane would leave half the wavefront idle: rows
+    // of 512 stepped halves ran at 45.4 us with 64 lanes and two loads each,
+    // 47.4 us with 32 lanes and two outer coordinates side by side.
+    if (p.nr >= 2 && rtotal > 0 && G == 64 && rin <= (int64_t)32 * V &&
+        env_ul("GPUARRAY_REDUX_LO", 1)) {
       const int64_t need = (rin + (int64_t)V * 4 - 1) / ((int64_t)V * 4);
       unsigned LI = 1;
       while (LI < 64 && (int64_t)LI < need) LI *= 2;
