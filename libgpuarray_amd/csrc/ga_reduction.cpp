@@ -538,8 +538,13 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
       return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Reduction axis %d is out of range or repeated", ax);
     reduced[ax] = 1;
   }
+  for (const GpuArray *d : {(const GpuArray *)d0, (const GpuArray *)d1})
+    if (d != nullptr && d->data == nullptr)
+      return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array has no buffer");
   for (unsigned k = 0; k < K; k++) {
     const GpuArray *s = srcs[k].a;
+    if (s->data == nullptr)
+      return ga_err_set(ctx->err, GA_INVALID_ERROR, "A source array has no buffer");
     const int want = gr->args[gr->arrays[k]].tc;
     if (s->typecode != want)
       return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Source has typecode %d, operator was made for %d",
@@ -1101,6 +1106,8 @@ int GpuArray_maxandargmax(GpuArray *dstMax, GpuArray *dstArgmax, const GpuArray 
                           unsigned reduxLen, const unsigned *reduxList) {
   if (dstMax == nullptr || dstArgmax == nullptr || src == nullptr || src->nd == 0 ||
       reduxLen == 0 || reduxLen > src->nd || reduxList == nullptr)
+    return GA_INVALID_ERROR;
+  if (src->data == nullptr || dstMax->data == nullptr || dstArgmax->data == nullptr)
     return GA_INVALID_ERROR;
   gpucontext *ctx = GpuArray_context(src);
   if (ctx == nullptr) return GA_INVALID_ERROR;

@@ -1,0 +1,62 @@
+"""Host logic of the library where there is no device: the tests of the GPU
+suite that never look at a kernel's result (argument rules, buffer
+bookkeeping, the memory cache's limits, flag and stride arithmetic, compile
+errors, read/write checks) run here against tests/mock_runtime/mock_hip.cpp,
+a preloaded stand-in for the HIP runtime whose buffers are host memory and
+whose kernel launches do nothing.  The C client runs through context
+teardown the same way (its numeric checks fail, by construction; it must not
+crash).  On a GPU box the same tests run for real under `-m gpu`."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST_ONLY = [
+    "tests/test_gpu_buffer_array.py::test_context_properties",
+    "tests/test_gpu_buffer_array.py::test_buffer_alloc_retain_release",
+    "tests/test_gpu_buffer_array.py::test_buffer_read_write_move",
+    "tests/test_gpu_buffer_array.py::test_empty_zeros_orders_and_errors",
+    "tests/test_gpu_buffer_array.py::test_memory_cache_limits",
+    "tests/test_gpu_ndarray_api.py::test_hash_and_bool",
+    "tests/test_gpu_ndarray_api.py::test_zeros_and_empty",
+    "tests/test_gpu_ndarray_api.py::test_write_and_read",
+    "tests/test_gpu_take1.py::test_complex_is_refused_like_other_kernels",
+    "tests/test_gpu_take1.py::test_argument_rules",
+    "tests/test_gpu_reduction.py::test_maxandargmax_argument_errors",
+    "tests/test_gpu_reduction.py::test_reduction_wrong_out_and_axis",
+    "tests/test_gpu_elemwise.py::test_zero_sized",
+    "tests/test_gpu_elemwise.py::test_new_reports_compile_errors",
+]
+
+
+@pytest.fixture(scope="module")
+def mock_runtime(tmp_path_factory):
+    out = tmp_path_factory.mktemp("mock") / "libmockhip.so"
+    subprocess.check_call(["g++", "-shared", "-fPIC", "-O1", "-I/opt/rocm/include",
+                           "-D__HIP_PLATFORM_AMD__",
+                           os.path.join(ROOT, "tests", "mock_runtime", "mock_hip.cpp"), "-o", str(out)])
+    return str(out)
+
+
+def test_host_only_tests_pass_without_a_device(mock_runtime):
+    env = dict(os.environ, LD_PRELOAD=mock_runtime)
+    r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-m", "gpu", "-p", "no:cacheprovider",
+                        "--timeout", "300"] + HOST_ONLY, cwd=ROOT, env=env, capture_output=True,
+                       text=True, timeout=900)
+    assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
+
+
+def test_c_client_survives_teardown_without_a_device(mock_runtime, tmp_path):
+    libdir = os.path.join(ROOT, "libgpuarray_amd")
+    exe = tmp_path / "client"
+    subprocess.check_call(["gcc", "-std=gnu99", "-O1", "-I", os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "c_client", "client.c"), "-o", str(exe),
+                           "-L", libdir, "-l:libgpuarray.so", "-Wl,-rpath," + libdir])
+    r = subprocess.run([str(exe)], env=dict(os.environ, LD_PRELOAD=mock_runtime),
+                       capture_output=True, text=True, timeout=300)
+    # kernels do nothing here, so the numeric checks fail (status 1); what is
+    # asked is that every host path, context teardown included, runs through
+    assert r.returncode in (0, 1), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+    assert "checks failed" in r.stdout or "all checks passed" in r.stdout
