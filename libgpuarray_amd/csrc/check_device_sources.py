@@ -86,6 +86,10 @@ def main():
     for lo in (4, 16):
         check("reduction %d outer coordinates side by side" % lo,
               gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | (lo << 16)))
+    for op, src in ((0, GA_FLOAT), (8, GA_FLOAT), (13, GA_UBYTE), (0, GA_HALF)):
+        check("reduction element-aligned loads with a ragged end, op %d type %d" % (op, src),
+              gen_r(op, src, GA_BOOL if op == 13 else GA_FLOAT, GA_LONG, 256, 4 if src == GA_FLOAT else 8,
+                    4 | (1 << 24)))
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),
@@ -108,7 +112,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "12 elementwise)" % (n + 16, m, t))
+          "12 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

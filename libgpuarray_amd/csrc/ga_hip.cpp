@@ -1303,6 +1303,16 @@ gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
   return ctx->scratch;
 }
 
+// Bytes from the start of a buffer that a kernel may read without leaving the
+// memory behind it: the cache block for the library's own allocations (a
+// multiple of 256), the stated size for memory wrapped by hip_make_buf.
+size_t ga_hip_readable_bytes(gpudata *b) {
+  hip_data *d = HD(b);
+  if (d->block != nullptr) return d->block->size;
+  if (!(d->flags & BUF_OWNED)) return d->sz;     // caller's memory
+  return (d->sz + 15) & ~(size_t)15;             // straight from the driver
+}
+
 unsigned int ga_hip_numprocs(gpucontext *c) { return HC(c)->numprocs; }
 void **ga_hip_redux_cache_slot(gpucontext *c) { return &HC(c)->redux_cache; }
 void **ga_hip_take1_cache_slot(gpucontext *c) { return &HC(c)->take1_cache; }

@@ -135,6 +135,9 @@ extern const char ga_reduce_kernels_src[];
 // reductions).  Work on a context is in stream order, so one buffer is
 // shared by consecutive calls.
 gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
+// Bytes from a buffer's start that lie inside the memory behind it (at least
+// its size; more when the allocation was rounded up).
+size_t ga_hip_readable_bytes(gpudata *b);
 // Number of compute units of the context's device.
 unsigned int ga_hip_numprocs(gpucontext *ctx);
 // Frees the strided-copy operator cache of a context (array.cpp).

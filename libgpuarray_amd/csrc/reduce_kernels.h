@@ -21,6 +21,11 @@
  *               advances by RD_ES elements per index (a [::2] or [::4] view), a
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
+ *   RD_TAIL     rows that are misaligned for the vector load or whose extent
+ *               is not a multiple of RD_VEC (one source, contiguous rows): a
+ *               row is read from the vector boundary at or below its start,
+ *               `sh` elements early, and every element is tested against
+ *               [sh, sh + extent); RD_ELSZ0 is the element size in bytes
  *   RD_U        loads in flight per lane
  *   RD_LO       redux_row: outer reduced coordinates handled side by side by
  *               the RD_G lanes when the inner reduced dim is short (1: none)
@@ -319,6 +324,20 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
 #define RD_LOAD(p) (*(p))
 #endif
 
+/* A use of a loaded value that no branch can skip.  The compiler waits for a
+ * load where its result is first used; when every use sits under a branch that
+ * some path skips, the result still counts as pending at the loop's back edge,
+ * and in the next round each load of the unit waits for the one before it
+ * (their destination registers may be in flight) instead of all being issued
+ * back to back.  Costs no instruction. */
+static __device__ inline void rd_touch(const ga_float v) { asm volatile("" ::"v"(v)); }
+static __device__ inline void rd_touch(const ga_double v) { asm volatile("" ::"v"(v)); }
+template <typename T>
+static __device__ inline void rd_touch(const T v) {
+  if (sizeof(T) > 4) asm volatile("" ::"v"((ga_ulong)v));
+  else asm volatile("" ::"v"((ga_uint)v));
+}
+
 /*@RD_GENERATED@*/
 
 /* Write the finished value(s) of one output. */
@@ -374,41 +393,89 @@ static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *
  *
  * Combination of the lane's elements of one unit.  ib, rml: index of element
  * 0 of the inner dim and index step per element. */
+#if RD_TAIL
+/* elements a row starts before its first one, and the pointer moved back by that */
+#define RD_SHIFT(ptr) ((ga_long)(((ga_size)(ptr) / RD_ELSZ0) % RD_VEC))
+#else
+#define RD_SHIFT(ptr) ((ga_long)0)
+#endif
+
+/* `rin` is the end of the row in the lane's coordinates (extent + sh), `sh`
+ * its start (0 unless RD_TAIL). */
 template <int LN>
 static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga_long rin,
-                                                ga_long ib, ga_long rml RD_SCALAR_FPARAMS) {
+                                                ga_long ib, ga_long rml, ga_long sh RD_SCALAR_FPARAMS) {
+  (void)sh;
 #if RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN
+#if RD_TAIL
+  /* A unit that touches an end of the row: the lane's first valid element can
+   * be anywhere.  No branch around a use of the loaded registers, here or
+   * below: a path that skips every use leaves the loads pending at the loop's
+   * back edge, and the next unit's loads then wait for one another. */
+  if (e0 < sh || e0 + (ga_long)(RD_U - 1) * LN * RD_VEC + RD_VEC > rin) {
+    RD_ACC_T bv = RD_NEUTRAL;
+    ga_int bp = 0;
+    bool found = false;
+#pragma unroll
+    for (int j = 0; j < RD_U; j++) {
+      const ga_long e = e0 + (ga_long)j * LN * RD_VEC;
+      const ga_long dl = sh - e, dh = rin - e;
+      const int lo = dl > RD_VEC ? RD_VEC : (int)dl;
+      const int hi = dh < 0 ? 0 : (dh > RD_VEC ? RD_VEC : (int)dh);
+#pragma unroll
+      for (int v = 0; v < RD_VEC; v++) {
+        const bool valid = v >= lo && v < hi;
+        const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
+#if RD_KIND == RD_K_MAX
+        const bool better = valid && (!found || val > bv);
+#else
+        const bool better = valid && (!found || val < bv);
+#endif
+        bv = better ? val : bv;
+        bp = better ? (j * LN * RD_VEC + v) : bp;
+        found = found || valid;
+      }
+    }
+    rd_acc r = rd_neutral();
+    r.v = found ? bv : r.v;
+#if RD_ARG
+    r.i = found ? ib + (e0 + bp - sh) * rml : r.i;
+#else
+    (void)ib; (void)rml;
+#endif
+    return r;
+  }
+#endif
   /* The lane's elements are visited in rising index order, so a strict
    * compare keeps the first of equals by itself; only the position inside
    * the unit (a small int) is tracked. */
-  rd_acc r = rd_neutral();
-  if (e0 < rin) {
-    RD_ACC_T bv = rd_elem(RD_UNIT_VAL(x, 0, 0), 0).v;
-    ga_int bp = 0;
+  /* (with RD_TAIL only units wholly inside the row come here) */
+  RD_ACC_T bv = rd_elem(RD_UNIT_VAL(x, 0, 0), 0).v;
+  ga_int bp = 0;
 #pragma unroll
-    for (int j = 0; j < RD_U; j++) {
-      if (e0 + (ga_long)j * LN * RD_VEC < rin) {
+  for (int j = 0; j < RD_U; j++) {
+    const bool in = RD_TAIL || e0 + (ga_long)j * LN * RD_VEC < rin;
 #pragma unroll
-        for (int v = 0; v < RD_VEC; v++) {
-          if (j == 0 && v == 0) continue;
-          const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
+    for (int v = 0; v < RD_VEC; v++) {
+      if (j == 0 && v == 0) continue;
+      const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
 #if RD_KIND == RD_K_MAX
-          const bool better = val > bv;
+      const bool better = in && val > bv;
 #else
-          const bool better = val < bv;
+      const bool better = in && val < bv;
 #endif
-          bv = better ? val : bv;
-          bp = better ? (j * LN * RD_VEC + v) : bp;
-        }
-      }
+      bv = better ? val : bv;
+      bp = better ? (j * LN * RD_VEC + v) : bp;
     }
-    r.v = bv;
-#if RD_ARG
-    r.i = ib + (e0 + bp) * rml;
-#else
-    (void)bp; (void)ib; (void)rml;
-#endif
   }
+  rd_acc r = rd_neutral();
+  const bool any = RD_TAIL || e0 < rin;
+  r.v = any ? bv : r.v;
+#if RD_ARG
+  r.i = any ? ib + (e0 + bp - sh) * rml : r.i;
+#else
+  (void)bp; (void)ib; (void)rml;
+#endif
   return r;
 #else
   rd_acc t[RD_U];
@@ -416,11 +483,23 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
   for (int j = 0; j < RD_U; j++) {
     const ga_long e = e0 + (ga_long)j * LN * RD_VEC;
     t[j] = rd_neutral();
+#if RD_TAIL
+    /* every element under a select, no branch (see above) */
+    const ga_long dl = sh - e, dh = rin - e;
+    const int lo = dl > RD_VEC ? RD_VEC : (int)dl;
+    const int hi = dh < 0 ? 0 : (dh > RD_VEC ? RD_VEC : (int)dh);
+#pragma unroll
+    for (int v = 0; v < RD_VEC; v++) {
+      const rd_acc c = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v - sh) * rml));
+      t[j] = (v >= lo && v < hi) ? c : t[j];
+    }
+#else
     if (e < rin) {
 #pragma unroll
       for (int v = 0; v < RD_VEC; v++)
-        t[j] = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v) * rml));
+        t[j] = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v - sh) * rml));
     }
+#endif
   }
   /* pairwise over the unit */
 #pragma unroll
@@ -487,8 +566,11 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
       const char *ub[RD_NSRC];
 #pragma unroll
       for (int s = 0; s < RD_NSRC; s++) ub[s] = srow[s] + rb[s];
-      rd_unit_load<RD_G / RD_LO>(x, ub, e0, rin, rstr);
-      acc = rd_combine(acc, rd_unit_combine<RD_G / RD_LO>(x, e0, rin, ib, rml RD_SCALAR_ARGS));
+      const ga_long sh = RD_SHIFT(ub[0]);
+      ub[0] -= sh * RD_ELSZ0;
+      rd_unit_load<RD_G / RD_LO>(x, ub, e0, rin + sh, rstr);
+      rd_unit_touch(x);
+      acc = rd_combine(acc, rd_unit_combine<RD_G / RD_LO>(x, e0, rin + sh, ib, rml, sh RD_SCALAR_ARGS));
     }
   }
   (void)seg;
@@ -507,8 +589,11 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
     const char *ub[RD_NSRC];
 #pragma unroll
     for (int s = 0; s < RD_NSRC; s++) ub[s] = srow[s] + rb[s];
-    rd_unit_load<RD_G>(x, ub, e0, rin, rstr);
-    acc = rd_combine(acc, rd_unit_combine<RD_G>(x, e0, rin, ib, rml RD_SCALAR_ARGS));
+    const ga_long sh = RD_SHIFT(ub[0]);
+    ub[0] -= sh * RD_ELSZ0;
+    rd_unit_load<RD_G>(x, ub, e0, rin + sh, rstr);
+    rd_unit_touch(x);
+    acc = rd_combine(acc, rd_unit_combine<RD_G>(x, e0, rin + sh, ib, rml, sh RD_SCALAR_ARGS));
 #if RD_INTERLEAVE
     k += ustep;   /* single reduced dim: the unit is the segment */
 #else
@@ -542,7 +627,7 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
  * first row is combined, so a wavefront whose row is a single load per lane
  * still has RD_RB loads in flight.  Only built for RD_G == 64. */
 #if RD_G == 64
-#if RD_RB == 1 && RD_L == 64
+#if RD_RB == 1 && RD_L == 64 && !RD_TAIL
 /* one row at a time; with upb > 1 the next row's loads are issued before the
  * current row is combined */
 KERNEL void __launch_bounds__(256)
@@ -583,7 +668,7 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       for (int k = 0; k < RD_NSRC; k++) nrow[k] = base[k] + nso[k];
       rd_unit_load<64>(nxt, nrow, e0, rin, rstr);
     }
-    rd_acc acc = rd_wave_reduce(rd_unit_combine<64>(cur, e0, rin, 0, rml RD_SCALAR_ARGS));
+    rd_acc acc = rd_wave_reduce(rd_unit_combine<64>(cur, e0, rin, 0, rml, 0 RD_SCALAR_ARGS));
     if (lane == 0)
       rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
     cur = nxt;
@@ -621,7 +706,7 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 
   for (; row0 < row_end; row0 += (64 / RD_L) * RD_RB) {
     rd_unit x[RD_RB];
-    ga_long d0o[RD_RB], d1o[RD_RB];
+    ga_long d0o[RD_RB], d1o[RD_RB], sh[RD_RB];
     const char *srow[RD_RB][RD_NSRC];
 #pragma unroll
     for (int b = 0; b < RD_RB; b++) {
@@ -629,14 +714,20 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       if (row >= row_end) row = row_end - 1;
       ga_long so[RD_NSRC];
       rd_row_offsets(p, row, so, &d0o[b], &d1o[b]);
+      const char *lp[RD_NSRC];
 #pragma unroll
-      for (int k = 0; k < RD_NSRC; k++) srow[b][k] = base[k] + so[k];
-      rd_unit_load<RD_L>(x[b], srow[b], e0, rin, rstr);
+      for (int k = 0; k < RD_NSRC; k++) lp[k] = srow[b][k] = base[k] + so[k];
+      sh[b] = RD_SHIFT(lp[0]);
+      lp[0] -= sh[b] * RD_ELSZ0;
+      rd_unit_load<RD_L>(x[b], lp, e0, rin + sh[b], rstr);
     }
+#pragma unroll
+    for (int b = RD_RB - 1; b >= 0; b--) rd_unit_touch(x[b]);
 #pragma unroll
     for (int b = 0; b < RD_RB; b++) {
       const ga_long row = row0 + b * (64 / RD_L) + sub;
-      rd_acc acc = rd_seg_reduce<RD_L>(rd_unit_combine<RD_L>(x[b], e0, rin, 0, rml RD_SCALAR_ARGS));
+      rd_acc acc = rd_seg_reduce<RD_L>(
+          rd_unit_combine<RD_L>(x[b], e0, rin + sh[b], 0, rml, sh[b] RD_SCALAR_ARGS));
       if (l == RD_L - 1 && row < row_end)
         rd_store(acc, srow[b], d0 + d0_off, d0o[b], d1 + d1_off, d1o[b], p.rtotal RD_SCALAR_ARGS);
     }

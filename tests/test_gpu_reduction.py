@@ -531,3 +531,28 @@ def test_several_outputs_per_lane(ctx, dtype):
     _check_ops(ctx, base[:, 1:], [0])
     _check_ops(ctx, base[:, :1000], [0])
     _check_ops(ctx, base[::2, 2:998:2], [0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64"])
+def test_ragged_and_misaligned_rows_take_vector_loads(ctx, dtype):
+    """Rows whose length is not a multiple of the load, or that start at an
+    address that is only element-aligned: every element still counts once."""
+    rng = np.random.default_rng(53)
+    for shape in ((300, 1023), (7, 4097), (64, 33), (1, 100003), (5, 4), (129, 17), (3, 70001)):
+        host = rng.integers(0, 40, size=shape).astype(dtype)
+        if dtype == "float16":
+            g, _ = to_gpu_view(host, ctx)
+            val, idx = R.maxandargmax(g, axis=1)
+            assert np.array_equal(np.asarray(val), host.max(axis=1))
+            assert np.array_equal(np.asarray(idx), host.argmax(axis=1))
+            got = np.asarray(R.sum(g, axis=1, dtype="float32"))
+            assert np.array_equal(got, host.astype(np.float32).sum(axis=1))     # small integers: exact
+            continue
+        _check_ops(ctx, host, [1])
+    base = rng.integers(0, 40, size=(50, 2051)).astype(dtype if dtype != "float16" else "float32")
+    _check_ops(ctx, base[:, 1:], [1])           # aligned length, misaligned start
+    _check_ops(ctx, base[:, 3:2050], [1])
+    _check_ops(ctx, base[::-1, 2:], [1])
+    flat = rng.integers(0, 40, size=(1 << 22) + 5).astype(dtype if dtype != "float16" else "float32")
+    _check_ops(ctx, flat[1:], [0])              # split over many groups, ragged end
+    _check_ops(ctx, flat[3:-1], [0])
