@@ -58,41 +58,7 @@ class GpuReduction(object):
                                     len(axes), arr, 0), self.context.ctx)
 
 
-class Argument(object):
-    """reference pygpu/tools.py:22-37"""
-
-    def __init__(self, dtype, name):
-        self.dtype = np.dtype(dtype)
-        self.name = name
-
-    def __hash__(self):
-        return hash(type(self)) ^ hash(self.dtype) ^ hash(self.name)
-
-    def __eq__(self, other):
-        return type(self) == type(other) and self.dtype == other.dtype and self.name == other.name
-
-
-class ArrayArg(Argument):
-    def isarray(self):
-        return True
-
-    def expr(self):
-        return "%s[i]" % (self.name,)
-
-
-class ScalarArg(Argument):
-    def isarray(self):
-        return False
-
-    def expr(self):
-        return self.name
-
-
-def as_argument(obj, name):
-    """reference pygpu/tools.py:15-19"""
-    if isinstance(obj, GpuArray):
-        return ArrayArg(obj.dtype, name)
-    return ScalarArg(np.asarray(obj).dtype, name)
+from .tools import Argument, ArrayArg, ScalarArg, as_argument  # noqa: E402,F401
 
 
 _C_TYPES = {
