@@ -65,8 +65,9 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
  * kernel in bits 16 and up (0 means 64).
  * unroll: loads in flight per lane in bits 0..7; rows per batch of the
  * short-row kernel in bits 8..15 (0 means 1); outer reduced coordinates the
- * row kernel handles side by side in bits 16..23 (0 means 1); bit 24: vector
- * loads with element alignment only and a ragged end of the row. */
+ * row kernel handles side by side in bits 16..23 (0 means 1); bit 24: rows
+ * read from the 16-byte boundary below their start, both ends masked; bit 25:
+ * also the kernel that stages short contiguous rows in LDS. */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

@@ -87,9 +87,14 @@ def main():
         check("reduction %d outer coordinates side by side" % lo,
               gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | (lo << 16)))
     for op, src in ((0, GA_FLOAT), (8, GA_FLOAT), (13, GA_UBYTE), (0, GA_HALF)):
-        check("reduction element-aligned loads with a ragged end, op %d type %d" % (op, src),
+        check("reduction rows read from the boundary below their start, op %d type %d" % (op, src),
               gen_r(op, src, GA_BOOL if op == 13 else GA_FLOAT, GA_LONG, 256, 4 if src == GA_FLOAT else 8,
                     4 | (1 << 24)))
+    for op, src, d0 in ((0, GA_FLOAT, GA_FLOAT), (8, GA_FLOAT, GA_FLOAT), (13, GA_UBYTE, GA_BOOL),
+                        (0, GA_HALF, GA_FLOAT), (4, GA_DOUBLE, GA_DOUBLE), (0, GA_INT, GA_LONG)):
+        check("reduction short rows staged in LDS, op %d type %d" % (op, src),
+              gen_r(op, src, d0, GA_LONG, 64, 1, 1 | (1 << 25)))
+        n += 1
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),

@@ -126,7 +126,8 @@ std::string neutral_for(rd_kind kind, int acc_tc) {
 
 struct variant {
   GpuKernel row = {nullptr, nullptr}, col = {nullptr, nullptr}, fin = {nullptr, nullptr},
-            wrows = {nullptr, nullptr};   // wrows only exists in 64-lane variants
+            wrows = {nullptr, nullptr},   // wrows only exists in 64-lane variants
+            srows = {nullptr, nullptr};   // the only kernel of a short-rows variant (opts bit 3)
 };
 
 struct dimrec {
@@ -244,6 +245,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
       vs.CV ? vs.CV : 1u, vs.LO ? vs.LO : 1u);
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
+  DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -399,7 +401,13 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   variant v;
   const char *names[4] = {"redux_row", "redux_col", "redux_final", "redux_wrows"};
   GpuKernel *ks[4] = {&v.row, &v.col, &v.fin, &v.wrows};
-  for (int i = 0; i < (vs.G == 64 ? 4 : 3); i++) {
+  int nk = vs.G == 64 ? 4 : 3;
+  if (vs.opts & 8u) {
+    names[0] = "redux_srows";
+    ks[0] = &v.srows;
+    nk = 1;
+  }
+  for (int i = 0; i < nk; i++) {
     err = GpuKernel_init(ks[i], ctx, 1, strs, lens, names[i], na, types.data(), kflags, nullptr);
     if (err != GA_NO_ERROR) {
       for (int j = 0; j < i; j++) GpuKernel_clear(ks[j]);
@@ -698,8 +706,8 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   }
 
   unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1, LO = 1;
-  bool wrows = false, tail = false;
-  size_t groups;
+  bool wrows = false, tail = false, srows = false;
+  size_t groups, lds_bytes = 0;
   if (use_row) {
     // Widest aligned load the layout allows, for a source whose inner reduced
     // stride is its element size: v elements, v*elsz bytes, everything the
@@ -861,6 +869,22 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
         const int64_t need = (rin_sz + (int64_t)V * 4 - 1) / ((int64_t)V * 4);
         L = 1;
         while (L < 64 && (int64_t)L < need) L *= 2;
+        // Up to 32 lanes, one load per lane and more lanes per row do better
+        // than four loads on few lanes (the batches keep the loads in flight):
+        // sums over rows of 32 floats 79.6 us with 2 lanes x 4 loads, 45.7 with
+        // 8 x 1; rows of 100: 42.0 with 8 x 4, 34.6 with 32 x 1; rows of 17:
+        // 76.9 -> 59.6.  Min/max carry an index through every cross-lane
+        // step, so they keep two loads per lane (rows of 64: 80 us with 16
+        // lanes, 67 with 8).
+        // (vector loads only: rows of 3 floats, element loads, 60 us with one
+        // lane per row and 74 with four).
+        if (V > 1) {
+          const int64_t per_lane = (int64_t)V * (minmax ? 2 : 1);
+          const int64_t need1 = (rin_sz + per_lane - 1) / per_lane;
+          unsigned l1 = 1;
+          while (l1 < 64 && (int64_t)l1 < need1) l1 *= 2;
+          if (l1 <= 32) L = l1;
+        }
         const unsigned long force = env_ul("GPUARRAY_REDUX_L", 0);
         if (force >= 1 && force <= 64 && (force & (force - 1)) == 0 &&
             (int64_t)force * V * 8 >= rin_sz)
@@ -878,6 +902,36 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
       p.upb = rpw;
       const int64_t waves = (nrows + rpw - 1) / rpw;
       groups = (size_t)((waves + 3) / 4);
+    }
+    // Rows of a few dozen elements that follow one another in memory: a group
+    // stages the bytes of up to 256 rows in LDS and every lane walks one row
+    // (redux_srows).  Measured on MI355X, 2^26 floats in rows of 8 / 17 / 33 /
+    // 64: sum 63 / 72 / 68 / 48 us with redux_wrows, 51 / 48 / 46 / 45 us
+    // staged; maxandargmax 73 / 76 / 78 / 56 against 59 / 53 / 53 / 72 us
+    // (its walk costs more per element, and 64 KiB of LDS per group leaves
+    // two groups per compute unit), hence the lower limit for min/max.
+    if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] &&
+        fsstr[0] == rin * elsz[0] && rin >= 2 &&
+        rin * elsz[0] <= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MAX_BYTES", minmax ? 160 : 256) &&
+        rin * elsz[0] > (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_BYTES", 16) &&
+        nrows >= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_ROWS", 512) * ncu &&
+        GpuArray_ISALIGNED(srcs[0].a) && env_ul("GPUARRAY_REDUX_SROWS", 1)) {
+      const GpuArray *s0 = srcs[0].a;
+      const size_t readable = ga_hip_readable_bytes(s0->data);
+      const size_t end = ((size_t)s0->offset + (size_t)(nrows * rin * elsz[0]) + 15) & ~(size_t)15;
+      if ((uintptr_t)s0->data->devptr % 16 == 0 && end <= readable) {
+        int64_t per_group = (65536 - 16) / (rin * elsz[0]);
+        if (per_group > 256) per_group = 256;
+        per_group &= ~(int64_t)63;   // whole wavefronts
+        if (per_group >= 64) {
+          srows = true;
+          wrows = false;
+          p.nsplit = 1;
+          p.upb = per_group;
+          groups = (size_t)((nrows + per_group - 1) / per_group);
+          lds_bytes = (size_t)(per_group * rin * elsz[0] + 16 + 15) & ~(size_t)15;
+        }
+      }
     }
   } else {
     const int64_t fin = p.fdim[p.nf - 1];
@@ -949,6 +1003,8 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
                      use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
                      (use_row && !wrows) ? LO : 1};
+  if (srows)   // one kernel, independent of the lane geometry
+    vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
   variant *var = nullptr;
   int err = get_variant(gr, vs, &var);
   if (err != GA_NO_ERROR) return err;
@@ -990,8 +1046,8 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   args.push_back(planbuf.data());
   for (void *sc : scalars) args.push_back(sc);
   size_t ls = 256;
-  GpuKernel *k1 = use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
-  if ((err = GpuKernel_call(k1, 1, &groups, &ls, 0, args.data())) != GA_NO_ERROR) return err;
+  GpuKernel *k1 = srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
+  if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
   if (p.nsplit > 1) {
     size_t fg = (size_t)((nrows + 3) / 4);
     if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args.data())) != GA_NO_ERROR) return err;
@@ -1018,7 +1074,8 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   V &= 0xffu;
   std::string s;
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
-                     ((U >> 16) & 0xffu ? 1u : 3u) | ((U >> 24) ? 4u : 0u), ES, 1,
+                     ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
+                         (((U >> 25) & 1u) ? 8u : 0u), ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};
@@ -1073,6 +1130,7 @@ void GpuReduction_free(GpuReduction *gr) {
     GpuKernel_clear(&kv.second.col);
     GpuKernel_clear(&kv.second.fin);
     if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
+    if (kv.second.srows.k != nullptr) GpuKernel_clear(&kv.second.srows);
   }
   delete gr;
 }

@@ -21,6 +21,7 @@
  *               advances by RD_ES elements per index (a [::2] or [::4] view), a
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
+ *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
  *   RD_TAIL     rows that are misaligned for the vector load or whose extent
  *               is not a multiple of RD_VEC (one source, contiguous rows): a
  *               row is read from the vector boundary at or below its start,
@@ -340,25 +341,25 @@ static __device__ inline void rd_touch(const T v) {
 
 /*@RD_GENERATED@*/
 
-/* Write the finished value(s) of one output. */
-static __device__ inline void rd_store(rd_acc a, const char *const *srow, char *d0, ga_long d0o,
-                                       char *d1, ga_long d1o, ga_long rtotal RD_SCALAR_FPARAMS) {
-#if RD_FLT && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN)
-  /* a NaN in the first position of the scan stays (see the header) */
-  if (rtotal > 0) {
-    rd_one o;
-    rd_one_load(o, srow);
-    const RD_ACC_T first = (RD_ACC_T)RD_ONE_VAL(o);
-    if (first != first) {
-      a.v = first;
+/* A NaN in the first position of a floating min/max scan stays (see the
+ * header): `first` is the value at that position. */
+#define RD_FIRST_RULE (RD_FLT && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN))
+static __device__ inline rd_acc rd_first_rule(rd_acc a, const RD_ACC_T first) {
+#if RD_FIRST_RULE
+  if (first != first) {
+    a.v = first;
 #if RD_ARG
-      a.i = 0;
+    a.i = 0;
 #endif
-    }
   }
 #else
-  (void)srow; (void)rtotal;
+  (void)first;
 #endif
+  return a;
+}
+
+/* Write the finished value(s) of one output. */
+static __device__ inline void rd_write(rd_acc a, char *d0, ga_long d0o, char *d1, ga_long d1o) {
 #if RD_HAS_D0
 #if RD_DST_HALF
   *(ga_half *)(d0 + d0o) = ga_float2half((float)a.v);
@@ -373,6 +374,23 @@ static __device__ inline void rd_store(rd_acc a, const char *const *srow, char *
 #else
   (void)d1; (void)d1o;
 #endif
+}
+
+/* The same for a caller that does not hold the scan's first value: it is
+ * fetched from the row again (one element per output; the short-row kernels,
+ * where that would double the traffic, pass it from their registers). */
+static __device__ inline void rd_store(rd_acc a, const char *const *srow, char *d0, ga_long d0o,
+                                       char *d1, ga_long d1o, ga_long rtotal RD_SCALAR_FPARAMS) {
+#if RD_FIRST_RULE
+  if (rtotal > 0) {
+    rd_one o;
+    rd_one_load(o, srow);
+    a = rd_first_rule(a, (RD_ACC_T)RD_ONE_VAL(o));
+  }
+#else
+  (void)srow; (void)rtotal;
+#endif
+  rd_write(a, d0, d0o, d1, d1o);
 }
 
 static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *pi, ga_long slot) {
@@ -669,8 +687,8 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       rd_unit_load<64>(nxt, nrow, e0, rin, rstr);
     }
     rd_acc acc = rd_wave_reduce(rd_unit_combine<64>(cur, e0, rin, 0, rml, 0 RD_SCALAR_ARGS));
-    if (lane == 0)
-      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
+    if (lane == 0)   /* which also holds the row's first element */
+      rd_write(rd_first_rule(acc, (RD_ACC_T)RD_UNIT_VAL(cur, 0, 0)), d0 + d0_off, d0o, d1 + d1_off, d1o);
     cur = nxt;
 #pragma unroll
     for (int k = 0; k < RD_NSRC; k++) srow[k] = nrow[k];
@@ -707,7 +725,6 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
   for (; row0 < row_end; row0 += (64 / RD_L) * RD_RB) {
     rd_unit x[RD_RB];
     ga_long d0o[RD_RB], d1o[RD_RB], sh[RD_RB];
-    const char *srow[RD_RB][RD_NSRC];
 #pragma unroll
     for (int b = 0; b < RD_RB; b++) {
       ga_long row = row0 + b * (64 / RD_L) + sub;
@@ -716,7 +733,7 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       rd_row_offsets(p, row, so, &d0o[b], &d1o[b]);
       const char *lp[RD_NSRC];
 #pragma unroll
-      for (int k = 0; k < RD_NSRC; k++) lp[k] = srow[b][k] = base[k] + so[k];
+      for (int k = 0; k < RD_NSRC; k++) lp[k] = base[k] + so[k];
       sh[b] = RD_SHIFT(lp[0]);
       lp[0] -= sh[b] * RD_ELSZ0;
       rd_unit_load<RD_L>(x[b], lp, e0, rin + sh[b], rstr);
@@ -728,12 +745,141 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       const ga_long row = row0 + b * (64 / RD_L) + sub;
       rd_acc acc = rd_seg_reduce<RD_L>(
           rd_unit_combine<RD_L>(x[b], e0, rin + sh[b], 0, rml, sh[b] RD_SCALAR_ARGS));
+#if RD_FIRST_RULE
+      /* Lane 0 of the row holds its first element (at position sh of its first
+       * load).  Where that is a NaN this lane writes the result itself, and
+       * the last lane, which holds the combination, stands back. */
+      RD_ACC_T first = (RD_ACC_T)RD_UNIT_VAL(x[b], 0, 0);
+#if RD_TAIL
+#pragma unroll
+      for (int v = 1; v < RD_VEC; v++)
+        if (sh[b] == v) first = (RD_ACC_T)RD_UNIT_VAL(x[b], 0, v);
+#endif
+      const bool first_nan = l == 0 && first != first;
+      const ga_ulong nan_rows = __builtin_amdgcn_ballot_w64(first_nan);
+      if (first_nan && row < row_end)
+        rd_write(rd_first_rule(acc, first), d0 + d0_off, d0o[b], d1 + d1_off, d1o[b]);
+      if (l == RD_L - 1 && row < row_end && !((nan_rows >> (lane - l)) & 1u))
+        rd_write(acc, d0 + d0_off, d0o[b], d1 + d1_off, d1o[b]);
+#else
       if (l == RD_L - 1 && row < row_end)
-        rd_store(acc, srow[b], d0 + d0_off, d0o[b], d1 + d1_off, d1o[b], p.rtotal RD_SCALAR_ARGS);
+        rd_write(acc, d0 + d0_off, d0o[b], d1 + d1_off, d1o[b]);
+#endif
     }
   }
 }
 #endif
+#endif
+
+#if RD_SROWS
+/* ---- redux_srows -----------------------------------------------------------
+ * Rows of a few dozen elements, one after the other in memory (one source,
+ * one reduced dim, unit stride, row pitch = row length).  redux_wrows spends
+ * its time on instructions per row there - address arithmetic, masks and
+ * cross-lane steps for a handful of elements.  Here a group copies the
+ * contiguous bytes of its p.upb <= 256 rows into LDS with 16-byte streaming
+ * loads (from the 16-byte boundary at or below the first row), and after one
+ * barrier lane t walks row t out of LDS: no cross-lane step, and per element
+ * one LDS read and the combine.  A lane starts t elements into its row when the
+ * row length is even, so that the lanes of a wavefront spread over the banks. */
+typedef ga_uint rd_chunk_t __attribute__((ext_vector_type(4)));
+
+KERNEL void __launch_bounds__(256)
+redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const rd_plan p RD_SCALAR_PARAMS) {
+  (void)part_v; (void)part_i;
+  extern __shared__ rd_chunk_t rd_staged[];
+  const ga_long per_group = p.upb;
+  const ga_long row0 = (ga_long)GID_0 * per_group;
+  ga_long nrow = p.nrows - row0;
+  if (nrow > per_group) nrow = per_group;
+  const ga_long rin = p.rdim[0], rml = p.rmul[0];
+
+  const char *base[RD_NSRC];
+  RD_SRC_BASES(base);
+  const char *begin = base[0] + row0 * p.fsstr[0][0];
+  const ga_size sh = (ga_size)begin & 15u;
+  const char *from = begin - sh;
+  const ga_long chunks = ((ga_long)sh + nrow * rin * RD_ELSZ0 + 15) >> 4;
+
+  for (ga_long c0 = LID_0; c0 < chunks; c0 += 256 * 8) {
+    rd_chunk_t t[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (c0 + j * 256 < chunks) t[j] = RD_LOAD((const rd_chunk_t *)(from + (c0 + j * 256) * 16));
+#pragma unroll
+    for (int j = 7; j >= 0; j--) rd_touch(t[j][0]);
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (c0 + j * 256 < chunks) rd_staged[c0 + j * 256] = t[j];
+  }
+  local_barrier();
+
+  if ((ga_long)LID_0 < nrow) {
+    typedef decltype(rd_one::x0) elem_t;
+    const elem_t *e = (const elem_t *)((const char *)rd_staged + sh) + (ga_long)LID_0 * rin;
+    const ga_int n = (ga_int)rin;
+    rd_acc acc = rd_neutral();
+#if RD_ARG && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN)
+    /* value and position inside the row (32 bits) while walking; the 64-bit
+     * index is formed once at the end */
+#if RD_KIND == RD_K_MAX
+#define RD_SR_BETTER(x, y) ((x) > (y))
+#else
+#define RD_SR_BETTER(x, y) ((x) < (y))
+#endif
+    RD_ACC_T bv;
+    ga_int bp;
+    if (n & 1) {
+      /* rising positions: a strict compare keeps the first of equals */
+      rd_one o;
+      o.x0 = e[0];
+      bv = rd_elem(RD_ONE_VAL(o), 0).v;
+      bp = 0;
+#pragma unroll 4
+      for (ga_int i = 1; i < n; i++) {
+        o.x0 = e[i];
+        const RD_ACC_T val = rd_elem(RD_ONE_VAL(o), 0).v;
+        const bool better = RD_SR_BETTER(val, bv);
+        bv = better ? val : bv;
+        bp = better ? i : bp;
+      }
+    } else {
+      ga_int pos = (ga_int)(LID_0 % (unsigned)n);
+      bv = RD_NEUTRAL;
+      bp = 0x7fffffff;
+#pragma unroll 4
+      for (ga_int i = 0; i < n; i++) {
+        rd_one o;
+        o.x0 = e[pos];
+        const RD_ACC_T val = rd_elem(RD_ONE_VAL(o), 0).v;
+        const bool better = RD_SR_BETTER(val, bv) || (val == bv && pos < bp);
+        bv = better ? val : bv;
+        bp = better ? pos : bp;
+        pos = (pos + 1 == n) ? 0 : pos + 1;
+      }
+    }
+#undef RD_SR_BETTER
+    acc.v = bv;
+    acc.i = (ga_long)bp * rml;
+#else
+    ga_int pos = (n & 1) ? 0 : (ga_int)(LID_0 % (unsigned)n);
+#pragma unroll 4
+    for (ga_int i = 0; i < n; i++) {
+      rd_one o;
+      o.x0 = e[pos];
+      acc = rd_combine(acc, rd_elem(RD_ONE_VAL(o), (ga_long)pos * rml));
+      pos = (pos + 1 == n) ? 0 : pos + 1;
+    }
+#endif
+    ga_long so[RD_NSRC], d0o, d1o;
+    rd_row_offsets(p, row0 + LID_0, so, &d0o, &d1o);
+    rd_one first;
+    first.x0 = e[0];
+    rd_write(rd_first_rule(acc, (RD_ACC_T)RD_ONE_VAL(first)), d0 + d0_off, d0o, d1 + d1_off, d1o);
+  }
+}
 #endif
 
 /* ---- redux_col -------------------------------------------------------------

@@ -502,6 +502,92 @@ def test_short_rows_share_a_wavefront(ctx, dtype):
     _check_ops(ctx, base[::-1, ::2], [1])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64", "int16"])
+def test_short_contiguous_rows_staged_in_lds(ctx, dtype, monkeypatch):
+    """Many short rows lying one after the other take the kernel that stages a
+    group's rows in LDS (here from 1000 rows on, so that the case stays
+    small): every row length up to the limit, starts off the 16-byte boundary,
+    a last group that is not full, ties, and NaN / signed zero placement."""
+    monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")
+    rng = np.random.default_rng(54)
+    item = np.dtype(dtype).itemsize
+    lengths = [n for n in (2, 3, 5, 6, 7, 8, 12, 16, 17, 31, 32, 33, 48, 63, 64, 100, 128, 255, 256)
+               if 16 < n * item <= 256]
+    for n in lengths:
+        rows = int(rng.integers(300, 1500))
+        flat = rng.integers(0, 12, size=rows * n + 7).astype(dtype)      # many ties
+        for off in (0, 1, 3):
+            host = flat[off:off + rows * n].reshape(rows, n)
+            if dtype == "float16":
+                g, _ = to_gpu_view(host, ctx)
+                val, idx = R.maxandargmax(g, axis=1)
+                assert np.array_equal(np.asarray(val), host.max(axis=1))
+                assert np.array_equal(np.asarray(idx), host.argmax(axis=1))
+                got = np.asarray(R.sum(g, axis=1, dtype="float32"))
+                assert np.array_equal(got, host.astype(np.float32).sum(axis=1))   # small integers: exact
+            else:
+                _check_ops(ctx, host, [1])
+    if dtype in ("float32", "float64"):
+        host = rng.standard_normal((2000, 33)).astype(dtype)
+        host[5, 0] = np.nan            # element 0: the result is NaN at index 0
+        host[6, 7] = np.nan            # elsewhere: ignored
+        host[7, :] = 0.0
+        host[7, 4] = -0.0              # equal to the zeros before it: index 0 stays
+        host[8, :] = -0.0
+        host[8, 9] = 0.0
+        g, _ = to_gpu_view(host, ctx)
+        val, idx = R.maxandargmax(g, axis=1)
+        val, idx = np.asarray(val), np.asarray(idx)
+        assert np.isnan(val[5]) and idx[5] == 0
+        assert val[6] == np.nanmax(host[6]) and idx[6] == np.nanargmax(host[6])
+        assert idx[7] == 0 and not np.signbit(val[7])
+        assert idx[8] == 0 and np.signbit(val[8])
+        keep = np.ones(2000, bool)
+        keep[[5, 6]] = False
+        assert np.array_equal(val[keep], host[keep].max(axis=1))
+        assert np.array_equal(idx[keep], host[keep].argmax(axis=1))
+    if dtype == "uint8":
+        host = (rng.random((5000, 40)) < 0.02).astype(dtype)
+        g, _ = to_gpu_view(host, ctx)
+        assert np.array_equal(np.asarray(R.any(g, axis=1)), host.any(axis=1))
+        assert np.array_equal(np.asarray(R.all(g, axis=1)), host.all(axis=1))
+        ones = np.ones((5000, 40), dtype)
+        ones[17, 39] = 0
+        g, _ = to_gpu_view(ones, ctx)
+        assert np.array_equal(np.asarray(R.all(g, axis=1)), ones.all(axis=1))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "float16"])
+@pytest.mark.parametrize("staged", [0, 1])
+def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, monkeypatch):
+    """The NaN rule of the sequential scan (a NaN stays only when it is the
+    first element) in the kernels that take it from their own registers: rows
+    sharing a wavefront in every lane geometry, rows shifted to a load
+    boundary, one row per wavefront, rows staged in LDS."""
+    monkeypatch.setenv("GPUARRAY_REDUX_SROWS", str(staged))
+    monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")
+    rng = np.random.default_rng(55)
+    for n in (2, 3, 4, 8, 15, 16, 33, 64, 100, 129, 250, 513, 1000, 1001):
+        rows = 131
+        host = rng.integers(-20, 20, size=(rows, n)).astype(dtype)
+        first = rng.choice(rows, 20, replace=False)
+        host[first[:10], 0] = np.nan                     # stays
+        host[first[10:], rng.integers(1, n, 10)] = np.nan   # ignored
+        host[first[3], :] = np.nan                       # all NaN
+        flat = np.concatenate([np.zeros(1, dtype), host.ravel()])
+        for view in (host, flat[1:].reshape(rows, n)):   # aligned, and one element off
+            g, _ = to_gpu_view(view, ctx)
+            for name, nanfn, argfn in (("maxandargmax", np.nanmax, np.nanargmax),
+                                       ("minandargmin", np.nanmin, np.nanargmin)):
+                val, idx = getattr(R, name)(g, axis=1)
+                val, idx = np.asarray(val), np.asarray(idx)
+                for r in range(rows):
+                    if np.isnan(view[r, 0]):
+                        assert np.isnan(val[r]) and idx[r] == 0, (name, n, r)
+                    else:
+                        assert val[r] == nanfn(view[r]) and idx[r] == argfn(view[r]), (name, n, r)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "int32", "float64"])
 def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
     rng = np.random.default_rng(51)
