@@ -144,12 +144,13 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 
 // ---- flat kernel --------------------------------------------------------------
 // elem(n, {data, byte offset | scalar}..., ga_vec)
-//   ga_vec != 0: every array base is aligned to a whole chunk of V elements
+//   ga_vec != 0: ga_vec - 1 elements into every array a whole chunk of V elements starts
 //   (16 bytes of the widest type).  Chunk c belongs to lane c % 256 of group
 //   (c / 256) % G; a lane issues the loads of its next U chunks (G*256 chunks
 //   apart, so every load instruction of a wavefront covers one contiguous
-//   kilobyte) before the first use.  The last n % V elements, and the whole
-//   range when ga_vec == 0, run one element per lane.
+//   kilobyte) before the first use.  The elements before the first chunk and
+//   after the last one, and the whole range when ga_vec == 0, run one element
+//   per lane.
 std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
   std::string s;
   const unsigned V = ge->vec, U = ge->unroll;
@@ -175,9 +176,13 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
               a.name.c_str(), ctype(a.typecode), a.name.c_str(), a.name.c_str());
   s += "const ga_size ga_gtid = (ga_size)GID_0 * LDIM_0 + LID_0;\n"
        "const ga_size ga_nthr = (ga_size)GDIM_0 * LDIM_0;\n"
-       "ga_size ga_done = 0;\n";
+       "ga_size ga_done = 0; (void)ga_done;\n";
   if (V > 1 || U > 1) {
-    appendf(s, "if (ga_vec) {\nconst ga_size ga_nchunks = n / %uu;\n", V);
+    // ga_vec - 1 leading elements come before the first whole chunk of every array
+    s += "if (ga_vec) {\nconst ga_size ga_head = ga_vec - 1u;\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) appendf(s, "%s_p += ga_head;\n", a.name.c_str());
+    appendf(s, "const ga_size ga_nchunks = (n - ga_head) / %uu;\n", V);
     if (ge->tile) {
       appendf(s, "const ga_size ga_ustep = 256;\n"
                  "for (ga_size ga_c0 = (ga_size)GID_0 * %uu + LID_0; ga_c0 - LID_0 < ga_nchunks; "
@@ -208,7 +213,7 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
     s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
     appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
-    appendf(s, "const ga_size i = ga_c * %uu + ga_v; (void)i;\n{\n", V);
+    appendf(s, "const ga_size i = ga_head + ga_c * %uu + ga_v; (void)i;\n{\n", V);
     for (const ge_arg &a : ge->args)
       if (a.is_array()) emit_load(ge, s, a, a.name + "_u[ga_u].e[ga_v]");
     s += ge->expr;
@@ -227,9 +232,22 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
                 a.name.c_str());
     }
     s += "}\n}\n";
-    appendf(s, "}\nga_done = ga_nchunks * %uu;\n}\n", V);
+    s += "}\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) appendf(s, "%s_p -= ga_head;\n", a.name.c_str());
+    appendf(s, "ga_done = ga_nchunks * %uu;\n", V);
+    // the elements before the first chunk and after the last one
+    s += "const ga_size ga_rest = n - ga_done;\nfor (ga_size ga_t = ga_gtid; ga_t < ga_rest; ga_t += ga_nthr) {\n"
+         "const ga_size i = ga_t < ga_head ? ga_t : ga_t + ga_done;\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_load(ge, s, a, a.name + "_p[i]");
+    s += ge->expr;
+    s += ";\n";
+    for (const ge_arg &a : ge->args)
+      if (a.is_array()) emit_store(ge, s, a, a.name + "_p[i]");
+    s += "}\nreturn;\n}\n";
   }
-  s += "for (ga_size i = ga_done + ga_gtid; i < n; i += ga_nthr) {\n";
+  s += "for (ga_size i = ga_gtid; i < n; i += ga_nthr) {\n";
   for (const ge_arg &a : ge->args)
     if (a.is_array()) emit_load(ge, s, a, a.name + "_p[i]");
   s += ge->expr;
@@ -850,22 +868,34 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   GpuKernel *k = &ge->k_flat;
   unsigned p = 0, l = 0;
   int err;
-  unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u;
+  unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u, head = ~0u;
   if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
   for (size_t i = 0; i < ge->args.size(); i++) {
     if (ge->args[i].is_array()) {
       GpuArray *a = (GpuArray *)args[i];
       size_t off = offs[l++];
-      size_t chunk = gpuarray_get_elsize(a->typecode) * ge->vec;
-      if (((uintptr_t)a->data->devptr + off) % chunk != 0) vec_ok = 0;
+      // Elements from this array's start to its next chunk boundary; the
+      // vector path needs the same count for every array (views cut the same
+      // way out of aligned arrays, x[1:] say, have it).
+      const size_t elsz = gpuarray_get_elsize(a->typecode), chunk = elsz * ge->vec;
+      const size_t mis = ((uintptr_t)a->data->devptr + off) % chunk;
+      if (mis % elsz != 0) {
+        vec_ok = 0;
+      } else {
+        const unsigned h = (unsigned)((chunk - mis) % chunk / elsz);
+        if (head == ~0u) head = h;
+        else if (head != h) vec_ok = 0;
+      }
       if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
       if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
     } else {
       if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
     }
   }
-  if (n < ge->vec) vec_ok = 0;
-  if ((err = GpuKernel_setarg(k, p++, &vec_ok)) != GA_NO_ERROR) return err;
+  if (head == ~0u) head = 0;
+  if (n < (size_t)head + ge->vec) vec_ok = 0;
+  unsigned int vec_arg = vec_ok ? 1u + head : 0u;
+  if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
 
   // Grid: one lane per chunk (or per element) up to a fixed number of groups
   // per compute unit; beyond that the lanes stride over the range.
@@ -875,7 +905,7 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   // only matters far beyond that size.
   const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 2048);
   size_t cap = (size_t)ga_hip_numprocs(ge->ctx) * (per_cu ? per_cu : 2048);
-  size_t units = vec_ok ? n / ge->vec : n;
+  size_t units = vec_ok ? (n - head) / ge->vec + 1 : n;
   size_t per_group = GE_LANES * (size_t)((vec_ok && ge->tile) ? ge->unroll : 1);
   size_t want = (units + per_group - 1) / per_group;
   size_t gs = want < 1 ? 1 : (want > cap ? cap : want);

@@ -184,6 +184,7 @@ struct variant_spec {
   unsigned L;         // redux_wrows: lanes per row
   unsigned CV;        // redux_col: adjacent outputs per lane
   unsigned LO;        // redux_row: outer reduced coordinates side by side
+  unsigned CY = 4;    // redux_col: lane rows of a group (4, 2 or 1), 256 / CY lanes along the free dim
 };
 
 const char *load_type_name(int tc) {
@@ -246,6 +247,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
+  DEF("#define RD_CY %u\n", vs.CY ? vs.CY : 4u);
 #undef DEF
 
 #define GEN(...) do { snprintf(line, sizeof(line), __VA_ARGS__); gen += line; } while (0)
@@ -367,8 +369,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
   char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
-           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO);
+  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
+           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY);
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -705,7 +707,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1, LO = 1;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1, LO = 1, CY = 4;
   bool wrows = false, tail = false, srows = false;
   size_t groups, lds_bytes = 0;
   if (use_row) {
@@ -935,6 +937,9 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     }
   } else {
     const int64_t fin = p.fdim[p.nf - 1];
+    CY = (unsigned)env_ul("GPUARRAY_REDUX_COL_ROWS", 4);
+    if (CY != 1 && CY != 2 && CY != 4) CY = 4;
+    const int64_t CX = 256 / CY;   // lanes along the free dim
     // Adjacent outputs per lane: as many as one 16-byte load of the widest
     // source holds, when the inner free dim is contiguous in every source and
     // every address a lane forms is a multiple of its load.
@@ -963,14 +968,14 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
       // few groups, take the widest one that still fills the chip unsplit.
       {
         const int64_t want = ncu * 4, outer_f = nrows / fin;
-        auto groups_at = [&](unsigned c) { return ((fin + 64 * c - 1) / (64 * c)) * outer_f; };
+        auto groups_at = [&](unsigned c) { return ((fin + CX * c - 1) / (CX * c)) * outer_f; };
         if (groups_at(cv) < want)
           for (unsigned c = cv / 2; c >= 1; c /= 2)
             if (groups_at(c) >= want) { cv = c; break; }
       }
       CV = cv;
     }
-    p.gx = (fin + 64 * CV - 1) / (64 * CV);
+    p.gx = (fin + CX * CV - 1) / (CX * CV);
     const int64_t outer = nrows / fin;
     const int64_t base_groups = p.gx * outer;
     int64_t nsplit = 1;
@@ -1003,6 +1008,7 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
   variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
                      use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
                      (use_row && !wrows) ? LO : 1};
+  if (!use_row) vs.CY = CY;
   if (srows)   // one kernel, independent of the lane geometry
     vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
   variant *var = nullptr;

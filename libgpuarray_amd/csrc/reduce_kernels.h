@@ -31,6 +31,8 @@
  *   RD_LO       redux_row: outer reduced coordinates handled side by side by
  *               the RD_G lanes when the inner reduced dim is short (1: none)
  *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
+ *   RD_CY       redux_col: lane rows of a group that share the reduced range
+ *               (4, 2 or 1); 256 / RD_CY lanes lie along the free dim
  *   RD_L        redux_wrows: lanes that share a row (power of two, <= 64);
  *               64 / RD_L rows sit side by side in a wavefront
  *   RD_RB       redux_wrows: sets of rows whose loads a wavefront issues together
@@ -882,6 +884,8 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 }
 #endif
 
+#define RD_CX (256 / RD_CY)   /* lanes along the free dim; RD_CY lane rows share the reduced range */
+
 /* ---- redux_col -------------------------------------------------------------
  * Lanes along the fastest free dim; a lane owns RD_CV adjacent outputs and
  * fetches them with one load (RD_CV > 1 needs that dim to be contiguous in
@@ -890,15 +894,15 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 KERNEL void __launch_bounds__(256)
 redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
           RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
-  __shared__ rd_acc lds[4][RD_CV][64];
-  const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
+  __shared__ rd_acc lds[RD_CY][RD_CV][RD_CX];
+  const unsigned tx = LID_0 % RD_CX, ty = LID_0 / RD_CX;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
   ga_long t = GID_0 / (unsigned)p.nsplit;
   const ga_long bx = t % p.gx;
   const ga_long fo = t / p.gx;   /* flat index over the outer free dims */
   const int fi_d = p.nf - 1;
   const ga_long fin = p.fdim[fi_d];
-  const ga_long fi = (bx * 64 + tx) * RD_CV;   /* first of the lane's outputs */
+  const ga_long fi = (bx * RD_CX + tx) * RD_CV;   /* first of the lane's outputs */
   const bool live = fi < fin;
 
   /* offsets of this lane's first output */
@@ -932,12 +936,12 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #pragma unroll
   for (int c = 0; c < RD_CV; c++) acc[c] = rd_neutral();
   if (live) {
-    for (ga_long j0 = r0 + ty; j0 < r1; j0 += 4 * RD_U) {
+    for (ga_long j0 = r0 + ty; j0 < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
       ga_long idx[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
-        const ga_long j = j0 + 4 * q;
+        const ga_long j = j0 + RD_CY * q;
         if (j < r1) {
           ga_long off[RD_NSRC], ix = 0, r = j;
 #pragma unroll
@@ -958,23 +962,26 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       }
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
-        if (j0 + 4 * q < r1) {
+        if (j0 + RD_CY * q < r1) {
 #pragma unroll
           for (int c = 0; c < RD_CV; c++)
             acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
         }
     }
   }
+#if RD_CY > 1
 #pragma unroll
   for (int c = 0; c < RD_CV; c++) lds[ty][c][tx] = acc[c];
   local_barrier();
+#else
+  (void)lds;
+#endif
   if (ty == 0 && live) {
 #pragma unroll
     for (int c = 0; c < RD_CV; c++) {
       rd_acc a = acc[c];
-      a = rd_combine(a, lds[1][c][tx]);
-      a = rd_combine(a, lds[2][c][tx]);
-      a = rd_combine(a, lds[3][c][tx]);
+#pragma unroll
+      for (int y = 1; y < RD_CY; y++) a = rd_combine(a, lds[y][c][tx]);
       const ga_long row = fo * fin + fi + c;
       if (p.nsplit == 1) {
         /* element 0 of the scan is at the start of the output's reduced range */

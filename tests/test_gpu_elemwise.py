@@ -17,6 +17,33 @@ pytestmark = pytest.mark.gpu
 lib = _lib.lib
 F16 = np.array([0x0000, 0x3c00, 0x4000, 0x4200, 0x4400, 0x4500, 0x4600, 0x4700, 0x4800, 0x4880],
                dtype=np.uint16).view(np.float16)
+@pytest.mark.parametrize("dts", [("uint8", "uint8", "uint8"), ("float16", "float16", "float16"),
+                                 ("float64", "float64", "float64"), ("float32", "float16", "float32"),
+                                 ("int16", "int64", "int32")])
+def test_views_cut_the_same_way_keep_vector_access(ctx, dts):
+    """Arrays that start the same number of elements off a chunk boundary
+    (x[k:] of aligned arrays) take vector access after a short head; other
+    combinations fall back to element access.  Either way every element is
+    computed once and nothing outside the views is written."""
+    rng = np.random.default_rng(77)
+    ta, tb, tc = dts
+    ge = ga.GpuElemwise(ctx, "c = a + b", [arg("a", ta, read=True), arg("b", tb, read=True),
+                                           arg("c", tc, write=True)], convert_f16=True)
+    pad = 40
+    for n in (1, 2, 5, 15, 16, 17, 31, 33, 1000, 4099, 100003):
+        a = rng.integers(0, 50, n + pad).astype(ta)
+        b = rng.integers(0, 50, n + pad).astype(tb)
+        for oa, ob, oc in ((1, 1, 1), (3, 3, 3), (15, 15, 15), (17, 17, 17), (1, 17, 33), (2, 1, 0),
+                           (0, 0, 5), (4, 4, 4), (8, 0, 0)):
+            ga_v, gb_v = to_gpu_view(a[oa:oa + n], ctx)[0], to_gpu_view(b[ob:ob + n], ctx)[0]
+            gc = gpuarray.zeros((n + pad,), tc, context=ctx)
+            ge(ga_v, gb_v, gc[oc:oc + n])
+            got = np.asarray(gc)
+            want = (a[oa:oa + n].astype(np.float64) + b[ob:ob + n].astype(np.float64)).astype(tc)
+            assert np.array_equal(got[oc:oc + n], want), (n, oa, ob, oc)
+            assert not got[:oc].any() and not got[oc + n:].any(), (n, oa, ob, oc)
+
+
 BCAST, NOCOLLAPSE, PAD = _lib.GE_BROADCAST, _lib.GE_NOCOLLAPSE, _lib.GE_PADSHAPE
 
 
