@@ -101,6 +101,7 @@ struct _GpuElemwise {
   unsigned int unroll = 1;  // chunks per lane and tile in the flat kernel
   bool tile = false;        // a group's chunks are adjacent (tile) or a grid apart
   bool nontemporal = true;  // streaming hint on the flat kernel's loads and stores
+  unsigned flat_nt_mask = ~0u;   // ... per array (bit k: array k)
   GpuKernel k_flat = {nullptr, nullptr};
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
@@ -144,7 +145,9 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 
 // ---- flat kernel --------------------------------------------------------------
 // elem(n, {data, byte offset | scalar}..., ga_vec)
-//   ga_vec != 0: ga_vec - 1 elements into every array a whole chunk of V elements starts
+//   ga_vec != 0: (ga_vec & 0xff) - 1 elements into every array a whole chunk of V
+//   elements starts, except the arrays k with bit 8 + k set, which are moved
+//   element by element
 //   (16 bytes of the widest type).  Chunk c belongs to lane c % 256 of group
 //   (c / 256) % G; a lane issues the loads of its next U chunks (G*256 chunks
 //   apart, so every load instruction of a wavefront covers one contiguous
@@ -179,7 +182,8 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
        "ga_size ga_done = 0; (void)ga_done;\n";
   if (V > 1 || U > 1) {
     // ga_vec - 1 leading elements come before the first whole chunk of every array
-    s += "if (ga_vec) {\nconst ga_size ga_head = ga_vec - 1u;\n";
+    // and bit 8 + k says that array k does not: it is then moved element by element
+    s += "if (ga_vec) {\nconst ga_size ga_head = (ga_vec & 0xffu) - 1u;\nconst ga_uint ga_mis = ga_vec >> 8;\n";
     for (const ge_arg &a : ge->args)
       if (a.is_array()) appendf(s, "%s_p += ga_head;\n", a.name.c_str());
     appendf(s, "const ga_size ga_nchunks = (n - ga_head) / %uu;\n", V);
@@ -199,15 +203,22 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
     }
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
     s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
+    unsigned ak = 0;
     for (const ge_arg &a : ge->args) {
-      if (!a.is_array() || !a.reads()) continue;
+      if (!a.is_array()) continue;
+      const unsigned bit = ak++;
+      if (!a.reads()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
-      if (ge->nontemporal)
+      appendf(s, "if (ga_mis & %uu) {\n#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) "
+                 "%s_u[ga_u].e[ga_v] = %s_p[ga_c * %uu + ga_v];\n} else {\n",
+              1u << bit, V, a.name.c_str(), a.name.c_str(), V);
+      if (ge->nontemporal && ((ge->flat_nt_mask >> bit) & 1u))
         appendf(s, "%s_u[ga_u].c = __builtin_nontemporal_load((const %s *)%s_p + ga_c);\n",
                 a.name.c_str(), chunk_type(cb), a.name.c_str());
       else
         appendf(s, "%s_u[ga_u].c = ((const %s *)%s_p)[ga_c];\n", a.name.c_str(), chunk_type(cb),
                 a.name.c_str());
+      s += "}\n";
     }
     s += "}\n}\n";
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
@@ -221,15 +232,22 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
     for (const ge_arg &a : ge->args)
       if (a.is_array()) emit_store(ge, s, a, a.name + "_u[ga_u].e[ga_v]");
     s += "}\n}\n";
+    ak = 0;
     for (const ge_arg &a : ge->args) {
-      if (!a.is_array() || !a.writes()) continue;
+      if (!a.is_array()) continue;
+      const unsigned bit = ak++;
+      if (!a.writes()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
-      if (ge->nontemporal)
+      appendf(s, "if (ga_mis & %uu) {\n#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) "
+                 "%s_p[ga_c * %uu + ga_v] = %s_u[ga_u].e[ga_v];\n} else {\n",
+              1u << bit, V, a.name.c_str(), V, a.name.c_str());
+      if (ge->nontemporal && ((ge->flat_nt_mask >> bit) & 1u))
         appendf(s, "__builtin_nontemporal_store(%s_u[ga_u].c, (%s *)%s_p + ga_c);\n",
                 a.name.c_str(), chunk_type(cb), a.name.c_str());
       else
         appendf(s, "((%s *)%s_p)[ga_c] = %s_u[ga_u].c;\n", chunk_type(cb), a.name.c_str(),
                 a.name.c_str());
+      s += "}\n";
     }
     s += "}\n}\n";
     s += "}\n";
@@ -869,32 +887,33 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   unsigned p = 0, l = 0;
   int err;
   unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u, head = ~0u;
+  std::vector<unsigned> heads;
   if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
   for (size_t i = 0; i < ge->args.size(); i++) {
     if (ge->args[i].is_array()) {
       GpuArray *a = (GpuArray *)args[i];
       size_t off = offs[l++];
-      // Elements from this array's start to its next chunk boundary; the
-      // vector path needs the same count for every array (views cut the same
-      // way out of aligned arrays, x[1:] say, have it).
+      // Elements from this array's start to its next chunk boundary.  The
+      // first written array (else the first array) sets the head of the
+      // vector path; an array with another count is moved element by element.
       const size_t elsz = gpuarray_get_elsize(a->typecode), chunk = elsz * ge->vec;
       const size_t mis = ((uintptr_t)a->data->devptr + off) % chunk;
-      if (mis % elsz != 0) {
-        vec_ok = 0;
-      } else {
-        const unsigned h = (unsigned)((chunk - mis) % chunk / elsz);
-        if (head == ~0u) head = h;
-        else if (head != h) vec_ok = 0;
-      }
+      if (mis % elsz != 0) vec_ok = 0;
+      heads.push_back((unsigned)((chunk - mis) % chunk / elsz));
+      if (head == ~0u && ge->args[i].writes()) head = heads.back();
       if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
       if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
     } else {
       if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
     }
   }
-  if (head == ~0u) head = 0;
-  if (n < (size_t)head + ge->vec) vec_ok = 0;
+  if (head == ~0u) head = heads.empty() ? 0 : heads[0];
+  if (n < (size_t)head + ge->vec || heads.size() > 24) vec_ok = 0;
   unsigned int vec_arg = vec_ok ? 1u + head : 0u;
+  for (size_t q = 0; vec_ok && q < heads.size(); q++)
+    if (heads[q] != head) vec_arg |= 1u << (8 + q);
+  if (!env_ul("GPUARRAY_ELEMWISE_MIXED_ALIGN", 1) && (vec_arg >> 8)) vec_arg = 0;
+  if (vec_arg == 0) vec_ok = 0;
   if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
 
   // Grid: one lane per chunk (or per element) up to a fixed number of groups
@@ -1232,6 +1251,7 @@ static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, 
   if (ge->unroll < 1) ge->unroll = 1;
   ge->tile = env_ul("GPUARRAY_ELEMWISE_TILE", 0) != 0;
   ge->nontemporal = env_ul("GPUARRAY_ELEMWISE_NT", 1) != 0;
+  ge->flat_nt_mask = (unsigned)env_ul("GPUARRAY_ELEMWISE_FLAT_NT_MASK", 0xffffffffu);
   return GA_NO_ERROR;
 }
 
