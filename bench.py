@@ -358,6 +358,41 @@ def per_config(ctx, ga, R):
     mm = ga.zeros((64, 1000), f32, context=ctx)
     mo, mi = ga.empty((64,), f32, context=ctx), ga.empty((64,), "int64", context=ctx)
     lat["maxandargmax_64x1000"] = {"device_us": round(time_calls(ctx, lambda i: op4(mm, [1], d0=mo, d1=mi), iters=100), 2)}
+    # the same small calls recorded once into a HIP graph on the library's stream and replayed
+    try:
+        import ctypes as C
+        from libgpuarray_amd import _lib
+        hip = C.CDLL("libamdhip64.so")
+        stream = C.c_void_p(_lib.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
+        sa, sb, sc = (ga.zeros((1 << 10,), f32, context=ctx) for _ in range(3))
+        per_graph = 100
+
+        def chain():
+            for _ in range(per_graph // 2):
+                elem(sa, sb, sc)
+                elem(sc, sb, sa)
+        chain()
+        ctx.sync()
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        if hip.hipStreamBeginCapture(stream, 0) == 0:
+            chain()
+            ok = hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+            ok = ok and hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+            if ok:
+                hip.hipGraphLaunch(gexec, stream)
+                ctx.sync()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    hip.hipGraphLaunch(gexec, stream)
+                ctx.sync()
+                lat["elemwise_n=1024_graph_replay"] = {
+                    "wall_us_per_call": round((time.perf_counter() - t0) / (20 * per_graph) * 1e6, 2),
+                    "calls_per_graph": per_graph}
+                hip.hipGraphExecDestroy(gexec)
+            if graph:
+                hip.hipGraphDestroy(graph)
+    except OSError:
+        pass
     res["latency"] = lat
     return res
 
