@@ -22,6 +22,7 @@
 #include "private.hpp"
 
 #include <algorithm>
+#include <array>
 #include <cctype>
 #include <map>
 #include <mutex>
@@ -156,7 +157,7 @@ struct _GpuReduction {
   bool mapped = false;        // an expression feeds the reduction
   int acc_tc = -1;            // mapped: accumulator (= value result) type
   std::string map_expr, preamble, reduce_expr, neutral;
-  std::map<std::string, variant> variants;
+  std::map<std::array<unsigned, 13>, variant> variants;   // by the fields of a variant_spec
   int src_tc() const { return args[arrays[0]].tc; }
   unsigned nsrc() const { return (unsigned)arrays.size(); }
 };
@@ -368,9 +369,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   gpucontext *ctx = gr->ctx;
-  char key[128];
-  snprintf(key, sizeof(key), "%d:%d:%u:%u:%u:%u:%u:%x:%u:%u:%u:%u:%u", vs.d0_tc, vs.d1_tc, vs.G, vs.V,
-           vs.U, vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY);
+  const std::array<unsigned, 13> key = {(unsigned)vs.d0_tc, (unsigned)vs.d1_tc, vs.G, vs.V, vs.U,
+                                        vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY};
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;

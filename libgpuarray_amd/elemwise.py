@@ -54,6 +54,16 @@ class GpuElemwise(object):
         flags = _lib.GE_CONVERT_F16 if convert_f16 else 0
         self.ge = lib.GpuElemwise_new(context.ctx, preamble.encode(), expr.encode(), n, arr, nd,
                                       flags)
+        # argument table of a call, reused: array slots take the address of the
+        # caller's GpuArray struct, scalar slots point at a value held here
+        self._ptrs = (C.c_void_p * max(n, 1))()
+        self._scalars = {}
+        for i, a in enumerate(self.args):
+            if a.scalar:
+                buf = np.zeros((), dtype=a.dtype)
+                self._scalars[i] = buf
+                self._ptrs[i] = buf.ctypes.data
+        self._slots = [(i, a.scalar, a.name) for i, a in enumerate(self.args)]
         if not self.ge:
             # the code is in the context's record; surface it like any other failure
             msg = context.error()
@@ -67,33 +77,31 @@ class GpuElemwise(object):
             self.ge = None
 
     def __call__(self, *values, **kwargs):
-        broadcast = kwargs.pop("broadcast", True)
-        padshape = kwargs.pop("padshape", True)
-        collapse = kwargs.pop("collapse", True)
+        flags = _lib.GE_BROADCAST | _lib.GE_PADSHAPE
         if kwargs:
-            raise TypeError("unexpected keyword arguments: %s" % (sorted(kwargs),))
-        if len(values) != len(self.args):
-            raise TypeError("expected %d arguments, got %d" % (len(self.args), len(values)))
-        keep = []
-        ptrs = (C.c_void_p * max(len(values), 1))()
-        for i, (a, v) in enumerate(zip(self.args, values)):
-            if a.scalar:
-                s = np.asarray(v, dtype=a.dtype).reshape(())
-                buf = np.ascontiguousarray(s)
-                keep.append(buf)
-                ptrs[i] = buf.ctypes.data
+            if not kwargs.pop("broadcast", True):
+                flags &= ~_lib.GE_BROADCAST
+            if not kwargs.pop("padshape", True):
+                flags &= ~_lib.GE_PADSHAPE
+            if not kwargs.pop("collapse", True):
+                flags |= _lib.GE_NOCOLLAPSE
+            if kwargs:
+                raise TypeError("unexpected keyword arguments: %s" % (sorted(kwargs),))
+        if len(values) != len(self._slots):
+            raise TypeError("expected %d arguments, got %d" % (len(self._slots), len(values)))
+        ptrs = self._ptrs
+        for i, scalar, name in self._slots:
+            v = values[i]
+            if scalar:
+                self._scalars[i][...] = v
             else:
-                if not isinstance(v, GpuArray):
-                    raise TypeError("argument %d (%s) must be a GpuArray" % (i, a.name))
-                ptrs[i] = C.addressof(v.ga)
-        flags = 0
-        if broadcast:
-            flags |= _lib.GE_BROADCAST
-        if padshape:
-            flags |= _lib.GE_PADSHAPE
-        if not collapse:
-            flags |= _lib.GE_NOCOLLAPSE
-        check(lib.GpuElemwise_call(self.ge, ptrs, flags), self.context.ctx)
+                try:
+                    ptrs[i] = v._addr
+                except AttributeError:
+                    raise TypeError("argument %d (%s) must be a GpuArray" % (i, name))
+        err = lib.GpuElemwise_call(self.ge, ptrs, flags)
+        if err:
+            check(err, self.context.ctx)
 
 
 def _dtype(o):

@@ -194,6 +194,8 @@ class GpuArray(object):
     def __init__(self, context):
         self.context = context
         self.ga = GpuArrayStruct()
+        self._addr = C.addressof(self.ga)   # of the C struct; fixed for the object's life
+        self._ref = C.byref(self.ga)
         self.base = None
 
     def __del__(self):
@@ -309,7 +311,7 @@ class GpuArray(object):
                      cls=type(self))
 
     def _ptr(self):
-        return C.byref(self.ga)
+        return self._ref
 
     def _check(self, err):
         check(err, self.context.ctx)

@@ -41,6 +41,7 @@ class GpuReduction(object):
         self.op = op
         self.dtype = np.dtype(dtype)
         self.gr = C.c_void_p()
+        self._axes = {}
         check(lib.GpuReduction_new(C.byref(self.gr), context.ctx, _OPS[op], ndf, ndr,
                                    dtype_to_typecode(dtype), 0), context.ctx)
 
@@ -51,11 +52,15 @@ class GpuReduction(object):
             self.gr = None
 
     def __call__(self, src, axes, d0=None, d1=None):
-        axes = list(axes)
-        arr = (C.c_int * _b.max(len(axes), 1))(*axes)
-        check(lib.GpuReduction_call(self.gr, d0._ptr() if d0 is not None else None,
-                                    d1._ptr() if d1 is not None else None, src._ptr(),
-                                    len(axes), arr, 0), self.context.ctx)
+        key = tuple(axes)
+        arr = self._axes.get(key)
+        if arr is None:            # the C array of an axis list, built once
+            arr = self._axes[key] = (C.c_int * _b.max(len(key), 1))(*key)
+        err = lib.GpuReduction_call(self.gr, d0._ref if d0 is not None else None,
+                                    d1._ref if d1 is not None else None, src._ref,
+                                    len(key), arr, 0)
+        if err:
+            check(err, self.context.ctx)
 
 
 from .tools import Argument, ArrayArg, ScalarArg, as_argument  # noqa: E402,F401
