@@ -539,178 +539,243 @@ struct src_view {
   std::vector<int64_t> strides;
 };
 
-int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
-                  const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
-                  unsigned reduxLen, const int *reduxList) {
-  gpucontext *ctx = gr->ctx;
-  const op_info &info = gr->info;
-  const unsigned K = gr->nsrc();
-  if ((info.has_d0 && d0 == nullptr) || (info.has_d1 && d1 == nullptr))
-    return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array required by the operation is NULL");
-  if (!info.has_d0) d0 = nullptr;
-  if (!info.has_d1) d1 = nullptr;
-  if (nd == 0 || reduxLen == 0 || reduxLen > nd || reduxList == nullptr)
-    return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
-                      "Invalid reduction: source nd = %u, %u axes to reduce", nd, reduxLen);
-  std::vector<char> reduced(nd, 0);
-  for (unsigned i = 0; i < reduxLen; i++) {
-    const int ax = reduxList[i];
-    if (ax < 0 || ax >= (int)nd || reduced[ax])
-      return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Reduction axis %d is out of range or repeated", ax);
-    reduced[ax] = 1;
-  }
-  for (const GpuArray *d : {(const GpuArray *)d0, (const GpuArray *)d1})
-    if (d != nullptr && d->data == nullptr)
-      return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array has no buffer");
-  for (unsigned k = 0; k < K; k++) {
-    const GpuArray *s = srcs[k].a;
-    if (s->data == nullptr)
-      return ga_err_set(ctx->err, GA_INVALID_ERROR, "A source array has no buffer");
-    const int want = gr->args[gr->arrays[k]].tc;
-    if (s->typecode != want)
-      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Source has typecode %d, operator was made for %d",
-                        s->typecode, want);
-    if (GpuArray_context(s) != ctx)
-      return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
-  }
-  if ((d0 && GpuArray_context(d0) != ctx) || (d1 && GpuArray_context(d1) != ctx))
-    return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
+// One call of an operator: argument checks, the dim lists and the plan the
+// kernels read, the choice of kernel family and lane geometry, the launch.
+class reduction_call {
+ public:
+  reduction_call(GpuReduction *gr_, GpuArray *d0_, GpuArray *d1_, unsigned nd_, const size_t *dims_,
+                 const std::vector<src_view> &srcs_, const std::vector<void *> &scalars_,
+                 unsigned reduxLen_, const int *reduxList_)
+      : gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
+        dims(dims_), srcs(srcs_), scalars(scalars_), reduxLen(reduxLen_), reduxList(reduxList_),
+        kind(info.kind), minmax(kind == K_MIN || kind == K_MAX),
+        logical(kind == K_ALL || kind == K_ANY),
+        planbuf(plan_bytes(K) / sizeof(int64_t), 0),
+        p(*reinterpret_cast<rd_plan *>(planbuf.data())),
+        fsstr(planbuf.data() + sizeof(rd_plan) / sizeof(int64_t)),
+        rsstr(fsstr + (size_t)K * RD_MAXD),
+        vecmask((1u << K) - 1) {}
 
-  // result types
-  const rd_kind kind = info.kind;
-  const bool minmax = kind == K_MIN || kind == K_MAX;
-  const bool logical = kind == K_ALL || kind == K_ANY;
-  int d0_tc = d0 ? d0->typecode : (gr->mapped ? gr->acc_tc : gr->src_tc());
-  const int d1_tc = d1 ? d1->typecode : GA_LONG;
-  if (d0) {
-    if (!GpuArray_ISWRITEABLE(d0)) return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination not writeable");
-    if (gr->mapped && !logical && d0_tc != gr->acc_tc)
-      return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
-                        "Result has typecode %d, the operator accumulates in %d", d0_tc, gr->acc_tc);
-    if (!gr->mapped && minmax && d0_tc != gr->src_tc())
-      return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max results must have the source's type");
-    if ((kind == K_AND || kind == K_OR || kind == K_XOR || logical) && !is_int_type(d0_tc))
-      return ga_err_set(ctx->err, GA_VALUE_ERROR, "Result of a logical/bitwise reduction must be an integer type");
-    if (!is_int_type(d0_tc) && !is_float_type(d0_tc))
-      return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Result typecode %d is not supported", d0_tc);
-  }
-  if (d1) {
-    if (!GpuArray_ISWRITEABLE(d1)) return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination not writeable");
-    if (d1_tc != GA_LONG && d1_tc != GA_ULONG)
-      return ga_err_set(ctx->err, GA_VALUE_ERROR, "Index results must be GA_LONG or GA_ULONG");
-  }
-
-  // free axes in ascending order must match the destinations' shapes
-  const unsigned nfree = nd - reduxLen;
-  for (GpuArray *d : {d0, d1}) {
-    if (d == nullptr) continue;
-    if (d->nd != nfree)
-      return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Destination has nd = %u, expected %u", d->nd, nfree);
-    unsigned k = 0;
-    for (unsigned ax = 0; ax < nd; ax++) {
-      if (reduced[ax]) continue;
-      if (d->dimensions[k] != dims[ax])
-        return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
-                          "Destination dimension %u is %zu, source axis %u is %zu", k,
-                          d->dimensions[k], ax, dims[ax]);
-      k++;
+  int run() {
+    int err;
+    if ((err = check_arguments()) != GA_NO_ERROR) return err;
+    if ((err = build_dims()) != GA_NO_ERROR || nrows == 0) return err;
+    fill_plan();
+    choose_family();
+    if (use_row) {
+      choose_row_loads();
+      row_geometry();
+      wrows_geometry();
+      srows_geometry();
+    } else {
+      col_geometry();
     }
+    if ((err = pick_variant()) != GA_NO_ERROR) return err;
+    return launch();
   }
 
-  // dim lists
-  std::vector<dimrec> fr, rd;
-  int64_t nrows = 1, rtotal = 1;
-  {
-    unsigned k = 0;
-    for (unsigned ax = 0; ax < nd; ax++) {
-      if (reduced[ax]) continue;
-      const int64_t dim = (int64_t)dims[ax];
-      nrows *= dim;
-      if (dim != 1) {
-        dimrec r;
-        memset(&r, 0, sizeof(r));
-        r.dim = dim;
-        for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
-        r.a = d0 ? (int64_t)d0->strides[k] : 0;
-        r.b = d1 ? (int64_t)d1->strides[k] : 0;
-        fr.push_back(r);
-      }
-      k++;
-    }
-    int64_t mul = 1;
-    for (unsigned i = reduxLen; i-- > 0;) {
-      const int ax = reduxList[i];
-      const int64_t dim = (int64_t)dims[ax];
-      rtotal *= dim;
-      if (dim != 1) {
-        dimrec r;
-        memset(&r, 0, sizeof(r));
-        r.dim = dim;
-        for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
-        r.a = mul;
-        rd.insert(rd.begin(), r);
-      }
-      mul *= dim;
-    }
-  }
-  if (nrows == 0) return GA_NO_ERROR;
-  if (rtotal == 0 && minmax)
-    return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max over an empty axis has no value");
-  if (rtotal == 0) rd.clear();
-  sort_and_fuse(fr, K, true);
-  sort_and_fuse(rd, K, false);
-  if (fr.size() > (size_t)RD_MAXD || rd.size() > (size_t)RD_MAXD)
-    return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR,
-                      "More than %d non-mergeable free or reduced dimensions", RD_MAXD);
-
+ private:
+  GpuReduction *gr;
+  gpucontext *ctx;
+  const op_info &info;
+  const unsigned K;                 // number of array sources
+  GpuArray *d0, *d1;
+  const unsigned nd;
+  const size_t *dims;
+  const std::vector<src_view> &srcs;
+  const std::vector<void *> &scalars;
+  const unsigned reduxLen;
+  const int *reduxList;
+  const rd_kind kind;
+  const bool minmax, logical;
+  int d0_tc = -1, d1_tc = GA_LONG;
+  std::vector<char> reduced;        // per source axis
+  std::vector<dimrec> fr, rd;       // free and reduced dims, slowest first, fused
+  int64_t nrows = 1, rtotal = 1;    // outputs, elements per output
   // plan = fixed part + per-source stride tables
-  std::vector<int64_t> planbuf(plan_bytes(K) / sizeof(int64_t), 0);
-  rd_plan &p = *reinterpret_cast<rd_plan *>(planbuf.data());
-  int64_t *fsstr = planbuf.data() + sizeof(rd_plan) / sizeof(int64_t);   // [K][RD_MAXD]
-  int64_t *rsstr = fsstr + (size_t)K * RD_MAXD;                           // [K][RD_MAXD]
-  p.nf = (int)fr.size();
-  p.nr = (int)rd.size();
-  for (int i = 0; i < p.nf; i++) {
-    p.fdim[i] = fr[i].dim; p.fd0str[i] = fr[i].a; p.fd1str[i] = fr[i].b;
-    for (unsigned q = 0; q < K; q++) fsstr[q * RD_MAXD + i] = fr[i].s[q];
-  }
-  for (int i = 0; i < p.nr; i++) {
-    p.rdim[i] = rd[i].dim; p.rmul[i] = rd[i].a;
-    for (unsigned q = 0; q < K; q++) rsstr[q * RD_MAXD + i] = rd[i].s[q];
-  }
-  p.nrows = nrows;
-  p.rtotal = rtotal;
-  p.nsplit = 1;
+  std::vector<int64_t> planbuf;
+  rd_plan &p;
+  int64_t *fsstr, *rsstr;           // [K][RD_MAXD] each
+  std::vector<int64_t> elsz;
+  int64_t elsz_max = 0, elsz_sum = 0, ncu = 1;
+  int64_t rin = 1, rstr = 0, fstr = 0;   // inner reduced extent and stride, inner free stride
+  int64_t rin_sz = 1;               // rin plus what a shifted row can gain
+  // kernel family and lane geometry
+  bool use_row = true, wrows = false, tail = false, srows = false;
+  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask, RB = 1, L = 64, CV = 1, LO = 1, CY = 4;
+  size_t groups = 0, lds_bytes = 0;
+  variant *var = nullptr;
 
-  int64_t elsz_max = 0, elsz_sum = 0;
-  std::vector<int64_t> elsz(K);
-  for (unsigned q = 0; q < K; q++) {
-    elsz[q] = (int64_t)gpuarray_get_elsize(gr->args[gr->arrays[q]].tc);
-    elsz_max = std::max(elsz_max, elsz[q]);
-    elsz_sum += elsz[q];
-  }
-  const int64_t ncu = (int64_t)ga_hip_numprocs(ctx);
-  const int64_t rin = p.nr ? p.rdim[p.nr - 1] : 1;
-  const int64_t rstr = p.nr ? rd[p.nr - 1].smax : 0;
-  const int64_t fstr = p.nf ? fr[p.nf - 1].smax : INT64_MAX;
+  int check_arguments() {
+    if ((info.has_d0 && d0 == nullptr) || (info.has_d1 && d1 == nullptr))
+      return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array required by the operation is NULL");
+    if (!info.has_d0) d0 = nullptr;
+    if (!info.has_d1) d1 = nullptr;
+    if (nd == 0 || reduxLen == 0 || reduxLen > nd || reduxList == nullptr)
+      return ga_err_fmt(ctx->err, GA_INVALID_ERROR,
+                        "Invalid reduction: source nd = %u, %u axes to reduce", nd, reduxLen);
+    reduced.assign(nd, 0);
+    for (unsigned i = 0; i < reduxLen; i++) {
+      const int ax = reduxList[i];
+      if (ax < 0 || ax >= (int)nd || reduced[ax])
+        return ga_err_fmt(ctx->err, GA_INVALID_ERROR, "Reduction axis %d is out of range or repeated", ax);
+      reduced[ax] = 1;
+    }
+    for (const GpuArray *d : {(const GpuArray *)d0, (const GpuArray *)d1})
+      if (d != nullptr && d->data == nullptr)
+        return ga_err_set(ctx->err, GA_INVALID_ERROR, "A destination array has no buffer");
+    for (unsigned k = 0; k < K; k++) {
+      const GpuArray *s = srcs[k].a;
+      if (s->data == nullptr)
+        return ga_err_set(ctx->err, GA_INVALID_ERROR, "A source array has no buffer");
+      const int want = gr->args[gr->arrays[k]].tc;
+      if (s->typecode != want)
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Source has typecode %d, operator was made for %d",
+                          s->typecode, want);
+      if (GpuArray_context(s) != ctx)
+        return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
+    }
+    if ((d0 && GpuArray_context(d0) != ctx) || (d1 && GpuArray_context(d1) != ctx))
+      return ga_err_set(ctx->err, GA_VALUE_ERROR, "Arrays belong to another context");
 
-  // Lanes along the reduced run unless the free run is the one that is
-  // contiguous in memory (or the reduced run is too short to feed a wavefront).
-  // Short reduced runs are fine when they are the only reduced dim: several
-  // rows then share a wavefront (redux_wrows).
-  bool use_row = p.nf == 0 || (rstr <= fstr && (rin >= 32 || p.nr <= 1)) ||
-                 (rin >= 4096 && rstr <= 4 * elsz_max);
-  if (rtotal == 0) use_row = true;
-  {
-    const char *force = getenv("GPUARRAY_REDUX_FAMILY");
-    if (force && strcmp(force, "row") == 0) use_row = true;
-    if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
+    // result types
+    d0_tc = d0 ? d0->typecode : (gr->mapped ? gr->acc_tc : gr->src_tc());
+    d1_tc = d1 ? d1->typecode : GA_LONG;
+    if (d0) {
+      if (!GpuArray_ISWRITEABLE(d0)) return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination not writeable");
+      if (gr->mapped && !logical && d0_tc != gr->acc_tc)
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                          "Result has typecode %d, the operator accumulates in %d", d0_tc, gr->acc_tc);
+      if (!gr->mapped && minmax && d0_tc != gr->src_tc())
+        return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max results must have the source's type");
+      if ((kind == K_AND || kind == K_OR || kind == K_XOR || logical) && !is_int_type(d0_tc))
+        return ga_err_set(ctx->err, GA_VALUE_ERROR,
+                          "Result of a logical/bitwise reduction must be an integer type");
+      if (!is_int_type(d0_tc) && !is_float_type(d0_tc))
+        return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Result typecode %d is not supported", d0_tc);
+    }
+    if (d1) {
+      if (!GpuArray_ISWRITEABLE(d1)) return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination not writeable");
+      if (d1_tc != GA_LONG && d1_tc != GA_ULONG)
+        return ga_err_set(ctx->err, GA_VALUE_ERROR, "Index results must be GA_LONG or GA_ULONG");
+    }
+
+    // free axes in ascending order must match the destinations' shapes
+    const unsigned nfree = nd - reduxLen;
+    for (GpuArray *d : {d0, d1}) {
+      if (d == nullptr) continue;
+      if (d->nd != nfree)
+        return ga_err_fmt(ctx->err, GA_VALUE_ERROR, "Destination has nd = %u, expected %u", d->nd, nfree);
+      unsigned k = 0;
+      for (unsigned ax = 0; ax < nd; ax++) {
+        if (reduced[ax]) continue;
+        if (d->dimensions[k] != dims[ax])
+          return ga_err_fmt(ctx->err, GA_VALUE_ERROR,
+                            "Destination dimension %u is %zu, source axis %u is %zu", k,
+                            d->dimensions[k], ax, dims[ax]);
+        k++;
+      }
+    }
+    return GA_NO_ERROR;
   }
 
-  unsigned G = 256, V = 1, U = 4, ES = 1, vecmask = (1u << K) - 1, RB = 1, L = 64, CV = 1, LO = 1, CY = 4;
-  bool wrows = false, tail = false, srows = false;
-  size_t groups, lds_bytes = 0;
-  if (use_row) {
+  // Free and reduced dim lists (extent-1 dims dropped, sorted, fused).
+  int build_dims() {
+    // dim lists
+    nrows = 1;
+    rtotal = 1;
+    {
+      unsigned k = 0;
+      for (unsigned ax = 0; ax < nd; ax++) {
+        if (reduced[ax]) continue;
+        const int64_t dim = (int64_t)dims[ax];
+        nrows *= dim;
+        if (dim != 1) {
+          dimrec r;
+          memset(&r, 0, sizeof(r));
+          r.dim = dim;
+          for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
+          r.a = d0 ? (int64_t)d0->strides[k] : 0;
+          r.b = d1 ? (int64_t)d1->strides[k] : 0;
+          fr.push_back(r);
+        }
+        k++;
+      }
+      int64_t mul = 1;
+      for (unsigned i = reduxLen; i-- > 0;) {
+        const int ax = reduxList[i];
+        const int64_t dim = (int64_t)dims[ax];
+        rtotal *= dim;
+        if (dim != 1) {
+          dimrec r;
+          memset(&r, 0, sizeof(r));
+          r.dim = dim;
+          for (unsigned q = 0; q < K; q++) r.s[q] = srcs[q].strides[ax];
+          r.a = mul;
+          rd.insert(rd.begin(), r);
+        }
+        mul *= dim;
+      }
+    }
+    if (nrows == 0) return GA_NO_ERROR;   // (run() sees nrows == 0 and stops)
+    if (rtotal == 0 && minmax)
+      return ga_err_set(ctx->err, GA_VALUE_ERROR, "min/max over an empty axis has no value");
+    if (rtotal == 0) rd.clear();
+    sort_and_fuse(fr, K, true);
+    sort_and_fuse(rd, K, false);
+    if (fr.size() > (size_t)RD_MAXD || rd.size() > (size_t)RD_MAXD)
+      return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR,
+                        "More than %d non-mergeable free or reduced dimensions", RD_MAXD);
+    return GA_NO_ERROR;
+  }
+
+  void fill_plan() {
+    // plan = fixed part + per-source stride tables
+    p.nf = (int)fr.size();
+    p.nr = (int)rd.size();
+    for (int i = 0; i < p.nf; i++) {
+      p.fdim[i] = fr[i].dim; p.fd0str[i] = fr[i].a; p.fd1str[i] = fr[i].b;
+      for (unsigned q = 0; q < K; q++) fsstr[q * RD_MAXD + i] = fr[i].s[q];
+    }
+    for (int i = 0; i < p.nr; i++) {
+      p.rdim[i] = rd[i].dim; p.rmul[i] = rd[i].a;
+      for (unsigned q = 0; q < K; q++) rsstr[q * RD_MAXD + i] = rd[i].s[q];
+    }
+    p.nrows = nrows;
+    p.rtotal = rtotal;
+    p.nsplit = 1;
+
+    elsz_max = elsz_sum = 0;
+    elsz.assign(K, 0);
+    for (unsigned q = 0; q < K; q++) {
+      elsz[q] = (int64_t)gpuarray_get_elsize(gr->args[gr->arrays[q]].tc);
+      elsz_max = std::max(elsz_max, elsz[q]);
+      elsz_sum += elsz[q];
+    }
+    ncu = (int64_t)ga_hip_numprocs(ctx);
+    rin = p.nr ? p.rdim[p.nr - 1] : 1;
+    rstr = p.nr ? rd[p.nr - 1].smax : 0;
+    fstr = p.nf ? fr[p.nf - 1].smax : INT64_MAX;
+  }
+
+  void choose_family() {
+    // Lanes along the reduced run unless the free run is the one that is
+    // contiguous in memory (or the reduced run is too short to feed a wavefront).
+    // Short reduced runs are fine when they are the only reduced dim: several
+    // rows then share a wavefront (redux_wrows).
+    use_row = p.nf == 0 || (rstr <= fstr && (rin >= 32 || p.nr <= 1)) ||
+                   (rin >= 4096 && rstr <= 4 * elsz_max);
+    if (rtotal == 0) use_row = true;
+    {
+      const char *force = getenv("GPUARRAY_REDUX_FAMILY");
+      if (force && strcmp(force, "row") == 0) use_row = true;
+      if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
+    }
+  }
+
+  // redux_row / redux_wrows: elements per load, element step, which sources
+  // take vector loads, shifted rows.
+  void choose_row_loads() {
     // Widest aligned load the layout allows, for a source whose inner reduced
     // stride is its element size: v elements, v*elsz bytes, everything the
     // lane's address is built from a multiple of that.
@@ -779,12 +844,17 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
         if (V > 1) vecmask = unit_mask;
       }
     }
+  }
+
+  // redux_row: lanes per output, loads in flight, outer coordinates side by
+  // side, units and splits.
+  void row_geometry() {
     // One wavefront per output when eight loads per lane cover the inner
     // reduced dim, four wavefronts otherwise.  Measured on MI355X: rows of
     // 8192 floats run at 6.7 TB/s with 256 lanes per row and 6.0 with 64;
     // rows of 512 stepped halves at 3.1 TB/s (useful) with 64 and 2.0 with 256.
     // a shifted row can be up to V-1 elements longer than its extent
-    const int64_t rin_sz = rin + (tail ? (int64_t)V - 1 : 0);
+    rin_sz = rin + (tail ? (int64_t)V - 1 : 0);
     G = (rin_sz <= (int64_t)64 * V * 8) ? 64 : 256;
     {
       const unsigned long force = env_ul("GPUARRAY_REDUX_G", 0);
@@ -854,11 +924,14 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     if (p.upb > 0) nsplit = (p.units + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;
     groups = (size_t)(rowgroups * nsplit);
+  }
+
+  void wrows_geometry() {
     // Short rows, one wavefront each, take the kernel without the unit loop.
     // A wavefront takes RB rows at a time and issues their loads together:
     // a row that is a single load per lane would otherwise leave the
     // wavefront with one load in flight.
-    if (G == 64 && nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
+    if (G == 64 && p.nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
       wrows = true;
       // Measured on MI355X: any() over 131072 rows of 512 stepped bytes 29.8 us
       // one row at a time, 24.8 us with batches of 4 and 8 rows per wavefront;
@@ -905,6 +978,9 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
       const int64_t waves = (nrows + rpw - 1) / rpw;
       groups = (size_t)((waves + 3) / 4);
     }
+  }
+
+  void srows_geometry() {
     // Rows of a few dozen elements that follow one another in memory: a group
     // stages the bytes of up to 256 rows in LDS and every lane walks one row
     // (redux_srows).  Measured on MI355X, 2^26 floats in rows of 8 / 17 / 33 /
@@ -935,7 +1011,9 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
         }
       }
     }
-  } else {
+  }
+
+  void col_geometry() {
     const int64_t fin = p.fdim[p.nf - 1];
     CY = (unsigned)env_ul("GPUARRAY_REDUX_COL_ROWS", 4);
     if (CY != 1 && CY != 2 && CY != 4) CY = 4;
@@ -998,67 +1076,77 @@ int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, con
     U = (unsigned)env_ul("GPUARRAY_REDUX_COL_U", 4);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 4;
   }
-  if (groups == 0 || groups > 0x7fffffffull)
-    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Reduction needs more groups than one launch has");
 
-  // bit 0: streaming loads; bit 1: interleaved splits (single reduced dim only)
-  unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
-  if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
-  if (use_row && tail) opts |= 4u;   // bit 2: element-aligned vector loads with a ragged end
-  variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
-                     use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
-                     (use_row && !wrows) ? LO : 1};
-  if (!use_row) vs.CY = CY;
-  if (srows)   // one kernel, independent of the lane geometry
-    vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
-  variant *var = nullptr;
-  int err = get_variant(gr, vs, &var);
-  if (err != GA_NO_ERROR) return err;
+  int pick_variant() {
+    if (groups == 0 || groups > 0x7fffffffull)
+      return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Reduction needs more groups than one launch has");
 
-  // partials of a split reduction live in the context's scratch buffer:
-  // values first, indices after, both 8-byte aligned
-  const int acc_tc = acc_typecode(gr, d0_tc);
-  const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
-  gpudata *scratch = ga_hip_scratch(ctx, 16);
-  size_t pi_off = 0;
-  if (p.nsplit > 1) {
-    const size_t slots = (size_t)nrows * (size_t)p.nsplit;
-    pi_off = (slots * accsz + 255) & ~(size_t)255;
-    scratch = ga_hip_scratch(ctx, pi_off + slots * 8);
+    // bit 0: streaming loads; bit 1: interleaved splits (single reduced dim only)
+    unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
+    if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
+    if (use_row && tail) opts |= 4u;   // bit 2: element-aligned vector loads with a ragged end
+    variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
+                       use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
+                       (use_row && !wrows) ? LO : 1};
+    if (!use_row) vs.CY = CY;
+    if (srows)   // one kernel, independent of the lane geometry
+      vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
+    return get_variant(gr, vs, &var);
   }
-  if (scratch == nullptr) return ctx->err->code;
 
-  // A destination the operation does not write still needs a valid pointer.
-  gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
-  size_t d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
-  std::vector<size_t> s_off(K);
+  int launch() {
+    // partials of a split reduction live in the context's scratch buffer:
+    // values first, indices after, both 8-byte aligned
+    const int acc_tc = acc_typecode(gr, d0_tc);
+    const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
+    gpudata *scratch = ga_hip_scratch(ctx, 16);
+    size_t pi_off = 0;
+    if (p.nsplit > 1) {
+      const size_t slots = (size_t)nrows * (size_t)p.nsplit;
+      pi_off = (slots * accsz + 255) & ~(size_t)255;
+      scratch = ga_hip_scratch(ctx, pi_off + slots * 8);
+    }
+    if (scratch == nullptr) return ctx->err->code;
 
-  // The two scratch views are passed as (buffer) arguments; the index part
-  // starts pi_off bytes in, which the kernels receive through a second
-  // gpudata wrapping the same memory.
-  struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + pi_off, ctx};
-  std::vector<void *> args;
-  for (unsigned q = 0; q < K; q++) {
-    s_off[q] = srcs[q].a->offset;
-    args.push_back(srcs[q].a->data);
-    args.push_back(&s_off[q]);
+    // A destination the operation does not write still needs a valid pointer.
+    gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
+    size_t d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
+    std::vector<size_t> s_off(K);
+
+    // The two scratch views are passed as (buffer) arguments; the index part
+    // starts pi_off bytes in, which the kernels receive through a second
+    // gpudata wrapping the same memory.
+    struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + pi_off, ctx};
+    std::vector<void *> args;
+    for (unsigned q = 0; q < K; q++) {
+      s_off[q] = srcs[q].a->offset;
+      args.push_back(srcs[q].a->data);
+      args.push_back(&s_off[q]);
+    }
+    args.push_back(d0b);
+    args.push_back(&d0_off);
+    args.push_back(d1b);
+    args.push_back(&d1_off);
+    args.push_back(scratch);
+    args.push_back(&pi_view);
+    args.push_back(planbuf.data());
+    for (void *sc : scalars) args.push_back(sc);
+    size_t ls = 256;
+    GpuKernel *k1 = srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
+    int err;
+    if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
+    if (p.nsplit > 1) {
+      size_t fg = (size_t)((nrows + 3) / 4);
+      if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args.data())) != GA_NO_ERROR) return err;
+    }
+    return GA_NO_ERROR;
   }
-  args.push_back(d0b);
-  args.push_back(&d0_off);
-  args.push_back(d1b);
-  args.push_back(&d1_off);
-  args.push_back(scratch);
-  args.push_back(&pi_view);
-  args.push_back(planbuf.data());
-  for (void *sc : scalars) args.push_back(sc);
-  size_t ls = 256;
-  GpuKernel *k1 = srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
-  if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
-  if (p.nsplit > 1) {
-    size_t fg = (size_t)((nrows + 3) / 4);
-    if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args.data())) != GA_NO_ERROR) return err;
-  }
-  return GA_NO_ERROR;
+};
+
+int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
+                  const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
+                  unsigned reduxLen, const int *reduxList) {
+  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList).run();
 }
 
 }  // namespace
