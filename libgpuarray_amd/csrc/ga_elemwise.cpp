@@ -990,233 +990,286 @@ int check_general(GpuElemwise *ge, void **args, int flags, size_t *n_out, unsign
 
 inline size_t sabs(ssize_t v) { return v < 0 ? (size_t)(-v) : (size_t)v; }
 
-int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
-  gpucontext *ctx = ge->ctx;
-  const unsigned na = ge->narray;
-  std::vector<size_t> &dims = ge->dims;
-  std::vector<std::vector<ssize_t>> &strs = ge->strs;
+// One call of the strided kernels: the arrays' layout brought into the order
+// the kernels walk it, the choice between the scalar, four-per-lane and
+// transposed-tile forms, the launch.
+class strided_call {
+ public:
+  strided_call(GpuElemwise *ge_, void **args_, size_t n_, unsigned nd_)
+      : ge(ge_), ctx(ge_->ctx), args(args_), n(n_), nd(nd_), na(ge_->narray), dims(ge_->dims),
+        strs(ge_->strs) {}
 
-  // which array is the (first) output, and per-array element sizes / offsets
-  std::vector<size_t> elsz(na), offs(na);
-  int outk = -1;
-  {
-    unsigned k = 0;
-    for (size_t i = 0; i < ge->args.size(); i++) {
-      if (!ge->args[i].is_array()) continue;
-      const GpuArray *v = (const GpuArray *)args[i];
-      elsz[k] = gpuarray_get_elsize(v->typecode);
-      offs[k] = v->offset;
-      if (outk < 0 && ge->args[i].writes()) outk = (int)k;
-      k++;
+  int run() {
+    describe_arrays();
+    normalise_layout();
+    if (is_one_dense_run()) return call_flat(ge, args, n, offs.data());
+    find_transposed_operands();
+    choose_offset_width();
+    choose_vector_access();
+    int err;
+    if ((err = choose_grid()) != GA_NO_ERROR) return err;
+    if ((err = get_kernel()) != GA_NO_ERROR) return err;
+    return launch();
+  }
+
+ private:
+  GpuElemwise *ge;
+  gpucontext *ctx;
+  void **args;
+  const size_t n;
+  unsigned nd;
+  const unsigned na;
+  std::vector<size_t> &dims;
+  std::vector<std::vector<ssize_t>> &strs;
+  std::vector<size_t> elsz, offs;   // per array: element size, byte offset of element 0
+  int outk = -1;                    // the (first) output among the arrays
+  unsigned tmask = 0;               // arrays read or written through transposed tiles
+  bool idx64 = false;               // 64-bit offsets in the kernel
+  bool vec4 = false;                // four elements per lane
+  unsigned umask = 0;               // vec4: arrays with 16-byte access along x
+  unsigned ntmask = 0;              // vec4: arrays touched once, streamed past the caches
+  size_t gx = 0, groups = 0;
+  unsigned ltx = 0, tile = 64;
+  GpuKernel *kernel = nullptr;
+
+  void describe_arrays() {
+    // which array is the (first) output, and per-array element sizes / offsets
+    elsz.assign(na, 0);
+    offs.assign(na, 0);
+    {
+      unsigned k = 0;
+      for (size_t i = 0; i < ge->args.size(); i++) {
+        if (!ge->args[i].is_array()) continue;
+        const GpuArray *v = (const GpuArray *)args[i];
+        elsz[k] = gpuarray_get_elsize(v->typecode);
+        offs[k] = v->offset;
+        if (outk < 0 && ge->args[i].writes()) outk = (int)k;
+        k++;
+      }
     }
   }
 
-  if (nd == 0) {  // 0-d arrays: one element
-    nd = 1;
-    dims.assign(1, 1);
-    for (auto &s : strs) s.assign(1, 0);
-  }
-
-  // Sort dims so the output's stride shrinks towards the last dim (stable),
-  // then drop size-1 dims and fuse runs.
-  {
-    std::vector<unsigned> order(nd);
-    for (unsigned j = 0; j < nd; j++) order[j] = j;
-    std::stable_sort(order.begin(), order.end(), [&](unsigned a, unsigned b) {
-      return sabs(strs[outk][a]) > sabs(strs[outk][b]);
-    });
-    std::vector<size_t> d2(nd);
-    for (unsigned j = 0; j < nd; j++) d2[j] = dims[order[j]];
-    dims = d2;
-    for (unsigned k = 0; k < na; k++) {
-      std::vector<ssize_t> s2(nd);
-      for (unsigned j = 0; j < nd; j++) s2[j] = strs[k][order[j]];
-      strs[k] = s2;
+  void normalise_layout() {
+    if (nd == 0) {  // 0-d arrays: one element
+      nd = 1;
+      dims.assign(1, 1);
+      for (auto &s : strs) s.assign(1, 0);
     }
-  }
-  ge->strp.resize(na);
-  for (unsigned k = 0; k < na; k++) ge->strp[k] = strs[k].data();
-  gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
 
-  // One evenly strided run with every array stepping by its own element
-  // size is the flat case again (all-Fortran inputs, sliced-then-dense...).
-  if (nd == 1) {
+    // Sort dims so the output's stride shrinks towards the last dim (stable),
+    // then drop size-1 dims and fuse runs.
+    {
+      std::vector<unsigned> order(nd);
+      for (unsigned j = 0; j < nd; j++) order[j] = j;
+      std::stable_sort(order.begin(), order.end(), [&](unsigned a, unsigned b) {
+        return sabs(strs[outk][a]) > sabs(strs[outk][b]);
+      });
+      std::vector<size_t> d2(nd);
+      for (unsigned j = 0; j < nd; j++) d2[j] = dims[order[j]];
+      dims = d2;
+      for (unsigned k = 0; k < na; k++) {
+        std::vector<ssize_t> s2(nd);
+        for (unsigned j = 0; j < nd; j++) s2[j] = strs[k][order[j]];
+        strs[k] = s2;
+      }
+    }
+    ge->strp.resize(na);
+    for (unsigned k = 0; k < na; k++) ge->strp[k] = strs[k].data();
+    gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
+  }
+
+  bool is_one_dense_run() const {
+    // One evenly strided run with every array stepping by its own element
+    // size is the flat case again (all-Fortran inputs, sliced-then-dense...).
+    if (nd != 1) return false;
     bool unit = true;
     for (unsigned k = 0; k < na && unit; k++)
       unit = dims[0] == 1 || strs[k][0] == (ssize_t)elsz[k];
-    if (unit) return call_flat(ge, args, n, offs.data());
+    return unit;
   }
 
-  // Transposed operands: small stride on some outer dim, large on x.
-  unsigned tmask = 0;
-  if (nd >= 2 && dims[nd - 1] >= 16) {
-    // candidate y axis: the outer dim on which most arrays have their
-    // smallest non-zero stride
-    std::vector<unsigned> votes(nd, 0);
-    std::vector<int> best(na, -1);
-    for (unsigned k = 0; k < na; k++) {
-      size_t sx = sabs(strs[k][nd - 1]);
-      if (sx == 0) continue;
-      int b = -1;
-      size_t bs = sx;
-      for (unsigned j = 0; j + 1 < nd; j++) {
-        size_t sj = sabs(strs[k][j]);
-        if (sj != 0 && sj < bs && sj <= 4 * elsz[k] && dims[j] >= 16) { bs = sj; b = (int)j; }
+  void find_transposed_operands() {
+    // Transposed operands: small stride on some outer dim, large on x.
+    if (nd >= 2 && dims[nd - 1] >= 16) {
+      // candidate y axis: the outer dim on which most arrays have their
+      // smallest non-zero stride
+      std::vector<unsigned> votes(nd, 0);
+      std::vector<int> best(na, -1);
+      for (unsigned k = 0; k < na; k++) {
+        size_t sx = sabs(strs[k][nd - 1]);
+        if (sx == 0) continue;
+        int b = -1;
+        size_t bs = sx;
+        for (unsigned j = 0; j + 1 < nd; j++) {
+          size_t sj = sabs(strs[k][j]);
+          if (sj != 0 && sj < bs && sj <= 4 * elsz[k] && dims[j] >= 16) { bs = sj; b = (int)j; }
+        }
+        best[k] = b;
+        if (b >= 0) votes[b]++;
       }
-      best[k] = b;
-      if (b >= 0) votes[b]++;
-    }
-    int y = -1;
-    for (unsigned j = 0; j + 1 < nd; j++)
-      if (votes[j] > 0 && (y < 0 || votes[j] > votes[y])) y = (int)j;
-    if (y >= 0) {
-      size_t lds = 0;
-      for (unsigned k = 0; k < na; k++)
-        if (best[k] == y) { tmask |= 1u << k; lds += 64 * 65 * elsz[k]; }
-      if (lds > 64 * 1024 || na > 31) tmask = 0;
-      if (tmask && (unsigned)y != nd - 2) {
-        // rotate y into position nd-2
-        size_t dy = dims[y];
-        dims.erase(dims.begin() + y);
-        dims.insert(dims.begin() + (nd - 2), dy);
-        for (unsigned k = 0; k < na; k++) {
-          ssize_t sy = strs[k][y];
-          strs[k].erase(strs[k].begin() + y);
-          strs[k].insert(strs[k].begin() + (nd - 2), sy);
+      int y = -1;
+      for (unsigned j = 0; j + 1 < nd; j++)
+        if (votes[j] > 0 && (y < 0 || votes[j] > votes[y])) y = (int)j;
+      if (y >= 0) {
+        size_t lds = 0;
+        for (unsigned k = 0; k < na; k++)
+          if (best[k] == y) { tmask |= 1u << k; lds += 64 * 65 * elsz[k]; }
+        if (lds > 64 * 1024 || na > 31) tmask = 0;
+        if (tmask && (unsigned)y != nd - 2) {
+          // rotate y into position nd-2
+          size_t dy = dims[y];
+          dims.erase(dims.begin() + y);
+          dims.insert(dims.begin() + (nd - 2), dy);
+          for (unsigned k = 0; k < na; k++) {
+            ssize_t sy = strs[k][y];
+            strs[k].erase(strs[k].begin() + y);
+            strs[k].insert(strs[k].begin() + (nd - 2), sy);
+          }
         }
       }
     }
   }
 
-  // 32-bit offsets when every reachable byte offset fits
-  bool idx64 = n >= (size_t)GA_SADDR32_MAX;
-  for (unsigned k = 0; k < na && !idx64; k++) {
-    size_t reach = elsz[k];
-    for (unsigned j = 0; j < nd; j++) reach += (dims[j] - 1) * sabs(strs[k][j]);
-    if (reach >= (size_t)GA_SADDR32_MAX) idx64 = true;
-  }
-
-  // Four elements per lane when the layout allows it (see gen_strided_vec).
-  bool vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % 4 == 0 &&
-              strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
-  unsigned umask = 0;
-  if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
-  for (unsigned k = 0; k < na && vec4; k++) {
-    if (elsz[k] > 8) { vec4 = false; break; }
-    const size_t q = 4 * elsz[k];
-    unsigned l2 = 0;
-    const GpuArray *v = nullptr;
-    for (size_t i = 0; i < ge->args.size(); i++)
-      if (ge->args[i].is_array() && l2++ == k) { v = (const GpuArray *)args[i]; break; }
-    const bool base_ok = ((uintptr_t)v->data->devptr + v->offset) % q == 0;
-    const bool tr = (tmask >> k) & 1u;
-    const unsigned unit_dim = tr ? nd - 2 : nd - 1;
-    bool aligned = base_ok && strs[k][unit_dim] == (ssize_t)elsz[k];
-    for (unsigned j = 0; j < nd && aligned; j++)
-      if (j != unit_dim && strs[k][j] % (ssize_t)q != 0) aligned = false;
-    if (tr) {
-      if (!aligned) vec4 = false;          // a transposed operand must be vector-accessible
-    } else if (aligned) {
-      umask |= 1u << k;
+  void choose_offset_width() {
+    // 32-bit offsets when every reachable byte offset fits
+    idx64 = n >= (size_t)GA_SADDR32_MAX;
+    for (unsigned k = 0; k < na && !idx64; k++) {
+      size_t reach = elsz[k];
+      for (unsigned j = 0; j < nd; j++) reach += (dims[j] - 1) * sabs(strs[k][j]);
+      if (reach >= (size_t)GA_SADDR32_MAX) idx64 = true;
     }
   }
-  if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
-  // arrays read or written exactly once per element stream past the caches
-  unsigned ntmask = 0;
-  if (vec4 && ge->nontemporal) {
-    for (unsigned k = 0; k < na; k++) {
-      bool once = true;
-      for (unsigned j = 0; j < nd && once; j++)
-        if (dims[j] > 1 && strs[k][j] == 0) once = false;
-      if (once) ntmask |= 1u << k;
+
+  void choose_vector_access() {
+    // Four elements per lane when the layout allows it (see gen_strided_vec).
+    vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % 4 == 0 &&
+                strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
+    if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
+    for (unsigned k = 0; k < na && vec4; k++) {
+      if (elsz[k] > 8) { vec4 = false; break; }
+      const size_t q = 4 * elsz[k];
+      unsigned l2 = 0;
+      const GpuArray *v = nullptr;
+      for (size_t i = 0; i < ge->args.size(); i++)
+        if (ge->args[i].is_array() && l2++ == k) { v = (const GpuArray *)args[i]; break; }
+      const bool base_ok = ((uintptr_t)v->data->devptr + v->offset) % q == 0;
+      const bool tr = (tmask >> k) & 1u;
+      const unsigned unit_dim = tr ? nd - 2 : nd - 1;
+      bool aligned = base_ok && strs[k][unit_dim] == (ssize_t)elsz[k];
+      for (unsigned j = 0; j < nd && aligned; j++)
+        if (j != unit_dim && strs[k][j] % (ssize_t)q != 0) aligned = false;
+      if (tr) {
+        if (!aligned) vec4 = false;          // a transposed operand must be vector-accessible
+      } else if (aligned) {
+        umask |= 1u << k;
+      }
     }
-    ntmask &= (unsigned)env_ul("GPUARRAY_ELEMWISE_NT_MASK", 0xffffffffu);
-  }
-
-  // launch geometry
-  size_t gx, groups;
-  unsigned ltx = 0, tile = 64;
-  if (tmask == 0) {
-    size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
-    // as many lanes along x as the inner extent needs (a power of two), the
-    // rest of the 256 along the rows: 2^24 floats in rows of 3 took 191 us
-    // with a floor of 16 lanes along x, 61 us without
-    ltx = 0;
-    while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
-    size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
-    size_t rows = n / dims[nd - 1];
-    gx = (inner + 4 * tx - 1) / (4 * tx);
-    groups = gx * ((rows + ty - 1) / ty);
-  } else {
-    // Transposed tiles.  A group takes a 64 x 64 tile (256 lanes) or a
-    // 128 x 128 tile (1024 lanes); the tiles of a plane are handed out in bands
-    // of `ltx` tile rows, down a band's rows first.  Measured on MI355X for
-    // out = in.T of n x n floats: n = 4096 (4096 small tiles) 26.8 us with
-    // small tiles in row-major order, 27.6-28.8 with large ones; n = 8192
-    // 112.6 us small row-major, 106.2 small in bands of 8, 91.3 / 93.3 / 89.8
-    // large in bands of 1 / 2 / 4.  So the large tile is used when it still
-    // gives every compute unit eight groups and its staging copies leave room
-    // for two groups per unit.
-    if (vec4) {
-      size_t lds128 = 0;
-      for (unsigned k = 0; k < na; k++)
-        if ((tmask >> k) & 1u) lds128 += (size_t)128 * 129 * elsz[k];
-      const size_t tiles128 = ((dims[nd - 1] + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
-                              (n / dims[nd - 1] / dims[nd - 2]);
-      tile = (tiles128 >= (size_t)8 * ga_hip_numprocs(ctx) && lds128 <= 80 * 1024) ? 128 : 64;
-      const unsigned long ft = env_ul("GPUARRAY_ELEMWISE_TTILE", 0);
-      if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
-      const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
-      ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", tile == 128 ? 4 : (tiles >= 8192 ? 8 : 1));
-      if (ltx < 1) ltx = 1;
+    if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
+    // arrays read or written exactly once per element stream past the caches
+    if (vec4 && ge->nontemporal) {
+      for (unsigned k = 0; k < na; k++) {
+        bool once = true;
+        for (unsigned j = 0; j < nd && once; j++)
+          if (dims[j] > 1 && strs[k][j] == 0) once = false;
+        if (once) ntmask |= 1u << k;
+      }
+      ntmask &= (unsigned)env_ul("GPUARRAY_ELEMWISE_NT_MASK", 0xffffffffu);
     }
-    gx = (dims[nd - 1] + tile - 1) / tile;
-    size_t gy = (dims[nd - 2] + tile - 1) / tile;
-    size_t outer = n / dims[nd - 1] / dims[nd - 2];
-    groups = gx * gy * outer;
-  }
-  if (!idx64 && (groups >= (size_t)GA_SADDR32_MAX || gx >= (size_t)GA_SADDR32_MAX)) idx64 = true;
-  if (groups > 0x7fffffffull || gx > 0xffffffffull)
-    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
-
-  char key[64];
-  snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-           vec4 ? umask : 0u, ntmask, tile);
-  GpuKernel *k;
-  auto it = ge->k_strided.find(key);
-  if (it != ge->k_strided.end()) {
-    k = &it->second;
-  } else {
-    std::vector<int> ktypes;
-    std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile)
-                           : gen_strided(ge, nd, idx64, tmask, ktypes);
-    GpuKernel nk = {nullptr, nullptr};
-    int err = build_kernel(ge, &nk, src, ktypes);
-    if (err != GA_NO_ERROR) return err;
-    k = &ge->k_strided.emplace(key, nk).first->second;
   }
 
-  unsigned p = 0, l = 0;
-  int err;
-  for (unsigned j = 0; j < nd; j++)
-    if ((err = GpuKernel_setarg(k, p++, &dims[j])) != GA_NO_ERROR) return err;
-  for (size_t i = 0; i < ge->args.size(); i++) {
-    if (ge->args[i].is_array()) {
-      GpuArray *v = (GpuArray *)args[i];
-      if ((err = GpuKernel_setarg(k, p++, v->data)) != GA_NO_ERROR) return err;
-      if ((err = GpuKernel_setarg(k, p++, &v->offset)) != GA_NO_ERROR) return err;
-      for (unsigned j = 0; j < nd; j++)
-        if ((err = GpuKernel_setarg(k, p++, &strs[l][j])) != GA_NO_ERROR) return err;
-      l++;
+  int choose_grid() {
+    // launch geometry
+    if (tmask == 0) {
+      size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
+      // as many lanes along x as the inner extent needs (a power of two), the
+      // rest of the 256 along the rows: 2^24 floats in rows of 3 took 191 us
+      // with a floor of 16 lanes along x, 61 us without
+      ltx = 0;
+      while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
+      size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
+      size_t rows = n / dims[nd - 1];
+      gx = (inner + 4 * tx - 1) / (4 * tx);
+      groups = gx * ((rows + ty - 1) / ty);
     } else {
-      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
+      // Transposed tiles.  A group takes a 64 x 64 tile (256 lanes) or a
+      // 128 x 128 tile (1024 lanes); the tiles of a plane are handed out in bands
+      // of `ltx` tile rows, down a band's rows first.  Measured on MI355X for
+      // out = in.T of n x n floats: n = 4096 (4096 small tiles) 26.8 us with
+      // small tiles in row-major order, 27.6-28.8 with large ones; n = 8192
+      // 112.6 us small row-major, 106.2 small in bands of 8, 91.3 / 93.3 / 89.8
+      // large in bands of 1 / 2 / 4.  So the large tile is used when it still
+      // gives every compute unit eight groups and its staging copies leave room
+      // for two groups per unit.
+      if (vec4) {
+        size_t lds128 = 0;
+        for (unsigned k = 0; k < na; k++)
+          if ((tmask >> k) & 1u) lds128 += (size_t)128 * 129 * elsz[k];
+        const size_t tiles128 = ((dims[nd - 1] + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
+                                (n / dims[nd - 1] / dims[nd - 2]);
+        tile = (tiles128 >= (size_t)8 * ga_hip_numprocs(ctx) && lds128 <= 80 * 1024) ? 128 : 64;
+        const unsigned long ft = env_ul("GPUARRAY_ELEMWISE_TTILE", 0);
+        if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
+        const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
+        ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", tile == 128 ? 4 : (tiles >= 8192 ? 8 : 1));
+        if (ltx < 1) ltx = 1;
+      }
+      gx = (dims[nd - 1] + tile - 1) / tile;
+      size_t gy = (dims[nd - 2] + tile - 1) / tile;
+      size_t outer = n / dims[nd - 1] / dims[nd - 2];
+      groups = gx * gy * outer;
     }
+    if (!idx64 && (groups >= (size_t)GA_SADDR32_MAX || gx >= (size_t)GA_SADDR32_MAX)) idx64 = true;
+    if (groups > 0x7fffffffull || gx > 0xffffffffull)
+      return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Iteration space needs more groups than one launch has");
+    return GA_NO_ERROR;
   }
-  unsigned int gx32 = (unsigned int)gx;
-  if ((err = GpuKernel_setarg(k, p++, &gx32)) != GA_NO_ERROR) return err;
-  if ((err = GpuKernel_setarg(k, p++, &ltx)) != GA_NO_ERROR) return err;
-  size_t ls = (vec4 && tmask) ? (size_t)tile * tile / 16 : 256;
-  return GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
+
+  int get_kernel() {
+    char key[64];
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, tile);
+    auto it = ge->k_strided.find(key);
+    if (it != ge->k_strided.end()) {
+      kernel = &it->second;
+    } else {
+      std::vector<int> ktypes;
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile)
+                             : gen_strided(ge, nd, idx64, tmask, ktypes);
+      GpuKernel nk = {nullptr, nullptr};
+      int err = build_kernel(ge, &nk, src, ktypes);
+      if (err != GA_NO_ERROR) return err;
+      kernel = &ge->k_strided.emplace(key, nk).first->second;
+    }
+    return GA_NO_ERROR;
+  }
+
+  int launch() {
+    unsigned p = 0, l = 0;
+    int err;
+    for (unsigned j = 0; j < nd; j++)
+      if ((err = GpuKernel_setarg(kernel, p++, &dims[j])) != GA_NO_ERROR) return err;
+    for (size_t i = 0; i < ge->args.size(); i++) {
+      if (ge->args[i].is_array()) {
+        GpuArray *v = (GpuArray *)args[i];
+        if ((err = GpuKernel_setarg(kernel, p++, v->data)) != GA_NO_ERROR) return err;
+        if ((err = GpuKernel_setarg(kernel, p++, &v->offset)) != GA_NO_ERROR) return err;
+        for (unsigned j = 0; j < nd; j++)
+          if ((err = GpuKernel_setarg(kernel, p++, &strs[l][j])) != GA_NO_ERROR) return err;
+        l++;
+      } else {
+        if ((err = GpuKernel_setarg(kernel, p++, args[i])) != GA_NO_ERROR) return err;
+      }
+    }
+    unsigned int gx32 = (unsigned int)gx;
+    if ((err = GpuKernel_setarg(kernel, p++, &gx32)) != GA_NO_ERROR) return err;
+    if ((err = GpuKernel_setarg(kernel, p++, &ltx)) != GA_NO_ERROR) return err;
+    size_t ls = (vec4 && tmask) ? (size_t)tile * tile / 16 : 256;
+    return GpuKernel_call(kernel, 1, &groups, &ls, 0, nullptr);
+  }
+};
+
+int call_general(GpuElemwise *ge, void **args, size_t n, unsigned nd) {
+  return strided_call(ge, args, n, nd).run();
 }
 
 }  // namespace
