@@ -141,6 +141,27 @@ def main():
               "avg_launch_us": round(sum_avg * 1e3, 2),
               "algorithmic_bytes_per_launch": sum_bytes}
 
+    # A second yardstick next to the published peak: what the driver's own
+    # device-to-device copy (hipMemcpyDtoDAsync on the library's stream)
+    # sustains on this box, reads plus writes.
+    import ctypes as C
+    from libgpuarray_amd import _lib as _L
+    hip = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p(_L.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
+    get_ptr = _L.extension("hip_get_ptr", C.c_void_p, [C.c_void_p])
+    src_p, dst_p = C.c_void_p(get_ptr(a.ga.data)), C.c_void_p(get_ptr(c.ga.data))
+    for i in range(3 + 10):
+        if i >= 3:
+            ctx.mark(2 * (i - 3))
+        assert hip.hipMemcpyDtoDAsync(dst_p, src_p, C.c_size_t(4 * n), stream) == 0
+        if i >= 3:
+            ctx.mark(2 * (i - 3) + 1)
+    ctx.sync()
+    copy_ms = float(np.mean([ctx.elapsed(2 * i, 2 * i + 1) for i in range(10)]))
+    copy_gbs = 8 * n / (copy_ms * 1e-3) / 1e9
+    roofline["driver_copy_GBps"] = round(copy_gbs, 1)
+    roofline["frac_of_driver_copy"] = round(achieved / copy_gbs, 4)
+
     cpu = cpu_baseline(a_h, b_h, x_h)
     out = {
         "metric": "achieved HBM GB/s for elemwise + reduce (fp32, 2^%d elements)" % args.log2n,

@@ -111,6 +111,15 @@ static void contiguous_strides(ssize_t *str, const size_t *dims, unsigned int nd
 
 extern "C" {
 
+// A struct that was cleared (or never filled) has no buffer and no context to
+// report through: INVALID with a message in the process-wide record, rather
+// than a fault further down.
+#define NEED_BUFFER(arr)                                                                    \
+  do {                                                                                      \
+    if ((arr) == nullptr || (arr)->data == nullptr)                                         \
+      return ga_err_set(ga_global_err, GA_INVALID_ERROR, "Array has no buffer (cleared?)"); \
+  } while (0)
+
 void GpuArray_fix_flags(GpuArray *a) {
   a->flags &= GA_WRITEABLE;
   if (GpuArray_is_c_contiguous(a)) a->flags |= GA_C_CONTIGUOUS;
@@ -219,7 +228,10 @@ int GpuArray_view(GpuArray *v, const GpuArray *a) {
   return GA_NO_ERROR;
 }
 
-int GpuArray_sync(GpuArray *a) { return gpudata_sync(a->data); }
+int GpuArray_sync(GpuArray *a) {
+  NEED_BUFFER(a);
+  return gpudata_sync(a->data);
+}
 
 // reference :243-313.  Per dim: start in [-1, len]; with step 0 the start
 // must be a valid index; otherwise stop in [-1, len] and the span must run in
@@ -468,6 +480,8 @@ gpucontext *GpuArray_context(const GpuArray *a) { return gpudata_context(a->data
 
 // reference :849-877
 int GpuArray_move(GpuArray *dst, const GpuArray *src) {
+  NEED_BUFFER(dst);
+  NEED_BUFFER(src);
   gpucontext *ctx = GpuArray_context(dst);
   if (!GpuArray_ISWRITEABLE(dst))
     return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array (dst) not writeable");
@@ -493,6 +507,7 @@ int GpuArray_move(GpuArray *dst, const GpuArray *src) {
 
 // reference :879-900
 int GpuArray_write(GpuArray *dst, const void *src, size_t src_sz) {
+  NEED_BUFFER(dst);
   gpucontext *ctx = GpuArray_context(dst);
   if (!GpuArray_ISWRITEABLE(dst))
     return ga_err_set(ctx->err, GA_VALUE_ERROR, "Destination array (dst) not writeable");
@@ -502,6 +517,7 @@ int GpuArray_write(GpuArray *dst, const void *src, size_t src_sz) {
 }
 
 int GpuArray_read(void *dst, size_t dst_sz, const GpuArray *src) {
+  NEED_BUFFER(src);
   gpucontext *ctx = GpuArray_context(src);
   if (!GpuArray_ISONESEGMENT(src))
     return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (src) not one segment");
@@ -509,6 +525,7 @@ int GpuArray_read(void *dst, size_t dst_sz, const GpuArray *src) {
 }
 
 int GpuArray_memset(GpuArray *a, int data) {
+  NEED_BUFFER(a);
   gpucontext *ctx = GpuArray_context(a);
   if (!GpuArray_ISONESEGMENT(a))
     return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (a) not one segment");
@@ -516,6 +533,7 @@ int GpuArray_memset(GpuArray *a, int data) {
 }
 
 int GpuArray_copy(GpuArray *res, const GpuArray *a, ga_order order) {
+  NEED_BUFFER(a);
   int err = GpuArray_empty(res, GpuArray_context(a), a->typecode, a->nd, a->dimensions, order);
   if (err != GA_NO_ERROR) return err;
   err = GpuArray_move(res, a);
@@ -525,6 +543,8 @@ int GpuArray_copy(GpuArray *res, const GpuArray *a, ga_order order) {
 
 // reference :913-932
 int GpuArray_transfer(GpuArray *res, const GpuArray *a) {
+  NEED_BUFFER(res);
+  NEED_BUFFER(a);
   gpucontext *ctx = GpuArray_context(res);
   if (!GpuArray_ISONESEGMENT(res))
     return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "Array (res) not one segment");

@@ -48,14 +48,6 @@ struct ge_arg {
 // per array and tile.
 constexpr unsigned GE_LANES = 256;
 
-unsigned long env_ul(const char *name, unsigned long dflt) {
-  const char *v = getenv(name);
-  if (v == nullptr || *v == 0) return dflt;
-  char *end = nullptr;
-  unsigned long r = strtoul(v, &end, 10);
-  return end == v ? dflt : r;
-}
-
 void appendf(std::string &s, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void appendf(std::string &s, const char *fmt, ...) {
   char buf[1024];

@@ -49,13 +49,6 @@ enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL,
 bool is_float_type(int tc) { return tc == GA_FLOAT || tc == GA_DOUBLE || tc == GA_HALF; }
 bool is_int_type(int tc) { return tc >= GA_BOOL && tc <= GA_ULONG; }
 
-unsigned long env_ul(const char *name, unsigned long dflt) {
-  const char *v = getenv(name);
-  if (v == nullptr || *v == 0) return dflt;
-  char *end = nullptr;
-  unsigned long r = strtoul(v, &end, 10);
-  return end == v ? dflt : r;
-}
 
 struct op_info {
   rd_kind kind;

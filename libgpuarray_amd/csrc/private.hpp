@@ -134,6 +134,15 @@ extern const char ga_reduce_kernels_src[];
 // Grow-only scratch buffer owned by the context (partials of two-pass
 // reductions).  Work on a context is in stream order, so one buffer is
 // shared by consecutive calls.
+// A tuning knob from the environment: its value as a number, `dflt` when unset or not one.
+inline unsigned long env_ul(const char *name, unsigned long dflt) {
+  const char *v = getenv(name);
+  if (v == nullptr || *v == 0) return dflt;
+  char *end = nullptr;
+  unsigned long r = strtoul(v, &end, 10);
+  return end == v ? dflt : r;
+}
+
 gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
 // Bytes from a buffer's start that lie inside the memory behind it (at least
 // its size; more when the allocation was rounded up).

@@ -95,6 +95,31 @@ def test_buffer_read_write_move(ctx):           # check_buffer.c:95-177
         lib.gpudata_release(b)
 
 
+def test_large_moves_take_the_copy_kernel(ctx, monkeypatch):
+    """buffer_move copies large ranges with the library's own kernel when source
+    and destination sit equally far from a 16-byte boundary (here from the
+    first byte on), with the driver's copy otherwise: same bytes either way,
+    nothing outside the range, and a cleared array struct is refused."""
+    monkeypatch.setenv("GPUARRAY_MOVE_KERNEL_MIN", "1")
+    rng = np.random.default_rng(31)
+    total = (1 << 20) + 200
+    h = rng.integers(0, 256, total).astype(np.uint8)
+    src = gpuarray.array(h, context=ctx)
+    for so, do, m in ((0, 0, 1 << 20), (3, 3, (1 << 20) + 17), (5, 21, (1 << 19) + 3), (7, 8, 1 << 19),
+                      (1, 1, 1), (2, 18, 15), (0, 16, 16), (9, 9, 40), (4, 4, 4099)):
+        dst = gpuarray.zeros((total,), "uint8", context=ctx)
+        dv, sv = dst[do:do + m], src[so:so + m]          # the views must outlive the call
+        assert lib.GpuArray_move(dv._ptr(), sv._ptr()) == 0
+        got = np.asarray(dst)
+        assert np.array_equal(got[do:do + m], h[so:so + m]), (so, do, m)
+        assert not got[:do].any() and not got[do + m:].any(), (so, do, m)
+    f = gpuarray.array(rng.standard_normal((700, 300)).astype(np.float32), context=ctx)
+    assert np.array_equal(np.asarray(f.copy()), np.asarray(f))
+    cleared = _lib.GpuArrayStruct()
+    assert lib.GpuArray_move(C.byref(cleared), f._ptr()) == _lib.GA_INVALID_ERROR
+    assert lib.GpuArray_read(h.ctypes.data, 4, C.byref(cleared)) == _lib.GA_INVALID_ERROR
+
+
 def test_user_kernel_through_gpukernel(ctx):
     # a kernel in the reference's dialect, launched with explicit geometry and
     # with GpuKernel_sched's geometry
