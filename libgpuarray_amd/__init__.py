@@ -17,7 +17,8 @@ from ._lib import GpuArrayException, UnsupportedException, LIB_PATH
 from . import gpuarray, elemwise, reduction, operations, basic, tools
 from .gpuarray import (GpuContext, GpuArray, GpuKernel, init, array, asarray, empty, zeros, zeros_like,
                        empty_like, ascontiguousarray, asfortranarray, may_share_memory,
-                       set_default_context, get_default_context, count_devices)
+                       set_default_context, get_default_context, count_devices, count_platforms,
+                       from_gpudata, register_dtype, api_version, abi_version)
 from .elemwise import GpuElemwise, arg, as_argument, elemwise1, elemwise2, ielemwise2, compare
 from .reduction import GpuReduction, ReductionKernel
 from ._array import ndgpuarray

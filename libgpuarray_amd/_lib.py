@@ -63,6 +63,14 @@ GA_CTX_PROP_TOTAL_GMEM = 9
 GA_CTX_PROP_FREE_GMEM = 10
 GA_CTX_PROP_MAXGSIZE0 = 12
 GA_CTX_PROP_MAXLSIZE0 = 15
+GA_CTX_PROP_MAXGSIZE1 = 13
+GA_CTX_PROP_MAXGSIZE2 = 14
+GA_CTX_PROP_MAXLSIZE1 = 16
+GA_CTX_PROP_MAXLSIZE2 = 17
+GA_CTX_PROP_UNIQUE_ID = 19
+GA_CTX_PROP_LARGEST_MEMBLOCK = 20
+GPUARRAY_API_VERSION = 2       # include/gpuarray/config.h
+GPUARRAY_ABI_VERSION = 3000    # include/gpuarray/abi_version.h
 GA_BUFFER_PROP_REFCNT = 513
 GA_BUFFER_PROP_SIZE = 514
 GA_KERNEL_PROP_MAXLSIZE = 1025

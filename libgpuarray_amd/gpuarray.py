@@ -12,7 +12,8 @@ import os
 import numpy as np
 
 from . import _lib
-from ._lib import lib, check, GpuArrayException, GpuArrayStruct, c_ssize_t
+from ._lib import lib, check, GpuArrayException, UnsupportedException, GpuArrayStruct, c_ssize_t
+from .dtypes import dtype_to_ctype  # noqa: F401  (part of this module's interface, as in the reference)
 
 # numpy dtype.num equals the typecode on LP64 Linux
 # (reference pygpu/gpuarray.pyx:101-116).
@@ -46,6 +47,41 @@ def count_devices(kind="hip", platform=0):
     n = C.c_uint(0)
     check(lib.gpu_get_device_count(kind.encode(), platform, C.byref(n)))
     return n.value
+
+
+def count_platforms(kind="hip"):
+    """reference pygpu/gpuarray.pyx:534-545"""
+    n = C.c_uint(0)
+    check(lib.gpu_get_platform_count(kind.encode(), C.byref(n)))
+    return n.value
+
+
+def api_version():
+    """(library API version, module version); reference pygpu/gpuarray.pyx:14-18"""
+    return (_lib.GPUARRAY_API_VERSION, 0)
+
+
+def abi_version():
+    """(major, minor) of the library ABI; reference pygpu/gpuarray.pyx:20-25"""
+    return (_lib.GPUARRAY_ABI_VERSION // 1000, _lib.GPUARRAY_ABI_VERSION % 1000)
+
+
+_registered = []   # the type records handed to the C table must stay alive
+
+
+def register_dtype(dtype, cname):
+    """Make a new element type known to the kernel generators under the C name
+    `cname`; returns its typecode (reference pygpu/gpuarray.pyx:120-158)."""
+    dtype = np.dtype(dtype)
+    name = cname.encode() if isinstance(cname, str) else bytes(cname)
+    rec = _lib.GpuArrayType(name, dtype.itemsize, dtype.alignment, 0)
+    typecode = lib.gpuarray_register_type(C.byref(rec), None)
+    if typecode == -1:
+        raise RuntimeError("Could not register type")
+    _registered.append((rec, name))
+    _TYPECODES[dtype] = typecode
+    _DTYPES[typecode] = dtype
+    return typecode
 
 
 class GpuContext(object):
@@ -96,7 +132,35 @@ class GpuContext(object):
     def bin_id(self):
         return self._prop(_lib.GA_CTX_PROP_BIN_ID, C.c_char_p).decode()
 
+    @property
+    def unique_id(self):
+        """PCI bus id of the device"""
+        buf = C.create_string_buffer(16)
+        check(lib.gpucontext_property(self.ctx, _lib.GA_CTX_PROP_UNIQUE_ID, buf), self.ctx)
+        return buf.value.decode()
+
+    @property
+    def ptr(self):
+        """the gpucontext pointer as an integer"""
+        return self.ctx.value
+
+    def __enter__(self):
+        # the reference makes a CUDA context current here (cuda_enter); every
+        # call of this backend selects its device itself
+        return self
+
+    def __exit__(self, t, v, tb):
+        return False
+
+    def __reduce__(self):
+        raise RuntimeError("Cannot pickle GpuContext object")
+
     numprocs = property(lambda s: s._prop(_lib.GA_CTX_PROP_NUMPROCS, C.c_uint))
+    maxlsize1 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXLSIZE1, C.c_size_t))
+    maxlsize2 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXLSIZE2, C.c_size_t))
+    maxgsize1 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXGSIZE1, C.c_size_t))
+    maxgsize2 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXGSIZE2, C.c_size_t))
+    largest_memblock = property(lambda s: s._prop(_lib.GA_CTX_PROP_LARGEST_MEMBLOCK, C.c_size_t))
     lmemsize = property(lambda s: s._prop(_lib.GA_CTX_PROP_LMEMSIZE, C.c_size_t))
     maxlsize0 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXLSIZE0, C.c_size_t))
     maxgsize0 = property(lambda s: s._prop(_lib.GA_CTX_PROP_MAXGSIZE0, C.c_size_t))
@@ -166,25 +230,64 @@ def _ensure_context(context):
 
 
 class flags(object):
-    """numpy-style flag view (reference pygpu/gpuarray.pyx:1390-1480)."""
+    """NumPy-style view of an array's flag word, by attribute or by NumPy's
+    flag names and one- or two-letter short forms (reference
+    pygpu/gpuarray.pyx:1190-1342)."""
+
+    _KEYS = {"C": "c_contiguous", "F": "f_contiguous", "W": "writeable", "B": "behaved",
+             "O": "owndata", "A": "aligned", "U": "updateifcopy", "CA": "carray", "FA": "farray",
+             "FNC": "fnc", "FORC": "forc", "CARRAY": "carray", "FARRAY": "farray",
+             "FORTRAN": "fortran", "BEHAVED": "behaved", "OWNDATA": "owndata",
+             "ALIGNED": "aligned", "WRITEABLE": "writeable", "CONTIGUOUS": "c_contiguous",
+             "UPDATEIFCOPY": "updateifcopy", "C_CONTIGUOUS": "c_contiguous",
+             "F_CONTIGUOUS": "f_contiguous"}
+    _BEHAVED = _lib.GA_ALIGNED | _lib.GA_WRITEABLE
 
     def __init__(self, fl):
-        self.fl = fl
+        self.fl = int(fl)
+
+    def __reduce__(self):
+        return (flags, (self.fl,))
 
     c_contiguous = property(lambda s: bool(s.fl & _lib.GA_C_CONTIGUOUS))
     f_contiguous = property(lambda s: bool(s.fl & _lib.GA_F_CONTIGUOUS))
+    contiguous = c_contiguous
+    fortran = f_contiguous
     aligned = property(lambda s: bool(s.fl & _lib.GA_ALIGNED))
     writeable = property(lambda s: bool(s.fl & _lib.GA_WRITEABLE))
-    contiguous = c_contiguous
-    fortran = property(lambda s: s.f_contiguous and not s.c_contiguous)
+    updateifcopy = property(lambda s: False)     # not supported
+    owndata = property(lambda s: True)           # no equivalent for device arrays
+    behaved = property(lambda s: (s.fl & s._BEHAVED) == s._BEHAVED)
+    carray = property(lambda s: s.behaved and s.c_contiguous)
     forc = property(lambda s: s.c_contiguous or s.f_contiguous)
+    fnc = property(lambda s: s.f_contiguous and not s.c_contiguous)
+    # any of F_CONTIGUOUS / ALIGNED / WRITEABLE set and not C-contiguous: NumPy's own definition
+    farray = property(lambda s: bool(s.fl & (_lib.GA_F_CONTIGUOUS | s._BEHAVED)) and not s.c_contiguous)
+    num = property(lambda s: s.fl)
 
-    def __getitem__(self, name):
-        return getattr(self, name.lower())
+    def __getitem__(self, key):
+        if isinstance(key, bytes):
+            key = key.decode()
+        if not isinstance(key, str) or key not in self._KEYS:
+            raise KeyError("Unknown flag")
+        return getattr(self, self._KEYS[key])
+
+    def __eq__(self, other):
+        if not isinstance(other, flags):
+            return NotImplemented
+        return self.fl == other.fl
+
+    def __ne__(self, other):
+        if not isinstance(other, flags):
+            return NotImplemented
+        return self.fl != other.fl
+
+    __hash__ = None
 
     def __repr__(self):
-        return "  C_CONTIGUOUS : %s\n  F_CONTIGUOUS : %s\n  WRITEABLE : %s\n  ALIGNED : %s" % (
-            self.c_contiguous, self.f_contiguous, self.writeable, self.aligned)
+        return "\n".join(" %s : %s" % (n.upper(), getattr(self, n)) for n in
+                         ("c_contiguous", "f_contiguous", "owndata", "writeable", "aligned",
+                          "updateifcopy"))
 
 
 class GpuArray(object):
@@ -377,6 +480,23 @@ class GpuArray(object):
                 else _lib.GA_C_ORDER
         self._check(lib.GpuArray_copy(res._ptr(), self._ptr(), o))
         return res
+
+    def transfer(self, new_ctx):
+        """A copy of this array in another context
+        (reference pygpu/gpuarray.pyx:1779-1791)."""
+        if not (self.flags.c_contiguous or self.flags.f_contiguous):
+            raise ValueError("transfer() only works for contigous source")
+        res = empty(self.shape, self.dtype, "C" if self.flags.c_contiguous else "F", context=new_ctx)
+        check(lib.GpuArray_transfer(res._ptr(), self._ptr()), new_ctx.ctx)
+        return res
+
+    @property
+    def data(self):
+        """The raw OpenCL buffer object in the reference
+        (pygpu/gpuarray.pyx:2223-2236): there is no such object here."""
+        raise TypeError("This is for OpenCL arrays.")
+
+    base_data = data
 
     def take1(self, idx):
         """Rows of `self` picked by the 1-D integer array `idx`
@@ -584,6 +704,41 @@ def from_strided(base, offset, shape, strides, dtype=None, writeable=True, cls=N
     tc = base.typecode if dtype is None else dtype_to_typecode(dtype)
     check(lib.GpuArray_fromdata(res._ptr(), base.ga.data, offset, tc, nd, dims, strs,
                                 1 if writeable else 0), base.context.ctx)
+    res.base = base
+    return res
+
+
+class _gpudata_owner(object):
+    """Stands for a buffer known only by its gpudata pointer."""
+
+    def __init__(self, context, data):
+        self.context = context
+        self.ga = GpuArrayStruct()
+        self.ga.data = data
+
+
+def from_gpudata(data, offset, dtype, shape, context=None, strides=None, writable=True, base=None,
+                 cls=None):
+    """An array over an existing buffer given as the integer value of its
+    gpudata pointer (the `gpudata` attribute of an array); C-contiguous
+    unless `strides` are given.  `base` is kept alive with the result
+    (reference pygpu/gpuarray.pyx:849-939).  As there, a wrong pointer takes
+    the interpreter down."""
+    context = _ensure_context(context)
+    try:
+        shape = tuple(shape)
+    except TypeError:
+        shape = (shape,)
+    if strides is not None and len(strides) != len(shape):
+        raise ValueError("strides must be the same length as shape")
+    dtype = np.dtype(dtype)
+    if not strides:
+        strides, step = [], dtype.itemsize
+        for d in reversed(shape):
+            strides.insert(0, step)
+            step *= d
+    res = from_strided(_gpudata_owner(context, data), offset, shape, strides, dtype=dtype,
+                       writeable=writable, cls=cls or GpuArray)
     res.base = base
     return res
 

@@ -9,7 +9,7 @@ import pytest
 
 import libgpuarray_amd as ga
 from libgpuarray_amd import gpuarray
-from support import gen_gpuarray
+from support import gen_gpuarray, to_gpu_view
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "float64", "int8", "int16", "uint8", "uint16", "int32", "int64", "uint32",
@@ -314,3 +314,94 @@ def test_getitem_w_int(ctx, dtype, offseted):              # :605-672
         _cmp(_a[k], a[k])
     with pytest.raises(NotImplementedError):
         _a[[0, 1]]
+
+
+def test_flags_object_follows_numpy(ctx):                 # pygpu/gpuarray.pyx:1190-1342
+    keys = ["C", "F", "W", "A", "B", "O", "CA", "FA", "FNC", "FORC", "CARRAY", "FARRAY", "FORTRAN",
+            "BEHAVED", "OWNDATA", "ALIGNED", "WRITEABLE", "CONTIGUOUS", "C_CONTIGUOUS",
+            "F_CONTIGUOUS"]
+    base = np.arange(24, dtype="float32").reshape(4, 6)
+    for view in (base, base.T, base[::2], base[:, ::2], base[1:2, :], np.asfortranarray(base)):
+        g, _ = to_gpu_view(view, ctx)
+        own = np.array(view, copy=True, order="K") if False else view
+        for k in keys:
+            if k in ("O", "OWNDATA"):
+                assert g.flags[k] is True          # always, by definition there
+                continue
+            assert g.flags[k] == own.flags[k], (k, view.strides)
+        assert g.flags["U"] is False and g.flags["UPDATEIFCOPY"] is False
+        assert g.flags.num == g.ga.flags and g.flags.fortran == g.flags.f_contiguous
+        assert g.flags == gpuarray.flags(g.ga.flags) and not (g.flags != gpuarray.flags(g.ga.flags))
+        assert g.flags[b"C"] == g.flags.c_contiguous
+    with pytest.raises(KeyError):
+        g.flags["X"]
+    with pytest.raises(KeyError):
+        g.flags[3]
+    import pickle
+    assert pickle.loads(pickle.dumps(g.flags)) == g.flags
+    assert "C_CONTIGUOUS" in repr(g.flags) and "UPDATEIFCOPY" in repr(g.flags)
+
+
+def test_module_interface(ctx):
+    assert gpuarray.api_version() == (2, 0) and gpuarray.abi_version() == (3, 0)
+    assert gpuarray.count_platforms("hip") == 1 and gpuarray.count_devices("hip", 0) >= 1
+    assert gpuarray.dtype_to_ctype(np.dtype("float32")) == "ga_float"
+    assert issubclass(gpuarray.UnsupportedException, gpuarray.GpuArrayException)
+    # context properties and protocol
+    assert ctx.ptr == ctx.ctx.value and len(ctx.unique_id) >= 7 and ":" in ctx.unique_id
+    assert ctx.maxlsize1 >= 1 and ctx.maxlsize2 >= 1 and ctx.maxgsize1 >= 1 and ctx.maxgsize2 >= 1
+    assert 0 < ctx.largest_memblock <= ctx.total_gmem
+    with ctx as c:
+        assert c is ctx
+    with pytest.raises(RuntimeError):
+        ctx.__reduce__()
+    # an array over the buffer of another one, by pointer value
+    h = np.arange(60, dtype="int32")
+    g = gpuarray.array(h, context=ctx)
+    v = gpuarray.from_gpudata(g.gpudata, 8, "int32", (4, 5), context=ctx, base=g)
+    assert v.base is g and np.array_equal(np.asarray(v), h[2:22].reshape(4, 5))
+    v2 = gpuarray.from_gpudata(g.gpudata, 0, "int32", 10, context=ctx, strides=(24,), writable=False,
+                               base=g)
+    assert np.array_equal(np.asarray(v2), h[::6]) and not v2.flags.writeable
+    with pytest.raises(ValueError):
+        gpuarray.from_gpudata(g.gpudata, 0, "int32", (2, 2), context=ctx, strides=(4,))
+    with pytest.raises(TypeError):
+        g.data
+    with pytest.raises(TypeError):
+        g.base_data
+
+
+def test_register_dtype_and_use_it(ctx):
+    """A caller-defined element type: registered under a C name, usable as the
+    element type of arrays and in kernels whose preamble declares it
+    (pygpu/gpuarray.pyx:120-158)."""
+    pair = np.dtype([("lo", "int32"), ("hi", "int32")])
+    tc = gpuarray.register_dtype(pair, "my_pair")
+    assert tc >= 512 and gpuarray.dtype_to_typecode(pair) == tc          # user range
+    assert gpuarray.typecode_to_dtype(tc) == pair
+    h = np.zeros(100, pair)
+    h["lo"] = np.arange(100)
+    h["hi"] = 7
+    g = gpuarray.array(h, context=ctx)
+    assert g.dtype == pair and g.itemsize == 8
+    back = np.asarray(g.copy())
+    assert np.array_equal(back["lo"], h["lo"]) and np.array_equal(back["hi"], h["hi"])
+    ew = ga.GpuElemwise(ctx, "o = p.lo + p.hi", [ga.arg("p", pair, read=True),
+                                                ga.arg("o", "int32", write=True)],
+                        preamble="typedef struct { int lo, hi; } my_pair;")
+    out = gpuarray.zeros((100,), "int32", context=ctx)
+    ew(g, out)
+    assert np.array_equal(np.asarray(out), h["lo"] + 7)
+
+
+def test_transfer_between_contexts(ctx):
+    other = gpuarray.init("hip0")
+    h = np.arange(1000, dtype="float32").reshape(10, 100)
+    g = gpuarray.array(h, context=ctx)
+    t = g.transfer(other)
+    assert t.context is other and np.array_equal(np.asarray(t), h)
+    f = gpuarray.array(np.asfortranarray(h), context=ctx)
+    tf = f.transfer(other)
+    assert tf.flags.f_contiguous and np.array_equal(np.asarray(tf), h)
+    with pytest.raises(ValueError):
+        g[:, ::2].transfer(other)
