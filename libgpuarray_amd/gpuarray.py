@@ -79,6 +79,8 @@ def register_dtype(dtype, cname):
     if typecode == -1:
         raise RuntimeError("Could not register type")
     _registered.append((rec, name))
+    from . import dtypes
+    dtypes._REGISTERED[dtype] = name.decode()
     _TYPECODES[dtype] = typecode
     _DTYPES[typecode] = dtype
     return typecode

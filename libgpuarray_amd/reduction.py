@@ -64,37 +64,27 @@ class GpuReduction(object):
 
 
 from .tools import Argument, ArrayArg, ScalarArg, as_argument  # noqa: E402,F401
+from .dtypes import parse_c_arg_backend  # noqa: E402
 
 
-_C_TYPES = {
-    "bool": "bool", "char": "int8", "signed char": "int8", "unsigned char": "uint8",
-    "short": "int16", "unsigned short": "uint16", "int": "int32", "unsigned": "uint32",
-    "unsigned int": "uint32", "long": "int64", "unsigned long": "uint64",
-    "long long": "int64", "unsigned long long": "uint64", "float": "float32",
-    "double": "float64", "half": "float16", "ga_half": "float16", "ga_bool": "bool",
-    "ga_byte": "int8", "ga_ubyte": "uint8", "ga_short": "int16", "ga_ushort": "uint16",
-    "ga_int": "int32", "ga_uint": "uint32", "ga_long": "int64", "ga_ulong": "uint64",
-    "ga_float": "float32", "ga_double": "float64",
-}
-_DECL_RE = re.compile(r"(\**)\s*([_a-zA-Z0-9]+)(\s*\[[ 0-9]*\])*\s*$")
 _INDEX_RE = re.compile(r"([a-zA-Z_][a-zA-Z0-9_]*)\[i\]")
 
 
 def parse_c_args(arguments):
     """"float *a, float *b, float s" -> (ArrayArg, ArrayArg, ScalarArg)
-    (reference pygpu/reduction.py:13-15, pygpu/dtypes.py:121-147)."""
-    res = []
-    for c_arg in arguments.split(","):
-        c_arg = c_arg.replace("const", "").replace("volatile", "").replace("GLOBAL_MEM", "")
-        m = _DECL_RE.search(c_arg)
-        if m is None:
-            raise ValueError("couldn't parse C declarator '%s'" % c_arg)
-        tp = " ".join(c_arg[:m.start()].split())
-        if tp not in _C_TYPES:
-            raise ValueError("unknown type '%s'" % tp)
-        cls = ArrayArg if (m.group(1) or m.group(3) is not None) else ScalarArg
-        res.append(cls(np.dtype(_C_TYPES[tp]), m.group(2)))
-    return tuple(res)
+    (reference pygpu/reduction.py:13-15)."""
+    return tuple(parse_c_arg_backend(c_arg.replace("GLOBAL_MEM", ""), ScalarArg, ArrayArg)
+                 for c_arg in arguments.split(","))
+
+
+def massage_op(operation):
+    """`a[i]` -> `a[0]` for every indexed name (reference pygpu/reduction.py:21-22)."""
+    return _INDEX_RE.sub(r"\g<1>[0]", operation)
+
+
+def _ceil_log2(x):
+    """Exponent of the nearest power of two at or above x (reference pygpu/reduction.py:25-30)."""
+    return int(x - 1).bit_length() if x > 0 else 0
 
 
 class ReductionKernel(object):
