@@ -37,6 +37,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # inside this process, so the figure is carried here for the shape it was
 # measured on.
 MEASURED_TRAFFIC = {28: 3219788085}
+MEASURED_TRAFFIC_SUM = {28: 1073816553}   # redux_row of the full sum, same file
 
 
 def main():
@@ -137,7 +138,9 @@ def main():
     sum_avg = float(sum_ms.mean())
     sum_gbs = sum_bytes / (sum_avg * 1e-3) / 1e9
     second = {"kernel": "redux_row + redux_final (full fp32 sum, two passes)",
+              "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
               "achieved": round(sum_gbs, 1), "frac": round(sum_gbs / HBM_PEAK_GBS, 4),
+              "traffic": MEASURED_TRAFFIC_SUM.get(args.log2n),
               "avg_launch_us": round(sum_avg * 1e3, 2),
               "algorithmic_bytes_per_launch": sum_bytes}
 
