@@ -332,7 +332,11 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
  * some path skips, the result still counts as pending at the loop's back edge,
  * and in the next round each load of the unit waits for the one before it
  * (their destination registers may be in flight) instead of all being issued
- * back to back.  Costs no instruction. */
+ * back to back.  Costs no instruction, but it makes the first use wait for
+ * all of the unit's loads; redux_row leaves it out (RD_TOUCH_ROW 0) for sums
+ * and the like over several sources, where the compiler orders the waits well
+ * by itself and the combination starts as the first loads arrive (dot product
+ * of two 2^27-float vectors: 153.6 us without it, 158.3 with). */
 static __device__ inline void rd_touch(const ga_float v) { asm volatile("" ::"v"(v)); }
 static __device__ inline void rd_touch(const ga_double v) { asm volatile("" ::"v"(v)); }
 template <typename T>
@@ -589,7 +593,9 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
       const ga_long sh = RD_SHIFT(ub[0]);
       ub[0] -= sh * RD_ELSZ0;
       rd_unit_load<RD_G / RD_LO>(x, ub, e0, rin + sh, rstr);
+#if RD_TOUCH_ROW
       rd_unit_touch(x);
+#endif
       acc = rd_combine(acc, rd_unit_combine<RD_G / RD_LO>(x, e0, rin + sh, ib, rml, sh RD_SCALAR_ARGS));
     }
   }
@@ -612,7 +618,9 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
     const ga_long sh = RD_SHIFT(ub[0]);
     ub[0] -= sh * RD_ELSZ0;
     rd_unit_load<RD_G>(x, ub, e0, rin + sh, rstr);
+#if RD_TOUCH_ROW
     rd_unit_touch(x);
+#endif
     acc = rd_combine(acc, rd_unit_combine<RD_G>(x, e0, rin + sh, ib, rml, sh RD_SCALAR_ARGS));
 #if RD_INTERLEAVE
     k += ustep;   /* single reduced dim: the unit is the segment */
