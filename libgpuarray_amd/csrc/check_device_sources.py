@@ -95,6 +95,13 @@ def main():
         check("reduction short rows staged in LDS, op %d type %d" % (op, src),
               gen_r(op, src, d0, GA_LONG, 64, 1, 1 | (1 << 25)))
         n += 1
+    GA_BYTE, GA_ULONG = 1, 8
+    for label, spec in (("sum of unsigned bytes", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8)),
+                        ("sum of signed bytes", (0, GA_BYTE, GA_LONG, GA_LONG, 256, 16, 8)),
+                        ("sum of bytes, shifted rows", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8 | (1 << 24))),
+                        ("all over stepped bytes", (12, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 4))):
+        check("reduction four bytes per operation: " + label, gen_r(*spec))
+        n += 1
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
     # an expression over several arrays and a scalar feeding the reduction
     margs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_HALF, 2),

@@ -41,7 +41,7 @@ struct rd_plan {
   int64_t fdim[RD_MAXD], fd0str[RD_MAXD], fd1str[RD_MAXD];
   int64_t rdim[RD_MAXD], rmul[RD_MAXD];
   int64_t nrows, rtotal, nseg, units, upb, gx, router;
-  int32_t nf, nr, nsplit, pad;
+  int32_t nf, nr, nsplit, split_major;
 };
 
 enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL, K_ANY, K_CUSTOM };
@@ -120,6 +120,7 @@ std::string neutral_for(rd_kind kind, int acc_tc) {
 
 struct variant {
   GpuKernel row = {nullptr, nullptr}, col = {nullptr, nullptr}, fin = {nullptr, nullptr},
+            fin_cols = {nullptr, nullptr},   // second pass after redux_col
             wrows = {nullptr, nullptr},   // wrows only exists in 64-lane variants
             srows = {nullptr, nullptr};   // the only kernel of a short-rows variant (opts bit 3)
 };
@@ -196,6 +197,12 @@ int acc_typecode(const GpuReduction *gr, int d0_tc) {
   return (kind == K_MIN || kind == K_MAX) ? gr->src_tc() : d0_tc;
 }
 
+// One-byte elements of a vector-loaded source are kept packed in 32-bit words
+// when a load holds whole words.
+bool packed_bytes(int tc, const variant_spec &vs) {
+  return gpuarray_get_elsize(tc) == 1 && (vs.V * vs.ES) % 4 == 0;
+}
+
 // The text that specialises reduce_kernels.h: `defs` goes in front of it,
 // `gen` replaces its @RD_GENERATED@ mark.
 int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string &defs,
@@ -243,6 +250,18 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
   DEF("#define RD_CY %u\n", vs.CY ? vs.CY : 4u);
   {
+    // One-byte elements under sum / any / all with an integer accumulator:
+    // the unit is combined four elements per 32-bit operation (RD_FAST8: 1
+    // unsigned, 2 signed).  Needs the plain operator on one source fetched
+    // with vector loads of whole 32-bit words.
+    const int stc = gr->args[gr->arrays[0]].tc;
+    const bool bytes = K == 1 && !gr->mapped && gpuarray_get_elsize(stc) == 1 && (vs.vecmask & 1u) &&
+                       (vs.V * vs.ES) % 4 == 0 && (vs.ES == 1 || vs.ES == 2 || vs.ES == 4) &&
+                       (kind == K_SUM || kind == K_ANY || kind == K_ALL) && !valf &&
+                       env_ul("GPUARRAY_REDUX_FAST8", 1);
+    DEF("#define RD_FAST8 %d\n", bytes ? (stc == GA_BYTE ? 2 : 1) : 0);
+  }
+  {
     // redux_row: an unconditional use after each unit's loads where the
     // combination puts every use under a branch (see rd_touch)
     bool half_src = false;
@@ -278,7 +297,13 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   for (unsigned k = 0; k < K; k++) {
     const int tc = gr->args[gr->arrays[k]].tc;
     const char *lt = load_type_name(tc);
-    if ((vs.vecmask >> k) & 1u) {
+    if (((vs.vecmask >> k) & 1u) && packed_bytes(tc, vs)) {
+      // One-byte elements stay packed in 32-bit words; an element is shifted
+      // out where it is used.  A vector of bytes would be taken apart right
+      // after each load, which makes every load wait for the one before it.
+      GEN("typedef ga_uint rd_pvec%u_t __attribute__((ext_vector_type(RD_PV / 4)));\n", k);
+      snprintf(line, sizeof(line), " rd_pvec%u_t x%u[RD_U];", k, k);
+    } else if ((vs.vecmask >> k) & 1u) {
       GEN("typedef %s rd_pvec%u_t __attribute__((ext_vector_type(RD_PV)));\n", lt, k);
       snprintf(line, sizeof(line), " rd_pvec%u_t x%u[RD_U];", k, k);
     } else {
@@ -329,7 +354,11 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   }
   gen += "  }\n}\n#define RD_UNIT_VAL(u, j, v) rd_map(";
   for (unsigned k = 0; k < K; k++) {
-    if ((vs.vecmask >> k) & 1u) GEN("%srd_w%u((u).x%u[j][(v) * RD_ES])", k ? ", " : "", k, k);
+    const int tck = gr->args[gr->arrays[k]].tc;
+    if (((vs.vecmask >> k) & 1u) && packed_bytes(tck, vs))
+      GEN("%srd_w%u((%s)((u).x%u[j][((v) * RD_ES) / 4] >> (8 * (((v) * RD_ES) %% 4))))", k ? ", " : "", k,
+          load_type_name(tck), k);
+    else if ((vs.vecmask >> k) & 1u) GEN("%srd_w%u((u).x%u[j][(v) * RD_ES])", k ? ", " : "", k, k);
     else GEN("%srd_w%u((u).x%u[j][v])", k ? ", " : "", k, k);
   }
   gen += " RD_SCALAR_ARGS)\n"
@@ -340,16 +369,37 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   for (unsigned k = 0; k < K; k++) GEN("%srd_w%u((o).x%u)", k ? ", " : "", k, k);
   gen += " RD_SCALAR_ARGS)\n";
   // RD_CV adjacent elements per source (redux_col)
-  for (unsigned k = 0; k < K; k++)
-    GEN("typedef %s rd_cv%u_t __attribute__((ext_vector_type(RD_CV)));\n",
-        load_type_name(gr->args[gr->arrays[k]].tc), k);
+  // One- and two-byte elements stay packed in 32-bit words here too (see the
+  // unit registers above); `words` is 0 for a source kept as a vector of its
+  // own element type.
+  std::vector<unsigned> words(K, 0);
+  const unsigned cvn = vs.CV ? vs.CV : 1;
+  for (unsigned k = 0; k < K; k++) {
+    const int tc = gr->args[gr->arrays[k]].tc;
+    const unsigned es = (unsigned)gpuarray_get_elsize(tc);
+    if ((es == 1 || es == 2) && (cvn * es) % 4 == 0) words[k] = cvn * es / 4;
+    if (words[k] == 1) GEN("typedef ga_uint rd_cv%u_t;\n", k);
+    else if (words[k] > 1) GEN("typedef ga_uint rd_cv%u_t __attribute__((ext_vector_type(%u)));\n", k, words[k]);
+    else GEN("typedef %s rd_cv%u_t __attribute__((ext_vector_type(RD_CV)));\n", load_type_name(tc), k);
+  }
   gen += "struct rd_cvec {";
   for (unsigned k = 0; k < K; k++) GEN(" rd_cv%u_t x%u;", k, k);
   gen += " };\nstatic __device__ inline void rd_cvec_load(rd_cvec &o, const char *const *p) {\n";
   for (unsigned k = 0; k < K; k++)
     GEN("  o.x%u = RD_LOAD((const rd_cv%u_t *)p[%u]);\n", k, k, k);
   gen += "}\n#define RD_CVEC_VAL(o, c) rd_map(";
-  for (unsigned k = 0; k < K; k++) GEN("%srd_w%u((o).x%u[c])", k ? ", " : "", k, k);
+  for (unsigned k = 0; k < K; k++) {
+    const int tc = gr->args[gr->arrays[k]].tc;
+    const unsigned es = (unsigned)gpuarray_get_elsize(tc), per = 4 / (es ? es : 4);
+    if (words[k] == 1)
+      GEN("%srd_w%u((%s)((o).x%u >> (%u * ((c) %% %u))))", k ? ", " : "", k, load_type_name(tc), k,
+          8 * es, per);
+    else if (words[k] > 1)
+      GEN("%srd_w%u((%s)((o).x%u[(c) / %u] >> (%u * ((c) %% %u))))", k ? ", " : "", k,
+          load_type_name(tc), k, per, 8 * es, per);
+    else
+      GEN("%srd_w%u((o).x%u[c])", k ? ", " : "", k, k);
+  }
   gen += " RD_SCALAR_ARGS)\n";
 #undef GEN
   return GA_NO_ERROR;
@@ -407,9 +457,9 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   for (int t : flag_types) kflags |= gpuarray_type_flags(t, -1);
   const unsigned na = (unsigned)types.size();
   variant v;
-  const char *names[4] = {"redux_row", "redux_col", "redux_final", "redux_wrows"};
-  GpuKernel *ks[4] = {&v.row, &v.col, &v.fin, &v.wrows};
-  int nk = vs.G == 64 ? 4 : 3;
+  const char *names[5] = {"redux_row", "redux_col", "redux_final", "redux_final_cols", "redux_wrows"};
+  GpuKernel *ks[5] = {&v.row, &v.col, &v.fin, &v.fin_cols, &v.wrows};
+  int nk = vs.G == 64 ? 5 : 4;
   if (vs.opts & 8u) {
     names[0] = "redux_srows";
     ks[0] = &v.srows;
@@ -1030,7 +1080,7 @@ class reduction_call {
     {
       unsigned cv = (unsigned)(16 / elsz_max);
       if (info.has_d1 && cv > 4) cv = 4;
-      if (cv > 8) cv = 8;
+      if (cv > (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16)) cv = (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16);
       for (unsigned q = 0; q < K; q++)
         if (fsstr[q * RD_MAXD + p.nf - 1] != elsz[q]) cv = 1;
       while (cv > 1) {
@@ -1078,6 +1128,15 @@ class reduction_call {
     p.upb = (rtotal + nsplit - 1) / nsplit;
     if (p.upb > 0) nsplit = (rtotal + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;
+    // Partials of a split column reduction: with many outputs they are laid
+    // out split-major, so that adjacent lanes write adjacent slots, and the
+    // second pass runs with lanes along the outputs (sum over axis 0 of
+    // 8192 x 8192 bytes 37.8 -> 32.8 us, of int16 41.0 -> 37.0); with few
+    // outputs that second pass would have too few lanes (1000 outputs over
+    // 256 splits: 51.6 -> 65.9 us), and they stay output-major for the
+    // wavefront-per-output pass.
+    const int64_t many = (int64_t)env_ul("GPUARRAY_REDUX_SPLIT_MAJOR_MIN", 4096);
+    p.split_major = (nsplit > 1 && nrows >= many) ? 1 : 0;
     groups = (size_t)(base_groups * nsplit);
     U = (unsigned)env_ul("GPUARRAY_REDUX_COL_U", 4);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 4;
@@ -1142,8 +1201,10 @@ class reduction_call {
     int err;
     if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
     if (p.nsplit > 1) {
-      size_t fg = (size_t)((nrows + 3) / 4);
-      if ((err = GpuKernel_call(&var->fin, 1, &fg, &ls, 0, args.data())) != GA_NO_ERROR) return err;
+      size_t fg = (size_t)(p.split_major ? (nrows + 63) / 64 : (nrows + 3) / 4);
+      if ((err = GpuKernel_call(p.split_major ? &var->fin_cols : &var->fin, 1, &fg, &ls, 0,
+                                args.data())) != GA_NO_ERROR)
+        return err;
     }
     return GA_NO_ERROR;
   }
@@ -1229,6 +1290,7 @@ void GpuReduction_free(GpuReduction *gr) {
     GpuKernel_clear(&kv.second.row);
     GpuKernel_clear(&kv.second.col);
     GpuKernel_clear(&kv.second.fin);
+    if (kv.second.fin_cols.k != nullptr) GpuKernel_clear(&kv.second.fin_cols);
     if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
     if (kv.second.srows.k != nullptr) GpuKernel_clear(&kv.second.srows);
   }

@@ -21,6 +21,8 @@
  *               advances by RD_ES elements per index (a [::2] or [::4] view), a
  *               load fetches RD_VEC*RD_ES contiguous elements and every
  *               RD_ES-th one is used
+ *   RD_FAST8    one-byte elements combined four per 32-bit operation (sum, any,
+ *               all; 1: unsigned bytes, 2: signed), 0: off
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
  *   RD_TAIL     rows that are misaligned for the vector load or whose extent
  *               is not a multiple of RD_VEC (one source, contiguous rows): a
@@ -104,7 +106,7 @@ struct rd_plan {
   ga_long upb;     /* work per split: units (row) or elements (col) */
   ga_long gx;      /* redux_col: groups along the inner free dim */
   ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates */
-  ga_int nf, nr, nsplit, pad;
+  ga_int nf, nr, nsplit, split_major;   /* split_major: layout of redux_col's partials */
   ga_long fsstr[RD_NSRC][RD_MAXD], rsstr[RD_NSRC][RD_MAXD];   /* per source */
 };
 
@@ -499,6 +501,61 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
   r.i = any ? ib + (e0 + bp - sh) * rml : r.i;
 #else
   (void)bp; (void)ib; (void)rml;
+#endif
+  return r;
+#elif RD_FAST8
+  /* One-byte elements, four per 32-bit operation.  `m` has 0xff in the bytes
+   * of a word that hold elements of the row (every RD_ES-th byte; none past
+   * the row's end; with RD_TAIL only those inside [sh, rin)).  Sum: a dot
+   * product of the word's four bytes with the 0/1 bytes of m & 0x01010101,
+   * accumulated in 32 bits over the unit (at most 8 loads x 16 bytes x 255).
+   * Any: the valid bytes or-ed together.  All: a zero among the valid bytes
+   * shows as (v - 0x01010101) & ~v & 0x80808080 with the other bytes forced
+   * to 0xff. */
+  (void)ib; (void)rml;
+  const ga_uint every = RD_ES == 1 ? 0xffffffffu : (RD_ES == 2 ? 0x00ff00ffu : 0x000000ffu);
+  ga_uint acc32 = 0;
+#pragma unroll
+  for (int j = 0; j < RD_U; j++) {
+    const ga_long e = e0 + (ga_long)j * LN * RD_VEC;
+#pragma unroll
+    for (int d = 0; d < RD_PV / 4; d++) {
+      const ga_uint wd = x.x0[j][d];   /* the unit keeps bytes packed in words */
+      ga_uint m = e < rin ? every : 0u;
+#if RD_TAIL
+      {   /* elements 4d .. 4d+3 of the load (RD_ES is 1 here) */
+        const ga_long first = e + 4 * d;
+        const ga_long lo = sh - first, hi = rin - first;   /* valid: lo <= byte < hi */
+        const ga_uint below = lo <= 0 ? 0u : (lo >= 4 ? 0xffffffffu : (1u << (8 * (int)lo)) - 1u);
+        const ga_uint upto = hi <= 0 ? 0u : (hi >= 4 ? 0xffffffffu : (1u << (8 * (int)hi)) - 1u);
+        m = upto & ~below;
+      }
+#endif
+#if RD_KIND == RD_K_SUM
+#if RD_FAST8 == 2
+      acc32 = (ga_uint)__builtin_amdgcn_sdot4((int)wd, (int)(m & 0x01010101u), (int)acc32, false);
+#else
+      acc32 = __builtin_amdgcn_udot4(wd, m & 0x01010101u, acc32, false);
+#endif
+#elif RD_KIND == RD_K_ANY
+      acc32 |= wd & m;
+#else
+      const ga_uint v = wd | ~m;
+      acc32 |= (v - 0x01010101u) & ~v & 0x80808080u;
+#endif
+    }
+  }
+  rd_acc r;
+#if RD_KIND == RD_K_SUM
+#if RD_FAST8 == 2
+  r.v = (RD_ACC_T)(ga_int)acc32;
+#else
+  r.v = (RD_ACC_T)acc32;
+#endif
+#elif RD_KIND == RD_K_ANY
+  r.v = acc32 != 0 ? 1 : 0;
+#else
+  r.v = acc32 == 0 ? 1 : 0;
 #endif
   return r;
 #else
@@ -999,7 +1056,10 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
         rd_store(a, sc, d0 + d0_off, d0o + c * p.fd0str[fi_d], d1 + d1_off,
                  d1o + c * p.fd1str[fi_d], p.rtotal RD_SCALAR_ARGS);
       } else {
-        rd_store_partial(a, part_v, part_i, row * p.nsplit + split);
+        /* with many outputs the partials lie split-major (adjacent lanes write
+         * adjacent slots, redux_final_cols reads them); else output-major */
+        rd_store_partial(a, part_v, part_i,
+                         p.split_major ? split * p.nrows + row : row * p.nsplit + split);
       }
     }
   }
@@ -1024,6 +1084,44 @@ redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_si
   }
   acc = rd_wave_reduce(acc);
   if (lane == 0) {
+    ga_long so[RD_NSRC], d0o, d1o;
+    rd_row_offsets(p, row, so, &d0o, &d1o);
+    const char *srow[RD_NSRC];
+    RD_SRC_BASES(srow);
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) srow[k] += so[k];
+    rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
+  }
+}
+
+/* The second pass after redux_col, whose partials lie split-major
+ * (slot = split * nrows + output): 64 adjacent outputs per group, lanes along
+ * the outputs so that every load of a wavefront is one contiguous run, the 4
+ * lane rows share the splits and meet in LDS. */
+KERNEL void __launch_bounds__(256)
+redux_final_cols(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
+                 RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
+  __shared__ rd_acc meet[4][64];
+  const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
+  const ga_long row = (ga_long)GID_0 * 64 + tx;
+  const bool live = row < p.nrows;
+  rd_acc acc = rd_neutral();
+  if (live) {
+    for (ga_long s = ty; s < p.nsplit; s += 4) {
+      rd_acc t;
+      t.v = part_v[s * p.nrows + row];
+#if RD_ARG
+      t.i = part_i[s * p.nrows + row];
+#endif
+      acc = rd_combine(acc, t);
+    }
+  }
+  meet[ty][tx] = acc;
+  local_barrier();
+  if (ty == 0 && live) {
+    acc = rd_combine(acc, meet[1][tx]);
+    acc = rd_combine(acc, meet[2][tx]);
+    acc = rd_combine(acc, meet[3][tx]);
     ga_long so[RD_NSRC], d0o, d1o;
     rd_row_offsets(p, row, so, &d0o, &d1o);
     const char *srow[RD_NSRC];

@@ -588,6 +588,56 @@ def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, monkeypatch):
                         assert val[r] == nanfn(view[r]) and idx[r] == argfn(view[r]), (name, n, r)
 
 
+@pytest.mark.parametrize("dtype", ["uint8", "int8", "bool"])
+def test_one_byte_elements_four_per_operation(ctx, dtype):
+    """sum / any / all over one-byte elements (combined a 32-bit word at a
+    time): extreme values, every alignment of start and end, stepped views,
+    long rows split over groups, rows sharing a wavefront."""
+    rng = np.random.default_rng(56)
+
+    def make(shape):
+        if dtype == "bool":
+            return rng.random(shape) < 0.5
+        info = np.iinfo(dtype)
+        h = rng.integers(info.min, info.max + 1, size=shape).astype(dtype)
+        h.reshape(-1)[::7] = info.max
+        h.reshape(-1)[3::11] = info.min
+        return h
+
+    def check(view, axes):
+        g, _ = to_gpu_view(view, ctx)
+        axes = tuple(axes)
+        want = view.sum(axis=axes, dtype=np.int64)
+        assert np.array_equal(np.asarray(R.sum(g, axis=axes, dtype="int64")), want)
+        if dtype != "int8":
+            assert np.array_equal(np.asarray(R.sum(g, axis=axes, dtype="uint32")), want.astype(np.uint32))
+        assert np.array_equal(np.asarray(R.any(g, axis=axes)), view.any(axis=axes))
+        assert np.array_equal(np.asarray(R.all(g, axis=axes)), view.all(axis=axes))
+
+    for shape in ((64, 8192), (300, 1000), (1000, 33), (513, 100), (7, 70001), (2000, 16), (3, 1 << 20)):
+        check(make(shape), [1])
+    flat = make((1 << 22) + 37)
+    for off, n in ((0, 1 << 22), (1, (1 << 22) + 3), (5, 1 << 21), (16, (1 << 22) - 15), (3, 100003)):
+        check(flat[off:off + n], [0])
+    base = make((256, 4096))
+    check(base[:, ::2], [1])
+    check(base[:, 1::4], [1])
+    check(base[:, 3:4001], [1])
+    check(base[::3, 5::2], [1])
+    # where any / all flip on a single element in every byte position of a word
+    for pos in range(0, 40):
+        z = np.zeros((4, 4099), dtype)
+        z[1, pos] = 1
+        z[2, 4098 - pos] = 1
+        o = np.ones((4, 4099), dtype)
+        o[1, pos] = 0
+        o[3, 4098 - pos] = 0
+        for h in (z, o, z[:, 1:], o[:, 2:4097]):
+            g, _ = to_gpu_view(h, ctx)
+            assert np.array_equal(np.asarray(R.any(g, axis=1)), h.any(axis=1)), pos
+            assert np.array_equal(np.asarray(R.all(g, axis=1)), h.all(axis=1)), pos
+
+
 @pytest.mark.parametrize("dtype", ["float32", "int32", "float64"])
 def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
     rng = np.random.default_rng(51)
