@@ -1043,10 +1043,15 @@ class reduction_call {
     // 64: sum 63 / 72 / 68 / 48 us with redux_wrows, 51 / 48 / 46 / 45 us
     // staged; maxandargmax 73 / 76 / 78 / 56 against 59 / 53 / 53 / 72 us
     // (its walk costs more per element, and 64 KiB of LDS per group leaves
-    // two groups per compute unit), hence the lower limit for min/max.
+    // two groups per compute unit), hence the lower limit for min/max.  Rows
+    // whose pitch is no multiple of 16 bytes cost redux_wrows a shifted,
+    // masked load pattern per row and stay here longer: 33 doubles (264
+    // bytes) sum / max 118 / 145 us there, 91 / 91 us staged; 40 doubles (320
+    // bytes, aligned) 89 / 100 against 95 / 121 us.
     if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] &&
         fsstr[0] == rin * elsz[0] && rin >= 2 &&
-        rin * elsz[0] <= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MAX_BYTES", minmax ? 160 : 256) &&
+        rin * elsz[0] <= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MAX_BYTES",
+                                         (rin * elsz[0]) % 16 != 0 ? 384 : (minmax ? 160 : 256)) &&
         rin * elsz[0] > (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_BYTES", 16) &&
         nrows >= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_ROWS", 512) * ncu &&
         GpuArray_ISALIGNED(srcs[0].a) && env_ul("GPUARRAY_REDUX_SROWS", 1)) {

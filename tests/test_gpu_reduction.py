@@ -511,8 +511,10 @@ def test_short_contiguous_rows_staged_in_lds(ctx, dtype, monkeypatch):
     monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")
     rng = np.random.default_rng(54)
     item = np.dtype(dtype).itemsize
-    lengths = [n for n in (2, 3, 5, 6, 7, 8, 12, 16, 17, 31, 32, 33, 48, 63, 64, 100, 128, 255, 256)
-               if 16 < n * item <= 256]
+    # up to 256 bytes per row, 384 where the row length is no multiple of 16 bytes
+    lengths = [n for n in (2, 3, 5, 6, 7, 8, 12, 16, 17, 31, 32, 33, 47, 48, 63, 64, 91, 100, 128, 181,
+                           255, 256, 333, 383)
+               if 16 < n * item <= (384 if (n * item) % 16 else 256)]
     for n in lengths:
         rows = int(rng.integers(300, 1500))
         flat = rng.integers(0, 12, size=rows * n + 7).astype(dtype)      # many ties
