@@ -640,7 +640,7 @@ def test_one_byte_elements_four_per_operation(ctx, dtype):
             assert np.array_equal(np.asarray(R.all(g, axis=1)), h.all(axis=1)), pos
 
 
-@pytest.mark.parametrize("dtype", ["float32", "int32", "float64"])
+@pytest.mark.parametrize("dtype", ["float32", "int32", "float64", "uint8", "int16"])
 def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
     rng = np.random.default_rng(51)
     for shape, axes in (((32, 16, 7, 7), (0, 2, 3)), ((16, 24, 16, 20), (1, 3)), ((9, 5, 3), (0, 2)),
@@ -652,10 +652,12 @@ def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
     _check_ops(ctx, host, (0, 2))
 
 
-@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float64", "float16"])
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "int8", "int16", "float64", "float16"])
 def test_several_outputs_per_lane(ctx, dtype):
     rng = np.random.default_rng(52)
-    for shape in ((300, 1000), (8, 4096), (1000, 256), (37, 20), (513, 772), (4, 64, 260)):
+    # (the 8192-wide cases have enough outputs for split-major partials)
+    for shape in ((300, 1000), (8, 4096), (1000, 256), (37, 20), (513, 772), (4, 64, 260), (2000, 8192),
+                  (5, 300, 4096)):
         host = rng.integers(0, 40, size=shape).astype(dtype)
         if dtype == "float16":
             g, _ = to_gpu_view(host, ctx)
