@@ -15,7 +15,7 @@ prints ONE JSON line:
                           own stream inside the timed region
   cpu_baseline            the CPU restatement of the reference's kernels
                           (oracle/, one host core) on a bounded sample
-  per_config              every BASELINE shape: GB/s, fraction of peak, us/call,
+  per_config              every configuration of the benchmark: GB/s, fraction of peak, us/call,
                           NumPy's time on the host next to it
 """
 import argparse
@@ -236,7 +236,7 @@ def host_time(fn, reps=3):
 
 
 def per_config(ctx, ga, R):
-    """Every BASELINE shape.  `cold` rotates over four buffer sets so that a
+    """Every configuration of the benchmark.  `cold` rotates over four buffer sets so that a
     footprint below the 256 MB Infinity Cache is not served from it; `warm`
     reuses one set."""
     res = {}
@@ -333,7 +333,7 @@ def per_config(ctx, ga, R):
               host_time(lambda: getattr(U[:, :, ::2], nm)(axis=2), reps=1), "useful bytes; stride-2 view")
     del gu, U
 
-    # Beyond the BASELINE shapes: an expression feeding a reduction in one pass
+    # Beyond the benchmark's own shapes: an expression feeding a reduction in one pass
     # (dot product of two 2^27 vectors; the two-pass alternative writes and
     # re-reads a 512 MiB temporary) and a row gather.
     n = 1 << 27

@@ -332,7 +332,7 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
 /* A use of a loaded value that no branch can skip.  The compiler waits for a
  * load where its result is first used; when every use sits under a branch that
  * some path skips, the result still counts as pending at the loop's back edge,
- * and in the next round each load of the unit waits for the one before it
+ * and in the next pass of the loop each load of the unit waits for the one before it
  * (their destination registers may be in flight) instead of all being issued
  * back to back.  Costs no instruction, but it makes the first use wait for
  * all of the unit's loads; redux_row leaves it out (RD_TOUCH_ROW 0) for sums

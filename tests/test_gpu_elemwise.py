@@ -1,7 +1,7 @@
 """GpuElemwise on the device, through the C ABI, against
   - the literal results of the reference's tests (tests/check_elemwise.c:39-880),
   - the CPU checker (oracle/) on seeded random layouts, bit for bit,
-  - NumPy at the BASELINE shapes.
+  - NumPy at the benchmark's shapes.
 Float expressions are compiled without contraction, so a*b+c is two roundings
 and results are bit-identical to the checker and to NumPy."""
 import ctypes as C
@@ -352,7 +352,7 @@ def test_zero_dimensional_and_size_one(ctx):
     assert np.asarray(c3).ravel()[0] == np.float32(6.5)
 
 
-# ---- BASELINE shapes -----------------------------------------------------------------
+# ---- the benchmark's shapes -----------------------------------------------------------------
 
 def test_config1_contiguous_2p24(ctx, oracle):
     rng = np.random.default_rng(0)

@@ -375,7 +375,7 @@ def test_sum_is_reproducible_run_to_run(ctx):
         assert np.asarray(R.sum(g)).tobytes() == first
 
 
-# ---- BASELINE shapes at full size -----------------------------------------------------
+# ---- the benchmark's shapes at full size -----------------------------------------------------
 
 def test_config3a_sum_axis1_8192(ctx, oracle):
     rng = np.random.default_rng(2)
