@@ -9,6 +9,7 @@ _CTYPES = {"bool": "ga_bool", "int8": "ga_byte", "uint8": "ga_ubyte", "int16": "
 
 
 _REGISTERED = {}     # dtype -> C name, for element types added with register_dtype
+_BY_DTYPE = {}       # dtype object -> C name of a built-in type (dtype.name is slow to form)
 NAME_TO_DTYPE = {}   # C spelling -> dtype, for parsing C argument lists
 
 
@@ -16,11 +17,16 @@ def dtype_to_ctype(dtype):
     """reference pygpu/dtypes.py:78-93 (the cluda spelling of a dtype)"""
     if dtype is None:
         raise ValueError("dtype may not be None")
+    try:
+        return _BY_DTYPE[dtype]        # the common case: a dtype object seen before
+    except (KeyError, TypeError):
+        pass
     dtype = np.dtype(dtype)
     if dtype in _REGISTERED:
         return _REGISTERED[dtype]
     try:
-        return _CTYPES[dtype.name]
+        res = _BY_DTYPE[dtype] = _CTYPES[dtype.name]
+        return res
     except KeyError:
         raise ValueError("unable to map dtype: %s" % (dtype,))
 

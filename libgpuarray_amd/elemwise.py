@@ -117,13 +117,44 @@ def as_argument(o, name, read=False, write=False):
     return arg(name, _dtype(o), scalar=not isinstance(o, GpuArray), read=read, write=write)
 
 
+def _kernel(context, oper, args, convert_f16):
+    """The GpuElemwise for an expression and argument signature, built once per
+    context: the helpers below are called per operation (every `a + b` of an
+    ndgpuarray), and building the C object costs several times a launch."""
+    cache = context.__dict__.setdefault("_elemwise_cache", {})
+    key = (oper, convert_f16, tuple((x.name, x.dtype.str, x.flags) for x in args))
+    k = cache.get(key)
+    if k is None:
+        if len(cache) >= 512:
+            cache.clear()
+        k = cache[key] = GpuElemwise(context, oper, args, convert_f16=convert_f16)
+    return k
+
+
+_common = {}
+
+
+def _common_dtype(a, b):
+    """get_common_dtype(a, b, True), remembered per pair of (dtype | Python scalar type)."""
+    ka = a.dtype if hasattr(a, "dtype") else type(a)
+    kb = b.dtype if hasattr(b, "dtype") else type(b)
+    try:
+        return _common[(ka, kb)]
+    except KeyError:
+        res = get_common_dtype(a, b, True)
+        if ka in (int, float, bool, complex) or hasattr(a, "dtype"):
+            if kb in (int, float, bool, complex) or hasattr(b, "dtype"):
+                _common[(ka, kb)] = res
+        return res
+
+
 def elemwise1(a, op, oper=None, op_tmpl="res = %(op)sa", out=None, convert_f16=True):
     """Unary op into a new (or given) array (reference pygpu/elemwise.py:24-39)."""
     args = (as_argument(a, "res", write=True), as_argument(a, "a", read=True))
     res = a._empty_like_me() if out is None else out
     if oper is None:
         oper = op_tmpl % {"op": op}
-    k = GpuElemwise(a.context, oper, args, convert_f16=convert_f16)
+    k = _kernel(a.context, oper, args, convert_f16)
     k(res, a)
     return res
 
@@ -144,7 +175,7 @@ def elemwise2(a, op, b, ary, odtype=None, oper=None,
     else:
         b_np = b
     if odtype is None:
-        odtype = get_common_dtype(a_np, b_np, True)
+        odtype = _common_dtype(a_np, b_np)
     odtype = np.dtype(odtype)
     args = [arg("res", odtype, write=True), as_argument(a, "a", read=True),
             as_argument(b, "b", read=True)]
@@ -164,7 +195,7 @@ def elemwise2(a, op, b, ary, odtype=None, oper=None,
         if convert_f16 and ot == np.dtype("float16"):
             ot = np.dtype("float32")
         oper = op_tmpl % {"op": op, "out_t": dtype_to_ctype(ot)}
-    k = GpuElemwise(ary.context, oper, args, convert_f16=convert_f16)
+    k = _kernel(ary.context, oper, args, convert_f16)
     k(res, a, b, broadcast=broadcast)
     return res
 
@@ -176,7 +207,7 @@ def ielemwise2(a, op, b, oper=None, op_tmpl="a = a %(op)s b", broadcast=False, c
     args = [as_argument(a, "a", read=True, write=True), as_argument(b, "b", read=True)]
     if oper is None:
         oper = op_tmpl % {"op": op}
-    k = GpuElemwise(a.context, oper, args, convert_f16=convert_f16)
+    k = _kernel(a.context, oper, args, convert_f16)
     k(a, b, broadcast=broadcast)
     return a
 

@@ -31,6 +31,10 @@ _DTYPES = {v: k for k, v in _TYPECODES.items()}
 
 def dtype_to_typecode(dtype):
     try:
+        return _TYPECODES[dtype]          # a dtype object: the common case
+    except (KeyError, TypeError):
+        pass
+    try:
         return _TYPECODES[np.dtype(dtype)]
     except KeyError:
         raise ValueError("don't know how to convert to dtype: %s" % (dtype,))
@@ -647,6 +651,11 @@ class GpuArray(object):
         return "gpuarray." + repr(np.asarray(self))
 
 
+_DIM_ARRAYS = {}     # rank -> ctypes array type of that many extents
+_ORDERS = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER,
+           "c": _lib.GA_C_ORDER, "f": _lib.GA_F_ORDER, "a": _lib.GA_ANY_ORDER}
+
+
 def _make(cls, context):
     return (cls or GpuArray)(context)
 
@@ -655,12 +664,15 @@ def empty(shape, dtype="float32", order="C", context=None, cls=None):
     ctx = _ensure_context(context)
     if isinstance(shape, (int, np.integer)):
         shape = (int(shape),)
-    shape = tuple(int(d) for d in shape)
     res = _make(cls, ctx)
-    dims = (C.c_size_t * max(len(shape), 1))(*shape)
-    o = {"C": _lib.GA_C_ORDER, "F": _lib.GA_F_ORDER, "A": _lib.GA_ANY_ORDER}[order.upper()]
-    check(lib.GpuArray_empty(res._ptr(), ctx.ctx, dtype_to_typecode(dtype), len(shape), dims, o),
-          ctx.ctx)
+    nd = len(shape)
+    dims = _DIM_ARRAYS.get(nd)
+    if dims is None:
+        dims = _DIM_ARRAYS[nd] = C.c_size_t * max(nd, 1)
+    err = lib.GpuArray_empty(res._ref, ctx.ctx, dtype_to_typecode(dtype), nd, dims(*shape),
+                             _ORDERS[order])
+    if err:
+        check(err, ctx.ctx)
     return res
 
 
