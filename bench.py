@@ -228,6 +228,19 @@ def time_calls(ctx, fn, iters=30, warm=5):
     return float(np.median(ms)) * 1e3   # microseconds
 
 
+def time_stream(ctx, fn, iters=40, warm=5):
+    """Microseconds per call when the calls are issued back to back: two marks
+    around all of them, so that launches overlap the kernels before them."""
+    for _ in range(warm):
+        fn(0)
+    ctx.sync()
+    ctx.mark(0)
+    for i in range(iters):
+        fn(i)
+    ctx.mark(1)
+    return ctx.elapsed(0, 1) * 1e3 / iters
+
+
 def host_time(fn, reps=3):
     t0 = time.perf_counter()
     for _ in range(reps):
@@ -242,12 +255,15 @@ def per_config(ctx, ga, R):
     res = {}
     rot = 4
 
-    def entry(name, nbytes, us_cold, us_warm, numpy_us, note=None):
+    def entry(name, nbytes, us_cold, us_warm, numpy_us, note=None, us_stream=None):
         e = {"algorithmic_bytes": nbytes, "us_per_call_cold": round(us_cold, 2),
              "GBps_cold": round(nbytes / us_cold / 1e3, 1),
              "frac_cold": round(nbytes / us_cold / 1e3 / HBM_PEAK_GBS, 4),
              "us_per_call_warm": round(us_warm, 2), "GBps_warm": round(nbytes / us_warm / 1e3, 1),
              "numpy_us_per_call": round(numpy_us, 1), "numpy_cores": 1}
+        if us_stream is not None:     # cold buffers, calls issued back to back
+            e["us_per_call_back_to_back"] = round(us_stream, 2)
+            e["GBps_back_to_back"] = round(nbytes / us_stream / 1e3, 1)
         if note:
             e["note"] = note
         res[name] = e
@@ -264,9 +280,11 @@ def per_config(ctx, ga, R):
             for _ in range(rot)]
     cold = time_calls(ctx, lambda i: elem(*sets[i % rot]))
     warm = time_calls(ctx, lambda i: elem(*sets[0]))
+    b2b = time_stream(ctx, lambda i: elem(*sets[i % rot]))
     c_h = np.empty_like(a_h)
     entry("C1_elemwise_2^24", 12 * n, cold, warm,
-          host_time(lambda: np.add(np.multiply(a_h, b_h, out=c_h), np.float32(0.5), out=c_h)))
+          host_time(lambda: np.add(np.multiply(a_h, b_h, out=c_h), np.float32(0.5), out=c_h)),
+          us_stream=b2b)
     del sets
 
     # C2: transposed view + two broadcast operands
@@ -280,8 +298,9 @@ def per_config(ctx, ga, R):
              ga.empty((4096, 4096), f32, context=ctx)) for _ in range(rot)]
     cold = time_calls(ctx, lambda i: k2(*sets[i % rot]))
     warm = time_calls(ctx, lambda i: k2(*sets[0]))
+    b2b = time_stream(ctx, lambda i: k2(*sets[i % rot]))
     entry("C2_transposed_broadcast_4096", 2 * 4096 * 4096 * 4 + 2 * 4096 * 4, cold, warm,
-          host_time(lambda: A.T + B * Cc))
+          host_time(lambda: A.T + B * Cc), us_stream=b2b)
     del sets
 
     # C3a: sum over axis 1 of (8192, 8192)
@@ -290,7 +309,9 @@ def per_config(ctx, ga, R):
     sets = [(ga.array(X, context=ctx), ga.empty((8192,), f32, context=ctx)) for _ in range(rot)]
     cold = time_calls(ctx, lambda i: op(sets[i % rot][0], [1], d0=sets[i % rot][1]))
     warm = time_calls(ctx, lambda i: op(sets[0][0], [1], d0=sets[0][1]))
-    entry("C3a_sum_axis1_8192x8192", 8192 * 8192 * 4 + 8192 * 4, cold, warm, host_time(lambda: X.sum(axis=1)))
+    b2b = time_stream(ctx, lambda i: op(sets[i % rot][0], [1], d0=sets[i % rot][1]))
+    entry("C3a_sum_axis1_8192x8192", 8192 * 8192 * 4 + 8192 * 4, cold, warm, host_time(lambda: X.sum(axis=1)),
+          us_stream=b2b)
     del sets
 
     # C4: maxandargmax over the last axis of (65536, 1000)
@@ -300,8 +321,9 @@ def per_config(ctx, ga, R):
              ga.empty((65536,), "int64", context=ctx)) for _ in range(rot)]
     cold = time_calls(ctx, lambda i: op4(sets[i % rot][0], [1], d0=sets[i % rot][1], d1=sets[i % rot][2]))
     warm = time_calls(ctx, lambda i: op4(sets[0][0], [1], d0=sets[0][1], d1=sets[0][2]))
+    b2b = time_stream(ctx, lambda i: op4(sets[i % rot][0], [1], d0=sets[i % rot][1], d1=sets[i % rot][2]))
     entry("C4_maxandargmax_65536x1000", 65536 * 1000 * 4 + 65536 * 12, cold, warm,
-          host_time(lambda: (L.max(axis=1), L.argmax(axis=1))))
+          host_time(lambda: (L.max(axis=1), L.argmax(axis=1))), us_stream=b2b)
     del sets, L, X, A
 
     # C5: stride-2 view of (256, 512, 1024); at most half of every fetched line is useful
