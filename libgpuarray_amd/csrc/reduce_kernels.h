@@ -34,7 +34,7 @@
  *               the RD_G lanes when the inner reduced dim is short (1: none)
  *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
  *   RD_CY       redux_col: lane rows of a group that share the reduced range
- *               (4, 2 or 1); 256 / RD_CY lanes lie along the free dim
+ *               (a power of two up to 16); 256 / RD_CY lanes lie along the free dim
  *   RD_L        redux_wrows: lanes that share a row (power of two, <= 64);
  *               64 / RD_L rows sit side by side in a wavefront
  *   RD_RB       redux_wrows: sets of rows whose loads a wavefront issues together

@@ -655,9 +655,10 @@ def test_short_inner_dim_with_outer_reduced_dims(ctx, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "int8", "int16", "float64", "float16"])
 def test_several_outputs_per_lane(ctx, dtype):
     rng = np.random.default_rng(52)
-    # (the 8192-wide cases have enough outputs for split-major partials)
+    # (the 8192-wide cases have enough outputs for split-major partials; the narrow ones
+    # take 8 or 16 lane rows)
     for shape in ((300, 1000), (8, 4096), (1000, 256), (37, 20), (513, 772), (4, 64, 260), (2000, 8192),
-                  (5, 300, 4096)):
+                  (5, 300, 4096), (3000, 64), (7, 1500, 32), (1201, 16), (900, 8), (4000, 100)):
         host = rng.integers(0, 40, size=shape).astype(dtype)
         if dtype == "float16":
             g, _ = to_gpu_view(host, ctx)
