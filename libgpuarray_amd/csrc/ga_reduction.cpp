@@ -1077,8 +1077,15 @@ class reduction_call {
   void col_geometry() {
     const int64_t fin = p.fdim[p.nf - 1];
     const unsigned long cy_forced = env_ul("GPUARRAY_REDUX_COL_ROWS", 0);
+    // Lane rows of a group: 8 (32 lanes along the free dim) when the reduced
+    // range is long, else 4.  Measured on MI355X with 4 / 8 / 16: per-channel
+    // sum of (64, 56, 56, 256) floats 45.2 / 40.9 / 39.7 us, max over the
+    // channels of (64, 256, 56, 56) 49.7 / 44.1 / 47.1, sum over axis 0 of
+    // 8192 x 8192 50.9 / 49.4 / 51.4, over the middle axis of 256 x 512 x 512
+    // 47.0 / 43.8 / 47.5; but 8 x 2^23 over axis 0 49.3 / 72.4 / 121 and
+    // 256 x 2^18 45.8 / 48.2 / 47.2.
     CY = (cy_forced == 1 || cy_forced == 2 || cy_forced == 4 || cy_forced == 8 || cy_forced == 16)
-             ? (unsigned)cy_forced : 4;
+             ? (unsigned)cy_forced : (rtotal >= 512 ? 8 : 4);
     int64_t CX = 256 / CY;   // lanes along the free dim
     // Adjacent outputs per lane: as many as one 16-byte load of the widest
     // source holds, when the inner free dim is contiguous in every source and
