@@ -42,6 +42,7 @@ struct rd_plan {
   int64_t rdim[RD_MAXD], rmul[RD_MAXD];
   int64_t nrows, rtotal, nseg, units, upb, gx, router;
   int32_t nf, nr, nsplit, split_major;
+  int32_t rising, reserved;
 };
 
 enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL, K_ANY, K_CUSTOM };
@@ -179,7 +180,7 @@ struct variant_spec {
   unsigned L;         // redux_wrows: lanes per row
   unsigned CV;        // redux_col: adjacent outputs per lane
   unsigned LO;        // redux_row: outer reduced coordinates side by side
-  unsigned CY = 4;    // redux_col: lane rows of a group (4, 2 or 1), 256 / CY lanes along the free dim
+  unsigned CY = 4;    // redux_col: lane rows of a group (1 to 16), 256 / CY lanes along the free dim
 };
 
 const char *load_type_name(int tc) {
@@ -800,6 +801,15 @@ class reduction_call {
     p.nrows = nrows;
     p.rtotal = rtotal;
     p.nsplit = 1;
+    // Does the flattened index grow with the position in the reduced range
+    // (dims slowest first)?  Then a scan in that order meets equal values
+    // lowest index first.
+    p.rising = rtotal < 0x7fffffff ? 1 : 0;
+    for (int i = 0; i + 1 < p.nr; i++)
+      if (p.rmul[i] < p.rdim[i + 1] * p.rmul[i + 1]) p.rising = 0;
+    for (int i = 0; i < p.nr; i++)
+      if (p.rmul[i] <= 0) p.rising = 0;
+    p.reserved = 0;
 
     elsz_max = elsz_sum = 0;
     elsz.assign(K, 0);
@@ -1092,7 +1102,7 @@ class reduction_call {
     // every address a lane forms is a multiple of its load.
     {
       unsigned cv = (unsigned)(16 / elsz_max);
-      if (info.has_d1 && cv > 4) cv = 4;
+      if (info.has_d1 && cv > 8) cv = 8;   // (value, index) pairs meet in LDS: 32 KiB per group at 8
       if (cv > (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16)) cv = (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16);
       for (unsigned q = 0; q < K; q++)
         if (fsstr[q * RD_MAXD + p.nf - 1] != elsz[q]) cv = 1;

@@ -107,6 +107,8 @@ struct rd_plan {
   ga_long gx;      /* redux_col: groups along the inner free dim */
   ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates */
   ga_int nf, nr, nsplit, split_major;   /* split_major: layout of redux_col's partials */
+  ga_int rising, reserved;   /* rising: the flattened index grows with the position in the
+                              * reduced range, and the range has fewer than 2^31 positions */
   ga_long fsstr[RD_NSRC][RD_MAXD], rsstr[RD_NSRC][RD_MAXD];   /* per source */
 };
 
@@ -949,6 +951,73 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 }
 #endif
 
+/* ---- helpers of redux_col ------------------------------------------------- */
+
+/* Position j of the flattened reduced range: byte offset in every source and
+ * flattened index in the caller's axis order.  32-bit divisions when the
+ * range allows it. */
+static __device__ inline void rd_col_at(const rd_plan &p, const ga_long j, ga_long *off, ga_long *ix) {
+  if (p.nr == 1) {
+#pragma unroll
+    for (int k = 0; k < RD_NSRC; k++) off[k] = j * p.rsstr[k][0];
+    *ix = j * p.rmul[0];
+    return;
+  }
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) off[k] = 0;
+  *ix = 0;
+  if (p.rtotal <= 0x7fffffffLL) {
+    ga_uint r = (ga_uint)j;
+    for (int d = p.nr - 1; d >= 0; d--) {
+      ga_uint c = r;
+      if (d > 0) {
+        const ga_uint n = (ga_uint)p.rdim[d];
+        const ga_uint qd = r / n;
+        c = r - qd * n;
+        r = qd;
+      }
+#pragma unroll
+      for (int k = 0; k < RD_NSRC; k++) off[k] += (ga_long)c * p.rsstr[k][d];
+      *ix += (ga_long)c * p.rmul[d];
+    }
+  } else {
+    ga_long r = j;
+    for (int d = p.nr - 1; d >= 0; d--) {
+      ga_long c = r;
+      if (d > 0) { c = r % p.rdim[d]; r = r / p.rdim[d]; }
+#pragma unroll
+      for (int k = 0; k < RD_NSRC; k++) off[k] += c * p.rsstr[k][d];
+      *ix += c * p.rmul[d];
+    }
+  }
+}
+
+static __device__ inline ga_long rd_col_index(const rd_plan &p, const ga_long j) {
+  ga_long off[RD_NSRC], ix;
+  rd_col_at(p, j, off, &ix);
+  return ix;
+}
+
+/* A lane's RD_CV adjacent elements at position j of the reduced range. */
+static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *srow, const ga_long j,
+                                           rd_cvec &x) {
+  ga_long off[RD_NSRC], ix;
+  rd_col_at(p, j, off, &ix);
+  const char *ep[RD_NSRC];
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) ep[k] = srow[k] + off[k];
+  rd_cvec_load(x, ep);
+}
+
+/* Arg-min/max and floating min/max scan a lane's elements in rising order
+ * with a strict compare when the plan says the index rises with them. */
+#define RD_COL_SCAN (RD_ARG && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN))
+#if RD_KIND == RD_K_MAX
+#define RD_COL_BETTER(a, b) ((a) > (b))
+#else
+#define RD_COL_BETTER(a, b) ((a) < (b))
+#endif
+
 #define RD_CX (256 / RD_CY)   /* lanes along the free dim; RD_CY lane rows share the reduced range */
 
 /* ---- redux_col -------------------------------------------------------------
@@ -1000,38 +1069,81 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   rd_acc acc[RD_CV];
 #pragma unroll
   for (int c = 0; c < RD_CV; c++) acc[c] = rd_neutral();
+#if RD_COL_SCAN
+  if (live && p.rising) {
+    /* The index grows with j and j fits 31 bits: a lane meets its elements in
+     * rising order, so a strict compare keeps the first of equals, and what
+     * it carries per output is the value and a 32-bit j. */
+    RD_ACC_T bv[RD_CV];
+    ga_int bj[RD_CV];
+#pragma unroll
+    for (int c = 0; c < RD_CV; c++) { bv[c] = RD_NEUTRAL; bj[c] = 0x7fffffff; }
+    ga_long j0 = r0 + ty;
+#if RD_U > 1
+    for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
+      rd_cvec x[RD_U];
+#pragma unroll
+      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+#pragma unroll
+      for (int q = 0; q < RD_U; q++) {
+#pragma unroll
+        for (int c = 0; c < RD_CV; c++) {
+          const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x[q], c), 0).v;
+          const bool better = RD_COL_BETTER(val, bv[c]);
+          bv[c] = better ? val : bv[c];
+          bj[c] = better ? (ga_int)(j0 + RD_CY * q) : bj[c];
+        }
+      }
+    }
+#endif
+    for (; j0 < r1; j0 += RD_CY) {
+      rd_cvec x;
+      rd_col_fetch(p, srow, j0, x);
+#pragma unroll
+      for (int c = 0; c < RD_CV; c++) {
+        const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x, c), 0).v;
+        const bool better = RD_COL_BETTER(val, bv[c]);
+        bv[c] = better ? val : bv[c];
+        bj[c] = better ? (ga_int)j0 : bj[c];
+      }
+    }
+    if (r0 + ty < r1) {
+#pragma unroll
+      for (int c = 0; c < RD_CV; c++) {
+        /* nothing beat the neutral value: every element equals it, the first stays */
+        const ga_long j = bj[c] == 0x7fffffff ? r0 + ty : (ga_long)bj[c];
+        acc[c].v = bv[c];
+        acc[c].i = rd_col_index(p, j);
+      }
+    }
+  } else
+#endif
   if (live) {
-    for (ga_long j0 = r0 + ty; j0 < r1; j0 += RD_CY * RD_U) {
+    ga_long j0 = r0 + ty;
+#if RD_U > 1
+    /* all RD_U loads of a batch lie inside the range: no test per load */
+    for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
       ga_long idx[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
-        const ga_long j = j0 + RD_CY * q;
-        if (j < r1) {
-          ga_long off[RD_NSRC], ix = 0, r = j;
-#pragma unroll
-          for (int k = 0; k < RD_NSRC; k++) off[k] = 0;
-          for (int d = p.nr - 1; d >= 0; d--) {
-            ga_long c;
-            if (d > 0) { c = r % p.rdim[d]; r = r / p.rdim[d]; } else { c = r; }
-#pragma unroll
-            for (int k = 0; k < RD_NSRC; k++) off[k] += c * p.rsstr[k][d];
-            ix += c * p.rmul[d];
-          }
-          const char *ep[RD_NSRC];
-#pragma unroll
-          for (int k = 0; k < RD_NSRC; k++) ep[k] = srow[k] + off[k];
-          rd_cvec_load(x[q], ep);
-          idx[q] = ix;
-        }
+        rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+        idx[q] = RD_ARG ? rd_col_index(p, j0 + RD_CY * q) : 0;
       }
 #pragma unroll
-      for (int q = 0; q < RD_U; q++)
-        if (j0 + RD_CY * q < r1) {
+      for (int q = 0; q < RD_U; q++) {
 #pragma unroll
-          for (int c = 0; c < RD_CV; c++)
-            acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
-        }
+        for (int c = 0; c < RD_CV; c++)
+          acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
+      }
+    }
+#endif
+    for (; j0 < r1; j0 += RD_CY) {
+      rd_cvec x;
+      rd_col_fetch(p, srow, j0, x);
+      const ga_long idx = RD_ARG ? rd_col_index(p, j0) : 0;
+#pragma unroll
+      for (int c = 0; c < RD_CV; c++) acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x, c), idx));
     }
   }
 #if RD_CY > 1

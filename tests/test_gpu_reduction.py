@@ -697,3 +697,57 @@ def test_ragged_and_misaligned_rows_take_vector_loads(ctx, dtype):
     flat = rng.integers(0, 40, size=(1 << 22) + 5).astype(dtype if dtype != "float16" else "float32")
     _check_ops(ctx, flat[1:], [0])              # split over many groups, ragged end
     _check_ops(ctx, flat[3:-1], [0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "float16", "int8", "uint8", "int16", "int32", "int64"])
+def test_column_scans_keep_the_first_of_equals(ctx, dtype):
+    """Arg-min/max (and floating min/max) with lanes along the free dim: a lane
+    scans its share of the reduced range in rising order with a strict compare
+    when the index rises along the scan, else with the index compare.  Columns
+    that hold only the scan's starting value (type minimum / maximum, -inf /
+    +inf), ties within a lane and between lanes and splits, NaN after the
+    first position, signed zeros; reduced ranges of one dim, of two dims in
+    index order, and of two dims whose memory order is not the index order."""
+    rng = np.random.default_rng(77)
+    dt = np.dtype(dtype)
+    lo, hi = ((-np.inf, np.inf) if dt.kind == "f" else (np.iinfo(dt).min, np.iinfo(dt).max))
+    for shape, axes in (((700, 96), (0,)), ((5000, 256), (0,)), ((9, 130, 64), (0, 1)),
+                        ((40, 2, 33, 128), (0, 2)), ((64, 8192), (0,)), ((2100, 8), (0,))):
+        host = rng.integers(0, 3, size=shape).astype(dt)                  # ties everywhere
+        cols = host.reshape(-1, shape[-1])
+        cols[:, 0] = lo                                                   # only the starting value of a max scan
+        cols[:, 1] = hi                                                   # ... of a min scan
+        cols[:, 2] = lo; cols[cols.shape[0] // 2:, 2] = hi
+        cols[:, 3] = hi; cols[cols.shape[0] // 3, 3] = lo
+        if dt.kind == "f":
+            cols[5, 4] = np.nan                                           # not first: passed over
+            cols[0, 5] = np.nan                                           # first: stays
+            cols[:, 6] = -0.0; cols[cols.shape[0] - 2, 6] = 0.0           # equal zeros
+            cols[:, 7] = 0.0; cols[3, 7] = -0.0
+        views = [host]
+        if len(axes) == 2:
+            # the same values with the two reduced dims swapped in memory: the scan no
+            # longer meets the elements in index order
+            order = list(range(host.ndim))
+            order[axes[0]], order[axes[1]] = order[axes[1]], order[axes[0]]
+            views.append(np.ascontiguousarray(host.transpose(order)).transpose(order))
+        for v in views:
+            g, _ = to_gpu_view(v, ctx)
+            moved = np.moveaxis(v, axes, range(v.ndim - len(axes), v.ndim))
+            flat = moved.reshape(moved.shape[:v.ndim - len(axes)] + (-1,))
+            for name, better in (("maxandargmax", np.greater), ("minandargmin", np.less)):
+                # sequential scan with a strict compare, as the reference's kernel does it
+                want_v = flat[..., 0].copy()
+                want_i = np.zeros(flat.shape[:-1], np.int64)
+                for j in range(1, flat.shape[-1]):
+                    b = better(flat[..., j], want_v)
+                    want_v = np.where(b, flat[..., j], want_v)
+                    want_i = np.where(b, j, want_i)
+                val, idx = getattr(R, name)(g, axis=axes)
+                assert np.array_equal(np.asarray(idx), want_i), (name, shape, axes, v.strides)
+                got = np.asarray(val)
+                bits = "u%d" % dt.itemsize
+                assert np.array_equal(got.view(bits), want_v.astype(dt).view(bits)), (name, shape, axes)
+                if dt.kind == "f":
+                    plain = np.asarray(getattr(R, name[:3])(g, axis=axes))
+                    assert np.array_equal(plain.view(bits), want_v.astype(dt).view(bits)), (name[:3], shape)
