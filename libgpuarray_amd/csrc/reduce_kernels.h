@@ -65,17 +65,21 @@
  *     inside a unit, then the cross-lane network below), so results are
  *     reproducible run to run.
  *
- * Four kernels:
+ * The kernels:
  *   redux_row    lanes run along the fastest REDUCED dim; RD_G lanes
  *                cooperate on one output; a row can be cut in `nsplit` pieces
  *                that each leave a partial.
  *   redux_wrows  the same for short rows (one pass of a wavefront covers a
  *                row): a wavefront takes several rows at a time and issues all
  *                their loads before it combines the first.
- *   redux_col    lanes run along the fastest FREE dim (coalesced), each lane
- *                owns one output and walks the reduced range; 4 lane rows
- *                share the range and meet in LDS.
- *   redux_final  second pass: combines the partials of one output.
+ *   redux_srows  many short contiguous rows: a group copies its rows to LDS
+ *                with full-width loads and each lane then walks one row.
+ *   redux_col    lanes run along the fastest FREE dim (coalesced), a lane owns
+ *                RD_CV adjacent outputs and walks the reduced range; RD_CY
+ *                lane rows share the range and meet in LDS.
+ *   redux_final, redux_final_cols  second pass: combine the partials of an
+ *                output (a wavefront per output; or lanes along the outputs
+ *                when the partials lie split-major).
  */
 #include "cluda.h"
 
