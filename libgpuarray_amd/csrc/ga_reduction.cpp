@@ -249,6 +249,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
+  DEF("#define RD_WANT %u\n", (vs.opts >> 4) & 3u);
   DEF("#define RD_CY %u\n", vs.CY ? vs.CY : 4u);
   {
     // One-byte elements under sum / any / all with an integer accumulator:
@@ -458,14 +459,22 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   for (int t : flag_types) kflags |= gpuarray_type_flags(t, -1);
   const unsigned na = (unsigned)types.size();
   variant v;
-  const char *names[5] = {"redux_row", "redux_col", "redux_final", "redux_final_cols", "redux_wrows"};
-  GpuKernel *ks[5] = {&v.row, &v.col, &v.fin, &v.fin_cols, &v.wrows};
-  int nk = vs.G == 64 ? 5 : 4;
-  if (vs.opts & 8u) {
-    names[0] = "redux_srows";
-    ks[0] = &v.srows;
-    nk = 1;
+  // the text holds the kernels of one family only (opts bits 4 and 5): a
+  // variant is compiled when its first call needs it, and that call waits
+  const char *names[6];
+  GpuKernel *ks[6];
+  int nk = 0;
+  auto want = [&](const char *name, GpuKernel *k) { names[nk] = name; ks[nk++] = k; };
+  if (vs.opts & 8u) want("redux_srows", &v.srows);
+  if (vs.opts & 16u) {
+    want("redux_row", &v.row);
+    if (vs.G == 64) want("redux_wrows", &v.wrows);
   }
+  if (vs.opts & 32u) {
+    want("redux_col", &v.col);
+    want("redux_final_cols", &v.fin_cols);
+  }
+  if (vs.opts & 48u) want("redux_final", &v.fin);
   for (int i = 0; i < nk; i++) {
     err = GpuKernel_init(ks[i], ctx, 1, strs, lens, names[i], na, types.data(), kflags, nullptr);
     if (err != GA_NO_ERROR) {
@@ -1185,6 +1194,7 @@ class reduction_call {
                        use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
                        (use_row && !wrows) ? LO : 1};
     if (!use_row) vs.CY = CY;
+    vs.opts |= use_row ? 16u : 32u;   // bits 4, 5: the family of kernels the text holds
     if (srows)   // one kernel, independent of the lane geometry
       vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
     return get_variant(gr, vs, &var);
@@ -1267,7 +1277,7 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   std::string s;
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
-                         (((U >> 25) & 1u) ? 8u : 0u), ES, 1,
+                         (((U >> 25) & 1u) ? 8u : 0u) | 48u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};
@@ -1287,7 +1297,7 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3, 1, vecmask, 1, 64, 1, 1};
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3 | 48u, 1, vecmask, 1, 64, 1, 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

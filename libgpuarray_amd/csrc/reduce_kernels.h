@@ -24,6 +24,9 @@
  *   RD_FAST8    one-byte elements combined four per 32-bit operation (sum, any,
  *               all; 1: unsigned bytes, 2: signed), 0: off
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
+ *   RD_WANT     which kernels the text holds: bit 0 the row family (redux_row,
+ *               redux_wrows), bit 1 the column family (redux_col,
+ *               redux_final_cols); redux_final with either
  *   RD_TAIL     rows that are misaligned for the vector load or whose extent
  *               is not a multiple of RD_VEC (one source, contiguous rows): a
  *               row is read from the vector boundary at or below its start,
@@ -597,6 +600,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
 #endif
 }
 
+#if RD_WANT & 1   /* the row family: redux_row, redux_wrows */
 KERNEL void __launch_bounds__(256)
 redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
           const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
@@ -844,6 +848,8 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 #endif
 #endif
 
+#endif   /* RD_WANT & 1 */
+
 #if RD_SROWS
 /* ---- redux_srows -----------------------------------------------------------
  * Rows of a few dozen elements, one after the other in memory (one source,
@@ -1024,6 +1030,7 @@ static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *
 
 #define RD_CX (256 / RD_CY)   /* lanes along the free dim; RD_CY lane rows share the reduced range */
 
+#if RD_WANT & 2   /* the column family: redux_col, redux_final_cols */
 /* ---- redux_col -------------------------------------------------------------
  * Lanes along the fastest free dim; a lane owns RD_CV adjacent outputs and
  * fetches them with one load (RD_CV > 1 needs that dim to be contiguous in
@@ -1181,6 +1188,9 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   }
 }
 
+#endif   /* RD_WANT & 2 */
+
+#if RD_WANT & 3
 /* ---- redux_final ------------------------------------------------------------
  * One wavefront per output: combine its nsplit partials and write the result. */
 KERNEL void __launch_bounds__(256)
@@ -1210,6 +1220,9 @@ redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_si
   }
 }
 
+#endif   /* RD_WANT & 3 */
+
+#if RD_WANT & 2
 /* The second pass after redux_col, whose partials lie split-major
  * (slot = split * nrows + output): 64 adjacent outputs per group, lanes along
  * the outputs so that every load of a wavefront is one contiguous run, the 4
@@ -1247,3 +1260,4 @@ redux_final_cols(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const 
     rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
   }
 }
+#endif   /* RD_WANT & 2 */
