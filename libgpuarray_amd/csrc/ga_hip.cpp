@@ -287,6 +287,7 @@ struct hip_context : _gpucontext {
   size_t live_modules = 0;   // loaded code objects, cached or still referenced
   gpudata *scratch = nullptr;
   size_t scratch_sz = 0;
+  gpudata *redux_counters = nullptr;   // zeroed counters of single-launch split reductions
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
   void *redux_cache = nullptr;
@@ -393,6 +394,7 @@ void ctx_destroy(hip_context *ctx) {
   // internal buffers do not count as owners, so they are still here
   if (ctx->errbuf) { hip_release(ctx->errbuf); ctx->errbuf = nullptr; }
   if (ctx->scratch) { hip_release(ctx->scratch); ctx->scratch = nullptr; }
+  if (ctx->redux_counters) { hip_release(ctx->redux_counters); ctx->redux_counters = nullptr; }
   ctx->mem.destroy();
   {
     // every kernel is gone by now (each one holds a reference to the context)
@@ -1420,6 +1422,19 @@ gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
   ctx->scratch = hip_alloc(c, want, nullptr, BUF_INTERNAL);
   if (ctx->scratch != nullptr) ctx->scratch_sz = want;
   return ctx->scratch;
+}
+
+gpudata *ga_hip_redux_counters(gpucontext *c) {
+  hip_context *ctx = HC(c);
+  if (ctx->redux_counters != nullptr) return ctx->redux_counters;
+  gpudata *b = hip_alloc(c, ga_hip_redux_counters_max * sizeof(uint32_t), nullptr, BUF_INTERNAL);
+  if (b == nullptr) return nullptr;
+  if (hip_memset(b, 0, 0) != GA_NO_ERROR) {
+    hip_release(b);
+    return nullptr;
+  }
+  ctx->redux_counters = b;
+  return b;
 }
 
 // Bytes from the start of a buffer that a kernel may read without leaving the

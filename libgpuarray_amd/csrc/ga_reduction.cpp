@@ -42,7 +42,7 @@ struct rd_plan {
   int64_t rdim[RD_MAXD], rmul[RD_MAXD];
   int64_t nrows, rtotal, nseg, units, upb, gx, router;
   int32_t nf, nr, nsplit, split_major;
-  int32_t rising, reserved;
+  int32_t rising, fused;
 };
 
 enum rd_kind { K_SUM, K_PROD, K_PRODNZ, K_MIN, K_MAX, K_AND, K_OR, K_XOR, K_ALL, K_ANY, K_CUSTOM };
@@ -439,7 +439,7 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
   if (err != GA_NO_ERROR) return err;
   const char *strs[1] = {s.c_str()};
   size_t lens[1] = {s.size()};
-  // sources (buffer, offset) ..., d0, d0_off, d1, d1_off, part_v, part_i, plan, scalars ...
+  // sources (buffer, offset) ..., d0, d0_off, d1, d1_off, part_v, part_i, done, plan, scalars ...
   std::vector<int> types;
   std::vector<int> flag_types;
   for (unsigned k = 0; k < gr->nsrc(); k++) {
@@ -447,7 +447,7 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
     types.push_back(GA_SIZE);
     flag_types.push_back(gr->args[gr->arrays[k]].tc);
   }
-  for (int t : {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_BUFFER, GA_BUFFER}) types.push_back(t);
+  for (int t : {GA_BUFFER, GA_SIZE, GA_BUFFER, GA_SIZE, GA_BUFFER, GA_BUFFER, GA_BUFFER}) types.push_back(t);
   types.push_back(ga_plan_typecode(plan_bytes(gr->nsrc())));
   for (unsigned i : gr->scalars) {
     types.push_back(gr->args[i].tc);
@@ -818,7 +818,7 @@ class reduction_call {
       if (p.rmul[i] < p.rdim[i + 1] * p.rmul[i + 1]) p.rising = 0;
     for (int i = 0; i < p.nr; i++)
       if (p.rmul[i] <= 0) p.rising = 0;
-    p.reserved = 0;
+    p.fused = 0;
 
     elsz_max = elsz_sum = 0;
     elsz.assign(K, 0);
@@ -991,7 +991,8 @@ class reduction_call {
     const int64_t target = ncu * per_cu;
     if (rowgroups < target && p.units >= 8) {
       nsplit = (target + rowgroups - 1) / rowgroups;
-      if (nsplit > p.units / 4) nsplit = p.units / 4;
+      const int64_t min_units = (int64_t)env_ul("GPUARRAY_REDUX_MIN_UNITS", 2);
+      if (nsplit > p.units / min_units) nsplit = p.units / min_units;
       if (nsplit > 65536) nsplit = 65536;
       if (nsplit < 1) nsplit = 1;
     }
@@ -1207,12 +1208,32 @@ class reduction_call {
     const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
     gpudata *scratch = ga_hip_scratch(ctx, 16);
     size_t pi_off = 0;
+    // A split reduction of moderate size ends in the launch that started it:
+    // its outputs (row kernel) or tiles of outputs (column kernel) have a
+    // counter each, and the piece that counts in last combines the partials.
+    // Measured on MI355X, one launch against two, calls timed one by one /
+    // issued back to back: sum of 2^16 floats 6.4 / 5.2 us against 8.4 / 8.7,
+    // of 2^20 7.0 / 5.3 against 8.4 / 8.6, of 2^22 (256 groups) 9.2 / 7.1
+    // against 8.7 / 8.6; with one group or more per compute unit waiting for
+    // its partial to be acknowledged before it counts in costs more than the
+    // second launch (2^24, 512 groups: 17.5 against 14.8 us).
+    gpudata *done = nullptr;
+    if (p.nsplit > 1) {
+      const size_t counters = use_row ? (size_t)nrows : groups / (size_t)p.nsplit;
+      const size_t fused_max = (size_t)ncu * env_ul("GPUARRAY_REDUX_FUSED", 1);   // 0 turns it off
+      if (groups <= fused_max && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
+          (done = ga_hip_redux_counters(ctx)) != nullptr) {
+        p.fused = 1;
+        if (!use_row) p.split_major = 1;
+      }
+    }
     if (p.nsplit > 1) {
       const size_t slots = (size_t)nrows * (size_t)p.nsplit;
       pi_off = (slots * accsz + 255) & ~(size_t)255;
       scratch = ga_hip_scratch(ctx, pi_off + slots * 8);
     }
     if (scratch == nullptr) return ctx->err->code;
+    if (!p.fused) done = scratch;   // not used then, but the kernels take a pointer
 
     // A destination the operation does not write still needs a valid pointer.
     gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
@@ -1235,13 +1256,14 @@ class reduction_call {
     args.push_back(&d1_off);
     args.push_back(scratch);
     args.push_back(&pi_view);
+    args.push_back(done);
     args.push_back(planbuf.data());
     for (void *sc : scalars) args.push_back(sc);
     size_t ls = 256;
     GpuKernel *k1 = srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
     int err;
     if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
-    if (p.nsplit > 1) {
+    if (p.nsplit > 1 && !p.fused) {
       size_t fg = (size_t)(p.split_major ? (nrows + 63) / 64 : (nrows + 3) / 4);
       if ((err = GpuKernel_call(p.split_major ? &var->fin_cols : &var->fin, 1, &fg, &ls, 0,
                                 args.data())) != GA_NO_ERROR)

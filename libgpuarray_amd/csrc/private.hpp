@@ -144,6 +144,11 @@ inline unsigned long env_ul(const char *name, unsigned long dflt) {
 }
 
 gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
+// Counters of split reductions that finish in one launch: a buffer of
+// ga_hip_redux_counters_max 32-bit zeros, made on first use; every kernel
+// that counts on it leaves it zeroed.  NULL (error set) when it cannot be made.
+constexpr size_t ga_hip_redux_counters_max = 16384;
+gpudata *ga_hip_redux_counters(gpucontext *ctx);
 // Bytes from a buffer's start that lie inside the memory behind it (at least
 // its size; more when the allocation was rounded up).
 size_t ga_hip_readable_bytes(gpudata *b);

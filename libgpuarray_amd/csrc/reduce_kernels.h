@@ -114,8 +114,10 @@ struct rd_plan {
   ga_long gx;      /* redux_col: groups along the inner free dim */
   ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates */
   ga_int nf, nr, nsplit, split_major;   /* split_major: layout of redux_col's partials */
-  ga_int rising, reserved;   /* rising: the flattened index grows with the position in the
-                              * reduced range, and the range has fewer than 2^31 positions */
+  ga_int rising, fused;   /* rising: the flattened index grows with the position in the
+                           * reduced range, and the range has fewer than 2^31 positions;
+                           * fused: the group that finishes an output's last piece also
+                           * combines its partials (no second pass) */
   ga_long fsstr[RD_NSRC][RD_MAXD], rsstr[RD_NSRC][RD_MAXD];   /* per source */
 };
 
@@ -410,6 +412,22 @@ static __device__ inline void rd_store(rd_acc a, const char *const *srow, char *
   rd_write(a, d0, d0o, d1, d1o);
 }
 
+/* The value the first-element rule looks at, for a caller that asks for it
+ * early so that the load is back by the time the result is (a second pass
+ * spends most of its few microseconds waiting for loads). */
+static __device__ inline RD_ACC_T rd_first_value(const char *const *srow, ga_long rtotal RD_SCALAR_FPARAMS) {
+#if RD_FIRST_RULE
+  if (rtotal > 0) {
+    rd_one o;
+    rd_one_load(o, srow);
+    return (RD_ACC_T)RD_ONE_VAL(o);
+  }
+#else
+  (void)srow; (void)rtotal;
+#endif
+  return RD_NEUTRAL;   /* not a NaN: the rule leaves the result alone */
+}
+
 static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *pi, ga_long slot) {
   pv[slot] = a.v;
 #if RD_ARG
@@ -417,6 +435,81 @@ static __device__ inline void rd_store_partial(rd_acc a, RD_ACC_T *pv, ga_long *
 #else
   (void)pi;
 #endif
+}
+
+/* ---- a split reduction finished in the same launch ---------------------------
+ * Every piece of an output leaves its partial and then counts itself in with
+ * an atomic add on the output's counter; the piece that brings the count to
+ * nsplit knows that all partials are there, reads them, combines them in slot
+ * order - so the result does not depend on which piece came last - writes the
+ * output and sets the counter back to zero for the next launch.  Nobody waits
+ * for anybody.
+ *
+ * The partials travel as device-scope atomic stores and loads (they pass the
+ * per-die L2 instead of resting in it), and a piece waits for its stores to
+ * be acknowledged before it counts in.  A device-scope release / acquire fence
+ * pair around plain stores and loads is the textbook form, but the release
+ * writes back the whole L2 once per piece: with 512 pieces a sum of 2^24
+ * floats went from 14.8 to 27 us.
+ *
+ * Launches that share the counters must not overlap (the library issues
+ * everything on one in-order stream). */
+template <typename T>
+static __device__ inline void rd_coherent_store(T *p, const T v) {
+  if (sizeof(T) == 8) {
+    union { T t; ga_ulong u; } x;
+    x.t = v;
+    __hip_atomic_store((ga_ulong *)p, x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    union { T t; ga_uint u; } x;
+    x.u = 0;
+    x.t = v;
+    __hip_atomic_store((ga_uint *)p, x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+template <typename T>
+static __device__ inline T rd_coherent_load(const T *p) {
+  if (sizeof(T) == 8) {
+    union { T t; ga_ulong u; } x;
+    x.u = __hip_atomic_load((const ga_ulong *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return x.t;
+  } else {
+    union { T t; ga_uint u; } x;
+    x.u = __hip_atomic_load((const ga_uint *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return x.t;
+  }
+}
+/* the host only asks for this path when the accumulator has 4 or 8 bytes */
+static __device__ inline void rd_publish_partial(rd_acc a, RD_ACC_T *pv, ga_long *pi, ga_long slot) {
+  rd_coherent_store(pv + slot, a.v);
+#if RD_ARG
+  rd_coherent_store(pi + slot, a.i);
+#else
+  (void)pi;
+#endif
+}
+static __device__ inline rd_acc rd_fetch_partial(const RD_ACC_T *pv, const ga_long *pi, ga_long slot) {
+  rd_acc t;
+  t.v = rd_coherent_load(pv + slot);
+#if RD_ARG
+  t.i = rd_coherent_load(pi + slot);
+#else
+  (void)pi;
+#endif
+  return t;
+}
+/* The wavefront's stores have been acknowledged when this returns (a
+ * device-scope store is acknowledged once it is past the L2), and the
+ * compiler moves no memory access across either of the two. */
+static __device__ inline void rd_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+static __device__ inline void rd_before_loads() { asm volatile("" ::: "memory"); }
+/* true for the caller that completes the count */
+static __device__ inline bool rd_count_in(ga_uint *counter, ga_uint total) {
+  const ga_uint before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return before + 1u == total;
+}
+static __device__ inline void rd_count_reset(ga_uint *counter) {
+  __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* ---- redux_row ------------------------------------------------------------- */
@@ -485,24 +578,50 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
    * compare keeps the first of equals by itself; only the position inside
    * the unit (a small int) is tracked. */
   /* (with RD_TAIL only units wholly inside the row come here) */
-  RD_ACC_T bv = rd_elem(RD_UNIT_VAL(x, 0, 0), 0).v;
-  ga_int bp = 0;
+  /* For one-byte elements with a position to track, RD_NCH scans run side by
+   * side (elements v, v + RD_NCH, ... of every load), each in rising order, so
+   * that one compare does not wait for the one before it; they meet at the
+   * end, the lower position winning a tie (maxandargmax of 2^28 bytes 127 ->
+   * 65 us).  Wider elements, and a plain integer max, which compiles to one
+   * instruction per element, measured a few percent slower that way. */
+#define RD_NCH ((RD_ARG && RD_ELSZ0 == 1 && RD_VEC >= 4) ? 4 : 1)
+  RD_ACC_T cv[RD_NCH];
+  ga_int cp[RD_NCH];
+#pragma unroll
+  for (int c = 0; c < RD_NCH; c++) {
+    cv[c] = rd_elem(RD_UNIT_VAL(x, 0, c), 0).v;
+    cp[c] = c;
+  }
 #pragma unroll
   for (int j = 0; j < RD_U; j++) {
     const bool in = RD_TAIL || e0 + (ga_long)j * LN * RD_VEC < rin;
 #pragma unroll
     for (int v = 0; v < RD_VEC; v++) {
-      if (j == 0 && v == 0) continue;
+      if (j == 0 && v < RD_NCH) continue;
+      const int c = v % RD_NCH;
       const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
 #if RD_KIND == RD_K_MAX
-      const bool better = in && val > bv;
+      const bool better = in && val > cv[c];
 #else
-      const bool better = in && val < bv;
+      const bool better = in && val < cv[c];
 #endif
-      bv = better ? val : bv;
-      bp = better ? (j * LN * RD_VEC + v) : bp;
+      cv[c] = better ? val : cv[c];
+      cp[c] = better ? (j * LN * RD_VEC + v) : cp[c];
     }
   }
+  RD_ACC_T bv = cv[0];
+  ga_int bp = cp[0];
+#pragma unroll
+  for (int c = 1; c < RD_NCH; c++) {
+#if RD_KIND == RD_K_MAX
+    const bool better = cv[c] > bv || (cv[c] == bv && cp[c] < bp);
+#else
+    const bool better = cv[c] < bv || (cv[c] == bv && cp[c] < bp);
+#endif
+    bv = better ? cv[c] : bv;
+    bp = better ? cp[c] : bp;
+  }
+#undef RD_NCH
   rd_acc r = rd_neutral();
   const bool any = RD_TAIL || e0 < rin;
   r.v = any ? bv : r.v;
@@ -603,7 +722,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
 #if RD_WANT & 1   /* the row family: redux_row, redux_wrows */
 KERNEL void __launch_bounds__(256)
 redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
-          const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+          const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
           const rd_plan p RD_SCALAR_PARAMS) {
   const unsigned rows_per_group = 256u / RD_G;
   const unsigned lane = LID_0 % RD_G;
@@ -628,6 +747,10 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
     srow[k] += so[k];
     rstr[k] = p.nr > 0 ? p.rsstr[k][ri] : 0;
   }
+
+  /* what the first-element rule looks at, asked for now and used at the end */
+  RD_ACC_T first = RD_NEUTRAL;
+  if (lane == 0) first = rd_first_value(srow, p.rtotal RD_SCALAR_ARGS);
 
   /* A split owns a contiguous range of units, or - for a single reduced dim
    * (RD_INTERLEAVE) - every nsplit-th unit, so that at any moment the splits
@@ -709,9 +832,43 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
 #endif
   if (lane == 0) {
     if (p.nsplit == 1)
-      rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
+      rd_write(rd_first_rule(acc, first), d0 + d0_off, d0o, d1 + d1_off, d1o);
+    else if (p.fused)
+      rd_publish_partial(acc, part_v, part_i, row * p.nsplit + split);
     else
       rd_store_partial(acc, part_v, part_i, row * p.nsplit + split);
+  }
+  if (p.nsplit > 1 && p.fused) {
+    /* uniform over the lanes that share the row: the group (RD_G == 256) or the wavefront */
+#if RD_G == 256
+    __shared__ ga_uint last_piece;
+    if (lane == 0) {
+      rd_stores_done();
+      last_piece = rd_count_in(done + row, (ga_uint)p.nsplit) ? 1u : 0u;
+    }
+    local_barrier();
+    if (!last_piece) return;
+#else
+    ga_uint last_piece = 0;
+    if (lane == 0) {
+      rd_stores_done();
+      last_piece = rd_count_in(done + row, (ga_uint)p.nsplit) ? 1u : 0u;
+    }
+    if (!__builtin_amdgcn_readfirstlane(last_piece)) return;
+#endif
+    rd_before_loads();
+    rd_acc all = rd_neutral();
+    for (ga_long s = lane; s < p.nsplit; s += RD_G)
+      all = rd_combine(all, rd_fetch_partial(part_v, part_i, row * p.nsplit + s));
+#if RD_G == 256
+    all = rd_block_reduce(all, lds);
+#else
+    all = rd_wave_reduce(all);
+#endif
+    if (lane == 0) {
+      rd_write(rd_first_rule(all, first), d0 + d0_off, d0o, d1 + d1_off, d1o);
+      rd_count_reset(done + row);
+    }
   }
 }
 
@@ -727,9 +884,9 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
  * current row is combined */
 KERNEL void __launch_bounds__(256)
 redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
-            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
             const rd_plan p RD_SCALAR_PARAMS) {
-  (void)part_v; (void)part_i;
+  (void)part_v; (void)part_i; (void)done;
   const unsigned lane = LID_0 & 63u;
   const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
   ga_long row = wave * p.upb;
@@ -779,9 +936,9 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
  * see a disabled lane. */
 KERNEL void __launch_bounds__(256)
 redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
-            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
             const rd_plan p RD_SCALAR_PARAMS) {
-  (void)part_v; (void)part_i;
+  (void)part_v; (void)part_i; (void)done;
   const unsigned lane = LID_0 & 63u;
   const unsigned sub = lane / RD_L, l = lane % RD_L;
   const ga_long wave = (ga_long)GID_0 * 4 + (LID_0 >> 6);
@@ -865,9 +1022,9 @@ typedef ga_uint rd_chunk_t __attribute__((ext_vector_type(4)));
 
 KERNEL void __launch_bounds__(256)
 redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
-            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
             const rd_plan p RD_SCALAR_PARAMS) {
-  (void)part_v; (void)part_i;
+  (void)part_v; (void)part_i; (void)done;
   extern __shared__ rd_chunk_t rd_staged[];
   const ga_long per_group = p.upb;
   const ga_long row0 = (ga_long)GID_0 * per_group;
@@ -1038,7 +1195,7 @@ static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *
 
 KERNEL void __launch_bounds__(256)
 redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
-          RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
+          RD_ACC_T *part_v, ga_long *part_i, ga_uint *done, const rd_plan p RD_SCALAR_PARAMS) {
   __shared__ rd_acc lds[RD_CY][RD_CV][RD_CX];
   const unsigned tx = LID_0 % RD_CX, ty = LID_0 / RD_CX;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
@@ -1181,10 +1338,51 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       } else {
         /* with many outputs the partials lie split-major (adjacent lanes write
          * adjacent slots, redux_final_cols reads them); else output-major */
-        rd_store_partial(a, part_v, part_i,
-                         p.split_major ? split * p.nrows + row : row * p.nsplit + split);
+        if (p.fused)
+          rd_publish_partial(a, part_v, part_i, split * p.nrows + row);
+        else
+          rd_store_partial(a, part_v, part_i,
+                           p.split_major ? split * p.nrows + row : row * p.nsplit + split);
       }
     }
+  }
+  if (p.nsplit > 1 && p.fused) {
+    /* one counter per tile of outputs (the groups that differ in `split` only);
+     * the partials lie split-major here */
+    __shared__ ga_uint last_piece;
+    rd_stores_done();   /* every lane that left partials */
+    local_barrier();
+    if (LID_0 == 0) last_piece = rd_count_in(done + t, (ga_uint)p.nsplit) ? 1u : 0u;
+    local_barrier();
+    if (!last_piece) return;
+    rd_before_loads();
+#pragma unroll
+    for (int c = 0; c < RD_CV; c++) {
+      rd_acc a = rd_neutral();
+      if (live)
+        for (ga_long s = ty; s < p.nsplit; s += RD_CY)
+          a = rd_combine(a, rd_fetch_partial(part_v, part_i, s * p.nrows + fo * fin + fi + c));
+      acc[c] = a;
+    }
+#if RD_CY > 1
+#pragma unroll
+    for (int c = 0; c < RD_CV; c++) lds[ty][c][tx] = acc[c];
+    local_barrier();
+#endif
+    if (ty == 0 && live) {
+#pragma unroll
+      for (int c = 0; c < RD_CV; c++) {
+        rd_acc a = acc[c];
+#pragma unroll
+        for (int y = 1; y < RD_CY; y++) a = rd_combine(a, lds[y][c][tx]);
+        const char *sc[RD_NSRC];
+#pragma unroll
+        for (int k = 0; k < RD_NSRC; k++) sc[k] = srow[k] + c * p.fsstr[k][fi_d];
+        rd_store(a, sc, d0 + d0_off, d0o + c * p.fd0str[fi_d], d1 + d1_off,
+                 d1o + c * p.fd1str[fi_d], p.rtotal RD_SCALAR_ARGS);
+      }
+    }
+    if (LID_0 == 0) rd_count_reset(done + t);
   }
 }
 
@@ -1195,10 +1393,18 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
  * One wavefront per output: combine its nsplit partials and write the result. */
 KERNEL void __launch_bounds__(256)
 redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
-            RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
+            RD_ACC_T *part_v, ga_long *part_i, ga_uint *done, const rd_plan p RD_SCALAR_PARAMS) {
   const unsigned lane = LID_0 & 63u;
   const ga_long row = (ga_long)GID_0 * 4 + (LID_0 >> 6);
   if (row >= p.nrows) return;
+  ga_long so[RD_NSRC], d0o, d1o;
+  rd_row_offsets(p, row, so, &d0o, &d1o);
+  const char *srow[RD_NSRC];
+  RD_SRC_BASES(srow);
+#pragma unroll
+  for (int k = 0; k < RD_NSRC; k++) srow[k] += so[k];
+  RD_ACC_T first = RD_NEUTRAL;
+  if (lane == 0) first = rd_first_value(srow, p.rtotal RD_SCALAR_ARGS);
   rd_acc acc = rd_neutral();
   for (ga_long s = lane; s < p.nsplit; s += 64) {
     rd_acc t;
@@ -1209,15 +1415,7 @@ redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_si
     acc = rd_combine(acc, t);
   }
   acc = rd_wave_reduce(acc);
-  if (lane == 0) {
-    ga_long so[RD_NSRC], d0o, d1o;
-    rd_row_offsets(p, row, so, &d0o, &d1o);
-    const char *srow[RD_NSRC];
-    RD_SRC_BASES(srow);
-#pragma unroll
-    for (int k = 0; k < RD_NSRC; k++) srow[k] += so[k];
-    rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
-  }
+  if (lane == 0) rd_write(rd_first_rule(acc, first), d0 + d0_off, d0o, d1 + d1_off, d1o);
 }
 
 #endif   /* RD_WANT & 3 */
@@ -1229,7 +1427,7 @@ redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_si
  * lane rows share the splits and meet in LDS. */
 KERNEL void __launch_bounds__(256)
 redux_final_cols(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size d1_off,
-                 RD_ACC_T *part_v, ga_long *part_i, const rd_plan p RD_SCALAR_PARAMS) {
+                 RD_ACC_T *part_v, ga_long *part_i, ga_uint *done, const rd_plan p RD_SCALAR_PARAMS) {
   __shared__ rd_acc meet[4][64];
   const unsigned tx = LID_0 & 63u, ty = LID_0 >> 6;
   const ga_long row = (ga_long)GID_0 * 64 + tx;

@@ -751,3 +751,70 @@ def test_column_scans_keep_the_first_of_equals(ctx, dtype):
                 if dt.kind == "f":
                     plain = np.asarray(getattr(R, name[:3])(g, axis=axes))
                     assert np.array_equal(plain.view(bits), want_v.astype(dt).view(bits)), (name[:3], shape)
+
+
+def test_split_reductions_finish_in_one_launch(ctx, monkeypatch):
+    """A reduction whose outputs are cut into pieces: the piece that finishes
+    last combines the partials in the same launch (a counter per output, or per
+    tile of outputs of the column kernel, that the launch leaves at zero).
+    Many such calls in a row on changing shapes, against NumPy, against the
+    two-launch path, and twice for bit-identical float results."""
+    rng = np.random.default_rng(91)
+    cases = []
+    for n in (1 << 16, (1 << 18) + 3, 1 << 20, (1 << 22) - 5):
+        cases.append(((n,), (0,)))
+    cases += [((4, 1 << 20), (1,)), ((16, 1 << 18), (1,)), ((3, 5, 1 << 16), (1, 2)),     # rows in pieces
+              ((4096, 256), (0,)), ((100000, 64), (0,)), ((70, 3000, 40), (1,)),          # columns in pieces
+              ((20000, 1000), (0,)), ((1 << 19, 8), (0,))]
+    for rep in range(2):
+        for dtype in ("float32", "int32", "float64"):
+            for shape, axes in cases:
+                host = rng.integers(-30, 30, size=shape).astype(dtype)
+                g, _ = to_gpu_view(host, ctx)
+                if host.dtype.kind == "i":
+                    got = np.asarray(R.sum(g, axis=axes, dtype="int64"))
+                    assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64)), (shape, axes)
+                else:
+                    got = np.asarray(R.sum(g, axis=axes))
+                    want = host.sum(axis=axes, dtype=np.float64)
+                    scale = np.abs(host).sum(axis=axes, dtype=np.float64)
+                    assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(scale, 1e-30)), (shape, axes)
+                    again = np.asarray(R.sum(g, axis=axes))
+                    assert np.array_equal(got.view("u%d" % got.dtype.itemsize),
+                                          again.view("u%d" % got.dtype.itemsize)), (shape, axes)
+                moved = np.moveaxis(host, axes, range(host.ndim - len(axes), host.ndim))
+                flat = moved.reshape(moved.shape[:host.ndim - len(axes)] + (-1,))
+                val, idx = R.maxandargmax(g, axis=axes)
+                assert np.array_equal(np.asarray(val), flat.max(axis=-1)), (shape, axes)
+                assert np.array_equal(np.asarray(idx), flat.argmax(axis=-1)), (shape, axes)
+    # the same slots of the partials carry other values in every call: a piece that
+    # read a leftover of the call before would show
+    for shape, axes in (((1 << 20,), (0,)), ((8, 1 << 18), (1,)), ((4096, 256), (0,))):
+        g = gpuarray.zeros(shape, "int32", context=ctx)
+        count = int(np.prod([shape[a] for a in axes]))
+        for k in range(1, 120):
+            g[...] = np.int32(k if k % 3 else -k)
+            got = np.asarray(R.sum(g, axis=axes, dtype="int64"))
+            assert np.all(got == count * (k if k % 3 else -k)), (shape, k)
+    # the two-launch path gives the same integers and indices
+    host = rng.integers(-30, 30, size=(100000, 64)).astype("int32")
+    flat = rng.integers(-30, 30, size=(1 << 20) + 1).astype("float32")
+    g, _ = to_gpu_view(host, ctx)
+    gf, _ = to_gpu_view(flat, ctx)
+    one = (np.asarray(R.sum(g, axis=0, dtype="int64")), np.asarray(R.maxandargmax(gf)[1]))
+    monkeypatch.setenv("GPUARRAY_REDUX_FUSED", "0")
+    two = (np.asarray(R.sum(g, axis=0, dtype="int64")), np.asarray(R.maxandargmax(gf)[1]))
+    monkeypatch.delenv("GPUARRAY_REDUX_FUSED")
+    assert np.array_equal(one[0], two[0]) and np.array_equal(one[0], host.sum(axis=0, dtype=np.int64))
+    assert one[1] == two[1] == flat.argmax()
+    # NaN in the first position of a cut row stays; later NaNs are passed over
+    x = rng.normal(size=1 << 20).astype("float32")
+    x[0] = np.nan
+    x[5000] = np.nan
+    gx, _ = to_gpu_view(x, ctx)
+    v, i = R.maxandargmax(gx)
+    assert np.isnan(np.asarray(v)) and int(np.asarray(i)) == 0
+    x[0] = -1.0
+    gx, _ = to_gpu_view(x, ctx)
+    v, i = R.maxandargmax(gx)
+    assert np.asarray(v) == np.nanmax(x) and int(np.asarray(i)) == int(np.nanargmax(x))
