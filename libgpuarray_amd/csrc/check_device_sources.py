@@ -83,6 +83,10 @@ def main():
         check("reduction %d outputs per lane" % cv,
               gen_r(8 if src != GA_UBYTE else 0, src, src if src != GA_UBYTE else GA_LONG, GA_LONG,
                     256, 1 | (cv << 16), 4))
+    for op, cv in ((13, 16), (12, 4), (13, 8)):
+        check("column any / all over bytes, op %d, %d outputs per lane" % (op, cv),
+              gen_r(op, GA_UBYTE, GA_BOOL, GA_LONG, 256, 1 | (cv << 16), 4))
+        n += 1
     for lo in (4, 16):
         check("reduction %d outer coordinates side by side" % lo,
               gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | (lo << 16)))

@@ -262,6 +262,13 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
                        (kind == K_SUM || kind == K_ANY || kind == K_ALL) && !valf &&
                        env_ul("GPUARRAY_REDUX_FAST8", 1);
     DEF("#define RD_FAST8 %d\n", bytes ? (stc == GA_BYTE ? 2 : 1) : 0);
+    // redux_col, any / all over one-byte elements: the words of a lane's load
+    // are or-ed whole (all: their zero-byte masks) and taken apart once at
+    // the end.
+    const unsigned cvn = vs.CV ? vs.CV : 1;
+    const bool col_bytes = K == 1 && !gr->mapped && gpuarray_get_elsize(stc) == 1 && cvn % 4 == 0 &&
+                           (kind == K_ANY || kind == K_ALL) && env_ul("GPUARRAY_REDUX_FAST8", 1);
+    DEF("#define RD_COL_FAST8 %d\n", col_bytes ? 1 : 0);
   }
   {
     // redux_row: an unconditional use after each unit's loads where the
@@ -403,6 +410,9 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
       GEN("%srd_w%u((o).x%u[c])", k ? ", " : "", k, k);
   }
   gen += " RD_SCALAR_ARGS)\n";
+  // word d of the first source's packed load (one- and two-byte elements)
+  if (words[0] == 1) gen += "#define RD_CVEC_WORD(o, d) ((o).x0)\n";
+  else if (words[0] > 1) gen += "#define RD_CVEC_WORD(o, d) ((o).x0[d])\n";
 #undef GEN
   return GA_NO_ERROR;
 }

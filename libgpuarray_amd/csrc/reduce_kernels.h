@@ -23,6 +23,7 @@
  *               RD_ES-th one is used
  *   RD_FAST8    one-byte elements combined four per 32-bit operation (sum, any,
  *               all; 1: unsigned bytes, 2: signed), 0: off
+ *   RD_COL_FAST8  redux_col: any / all over one-byte elements work on whole words
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
  *   RD_WANT     which kernels the text holds: bit 0 the row family (redux_row,
  *               redux_wrows), bit 1 the column family (redux_col,
@@ -1286,6 +1287,43 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     }
   } else
 #endif
+#if RD_COL_FAST8
+  if (live) {
+    /* any / all over bytes: bit 8c+7 of word c/4 of `seen` says that byte c of
+     * some load was non-zero (any) or zero (all); exact per byte (the sum of
+     * the low seven bits and 0x7f carries into bit 7 and no further) */
+    ga_uint seen[RD_CV / 4];
+#pragma unroll
+    for (int d = 0; d < RD_CV / 4; d++) seen[d] = 0;
+#define RD_COL_BYTES_SEEN(xx)                                                              \
+  _Pragma("unroll") for (int d = 0; d < RD_CV / 4; d++) {                                  \
+    const ga_uint wd = RD_CVEC_WORD(xx, d);                                                \
+    const ga_uint nz = (((wd & 0x7f7f7f7fu) + 0x7f7f7f7fu) | wd) & 0x80808080u;            \
+    seen[d] |= RD_KIND == RD_K_ANY ? nz : (nz ^ 0x80808080u);                              \
+  }
+    ga_long j0 = r0 + ty;
+#if RD_U > 1
+    for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
+      rd_cvec x[RD_U];
+#pragma unroll
+      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+#pragma unroll
+      for (int q = 0; q < RD_U; q++) { RD_COL_BYTES_SEEN(x[q]) }
+    }
+#endif
+    for (; j0 < r1; j0 += RD_CY) {
+      rd_cvec x;
+      rd_col_fetch(p, srow, j0, x);
+      RD_COL_BYTES_SEEN(x)
+    }
+#undef RD_COL_BYTES_SEEN
+#pragma unroll
+    for (int c = 0; c < RD_CV; c++) {
+      const ga_uint bit = (seen[c / 4] >> (8 * (c % 4) + 7)) & 1u;
+      acc[c].v = RD_KIND == RD_K_ANY ? bit : (bit ^ 1u);
+    }
+  }
+#else
   if (live) {
     ga_long j0 = r0 + ty;
 #if RD_U > 1
@@ -1314,6 +1352,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       for (int c = 0; c < RD_CV; c++) acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x, c), idx));
     }
   }
+#endif
 #if RD_CY > 1
 #pragma unroll
   for (int c = 0; c < RD_CV; c++) lds[ty][c][tx] = acc[c];

@@ -818,3 +818,32 @@ def test_split_reductions_finish_in_one_launch(ctx, monkeypatch):
     gx, _ = to_gpu_view(x, ctx)
     v, i = R.maxandargmax(gx)
     assert np.asarray(v) == np.nanmax(x) and int(np.asarray(i)) == int(np.nanargmax(x))
+
+
+@pytest.mark.parametrize("dtype", ["uint8", "int8", "bool"])
+def test_any_all_over_columns_of_bytes(ctx, dtype):
+    """any / all with lanes along the free dim over one-byte elements: the
+    words of a lane's load are combined whole and taken apart at the end.
+    Values 0x01, 0x7f, 0x80, 0xff and 0 next to one another in a word (a test
+    of one byte must not leak into its neighbours), 4, 8 and 16 columns per
+    lane, split and unsplit ranges, a single element that flips a column."""
+    rng = np.random.default_rng(57)
+    vals = np.array([0, 1, 0x7f, 0x80, 0xff, 0, 0, 2], np.uint8)
+    for shape in ((300, 1024), (4096, 256), (37, 64), (5000, 4096), (9, 130, 128), (1000, 20)):
+        raw = vals[rng.integers(0, len(vals), size=shape)]
+        host = (raw != 0) if dtype == "bool" else raw.view(dtype) if dtype == "int8" else raw
+        cols = host.reshape(-1, shape[-1])
+        cols[:, 0] = 0                       # any: false
+        cols[:, 1] = 1 if dtype != "int8" else -128   # all: true
+        cols[:, 2] = 0; cols[cols.shape[0] // 2, 2] = 1     # one element makes any true
+        cols[:, 3] = 1; cols[cols.shape[0] - 1, 3] = 0      # one element makes all false
+        cols[:, 5] = 0                                       # a zero column between non-zero ones
+        cols[:, 4] = 1; cols[:, 6] = 1
+        axes = tuple(range(host.ndim - 1))
+        for view in (host, host[..., 4:], host[1::2]):
+            g, _ = to_gpu_view(view, ctx)
+            assert np.array_equal(np.asarray(R.any(g, axis=axes)), view.any(axis=axes)), (shape, view.shape)
+            assert np.array_equal(np.asarray(R.all(g, axis=axes)), view.all(axis=axes)), (shape, view.shape)
+            if view.ndim == 3:
+                assert np.array_equal(np.asarray(R.any(g, axis=(1,))), view.any(axis=1))
+                assert np.array_equal(np.asarray(R.all(g, axis=(0,))), view.all(axis=0))
