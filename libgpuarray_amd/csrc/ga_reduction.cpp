@@ -1146,8 +1146,11 @@ class reduction_call {
       {
         const int64_t want = ncu * 4, outer_f = nrows / fin;
         auto groups_at = [&](unsigned c) { return ((fin + CX * c - 1) / (CX * c)) * outer_f; };
+        // ... but not with less than 256 contiguous bytes per row and group:
+        // sums over axis 0 of 4096 x 65536 bytes ran at 108 us with two
+        // columns per lane (64 bytes per row and group).
         if (groups_at(cv) < want)
-          for (unsigned c = cv / 2; c >= 1; c /= 2)
+          for (unsigned c = cv / 2; c >= 1 && (int64_t)c * elsz_max * CX >= 256; c /= 2)
             if (groups_at(c) >= want) { cv = c; break; }
       }
       CV = cv;

@@ -1248,7 +1248,6 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #pragma unroll
     for (int c = 0; c < RD_CV; c++) { bv[c] = RD_NEUTRAL; bj[c] = 0x7fffffff; }
     ga_long j0 = r0 + ty;
-#if RD_U > 1
     for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
 #pragma unroll
@@ -1264,17 +1263,22 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
         }
       }
     }
-#endif
-    for (; j0 < r1; j0 += RD_CY) {
-      rd_cvec x;
-      rd_col_fetch(p, srow, j0, x);
+    if (j0 < r1) {   /* the last, partial batch: its loads go out together too */
+      rd_cvec x[RD_U];
 #pragma unroll
-      for (int c = 0; c < RD_CV; c++) {
-        const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x, c), 0).v;
-        const bool better = RD_COL_BETTER(val, bv[c]);
-        bv[c] = better ? val : bv[c];
-        bj[c] = better ? (ga_int)j0 : bj[c];
-      }
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+#pragma unroll
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) {
+#pragma unroll
+          for (int c = 0; c < RD_CV; c++) {
+            const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x[q], c), 0).v;
+            const bool better = RD_COL_BETTER(val, bv[c]);
+            bv[c] = better ? val : bv[c];
+            bj[c] = better ? (ga_int)(j0 + RD_CY * q) : bj[c];
+          }
+        }
     }
     if (r0 + ty < r1) {
 #pragma unroll
@@ -1302,7 +1306,6 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     seen[d] |= RD_KIND == RD_K_ANY ? nz : (nz ^ 0x80808080u);                              \
   }
     ga_long j0 = r0 + ty;
-#if RD_U > 1
     for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
 #pragma unroll
@@ -1310,11 +1313,14 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #pragma unroll
       for (int q = 0; q < RD_U; q++) { RD_COL_BYTES_SEEN(x[q]) }
     }
-#endif
-    for (; j0 < r1; j0 += RD_CY) {
-      rd_cvec x;
-      rd_col_fetch(p, srow, j0, x);
-      RD_COL_BYTES_SEEN(x)
+    if (j0 < r1) {   /* the last, partial batch */
+      rd_cvec x[RD_U];
+#pragma unroll
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+#pragma unroll
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) { RD_COL_BYTES_SEEN(x[q]) }
     }
 #undef RD_COL_BYTES_SEEN
 #pragma unroll
@@ -1326,7 +1332,6 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #else
   if (live) {
     ga_long j0 = r0 + ty;
-#if RD_U > 1
     /* all RD_U loads of a batch lie inside the range: no test per load */
     for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
@@ -1343,13 +1348,22 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
           acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
       }
     }
-#endif
-    for (; j0 < r1; j0 += RD_CY) {
-      rd_cvec x;
-      rd_col_fetch(p, srow, j0, x);
-      const ga_long idx = RD_ARG ? rd_col_index(p, j0) : 0;
+    if (j0 < r1) {   /* the last, partial batch: its loads go out together too */
+      rd_cvec x[RD_U];
+      ga_long idx[RD_U];
 #pragma unroll
-      for (int c = 0; c < RD_CV; c++) acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x, c), idx));
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) {
+          rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+          idx[q] = RD_ARG ? rd_col_index(p, j0 + RD_CY * q) : 0;
+        }
+#pragma unroll
+      for (int q = 0; q < RD_U; q++)
+        if (j0 + RD_CY * q < r1) {
+#pragma unroll
+          for (int c = 0; c < RD_CV; c++)
+            acc[c] = rd_combine(acc[c], rd_elem(RD_CVEC_VAL(x[q], c), idx[q]));
+        }
     }
   }
 #endif
