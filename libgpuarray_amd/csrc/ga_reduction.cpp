@@ -1172,7 +1172,11 @@ class reduction_call {
     // 8 groups per compute unit; four outputs per lane 50.1 / 45.8 / 50.5 /
     // 49.6 us with 3-4 groups, and 60 / 84 / 61 / 51 us with 8 (the second
     // shape then splits its 256 rows for nothing).
-    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? 4 : 8);
+    // Three against four groups per unit, later, with eight lane rows: bytes
+    // 16384 x 16384 54.3 -> 49.5 us, floats 65536 x 1000 48.6 -> 46.3,
+    // 8192 x 8192 49.3 -> 48.1, halves 2048 x 65536 48.2 -> 46.1; two groups
+    // were faster still for 2- and 4-byte elements and slower for bytes (59.5).
+    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? 3 : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
       if (nsplit > rtotal / 64) nsplit = rtotal / 64;
