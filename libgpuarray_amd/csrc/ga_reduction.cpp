@@ -882,6 +882,7 @@ class reduction_call {
       const int64_t es = rsstr[p.nr - 1] / elsz[0];
       if (es == 1 || es == 2 || es == 4) {
         unsigned v = (unsigned)(16 / (elsz[0] * es));
+        if (v < 1) v = 1;   // 8-byte elements four apart: no load holds two of them
         size_t bufsz = 0;
         gpudata_property(s0->data, GA_BUFFER_PROP_SIZE, &bufsz);
         int64_t last = (int64_t)s0->offset;   // byte offset of the farthest element

@@ -847,3 +847,29 @@ def test_any_all_over_columns_of_bytes(ctx, dtype):
             if view.ndim == 3:
                 assert np.array_equal(np.asarray(R.any(g, axis=(1,))), view.any(axis=1))
                 assert np.array_equal(np.asarray(R.all(g, axis=(0,))), view.all(axis=0))
+
+
+@pytest.mark.parametrize("dtype", ["float64", "int64", "float32", "int16", "uint8"])
+def test_stepped_inner_dim_of_every_width(ctx, dtype):
+    """Reduced rows that take every 2nd, 3rd or 4th element (8-byte elements
+    four apart leave no load that holds two of them)."""
+    rng = np.random.default_rng(93)
+    for shape in ((16, 4), (300, 4000), (5, 70001), (2000, 64)):
+        base = rng.integers(0, 50, size=shape).astype(dtype)
+        for step in (2, 3, 4):
+            for view in (base[:, ::step], base[:, 1::step], base[:, :1], base[::step, ::step]):
+                _check_ops(ctx, view, [1])
+                _check_ops(ctx, view, [0, 1])
+
+
+def test_stepped_eight_byte_rows_are_planned(ctx):
+    """The planner's arithmetic alone (no look at the values): an 8-byte
+    element type whose reduced dim steps by four elements."""
+    base = np.zeros((16, 4), np.float64)
+    g, _ = to_gpu_view(base[:, :1], ctx)
+    for axes in ((0, 1), (0,), (1,)):
+        assert np.asarray(R.sum(g, axis=axes)).shape == base[:, :1].sum(axis=axes).shape
+        v, i = R.maxandargmax(g, axis=axes)
+        assert np.asarray(i).dtype == np.int64
+    g, _ = to_gpu_view(np.zeros((64, 4096), np.int64)[:, ::4], ctx)
+    assert np.asarray(R.sum(g, axis=1)).shape == (64,)

@@ -26,6 +26,7 @@ HOST_ONLY = [
     "tests/test_gpu_take1.py::test_argument_rules",
     "tests/test_gpu_reduction.py::test_maxandargmax_argument_errors",
     "tests/test_gpu_reduction.py::test_reduction_wrong_out_and_axis",
+    "tests/test_gpu_reduction.py::test_stepped_eight_byte_rows_are_planned",
     "tests/test_gpu_elemwise.py::test_zero_sized",
     "tests/test_gpu_elemwise.py::test_new_reports_compile_errors",
     "tests/test_gpu_tools.py",
