@@ -1,0 +1,52 @@
+"""Helper of test_host_logic_without_device.py (not collected by pytest): drives
+the reduction and elementwise planners over random element types, shapes,
+steps, offsets and axis sets against the stand-in runtime, whose launches do
+nothing.  What is asked is that every call returns (no crash in the host
+arithmetic that picks vector widths, lane geometry and splits) with a result
+of the right shape."""
+import sys
+
+import numpy as np
+
+sys.path.insert(0, ".")
+sys.path.insert(0, "tests")
+import libgpuarray_amd as ga                      # noqa: E402
+from libgpuarray_amd import reduction as R        # noqa: E402
+from libgpuarray_amd.elemwise import elemwise2    # noqa: E402
+from support import to_gpu_view                   # noqa: E402
+
+ctx = ga.init("hip0")
+rng = np.random.default_rng(int(sys.argv[1]))
+cases = int(sys.argv[2])
+pool = [1, 2, 3, 4, 5, 7, 8, 16, 17, 31, 32, 33, 64, 100, 129, 250, 256, 257, 1000, 1023, 4099]
+types = ["int8", "uint8", "int16", "int32", "int64", "float16", "float32", "float64", "bool"]
+for case in range(cases):
+    nd = int(rng.integers(1, 5))
+    while True:
+        shape = tuple(int(rng.choice(pool)) for _ in range(nd))
+        if np.prod(shape) <= 2_000_000:
+            break
+    dt = str(rng.choice(types))
+    steps = [int(rng.choice([1, 1, 2, 3, 4])) for _ in shape]
+    base = np.zeros(tuple(s * st + int(rng.integers(0, 4)) for s, st in zip(shape, steps)), dt)
+    idx = []
+    for s, st, b in zip(shape, steps, base.shape):
+        start = int(rng.integers(0, b - (s - 1) * st))
+        idx.append(slice(start, start + (s - 1) * st + 1, st))
+    view = base[tuple(idx)]
+    if nd > 1 and rng.random() < 0.3:
+        view = view.transpose(rng.permutation(nd))
+    k = int(rng.integers(1, nd + 1))
+    axes = tuple(sorted(rng.choice(nd, k, replace=False).tolist()))
+    g, _ = to_gpu_view(view, ctx)
+    want = view.sum(axis=axes).shape
+    print(case, dt, view.shape, view.strides, axes, flush=True)
+    assert np.asarray(R.sum(g, axis=axes)).shape == want
+    assert np.asarray(R.any(g, axis=axes)).shape == want
+    if dt != "bool":
+        assert np.asarray(R.max(g, axis=axes)).shape == want
+        v, i = R.maxandargmax(g, axis=axes)
+        assert np.asarray(i).shape == want
+    if dt != "bool":
+        assert elemwise2(g, "+", g, g).shape == view.shape
+print("planner ok")

@@ -62,3 +62,14 @@ def test_c_client_survives_teardown_without_a_device(mock_runtime, tmp_path):
     # asked is that every host path, context teardown included, runs through
     assert r.returncode in (0, 1), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
     assert "checks failed" in r.stdout or "all checks passed" in r.stdout
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_planners_survive_random_layouts(mock_runtime, seed):
+    """Random element types, shapes, steps (1 to 4), offsets, transposes and
+    axis sets through the reduction and elementwise planners (an 8-byte type
+    stepping by four once gave the row planner a vector width of zero)."""
+    r = subprocess.run([sys.executable, os.path.join("tests", "planner_random_layouts.py"), str(seed), "100"],
+                       cwd=ROOT, env=dict(os.environ, LD_PRELOAD=mock_runtime), capture_output=True,
+                       text=True, timeout=900)
+    assert r.returncode == 0 and "planner ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
