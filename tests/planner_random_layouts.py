@@ -49,4 +49,12 @@ for case in range(cases):
         assert np.asarray(i).shape == want
     if dt != "bool":
         assert elemwise2(g, "+", g, g).shape == view.shape
+    # the copy family: a contiguous copy in either order, a cast, an assignment
+    # through a stepped key, a gather along the first axis
+    assert g.copy("C").shape == view.shape and g.copy("F").shape == view.shape
+    assert g.astype("float32" if dt != "float32" else "int32").shape == view.shape
+    if view.shape[0] > 1:
+        g[::2] = g[::2].copy()
+        picks = rng.integers(0, view.shape[0], size=int(rng.integers(1, 40)))
+        assert g.take1(ga.array(picks, context=ctx)).shape == (len(picks),) + view.shape[1:]
 print("planner ok")
