@@ -73,3 +73,12 @@ def test_planners_survive_random_layouts(mock_runtime, seed):
                        cwd=ROOT, env=dict(os.environ, LD_PRELOAD=mock_runtime), capture_output=True,
                        text=True, timeout=900)
     assert r.returncode == 0 and "planner ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
+
+
+def test_views_follow_numpy_on_random_chains(mock_runtime):
+    """Chains of indexing, transposition and reshaping: shape, strides, byte
+    offset and contiguity flags against NumPy's at every step."""
+    r = subprocess.run([sys.executable, os.path.join("tests", "views_random_walk.py"), "0", "3000"],
+                       cwd=ROOT, env=dict(os.environ, LD_PRELOAD=mock_runtime), capture_output=True,
+                       text=True, timeout=600)
+    assert r.returncode == 0 and "views ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
