@@ -7,6 +7,8 @@ elements followed by the full fp32 sum of a 2^28-element array (two-pass grid
 reduction).  Inputs are resident in HBM before the timed region.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+    python bench.py --only NAME [--steps K]     one kernel per step, for profiler runs
+    python bench.py --list                      the names --only takes
 
 prints ONE JSON line:
   metric / value / unit   achieved algorithmic GB/s of the step
@@ -14,11 +16,14 @@ prints ONE JSON line:
                           its launches timed with HIP events on the library's
                           own stream inside the timed region
   cpu_baseline            the CPU restatement of the reference's kernels
-                          (oracle/, one host core) on a bounded sample
-  per_config              every configuration of the benchmark: GB/s, fraction of peak, us/call,
-                          NumPy's time on the host next to it
+                          (oracle/, one host core) on a bounded sample, NumPy
+                          next to it, and what a probe for a CPU OpenCL device
+                          (the reference's own backend) found
+  per_config              every configuration of the benchmark: GB/s, fraction
+                          of peak, us/call, NumPy's time on the host next to it
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -30,193 +35,34 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
-# HBM bytes per launch of the flat elementwise kernel at 2^28 elements, from
-# two counter runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known
-# size; the runs and the arithmetic are in
-# profiles/elem_flat_fp32_2p28_hbm_traffic.md.  Counters cannot be read from
-# inside this process, so the figure is carried here for the shape it was
-# measured on.
-MEASURED_TRAFFIC = {28: 3219920146}
-MEASURED_TRAFFIC_SUM = {28: 1073807338}   # redux_row of the full sum, same file
+
+# HBM bytes per call measured with the profiler's byte counters (two runs per
+# configuration, FETCH_SIZE then WRITE_SIZE, each scaled by what the same
+# counter reads for a copy kernel of known size).  Counters cannot be read
+# from inside this process, so the figures are carried here, each with the
+# hash of the kernel text it was measured on (hip_last_launch_hash): when the
+# kernel being timed is generated differently, the figure does not describe
+# it any more and the line says "traffic": null.  The runs and the arithmetic
+# are in profiles/hbm_traffic_all_configs.md.
+MEASURED_TRAFFIC = {
+    # name: (kernel text hash, HBM bytes per call)
+}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--quick", action="store_true", help="skip the per-config table")
-    ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count")
-    ap.add_argument("--only", choices=["step", "elem", "sum", "copy"], default="step",
-                    help="launch only one kernel per step (for profiler runs): the elementwise "
-                         "kernel, the sum, or a plain copy dst = src of the same size whose "
-                         "traffic is known (4*n read + 4*n written) to scale byte counters by")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
-                 "(--gpus %d refused; run with --gpus 1)" % args.gpus)
-
-    import libgpuarray_amd as ga
-    from libgpuarray_amd import reduction as R
-
-    ctx = ga.init("hip0")
-    n = 1 << args.log2n
-    K, W = args.steps, args.warmup
-
-    # ---- synthetic inputs, resident before timing -------------------------------
-    rng = np.random.default_rng(0)
-    a_h = rng.uniform(-1, 1, n).astype(np.float32)
-    b_h = rng.uniform(-1, 1, n).astype(np.float32)
-    x_h = np.random.default_rng(3).standard_normal(n, dtype=np.float32)
-    a, b, x = (ga.array(v, context=ctx) for v in (a_h, b_h, x_h))
-    c = ga.empty((n,), "float32", context=ctx)
-    s = ga.empty((), "float32", context=ctx)
-    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f",
-                          [ga.arg("a", "float32", read=True), ga.arg("b", "float32", read=True),
-                           ga.arg("c", "float32", write=True)])
-    summ = ga.GpuReduction(ctx, "sum", "float32")
-
-    copy = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", "float32", read=True),
-                                             ga.arg("dst", "float32", write=True)])
-    only = args.only
-
-    def step(i=None):
-        if i is not None:
-            ctx.mark(3 * i)
-        if only in ("step", "elem"):
-            elem(a, b, c)
-        elif only == "copy":
-            copy(a, c)
-        if i is not None:
-            ctx.mark(3 * i + 1)
-        if only in ("step", "sum"):
-            summ(x, [0], d0=s)
-        if i is not None:
-            ctx.mark(3 * i + 2)
-
-    for _ in range(W):
-        step()
-    ctx.sync()
-    t0 = time.perf_counter()
-    for i in range(K):
-        step(i)
-    ctx.sync()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / K
-
-    elem_ms = np.array([ctx.elapsed(3 * i, 3 * i + 1) for i in range(K)])
-    sum_ms = np.array([ctx.elapsed(3 * i + 1, 3 * i + 2) for i in range(K)])
-    elem_bytes = 3 * 4 * n
-    sum_bytes = 4 * n + 4
-    step_bytes = elem_bytes + sum_bytes
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
-
-    if only != "step":
-        # profiler run: report the one kernel that was launched and stop
-        ms = elem_ms if only in ("elem", "copy") else sum_ms
-        nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
-        print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
-                          "bytes_per_launch": nbytes,
-                          "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1)}))
-        return
-
-    # parity spot-check of what was just timed
-    got = np.asarray(c[:4096])
-    assert np.array_equal(got, a_h[:4096] * b_h[:4096] + np.float32(0.5)), "elementwise result wrong"
-    ref_sum = float(x_h.sum(dtype=np.float64))
-    assert abs(float(np.asarray(s)) - ref_sum) <= 1e-5 * abs(ref_sum), "sum result wrong"
-
-    elem_avg = float(elem_ms.mean())
-    achieved = elem_bytes / (elem_avg * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "elem (flat GpuElemwise kernel, c = a*b + 0.5f)",
-                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC.get(args.log2n),
-                "avg_launch_us": round(elem_avg * 1e3, 2),
-                "median_launch_us": round(float(np.median(elem_ms)) * 1e3, 2),
-                "algorithmic_bytes_per_launch": elem_bytes}
-    sum_avg = float(sum_ms.mean())
-    sum_gbs = sum_bytes / (sum_avg * 1e-3) / 1e9
-    second = {"kernel": "redux_row + redux_final (full fp32 sum, two passes)",
-              "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
-              "achieved": round(sum_gbs, 1), "frac": round(sum_gbs / HBM_PEAK_GBS, 4),
-              "traffic": MEASURED_TRAFFIC_SUM.get(args.log2n),
-              "avg_launch_us": round(sum_avg * 1e3, 2),
-              "algorithmic_bytes_per_launch": sum_bytes}
-
-    # A second yardstick next to the published peak: what the driver's own
-    # device-to-device copy (hipMemcpyDtoDAsync on the library's stream)
-    # sustains on this box, reads plus writes.
-    import ctypes as C
-    from libgpuarray_amd import _lib as _L
-    hip = C.CDLL("libamdhip64.so")
-    stream = C.c_void_p(_L.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
-    get_ptr = _L.extension("hip_get_ptr", C.c_void_p, [C.c_void_p])
-    src_p, dst_p = C.c_void_p(get_ptr(a.ga.data)), C.c_void_p(get_ptr(c.ga.data))
-    for i in range(3 + 10):
-        if i >= 3:
-            ctx.mark(2 * (i - 3))
-        assert hip.hipMemcpyDtoDAsync(dst_p, src_p, C.c_size_t(4 * n), stream) == 0
-        if i >= 3:
-            ctx.mark(2 * (i - 3) + 1)
-    ctx.sync()
-    copy_ms = float(np.mean([ctx.elapsed(2 * i, 2 * i + 1) for i in range(10)]))
-    copy_gbs = 8 * n / (copy_ms * 1e-3) / 1e9
-    roofline["driver_copy_GBps"] = round(copy_gbs, 1)
-    roofline["frac_of_driver_copy"] = round(achieved / copy_gbs, 4)
-
-    cpu = cpu_baseline(a_h, b_h, x_h)
-    out = {
-        "metric": "achieved HBM GB/s for elemwise + reduce (fp32, 2^%d elements)" % args.log2n,
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "fp32 elementwise c=a*b+0.5f over 2^%d contiguous elements + "
-                               "full fp32 sum of 2^%d elements (two-pass grid reduction); "
-                               "seeds 0 and 3" % (args.log2n, args.log2n),
-                   "bytes_per_step": step_bytes, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "roofline_sum": second, "cpu_baseline": cpu,
-        "device": ctx.devname,
-    }
-    del a, b, c, x, a_h, b_h, x_h
-    if not args.quick:
-        out["per_config"] = per_config(ctx, ga, R)
-    print(json.dumps(out))
+def traffic_for(name, kernel_hash):
+    rec = MEASURED_TRAFFIC.get(name)
+    if rec is None:
+        return None, "no counter run recorded for this configuration"
+    if rec[0] != kernel_hash:
+        return None, ("the counter run was made on kernel text %s; the kernel timed here is %s"
+                      % (rec[0], kernel_hash))
+    return rec[1], None
 
 
-def cpu_baseline(a_h, b_h, x_h):
-    """The reference's kernels restated on the CPU (oracle/), one core, on the
-    first 2^26 elements of the same inputs, twenty repetitions (about 10 s)."""
-    from oracle import oracle as O
-    m = min(1 << 26, a_h.size)
-    a, b, x = a_h[:m], b_h[:m], x_h[:m]
-    c = np.empty(m, np.float32)
-    reps = 20
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        O.elemwise_contig_muladd(a, b, c)           # flat kernel, src/gpuarray_elemwise.c:472-532
-    t1 = time.perf_counter()
-    for _ in range(reps):
-        O.reduk("sum", x, [0], "float32", ls=256)   # one group of 256 lanes, pygpu/reduction.py:85-132
-    t2 = time.perf_counter()
-    te, ts = (t1 - t0) / reps, (t2 - t1) / reps
-    tn0 = time.perf_counter()
-    for _ in range(reps):
-        np.add(np.multiply(a, b, out=c), np.float32(0.5), out=c)
-        x.sum()
-    tn = (time.perf_counter() - tn0) / reps
-    bytes_ = 16 * m + 4
-    return {"value": round(bytes_ / (te + ts) / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "first 2^26 elements of the same inputs, %d repetitions; elementwise %.3f s, "
-                      "sum %.3f s per repetition" % (reps, te, ts),
-            "reference_opencl_path": "not runnable (no CPU OpenCL device on the box; the reference "
-                                     "tree does not travel there)",
-            "numpy_value": round(bytes_ / tn / 1e9, 3),
-            "host_cpu_count": os.cpu_count(),
-            "host_affinity": len(os.sched_getaffinity(0))}
-
+# ---- timing helpers -----------------------------------------------------------------
 
 def time_calls(ctx, fn, iters=30, warm=5):
+    """Median microseconds between two marks around one call."""
     for _ in range(warm):
         fn(0)
     ctx.sync()
@@ -225,7 +71,24 @@ def time_calls(ctx, fn, iters=30, warm=5):
         fn(i)
         ctx.mark(2 * i + 1)
     ms = np.array([ctx.elapsed(2 * i, 2 * i + 1) for i in range(iters)])
-    return float(np.median(ms)) * 1e3   # microseconds
+    return float(np.median(ms)) * 1e3
+
+
+def time_kernels(ctx, fn, iters=30, warm=3):
+    """Median microseconds one call's kernels run on the device: every launch
+    carries its own start and stop event, the durations of the launches of one
+    call are added up.  Returns (us, launches per call)."""
+    for _ in range(warm):
+        fn(0)
+    ctx.sync()
+    ctx.kernel_timing(True)
+    for i in range(iters):
+        fn(i)
+    ms = np.array(ctx.kernel_times())
+    ctx.kernel_timing(False)
+    per = max(len(ms) // iters, 1)
+    per_call = ms[:per * iters].reshape(iters, per).sum(axis=1)
+    return float(np.median(per_call)) * 1e3, per
 
 
 def time_stream(ctx, fn, iters=40, warm=5):
@@ -248,46 +111,35 @@ def host_time(fn, reps=3):
     return (time.perf_counter() - t0) / reps * 1e6
 
 
-def per_config(ctx, ga, R):
-    """Every configuration of the benchmark.  `cold` rotates over four buffer sets so that a
-    footprint below the 256 MB Infinity Cache is not served from it; `warm`
-    reuses one set."""
-    res = {}
-    rot = 4
+# ---- the configurations -------------------------------------------------------------
+# Each builder returns a dict: bytes (algorithmic bytes per call), call(i) (one
+# call on buffer set i), sets (number of independent buffer sets; > 1 when the
+# footprint is below the 256 MB Infinity Cache, so that rotating over them
+# shows HBM and not the cache), numpy (the same work on the host), check()
+# (parity of the last call against NumPy, run outside any timed region), note.
 
-    def entry(name, nbytes, us_cold, us_warm, numpy_us, note=None, us_stream=None):
-        e = {"algorithmic_bytes": nbytes, "us_per_call_cold": round(us_cold, 2),
-             "GBps_cold": round(nbytes / us_cold / 1e3, 1),
-             "frac_cold": round(nbytes / us_cold / 1e3 / HBM_PEAK_GBS, 4),
-             "us_per_call_warm": round(us_warm, 2), "GBps_warm": round(nbytes / us_warm / 1e3, 1),
-             "numpy_us_per_call": round(numpy_us, 1), "numpy_cores": 1}
-        if us_stream is not None:     # cold buffers, calls issued back to back
-            e["us_per_call_back_to_back"] = round(us_stream, 2)
-            e["GBps_back_to_back"] = round(nbytes / us_stream / 1e3, 1)
-        if note:
-            e["note"] = note
-        res[name] = e
+f32 = "float32"
+ROT = 4
 
-    f32 = "float32"
-    # C1: contiguous 2^24
+
+def cfg_c1(ctx, ga, R):
     n = 1 << 24
     rng = np.random.default_rng(0)
     a_h, b_h = rng.uniform(-1, 1, n).astype(np.float32), rng.uniform(-1, 1, n).astype(np.float32)
-    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [ga.arg("a", f32, read=True),
-                                                   ga.arg("b", f32, read=True),
+    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [ga.arg("a", f32, read=True), ga.arg("b", f32, read=True),
                                                    ga.arg("c", f32, write=True)])
     sets = [(ga.array(a_h, context=ctx), ga.array(b_h, context=ctx), ga.empty((n,), f32, context=ctx))
-            for _ in range(rot)]
-    cold = time_calls(ctx, lambda i: elem(*sets[i % rot]))
-    warm = time_calls(ctx, lambda i: elem(*sets[0]))
-    b2b = time_stream(ctx, lambda i: elem(*sets[i % rot]))
+            for _ in range(ROT)]
     c_h = np.empty_like(a_h)
-    entry("C1_elemwise_2^24", 12 * n, cold, warm,
-          host_time(lambda: np.add(np.multiply(a_h, b_h, out=c_h), np.float32(0.5), out=c_h)),
-          us_stream=b2b)
-    del sets
 
-    # C2: transposed view + two broadcast operands
+    def check():
+        want = a_h * b_h + np.float32(0.5)
+        return all(np.array_equal(np.asarray(s[2]), want) for s in sets)
+    return {"bytes": 12 * n, "call": lambda i: elem(*sets[i % ROT]), "sets": ROT, "check": check,
+            "numpy": lambda: np.add(np.multiply(a_h, b_h, out=c_h), np.float32(0.5), out=c_h)}
+
+
+def cfg_c2(ctx, ga, R):
     rng = np.random.default_rng(1)
     A = rng.normal(0, 1, (4096, 4096)).astype(np.float32)
     B = rng.normal(0, 1, (1, 4096)).astype(np.float32)
@@ -295,76 +147,111 @@ def per_config(ctx, ga, R):
     k2 = ga.GpuElemwise(ctx, "out = a + b*c", [ga.arg("a", f32, read=True), ga.arg("b", f32, read=True),
                                                ga.arg("c", f32, read=True), ga.arg("out", f32, write=True)])
     sets = [(ga.array(A, context=ctx).T, ga.array(B, context=ctx), ga.array(Cc, context=ctx),
-             ga.empty((4096, 4096), f32, context=ctx)) for _ in range(rot)]
-    cold = time_calls(ctx, lambda i: k2(*sets[i % rot]))
-    warm = time_calls(ctx, lambda i: k2(*sets[0]))
-    b2b = time_stream(ctx, lambda i: k2(*sets[i % rot]))
-    entry("C2_transposed_broadcast_4096", 2 * 4096 * 4096 * 4 + 2 * 4096 * 4, cold, warm,
-          host_time(lambda: A.T + B * Cc), us_stream=b2b)
-    del sets
+             ga.empty((4096, 4096), f32, context=ctx)) for _ in range(ROT)]
 
-    # C3a: sum over axis 1 of (8192, 8192)
+    def check():
+        want = A.T + B * Cc
+        return all(np.array_equal(np.asarray(s[3]), want) for s in sets)
+    return {"bytes": 2 * 4096 * 4096 * 4 + 2 * 4096 * 4, "call": lambda i: k2(*sets[i % ROT]), "sets": ROT,
+            "check": check, "numpy": lambda: A.T + B * Cc}
+
+
+def cfg_c3a(ctx, ga, R):
     X = np.random.default_rng(2).standard_normal((8192, 8192), dtype=np.float32)
     op = ga.GpuReduction(ctx, "sum", f32)
-    sets = [(ga.array(X, context=ctx), ga.empty((8192,), f32, context=ctx)) for _ in range(rot)]
-    cold = time_calls(ctx, lambda i: op(sets[i % rot][0], [1], d0=sets[i % rot][1]))
-    warm = time_calls(ctx, lambda i: op(sets[0][0], [1], d0=sets[0][1]))
-    b2b = time_stream(ctx, lambda i: op(sets[i % rot][0], [1], d0=sets[i % rot][1]))
-    entry("C3a_sum_axis1_8192x8192", 8192 * 8192 * 4 + 8192 * 4, cold, warm, host_time(lambda: X.sum(axis=1)),
-          us_stream=b2b)
-    del sets
+    sets = [(ga.array(X, context=ctx), ga.empty((8192,), f32, context=ctx)) for _ in range(ROT)]
 
-    # C4: maxandargmax over the last axis of (65536, 1000)
+    def check():
+        want = X.sum(axis=1, dtype=np.float64)
+        mag = np.abs(X).sum(axis=1, dtype=np.float64)
+        tol = np.where(np.abs(want) >= 1e-3 * mag, 1e-5 * np.abs(want), 8 * 2.0 ** -24 * mag)
+        return all(np.all(np.abs(np.asarray(s[1]).astype(np.float64) - want) <= tol) for s in sets)
+    return {"bytes": 8192 * 8192 * 4 + 8192 * 4, "sets": ROT, "check": check,
+            "call": lambda i: op(sets[i % ROT][0], [1], d0=sets[i % ROT][1]),
+            "numpy": lambda: X.sum(axis=1)}
+
+
+def cfg_c4(ctx, ga, R):
     L = np.random.default_rng(4).normal(0, 2, (65536, 1000)).astype(np.float32)
     op4 = ga.GpuReduction(ctx, "maxandargmax", f32)
     sets = [(ga.array(L, context=ctx), ga.empty((65536,), f32, context=ctx),
-             ga.empty((65536,), "int64", context=ctx)) for _ in range(rot)]
-    cold = time_calls(ctx, lambda i: op4(sets[i % rot][0], [1], d0=sets[i % rot][1], d1=sets[i % rot][2]))
-    warm = time_calls(ctx, lambda i: op4(sets[0][0], [1], d0=sets[0][1], d1=sets[0][2]))
-    b2b = time_stream(ctx, lambda i: op4(sets[i % rot][0], [1], d0=sets[i % rot][1], d1=sets[i % rot][2]))
-    entry("C4_maxandargmax_65536x1000", 65536 * 1000 * 4 + 65536 * 12, cold, warm,
-          host_time(lambda: (L.max(axis=1), L.argmax(axis=1))), us_stream=b2b)
-    del sets, L, X, A
+             ga.empty((65536,), "int64", context=ctx)) for _ in range(ROT)]
 
-    # C5: stride-2 view of (256, 512, 1024); at most half of every fetched line is useful
-    shape = (256, 512, 1024)
-    H = np.random.default_rng(5).uniform(-4, 4, shape).astype(np.float16)
+    def check():
+        wm, wa = L.max(axis=1), L.argmax(axis=1)
+        return all(np.array_equal(np.asarray(s[1]), wm) and np.array_equal(np.asarray(s[2]), wa)
+                   for s in sets)
+    return {"bytes": 65536 * 1000 * 4 + 65536 * 12, "sets": ROT, "check": check,
+            "call": lambda i: op4(sets[i % ROT][0], [1], d0=sets[i % ROT][1], d1=sets[i % ROT][2]),
+            "numpy": lambda: (L.max(axis=1), L.argmax(axis=1))}
+
+
+C5_SHAPE = (256, 512, 1024)
+C5_NOTE = ("useful bytes of a stride-2 view: every fetched line is half used, so the ceiling in "
+           "useful bytes is 50 % of peak (268 MB footprint: no cold/warm split)")
+
+
+def cfg_c5_f16(ctx, ga, R):
+    H = np.random.default_rng(5).uniform(-4, 4, C5_SHAPE).astype(np.float16)
     gh = ga.array(H, context=ctx)[:, :, ::2]
     o5 = ga.empty((512,), f32, context=ctx)
     oph = ga.GpuReduction(ctx, "sum", "float16")
-    us = time_calls(ctx, lambda i: oph(gh, [0, 2], d0=o5))
-    entry("C5_fp16_sum_axes02", 256 * 512 * 512 * 2 + 2048, us, us,
-          host_time(lambda: H[:, :, ::2].sum(axis=(0, 2), dtype=np.float32), reps=1),
-          "useful bytes; physical traffic is ~2x (stride-2 view, 268 MB footprint: no cold/warm split)")
-    del gh, H
-    I = np.random.default_rng(6).integers(-1000, 1001, shape, dtype=np.int32)
+
+    def check():
+        want = H[:, :, ::2].astype(np.float64).sum(axis=(0, 2))
+        return bool(np.all(np.abs(np.asarray(o5) - want) <= 1e-2 * np.abs(want) + 1e-2 * 4 * 256))
+    return {"bytes": 256 * 512 * 512 * 2 + 2048, "call": lambda i: oph(gh, [0, 2], d0=o5), "sets": 1,
+            "check": check, "numpy": lambda: H[:, :, ::2].sum(axis=(0, 2), dtype=np.float32),
+            "numpy_reps": 1, "note": C5_NOTE}
+
+
+def cfg_c5_i32(ctx, ga, R):
+    I = np.random.default_rng(6).integers(-1000, 1001, C5_SHAPE, dtype=np.int32)
     gi = ga.array(I, context=ctx)[:, :, ::2]
     o5i = ga.empty((256, 512), "int64", context=ctx)
     opi = ga.GpuReduction(ctx, "sum", "int32")
-    us = time_calls(ctx, lambda i: opi(gi, [1], d0=o5i))
-    entry("C5_int32_sum_axis1", 256 * 512 * 512 * 4 + 256 * 512 * 8, us, us,
-          host_time(lambda: I[:, :, ::2].sum(axis=1), reps=1), "useful bytes; stride-2 view")
-    del gi, I
-    U = (np.random.default_rng(7).random(shape) < 1e-4).astype(np.uint8)
-    gu = ga.array(U, context=ctx)[:, :, ::2]
-    ob = ga.empty((256, 512), "bool", context=ctx)
-    for nm in ("any", "all"):
-        opb = ga.GpuReduction(ctx, nm, "uint8")
-        us = time_calls(ctx, lambda i: opb(gu, [2], d0=ob))
-        entry("C5_uint8_%s_axis2" % nm, 256 * 512 * 512 + 256 * 512, us, us,
-              host_time(lambda: getattr(U[:, :, ::2], nm)(axis=2), reps=1), "useful bytes; stride-2 view")
-    del gu, U
+    return {"bytes": 256 * 512 * 512 * 4 + 256 * 512 * 8, "call": lambda i: opi(gi, [1], d0=o5i), "sets": 1,
+            "check": lambda: np.array_equal(np.asarray(o5i), I[:, :, ::2].sum(axis=1, dtype=np.int64)),
+            "numpy": lambda: I[:, :, ::2].sum(axis=1), "numpy_reps": 1, "note": C5_NOTE}
 
-    # Beyond the benchmark's own shapes: an expression feeding a reduction in one pass
-    # (dot product of two 2^27 vectors; the two-pass alternative writes and
-    # re-reads a 512 MiB temporary) and a row gather.
+
+def _cfg_c5_u8(nm):
+    def build(ctx, ga, R):
+        U = (np.random.default_rng(7).random(C5_SHAPE) < 1e-4).astype(np.uint8)
+        gu = ga.array(U, context=ctx)[:, :, ::2]
+        ob = ga.empty((256, 512), "bool", context=ctx)
+        opb = ga.GpuReduction(ctx, nm, "uint8")
+        return {"bytes": 256 * 512 * 512 + 256 * 512, "call": lambda i: opb(gu, [2], d0=ob), "sets": 1,
+                "check": lambda: np.array_equal(np.asarray(ob), getattr(U[:, :, ::2], nm)(axis=2)),
+                "numpy": lambda: getattr(U[:, :, ::2], nm)(axis=2), "numpy_reps": 1, "note": C5_NOTE}
+    return build
+
+
+def cfg_dot(ctx, ga, R):
+    # Beyond the benchmark's own shapes: an expression feeding a reduction in
+    # one pass (dot product of two 2^27 vectors; the two-pass alternative
+    # writes and re-reads a 512 MiB temporary).
     n = 1 << 27
     rng = np.random.default_rng(8)
     p_h, q_h = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
     gp, gq = ga.array(p_h, context=ctx), ga.array(q_h, context=ctx)
     dot = R.MapReduction(ctx, "sum", f32, "p*q", [R.ArrayArg(f32, "p"), R.ArrayArg(f32, "q")])
     od = ga.empty((), f32, context=ctx)
-    us = time_calls(ctx, lambda i: dot([gp, gq], [0], d0=od))
+
+    def check():
+        want = float(np.dot(p_h.astype(np.float64), q_h.astype(np.float64)))
+        mag = float(np.dot(np.abs(p_h).astype(np.float64), np.abs(q_h).astype(np.float64)))
+        return abs(float(np.asarray(od)) - want) <= max(1e-5 * abs(want), 8 * 2.0 ** -24 * mag)
+    return {"bytes": 8 * n + 4, "call": lambda i: dot([gp, gq], [0], d0=od), "sets": 1, "check": check,
+            "numpy": lambda: np.dot(p_h, q_h), "note": "one kernel pass over both inputs"}
+
+
+def cfg_dot_two_pass(ctx, ga, R):
+    n = 1 << 27
+    rng = np.random.default_rng(8)
+    p_h, q_h = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
+    gp, gq = ga.array(p_h, context=ctx), ga.array(q_h, context=ctx)
+    od = ga.empty((), f32, context=ctx)
     tmp = ga.empty((n,), f32, context=ctx)
     mul = ga.GpuElemwise(ctx, "t = p*q", [ga.arg("p", f32, read=True), ga.arg("q", f32, read=True),
                                           ga.arg("t", f32, write=True)])
@@ -373,21 +260,83 @@ def per_config(ctx, ga, R):
     def two_pass(i):
         mul(gp, gq, tmp)
         opsum(tmp, [0], d0=od)
-    us2 = time_calls(ctx, two_pass)
-    entry("F4_dot_2x2^27_fused", 8 * n + 4, us, us, host_time(lambda: np.dot(p_h, q_h)),
-          "one kernel pass; elementwise-then-sum takes %.1f us for the same result" % us2)
-    del gp, gq, tmp, p_h, q_h
+    return {"bytes": 8 * n + 4, "call": two_pass, "sets": 1, "numpy": lambda: np.dot(p_h, q_h),
+            "note": "the same result as F4_dot_2x2^27_fused by elementwise multiply, then sum: "
+                    "16 bytes per element instead of 8 cross the memory bus"}
+
+
+def cfg_take1(ctx, ga, R):
     rows, width = 65536, 1024
     V = np.random.default_rng(9).standard_normal((rows, width), dtype=np.float32)
     idx = np.random.default_rng(10).permutation(rows)
     gv, gidx = ga.array(V, context=ctx), ga.array(idx, context=ctx)
-    us = time_calls(ctx, lambda i: gv.take1(gidx))
-    entry("F2_take1_65536x1024_rows", 2 * rows * width * 4 + rows * 8, us, us,
-          host_time(lambda: V.take(idx, axis=0)), "includes the result's allocation and the bounds-flag read-back")
-    del gv, gidx, V
+    last = [None]
 
-    # launch-latency floor: small shapes, host-side wall time per call included
+    def call(i):
+        last[0] = gv.take1(gidx)
+    return {"bytes": 2 * rows * width * 4 + rows * 8, "call": call, "sets": 1,
+            "check": lambda: np.array_equal(np.asarray(last[0]), V.take(idx, axis=0)),
+            "numpy": lambda: V.take(idx, axis=0),
+            "note": "includes the result's allocation and the bounds-flag read-back"}
+
+
+CONFIGS = [
+    ("C1_elemwise_2^24", cfg_c1),
+    ("C2_transposed_broadcast_4096", cfg_c2),
+    ("C3a_sum_axis1_8192x8192", cfg_c3a),
+    ("C4_maxandargmax_65536x1000", cfg_c4),
+    ("C5_fp16_sum_axes02", cfg_c5_f16),
+    ("C5_int32_sum_axis1", cfg_c5_i32),
+    ("C5_uint8_any_axis2", _cfg_c5_u8("any")),
+    ("C5_uint8_all_axis2", _cfg_c5_u8("all")),
+    ("F4_dot_2x2^27_fused", cfg_dot),
+    ("F4_dot_2x2^27_two_pass", cfg_dot_two_pass),
+    ("F2_take1_65536x1024_rows", cfg_take1),
+]
+STEP_MODES = ("step", "elem", "sum", "copy")
+
+
+def measure_config(ctx, name, cfg):
+    nbytes, call, sets = cfg["bytes"], cfg["call"], cfg["sets"]
+    call(0)
+    khash = ctx.last_launch_hash()
+    cold = time_calls(ctx, call)
+    kern, launches = time_kernels(ctx, call)
+    e = {"algorithmic_bytes": nbytes,
+         "us_per_call_cold": round(cold, 2), "GBps_cold": round(nbytes / cold / 1e3, 1),
+         "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 4),
+         "kernel_us_cold": round(kern, 2), "GBps_kernel_cold": round(nbytes / kern / 1e3, 1),
+         "frac_kernel_cold": round(nbytes / kern / 1e3 / HBM_PEAK_GBS, 4),
+         "launches_per_call": launches, "kernel_text_hash": khash}
+    if sets > 1:
+        warm = time_calls(ctx, lambda i: call(0))
+        e["us_per_call_warm"] = round(warm, 2)
+        e["GBps_warm"] = round(nbytes / warm / 1e3, 1)
+    b2b = time_stream(ctx, call)
+    e["us_per_call_back_to_back"] = round(b2b, 2)
+    e["GBps_back_to_back"] = round(nbytes / b2b / 1e3, 1)
+    traffic, why = traffic_for(name, khash)
+    e["traffic"] = traffic
+    if traffic is not None:
+        e["traffic_over_algorithmic"] = round(traffic / nbytes, 4)
+    else:
+        e["traffic_note"] = why
+    if "check" in cfg:
+        ctx.sync()
+        e["parity_ok"] = bool(cfg["check"]())
+        assert e["parity_ok"], "%s: result differs from NumPy" % name
+    e["numpy_us_per_call"] = round(host_time(cfg["numpy"], reps=cfg.get("numpy_reps", 3)), 1)
+    e["numpy_cores"] = 1
+    if cfg.get("note"):
+        e["note"] = cfg["note"]
+    return e
+
+
+def latency_table(ctx, ga):
+    """Launch-latency floor: small shapes, host-side wall time per call included."""
     lat = {}
+    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [ga.arg("a", f32, read=True), ga.arg("b", f32, read=True),
+                                                   ga.arg("c", f32, write=True)])
     for m in (1, 1 << 10, 1 << 16):
         sa, sb, sc = (ga.zeros((m,), f32, context=ctx) for _ in range(3))
         dev_us = time_calls(ctx, lambda i: elem(sa, sb, sc), iters=100)
@@ -398,15 +347,17 @@ def per_config(ctx, ga, R):
         ctx.sync()
         lat["elemwise_n=%d" % m] = {"device_us": round(dev_us, 2),
                                     "wall_us_per_call": round((time.perf_counter() - t0) / 200 * 1e6, 2)}
+    op = ga.GpuReduction(ctx, "sum", f32)
+    op4 = ga.GpuReduction(ctx, "maxandargmax", f32)
     sm = ga.zeros((64, 64), f32, context=ctx)
     so = ga.empty((64,), f32, context=ctx)
     lat["sum_64x64_axis1"] = {"device_us": round(time_calls(ctx, lambda i: op(sm, [1], d0=so), iters=100), 2)}
     mm = ga.zeros((64, 1000), f32, context=ctx)
     mo, mi = ga.empty((64,), f32, context=ctx), ga.empty((64,), "int64", context=ctx)
-    lat["maxandargmax_64x1000"] = {"device_us": round(time_calls(ctx, lambda i: op4(mm, [1], d0=mo, d1=mi), iters=100), 2)}
+    lat["maxandargmax_64x1000"] = {
+        "device_us": round(time_calls(ctx, lambda i: op4(mm, [1], d0=mo, d1=mi), iters=100), 2)}
     # the same small calls recorded once into a HIP graph on the library's stream and replayed
     try:
-        import ctypes as C
         from libgpuarray_amd import _lib
         hip = C.CDLL("libamdhip64.so")
         stream = C.c_void_p(_lib.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
@@ -439,8 +390,298 @@ def per_config(ctx, ga, R):
                 hip.hipGraphDestroy(graph)
     except OSError:
         pass
-    res["latency"] = lat
+    return lat
+
+
+# ---- the CPU leg ----------------------------------------------------------------------
+
+def probe_opencl_cpu():
+    """Looks for a CPU OpenCL device, the kind the reference's OpenCL backend
+    would run on (PoCL): platform and device counts as found, nothing else is
+    touched.  The reference tree does not travel to the GPU box; its generated
+    kernels do, as fixtures (tests/golden/reference_kernels/), with a host
+    runner that applies the reference's launch rule (oracle/opencl_runner.py),
+    used only when this probe finds a CPU device."""
+    CL_DEVICE_TYPE_CPU, CL_DEVICE_TYPE_ALL = 1 << 1, 0xFFFFFFFF
+    res = {"library": None, "platforms": 0, "cpu_devices": 0, "devices_of_any_type": 0}
+    cl = None
+    for name in ("libOpenCL.so.1", "libOpenCL.so"):
+        try:
+            cl = C.CDLL(name)
+            res["library"] = name
+            break
+        except OSError:
+            continue
+    if cl is None:
+        res["status"] = "not runnable (no OpenCL loader library on the box)"
+        return res
+    nplat = C.c_uint(0)
+    if cl.clGetPlatformIDs(0, None, C.byref(nplat)) != 0 or nplat.value == 0:
+        res["status"] = "not runnable (the OpenCL loader reports no platform)"
+        return res
+    plats = (C.c_void_p * nplat.value)()
+    cl.clGetPlatformIDs(nplat.value, plats, None)
+    res["platforms"] = int(nplat.value)
+    cl.clGetDeviceIDs.argtypes = [C.c_void_p, C.c_ulong, C.c_uint, C.c_void_p, C.POINTER(C.c_uint)]
+    for p in plats:
+        for key, kind in (("cpu_devices", CL_DEVICE_TYPE_CPU), ("devices_of_any_type", CL_DEVICE_TYPE_ALL)):
+            nd = C.c_uint(0)
+            if cl.clGetDeviceIDs(p, kind, 0, None, C.byref(nd)) == 0:
+                res[key] += int(nd.value)
+    res["status"] = ("CPU OpenCL device present" if res["cpu_devices"] else
+                     "not runnable (no CPU OpenCL device on the box: %d platform(s), %d device(s) of other "
+                     "types; the reference tree does not travel there)"
+                     % (res["platforms"], res["devices_of_any_type"]))
     return res
+
+
+def cpu_baseline(a_h, b_h, x_h):
+    """The reference's kernels restated on the CPU (oracle/), one core, on the
+    first 2^26 elements of the same inputs, twenty repetitions (about 10 s)."""
+    from oracle import oracle as O
+    m = min(1 << 26, a_h.size)
+    a, b, x = a_h[:m], b_h[:m], x_h[:m]
+    c = np.empty(m, np.float32)
+    reps = 20
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        O.elemwise_contig_muladd(a, b, c)           # flat kernel, src/gpuarray_elemwise.c:472-532
+    t1 = time.perf_counter()
+    for _ in range(reps):
+        O.reduk("sum", x, [0], "float32", ls=256)   # one group of 256 lanes, pygpu/reduction.py:85-132
+    t2 = time.perf_counter()
+    te, ts = (t1 - t0) / reps, (t2 - t1) / reps
+    tn0 = time.perf_counter()
+    for _ in range(reps):
+        np.add(np.multiply(a, b, out=c), np.float32(0.5), out=c)
+        x.sum()
+    tn = (time.perf_counter() - tn0) / reps
+    bytes_ = 16 * m + 4
+    out = {"value": round(bytes_ / (te + ts) / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": "first 2^26 elements of the same inputs, %d repetitions; elementwise %.3f s, "
+                     "sum %.3f s per repetition" % (reps, te, ts),
+           "numpy_value": round(bytes_ / tn / 1e9, 3),
+           "host_cpu_count": os.cpu_count(),
+           "host_affinity": len(os.sched_getaffinity(0))}
+    probe = probe_opencl_cpu()
+    out["reference_opencl_path"] = probe["status"]
+    out["opencl_probe"] = {k: probe[k] for k in ("library", "platforms", "cpu_devices", "devices_of_any_type")}
+    if probe["cpu_devices"]:
+        try:
+            from oracle import opencl_runner
+            out["reference_opencl"] = opencl_runner.run_contig_muladd(a, b, device_type="cpu")
+        except Exception as e:   # the probe saw a device that then could not be used
+            out["reference_opencl"] = {"error": repr(e)}
+    return out
+
+
+# ---- main -----------------------------------------------------------------------------
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="skip the per-config table")
+    ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count")
+    ap.add_argument("--list", action="store_true", help="print the names --only takes")
+    ap.add_argument("--only", default="step",
+                    help="launch only one kernel per step (for profiler runs): 'elem', 'sum', or 'copy' "
+                         "(a plain copy dst = src of 2^log2n floats whose traffic is known, 4*n read + "
+                         "4*n written, to scale byte counters by), or the name of a per-config entry")
+    args = ap.parse_args()
+    names = [n for n, _ in CONFIGS]
+    if args.list:
+        print("\n".join(list(STEP_MODES) + names))
+        return
+    if args.only not in STEP_MODES and args.only not in names:
+        sys.exit("--only %s: not one of %s" % (args.only, ", ".join(list(STEP_MODES) + names)))
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
+                 "(--gpus %d refused; run with --gpus 1)" % args.gpus)
+
+    import libgpuarray_amd as ga
+    from libgpuarray_amd import reduction as R
+
+    ctx = ga.init("hip0")
+    K, W = args.steps, args.warmup
+
+    if args.only in names:
+        # profiler run of one configuration: K calls, rotating over its buffer sets
+        cfg = dict(CONFIGS)[args.only](ctx, ga, R)
+        for i in range(W):
+            cfg["call"](i)
+        ctx.sync()
+        khash = ctx.last_launch_hash()
+        ctx.mark(0)
+        for i in range(K):
+            cfg["call"](i)
+        ctx.mark(1)
+        us = ctx.elapsed(0, 1) * 1e3 / K
+        print(json.dumps({"only": args.only, "calls": K, "warmup_calls": W, "us_per_call_back_to_back": round(us, 2),
+                          "algorithmic_bytes_per_call": cfg["bytes"], "kernel_text_hash": khash,
+                          "GBps": round(cfg["bytes"] / us / 1e3, 1)}))
+        return
+
+    n = 1 << args.log2n
+    # ---- synthetic inputs, resident before timing -------------------------------
+    rng = np.random.default_rng(0)
+    a_h = rng.uniform(-1, 1, n).astype(np.float32)
+    b_h = rng.uniform(-1, 1, n).astype(np.float32)
+    x_h = np.random.default_rng(3).standard_normal(n, dtype=np.float32)
+    a, b, x = (ga.array(v, context=ctx) for v in (a_h, b_h, x_h))
+    c = ga.empty((n,), "float32", context=ctx)
+    s = ga.empty((), "float32", context=ctx)
+    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f",
+                          [ga.arg("a", "float32", read=True), ga.arg("b", "float32", read=True),
+                           ga.arg("c", "float32", write=True)])
+    summ = ga.GpuReduction(ctx, "sum", "float32")
+    copy = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", "float32", read=True),
+                                             ga.arg("dst", "float32", write=True)])
+    only = args.only
+    hashes = {}
+
+    def step(i=None):
+        if i is not None:
+            ctx.mark(3 * i)
+        if only in ("step", "elem"):
+            elem(a, b, c)
+            hashes["elem"] = ctx.last_launch_hash()
+        elif only == "copy":
+            copy(a, c)
+        if i is not None:
+            ctx.mark(3 * i + 1)
+        if only in ("step", "sum"):
+            summ(x, [0], d0=s)
+        if i is not None:
+            ctx.mark(3 * i + 2)
+
+    for _ in range(W):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(i)
+    ctx.sync()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K
+
+    elem_ms = np.array([ctx.elapsed(3 * i, 3 * i + 1) for i in range(K)])
+    sum_ms = np.array([ctx.elapsed(3 * i + 1, 3 * i + 2) for i in range(K)])
+    elem_bytes = 3 * 4 * n
+    sum_bytes = 4 * n + 4
+    step_bytes = elem_bytes + sum_bytes
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    if only != "step":
+        # profiler run: report the one kernel that was launched and stop
+        ms = elem_ms if only in ("elem", "copy") else sum_ms
+        nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
+        print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
+                          "bytes_per_launch": nbytes, "kernel_text_hash": ctx.last_launch_hash(),
+                          "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1)}))
+        return
+
+    # The same kernels once more with a start and a stop event on every
+    # dispatch: their own durations, the figure a kernel trace reports.
+    ctx.kernel_timing(True)
+    KT = min(K, 20)
+    for _ in range(KT):
+        elem(a, b, c)
+    elem_kernel_ms = np.array(ctx.kernel_times())
+    ctx.kernel_timing(True)
+    for _ in range(KT):
+        summ(x, [0], d0=s)
+    sum_kernel_ms = np.array(ctx.kernel_times())
+    ctx.kernel_timing(False)
+    sum_launches = max(len(sum_kernel_ms) // KT, 1)
+    sum_kernel_ms = sum_kernel_ms[:sum_launches * KT].reshape(KT, sum_launches).sum(axis=1)
+    hashes["sum"] = ctx.last_launch_hash()
+
+    # parity of what was just timed: the whole output, outside the timed region
+    got = np.asarray(c)
+    want = a_h * b_h + np.float32(0.5)
+    assert np.array_equal(got, want), "elementwise result wrong (%d of %d elements differ)" % (
+        int(np.count_nonzero(got != want)), n)
+    del got, want
+    ref_sum = float(x_h.sum(dtype=np.float64))
+    sum_rel_err = abs(float(np.asarray(s)) - ref_sum) / abs(ref_sum)
+    assert sum_rel_err <= 1e-5, "sum result wrong (relative error %.3g)" % sum_rel_err
+
+    elem_avg = float(elem_ms.mean())
+    achieved = elem_bytes / (elem_avg * 1e-3) / 1e9
+    tname = "elem_2^%d" % args.log2n
+    traffic, why = traffic_for(tname, hashes["elem"])
+    roofline = {"bound": "hbm", "kernel": "elem (flat GpuElemwise kernel, c = a*b + 0.5f)",
+                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": traffic,
+                "avg_launch_us": round(elem_avg * 1e3, 2),
+                "median_launch_us": round(float(np.median(elem_ms)) * 1e3, 2),
+                "kernel_us": round(float(elem_kernel_ms.mean()) * 1e3, 2),
+                "kernel_text_hash": hashes["elem"],
+                "parity": "all 2^%d outputs equal NumPy's" % args.log2n,
+                "algorithmic_bytes_per_launch": elem_bytes}
+    if traffic is None:
+        roofline["traffic_note"] = why
+    sum_avg = float(sum_ms.mean())
+    sum_gbs = sum_bytes / (sum_avg * 1e-3) / 1e9
+    traffic_s, why_s = traffic_for("sum_2^%d" % args.log2n, hashes["sum"])
+    second = {"kernel": "redux_row + redux_final (full fp32 sum, two passes)",
+              "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+              "achieved": round(sum_gbs, 1), "frac": round(sum_gbs / HBM_PEAK_GBS, 4),
+              "traffic": traffic_s,
+              "avg_launch_us": round(sum_avg * 1e3, 2),
+              "kernel_us": round(float(sum_kernel_ms.mean()) * 1e3, 2),
+              "kernel_text_hash": hashes["sum"],
+              "relative_error": float("%.3g" % sum_rel_err),
+              "algorithmic_bytes_per_launch": sum_bytes}
+    if traffic_s is None:
+        second["traffic_note"] = why_s
+
+    # A second yardstick next to the published peak: what the driver's own
+    # device-to-device copy (hipMemcpyDtoDAsync on the library's stream)
+    # sustains on this box, reads plus writes.
+    from libgpuarray_amd import _lib as _L
+    hip = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p(_L.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
+    get_ptr = _L.extension("hip_get_ptr", C.c_void_p, [C.c_void_p])
+    src_p, dst_p = C.c_void_p(get_ptr(a.ga.data)), C.c_void_p(get_ptr(c.ga.data))
+    for i in range(3 + 10):
+        if i >= 3:
+            ctx.mark(2 * (i - 3))
+        assert hip.hipMemcpyDtoDAsync(dst_p, src_p, C.c_size_t(4 * n), stream) == 0
+        if i >= 3:
+            ctx.mark(2 * (i - 3) + 1)
+    ctx.sync()
+    copy_ms = float(np.mean([ctx.elapsed(2 * i, 2 * i + 1) for i in range(10)]))
+    copy_gbs = 8 * n / (copy_ms * 1e-3) / 1e9
+    roofline["driver_copy_GBps"] = round(copy_gbs, 1)
+    roofline["frac_of_driver_copy"] = round(achieved / copy_gbs, 4)
+
+    cpu = cpu_baseline(a_h, b_h, x_h)
+    out = {
+        "metric": "achieved HBM GB/s for elemwise + reduce (fp32, 2^%d elements)" % args.log2n,
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fp32 elementwise c=a*b+0.5f over 2^%d contiguous elements + "
+                               "full fp32 sum of 2^%d elements (two-pass grid reduction); "
+                               "seeds 0 and 3" % (args.log2n, args.log2n),
+                   "bytes_per_step": step_bytes, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+        "roofline": roofline, "roofline_sum": second, "cpu_baseline": cpu,
+        "device": ctx.devname,
+    }
+    del a, b, c, x, a_h, b_h, x_h
+    if not args.quick:
+        res = {}
+        for name, build in CONFIGS:
+            cfg = build(ctx, ga, R)
+            res[name] = measure_config(ctx, name, cfg)
+            del cfg
+        res["latency"] = latency_table(ctx, ga)
+        out["per_config"] = res
+    print(json.dumps(out))
 
 
 if __name__ == "__main__":

@@ -37,6 +37,20 @@ typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
  * < 0 on error. */
 typedef int (*ga_hip_event_record_fn)(gpucontext *ctx, unsigned int slot);
 typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsigned int b);
+/* "hip_kernel_timing": on != 0 drops earlier records and gives every kernel
+ * launch of the context from now on its own start and stop event (the
+ * distance between them is the kernel's duration on the device, without the
+ * gap between a mark on the stream and the kernel's start); on == 0 returns to
+ * plain launches.  "hip_kernel_times": waits for the last recorded launch and
+ * writes the durations, in milliseconds and in launch order, to out[0..max);
+ * returns the number of launches recorded, < 0 on error. */
+typedef int (*ga_hip_kernel_timing_fn)(gpucontext *ctx, int on);
+typedef int (*ga_hip_kernel_times_fn)(gpucontext *ctx, float *out, unsigned int max);
+/* "hip_last_launch_hash": 64-bit FNV-1a hash of the source text, followed by
+ * the entry point's name, of the kernel the context launched last (0 before
+ * the first launch): ties a measurement to the generated kernel it was made
+ * on. */
+typedef unsigned long long (*ga_hip_last_launch_hash_fn)(gpucontext *ctx);
 /* "hip_take1_source": kernel text of GpuArray_take1 for result/source/index
  * typecodes and `tnd` collapsed trailing dims; chunks != 0: the variant that
  * moves dense aligned rows as 16-byte chunks. */

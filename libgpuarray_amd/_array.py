@@ -1,138 +1,123 @@
-"""`ndgpuarray`: GpuArray with NumPy's arithmetic, comparison and reduction
-methods, every one a GpuElemwise or reduction call on the device (reference
-pygpu/_array.py:10-294).  Result types are what NumPy gives for the same
-operands; integer `/`, `//` and `%` are C's (truncating) as in the reference,
-which agrees with NumPy for non-negative operands.
+"""`ndgpuarray`: a GpuArray that behaves like a NumPy array under Python's
+operators and the sum/prod/any/all/min/max methods.  Every operation is one
+GpuElemwise or GpuReduction call on the device.
 
-Beyond the reference: min and max (commented out there, :264-280) are
-provided on top of the C reductions.
+The rules are those of the reference's class of the same name
+(pygpu/_array.py:10-294), stated here as a table instead of one method per
+operator:
+
+  result type      what NumPy gives for the same operands (dtypes.get_common_dtype),
+                   for `/` the type of NumPy's true division
+  + - *            computed in the result type
+  / // %           on integers C's truncating division and remainder (equal to
+                   NumPy's for operands of one sign); `//` on floating results is
+                   floor(a / b), `%` is fmod(a, b)
+  op=              computed in C's own promotion of the two operand types and
+                   stored back into the left array's type; floating forms as above
+  comparisons      element-wise, bool result
+  sum, prod        accumulate in the result type, small integers widened to the
+                   platform integer (reference :250-262, :282-294)
+  any, all         truth values, bool result (reference :238-248)
+  min, max, argmin, argmax   not in the reference (commented out, :264-280)
 """
 import numpy as np
 
 from . import gpuarray
+from . import reduction as _red
 from .dtypes import dtype_to_ctype, get_common_dtype, get_np_obj
 from .elemwise import GpuElemwise, arg, as_argument, compare, elemwise1, elemwise2, ielemwise2
-from . import reduction as _red
+
+_F16, _F32, _F64 = np.dtype("float16"), np.dtype("float32"), np.dtype("float64")
+
+# operator -> (C symbol, form used when the computation is floating, else None)
+_BINARY = {
+    "add": ("+", None),
+    "sub": ("-", None),
+    "mul": ("*", None),
+    "truediv": ("/", None),
+    "floordiv": ("/", "floor({x} / {y})"),
+    "mod": ("%", "fmod({x}, {y})"),
+}
+_COMPARE = {"lt": "<", "le": "<=", "eq": "==", "ne": "!=", "ge": ">=", "gt": ">"}
 
 
-def _div_result(a, b):
-    return np.asarray(get_np_obj(a) / get_np_obj(b)).dtype
+def _compute_ctype(dt):
+    """C type a result of dtype `dt` is computed in (halves are computed as floats)."""
+    return dtype_to_ctype(_F32 if dt == _F16 else dt)
+
+
+def _statement(dst, sym, float_form, ctype, x="a", y="b"):
+    """`dst = x <op> y`; with a C type, both operands are converted to it first."""
+    if ctype is not None:
+        x, y = "(%s)%s" % (ctype, x), "(%s)%s" % (ctype, y)
+    if float_form is not None and ctype in ("ga_float", "ga_double", "float", "double"):
+        return "%s = %s" % (dst, float_form.format(x=x, y=y))
+    return "%s = %s %s %s" % (dst, x, sym, y)
+
+
+def _result_dtype(name, x, y):
+    if name == "truediv":
+        return np.asarray(get_np_obj(x) / get_np_obj(y)).dtype
+    return get_common_dtype(x, y, True)
+
+
+def _inplace_ctype(name, self, other):
+    """Type an `op=` is computed in: C's promotion of the operands, except that
+    the floating forms of `/`, `//` and `%` are spelled with explicit casts."""
+    if name not in ("truediv", "floordiv", "mod"):
+        return None
+    mine, theirs = self.dtype, np.asarray(get_np_obj(other)).dtype
+    kinds = (mine, theirs) if name != "floordiv" else (mine,)
+    if _F64 in kinds:
+        return "double"
+    if _F32 in kinds or _F16 in kinds:
+        return "float"
+    return None
+
+
+def _make_binary(name):
+    sym, float_form = _BINARY[name]
+
+    def apply(x, y, like):
+        dt = np.dtype(_result_dtype(name, x, y))
+        oper = _statement("res", sym, float_form, _compute_ctype(dt))
+        return elemwise2(x, sym, y, like, odtype=dt, oper=oper, broadcast=True)
+
+    def forward(self, other):
+        return apply(self, other, self)
+
+    def reflected(self, other):
+        return apply(other, self, self)
+
+    def inplace(self, other):
+        oper = _statement("a", sym, float_form, _inplace_ctype(name, self, other))
+        return ielemwise2(self, sym, other, oper=oper, broadcast=True)
+    return forward, reflected, inplace
+
+
+def _make_compare(sym):
+    def method(self, other):
+        return compare(self, sym, other, broadcast=True)
+    return method
 
 
 class ndgpuarray(gpuarray.GpuArray):
-    # add
-    def __add__(self, other):
-        return elemwise2(self, "+", other, self, broadcast=True)
+    __hash__ = None      # == compares element-wise, so instances cannot be dictionary keys
 
-    def __radd__(self, other):
-        return elemwise2(other, "+", self, self, broadcast=True)
-
-    def __iadd__(self, other):
-        return ielemwise2(self, "+", other, broadcast=True)
-
-    # sub
-    def __sub__(self, other):
-        return elemwise2(self, "-", other, self, broadcast=True)
-
-    def __rsub__(self, other):
-        return elemwise2(other, "-", self, self, broadcast=True)
-
-    def __isub__(self, other):
-        return ielemwise2(self, "-", other, broadcast=True)
-
-    # mul
-    def __mul__(self, other):
-        return elemwise2(self, "*", other, self, broadcast=True)
-
-    def __rmul__(self, other):
-        return elemwise2(other, "*", self, self, broadcast=True)
-
-    def __imul__(self, other):
-        return ielemwise2(self, "*", other, broadcast=True)
-
-    # truediv
-    def __truediv__(self, other):
-        return elemwise2(self, "/", other, self, odtype=_div_result(self, other), broadcast=True)
-
-    def __rtruediv__(self, other):
-        return elemwise2(other, "/", self, self, odtype=_div_result(other, self), broadcast=True)
-
-    def __itruediv__(self, other):
-        np2 = np.asarray(get_np_obj(other))
-        kw = {"broadcast": True}
-        if self.dtype == np.float32 or np2.dtype == np.float32:
-            kw["op_tmpl"] = "a = (float)a / (float)b"
-        if self.dtype == np.float64 or np2.dtype == np.float64:
-            kw["op_tmpl"] = "a = (double)a / (double)b"
-        return ielemwise2(self, "/", other, **kw)
-
-    # floordiv
-    def __floordiv__(self, other):
-        out_dtype = get_common_dtype(self, other, True)
-        kw = {"broadcast": True}
-        if out_dtype.kind == "f":
-            kw["op_tmpl"] = "res = floor((%(out_t)s)a / (%(out_t)s)b)"
-        return elemwise2(self, "/", other, self, odtype=out_dtype, **kw)
-
-    def __rfloordiv__(self, other):
-        out_dtype = get_common_dtype(other, self, True)
-        kw = {"broadcast": True}
-        if out_dtype.kind == "f":
-            kw["op_tmpl"] = "res = floor((%(out_t)s)a / (%(out_t)s)b)"
-        return elemwise2(other, "/", self, self, odtype=out_dtype, **kw)
-
-    def __ifloordiv__(self, other):
-        kw = {"broadcast": True}
-        if self.dtype == np.float32:
-            kw["op_tmpl"] = "a = floor((float)a / (float)b)"
-        if self.dtype == np.float64:
-            kw["op_tmpl"] = "a = floor((double)a / (double)b)"
-        return ielemwise2(self, "/", other, **kw)
-
-    # mod
-    def __mod__(self, other):
-        out_dtype = get_common_dtype(self, other, True)
-        kw = {"broadcast": True}
-        if out_dtype.kind == "f":
-            kw["op_tmpl"] = "res = fmod((%(out_t)s)a, (%(out_t)s)b)"
-        return elemwise2(self, "%", other, self, odtype=out_dtype, **kw)
-
-    def __rmod__(self, other):
-        out_dtype = get_common_dtype(other, self, True)
-        kw = {"broadcast": True}
-        if out_dtype.kind == "f":
-            kw["op_tmpl"] = "res = fmod((%(out_t)s)a, (%(out_t)s)b)"
-        return elemwise2(other, "%", self, self, odtype=out_dtype, **kw)
-
-    def __imod__(self, other):
-        out_dtype = get_common_dtype(self, other, self.dtype == np.float64)
-        kw = {"broadcast": True}
-        if out_dtype == np.float32:
-            kw["op_tmpl"] = "a = fmod((float)a, (float)b)"
-        if out_dtype == np.float64:
-            kw["op_tmpl"] = "a = fmod((double)a, (double)b)"
-        return ielemwise2(self, "%", other, **kw)
-
-    # divmod
-    def _divmod(self, a, b):
-        a_np, b_np = a, b
-        if not isinstance(a, gpuarray.GpuArray):
-            a = np.asarray(a)
-        if not isinstance(b, gpuarray.GpuArray):
-            b = np.asarray(b)
-        odtype = get_common_dtype(a_np, b_np, True)
-        args = [arg("div", odtype, write=True), arg("mod", odtype, write=True),
-                as_argument(a, "a", read=True), as_argument(b, "b", read=True)]
-        div = self._empty_like_me(dtype=odtype)
-        mod = self._empty_like_me(dtype=odtype)
-        if odtype.kind == "f":
-            tmpl = ("div = floor((%(out_t)s)a / (%(out_t)s)b),"
-                    "mod = fmod((%(out_t)s)a, (%(out_t)s)b)")
-        else:
-            tmpl = "div = (%(out_t)s)a / (%(out_t)s)b,mod = a %% b"
-        k = GpuElemwise(self.context, tmpl % {"out_t": dtype_to_ctype(odtype)}, args)
-        k(div, mod, a, b, broadcast=True)
-        return (div, mod)
+    def _divmod(self, x, y):
+        """(x // y, x % y) from one kernel with two outputs."""
+        dt = np.dtype(get_common_dtype(x, y, True))
+        ct = _compute_ctype(dt)
+        xs = x if isinstance(x, gpuarray.GpuArray) else np.asarray(x)
+        ys = y if isinstance(y, gpuarray.GpuArray) else np.asarray(y)
+        quot, rem = self._empty_like_me(dtype=dt), self._empty_like_me(dtype=dt)
+        oper = "%s; %s" % (_statement("quot", "/", _BINARY["floordiv"][1], ct),
+                           _statement("rem", "%", _BINARY["mod"][1], ct))
+        k = GpuElemwise(self.context, oper,
+                        [arg("quot", dt, write=True), arg("rem", dt, write=True),
+                         as_argument(xs, "a", read=True), as_argument(ys, "b", read=True)])
+        k(quot, rem, xs, ys, broadcast=True)
+        return quot, rem
 
     def __divmod__(self, other):
         return self._divmod(self, other)
@@ -147,65 +132,42 @@ class ndgpuarray(gpuarray.GpuArray):
         return elemwise1(self, "+")
 
     def __abs__(self):
-        if self.dtype.kind == "u":
+        kind, size = self.dtype.kind, self.dtype.itemsize
+        if kind in "ub":
             return self.copy()
-        if self.dtype.kind == "f":
+        if kind == "f":
             oper = "res = fabs(a)"
-        elif self.dtype.itemsize < 4:
-            oper = "res = abs((int)a)"
-        elif self.dtype.itemsize == 8:
-            oper = "res = a < 0 ? -a : a"
+        elif size == 8:
+            oper = "res = a < 0 ? -a : a"       # no 64-bit abs() in the device dialect
         else:
-            oper = "res = abs(a)"
+            oper = "res = abs((int)a)" if size < 4 else "res = abs(a)"
         return elemwise1(self, None, oper=oper)
-
-    # richcmp
-    def __lt__(self, other):
-        return compare(self, "<", other, broadcast=True)
-
-    def __le__(self, other):
-        return compare(self, "<=", other, broadcast=True)
-
-    def __eq__(self, other):
-        return compare(self, "==", other, broadcast=True)
-
-    def __ne__(self, other):
-        return compare(self, "!=", other, broadcast=True)
-
-    def __ge__(self, other):
-        return compare(self, ">=", other, broadcast=True)
-
-    def __gt__(self, other):
-        return compare(self, ">", other, broadcast=True)
-
-    __hash__ = None
 
     @property
     def T(self):
-        if self.ndim < 2:
-            return self
-        return self.transpose()
+        return self.transpose() if self.ndim >= 2 else self
 
-    # reductions
-    def all(self, axis=None, out=None):
+    # -- reductions ---------------------------------------------------------------
+    def _logical(self, c_op, neutral, axis, out):
         if self.ndim == 0:
             return self.copy()
-        return _red.reduce1(self, "&&", "1", np.dtype("bool"), axis=axis, out=out)
+        return _red.reduce1(self, c_op, neutral, np.dtype("bool"), axis=axis, out=out)
+
+    def all(self, axis=None, out=None):
+        return self._logical("&&", "1", axis, out)
 
     def any(self, axis=None, out=None):
-        if self.ndim == 0:
-            return self.copy()
-        return _red.reduce1(self, "||", "0", np.dtype("bool"), axis=axis, out=out)
+        return self._logical("||", "0", axis, out)
 
-    def prod(self, axis=None, dtype=None, out=None):
-        if dtype is None:
-            dtype = _red._upcast(self.dtype)
-        return _red.reduce1(self, "*", "1", dtype, axis=axis, out=out)
+    def _arith(self, c_op, neutral, axis, dtype, out):
+        return _red.reduce1(self, c_op, neutral, _red._upcast(self.dtype) if dtype is None else dtype,
+                            axis=axis, out=out)
 
     def sum(self, axis=None, dtype=None, out=None):
-        if dtype is None:
-            dtype = _red._upcast(self.dtype)
-        return _red.reduce1(self, "+", "0", dtype, axis=axis, out=out)
+        return self._arith("+", "0", axis, dtype, out)
+
+    def prod(self, axis=None, dtype=None, out=None):
+        return self._arith("*", "1", axis, dtype, out)
 
     def max(self, axis=None, out=None):
         return _red.max(self, axis=axis, out=out)
@@ -218,3 +180,15 @@ class ndgpuarray(gpuarray.GpuArray):
 
     def argmin(self, axis=None):
         return _red.argmin(self, axis=axis)
+
+
+for _name in _BINARY:
+    _f, _r, _i = _make_binary(_name)
+    for _prefix, _fn in (("", _f), ("r", _r), ("i", _i)):
+        _fn.__name__ = "__%s%s__" % (_prefix, _name)
+        setattr(ndgpuarray, _fn.__name__, _fn)
+for _name, _sym in _COMPARE.items():
+    _m = _make_compare(_sym)
+    _m.__name__ = "__%s__" % _name
+    setattr(ndgpuarray, _m.__name__, _m)
+del _name, _sym, _f, _r, _i, _m, _prefix, _fn

@@ -25,6 +25,16 @@
 #include <unordered_map>
 #include <vector>
 
+// Launch with a start and a stop event attached to the dispatch
+// (declared in <hip/hip_ext.h>, which needs the device-side headers).
+extern "C" hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX,
+                                               uint32_t globalWorkSizeY, uint32_t globalWorkSizeZ,
+                                               uint32_t localWorkSizeX, uint32_t localWorkSizeY,
+                                               uint32_t localWorkSizeZ, size_t sharedMemBytes,
+                                               hipStream_t hStream, void **kernelParams, void **extra,
+                                               hipEvent_t startEvent, hipEvent_t stopEvent,
+                                               uint32_t flags);
+
 namespace {
 
 struct hip_module {
@@ -287,9 +297,16 @@ struct hip_context : _gpucontext {
   size_t live_modules = 0;   // loaded code objects, cached or still referenced
   gpudata *scratch = nullptr;
   size_t scratch_sz = 0;
+  std::vector<gpudata *> retired_scratch;   // outgrown scratch buffers, kept until teardown
   gpudata *redux_counters = nullptr;   // zeroed counters of single-launch split reductions
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
+  // hip_kernel_timing: while on, every launch carries its own start and stop
+  // event (pairs [2i], [2i+1] of ktime_ev; ktime_n launches recorded so far)
+  bool ktime_on = false;
+  std::vector<hipEvent_t> ktime_ev;
+  size_t ktime_n = 0;
+  uint64_t last_launch_hash = 0;   // text_hash of the kernel launched last
   void *redux_cache = nullptr;
   void *take1_cache = nullptr;
   mem_cache mem;
@@ -339,6 +356,7 @@ struct hip_kernel : _gpukernel {
   unsigned char *argstore;
   void **args;           // what setarg recorded: gpudata* or pointer into argstore
   size_t maxlsize;
+  uint64_t text_hash;    // FNV-1a of the source text followed by the entry point's name
 };
 
 inline hip_context *HC(gpucontext *c) { return static_cast<hip_context *>(c); }
@@ -394,6 +412,8 @@ void ctx_destroy(hip_context *ctx) {
   // internal buffers do not count as owners, so they are still here
   if (ctx->errbuf) { hip_release(ctx->errbuf); ctx->errbuf = nullptr; }
   if (ctx->scratch) { hip_release(ctx->scratch); ctx->scratch = nullptr; }
+  for (gpudata *b : ctx->retired_scratch) hip_release(b);
+  ctx->retired_scratch.clear();
   if (ctx->redux_counters) { hip_release(ctx->redux_counters); ctx->redux_counters = nullptr; }
   ctx->mem.destroy();
   {
@@ -406,6 +426,7 @@ void ctx_destroy(hip_context *ctx) {
     }
   }
   for (hipEvent_t e : ctx->evpool) (void)hipEventDestroy(e);
+  for (hipEvent_t e : ctx->ktime_ev) (void)hipEventDestroy(e);
   if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
   if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -488,7 +509,6 @@ gpucontext *hip_init(gpucontext_props *p) {
   size_t alen = strcspn(arch, ":");
   snprintf(ctx->bin_id, sizeof(ctx->bin_id), "%.*s", (int)alen, arch);
 #undef INIT_TRY
-
   {
     const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
     if (dc != nullptr && *dc != 0) ctx->disk_cache = dc;
@@ -1092,6 +1112,12 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
       maxt <= 0)
     maxt = (int)ctx->maxthreads;
   k->maxlsize = (size_t)maxt;
+  {
+    uint64_t h = 1469598103934665603ull;
+    for (unsigned char ch : m->key) h = (h ^ ch) * 1099511628211ull;
+    for (const char *c = fname; *c; c++) h = (h ^ (unsigned char)*c) * 1099511628211ull;
+    k->text_hash = h;
+  }
   m->refcnt++;
   ctx->refcnt++;
   *out = k;
@@ -1174,6 +1200,24 @@ int hip_callkernel(gpukernel *kk, unsigned int n, const size_t *gs, const size_t
   }
   int err;
   if ((err = enter(ctx)) != GA_NO_ERROR) return err;
+  ctx->last_launch_hash = k->text_hash;
+  // Timed launches (the hip_kernel_timing hook): the dispatch itself carries
+  // a start and a stop event, so their distance is the kernel's own duration,
+  // without the gap between a mark on the stream and the kernel's start.
+  if (ctx->ktime_on && (uint64_t)g[0] * l[0] <= 0xffffffffull && (uint64_t)g[1] * l[1] <= 0xffffffffull &&
+      (uint64_t)g[2] * l[2] <= 0xffffffffull) {
+    while (ctx->ktime_ev.size() < 2 * (ctx->ktime_n + 1)) {
+      hipEvent_t e = nullptr;
+      HIP_TRY(ctx, hipEventCreate(&e));
+      ctx->ktime_ev.push_back(e);
+    }
+    HIP_TRY(ctx, hipExtModuleLaunchKernel(k->fn, g[0] * l[0], g[1] * l[1], g[2] * l[2], l[0], l[1], l[2],
+                                          shared, ctx->stream, params, nullptr,
+                                          ctx->ktime_ev[2 * ctx->ktime_n],
+                                          ctx->ktime_ev[2 * ctx->ktime_n + 1], 0));
+    ctx->ktime_n++;
+    return GA_NO_ERROR;
+  }
   HIP_TRY(ctx, hipModuleLaunchKernel(k->fn, g[0], g[1], g[2], l[0], l[1], l[2],
                                      (unsigned int)shared, ctx->stream, params, nullptr));
   return GA_NO_ERROR;
@@ -1374,6 +1418,35 @@ float ext_event_elapsed(gpucontext *c, unsigned int a, unsigned int b) {
   return ms;
 }
 
+// Per-launch timing.  on != 0: forget earlier records and give every launch
+// from now on its own pair of events; on == 0: back to plain launches (the
+// records stay readable).
+int ext_kernel_timing(gpucontext *c, int on) {
+  hip_context *ctx = HC(c);
+  if (on) ctx->ktime_n = 0;
+  ctx->ktime_on = on != 0;
+  return GA_NO_ERROR;
+}
+
+// Durations in milliseconds of the launches recorded since timing was turned
+// on, in launch order, into out[0..max); waits for the last of them.  Returns
+// how many were recorded, < 0 on error.
+int ext_kernel_times(gpucontext *c, float *out, unsigned int max) {
+  hip_context *ctx = HC(c);
+  if (enter(ctx) != GA_NO_ERROR) return -1;
+  const size_t n = ctx->ktime_n;
+  if (n > 0 && hipEventSynchronize(ctx->ktime_ev[2 * n - 1]) != hipSuccess) return -1;
+  for (size_t i = 0; i < n && i < max; i++)
+    if (hipEventElapsedTime(&out[i], ctx->ktime_ev[2 * i], ctx->ktime_ev[2 * i + 1]) != hipSuccess)
+      return -1;
+  return (int)n;
+}
+
+// Identifies the text of the kernel the context launched last: a 64-bit hash
+// of its source followed by its entry point's name.  Lets a measurement say
+// which generated kernel it belongs to.
+uint64_t ext_last_launch_hash(gpucontext *c) { return HC(c)->last_launch_hash; }
+
 // Entries in the hot, warm and cold lists of the module cache, and the number
 // of code objects currently loaded (cached or kept alive by a kernel).
 int ext_module_cache_stats(gpucontext *c, size_t out[4]) {
@@ -1394,6 +1467,9 @@ const ext_entry k_exts[] = {
     {"hip_time_end", (void *)ext_time_end},
     {"hip_event_record", (void *)ext_event_record},
     {"hip_event_elapsed", (void *)ext_event_elapsed},
+    {"hip_kernel_timing", (void *)ext_kernel_timing},
+    {"hip_kernel_times", (void *)ext_kernel_times},
+    {"hip_last_launch_hash", (void *)ext_last_launch_hash},
     {"hip_elemwise_source", (void *)ga_elemwise_gen_source},
     {"hip_reduction_source", (void *)ga_reduction_gen_source},
     {"hip_mapreduce_source", (void *)ga_mapreduce_gen_source},
@@ -1410,23 +1486,33 @@ extern "C" void *gpuarray_get_extension(const char *name) {
   return nullptr;
 }
 
+// A scratch buffer that is outgrown is kept until the context goes: launches
+// already recorded into a HIP graph hold its address, and a block given back
+// to the memory cache would be handed to the caller's next array while every
+// replay of that graph still writes partials into it.  Sizes double, so the
+// buffers kept this way add up to less than the one in use.
 gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
   hip_context *ctx = HC(c);
   if (ctx->scratch != nullptr && ctx->scratch_sz >= bytes) return ctx->scratch;
-  if (ctx->scratch != nullptr) {
-    hip_release(ctx->scratch);   // hipFree waits for queued users
-    ctx->scratch = nullptr;
-    ctx->scratch_sz = 0;
-  }
-  size_t want = bytes < ((size_t)1 << 20) ? ((size_t)1 << 20) : bytes;
-  ctx->scratch = hip_alloc(c, want, nullptr, BUF_INTERNAL);
-  if (ctx->scratch != nullptr) ctx->scratch_sz = want;
+  size_t want = ctx->scratch_sz ? ctx->scratch_sz * 2 : ((size_t)1 << 20);
+  while (want < bytes) want *= 2;
+  gpudata *grown = hip_alloc(c, want, nullptr, BUF_INTERNAL);
+  if (grown == nullptr && want > bytes) grown = hip_alloc(c, want = bytes, nullptr, BUF_INTERNAL);
+  if (grown == nullptr) return nullptr;
+  if (ctx->scratch != nullptr) ctx->retired_scratch.push_back(ctx->scratch);
+  ctx->scratch = grown;
+  ctx->scratch_sz = want;
   return ctx->scratch;
 }
 
 gpudata *ga_hip_redux_counters(gpucontext *c) {
   hip_context *ctx = HC(c);
   if (ctx->redux_counters != nullptr) return ctx->redux_counters;
+  // Not while the stream records a graph: the memset that zeroes the counters
+  // would be recorded instead of run.  The caller then takes two launches.
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+  else if (cap != hipStreamCaptureStatusNone) return nullptr;
   gpudata *b = hip_alloc(c, ga_hip_redux_counters_max * sizeof(uint32_t), nullptr, BUF_INTERNAL);
   if (b == nullptr) return nullptr;
   if (hip_memset(b, 0, 0) != GA_NO_ERROR) {

@@ -201,6 +201,25 @@ class GpuContext(object):
             raise GpuArrayException("event timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
         return ms
 
+    def last_launch_hash(self):
+        """Hash (hex) of the text and entry point of the kernel launched last."""
+        fn = _lib.extension("hip_last_launch_hash", C.c_ulonglong, [C.c_void_p])
+        return "%016x" % fn(self.ctx)
+
+    def kernel_timing(self, on=True):
+        """Give every launch from now on its own start and stop event."""
+        fn = _lib.extension("hip_kernel_timing", C.c_int, [C.c_void_p, C.c_int])
+        check(fn(self.ctx, 1 if on else 0), self.ctx)
+
+    def kernel_times(self, limit=65536):
+        """Milliseconds of each launch recorded since kernel_timing(True)."""
+        fn = _lib.extension("hip_kernel_times", C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.c_uint])
+        buf = (C.c_float * limit)()
+        n = fn(self.ctx, buf, limit)
+        if n < 0:
+            raise GpuArrayException("kernel timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
+        return list(buf[:min(n, limit)])
+
     def sync(self):
         # any buffer of the context syncs the one stream; use the error buffer
         eb = C.c_void_p()

@@ -5,6 +5,7 @@
 // copies are memcpy, a kernel launch does nothing: no result of a kernel means
 // anything here, and nothing the library ships may link or load this file.
 #include <hip/hip_runtime_api.h>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <cstdio>
@@ -41,10 +42,12 @@ hipError_t hipMemcpyDtoHAsync(void *d, hipDeviceptr_t s, size_t n, hipStream_t) 
 hipError_t hipMemcpyDtoDAsync(hipDeviceptr_t d, hipDeviceptr_t s, size_t n, hipStream_t) { memmove(d, s, n); return hipSuccess; }
 hipError_t hipMemcpyPeerAsync(void *d, int, const void *s, int, size_t n, hipStream_t) { memmove(d, s, n); return hipSuccess; }
 hipError_t hipMemsetD8Async(hipDeviceptr_t d, unsigned char v, size_t n, hipStream_t) { memset(d, v, n); return hipSuccess; }
+hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus *s) { *s = hipStreamCaptureStatusNone; return hipSuccess; }
 hipError_t hipModuleLoadData(hipModule_t *m, const void *) { *m = (hipModule_t)malloc(8); return hipSuccess; }
 hipError_t hipModuleUnload(hipModule_t m) { free(m); return hipSuccess; }
 hipError_t hipModuleGetFunction(hipFunction_t *f, hipModule_t, const char *) { *f = (hipFunction_t)0x30; return hipSuccess; }
 hipError_t hipFuncGetAttribute(int *v, hipFunction_attribute, hipFunction_t) { *v = 1024; return hipSuccess; }
+hipError_t hipExtModuleLaunchKernel(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, size_t, hipStream_t, void **, void **, hipEvent_t, hipEvent_t, uint32_t) { return hipSuccess; }
 hipError_t hipModuleLaunchKernel(hipFunction_t, unsigned gx, unsigned, unsigned, unsigned bx, unsigned, unsigned, unsigned, hipStream_t, void **params, void **) {
   (void)gx; (void)bx; (void)params; return hipSuccess; }
 }

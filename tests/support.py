@@ -76,3 +76,26 @@ def gen_gpuarray(shape_orig, dtype="float32", offseted_outer=False, offseted_inn
 
 def arg(name, dtype, read=False, write=False, scalar=False):
     return ga.arg(name, dtype, read=read, write=write, scalar=scalar)
+
+
+def check_float_sum(got, truth64, mag64, rtol=1e-5, cancel=1e-3, what=""):
+    """A floating sum against the float64 sum `truth64` of the same elements.
+
+    The bound is rtol * |sum| wherever the sum is not a cancellation, i.e.
+    |sum| >= cancel * (sum of magnitudes `mag64`).  Below that the relative
+    criterion is ill-posed (the exact sum can be 0), and the bound is what any
+    summation order of float32 values can promise: 8 * 2^-24 * sum of
+    magnitudes.  Returns the largest relative error among the results held to
+    rtol and the fraction of results that took the fallback, so that callers
+    can bound and report both."""
+    got = np.asarray(got, dtype=np.float64)
+    truth64 = np.asarray(truth64, dtype=np.float64)
+    mag64 = np.asarray(mag64, dtype=np.float64)
+    err = np.abs(got - truth64)
+    strict = np.abs(truth64) >= cancel * mag64
+    bound = np.where(strict, rtol * np.abs(truth64), 8 * 2.0 ** -24 * mag64)
+    bad = err > bound
+    assert not bad.any(), "%s: %d results outside the bound, worst error %.3g against %.3g" % (
+        what, int(bad.sum()), float(err[bad].max()), float(bound[bad].min()))
+    rel = err[strict] / np.abs(truth64[strict]) if strict.any() else np.zeros(1)
+    return float(rel.max()), float(1.0 - strict.mean())

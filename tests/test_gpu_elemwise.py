@@ -274,6 +274,27 @@ def test_dtype_matrix_copy_cast_vs_numpy(ctx):
             assert np.array_equal(got, n.T.astype(dd)), (sd, dd)
 
 
+def test_cast_to_bool_stores_the_truth_value_not_the_low_byte(ctx):
+    """A deliberate difference from the reference.  Its GA_BOOL is an unsigned
+    char (`ga_bool`, src/cluda_opencl.h:26), so a casting copy `dst = src` into
+    a bool array converts to unsigned char: 62.5 becomes 62, 256 becomes 0, 257
+    becomes 1.  Here the copy stores `src != 0`, NumPy's astype(bool): 1, 1, 1.
+    Both results are spelled out so that the difference stays visible."""
+    for dtype, values in (("float32", [0.0, 1.0, 62.5, -3.0, 0.25]),
+                          ("int32", [0, 1, 255, 256, 257, 512, -1]),
+                          ("int64", [0, 1 << 8, 1 << 32, 3])):
+        host = np.array(values, dtype=dtype)
+        got = np.asarray(gpuarray.array(host, context=ctx).astype("bool")).view(np.uint8)
+        with np.errstate(invalid="ignore"):
+            reference_would_store = host.astype(np.int64).astype(np.uint8)   # C's conversion to unsigned char
+        here = (host != 0).astype(np.uint8)
+        assert np.array_equal(got, here), (dtype, got)
+        if dtype == "int32":
+            assert reference_would_store.tolist() == [0, 1, 255, 0, 1, 0, 255]
+            assert here.tolist() == [0, 1, 1, 1, 1, 1, 1]
+        assert np.array_equal(got != 0, host.astype(bool))
+
+
 def test_all_fortran_inputs_take_the_flat_path(ctx):
     rng = np.random.default_rng(8)
     a = np.asfortranarray(rng.normal(size=(130, 70)).astype(np.float32))

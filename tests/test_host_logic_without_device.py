@@ -82,3 +82,4 @@ def test_views_follow_numpy_on_random_chains(mock_runtime):
                        cwd=ROOT, env=dict(os.environ, LD_PRELOAD=mock_runtime), capture_output=True,
                        text=True, timeout=600)
     assert r.returncode == 0 and "views ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
+

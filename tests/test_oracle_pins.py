@@ -162,6 +162,33 @@ def test_c_check_agrees_with_the_python_check(case, oracle):
         assert all(g == 0 for g, d in zip(got, dims) if d == 1)
 
 
+@pytest.mark.parametrize("case", KATS["planned_iteration_spaces"]["cases"], ids=lambda c: c["name"][:12])
+def test_planned_iteration_space_of_the_strided_configurations(case, oracle):
+    """The iteration space the reference plans for configuration 2 (two
+    dimensions that do not merge, 32-bit offsets) and for the stride-2 views of
+    configuration 5 (one dimension of 67 108 864 elements, source stride twice
+    the item size): the checker's check_basic and the library's exported
+    gpuarray_elemwise_collapse both have to arrive there."""
+    from numpy.lib.stride_tricks import as_strided
+    from test_types_util import lib_collapse
+    dt = {1: np.uint8, 2: np.float16, 4: np.float32}[case["itemsize"]]
+    # views of a one-element buffer: only shapes and strides are looked at
+    arrays = [as_strided(np.zeros(1, dtype=dt), shape=a["shape"], strides=a["strides"], writeable=False)
+              for a in case["arrays"]]
+    is_out = [i == case["out"] for i in range(len(arrays))]
+    err, nd, dims, strs, n, call32 = oracle.check_basic(arrays, is_out, BCAST if case["broadcast"] else 0)
+    assert err == 0
+    assert (nd, list(dims), n, call32) == (case["nd"], case["dims"], case["n"], case["call32"])
+    assert [list(s) for s in strs] == case["strs"]
+    # the library's collapse on the broadcast-adjusted strides (a size-1 input dim has stride 0)
+    full = case["arrays"][case["out"]]["shape"]
+    rows = [[0 if a["shape"][i] == 1 and full[i] != 1 else a["strides"][i] for i in range(len(full))]
+            for a in case["arrays"]]
+    lnd, ldims, lstrs = lib_collapse(list(full), rows)
+    assert (lnd, list(ldims)) == (case["nd"], case["dims"])
+    assert [list(s) for s in lstrs] == case["strs"]
+
+
 def test_checker_elemwise_equals_numpy_on_random_views(oracle):
     rng = np.random.default_rng(21)
     for _ in range(60):
