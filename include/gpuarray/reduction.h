@@ -76,6 +76,33 @@ GPUARRAY_PUBLIC int GpuReduction_call(const GpuReduction *gr, GpuArray *d0,
                                       unsigned reduxLen, const int *reduxList,
                                       int flags);
 
+/* GpuReduction_call for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.
+ *
+ * Same arguments, rules and results as GpuReduction_call (operators made by
+ * GpuReduction_new only).  Where GpuReduction_call keeps the partial results
+ * of a split reduction in a buffer the context allocates and grows, this
+ * entry point keeps them in a device array that is part of the library
+ * itself, GA_REDUCTION_NOALLOC_SCRATCH bytes on every GPU the library runs
+ * on, looked up once when the context is made; it calls no allocating
+ * routine, and a split reduction always ends in a second launch.
+ *   GA_UNSUPPORTED_ERROR  the kernels for this layout are not built yet
+ *                         (building loads a code object, which allocates):
+ *                         call GpuReduction_call once on arrays of the same
+ *                         types and layout first.
+ *   GA_XLARGE_ERROR       the partials (outputs x pieces x 12 or 16 bytes)
+ *                         would not fit GA_REDUCTION_NOALLOC_SCRATCH.
+ * All calls on one GPU share that GPU's array: calls issued on one context
+ * run in order on its stream; calls on different contexts of the same GPU
+ * that overlap in time race, and must be ordered by the caller. */
+#define GA_REDUCTION_NOALLOC_SCRATCH ((size_t)4 << 20)
+GPUARRAY_PUBLIC int GpuReduction_call_noalloc(const GpuReduction *gr,
+                                              GpuArray *d0, GpuArray *d1,
+                                              const GpuArray *s0,
+                                              unsigned reduxLen,
+                                              const int *reduxList, int flags);
+
 /* A reduction fed by an elementwise expression over several arguments, in one
  * pass over memory: the C counterpart of the reference's
  * ReductionKernel(map_expr=..., arguments=...) (pygpu/reduction.py:137-291,

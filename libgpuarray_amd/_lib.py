@@ -228,6 +228,8 @@ SIGNATURES = {
     "GpuReduction_free": (None, [C.c_void_p]),
     "GpuReduction_call": (C.c_int, [C.c_void_p, PA, PA, PA, C.c_uint, C.POINTER(C.c_int),
                                     C.c_int]),
+    "GpuReduction_call_noalloc": (C.c_int, [C.c_void_p, PA, PA, PA, C.c_uint, C.POINTER(C.c_int),
+                                            C.c_int]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

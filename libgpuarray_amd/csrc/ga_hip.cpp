@@ -298,6 +298,8 @@ struct hip_context : _gpucontext {
   gpudata *scratch = nullptr;
   size_t scratch_sz = 0;
   std::vector<gpudata *> retired_scratch;   // outgrown scratch buffers, kept until teardown
+  void *static_scratch = nullptr;           // this device's copy of the static scratch array
+  int static_scratch_err = 0;               // HIP error code of its lookup
   gpudata *redux_counters = nullptr;   // zeroed counters of single-launch split reductions
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
@@ -509,6 +511,10 @@ gpucontext *hip_init(gpucontext_props *p) {
   size_t alen = strcspn(arch, ":");
   snprintf(ctx->bin_id, sizeof(ctx->bin_id), "%.*s", (int)alen, arch);
 #undef INIT_TRY
+  // Where this device keeps the library's static scratch array (the partials
+  // of GpuReduction_call_noalloc).  A failed lookup only disables that entry
+  // point, which then reports the code kept here.
+  ctx->static_scratch_err = ga_static_scratch_setup(dev, &ctx->static_scratch);
   {
     const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
     if (dc != nullptr && *dc != 0) ctx->disk_cache = dc;
@@ -1503,6 +1509,13 @@ gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
   ctx->scratch = grown;
   ctx->scratch_sz = want;
   return ctx->scratch;
+}
+
+void *ga_hip_static_scratch(gpucontext *c, const char **why) {
+  hip_context *ctx = HC(c);
+  if (why != nullptr)
+    *why = ctx->static_scratch != nullptr ? "" : hipGetErrorString((hipError_t)ctx->static_scratch_err);
+  return ctx->static_scratch;
 }
 
 gpudata *ga_hip_redux_counters(gpucontext *c) {

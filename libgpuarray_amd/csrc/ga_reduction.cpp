@@ -435,7 +435,9 @@ int variant_source(const GpuReduction *gr, const variant_spec &vs, std::string &
 
 size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * RD_MAXD * sizeof(int64_t); }
 
-int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
+// `may_build` false: only a variant whose kernels are loaded already will do
+// (building one loads a code object, and that allocates device memory).
+int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out, bool may_build = true) {
   gpucontext *ctx = gr->ctx;
   const std::array<unsigned, 13> key = {(unsigned)vs.d0_tc, (unsigned)vs.d1_tc, vs.G, vs.V, vs.U,
                                         vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY};
@@ -444,6 +446,11 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out) {
     *out = &it->second;
     return GA_NO_ERROR;
   }
+  if (!may_build)
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR,
+                      "GpuReduction_call_noalloc: the kernels for arrays of this layout are not "
+                      "built yet, and building them allocates; run GpuReduction_call once on "
+                      "arrays of this layout first");
   std::string s;
   int err = variant_source(gr, vs, s, ctx->err);
   if (err != GA_NO_ERROR) return err;
@@ -621,8 +628,8 @@ class reduction_call {
  public:
   reduction_call(GpuReduction *gr_, GpuArray *d0_, GpuArray *d1_, unsigned nd_, const size_t *dims_,
                  const std::vector<src_view> &srcs_, const std::vector<void *> &scalars_,
-                 unsigned reduxLen_, const int *reduxList_)
-      : gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
+                 unsigned reduxLen_, const int *reduxList_, bool noalloc_ = false)
+      : noalloc(noalloc_), gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
         dims(dims_), srcs(srcs_), scalars(scalars_), reduxLen(reduxLen_), reduxList(reduxList_),
         kind(info.kind), minmax(kind == K_MIN || kind == K_MAX),
         logical(kind == K_ALL || kind == K_ANY),
@@ -651,6 +658,9 @@ class reduction_call {
   }
 
  private:
+  // true: partials go to the device's static scratch array, kernels must be
+  // loaded already, and nothing on the way allocates device memory
+  const bool noalloc;
   GpuReduction *gr;
   gpucontext *ctx;
   const op_info &info;
@@ -1216,7 +1226,7 @@ class reduction_call {
     vs.opts |= use_row ? 16u : 32u;   // bits 4, 5: the family of kernels the text holds
     if (srows)   // one kernel, independent of the lane geometry
       vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
-    return get_variant(gr, vs, &var);
+    return get_variant(gr, vs, &var, !noalloc);
   }
 
   int launch() {
@@ -1224,7 +1234,21 @@ class reduction_call {
     // values first, indices after, both 8-byte aligned
     const int acc_tc = acc_typecode(gr, d0_tc);
     const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
-    gpudata *scratch = ga_hip_scratch(ctx, 16);
+    // A view of the static scratch array, for calls that may not allocate: a
+    // gpudata is only read through its leading {device pointer, context}.
+    struct { void *devptr; gpucontext *ctx; } static_view = {nullptr, ctx};
+    gpudata *scratch = nullptr;
+    if (noalloc) {
+      const char *why = "";
+      static_view.devptr = ga_hip_static_scratch(ctx, &why);
+      if (static_view.devptr == nullptr)
+        return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
+                          "GpuReduction_call_noalloc: the static scratch array was not found on "
+                          "this device when the context was made (%s)", why);
+      scratch = reinterpret_cast<gpudata *>(&static_view);
+    } else {
+      scratch = ga_hip_scratch(ctx, 16);
+    }
     size_t pi_off = 0;
     // A split reduction of moderate size ends in the launch that started it:
     // its outputs (row kernel) or tiles of outputs (column kernel) have a
@@ -1235,8 +1259,11 @@ class reduction_call {
     // against 8.7 / 8.6; with one group or more per compute unit waiting for
     // its partial to be acknowledged before it counts in costs more than the
     // second launch (2^24, 512 groups: 17.5 against 14.8 us).
+    // Calls on the static scratch array always take two launches: the second
+    // reads only what the first has written, so nothing there has to start
+    // at zero.
     gpudata *done = nullptr;
-    if (p.nsplit > 1) {
+    if (p.nsplit > 1 && !noalloc) {
       const size_t counters = use_row ? (size_t)nrows : groups / (size_t)p.nsplit;
       const size_t fused_max = (size_t)ncu * env_ul("GPUARRAY_REDUX_FUSED", 1);   // 0 turns it off
       if (groups <= fused_max && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
@@ -1248,7 +1275,16 @@ class reduction_call {
     if (p.nsplit > 1) {
       const size_t slots = (size_t)nrows * (size_t)p.nsplit;
       pi_off = (slots * accsz + 255) & ~(size_t)255;
-      scratch = ga_hip_scratch(ctx, pi_off + slots * 8);
+      const size_t need = pi_off + slots * 8;
+      if (noalloc) {
+        if (need > ga_static_scratch_bytes)
+          return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
+                            "GpuReduction_call_noalloc: this reduction is split into %zu partial "
+                            "results that take %zu bytes; the static scratch array holds %zu",
+                            slots, need, (size_t)ga_static_scratch_bytes);
+      } else {
+        scratch = ga_hip_scratch(ctx, need);
+      }
     }
     if (scratch == nullptr) return ctx->err->code;
     if (!p.fused) done = scratch;   // not used then, but the kernels take a pointer
@@ -1293,8 +1329,8 @@ class reduction_call {
 
 int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
                   const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
-                  unsigned reduxLen, const int *reduxList) {
-  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList).run();
+                  unsigned reduxLen, const int *reduxList, bool noalloc = false) {
+  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList, noalloc).run();
 }
 
 }  // namespace
@@ -1390,6 +1426,21 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
   srcs[0].a = s0;
   srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);
   return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, srcs, {}, reduxLen, reduxList);
+}
+
+int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1,
+                              const GpuArray *s0, unsigned reduxLen, const int *reduxList,
+                              int flags) {
+  (void)flags;
+  GpuReduction *gr = const_cast<GpuReduction *>(cgr);
+  if (gr == nullptr || s0 == nullptr) return GA_INVALID_ERROR;
+  if (gr->nsrc() != 1 || !gr->scalars.empty())
+    return ga_err_set(gr->ctx->err, GA_INVALID_ERROR,
+                      "GpuReduction_call_noalloc takes operators made by GpuReduction_new");
+  std::vector<src_view> srcs(1);
+  srcs[0].a = s0;
+  srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);
+  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, srcs, {}, reduxLen, reduxList, true);
 }
 
 int GpuReduction_call_map(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, void **args,

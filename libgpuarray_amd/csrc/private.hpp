@@ -149,6 +149,16 @@ gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
 // that counts on it leaves it zeroed.  NULL (error set) when it cannot be made.
 constexpr size_t ga_hip_redux_counters_max = 16384;
 gpudata *ga_hip_redux_counters(gpucontext *ctx);
+// The scratch of GpuReduction_call_noalloc: a file-scope device array of
+// ga_static_scratch_bytes bytes in ga_static_scratch.hip, one copy per GPU.
+// ga_static_scratch_setup, called with device `dev` current, looks its
+// address on that device up once and returns it in *ptr (0 on success, else
+// the HIP error code; *ptr is then NULL).
+constexpr size_t ga_static_scratch_bytes = GA_REDUCTION_NOALLOC_SCRATCH;
+int ga_static_scratch_setup(int dev, void **ptr);
+// The address found for the context's device when the context was made, NULL
+// when the lookup failed (the reason is then in *why, if not NULL).
+void *ga_hip_static_scratch(gpucontext *ctx, const char **why);
 // Bytes from a buffer's start that lie inside the memory behind it (at least
 // its size; more when the allocation was rounded up).
 size_t ga_hip_readable_bytes(gpudata *b);

@@ -51,14 +51,16 @@ class GpuReduction(object):
             lib.GpuReduction_free(gr)
             self.gr = None
 
-    def __call__(self, src, axes, d0=None, d1=None):
+    def __call__(self, src, axes, d0=None, d1=None, noalloc=False):
+        """noalloc=True goes through GpuReduction_call_noalloc: partials in the
+        library's static device array, no allocation on the way."""
         key = tuple(axes)
         arr = self._axes.get(key)
         if arr is None:            # the C array of an axis list, built once
             arr = self._axes[key] = (C.c_int * _b.max(len(key), 1))(*key)
-        err = lib.GpuReduction_call(self.gr, d0._ref if d0 is not None else None,
-                                    d1._ref if d1 is not None else None, src._ref,
-                                    len(key), arr, 0)
+        fn = lib.GpuReduction_call_noalloc if noalloc else lib.GpuReduction_call
+        err = fn(self.gr, d0._ref if d0 is not None else None,
+                 d1._ref if d1 is not None else None, src._ref, len(key), arr, 0)
         if err:
             check(err, self.context.ctx)
 

@@ -83,3 +83,39 @@ def test_views_follow_numpy_on_random_chains(mock_runtime):
                        text=True, timeout=600)
     assert r.returncode == 0 and "views ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
 
+
+NOALLOC_SCRIPT = r"""
+import ctypes as C, os, sys
+import numpy as np
+sys.path.insert(0, os.getcwd())
+import libgpuarray_amd as ga
+from libgpuarray_amd import _lib
+mock = C.CDLL(os.environ["LD_PRELOAD"])
+calls = C.c_ulong.in_dll(mock, "mock_allocating_calls")
+ctx = ga.init("hip0")
+for dtype, shape, axes, d1 in (("float32", (1 << 22,), [0], False), ("int32", (6, 1 << 18), [1], False),
+                               ("float32", (1 << 14, 256), [0], True), ("float32", (4096, 100), [1], False)):
+    op = ga.GpuReduction(ctx, "maxandargmax" if d1 else "sum", dtype)
+    src = ga.zeros(shape, dtype, context=ctx)
+    oshape = tuple(d for k, d in enumerate(shape) if k not in axes)
+    d0 = ga.empty(oshape, dtype, context=ctx)
+    di = ga.empty(oshape, "int64", context=ctx) if d1 else None
+    op(src, axes, d0=d0, d1=di)                     # builds the kernels, grows the context's scratch
+    before = calls.value
+    for _ in range(3):
+        op(src, axes, d0=d0, d1=di, noalloc=True)
+    assert calls.value == before, (dtype, shape, calls.value - before)
+    op(src, axes, d0=d0, d1=di)
+print("noalloc ok")
+"""
+
+
+def test_noalloc_entry_point_calls_nothing_that_allocates(mock_runtime):
+    """GpuReduction_call_noalloc between two counts of the stand-in runtime's
+    allocating calls (hipMalloc, hipFree, hipHostMalloc, hipHostFree,
+    hipModuleLoadData, hipEventCreate): none may happen, for split and unsplit
+    reductions, with and without an index result."""
+    r = subprocess.run([sys.executable, "-c", NOALLOC_SCRIPT], cwd=ROOT,
+                       env=dict(os.environ, LD_PRELOAD=mock_runtime), capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0 and "noalloc ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
