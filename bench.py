@@ -265,19 +265,23 @@ def cfg_dot_two_pass(ctx, ga, R):
                     "16 bytes per element instead of 8 cross the memory bus"}
 
 
-def cfg_take1(ctx, ga, R):
-    rows, width = 65536, 1024
-    V = np.random.default_rng(9).standard_normal((rows, width), dtype=np.float32)
-    idx = np.random.default_rng(10).permutation(rows)
-    gv, gidx = ga.array(V, context=ctx), ga.array(idx, context=ctx)
-    last = [None]
+def _cfg_take1(check):
+    def build(ctx, ga, R):
+        rows, width = 65536, 1024
+        V = np.random.default_rng(9).standard_normal((rows, width), dtype=np.float32)
+        idx = np.random.default_rng(10).permutation(rows)
+        gv, gidx = ga.array(V, context=ctx), ga.array(idx, context=ctx)
+        last = [None]
 
-    def call(i):
-        last[0] = gv.take1(gidx)
-    return {"bytes": 2 * rows * width * 4 + rows * 8, "call": call, "sets": 1,
-            "check": lambda: np.array_equal(np.asarray(last[0]), V.take(idx, axis=0)),
-            "numpy": lambda: V.take(idx, axis=0),
-            "note": "includes the result's allocation and the bounds-flag read-back"}
+        def call(i):
+            last[0] = gv.take1(gidx, check=check)
+        return {"bytes": 2 * rows * width * 4 + rows * 8, "call": call, "sets": 1,
+                "check": lambda: np.array_equal(np.asarray(last[0]), V.take(idx, axis=0)),
+                "numpy": lambda: V.take(idx, axis=0),
+                "note": ("includes the result's allocation and the wait for the bounds flag "
+                         "(check_error = 1, the reference's default)") if check else
+                        "includes the result's allocation; check_error = 0, so the call does not wait"}
+    return build
 
 
 CONFIGS = [
@@ -291,7 +295,8 @@ CONFIGS = [
     ("C5_uint8_all_axis2", _cfg_c5_u8("all")),
     ("F4_dot_2x2^27_fused", cfg_dot),
     ("F4_dot_2x2^27_two_pass", cfg_dot_two_pass),
-    ("F2_take1_65536x1024_rows", cfg_take1),
+    ("F2_take1_65536x1024_rows", _cfg_take1(True)),
+    ("F2_take1_65536x1024_rows_unchecked", _cfg_take1(False)),
 ]
 STEP_MODES = ("step", "elem", "sum", "copy")
 
@@ -466,13 +471,40 @@ def cpu_baseline(a_h, b_h, x_h):
     probe = probe_opencl_cpu()
     out["reference_opencl_path"] = probe["status"]
     out["opencl_probe"] = {k: probe[k] for k in ("library", "platforms", "cpu_devices", "devices_of_any_type")}
-    if probe["cpu_devices"]:
-        try:
-            from oracle import opencl_runner
-            out["reference_opencl"] = opencl_runner.run_contig_muladd(a, b, device_type="cpu")
-        except Exception as e:   # the probe saw a device that then could not be used
-            out["reference_opencl"] = {"error": repr(e)}
+    # The reference's generated kernels (fixtures) under its launch rule, in a
+    # child process of their own (an OpenCL runtime next to this process's HIP
+    # context is not something to rely on): on a CPU device when the box has
+    # one, which is the reference leg the benchmark asks for, and, as a further
+    # yardstick, on this GPU through its OpenCL driver when that is the only
+    # device the probe found.
+    kind = "cpu" if probe["cpu_devices"] else ("gpu" if probe["devices_of_any_type"] else None)
+    if kind is not None:
+        cases = ["c1:24", "c1:28", "c2:4096", "c3a:8192"] if kind == "gpu" else ["c1:24", "c2:2048", "c3a:2048"]
+        out["reference_kernels_via_opencl"] = run_reference_kernels(kind, cases)
     return out
+
+
+def run_reference_kernels(device_type, cases):
+    import subprocess
+    res = {"device_type": device_type,
+           "what": "kernel texts the reference generates (tests/golden/reference_kernels), launched with "
+                   "GpuKernel_sched's geometry by oracle/opencl_runner.py; wall time per launch over "
+                   "several launches between two clFinish"}
+    try:
+        r = subprocess.run([sys.executable, "-m", "oracle.opencl_runner", "--device-type", device_type] + cases,
+                           cwd=ROOT, capture_output=True, text=True, timeout=240)
+        rows = []
+        for line in r.stdout.splitlines():
+            try:
+                rows.append(json.loads(line))
+            except ValueError:
+                pass
+        res["cases"] = rows
+        if r.returncode != 0:
+            res["error"] = (r.stderr or "")[-400:]
+    except Exception as e:
+        res["error"] = repr(e)
+    return res
 
 
 # ---- main -----------------------------------------------------------------------------
@@ -518,9 +550,12 @@ def main():
             cfg["call"](i)
         ctx.mark(1)
         us = ctx.elapsed(0, 1) * 1e3 / K
+        kern, launches = time_kernels(ctx, cfg["call"], iters=K, warm=0)
         print(json.dumps({"only": args.only, "calls": K, "warmup_calls": W, "us_per_call_back_to_back": round(us, 2),
+                          "kernel_us": round(kern, 2), "launches_per_call": launches,
                           "algorithmic_bytes_per_call": cfg["bytes"], "kernel_text_hash": khash,
-                          "GBps": round(cfg["bytes"] / us / 1e3, 1)}))
+                          "GBps": round(cfg["bytes"] / us / 1e3, 1),
+                          "GBps_kernel": round(cfg["bytes"] / kern / 1e3, 1)}))
         return
 
     n = 1 << args.log2n
@@ -577,9 +612,12 @@ def main():
         # profiler run: report the one kernel that was launched and stop
         ms = elem_ms if only in ("elem", "copy") else sum_ms
         nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
+        kern, launches = time_kernels(ctx, lambda i: step(), iters=K, warm=0)
         print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
+                          "kernel_us": round(kern, 2), "launches_per_call": launches,
                           "bytes_per_launch": nbytes, "kernel_text_hash": ctx.last_launch_hash(),
-                          "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1)}))
+                          "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1),
+                          "GBps_kernel": round(nbytes / kern / 1e3, 1)}))
         return
 
     # The same kernels once more with a start and a stop event on every

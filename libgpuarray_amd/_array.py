@@ -63,11 +63,21 @@ def _result_dtype(name, x, y):
 
 def _inplace_ctype(name, self, other):
     """Type an `op=` is computed in: C's promotion of the operands, except that
-    the floating forms of `/`, `//` and `%` are spelled with explicit casts."""
+    the floating forms of `/`, `//` and `%` are spelled with explicit casts
+    (reference pygpu/_array.py:59-68, :89-96, :121-131):
+      /=   double if either side is float64, else float if either is float32
+      //=  by the left array's type alone
+      %=   by the common type, double only when the left array is float64 (so
+           that a float32 array and a Python float meet in float32, as in NumPy)."""
     if name not in ("truediv", "floordiv", "mod"):
         return None
     mine, theirs = self.dtype, np.asarray(get_np_obj(other)).dtype
-    kinds = (mine, theirs) if name != "floordiv" else (mine,)
+    if name == "mod":
+        kinds = (np.dtype(get_common_dtype(self, other, mine == _F64)),)
+    elif name == "floordiv":
+        kinds = (mine,)
+    else:
+        kinds = (mine, theirs)
     if _F64 in kinds:
         return "double"
     if _F32 in kinds or _F16 in kinds:

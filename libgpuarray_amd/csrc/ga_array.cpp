@@ -710,6 +710,8 @@ static std::string take1_source(bool chunks, int a_tc, int v_tc, int i_tc, unsig
          "  if (row >= n0) return;\n"
          "  const ga_size x0 = (ga_size)(GID_0 % gx) * (4u << lsh) + lane;\n"
          "  ind = (GLOBAL_MEM const " + ti->cluda_name + " *)((GLOBAL_MEM const char *)ind + i_off);\n"
+         // as the reference (`ssize ii0 = ind[i0]`, src/gpuarray_array.c:385-391): an
+         // unsigned 64-bit index of 2^63 or more is seen as negative and wraps once
          "  ga_long ii = (ga_long)ind[row];\n"
          "  if (ii < 0) ii += (ga_long)d0;\n"
          "  if (ii < 0 || ii >= (ga_long)d0) { if (lane == 0) *err = -1; return; }\n"
@@ -882,6 +884,11 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
   GpuKernel_setarg(k, p++, &lsh);
   GpuKernel_setarg(k, p++, errbuf);
   size_t groups = gx * gy, ls = 256;
+  // The error word belongs to the context and is sticky, as in the reference
+  // (src/gpuarray_array.c:480, :534-543): a kernel sets it on a bad index
+  // whether or not its caller asked for the check, and the next call that does
+  // ask reports it and clears it - also when the bad index was an earlier
+  // call's.
   err = GpuKernel_call(k, 1, &groups, &ls, 0, nullptr);
   if (check_error && err == GA_NO_ERROR) {
     int kerr = 0;

@@ -673,6 +673,14 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
               ge->args[j].name.c_str(), T, T + 1);
   // T x T tile, T*T/16 lanes: ga_lo picks a quad along one axis, ga_hi a line
   // along the other; four passes of T/4 lines cover the tile
+  // Lane -> (quad ga_lo, line ga_hi): the quad from the low bits, so that 16
+  // adjacent lanes touch 256 contiguous bytes of one line.  With a row pitch
+  // of T + 1 words this puts two (T = 64) or four (T = 128) of every 32 lanes
+  // on the same local-memory bank in both phases (the bank-conflict counter
+  // reads half of the LDS cycles for T = 64); a lane order that avoids it (8
+  // quads x 4 lines per 32 lanes) halves the contiguous run to 128 bytes and
+  // measured no faster at 4096 x 4096 and 4 to 10 % slower at 8192 x 8192 and
+  // 16384 x 16384: the kernel waits on memory, not on LDS.
   appendf(s, "const %s ga_lo = LID_0 & %uu;\nconst %s ga_hi = LID_0 / %uu;\n", N, Q - 1, N, Q);
   appendf(s, "const %s ga_gy = ((%s)dim%u + %uu) / %uu;\n", N, N, yd, T - 1, T);
   // Tiles of one plane are handed out in bands of ga_ltx tile rows, walking
@@ -682,12 +690,29 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   appendf(s, "const %s ga_pl = ga_gx * ga_gy;\n", N);
   appendf(s, "%s ga_r = GID_0 / ga_pl;\n", N);
   appendf(s, "const %s ga_g = GID_0 - ga_r * ga_pl;\n", N);
-  appendf(s, "const %s ga_band = ga_g / (ga_ltx * ga_gx);\n", N);
-  appendf(s, "const %s ga_in = ga_g - ga_band * ga_ltx * ga_gx;\n", N);
-  appendf(s, "const %s ga_left = ga_gy - ga_band * ga_ltx;\n", N);
-  appendf(s, "const %s ga_bh = ga_left < (%s)ga_ltx ? ga_left : (%s)ga_ltx;\n", N, N, N);
-  appendf(s, "const %s ga_bx = ga_in / ga_bh;\n", N);
-  appendf(s, "const %s ga_by = ga_band * ga_ltx + (ga_in - ga_bx * ga_bh);\n", N);
+  // Low half of ga_ltx = 0: diagonal order instead.  The plane is cut into
+  // panels of ga_pw tile columns (high half of ga_ltx; 0: one panel), and tile
+  // row r of a panel is walked along a diagonal, (bx, (r + bx) mod gy):
+  // consecutive groups then differ in both coordinates, so neither the rows
+  // they read nor the rows they write start a whole number of row pitches
+  // apart (with a power-of-two pitch such rows fall on the same memory
+  // channels), while a panel keeps the groups that run together within a
+  // bounded span of the output's rows.
+  appendf(s, "%s ga_bx, ga_by;\nconst %s ga_ord = ga_ltx & 0xffffu;\n", N, N);
+  s += "if (ga_ord == 0u) {\n";
+  appendf(s, "%s ga_pw = ga_ltx >> 16;\nif (ga_pw == 0u || ga_pw > ga_gx) ga_pw = ga_gx;\n", N);
+  appendf(s, "const %s ga_pn = ga_g / (ga_pw * ga_gy);\n", N);
+  appendf(s, "const %s ga_pl2 = ga_g - ga_pn * ga_pw * ga_gy;\n", N);
+  appendf(s, "const %s ga_rest = ga_gx - ga_pn * ga_pw;\n", N);
+  appendf(s, "const %s ga_w = ga_rest < ga_pw ? ga_rest : ga_pw;\n", N);
+  appendf(s, "const %s ga_tr = ga_pl2 / ga_w;\n", N);
+  appendf(s, "const %s ga_tc = ga_pl2 - ga_tr * ga_w;\n", N);
+  s += "ga_bx = ga_pn * ga_pw + ga_tc;\nga_by = (ga_tr + ga_tc) % ga_gy;\n} else {\n";
+  appendf(s, "const %s ga_band = ga_g / (ga_ord * ga_gx);\n", N);
+  appendf(s, "const %s ga_in = ga_g - ga_band * ga_ord * ga_gx;\n", N);
+  appendf(s, "const %s ga_left = ga_gy - ga_band * ga_ord;\n", N);
+  appendf(s, "const %s ga_bh = ga_left < ga_ord ? ga_left : ga_ord;\n", N);
+  s += "ga_bx = ga_in / ga_bh;\nga_by = ga_band * ga_ord + (ga_in - ga_bx * ga_bh);\n}\n";
   for (const ge_arg &a : ge->args)
     if (a.is_array()) appendf(s, "%s %s_o = 0;\n", I, a.name.c_str());
   if (nd >= 3) {
@@ -1184,26 +1209,51 @@ class strided_call {
       groups = gx * ((rows + ty - 1) / ty);
     } else {
       // Transposed tiles.  A group takes a 64 x 64 tile (256 lanes) or a
-      // 128 x 128 tile (1024 lanes); the tiles of a plane are handed out in bands
-      // of `ltx` tile rows, down a band's rows first.  Measured on MI355X for
-      // out = in.T of n x n floats: n = 4096 (4096 small tiles) 26.8 us with
-      // small tiles in row-major order, 27.6-28.8 with large ones; n = 8192
-      // 112.6 us small row-major, 106.2 small in bands of 8, 91.3 / 93.3 / 89.8
-      // large in bands of 1 / 2 / 4.  So the large tile is used when it still
-      // gives every compute unit eight groups and its staging copies leave room
-      // for two groups per unit.
+      // 128 x 128 tile (1024 lanes).  The tiles of a plane are handed out
+      // either in bands of `ltx` tile rows, down a band's rows first, or
+      // (ltx = 0) along diagonals, so that groups running together differ in
+      // both tile coordinates.  Measured on MI355X, kernel time of
+      // out = in.T of floats, small / large tiles, each in row-major order
+      // (bands of 1), bands of 8 and diagonal order:
+      //    4096 x  4096   24.5  25.3  24.4 |  24.8  23.9  23.6 us
+      //    8192 x  8192  108.9 103.1  93.4 |  88.1  88.1  82.1
+      //   16384 x 16384  433   471   406   | 364   422   398
+      //    2048 x 16384   51.1  52.5  48.7 |  47.0  49.5  44.9
+      //   16384 x  2048   50.8  53.4  61.1 |  48.2  47.0  53.8
+      //    6144 x  6144   54.5  56.7  57.4 |  53.6  53.7  57.3
+      //    3000 x  5000   31.1  29.5  36.6 |  27.3  27.5  28.7
+      // and the same in.T with two broadcast operands on 4096 x 4096 25.7 /
+      // 25.7 / 24.9 | 26.1 / 25.8 / 25.1 (a plain copy of as many bytes: 22.3).
+      // So: the large tile from half a group per compute unit on, when its
+      // staging copies leave room for two groups per unit; diagonal
+      // order when every row pitch involved is a power of two of 4 to 32 KiB
+      // (rows that many bytes apart fall on the same memory channels, and
+      // row-major order then has all groups of a tile row read such rows);
+      // row-major order otherwise.
       if (vec4) {
         size_t lds128 = 0;
         for (unsigned k = 0; k < na; k++)
           if ((tmask >> k) & 1u) lds128 += (size_t)128 * 129 * elsz[k];
         const size_t tiles128 = ((dims[nd - 1] + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
                                 (n / dims[nd - 1] / dims[nd - 2]);
-        tile = (tiles128 >= (size_t)8 * ga_hip_numprocs(ctx) && lds128 <= 80 * 1024) ? 128 : 64;
+        // large against small tiles on smaller planes: 1536 x 1536 4.6 / 4.9 us,
+        // 2048 x 2048 6.2 / 6.9, 16 planes of 512 x 512 6.0 / 6.6, 3072 x 3072
+        // 15.3 / 14.8, 1024 x 1024 4.2 / 4.2
+        const size_t min128 = env_ul("GPUARRAY_ELEMWISE_TTILE_MIN", ga_hip_numprocs(ctx) / 2);
+        tile = (tiles128 >= min128 && lds128 <= 80 * 1024) ? 128 : 64;
         const unsigned long ft = env_ul("GPUARRAY_ELEMWISE_TTILE", 0);
         if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
         const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
-        ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", tile == 128 ? 4 : (tiles >= 8192 ? 8 : 1));
-        if (ltx < 1) ltx = 1;
+        bool aliasing = true;   // every pitch a power of two of 4 to 32 KiB
+        for (unsigned k = 0; k < na && aliasing; k++) {
+          // operands that are broadcast along x or y are a row or a column, not a plane
+          if (strs[k][nd - 1] == 0 || strs[k][nd - 2] == 0) continue;
+          const size_t pitch = sabs(strs[k][((tmask >> k) & 1u) ? nd - 1 : nd - 2]);
+          aliasing = (pitch & (pitch - 1)) == 0 && pitch >= 4096 && pitch <= 32768;
+        }
+        const unsigned long dflt = aliasing ? 0 : (tile == 128 ? 1 : (tiles >= 8192 ? 8 : 1));
+        ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", dflt) & 0xffffu;
+        if (ltx == 0) ltx |= ((unsigned)env_ul("GPUARRAY_ELEMWISE_PANEL", 0) & 0xffffu) << 16;
       }
       gx = (dims[nd - 1] + tile - 1) / tile;
       size_t gy = (dims[nd - 2] + tile - 1) / tile;

@@ -17,6 +17,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <iterator>
 #include <list>
 #include <map>
@@ -511,10 +512,19 @@ gpucontext *hip_init(gpucontext_props *p) {
   size_t alen = strcspn(arch, ":");
   snprintf(ctx->bin_id, sizeof(ctx->bin_id), "%.*s", (int)alen, arch);
 #undef INIT_TRY
+  // Every kernel is compiled for gfx950 (wave64, its DPP and LDS forms): say
+  // so here rather than at the first module load on another ISA.
+  if (strcmp(ctx->bin_id, "gfx950") != 0 && env_ul("GPUARRAY_ALLOW_OTHER_ISA", 0) == 0) {
+    ga_err_fmt(ga_global_err, GA_DEVSUP_ERROR,
+               "Device %d is %s; this library generates code for gfx950 (MI355X) only", dev, ctx->bin_id);
+    ctx_destroy(ctx);
+    return nullptr;
+  }
   // Where this device keeps the library's static scratch array (the partials
   // of GpuReduction_call_noalloc).  A failed lookup only disables that entry
   // point, which then reports the code kept here.
   ctx->static_scratch_err = ga_static_scratch_setup(dev, &ctx->static_scratch);
+
   {
     const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
     if (dc != nullptr && *dc != 0) ctx->disk_cache = dc;
@@ -916,6 +926,11 @@ std::string disk_key(const std::string &src, const char *isa) {
   std::string k = "ga-hip-kcache-1|";
   int maj = 0, min = 0;
   if (hiprtcVersion(&maj, &min) == HIPRTC_SUCCESS) k += std::to_string(maj) + "." + std::to_string(min);
+  // the runtime's full version too: a patch release of the compiler must not
+  // be served code objects its predecessor made
+  int rtv = 0;
+  if (hipRuntimeGetVersion(&rtv) == hipSuccess) k += "/" + std::to_string(rtv);
+  else (void)hipGetLastError();
   k += "|";
   k += isa;
   for (const char *o : k_rtc_opts) { k += "|"; k += o; }
@@ -989,7 +1004,9 @@ bool disk_load(const std::string &dir, const std::string &key, std::vector<char>
 
 void disk_store(const std::string &dir, const std::string &key, const std::vector<char> &code) {
   std::string path = disk_path(dir, key, true);
-  std::string tmp = path + ".tmp." + std::to_string((long)getpid());
+  // unique per store: two contexts or threads of one process may store the same key
+  static std::atomic<unsigned long> serial{0};
+  std::string tmp = path + ".tmp." + std::to_string((long)getpid()) + "." + std::to_string(serial++);
   FILE *f = fopen(tmp.c_str(), "wb");
   if (f == nullptr) return;   // a cache that cannot be written is only slower
   unsigned char hdr[16];

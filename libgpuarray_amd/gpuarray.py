@@ -523,16 +523,20 @@ class GpuArray(object):
 
     base_data = data
 
-    def take1(self, idx):
+    def take1(self, idx, check=True):
         """Rows of `self` picked by the 1-D integer array `idx`
         (reference pygpu/gpuarray.pyx:2098-2113): negative entries count from
-        the end, an entry out of range raises IndexError."""
+        the end, an entry out of range raises IndexError.  check=False is
+        GpuArray_take1's check_error = 0: the call does not wait for the
+        kernel to read the bounds flag back, a row whose index is out of range
+        keeps what the result's memory held, and the flag stays set for the
+        next checked call (reference src/gpuarray_array.c:534-543)."""
         if idx.ndim != 1:
             raise ValueError("Expected index with nd=1")
         if self.ndim == 0:
             raise _lib.GpuArrayException("take1 of a 0-d array", _lib.GA_INVALID_ERROR)
         res = empty((idx.shape[0],) + self.shape[1:], self.dtype, context=self.context)
-        err = lib.GpuArray_take1(res._ptr(), self._ptr(), idx._ptr(), 1)
+        err = lib.GpuArray_take1(res._ptr(), self._ptr(), idx._ptr(), 1 if check else 0)
         if err == _lib.GA_VALUE_ERROR:
             msg = lib.gpucontext_error(self.context.ctx, err)
             raise IndexError(msg.decode(errors="replace") if msg else "Index out of bounds")

@@ -224,14 +224,15 @@ class MapReduction(object):
               self.context.ctx)
 
 
-_cache = {}
-
-
 def _operator(context, op, dtype):
-    key = (id(context), op, np.dtype(dtype).str)
-    r = _cache.get(key)
-    if r is None or r.context is not context:
-        r = _cache[key] = GpuReduction(context, op, dtype)
+    """The GpuReduction for (op, dtype), kept on the context object itself (as
+    the elementwise helpers keep theirs), so that dropping the context frees
+    the operators and, with them, the context's device memory."""
+    cache = context.__dict__.setdefault("_reduction_cache", {})
+    key = (op, np.dtype(dtype).str)
+    r = cache.get(key)
+    if r is None:
+        r = cache[key] = GpuReduction(context, op, dtype)
     return r
 
 

@@ -267,3 +267,50 @@ def run_reduk_sum_axis1(x, device_type="cpu", reps=3):
                 "max_relative_error": rel}
     finally:
         sess.close()
+
+
+def main(argv=None):
+    """python -m oracle.opencl_runner --device-type gpu c1:24 c2:4096 c3a:8192
+    One JSON line per case: the reference's kernel for that configuration on the
+    first OpenCL device of the type (c1:L = 2^L elements, c2:N = N x N,
+    c3a:N = sum over axis 1 of N x N), inputs from the benchmark's seeds."""
+    import argparse
+    import json
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--device-type", default="cpu", choices=sorted(DEVICE_TYPES))
+    ap.add_argument("cases", nargs="+")
+    args = ap.parse_args(argv)
+    for case in args.cases:
+        kind, size = case.split(":")
+        size = int(size)
+        try:
+            if kind == "c1":
+                rng = np.random.default_rng(0)
+                n = 1 << size
+                a = rng.uniform(-1, 1, n).astype(np.float32)
+                b = rng.uniform(-1, 1, n).astype(np.float32)
+                res = run_contig_muladd(a, b, args.device_type)
+                res["algorithmic_bytes"] = 12 * n
+            elif kind == "c2":
+                rng = np.random.default_rng(1)
+                A = rng.normal(0, 1, (size, size)).astype(np.float32)
+                B = rng.normal(0, 1, (1, size)).astype(np.float32)
+                Cc = rng.normal(0, 1, (size, 1)).astype(np.float32)
+                res = run_strided_broadcast(A.T, B, Cc, args.device_type)
+                res["algorithmic_bytes"] = 8 * size * size + 8 * size
+            elif kind == "c3a":
+                X = np.random.default_rng(2).standard_normal((size, size), dtype=np.float32)
+                res = run_reduk_sum_axis1(X, args.device_type)
+                res["algorithmic_bytes"] = 4 * size * size + 4 * size
+            else:
+                raise ValueError("unknown case " + case)
+            res["GBps"] = round(res["algorithmic_bytes"] / res["seconds_per_launch"] / 1e9, 1)
+            res["us_per_launch"] = round(res.pop("seconds_per_launch") * 1e6, 2)
+        except Exception as e:   # one case failing does not hide the others
+            res = {"error": repr(e)}
+        res["case"] = case
+        print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -85,7 +85,10 @@ def check_float_sum(got, truth64, mag64, rtol=1e-5, cancel=1e-3, what=""):
     |sum| >= cancel * (sum of magnitudes `mag64`).  Below that the relative
     criterion is ill-posed (the exact sum can be 0), and the bound is what any
     summation order of float32 values can promise: 8 * 2^-24 * sum of
-    magnitudes.  Returns the largest relative error among the results held to
+    magnitudes.  cancel = 1e-3 suits long sums (thousands of elements, where
+    partial sums stay far below the sum of magnitudes); for sums of a few dozen
+    elements a single rounding of a partial sum exceeds rtol * |sum| once the
+    result is below 1e-2 of the magnitudes.  Returns the largest relative error among the results held to
     rtol and the fraction of results that took the fallback, so that callers
     can bound and report both."""
     got = np.asarray(got, dtype=np.float64)

@@ -448,14 +448,17 @@ def test_linearity_at_full_size(ctx):
         assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("tile,band", [(64, 1), (64, 3), (64, 8), (128, 1), (128, 2), (128, 5)])
-def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band):
-    """Every tile size and band height of the transposed kernels, on extents
-    that leave ragged tiles and a partial last band, with one and with two
-    transposed operands, a transposed result, several planes and 8-byte
-    elements: bit-exact against NumPy."""
+@pytest.mark.parametrize("tile,band,panel", [(64, 0, 0), (64, 0, 3), (64, 1, 0), (64, 3, 0), (64, 8, 0),
+                                             (128, 0, 0), (128, 0, 2), (128, 1, 0), (128, 2, 0), (128, 5, 0)])
+def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band, panel):
+    """Every tile size and tile order of the transposed kernels (bands of
+    `band` tile rows; 0: diagonals, within panels of `panel` tile columns), on
+    extents that leave ragged tiles, a partial last band and a narrower last
+    panel, with one and with two transposed operands, a transposed result,
+    several planes and 8-byte elements: bit-exact against NumPy."""
     monkeypatch.setenv("GPUARRAY_ELEMWISE_TTILE", str(tile))
     monkeypatch.setenv("GPUARRAY_ELEMWISE_BAND", str(band))
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_PANEL", str(panel))
     rng = np.random.default_rng(40 + tile + band)
     f32 = "float32"
     k2 = ga.GpuElemwise(ctx, "out = a + b*c", [arg("a", f32, read=True), arg("b", f32, read=True),

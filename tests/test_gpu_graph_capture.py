@@ -88,3 +88,57 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
     finally:
         hip.hipGraphExecDestroy(gexec)
         hip.hipGraphDestroy(graph)
+
+
+def test_scratch_that_a_graph_recorded_is_never_handed_out_again(monkeypatch):
+    """A graph holds the address of the scratch buffer its split reductions
+    write partials to.  When a later, larger split reduction outgrows that
+    buffer, the old one must stay out of circulation: were it given back to
+    the memory cache, the caller's next array could land on it and every
+    replay would write partials into that array.  A context of its own, so
+    that the scratch buffer starts at its smallest size whatever ran before."""
+    if ga.count_devices() == 0:
+        pytest.skip("no HIP device")
+    ctx = ga.init("hip0")
+    hip = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p(_lib.extension("hip_get_stream", C.c_void_p, [C.c_void_p])(ctx.ctx))
+    f32 = "float32"
+    rsum = ga.GpuReduction(ctx, "sum", f32)
+    n = 1 << 24
+    hx = np.random.default_rng(91).standard_normal(n).astype(np.float32)
+    x = gpuarray.array(hx, context=ctx)
+    tot = gpuarray.zeros((), f32, context=ctx)
+    rsum(x, [0], d0=tot)                 # two launches: partials rest in the scratch buffer (1 MiB)
+    ctx.sync()
+    want = float(np.asarray(tot))
+    assert abs(want - float(hx.sum(dtype=np.float64))) <= 1e-5 * abs(float(hx.sum(dtype=np.float64)))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0
+    try:
+        rsum(x, [0], d0=tot)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+    try:
+        # an eager split reduction whose partials outgrow that buffer: 8 pieces
+        # for each of 65536 columns, 6 MiB
+        monkeypatch.setenv("GPUARRAY_REDUX_GROUPS_PER_CU", "256")
+        wide = gpuarray.zeros((512, 65536), f32, context=ctx)
+        cols = gpuarray.empty((65536,), f32, context=ctx)
+        rsum(wide, [0], d0=cols)
+        monkeypatch.delenv("GPUARRAY_REDUX_GROUPS_PER_CU")
+        ctx.sync()
+        # arrays made now take whatever blocks the cache has free
+        fresh = [gpuarray.array(np.full(1 << 16, 5.0, np.float32), context=ctx) for _ in range(32)]
+        for k in range(3):
+            tot.write(np.float32(-1))
+            ctx.sync()
+            assert hip.hipGraphLaunch(gexec, stream) == 0
+            ctx.sync()
+            assert float(np.asarray(tot)) == want, k
+            for f in fresh:
+                assert np.all(np.asarray(f) == 5.0), "a replay wrote into an array allocated after the capture"
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)

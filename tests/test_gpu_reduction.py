@@ -25,13 +25,17 @@ def np_maxandargmax(x, redux, op="max"):
     return (y.max(-1), y.argmax(-1)) if op == "max" else (y.min(-1), y.argmin(-1))
 
 
-def assert_sum_close(got, x64sum, abs64sum, rtol=1e-5):
-    """1e-5 of the float64 sum wherever the sum is not a cancellation (at least
-    1e-3 of the sum of magnitudes); 8 float32 epsilons of the sum of magnitudes
-    below that, where a relative bound on a result near zero means nothing.
-    Returns (largest relative error among the results held to rtol, fraction
-    of results that took the fallback)."""
-    return check_float_sum(got, x64sum, abs64sum, rtol=rtol)
+def assert_sum_close(got, x64sum, abs64sum, rtol=1e-5, cancel=1e-2):
+    """1e-5 of the float64 sum wherever the sum is not a cancellation; 8
+    float32 epsilons of the sum of magnitudes below that, where a relative
+    bound on a result near zero means nothing.  The layout tests, whose sums
+    have as few as three elements, call a result a cancellation when it is
+    below 1e-2 of the sum of magnitudes: one rounding of one partial sum of
+    that size is already 1e-5 of such a result in float32, whatever the order.
+    The benchmark's long sums are held to 1e-3 (cancel=1e-3).  Returns (largest
+    relative error among the results held to rtol, fraction of results that
+    took the fallback)."""
+    return check_float_sum(got, x64sum, abs64sum, rtol=rtol, cancel=cancel)
 
 
 # ---- the reference's four tests ------------------------------------------------------
@@ -398,7 +402,7 @@ def test_config3a_sum_axis1_8192(ctx, oracle):
     got = np.asarray(R.sum(g, axis=1))
     # float64 sums without a float64 copy of the array
     want, mag = x.sum(axis=1, dtype=np.float64), np.abs(x).sum(axis=1, dtype=np.float64)
-    worst, fallback = assert_sum_close(got, want, mag)
+    worst, fallback = assert_sum_close(got, want, mag, cancel=1e-3)
     # Rows of 8192 N(0,1) values: |sum| ~ 90, sum of magnitudes ~ 6536, so
     # about 6 % of the rows are cancellations below 1e-3 of it; every other
     # row is held to 1e-5 relative.
@@ -411,7 +415,7 @@ def test_config3a_sum_axis1_8192(ctx, oracle):
     # and the other axis (column kernel)
     got0 = np.asarray(R.sum(g, axis=0))
     worst0, fallback0 = assert_sum_close(got0, x.sum(axis=0, dtype=np.float64),
-                                         np.abs(x).sum(axis=0, dtype=np.float64))
+                                         np.abs(x).sum(axis=0, dtype=np.float64), cancel=1e-3)
     assert fallback0 <= 0.08, fallback0
     _record("sum axis 0 of 8192x8192", max_relative_error=worst0, rows_on_fallback=fallback0)
 
