@@ -46,6 +46,20 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # are in profiles/hbm_traffic_all_configs.md.
 MEASURED_TRAFFIC = {
     # name: (kernel text hash, HBM bytes per call)
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201267465),
+    "C2_transposed_broadcast_4096": ("31f225248b8a2bfc", 134377945),
+    "C3a_sum_axis1_8192x8192": ("af7b7879c9561f8e", 268801984),
+    "C4_maxandargmax_65536x1000": ("477bbd70f85a432b", 263560871),
+    "C5_fp16_sum_axes02": ("f7232deb541fe4a7", 269751876),
+    "C5_int32_sum_axis1": ("3b05a07392f4de39", 538046866),
+    "C5_uint8_all_axis2": ("ece4e206d7eb6e28", 134404991),
+    "C5_uint8_any_axis2": ("370ef90477d5a858", 134388338),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538713359),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538715569),
+    "F4_dot_2x2^27_fused": ("7ba3850e95efbaa6", 1073828760),
+    "F4_dot_2x2^27_two_pass": ("32a750908c0f762d", 2146824867),
+    "elem_2^28": ("712fba8f0b8a6108", 3219703989),
+    "sum_2^28": ("32a750908c0f762d", 1073816083),
 }
 
 
@@ -156,6 +170,20 @@ def cfg_c2(ctx, ga, R):
             "check": check, "numpy": lambda: A.T + B * Cc}
 
 
+def cfg_transpose(ctx, ga, R):
+    # Beyond the benchmark's own shapes: a pure transposing copy, the pattern
+    # configuration 2 contains, at a size where the chip is full.
+    n = 8192
+    A = np.random.default_rng(11).standard_normal((n, n), dtype=np.float32)
+    k = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", f32, read=True), ga.arg("dst", f32, write=True)])
+    rot = 2
+    sets = [(ga.array(A, context=ctx).T, ga.empty((n, n), f32, context=ctx)) for _ in range(rot)]
+    return {"bytes": 8 * n * n, "call": lambda i: k(*sets[i % rot]), "sets": 1,
+            "check": lambda: all(np.array_equal(np.asarray(s_[1]), A.T) for s_ in sets),
+            "numpy": lambda: np.ascontiguousarray(A.T), "numpy_reps": 1,
+            "note": "out = in.T of 8192 x 8192 floats (512 MiB of traffic; two buffer sets)"}
+
+
 def cfg_c3a(ctx, ga, R):
     X = np.random.default_rng(2).standard_normal((8192, 8192), dtype=np.float32)
     op = ga.GpuReduction(ctx, "sum", f32)
@@ -187,8 +215,9 @@ def cfg_c4(ctx, ga, R):
 
 
 C5_SHAPE = (256, 512, 1024)
-C5_NOTE = ("useful bytes of a stride-2 view: every fetched line is half used, so the ceiling in "
-           "useful bytes is 50 % of peak (268 MB footprint: no cold/warm split)")
+C5_NOTE = ("useful bytes of a stride-2 view: every fetched line is half used (the byte counters read "
+           "1.997 to 2.010 x the useful bytes, traffic_over_algorithmic), so the ceiling in useful "
+           "bytes is 50 % of peak (268 MB footprint: no cold/warm split)")
 
 
 def cfg_c5_f16(ctx, ga, R):
@@ -287,6 +316,7 @@ def _cfg_take1(check):
 CONFIGS = [
     ("C1_elemwise_2^24", cfg_c1),
     ("C2_transposed_broadcast_4096", cfg_c2),
+    ("X_transpose_8192x8192", cfg_transpose),
     ("C3a_sum_axis1_8192x8192", cfg_c3a),
     ("C4_maxandargmax_65536x1000", cfg_c4),
     ("C5_fp16_sum_axes02", cfg_c5_f16),
@@ -575,19 +605,29 @@ def main():
                                              ga.arg("dst", "float32", write=True)])
     only = args.only
     hashes = {}
+    # Below the target size the one-kernel modes rotate over four copies of the
+    # buffers, so that a footprint the 256 MB Infinity Cache could hold is
+    # measured from HBM (the step itself is only ever run at sizes far above).
+    sets = [(a, b, c, x)]
+    if only != "step" and 16 * n <= (1 << 30):
+        sets += [(ga.array(a_h, context=ctx), ga.array(b_h, context=ctx), ga.empty((n,), "float32", context=ctx),
+                  ga.array(x_h, context=ctx)) for _ in range(3)]
+    calls = [0]
 
     def step(i=None):
+        a_, b_, c_, x_ = sets[calls[0] % len(sets)]
+        calls[0] += 1
         if i is not None:
             ctx.mark(3 * i)
         if only in ("step", "elem"):
-            elem(a, b, c)
+            elem(a_, b_, c_)
             hashes["elem"] = ctx.last_launch_hash()
         elif only == "copy":
-            copy(a, c)
+            copy(a_, c_)
         if i is not None:
             ctx.mark(3 * i + 1)
         if only in ("step", "sum"):
-            summ(x, [0], d0=s)
+            summ(x_, [0], d0=s)
         if i is not None:
             ctx.mark(3 * i + 2)
 
@@ -615,7 +655,8 @@ def main():
         kern, launches = time_kernels(ctx, lambda i: step(), iters=K, warm=0)
         print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
                           "kernel_us": round(kern, 2), "launches_per_call": launches,
-                          "bytes_per_launch": nbytes, "kernel_text_hash": ctx.last_launch_hash(),
+                          "bytes_per_launch": nbytes, "buffer_sets": len(sets),
+                          "kernel_text_hash": ctx.last_launch_hash(),
                           "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1),
                           "GBps_kernel": round(nbytes / kern / 1e3, 1)}))
         return

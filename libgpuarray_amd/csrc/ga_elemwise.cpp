@@ -95,6 +95,9 @@ struct _GpuElemwise {
   bool nontemporal = true;  // streaming hint on the flat kernel's loads and stores
   unsigned flat_nt_mask = ~0u;   // ... per array (bit k: array k)
   GpuKernel k_flat = {nullptr, nullptr};
+  // the flat kernel with 2 or 4 adjacent chunks per lane, built on first use
+  std::map<unsigned, GpuKernel> k_flat_tiled;
+  bool flat_forced = false;   // the environment fixed the flat kernel's shape
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
   // planning scratch
@@ -146,9 +149,10 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 //   kilobyte) before the first use.  The elements before the first chunk and
 //   after the last one, and the whole range when ga_vec == 0, run one element
 //   per lane.
-std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
+std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned unroll = 0, int tiled = -1) {
   std::string s;
-  const unsigned V = ge->vec, U = ge->unroll;
+  const unsigned V = ge->vec, U = unroll ? unroll : ge->unroll;
+  const bool tile = tiled < 0 ? ge->tile : tiled != 0;
   emit_header(ge, s);
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size n";
   ktypes.push_back(GA_SIZE);
@@ -179,7 +183,7 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes) {
     for (const ge_arg &a : ge->args)
       if (a.is_array()) appendf(s, "%s_p += ga_head;\n", a.name.c_str());
     appendf(s, "const ga_size ga_nchunks = (n - ga_head) / %uu;\n", V);
-    if (ge->tile) {
+    if (tile) {
       appendf(s, "const ga_size ga_ustep = 256;\n"
                  "for (ga_size ga_c0 = (ga_size)GID_0 * %uu + LID_0; ga_c0 - LID_0 < ga_nchunks; "
                  "ga_c0 += (ga_size)GDIM_0 * %uu) {\n", 256 * U, 256 * U);
@@ -900,29 +904,21 @@ int check_flat(GpuElemwise *ge, void **args, size_t *n_out, bool *flat) {
 // Launch the flat kernel over n elements; offs[k] is the byte offset of
 // array k's first element in its buffer.
 int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
-  GpuKernel *k = &ge->k_flat;
-  unsigned p = 0, l = 0;
+  unsigned l = 0;
   int err;
   unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u, head = ~0u;
   std::vector<unsigned> heads;
-  if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
   for (size_t i = 0; i < ge->args.size(); i++) {
-    if (ge->args[i].is_array()) {
-      GpuArray *a = (GpuArray *)args[i];
-      size_t off = offs[l++];
-      // Elements from this array's start to its next chunk boundary.  The
-      // first written array (else the first array) sets the head of the
-      // vector path; an array with another count is moved element by element.
-      const size_t elsz = gpuarray_get_elsize(a->typecode), chunk = elsz * ge->vec;
-      const size_t mis = ((uintptr_t)a->data->devptr + off) % chunk;
-      if (mis % elsz != 0) vec_ok = 0;
-      heads.push_back((unsigned)((chunk - mis) % chunk / elsz));
-      if (head == ~0u && ge->args[i].writes()) head = heads.back();
-      if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
-      if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
-    } else {
-      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
-    }
+    if (!ge->args[i].is_array()) continue;
+    GpuArray *a = (GpuArray *)args[i];
+    // Elements from this array's start to its next chunk boundary.  The
+    // first written array (else the first array) sets the head of the
+    // vector path; an array with another count is moved element by element.
+    const size_t elsz = gpuarray_get_elsize(a->typecode), chunk = elsz * ge->vec;
+    const size_t mis = ((uintptr_t)a->data->devptr + offs[l++]) % chunk;
+    if (mis % elsz != 0) vec_ok = 0;
+    heads.push_back((unsigned)((chunk - mis) % chunk / elsz));
+    if (head == ~0u && ge->args[i].writes()) head = heads.back();
   }
   if (head == ~0u) head = heads.empty() ? 0 : heads[0];
   if (n < (size_t)head + ge->vec || heads.size() > 24) vec_ok = 0;
@@ -931,7 +927,6 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
     if (heads[q] != head) vec_arg |= 1u << (8 + q);
   if (!env_ul("GPUARRAY_ELEMWISE_MIXED_ALIGN", 1) && (vec_arg >> 8)) vec_arg = 0;
   if (vec_arg == 0) vec_ok = 0;
-  if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
 
   // Grid: one lane per chunk (or per element) up to a fixed number of groups
   // per compute unit; beyond that the lanes stride over the range.
@@ -939,10 +934,55 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   // lane over the whole range sustains 6.5 TB/s, a grid capped at 8..64 groups
   // per compute unit that strides over the range 4.2..5.2 TB/s.  So the cap
   // only matters far beyond that size.
+  const size_t ncu = ga_hip_numprocs(ge->ctx);
   const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 2048);
-  size_t cap = (size_t)ga_hip_numprocs(ge->ctx) * (per_cu ? per_cu : 2048);
+  size_t cap = ncu * (per_cu ? per_cu : 2048);
   size_t units = vec_ok ? (n - head) / ge->vec + 1 : n;
-  size_t per_group = GE_LANES * (size_t)((vec_ok && ge->tile) ? ge->unroll : 1);
+  // A compute unit holds eight groups of this kernel at a time.  A grid of
+  // one to two such fills runs its second, partial fill at a fraction of the
+  // chip: two adjacent chunks per lane (four up to four fills) make it a
+  // single fill.  Measured on MI355X, c = a*b + 0.5f on floats, kernel time
+  // with 1 / 2 / 4 chunks per lane: 3 * 2^20 elements 8.3 / 7.3 / 8.5 us, 2^22
+  // 10.0 / 8.9 / 9.9, 3 * 2^21 13.7 / 13.7 / 12.5, 2^23 17.3 / 18.0 / 16.5;
+  // below (2^21: 5.8 / 6.4 / 7.8) and above (3 * 2^22: 25.0 / 26.3 / 26.9,
+  // 2^24 32.6 / 34.1 / 35.3, 2^28 496 / 509 / 531) one chunk per lane is best.
+  unsigned tiled_u = 0;
+  if (vec_ok && !ge->flat_forced && !ge->tile) {
+    // whole chunks only: the extra unit that covers head and tail does not add a group's worth of work
+    const size_t g1 = (units - 1 + GE_LANES - 1) / GE_LANES, fill = ncu * 8;
+    if (g1 > fill && g1 <= 2 * fill) tiled_u = 2;
+    else if (g1 > 2 * fill && g1 <= 4 * fill) tiled_u = 4;
+  }
+  GpuKernel *k = &ge->k_flat;
+  if (tiled_u) {
+    auto it = ge->k_flat_tiled.find(tiled_u);
+    if (it == ge->k_flat_tiled.end()) {
+      std::vector<int> ktypes;
+      std::string src = gen_flat(ge, ktypes, tiled_u, 1);
+      GpuKernel nk = {nullptr, nullptr};
+      if ((err = build_kernel(ge, &nk, src, ktypes)) != GA_NO_ERROR) return err;
+      it = ge->k_flat_tiled.emplace(tiled_u, nk).first;
+    }
+    k = &it->second;
+  }
+  const bool tile = tiled_u ? true : ge->tile;
+  const unsigned unroll = tiled_u ? tiled_u : ge->unroll;
+
+  unsigned p = 0;
+  l = 0;
+  if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (ge->args[i].is_array()) {
+      GpuArray *a = (GpuArray *)args[i];
+      size_t off = offs[l++];
+      if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
+      if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
+    } else {
+      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
+    }
+  }
+  if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
+  size_t per_group = GE_LANES * (size_t)((vec_ok && tile) ? unroll : 1);
   size_t want = (units + per_group - 1) / per_group;
   size_t gs = want < 1 ? 1 : (want > cap ? cap : want);
   size_t ls = GE_LANES;
@@ -1342,6 +1382,7 @@ static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, 
   // many arrays are live at once
   ge->vec = maxel >= 16 ? 1 : (unsigned)(16 / maxel);
   ge->unroll = ge->narray <= 8 ? 2 : 1;
+  ge->flat_forced = getenv("GPUARRAY_ELEMWISE_UNROLL") != nullptr || getenv("GPUARRAY_ELEMWISE_TILE") != nullptr;
   ge->unroll = (unsigned)env_ul("GPUARRAY_ELEMWISE_UNROLL", ge->unroll);
   if (ge->unroll < 1) ge->unroll = 1;
   ge->tile = env_ul("GPUARRAY_ELEMWISE_TILE", 0) != 0;
@@ -1404,6 +1445,7 @@ GpuElemwise *GpuElemwise_new(gpucontext *ctx, const char *preamble, const char *
 void GpuElemwise_free(GpuElemwise *ge) {
   if (ge == nullptr) return;
   if (ge->k_flat.k != nullptr || ge->k_flat.args != nullptr) GpuKernel_clear(&ge->k_flat);
+  for (auto &kv : ge->k_flat_tiled) GpuKernel_clear(&kv.second);
   for (auto &kv : ge->k_strided) GpuKernel_clear(&kv.second);
   delete ge;
 }

@@ -313,7 +313,10 @@ def test_all_fortran_inputs_take_the_flat_path(ctx):
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 65, 255, 256, 257, 1023, 4095, 4096, 4097,
-                               65535, 1 << 20, (1 << 20) + 1, (1 << 22) + 3])
+                               65535, 1 << 20, (1 << 20) + 1, (1 << 22) + 3,
+                               # grids of one to four chip fills: two / four adjacent chunks per lane
+                               (1 << 21) + 1021, (3 << 20) + 1, (1 << 22) - 5, (3 << 21) + 3, (1 << 23) - 1,
+                               (1 << 23) + 1])
 def test_flat_sizes_tails_and_misalignment(n, ctx, oracle):
     rng = np.random.default_rng(n)
     a = rng.uniform(-1, 1, n + 3).astype(np.float32)
