@@ -58,6 +58,8 @@ def main():
     check("elemwise strided vec4 plain, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 2, 0, 0b101 << 16))
     check("elemwise strided vec4 transposed, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 4, 3, 1, 0b001 | (0b110 << 16)))
+    check("elemwise flat, 2 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 5, 0, 0, 0))
+    check("elemwise flat, 4 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 6, 0, 0, 0))
     hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
     check("elemwise half->double copy", gen_e(b"", b"dst = src", 2, hargs, 2, 0, 0, 0, 0))
     n = 0
@@ -128,7 +130,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "12 elementwise)" % (n + 20, m, t))
+          "14 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

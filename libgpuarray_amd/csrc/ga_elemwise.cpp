@@ -1407,7 +1407,9 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // strided: 0 flat, 1 strided one element per lane, 2 strided four elements per
   // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride),
   // 3 the same with streaming 16-byte accesses on every array, 4 as 3 with
-  // 128 x 128 transposed tiles
+  // 128 x 128 transposed tiles; 5 and 6: the flat kernel with 2 and 4 adjacent
+  // chunks per lane
+  if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided == 4 ? 128 : 64)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)

@@ -968,6 +968,23 @@ class reduction_call {
     while (U > 1 && per_pass * (U / 2) >= rin_sz) U /= 2;
     int64_t outer = 1;
     for (int i = 0; i + 1 < p.nr; i++) outer *= p.rdim[i];
+    // A few rows of moderate length are a matter of latency, not of bandwidth:
+    // with eight loads per lane and unit such a row is cut into a handful of
+    // pieces, and each lane then walks a long chain of dependent operations
+    // (for min/max a compare and two selects per element).  Fewer loads per
+    // unit give more units, hence more pieces.  Measured on MI355X, one row of
+    // 2^16 / 2^18 floats, kernel time with 8 / 4 / 2 loads per unit: max 6.8 /
+    // 5.8 / 5.5 and 6.8 / 6.0 / 5.5 us, sum 4.4 / 4.0 / 4.0 and 4.3 / 4.1 / 4.1;
+    // 2^20 floats 7.4 / 7.3 / 7.9 (enough pieces as it is), 2^14 floats 4.7 / 5.0
+    // / 5.5 (too short to be worth cutting at all).
+    if (env_ul("GPUARRAY_REDUX_U", 0) == 0 && rtotal >= 49152) {
+      const int64_t rowgroups_now = (nrows + 256 / G - 1) / (256 / G);
+      auto pieces = [&](unsigned u) {
+        const int64_t units_u = outer * ((rin_sz + per_pass * u - 1) / (per_pass * u));
+        return rowgroups_now * (units_u / 2);
+      };
+      while (U > 2 && pieces(U) < 64) U /= 2;
+    }
     // Several reduced dims with a short inner one (statistics over the batch
     // and a small spatial extent, say): the lanes a row does not need take
     // further outer reduced coordinates.  LI lanes cover the inner dim with up

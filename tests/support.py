@@ -100,5 +100,6 @@ def check_float_sum(got, truth64, mag64, rtol=1e-5, cancel=1e-3, what=""):
     bad = err > bound
     assert not bad.any(), "%s: %d results outside the bound, worst error %.3g against %.3g" % (
         what, int(bad.sum()), float(err[bad].max()), float(bound[bad].min()))
-    rel = err[strict] / np.abs(truth64[strict]) if strict.any() else np.zeros(1)
+    den = np.abs(truth64[strict])       # an all-zero row is "strict" with truth 0: its error is 0 too
+    rel = err[strict] / np.where(den > 0, den, 1.0) if strict.any() else np.zeros(1)
     return float(rel.max()), float(1.0 - strict.mean())

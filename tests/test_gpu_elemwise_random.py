@@ -70,3 +70,68 @@ def test_random_elementwise_matches_numpy(ctx, seed):
         memory = expected if expected.flags.c_contiguous else expected.T
         np.ndarray(c.shape, dtype=c.dtype, buffer=memory, offset=offset, strides=c.strides)[...] = want
         assert np.array_equal(read_root(croot, root), expected), what
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_large_planes_and_flat_size_classes_match_numpy(ctx, monkeypatch, seed):
+    """The paths whose launch shape depends on size: transposed operands over
+    planes of up to 14 x 14 large tiles with ragged edges (tile size, band
+    height, diagonal order and panel width drawn per case, or left to the
+    library), a transposed result, several planes; and the flat kernel at two
+    to eight million elements, where it moves two or four adjacent chunks per
+    lane, with views that start off a 16-byte boundary.  Values are small
+    integers, so every type's result is exact: bit for bit against NumPy."""
+    from libgpuarray_amd import gpuarray
+    rng = np.random.default_rng(700 + seed)
+    kernels = {}
+
+    def kernel(dt, expr, names):
+        if (dt, expr) not in kernels:
+            args = [arg(n, dt, read=True) for n in names[:-1]] + [arg(names[-1], dt, write=True)]
+            kernels[(dt, expr)] = ga.GpuElemwise(ctx, expr, args, convert_f16=True)
+        return kernels[(dt, expr)]
+
+    def values(shape, dt):
+        return rng.integers(0, 11, size=shape).astype(dt)
+
+    for case in range(10):
+        for knob in ("GPUARRAY_ELEMWISE_TTILE", "GPUARRAY_ELEMWISE_BAND", "GPUARRAY_ELEMWISE_PANEL"):
+            monkeypatch.delenv(knob, raising=False)
+        dt = str(rng.choice(["float32", "float32", "float64", "int16"]))
+        mode = int(rng.integers(0, 4))
+        if mode <= 1:
+            if rng.random() < 0.5:
+                monkeypatch.setenv("GPUARRAY_ELEMWISE_TTILE", str(rng.choice([64, 128])))
+            if rng.random() < 0.6:
+                monkeypatch.setenv("GPUARRAY_ELEMWISE_BAND", str(rng.choice([0, 0, 1, 2, 8])))
+                monkeypatch.setenv("GPUARRAY_ELEMWISE_PANEL", str(rng.choice([0, 0, 1, 3, 16])))
+            ny = int(rng.integers(1, 14)) * 128 + int(rng.choice([0, 0, 4, 8, 60, 100]))
+            nx = int(rng.integers(1, 14)) * 128 + int(rng.choice([0, 0, 4, 12, 64, 124]))
+            planes = int(rng.choice([1, 1, 1, 2, 5]))
+            lead = (planes,) if planes > 1 else ()
+            swap = list(range(len(lead))) + [len(lead) + 1, len(lead)]
+            a = values(lead + (nx, ny), dt)
+            a_t = np.swapaxes(a, -1, -2)
+            g_t = gpuarray.array(a, context=ctx).transpose(swap)
+            if mode == 0:       # transposed input, two broadcast inputs
+                b, c = values((1,) * len(lead) + (1, nx), dt), values((1,) * len(lead) + (ny, 1), dt)
+                out = gpuarray.empty(lead + (ny, nx), dt, context=ctx)
+                kernel(dt, "o = a + b*c", "abco")(g_t, gpuarray.array(b, context=ctx), gpuarray.array(c, context=ctx), out)
+                want = (a_t + b * c).astype(dt)
+            else:               # transposed result, a plain and a transposed input
+                x = values(lead + (ny, nx), dt)
+                out = gpuarray.empty(lead + (nx, ny), dt, context=ctx).transpose(swap)
+                kernel(dt, "o = a + b", "abo")(gpuarray.array(x, context=ctx), g_t, out)
+                want = (x + a_t).astype(dt)
+            assert np.array_equal(np.asarray(out), want), (seed, case, dt, mode, ny, nx, planes)
+        else:
+            n = int(rng.choice([1 << 21, 3 << 20, 1 << 22, 3 << 21, 1 << 23])) + int(rng.integers(-3000, 3000))
+            off = int(rng.choice([0, 0, 1, 3]))
+            dst_off = off if mode == 2 else 0       # mode 3: the result starts at another offset than the inputs
+            a, b = values(n + 4, dt), values(n + 4, dt)
+            whole = gpuarray.zeros((n + 4,), dt, context=ctx)
+            kernel(dt, "o = a + b", "abo")(gpuarray.array(a, context=ctx)[off:off + n],
+                                           gpuarray.array(b, context=ctx)[off:off + n], whole[dst_off:dst_off + n])
+            got = np.asarray(whole)
+            assert np.array_equal(got[dst_off:dst_off + n], (a[off:off + n] + b[off:off + n]).astype(dt)), (seed, case, dt, n, off)
+            assert not got[:dst_off].any() and not got[dst_off + n:].any(), (seed, case, "outside the view")
