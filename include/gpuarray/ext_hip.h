@@ -68,7 +68,10 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * staged through LDS; bits 16..: arrays with unit stride along x), 3 the
  * same with the streaming hint on every array's 16-byte accesses, 4 as 3
  * with 128 x 128 transposed tiles (1024 lanes), 5 / 6 the flat kernel with 2 /
- * 4 adjacent chunks per lane. */
+ * 4 adjacent chunks per lane, 7 as 4 with every array in neither mask taken
+ * as constant along x (one load for a lane's four elements), 8 as 4 with
+ * every read-only array outside the LDS mask taken as constant along y (one
+ * load for a lane's four rows). */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
                                            unsigned int n, void *args, int flags,
                                            int strided, unsigned int nd, int idx64,

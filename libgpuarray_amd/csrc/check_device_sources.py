@@ -1,9 +1,10 @@
 """Compile every device-side text for gfx950, without a device.
 
-The library compiles kernels at run time with hipRTC; this script asks the
+The library compiles kernels at run time through the code-object manager
+(libamd_comgr); this script asks the
 freshly built library for representative kernel texts (flat and strided
 elementwise variants, every reduction operation) and runs each through the
-same hipRTC invocation the library uses.  It is the "does the device code
+same compile the library uses.  It is the "does the device code
 build" check of the build step.
 """
 import ctypes as C
@@ -58,6 +59,12 @@ def main():
     check("elemwise strided vec4 plain, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 2, 0, 0b101 << 16))
     check("elemwise strided vec4 transposed, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 4, 3, 1, 0b001 | (0b110 << 16)))
+    check("elemwise strided vec4 transposed, 128-tiles, operand constant along x",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 7, 2, 0, 0b001 | (0b100 << 16)))
+    check("elemwise strided vec4 transposed, 128-tiles, operands constant along y",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 8, 2, 0, 0b001 | (0b110 << 16)))
+    check("elemwise strided vec4 plain, operand constant along x",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 7, 2, 0, 0b100 << 16))
     check("elemwise flat, 2 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 5, 0, 0, 0))
     check("elemwise flat, 4 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 6, 0, 0, 0))
     hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
@@ -130,7 +137,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "14 elementwise)" % (n + 20, m, t))
+          "17 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

@@ -516,7 +516,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
-                            unsigned tile = 64) {
+                            unsigned tile = 64, unsigned zmask = 0) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
@@ -553,6 +553,15 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   }
   auto is_t = [&](size_t j) { return aidx[j] >= 0 && ((tmask >> aidx[j]) & 1u); };
   auto is_u = [&](size_t j) { return aidx[j] >= 0 && ((umask >> aidx[j]) & 1u); };
+  // read-only arrays whose stride along x is zero: one load serves a lane's four elements
+  auto is_z = [&](size_t j) {
+    return aidx[j] >= 0 && ((zmask >> aidx[j]) & 1u) && !ge->args[j].writes();
+  };
+  // the same along y (bits 16.. of zmask; transposed variant only): one load
+  // serves the four rows a lane works on
+  auto is_y = [&](size_t j) {
+    return aidx[j] >= 0 && ((zmask >> (16 + aidx[j])) & 1u) && !ge->args[j].writes();
+  };
   auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * 4); };
   // 16-byte accesses of arrays whose every element is touched once carry the
   // streaming hint (ntmask); broadcast operands stay cacheable
@@ -628,6 +637,10 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       if (!a.is_array() || !a.reads()) continue;
       if (is_u(j)) {
         s += quad_load(j, a.name + "_u[ga_e].c", quad_at(a, a.name + "_o", "ga_x"));
+      } else if (is_z(j)) {
+        appendf(s, "%s_u[ga_e].e[0] = %s;\n", a.name.c_str(), elem_at(a, a.name + "_o", "0").c_str());
+        for (int i = 1; i < 4; i++)
+          appendf(s, "%s_u[ga_e].e[%d] = %s_u[ga_e].e[0];\n", a.name.c_str(), i, a.name.c_str());
       } else {
         for (int i = 0; i < 4; i++) {
           char xi[32];
@@ -744,6 +757,43 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     if (ge->args[j].reads()) any_tr = true;
     if (ge->args[j].writes()) any_tw = true;
   }
+  // loads of the operands that phase 2 reads straight from memory
+  auto emit_direct_loads = [&]() {
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (a.is_array() && !is_t(j))
+        appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), a.name.c_str());
+    }
+    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!a.is_array() || is_t(j) || !a.reads()) continue;
+      if (is_y(j)) s += "if (ga_k == 0) {\n";
+      if (is_u(j)) {
+        std::string pe;
+        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
+                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
+        s += quad_load(j, a.name + "_u[ga_k].c", pe);
+      } else if (is_z(j)) {
+        appendf(s, "%s_u[ga_k].e[0] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(),
+                ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "0").c_str());
+        for (int i = 1; i < 4; i++)
+          appendf(s, "%s_u[ga_k].e[%d] = %s_u[ga_k].e[0];\n", a.name.c_str(), i, a.name.c_str());
+      } else {
+        for (int i = 0; i < 4; i++) {
+          char xi[48];
+          snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
+          appendf(s, "%s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), i,
+                  ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
+        }
+      }
+      // a lane's row 0 is in range whenever one of its later rows is
+      if (is_y(j)) appendf(s, "} else {\n%s_u[ga_k].c = %s_u[0].c;\n}\n", a.name.c_str(), a.name.c_str());
+    }
+    s += "}\n}\n";
+  };
   // phase 1: transposed reads.  lane: y quad ga_lo (y = 4*ga_lo..+3), x column ga_hi + 16k
   if (any_tr) {
     for (size_t j = 0; j < ge->args.size(); j++) {
@@ -766,6 +816,9 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       }
     }
     s += "}\n}\n";
+    // the direct operands of phase 2 are asked for here, behind the tile's
+    // loads and before the barrier, so that their latency is not paid after it
+    emit_direct_loads();
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
     appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
@@ -779,32 +832,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     s += "}\n}\nlocal_barrier();\n";
   }
   // phase 2: the expression.  lane: x quad ga_lo (x = 4*ga_lo..+3), y row ga_hi + 16k
-  for (size_t j = 0; j < ge->args.size(); j++) {
-    const ge_arg &a = ge->args[j];
-    if (a.is_array() && !is_t(j))
-      appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), a.name.c_str());
-  }
-  s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
-  for (size_t j = 0; j < ge->args.size(); j++) {
-    const ge_arg &a = ge->args[j];
-    if (!a.is_array() || is_t(j) || !a.reads()) continue;
-    if (is_u(j)) {
-      std::string pe;
-      appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
-              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
-      s += quad_load(j, a.name + "_u[ga_k].c", pe);
-    } else {
-      for (int i = 0; i < 4; i++) {
-        char xi[48];
-        snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
-        appendf(s, "%s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), i,
-                ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
-      }
-    }
-  }
-  s += "}\n}\n";
+  if (!any_tr) emit_direct_loads();
   s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
   appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
   appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
@@ -1085,6 +1113,7 @@ class strided_call {
   bool vec4 = false;                // four elements per lane
   unsigned umask = 0;               // vec4: arrays with 16-byte access along x
   unsigned ntmask = 0;              // vec4: arrays touched once, streamed past the caches
+  unsigned zmask = 0;               // vec4: arrays whose stride along x (bits 16..: along y) is zero
   size_t gx = 0, groups = 0;
   unsigned ltx = 0, tile = 64;
   GpuKernel *kernel = nullptr;
@@ -1219,7 +1248,11 @@ class strided_call {
         if (!aligned) vec4 = false;          // a transposed operand must be vector-accessible
       } else if (aligned) {
         umask |= 1u << k;
+      } else if (strs[k][nd - 1] == 0 && env_ul("GPUARRAY_ELEMWISE_ZMASK", 1) != 0) {
+        zmask |= 1u << k;
       }
+      if (!tr && tmask && k < 16 && strs[k][nd - 2] == 0 && env_ul("GPUARRAY_ELEMWISE_ZMASK", 1) != 0)
+        zmask |= 1u << (16 + k);
     }
     if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
     // arrays read or written exactly once per element stream past the caches
@@ -1308,14 +1341,14 @@ class strided_call {
 
   int get_kernel() {
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-             vec4 ? umask : 0u, ntmask, tile);
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
@@ -1408,10 +1441,13 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // lane (then bits 16.. of tmask carry the mask of arrays with unit x stride),
   // 3 the same with streaming 16-byte accesses on every array, 4 as 3 with
   // 128 x 128 transposed tiles; 5 and 6: the flat kernel with 2 and 4 adjacent
-  // chunks per lane
+  // chunks per lane; 7 as 4, every array in neither mask taken as constant along x;
+  // 8 as 4, every array that is not staged through LDS taken as constant along y
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
-                                                   strided >= 3 ? 0xffffffffu : 0u, strided == 4 ? 128 : 64)
+                                                   strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
+                                                   strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
+                                                   : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

@@ -128,6 +128,7 @@ int GpuArray_is_aligned(const GpuArray *a);
 
 // ---- HIP backend hooks used by the generators ------------------------------
 // Device prelude and reduction templates, embedded at build time.
+extern const char ga_device_rt_src[];
 extern const char ga_cluda_hip_src[];
 extern const char ga_reduce_kernels_src[];
 

@@ -1,7 +1,7 @@
 // TEST INFRASTRUCTURE ONLY: host-memory stand-ins for the HIP runtime calls the
 // backend makes, preloaded by tests that exercise the library's HOST logic where
 // there is no device (argument checks, buffer bookkeeping, the memory cache,
-// compile errors from hipRTC, context teardown).  Buffers are host allocations,
+// compile errors, context teardown).  Buffers are host allocations,
 // copies are memcpy, a kernel launch does nothing: no result of a kernel means
 // anything here, and nothing the library ships may link or load this file.
 #include <hip/hip_runtime_api.h>

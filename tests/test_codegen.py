@@ -1,4 +1,4 @@
-"""Generated kernel text compiles for gfx950 (hipRTC needs no device), and the
+"""Generated kernel text compiles for gfx950 (the compiler needs no device), and the
 device prelude offers the vocabulary kernels written for the reference use.
 No kernel is launched here."""
 import ctypes as C

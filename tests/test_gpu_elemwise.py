@@ -474,6 +474,11 @@ def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band, panel):
         k2(gpuarray.array(a, context=ctx).T, gpuarray.array(b, context=ctx),
            gpuarray.array(c, context=ctx), out)
         assert np.array_equal(np.asarray(out), a.T + b * c), (ny, nx)
+        # an operand that is constant along both axes
+        s11 = rng.standard_normal((1, 1)).astype(np.float32)
+        k2(gpuarray.array(a, context=ctx).T, gpuarray.array(s11, context=ctx),
+           gpuarray.array(c, context=ctx), out)
+        assert np.array_equal(np.asarray(out), a.T + s11 * c), (ny, nx)
         # two transposed inputs
         a2 = rng.standard_normal((nx, ny)).astype(np.float32)
         k2(gpuarray.array(a, context=ctx).T, gpuarray.array(a2, context=ctx).T,
