@@ -85,7 +85,10 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
  * short-row kernel in bits 8..15 (0 means 1); outer reduced coordinates the
  * row kernel handles side by side in bits 16..23 (0 means 1); bit 24: rows
  * read from the 16-byte boundary below their start, both ends masked; bit 25:
- * also the kernel that stages short contiguous rows in LDS. */
+ * also the kernel that stages short contiguous rows in LDS; bit 26: the column
+ * kernel of min / max scans in rising index order; bit 27: the kernel for rows
+ * that one pass of a wavefront covers in place of the general row kernel
+ * (64 lanes per output only). */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

@@ -47,6 +47,7 @@ def main():
             raise SystemExit("%s: does not compile for gfx950:\n%s" % (label, (log.value or b"").decode()))
 
     GA_FLOAT, GA_HALF, GA_INT, GA_LONG, GA_UBYTE, GA_BOOL, GA_DOUBLE = 11, 23, 5, 7, 2, 0, 12
+    WROWS = 1 << 27      # the wave-per-row kernel in place of the general row kernel
     args = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"b", GA_FLOAT, 2),
                              ElemwiseArg(b"c", GA_FLOAT, 4))
     check("elemwise flat", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 0, 0, 0, 0))
@@ -79,19 +80,25 @@ def main():
                 d0 = GA_BOOL
             check("reduction op=%d src=%d" % (op, src), gen_r(op, src, d0, GA_LONG, 256, 4, 4))
             n += 1
-    check("reduction wave-per-row", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4))
+    check("reduction 64 lanes per output, general row kernel", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4))
+    check("reduction wave-per-row", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | WROWS))
     check("reduction bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1))
+    check("reduction bytes, wave-per-row", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1 | WROWS))
     # element step 2 inside a load (a [::2] view): 8 used of 16 fetched bytes
-    check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1))
+    check("reduction stepped bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1 | WROWS))
     check("reduction stepped halves", gen_r(0, GA_HALF, GA_FLOAT, GA_LONG, 256, 4 | (2 << 8), 1))
-    check("reduction short rows in batches of 4", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1 | (4 << 8)))
+    check("reduction short rows in batches of 4", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 1 | (4 << 8) | WROWS))
     for lanes in (1, 2, 8, 16, 32):
         check("reduction %d lanes per row" % lanes,
-              gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64 | (lanes << 16), 4, 2 | (2 << 8)))
+              gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64 | (lanes << 16), 4, 2 | (2 << 8) | WROWS))
     for cv, src in ((4, GA_FLOAT), (2, GA_DOUBLE), (8, GA_UBYTE)):
         check("reduction %d outputs per lane" % cv,
               gen_r(8 if src != GA_UBYTE else 0, src, src if src != GA_UBYTE else GA_LONG, GA_LONG,
                     256, 1 | (cv << 16), 4))
+    for op, src in ((8, GA_FLOAT), (4, GA_HALF), (6, GA_INT)):
+        check("column min / max in rising index order, op %d type %d" % (op, src),
+              gen_r(op, src, src, GA_LONG, 256, 1 | (4 << 16), 4 | (1 << 26)))
+        n += 1
     for op, cv in ((13, 16), (12, 4), (13, 8)):
         check("column any / all over bytes, op %d, %d outputs per lane" % (op, cv),
               gen_r(op, GA_UBYTE, GA_BOOL, GA_LONG, 256, 1 | (cv << 16), 4))
@@ -112,7 +119,7 @@ def main():
     for label, spec in (("sum of unsigned bytes", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8)),
                         ("sum of signed bytes", (0, GA_BYTE, GA_LONG, GA_LONG, 256, 16, 8)),
                         ("sum of bytes, shifted rows", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8 | (1 << 24))),
-                        ("all over stepped bytes", (12, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 4))):
+                        ("all over stepped bytes", (12, GA_UBYTE, GA_BOOL, GA_LONG, 64, 8 | (2 << 8), 4 | WROWS))):
         check("reduction four bytes per operation: " + label, gen_r(*spec))
         n += 1
     check("reduction scalar loads", gen_r(8, GA_DOUBLE, GA_DOUBLE, GA_LONG, 64, 1, 8))
@@ -124,7 +131,7 @@ def main():
                               (14, b"a + b", b"0", GA_DOUBLE), (13, None, None, GA_FLOAT),
                               (14, b"max(a, b)", b"-INFINITY", GA_HALF)]:
         d0 = GA_BOOL if op == 13 else acc
-        for G, V, U, mask in [(256, 4, 4, 0b11), (64, 4, 2, 0b01), (256, 1, 4, 0b11)]:
+        for G, V, U, mask in [(256, 4, 4, 0b11), (64, 4, 2, 0b01), (64, 4, 2 | WROWS, 0b01), (256, 1, 4, 0b11)]:
             check("map-reduce op=%d G=%d V=%d mask=%x" % (op, G, V, mask),
                   gen_m(op, red, neu, acc, b"", b"s*a*b", 3, margs, d0, G, V, U, mask))
             m += 1

@@ -249,7 +249,10 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
-  DEF("#define RD_WANT %u\n", (vs.opts >> 4) & 3u);
+  // opts bits 4, 5: redux_row / redux_col; bit 7: redux_wrows in place of redux_row; bit 8: second pass
+  DEF("#define RD_WANT %u\n", ((vs.opts & 128u) ? 4u : (vs.opts >> 4) & 1u) | ((vs.opts >> 4) & 2u) |
+                                  ((vs.opts & 256u) ? 8u : 0u));
+  DEF("#define RD_RISING %u\n", (vs.opts >> 6) & 1u);
   DEF("#define RD_CY %u\n", vs.CY ? vs.CY : 4u);
   {
     // One-byte elements under sum / any / all with an integer accumulator:
@@ -476,22 +479,22 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out, bool ma
   for (int t : flag_types) kflags |= gpuarray_type_flags(t, -1);
   const unsigned na = (unsigned)types.size();
   variant v;
-  // the text holds the kernels of one family only (opts bits 4 and 5): a
-  // variant is compiled when its first call needs it, and that call waits
+  // the text holds only the kernels its calls launch (opts bits 4, 5, 7, 8):
+  // a variant is compiled when its first call needs it, and that call waits
   const char *names[6];
   GpuKernel *ks[6];
   int nk = 0;
   auto want = [&](const char *name, GpuKernel *k) { names[nk] = name; ks[nk++] = k; };
   if (vs.opts & 8u) want("redux_srows", &v.srows);
   if (vs.opts & 16u) {
-    want("redux_row", &v.row);
-    if (vs.G == 64) want("redux_wrows", &v.wrows);
+    if (vs.opts & 128u) want("redux_wrows", &v.wrows);
+    else want("redux_row", &v.row);
   }
   if (vs.opts & 32u) {
     want("redux_col", &v.col);
-    want("redux_final_cols", &v.fin_cols);
+    if (vs.opts & 256u) want("redux_final_cols", &v.fin_cols);
   }
-  if (vs.opts & 48u) want("redux_final", &v.fin);
+  if ((vs.opts & 48u) && (vs.opts & 256u)) want("redux_final", &v.fin);
   for (int i = 0; i < nk; i++) {
     err = GpuKernel_init(ks[i], ctx, 1, strs, lens, names[i], na, types.data(), kflags, nullptr);
     if (err != GA_NO_ERROR) {
@@ -1241,6 +1244,13 @@ class reduction_call {
                        (use_row && !wrows) ? LO : 1};
     if (!use_row) vs.CY = CY;
     vs.opts |= use_row ? 16u : 32u;   // bits 4, 5: the family of kernels the text holds
+    if (wrows) vs.opts |= 128u;         // bit 7: redux_wrows, not redux_row
+    // bit 8: the kernels of the second pass too.  Beside redux_col always: they
+    // compile in a fraction of its time, and a split and an unsplit call then
+    // share one text.
+    if (p.nsplit > 1 || !use_row) vs.opts |= 256u;
+    // bit 6: redux_col meets a lane's elements in rising index order (min, max and their arg forms)
+    if (!use_row && p.rising && (gr->info.kind == K_MAX || gr->info.kind == K_MIN)) vs.opts |= 64u;
     if (srows)   // one kernel, independent of the lane geometry
       vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
     return get_variant(gr, vs, &var, !noalloc);
@@ -1370,7 +1380,8 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   std::string s;
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
-                         (((U >> 25) & 1u) ? 8u : 0u) | 48u, ES, 1,
+                         (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
+                         (((U >> 27) & 1u) ? 128u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};
@@ -1390,7 +1401,9 @@ GPUARRAY_PUBLIC char *ga_mapreduce_gen_source(int op, const char *reduce_expr, c
                     preamble, map_expr, n, args) != GA_NO_ERROR)
     return nullptr;
   std::string s;
-  variant_spec vs = {d0_tc, GA_LONG, G, V, U, 3 | 48u, 1, vecmask, 1, 64, 1, 1};
+  // bit 27 of U: redux_wrows in place of redux_row (G = 64 only)
+  variant_spec vs = {d0_tc, GA_LONG, G, V, U & 0xffu, 3 | 48u | 256u | (((U >> 27) & 1u) ? 128u : 0u),
+                     1, vecmask, 1, 64, 1, 1};
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;

@@ -25,9 +25,9 @@
  *               all; 1: unsigned bytes, 2: signed), 0: off
  *   RD_COL_FAST8  redux_col: any / all over one-byte elements work on whole words
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
- *   RD_WANT     which kernels the text holds: bit 0 the row family (redux_row,
- *               redux_wrows), bit 1 the column family (redux_col,
- *               redux_final_cols); redux_final with either
+ *   RD_WANT     which kernels the text holds: bit 0 redux_row, bit 1 redux_col,
+ *               bit 2 redux_wrows, bit 3 the second pass (redux_final, and
+ *               redux_final_cols beside redux_col)
  *   RD_TAIL     rows that are misaligned for the vector load or whose extent
  *               is not a multiple of RD_VEC (one source, contiguous rows): a
  *               row is read from the vector boundary at or below its start,
@@ -36,6 +36,7 @@
  *   RD_U        loads in flight per lane
  *   RD_LO       redux_row: outer reduced coordinates handled side by side by
  *               the RD_G lanes when the inner reduced dim is short (1: none)
+ *   RD_RISING   redux_col: the flattened index grows along the scan and fits 31 bits
  *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
  *   RD_CY       redux_col: lane rows of a group that share the reduced range
  *               (a power of two up to 16); 256 / RD_CY lanes lie along the free dim
@@ -720,7 +721,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
 #endif
 }
 
-#if RD_WANT & 1   /* the row family: redux_row, redux_wrows */
+#if RD_WANT & 1   /* redux_row */
 KERNEL void __launch_bounds__(256)
 redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
           const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
@@ -873,6 +874,9 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
   }
 }
 
+#endif   /* RD_WANT & 1 */
+
+#if RD_WANT & 4
 /* ---- redux_wrows -----------------------------------------------------------
  * Rows that one pass of a wavefront covers (at most one reduced dim, one
  * unit per row, no split).  Wavefront w owns rows [w*upb, (w+1)*upb) and takes
@@ -1006,7 +1010,7 @@ redux_wrows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 #endif
 #endif
 
-#endif   /* RD_WANT & 1 */
+#endif   /* RD_WANT & 4 */
 
 #if RD_SROWS
 /* ---- redux_srows -----------------------------------------------------------
@@ -1178,8 +1182,9 @@ static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *
 }
 
 /* Arg-min/max and floating min/max scan a lane's elements in rising order
- * with a strict compare when the plan says the index rises with them. */
-#define RD_COL_SCAN (RD_ARG && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN))
+ * with a strict compare when the plan says the index rises with them
+ * (RD_RISING: decided per variant, so that a text holds one of the two scans). */
+#define RD_COL_SCAN (RD_RISING && RD_ARG && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN))
 #if RD_KIND == RD_K_MAX
 #define RD_COL_BETTER(a, b) ((a) > (b))
 #else
@@ -1188,7 +1193,7 @@ static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *
 
 #define RD_CX (256 / RD_CY)   /* lanes along the free dim; RD_CY lane rows share the reduced range */
 
-#if RD_WANT & 2   /* the column family: redux_col, redux_final_cols */
+#if RD_WANT & 2   /* redux_col */
 /* ---- redux_col -------------------------------------------------------------
  * Lanes along the fastest free dim; a lane owns RD_CV adjacent outputs and
  * fetches them with one load (RD_CV > 1 needs that dim to be contiguous in
@@ -1239,7 +1244,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #pragma unroll
   for (int c = 0; c < RD_CV; c++) acc[c] = rd_neutral();
 #if RD_COL_SCAN
-  if (live && p.rising) {
+  if (live) {
     /* The index grows with j and j fits 31 bits: a lane meets its elements in
      * rising order, so a strict compare keeps the first of equals, and what
      * it carries per output is the value and a 32-bit j. */
@@ -1289,9 +1294,8 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
         acc[c].i = rd_col_index(p, j);
       }
     }
-  } else
-#endif
-#if RD_COL_FAST8
+  }
+#elif RD_COL_FAST8
   if (live) {
     /* any / all over bytes: bit 8c+7 of word c/4 of `seen` says that byte c of
      * some load was non-zero (any) or zero (all); exact per byte (the sum of
@@ -1441,7 +1445,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 
 #endif   /* RD_WANT & 2 */
 
-#if RD_WANT & 3
+#if RD_WANT & 8
 /* ---- redux_final ------------------------------------------------------------
  * One wavefront per output: combine its nsplit partials and write the result. */
 KERNEL void __launch_bounds__(256)
@@ -1471,9 +1475,9 @@ redux_final(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_si
   if (lane == 0) rd_write(rd_first_rule(acc, first), d0 + d0_off, d0o, d1 + d1_off, d1o);
 }
 
-#endif   /* RD_WANT & 3 */
+#endif   /* RD_WANT & 8 */
 
-#if RD_WANT & 2
+#if (RD_WANT & 10) == 10
 /* The second pass after redux_col, whose partials lie split-major
  * (slot = split * nrows + output): 64 adjacent outputs per group, lanes along
  * the outputs so that every load of a wavefront is one contiguous run, the 4
@@ -1511,4 +1515,4 @@ redux_final_cols(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const 
     rd_store(acc, srow, d0 + d0_off, d0o, d1 + d1_off, d1o, p.rtotal RD_SCALAR_ARGS);
   }
 }
-#endif   /* RD_WANT & 2 */
+#endif   /* RD_WANT & 2 and & 8 */
