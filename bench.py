@@ -46,20 +46,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # are in profiles/hbm_traffic_all_configs.md.
 MEASURED_TRAFFIC = {
     # name: (kernel text hash, HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201267465),
-    "C2_transposed_broadcast_4096": ("31f225248b8a2bfc", 134377945),
-    "C3a_sum_axis1_8192x8192": ("af7b7879c9561f8e", 268801984),
-    "C4_maxandargmax_65536x1000": ("477bbd70f85a432b", 263560871),
-    "C5_fp16_sum_axes02": ("f7232deb541fe4a7", 269751876),
-    "C5_int32_sum_axis1": ("3b05a07392f4de39", 538046866),
-    "C5_uint8_all_axis2": ("ece4e206d7eb6e28", 134404991),
-    "C5_uint8_any_axis2": ("370ef90477d5a858", 134388338),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538713359),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538715569),
-    "F4_dot_2x2^27_fused": ("7ba3850e95efbaa6", 1073828760),
-    "F4_dot_2x2^27_two_pass": ("32a750908c0f762d", 2146824867),
-    "elem_2^28": ("712fba8f0b8a6108", 3219703989),
-    "sum_2^28": ("32a750908c0f762d", 1073816083),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201245895),
+    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134364953),
+    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536632293),
+    "C3a_sum_axis1_8192x8192": ("6bb5930cba48f24d", 268796082),
+    "C4_maxandargmax_65536x1000": ("94e3fb8deeaa47db", 263492430),
+    "C5_fp16_sum_axes02": ("0710d60b15ffb320", 269738296),
+    "C5_int32_sum_axis1": ("bfbeb275e179ec1d", 538046592),
+    "C5_uint8_all_axis2": ("a288cba458843516", 134404659),
+    "C5_uint8_any_axis2": ("3ede830847c544a6", 134384141),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538650774),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538640178),
+    "F4_dot_2x2^27_fused": ("8b91825f2a4ea231", 1073828510),
+    "F4_dot_2x2^27_two_pass": ("7e9e7822441d76b0", 2146676265),
+    "elem_2^28": ("712fba8f0b8a6108", 3219404349),
+    "sum_2^28": ("7e9e7822441d76b0", 1073816039),
 }
 
 
