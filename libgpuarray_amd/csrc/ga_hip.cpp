@@ -885,7 +885,7 @@ std::string join_sources(unsigned int count, const char **strs, const size_t *le
 // program, whose parse alone takes 0.24 s per kernel; an empty kernel compiles
 // in 0.035 s this way.  Needs no device.
 struct comgr_objects {
-  amd_comgr_data_t src = {0}, hdr = {0};
+  amd_comgr_data_t src = {0}, hdr = {0}, hip_hdr = {0};
   amd_comgr_data_set_t in = {0}, rel = {0}, exe = {0};
   amd_comgr_action_info_t compile = {0}, link = {0};
   ~comgr_objects() {
@@ -896,6 +896,7 @@ struct comgr_objects {
     if (exe.handle) amd_comgr_destroy_data_set(exe);
     if (src.handle) amd_comgr_release_data(src);
     if (hdr.handle) amd_comgr_release_data(hdr);
+    if (hip_hdr.handle) amd_comgr_release_data(hip_hdr);
   }
 };
 
@@ -938,11 +939,18 @@ int rtc_compile(const std::string &src, std::vector<char> &code, std::string &lo
     COMGR_TRY(amd_comgr_create_data(AMD_COMGR_DATA_KIND_INCLUDE, &o.hdr));
     COMGR_TRY(amd_comgr_set_data(o.hdr, strlen(ga_cluda_hip_src), ga_cluda_hip_src));
     COMGR_TRY(amd_comgr_set_data_name(o.hdr, "cluda.h"));
+    // kernel text written for hipcc may include the runtime header: what it
+    // would use of it is already there
+    static const char k_empty_header[] = "#pragma once\n";
+    COMGR_TRY(amd_comgr_create_data(AMD_COMGR_DATA_KIND_INCLUDE, &o.hip_hdr));
+    COMGR_TRY(amd_comgr_set_data(o.hip_hdr, sizeof(k_empty_header) - 1, k_empty_header));
+    COMGR_TRY(amd_comgr_set_data_name(o.hip_hdr, "hip/hip_runtime.h"));
     COMGR_TRY(amd_comgr_create_data_set(&o.in));
     COMGR_TRY(amd_comgr_create_data_set(&o.rel));
     COMGR_TRY(amd_comgr_create_data_set(&o.exe));
     COMGR_TRY(amd_comgr_data_set_add(o.in, o.src));
     COMGR_TRY(amd_comgr_data_set_add(o.in, o.hdr));
+    COMGR_TRY(amd_comgr_data_set_add(o.in, o.hip_hdr));
     COMGR_TRY(amd_comgr_create_action_info(&o.compile));
     COMGR_TRY(amd_comgr_action_info_set_language(o.compile, AMD_COMGR_LANGUAGE_HIP));
     COMGR_TRY(amd_comgr_action_info_set_isa_name(o.compile, k_isa_name));

@@ -116,6 +116,53 @@ KERNEL void k(GLOBAL_MEM ga_float *x, ga_size n, GLOBAL_MEM ga_half *h, GLOBAL_M
     assert err == 0, log
 
 
+def test_device_runtime_vocabulary_without_toolchain_headers():
+    """Kernel text is compiled without the toolchain's HIP headers; the
+    library's own device runtime supplies what kernels may use: the HIP
+    spelling of kernels and indices, atomics, and the C math library with
+    <cmath>-style overloads (float stays float, integers go to double)."""
+    user = b"""#include <hip/hip_runtime.h>
+template <class A, class B> struct same_t { static const bool v = false; };
+template <class A> struct same_t<A, A> { static const bool v = true; };
+static_assert(same_t<decltype(exp(1.0f)), float>::v, "exp(float) is the float function");
+static_assert(same_t<decltype(exp(1)), double>::v, "integers promote to double");
+static_assert(same_t<decltype(pow(2.0f, 3.0f)), float>::v, "pow(float, float)");
+static_assert(same_t<decltype(pow(2.0f, 3)), float>::v, "pow(float, int)");
+static_assert(same_t<decltype(pow(2.0f, 3.0)), double>::v, "mixed arguments promote");
+static_assert(same_t<decltype(fmod(2.0f, 3)), double>::v, "mixed arguments promote");
+static_assert(same_t<decltype(fabs(-1.0f)), float>::v, "fabs(float)");
+static_assert(same_t<decltype(abs(-1.0f)), float>::v, "abs(float)");
+static_assert(same_t<decltype(abs(-1LL)), long long>::v, "abs(long long)");
+static_assert(same_t<decltype(min(1u, 2u)), unsigned>::v, "min(unsigned, unsigned)");
+extern "C" __global__ void __launch_bounds__(256) k(float *x, double *d, int *cnt, unsigned long long *big, int n) {
+  __shared__ float tile[256];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  tile[threadIdx.x] = i < n ? x[i] : 0.0f;
+  __syncthreads();
+  if (i >= n) return;
+  float v = tile[threadIdx.x ^ 1];
+  v = expf(v) + logf(v) + log2(v) + log10(v) + log1p(v) + expm1(v) + exp2(v) + exp10(v);
+  v += sin(v) + cos(v) + tan(v) + asin(v) + acos(v) + atan(v) + atan2(v, 2.0f) + sinh(v) + cosh(v) + tanh(v);
+  v += asinh(v) + acosh(v) + atanh(v) + sqrt(v) + rsqrt(v) + cbrt(v) + hypot(v, 1.0f) + pow(v, 1.5f);
+  v += floor(v) + ceil(v) + trunc(v) + round(v) + rint(v) + nearbyint(v) + fmod(v, 3.0f) + remainder(v, 3.0f);
+  v += fmin(v, 1.0f) + fmax(v, 1.0f) + fdim(v, 1.0f) + copysign(v, -1.0f) + fma(v, v, v) + ldexp(v, 2);
+  v += erf(v) + erfc(v) + lgamma(v) + tgamma(v) + nextafter(v, 0.0f) + logb(v) + (float)ilogb(v);
+  float ip, sn, cs; int e, q;
+  v += modf(v, &ip) + ip + frexp(v, &e) + (float)e + remquo(v, 3.0f, &q) + (float)q;
+  sincos(v, &sn, &cs);
+  v += sn + cs + (isnan(v) || isinf(v) || !isfinite(v) || signbit(v) ? 1.0f : 0.0f);
+  v += (float)(lrint(v) + llrint(v) + lround(v) + llround(v));
+  d[i] = exp((double)v) + pow((double)v, 2) + sqrt(i) + erf((double)v) + fmod((double)v, 2.0) + fabs((double)v);
+  x[i] = v + (float)min(i, n) + (float)max(i, 3) + (float)abs(i - 7) + (float)(__popc(i) + __clz(i) + __ffs(i));
+  atomicAdd(cnt, 1); atomicAdd(x, 1.0f); atomicAdd(d, 1.0); atomicAdd(big, 1ull);
+  atomicMax(cnt, i); atomicMin(cnt, i); atomicExch(cnt, 2); atomicCAS(cnt, 2, 3); atomicOr(cnt, 1); atomicAnd(cnt, 7);
+  if (gridDim.x > 1000000 && blockIdx.y + blockIdx.z + threadIdx.y + threadIdx.z + blockDim.y + gridDim.z > 5) __threadfence();
+}
+"""
+    err, log = compile_src(user)
+    assert err == 0, log
+
+
 def test_bad_expression_is_a_compile_error_with_a_log():
     src = take_string(gen_elemwise(b"", b"c = a +* undefined_name", 3, args_of(F32), 0, 0, 0, 0, 0))
     err, log = compile_src(src)

@@ -496,3 +496,69 @@ def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band, panel):
     o = gpuarray.empty((3, 392, 264), "float64", context=ctx)
     kd(gpuarray.array(p, context=ctx).transpose(0, 2, 1), o)
     assert np.array_equal(np.asarray(o), p.transpose(0, 2, 1) * 2.0)
+
+
+def test_math_library_functions_match_numpy(ctx):
+    """The C math library as kernels see it (the library's own device runtime
+    maps it to compiler builtins and the device library): every function on
+    float32 and float64 arrays against NumPy / SciPy, to a few units in the
+    last place; the rounding functions, fabs, fmin / fmax, copysign, sqrt and
+    fmod exactly."""
+    import scipy.special as sp
+    rng = np.random.default_rng(77)
+    n = 4096
+    pos = rng.uniform(0.05, 20.0, n)
+    sym = rng.uniform(-6.0, 6.0, n)
+    unit = rng.uniform(-0.98, 0.98, n)
+    other = rng.uniform(0.5, 4.0, n)
+    with np.errstate(all="ignore"):
+        cases = [
+            ("exp(a)", sym, None, np.exp, 4), ("exp2(a)", sym, None, np.exp2, 4),
+            ("exp10(a)", sym, None, lambda x: np.power(x.dtype.type(10), x), 4),
+            ("expm1(a)", sym, None, np.expm1, 4), ("log(a)", pos, None, np.log, 4),
+            ("log2(a)", pos, None, np.log2, 4), ("log10(a)", pos, None, np.log10, 4),
+            ("log1p(a)", pos, None, np.log1p, 4), ("sqrt(a)", pos, None, np.sqrt, 0),
+            ("rsqrt(a)", pos, None, lambda x: 1 / np.sqrt(x), 4), ("cbrt(a)", sym, None, np.cbrt, 4),
+            ("sin(a)", sym, None, np.sin, 4), ("cos(a)", sym, None, np.cos, 4),
+            ("tan(a)", unit, None, np.tan, 6), ("asin(a)", unit, None, np.arcsin, 6),
+            ("acos(a)", unit, None, np.arccos, 6), ("atan(a)", sym, None, np.arctan, 4),
+            ("sinh(a)", sym, None, np.sinh, 6), ("cosh(a)", sym, None, np.cosh, 6),
+            ("tanh(a)", sym, None, np.tanh, 6), ("asinh(a)", sym, None, np.arcsinh, 6),
+            ("acosh(a)", other + 1, None, np.arccosh, 6), ("atanh(a)", unit, None, np.arctanh, 8),
+            ("erf(a)", sym, None, sp.erf, 8), ("erfc(a)", unit, None, sp.erfc, 8),
+            ("lgamma(a)", pos, None, sp.gammaln, 64), ("tgamma(a)", other, None, sp.gamma, 16),
+            ("floor(a)", sym, None, np.floor, 0), ("ceil(a)", sym, None, np.ceil, 0),
+            ("trunc(a)", sym, None, np.trunc, 0), ("rint(a)", sym, None, np.rint, 0),
+            ("fabs(a)", sym, None, np.abs, 0),
+            ("round(a)", sym, None, lambda x: np.copysign(np.floor(np.abs(x) + x.dtype.type(0.5)), x), 0),
+            ("pow(a, b)", pos, other, np.power, 16), ("atan2(a, b)", sym, other, np.arctan2, 6),
+            ("hypot(a, b)", sym, other, np.hypot, 4), ("fmod(a, b)", sym, other, np.fmod, 0),
+            ("fmin(a, b)", sym, other, np.fmin, 0), ("fmax(a, b)", sym, other, np.fmax, 0),
+            ("copysign(a, b)", sym, -other, np.copysign, 0),
+        ]
+        for dt in ("float32", "float64"):
+            eps = np.finfo(dt).eps
+            for expr, xa, xb, fn, ulps in cases:
+                a = xa.astype(dt)
+                b = (xb if xb is not None else other).astype(dt)
+                want = fn(a, b) if xb is not None else fn(a)
+                k = ga.GpuElemwise(ctx, "c = " + expr, [arg("a", dt, read=True), arg("b", dt, read=True),
+                                                         arg("c", dt, write=True)])
+                out = gpuarray.empty((n,), dt, context=ctx)
+                k(gpuarray.array(a, context=ctx), gpuarray.array(b, context=ctx), out)
+                got = np.asarray(out)
+                assert got.dtype == np.dtype(dt)
+                if ulps == 0:
+                    assert np.array_equal(got, want.astype(dt)), (expr, dt)
+                else:
+                    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+                    tol = ulps * eps * np.maximum(np.abs(want.astype(np.float64)), 1e-30)
+                    if expr in ("sin(a)", "cos(a)", "lgamma(a)"):
+                        tol = np.maximum(tol, ulps * eps)      # results near a zero of the function
+                    assert (err <= tol).all(), (expr, dt, float((err / tol).max()))
+    # integer arguments go to the double function, as in <cmath>
+    k = ga.GpuElemwise(ctx, "c = sqrt(a) + pow(a, 2)", [arg("a", "int32", read=True), arg("c", "float64", write=True)])
+    ia = rng.integers(0, 1000, n).astype("int32")
+    out = gpuarray.empty((n,), "float64", context=ctx)
+    k(gpuarray.array(ia, context=ctx), out)
+    assert np.allclose(np.asarray(out), np.sqrt(ia.astype(np.float64)) + ia.astype(np.float64) ** 2, rtol=1e-15)
