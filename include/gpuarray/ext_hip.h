@@ -32,7 +32,9 @@ typedef int (*ga_hip_time_begin_fn)(gpucontext *ctx);
 typedef float (*ga_hip_time_end_fn)(gpucontext *ctx);
 
 /* "hip_event_record": put timing mark number `slot` on the context's stream
- * (marks are created on first use and reused); does not wait.
+ * (marks are created on first use and reused); does not wait.  The marks'
+ * events are made without the system-scope fence (hipEventDisableSystemFence):
+ * they time the stream and publish nothing to the host.
  * "hip_event_elapsed": milliseconds from mark a to mark b; waits for b;
  * < 0 on error. */
 typedef int (*ga_hip_event_record_fn)(gpucontext *ctx, unsigned int slot);

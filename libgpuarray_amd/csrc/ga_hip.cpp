@@ -1504,14 +1504,20 @@ extern "C" char *ga_mapreduce_gen_source(int op, const char *reduce_expr, const 
 namespace {
 
 // Numbered timing marks on the context's stream: record as many as wanted
-// without waiting, read the spans afterwards.
+// without waiting, read the spans afterwards.  A mark orders nothing for the
+// host (ext_event_elapsed waits for the later mark itself), so its event is
+// made without the system-scope fence a default event carries: with that
+// fence every mark has the device write its caches back for the host to see,
+// which put 1.5 us between two marks around one kernel (2^24-element flat
+// kernel: 34.96 us between default events, 33.45 between these, 32.4 for the
+// kernel's own dispatch).  GPUARRAY_MARK_EVENT_FLAGS overrides the flags.
 int ext_event_record(gpucontext *c, unsigned int slot) {
   hip_context *ctx = HC(c);
   int err;
   if ((err = enter(ctx)) != GA_NO_ERROR) return err;
   while (ctx->evpool.size() <= slot) {
     hipEvent_t e = nullptr;
-    HIP_TRY(ctx, hipEventCreate(&e));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&e, (unsigned)env_ul("GPUARRAY_MARK_EVENT_FLAGS", hipEventDisableSystemFence)));
     ctx->evpool.push_back(e);
   }
   HIP_TRY(ctx, hipEventRecord(ctx->evpool[slot], ctx->stream));

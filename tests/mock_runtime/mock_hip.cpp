@@ -35,6 +35,7 @@ hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { *s = (hipStream_
 hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
 hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 hipError_t hipEventCreate(hipEvent_t *e) { mock_allocating_calls++; *e = (hipEvent_t)0x20; return hipSuccess; }
+hipError_t hipEventCreateWithFlags(hipEvent_t *e, unsigned) { mock_allocating_calls++; *e = (hipEvent_t)0x20; return hipSuccess; }
 hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
 hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
 hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
