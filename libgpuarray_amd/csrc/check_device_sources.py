@@ -139,7 +139,8 @@ def main():
     t = 0
     for chunks, a_tc, v_tc, i_tc, tnd in [(1, GA_FLOAT, GA_FLOAT, GA_LONG, 1), (0, GA_FLOAT, GA_FLOAT, GA_INT, 1),
                                           (0, GA_DOUBLE, GA_FLOAT, GA_UBYTE, 3), (0, GA_HALF, GA_HALF, GA_LONG, 2),
-                                          (0, GA_BOOL, GA_BOOL, GA_LONG, 1)]:
+                                          (0, GA_BOOL, GA_BOOL, GA_LONG, 1), (2, GA_FLOAT, GA_FLOAT, GA_LONG, 1),
+                                          (2, GA_FLOAT, GA_FLOAT, GA_UBYTE, 1)]:
         check("take1 chunks=%d types=%d,%d,%d nd=%d" % (chunks, a_tc, v_tc, i_tc, tnd),
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1

@@ -156,3 +156,28 @@ def test_large_gather_roundtrip(ctx):
     back = t.take1(gpuarray.array(inv, context=ctx))
     assert np.array_equal(np.asarray(back).view(np.uint32), v.view(np.uint32))
     assert np.array_equal(np.asarray(t[:64]).view(np.uint32), v[perm[:64]].view(np.uint32))
+
+
+@pytest.mark.parametrize("width", [4, 12, 32, 100, 256, 512, 516])
+def test_short_dense_rows(ctx, oracle, width):
+    """Rows of at most 128 sixteen-byte chunks take their own kernel (a lane
+    moves one chunk of four rows): widths around its limits, row counts that
+    leave groups partly empty, negative indices, and rows with a bad index
+    left untouched."""
+    rng = np.random.default_rng(width)
+    for rows, n in ((1000, 1), (37, 5), (300, 1027), (5000, 4099)):
+        v = rng.integers(0, 1 << 30, size=(rows, width), dtype=np.int32)
+        idx = rng.integers(-rows, rows, size=n)
+        g = gpuarray.array(v, context=ctx)
+        got = np.asarray(g.take1(gpuarray.array(idx, context=ctx)))
+        want, err = oracle.take1(v, idx)
+        assert err == 0 and np.array_equal(got, want), (rows, n)
+    bad = idx.copy()
+    bad[[0, n // 2, n - 1]] = [rows, -rows - 1, rows + 7]
+    out = gpuarray.array(np.full((n, width), -7, dtype=np.int32), context=ctx)
+    gi = gpuarray.array(bad, context=ctx)
+    assert _lib.lib.GpuArray_take1(out._ptr(), g._ptr(), gi._ptr(), 0) == _lib.GA_NO_ERROR
+    want, err = oracle.take1(v, bad, out=np.full((n, width), -7, dtype=np.int32))
+    assert err == -1 and np.array_equal(np.asarray(out), want)
+    with pytest.raises(IndexError):                 # the flag the unchecked call left
+        g.take1(gpuarray.array(np.array([0]), context=ctx))
