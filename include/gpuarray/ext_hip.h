@@ -73,7 +73,9 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * 4 adjacent chunks per lane, 7 as 4 with every array in neither mask taken
  * as constant along x (one load for a lane's four elements), 8 as 4 with
  * every read-only array outside the LDS mask taken as constant along y (one
- * load for a lane's four rows). */
+ * load for a lane's four rows), 9 the flat kernel with the arrays in tmask
+ * (read-only, broadcast against the dense ones) read through the coordinates
+ * of the flat index in nd = 2 or 3 dims. */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
                                            unsigned int n, void *args, int flags,
                                            int strided, unsigned int nd, int idx64,

@@ -66,6 +66,10 @@ def main():
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 8, 2, 0, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 plain, operand constant along x",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 7, 2, 0, 0b100 << 16))
+    check("elemwise flat, one operand read through the flat index's coordinates, 2 dims",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 2, 0, 0b010))
+    check("elemwise flat, two operands read through the flat index's coordinates, 3 dims",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 3, 0, 0b011))
     check("elemwise flat, 2 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 5, 0, 0, 0))
     check("elemwise flat, 4 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 6, 0, 0, 0))
     hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
@@ -145,7 +149,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "17 elementwise)" % (n + 20, m, t))
+          "19 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

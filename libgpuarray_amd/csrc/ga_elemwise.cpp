@@ -29,6 +29,7 @@
 #include "private.hpp"
 
 #include <algorithm>
+#include <array>
 #include <map>
 #include <string>
 #include <vector>
@@ -97,6 +98,9 @@ struct _GpuElemwise {
   GpuKernel k_flat = {nullptr, nullptr};
   // the flat kernel with 2 or 4 adjacent chunks per lane, built on first use
   std::map<unsigned, GpuKernel> k_flat_tiled;
+  // the flat kernel with some read-only operands addressed through the
+  // coordinates of the flat index (broadcast operands), by (mask, dims)
+  std::map<unsigned, GpuKernel> k_flat_periodic;
   bool flat_forced = false;   // the environment fixed the flat kernel's shape
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
@@ -149,10 +153,53 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 //   kilobyte) before the first use.  The elements before the first chunk and
 //   after the last one, and the whole range when ga_vec == 0, run one element
 //   per lane.
-std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned unroll = 0, int tiled = -1) {
+//
+// pmask != 0 (bit k: array k): those read-only arrays are not walked as one
+// dense run but addressed through the coordinates of the flat index in an
+// iteration space of pnd (2 or 3) dims, (d0,) d1, d2: element i of the run is
+// (c0, c1, c2) = (i / (d1 d2), i / d2 % d1, i % d2) and the operand's element
+// is ps0 c0 + ps1 c1 + ps2 c2 bytes in.  That is how operands broadcast
+// against dense arrays are read (a bias row, a per-row or per-channel factor)
+// whatever the extents are: the dense arrays keep their 16-byte chunks.  The
+// two divisions are multiplications by 2^k / d rounded up (n < 2^31), once
+// per chunk; a lane steps the coordinates through its chunk's elements.
+// Extra parameters, after ga_vec: d1, d2, the two multipliers and shifts,
+// then ps0, ps1, ps2 per such array.
+std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned unroll = 0, int tiled = -1,
+                     unsigned pmask = 0, unsigned pnd = 2) {
   std::string s;
   const unsigned V = ge->vec, U = unroll ? unroll : ge->unroll;
   const bool tile = tiled < 0 ? ge->tile : tiled != 0;
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto is_p = [&](const ge_arg &a) {
+    const size_t j = (size_t)(&a - ge->args.data());
+    return aidx[j] >= 0 && ((pmask >> aidx[j]) & 1u);
+  };
+  // lvalue of a periodic operand's element at coordinates named c0/c1/c2
+  auto p_elem = [&](const ge_arg &a, const char *c0, const char *c1, const char *c2) {
+    std::string e;
+    appendf(e, "*(GLOBAL_MEM const %s *)((GLOBAL_MEM const char *)%s_p + (ga_ssize)%s * %s_ps0 + "
+               "(ga_ssize)%s * %s_ps1 + (ga_ssize)%s * %s_ps2)",
+            ctype(a.typecode), a.name.c_str(), c0, a.name.c_str(), c1, a.name.c_str(), c2, a.name.c_str());
+    return e;
+  };
+  // coordinates of flat index `idx` into ga_p0, ga_p1, ga_p2
+  auto p_coords = [&](const char *idx) {
+    std::string e;
+    appendf(e, "ga_uint ga_p0 = 0, ga_p1, ga_p2;\n{ const ga_uint ga_fi = (ga_uint)(%s);\n"
+               "const ga_uint ga_q = (ga_uint)(((ga_ulong)ga_fi * ga_m2) >> ga_k2);\n"
+               "ga_p2 = ga_fi - ga_q * ga_d2;\n", idx);
+    if (pnd == 3)
+      e += "ga_p0 = (ga_uint)(((ga_ulong)ga_q * ga_m1) >> ga_k1);\nga_p1 = ga_q - ga_p0 * ga_d1;\n}\n";
+    else
+      e += "ga_p1 = ga_q;\n}\n";
+    return e;
+  };
   emit_header(ge, s);
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size n";
   ktypes.push_back(GA_SIZE);
@@ -167,8 +214,21 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
       ktypes.push_back(a.typecode);
     }
   }
-  s += ", const ga_uint ga_vec) {\n";
+  s += ", const ga_uint ga_vec";
   ktypes.push_back(GA_UINT);
+  if (pmask) {
+    s += ", const ga_uint ga_d1, const ga_uint ga_d2, const ga_ulong ga_m1, const ga_uint ga_k1, "
+         "const ga_ulong ga_m2, const ga_uint ga_k2";
+    for (int t : {GA_UINT, GA_UINT, GA_ULONG, GA_UINT, GA_ULONG, GA_UINT}) ktypes.push_back(t);
+    for (const ge_arg &a : ge->args)
+      if (is_p(a)) {
+        appendf(s, ", const ga_ssize %s_ps0, const ga_ssize %s_ps1, const ga_ssize %s_ps2",
+                a.name.c_str(), a.name.c_str(), a.name.c_str());
+        for (int q = 0; q < 3; q++) ktypes.push_back(GA_SSIZE);
+      }
+  }
+  s += ") {\n";
+  if (pmask) s += "(void)ga_d1; (void)ga_m1; (void)ga_k1;\n";
   for (const ge_arg &a : ge->args)
     if (a.is_array())
       appendf(s, "%s_p = (GLOBAL_MEM %s *)((GLOBAL_MEM char *)%s_p + %s_offset);\n",
@@ -181,7 +241,7 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     // and bit 8 + k says that array k does not: it is then moved element by element
     s += "if (ga_vec) {\nconst ga_size ga_head = (ga_vec & 0xffu) - 1u;\nconst ga_uint ga_mis = ga_vec >> 8;\n";
     for (const ge_arg &a : ge->args)
-      if (a.is_array()) appendf(s, "%s_p += ga_head;\n", a.name.c_str());
+      if (a.is_array() && !is_p(a)) appendf(s, "%s_p += ga_head;\n", a.name.c_str());
     appendf(s, "const ga_size ga_nchunks = (n - ga_head) / %uu;\n", V);
     if (tile) {
       appendf(s, "const ga_size ga_ustep = 256;\n"
@@ -199,11 +259,24 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     }
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
     s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
+    if (pmask) {
+      // the coordinates of the chunk's first element, then stepped through the chunk
+      char idx[64];
+      snprintf(idx, sizeof(idx), "ga_head + ga_c * %uu", V);
+      s += "{\n" + p_coords(idx);
+      appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
+      for (const ge_arg &a : ge->args)
+        if (is_p(a))
+          appendf(s, "%s_u[ga_u].e[ga_v] = %s;\n", a.name.c_str(), p_elem(a, "ga_p0", "ga_p1", "ga_p2").c_str());
+      s += "if (++ga_p2 == ga_d2) { ga_p2 = 0; ";
+      s += pnd == 3 ? "if (++ga_p1 == ga_d1) { ga_p1 = 0; ga_p0++; } }\n" : "ga_p1++; }\n";
+      s += "}\n}\n";
+    }
     unsigned ak = 0;
     for (const ge_arg &a : ge->args) {
       if (!a.is_array()) continue;
       const unsigned bit = ak++;
-      if (!a.reads()) continue;
+      if (!a.reads() || is_p(a)) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
       appendf(s, "if (ga_mis & %uu) {\n#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) "
                  "%s_u[ga_u].e[ga_v] = %s_p[ga_c * %uu + ga_v];\n} else {\n",
@@ -248,13 +321,14 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     s += "}\n}\n";
     s += "}\n";
     for (const ge_arg &a : ge->args)
-      if (a.is_array()) appendf(s, "%s_p -= ga_head;\n", a.name.c_str());
+      if (a.is_array() && !is_p(a)) appendf(s, "%s_p -= ga_head;\n", a.name.c_str());
     appendf(s, "ga_done = ga_nchunks * %uu;\n", V);
     // the elements before the first chunk and after the last one
     s += "const ga_size ga_rest = n - ga_done;\nfor (ga_size ga_t = ga_gtid; ga_t < ga_rest; ga_t += ga_nthr) {\n"
          "const ga_size i = ga_t < ga_head ? ga_t : ga_t + ga_done;\n";
+    if (pmask) s += p_coords("i");
     for (const ge_arg &a : ge->args)
-      if (a.is_array()) emit_load(ge, s, a, a.name + "_p[i]");
+      if (a.is_array()) emit_load(ge, s, a, is_p(a) ? p_elem(a, "ga_p0", "ga_p1", "ga_p2") : a.name + "_p[i]");
     s += ge->expr;
     s += ";\n";
     for (const ge_arg &a : ge->args)
@@ -262,8 +336,9 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     s += "}\nreturn;\n}\n";
   }
   s += "for (ga_size i = ga_gtid; i < n; i += ga_nthr) {\n";
+  if (pmask) s += p_coords("i");
   for (const ge_arg &a : ge->args)
-    if (a.is_array()) emit_load(ge, s, a, a.name + "_p[i]");
+    if (a.is_array()) emit_load(ge, s, a, is_p(a) ? p_elem(a, "ga_p0", "ga_p1", "ga_p2") : a.name + "_p[i]");
   s += ge->expr;
   s += ";\n";
   for (const ge_arg &a : ge->args)
@@ -929,16 +1004,33 @@ int check_flat(GpuElemwise *ge, void **args, size_t *n_out, bool *flat) {
   return GA_NO_ERROR;
 }
 
+// Operands of a flat call that are addressed through the coordinates of the
+// flat index (see gen_flat): which arrays, the iteration space, the
+// multipliers that stand in for the divisions, byte strides per array.
+struct flat_periodic {
+  unsigned pmask = 0, pnd = 2;
+  unsigned d1 = 1, d2 = 1, k1 = 0, k2 = 0;
+  uint64_t m1 = 0, m2 = 0;
+  std::vector<std::array<ssize_t, 3>> ps;   // indexed by array
+};
+
 // Launch the flat kernel over n elements; offs[k] is the byte offset of
 // array k's first element in its buffer.
-int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
+int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
+              const flat_periodic *pi = nullptr) {
   unsigned l = 0;
   int err;
   unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u, head = ~0u;
   std::vector<unsigned> heads;
+  const unsigned pmask = pi ? pi->pmask : 0u;
   for (size_t i = 0; i < ge->args.size(); i++) {
     if (!ge->args[i].is_array()) continue;
     GpuArray *a = (GpuArray *)args[i];
+    if ((pmask >> heads.size()) & 1u) {   // not walked in chunks: no say in the alignment
+      heads.push_back(~0u);
+      l++;
+      continue;
+    }
     // Elements from this array's start to its next chunk boundary.  The
     // first written array (else the first array) sets the head of the
     // vector path; an array with another count is moved element by element.
@@ -952,7 +1044,7 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   if (n < (size_t)head + ge->vec || heads.size() > 24) vec_ok = 0;
   unsigned int vec_arg = vec_ok ? 1u + head : 0u;
   for (size_t q = 0; vec_ok && q < heads.size(); q++)
-    if (heads[q] != head) vec_arg |= 1u << (8 + q);
+    if (heads[q] != head && heads[q] != ~0u) vec_arg |= 1u << (8 + q);
   if (!env_ul("GPUARRAY_ELEMWISE_MIXED_ALIGN", 1) && (vec_arg >> 8)) vec_arg = 0;
   if (vec_arg == 0) vec_ok = 0;
 
@@ -975,7 +1067,7 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
   // below (2^21: 5.8 / 6.4 / 7.8) and above (3 * 2^22: 25.0 / 26.3 / 26.9,
   // 2^24 32.6 / 34.1 / 35.3, 2^28 496 / 509 / 531) one chunk per lane is best.
   unsigned tiled_u = 0;
-  if (vec_ok && !ge->flat_forced && !ge->tile) {
+  if (vec_ok && !ge->flat_forced && !ge->tile && pi == nullptr) {
     // whole chunks only: the extra unit that covers head and tail does not add a group's worth of work
     const size_t g1 = (units - 1 + GE_LANES - 1) / GE_LANES, fill = ncu * 8;
     if (g1 > fill && g1 <= 2 * fill) tiled_u = 2;
@@ -990,6 +1082,18 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
       GpuKernel nk = {nullptr, nullptr};
       if ((err = build_kernel(ge, &nk, src, ktypes)) != GA_NO_ERROR) return err;
       it = ge->k_flat_tiled.emplace(tiled_u, nk).first;
+    }
+    k = &it->second;
+  }
+  if (pi != nullptr) {
+    const unsigned key = (pi->pmask << 2) | pi->pnd;
+    auto it = ge->k_flat_periodic.find(key);
+    if (it == ge->k_flat_periodic.end()) {
+      std::vector<int> ktypes;
+      std::string src = gen_flat(ge, ktypes, 0, -1, pi->pmask, pi->pnd);
+      GpuKernel nk = {nullptr, nullptr};
+      if ((err = build_kernel(ge, &nk, src, ktypes)) != GA_NO_ERROR) return err;
+      it = ge->k_flat_periodic.emplace(key, nk).first;
     }
     k = &it->second;
   }
@@ -1010,6 +1114,18 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs) {
     }
   }
   if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
+  if (pi != nullptr) {
+    GpuKernel_setarg(k, p++, (void *)&pi->d1);
+    GpuKernel_setarg(k, p++, (void *)&pi->d2);
+    GpuKernel_setarg(k, p++, (void *)&pi->m1);
+    GpuKernel_setarg(k, p++, (void *)&pi->k1);
+    GpuKernel_setarg(k, p++, (void *)&pi->m2);
+    GpuKernel_setarg(k, p++, (void *)&pi->k2);
+    for (size_t q = 0; q < pi->ps.size(); q++)
+      if ((pi->pmask >> q) & 1u)
+        for (int j = 0; j < 3; j++)
+          if ((err = GpuKernel_setarg(k, p++, (void *)&pi->ps[q][j])) != GA_NO_ERROR) return err;
+  }
   size_t per_group = GE_LANES * (size_t)((vec_ok && tile) ? unroll : 1);
   size_t want = (units + per_group - 1) / per_group;
   size_t gs = want < 1 ? 1 : (want > cap ? cap : want);
@@ -1091,6 +1207,10 @@ class strided_call {
     find_transposed_operands();
     choose_offset_width();
     choose_vector_access();
+    {
+      flat_periodic pi;
+      if (dense_with_broadcast_operands(pi)) return call_flat(ge, args, n, offs.data(), &pi);
+    }
     int err;
     if ((err = choose_grid()) != GA_NO_ERROR) return err;
     if ((err = get_kernel()) != GA_NO_ERROR) return err;
@@ -1172,6 +1292,67 @@ class strided_call {
     for (unsigned k = 0; k < na && unit; k++)
       unit = dims[0] == 1 || strs[k][0] == (ssize_t)elsz[k];
     return unit;
+  }
+
+  // Dense arrays (one run in C order over the collapsed dims) combined with
+  // read-only operands that are broadcast along at least one dim: the flat
+  // kernel walks the dense arrays in 16-byte chunks whatever the extents are
+  // and reads the broadcast operands through the coordinates of the flat
+  // index.  Taken when the four-per-lane strided kernel cannot be (an inner
+  // extent that is not a multiple of 4, rows off a 16-byte boundary), where
+  // the other choice is one element per lane and one row per lane group.
+  // Measured on MI355X, kernel time, floats: (2^24, 3) + (1, 3) 161 -> 60 us,
+  // (65536, 1001) + (1, 1001) 125 -> 88, (2^22, 17) + (1, 17) 307 -> 90,
+  // (2^22, 10) * (2^22, 1) 159 -> 51, (2^20, 3, 5) + (1, 3, 1) 55 -> 21.
+  // Where the four-per-lane kernel can be taken it stays, except when every
+  // broadcast operand is constant along the inner dim and a dense array is
+  // read: (8192, 8192) * (8192, 1) 86 -> 80 us, (4096, 10, 4096) * (1, 10, 1)
+  // 220 -> 201, (64, 3, 512, 512) - (1, 3, 1, 1) 65 -> 61; with an operand
+  // that varies along the inner dim the strided kernel is the faster one
+  // ((8192, 8192) + (1, 8192) 87 against 92 us, channels last 79 against 94),
+  // and so it is when nothing dense is read (outer product 49 against 79).
+  bool dense_with_broadcast_operands(flat_periodic &pi) const {
+    const unsigned long mode = env_ul("GPUARRAY_ELEMWISE_PERIODIC", 1);
+    if (mode == 0 || tmask != 0) return false;
+    bool inner_constant = true, dense_read = false;
+    if ((nd != 2 && nd != 3) || n >= ((size_t)1 << 31) || na > 24) return false;
+    pi.ps.assign(na, std::array<ssize_t, 3>{{0, 0, 0}});
+    unsigned l = 0;
+    for (size_t i = 0; i < ge->args.size(); i++) {
+      if (!ge->args[i].is_array()) continue;
+      const unsigned k = l++;
+      bool dense = true;
+      size_t run = elsz[k];
+      for (unsigned j = nd; j-- > 0;) {
+        if (strs[k][j] != (ssize_t)run) dense = false;
+        run *= dims[j];
+      }
+      if (dense) {
+        dense_read = dense_read || ge->args[i].reads();
+        continue;
+      }
+      bool has_zero = false;
+      for (unsigned j = 0; j < nd; j++) has_zero = has_zero || strs[k][j] == 0;
+      const ssize_t sx = strs[k][nd - 1];
+      if (ge->args[i].writes() || !has_zero || (sx != 0 && sx != (ssize_t)elsz[k])) return false;
+      inner_constant = inner_constant && sx == 0;
+      pi.pmask |= 1u << k;
+      for (unsigned j = 0; j < nd; j++) pi.ps[k][3 - nd + j] = strs[k][j];
+    }
+    if (pi.pmask == 0) return false;
+    if (vec4 && mode != 2 && !(inner_constant && dense_read)) return false;
+    pi.pnd = nd;
+    auto magic = [](unsigned d, uint64_t &m, unsigned &k) {
+      unsigned c = 0;
+      while (((uint64_t)1 << c) < d) c++;
+      k = 31 + c;                                   // exact for dividends below 2^31
+      m = (((uint64_t)1 << k) + d - 1) / d;
+    };
+    pi.d2 = (unsigned)dims[nd - 1];
+    pi.d1 = (unsigned)dims[nd - 2];
+    magic(pi.d2, pi.m2, pi.k2);
+    magic(pi.d1, pi.m1, pi.k1);
+    return true;
   }
 
   void find_transposed_operands() {
@@ -1444,6 +1625,8 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // chunks per lane; 7 as 4, every array in neither mask taken as constant along x;
   // 8 as 4, every array that is not staged through LDS taken as constant along y
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
+  // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
+  if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
@@ -1484,6 +1667,7 @@ void GpuElemwise_free(GpuElemwise *ge) {
   if (ge == nullptr) return;
   if (ge->k_flat.k != nullptr || ge->k_flat.args != nullptr) GpuKernel_clear(&ge->k_flat);
   for (auto &kv : ge->k_flat_tiled) GpuKernel_clear(&kv.second);
+  for (auto &kv : ge->k_flat_periodic) GpuKernel_clear(&kv.second);
   for (auto &kv : ge->k_strided) GpuKernel_clear(&kv.second);
   delete ge;
 }

@@ -562,3 +562,53 @@ def test_math_library_functions_match_numpy(ctx):
     out = gpuarray.empty((n,), "float64", context=ctx)
     k(gpuarray.array(ia, context=ctx), out)
     assert np.allclose(np.asarray(out), np.sqrt(ia.astype(np.float64)) + ia.astype(np.float64) ** 2, rtol=1e-15)
+
+
+@pytest.mark.parametrize("mode", ["1", "2", "0"])
+def test_dense_arrays_with_broadcast_operands(ctx, oracle, monkeypatch, mode):
+    """Dense arrays combined with operands broadcast along some dims take the
+    flat kernel, which reads the broadcast operands through the coordinates of
+    the flat index (mode 1: where four elements per lane are not possible;
+    2: always; 0: never): two and three collapsed dims, extents that are not
+    multiples of 4, a misaligned first element, a strided column, several
+    broadcast operands, mixed types, 8- and 1-byte elements; bit for bit
+    against NumPy."""
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_PERIODIC", mode)
+    rng = np.random.default_rng(91)
+    f32 = "float32"
+    k3 = ga.GpuElemwise(ctx, "o = a * b + c", [arg("a", f32, read=True), arg("b", f32, read=True),
+                                                arg("c", f32, read=True), arg("o", f32, write=True)])
+    def run(k, ins, shape, dt=f32):
+        out = gpuarray.empty(shape, dt, context=ctx)
+        k(*ins, out, broadcast=True)
+        return np.asarray(out)
+    for R, Cn in ((1000, 3), (517, 10), (300, 1001), (64, 17), (5, 1), (1, 7), (4099, 5)):
+        a = rng.standard_normal((R, Cn)).astype(f32)
+        row = rng.standard_normal((1, Cn)).astype(f32)
+        col = rng.standard_normal((R, 1)).astype(f32)
+        g = lambda x: gpuarray.array(x, context=ctx)
+        assert np.array_equal(run(k3, [g(a), g(row), g(col)], (R, Cn)), a * row + col), (R, Cn)
+        assert np.array_equal(run(k3, [g(row), g(a), g(a)], (R, Cn)), row * a + a), (R, Cn)
+        # the dense operand starts off a 16-byte boundary; the column is a strided view
+        wide = rng.standard_normal((R + 1, Cn)).astype(f32)
+        mat = rng.standard_normal((R, 6)).astype(f32)
+        gw, gm = g(wide), g(mat)
+        got = run(k3, [gw[1:], g(row), gm[:, 2:3]], (R, Cn))
+        assert np.array_equal(got, wide[1:] * row + mat[:, 2:3]), (R, Cn)
+    # three dims: per-channel operands, and one that varies along two dims
+    for shape in ((7, 3, 5), (33, 10, 257), (2, 5, 4099), (129, 3, 1)):
+        a = rng.standard_normal(shape).astype(f32)
+        ch = rng.standard_normal((1, shape[1], 1)).astype(f32)
+        nb = rng.standard_normal((shape[0], 1, shape[2])).astype(f32)
+        g = lambda x: gpuarray.array(x, context=ctx)
+        assert np.array_equal(run(k3, [g(a), g(ch), g(nb)], shape), a * ch + nb), shape
+        assert np.array_equal(run(k3, [g(a), g(ch), g(ch)], shape), a * ch + ch), shape
+    # other element sizes and mixed types
+    kd = ga.GpuElemwise(ctx, "o = a + b", [arg("a", "float64", read=True), arg("b", f32, read=True),
+                                            arg("o", "float64", write=True)])
+    a = rng.standard_normal((257, 9)); b = rng.standard_normal((1, 9)).astype(f32)
+    assert np.array_equal(run(kd, [gpuarray.array(a, context=ctx), gpuarray.array(b, context=ctx)], (257, 9), "float64"), a + b)
+    kb = ga.GpuElemwise(ctx, "o = a ^ b", [arg("a", "uint8", read=True), arg("b", "uint8", read=True),
+                                            arg("o", "uint8", write=True)])
+    a = rng.integers(0, 256, (301, 37), dtype=np.uint8); b = rng.integers(0, 256, (301, 1), dtype=np.uint8)
+    assert np.array_equal(run(kb, [gpuarray.array(a, context=ctx), gpuarray.array(b, context=ctx)], (301, 37), "uint8"), a ^ b)
