@@ -845,3 +845,55 @@ def test_stepped_eight_byte_rows_are_planned(ctx):
         assert np.asarray(i).dtype == np.int64
     g, _ = to_gpu_view(np.zeros((64, 4096), np.int64)[:, ::4], ctx)
     assert np.asarray(R.sum(g, axis=1)).shape == (64,)
+
+
+@pytest.mark.parametrize("fold", ["1", "0"])
+def test_leading_dims_with_short_kept_rows_are_folded(ctx, monkeypatch, fold):
+    """Reducing the leading dims of a dense array whose kept rows are short or
+    off a 16-byte boundary goes through folded rows (every m rows taken as one,
+    then the m copies of each output combined): every operation that may be
+    regrouped, integer and floating types, one and two leading dims, row
+    counts with and without a usable divisor, a strided destination; against
+    NumPy, and with folding switched off."""
+    monkeypatch.setenv("GPUARRAY_REDUX_FOLD", fold)
+    rng = np.random.default_rng(71)
+    for shape, axes in (((1 << 20, 10), (0,)), ((1 << 21, 3), (0,)), ((16384, 1001), (0,)),
+                        ((1024, 1024, 4), (0, 1)), ((1048573, 5), (0,)), ((3 * (1 << 18), 6, 2), (0,)),
+                        ((1 << 22, 1), (0,))):
+        for dt in ("float32", "int32", "int8", "float16", "uint8"):
+            if np.prod(shape) * np.dtype(dt).itemsize < (4 << 20):
+                continue
+            host = rng.integers(-3 if np.dtype(dt).kind in "if" else 0, 4, size=shape).astype(dt)
+            g = gpuarray.array(host, context=ctx)
+            kept = tuple(d for i, d in enumerate(shape) if i not in axes)
+            got = np.asarray(R.sum(g, axis=axes, dtype="int64" if np.dtype(dt).kind in "iu" else "float32"))
+            assert got.shape == kept
+            assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64).astype(got.dtype)), (shape, dt, "sum")
+            for name, npf in (("all", np.all), ("any", np.any)):
+                got = np.asarray(R._reduce_named(g, name, np.dtype("bool"), axis=axes))
+                assert np.array_equal(got, npf(host, axis=axes)), (shape, dt, name)
+            if np.dtype(dt).kind in "iu":
+                for name, npf in (("max", np.max), ("min", np.min)):
+                    assert np.array_equal(np.asarray(getattr(R, name)(g, axis=axes)), npf(host, axis=axes)), (shape, dt, name)
+                for name, npf in (("and", np.bitwise_and), ("or", np.bitwise_or), ("xor", np.bitwise_xor)):
+                    got = np.asarray(R._reduce_named(g, name, np.dtype(dt), axis=axes))
+                    assert np.array_equal(got, npf.reduce(host, axis=axes)), (shape, dt, name)
+            else:
+                # arg-reductions and floating min / max keep the order of the scan: not folded, still right
+                val, idx = R.maxandargmax(g, axis=axes)
+                moved = host.reshape(-1, int(np.prod(kept)))
+                assert np.array_equal(np.asarray(val).ravel(), moved.max(axis=0))
+                assert np.array_equal(np.asarray(idx).ravel(), moved.argmax(axis=0))
+    # products (of +-1, so that nothing overflows), float sums to tolerance, a strided destination
+    host = rng.choice(np.array([1.0, -1.0], dtype=np.float32), size=(1 << 20, 6))
+    g = gpuarray.array(host, context=ctx)
+    got = np.asarray(R._reduce_named(g, "prod", np.dtype("float32"), axis=(0,)))
+    assert np.array_equal(got, np.prod(host.astype(np.float64), axis=0).astype(np.float32))
+    host = rng.standard_normal((1 << 20, 10)).astype(np.float32) + np.float32(0.5)
+    g = gpuarray.array(host, context=ctx)
+    wide = gpuarray.zeros((10, 3), "float32", context=ctx)
+    o = ga.GpuReduction(ctx, "sum", "float32")
+    o(g, [0], d0=wide[:, 1])
+    x64 = host.astype(np.float64)
+    assert_sum_close(np.asarray(wide)[:, 1], x64.sum(axis=0), np.abs(x64).sum(axis=0))
+    assert not np.asarray(wide)[:, [0, 2]].any()
