@@ -857,9 +857,10 @@ def test_leading_dims_with_short_kept_rows_are_folded(ctx, monkeypatch, fold):
     NumPy, and with folding switched off."""
     monkeypatch.setenv("GPUARRAY_REDUX_FOLD", fold)
     rng = np.random.default_rng(71)
-    for shape, axes in (((1 << 20, 10), (0,)), ((1 << 21, 3), (0,)), ((16384, 1001), (0,)),
-                        ((1024, 1024, 4), (0, 1)), ((1048573, 5), (0,)), ((3 * (1 << 18), 6, 2), (0,)),
-                        ((1 << 22, 1), (0,))):
+    cases = (((1 << 20, 10), (0,)), ((1 << 21, 3), (0,)), ((16384, 1001), (0,)),
+             ((1024, 1024, 4), (0, 1)), ((1048573, 5), (0,)), ((3 * (1 << 18), 6, 2), (0,)),
+             ((1 << 22, 1), (0,)))
+    for shape, axes in cases if fold == "1" else cases[:2]:
         for dt in ("float32", "int32", "int8", "float16", "uint8"):
             if np.prod(shape) * np.dtype(dt).itemsize < (4 << 20):
                 continue
