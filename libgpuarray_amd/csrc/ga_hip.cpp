@@ -1629,14 +1629,24 @@ void *ga_hip_static_scratch(gpucontext *c, const char **why) {
   return ctx->static_scratch;
 }
 
+// Is the context's stream recording a graph?  Work recorded now runs again at
+// every replay, on the addresses it was recorded with.
+bool ga_hip_capturing(gpucontext *c) {
+  hip_context *ctx = HC(c);
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return cap != hipStreamCaptureStatusNone;
+}
+
 gpudata *ga_hip_redux_counters(gpucontext *c) {
   hip_context *ctx = HC(c);
   if (ctx->redux_counters != nullptr) return ctx->redux_counters;
   // Not while the stream records a graph: the memset that zeroes the counters
   // would be recorded instead of run.  The caller then takes two launches.
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
-  else if (cap != hipStreamCaptureStatusNone) return nullptr;
+  if (ga_hip_capturing(c)) return nullptr;
   gpudata *b = hip_alloc(c, ga_hip_redux_counters_max * sizeof(uint32_t), nullptr, BUF_INTERNAL);
   if (b == nullptr) return nullptr;
   if (hip_memset(b, 0, 0) != GA_NO_ERROR) {

@@ -634,8 +634,8 @@ class reduction_call {
  public:
   reduction_call(GpuReduction *gr_, GpuArray *d0_, GpuArray *d1_, unsigned nd_, const size_t *dims_,
                  const std::vector<src_view> &srcs_, const std::vector<void *> &scalars_,
-                 unsigned reduxLen_, const int *reduxList_, bool noalloc_ = false)
-      : noalloc(noalloc_), gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
+                 unsigned reduxLen_, const int *reduxList_, bool noalloc_ = false, size_t scratch_skip_ = 0)
+      : noalloc(noalloc_), scratch_skip(scratch_skip_), gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
         dims(dims_), srcs(srcs_), scalars(scalars_), reduxLen(reduxLen_), reduxList(reduxList_),
         kind(info.kind), minmax(kind == K_MIN || kind == K_MAX),
         logical(kind == K_ALL || kind == K_ANY),
@@ -667,6 +667,9 @@ class reduction_call {
   // true: partials go to the device's static scratch array, kernels must be
   // loaded already, and nothing on the way allocates device memory
   const bool noalloc;
+  // bytes at the start of the context's scratch buffer that belong to the
+  // caller (fold_rows keeps its folded partial results there)
+  const size_t scratch_skip;
   GpuReduction *gr;
   gpucontext *ctx;
   const op_info &info;
@@ -1277,7 +1280,7 @@ class reduction_call {
                           "this device when the context was made (%s)", why);
       scratch = reinterpret_cast<gpudata *>(&static_view);
     } else {
-      scratch = ga_hip_scratch(ctx, 16);
+      scratch = ga_hip_scratch(ctx, scratch_skip + 16);
     }
     size_t pi_off = 0;
     // A split reduction of moderate size ends in the launch that started it:
@@ -1313,7 +1316,7 @@ class reduction_call {
                             "results that take %zu bytes; the static scratch array holds %zu",
                             slots, need, (size_t)ga_static_scratch_bytes);
       } else {
-        scratch = ga_hip_scratch(ctx, need);
+        scratch = ga_hip_scratch(ctx, scratch_skip + need);
       }
     }
     if (scratch == nullptr) return ctx->err->code;
@@ -1327,7 +1330,8 @@ class reduction_call {
     // The two scratch views are passed as (buffer) arguments; the index part
     // starts pi_off bytes in, which the kernels receive through a second
     // gpudata wrapping the same memory.
-    struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + pi_off, ctx};
+    struct { void *devptr; gpucontext *ctx; } pv_view = {(char *)scratch->devptr + scratch_skip, ctx};
+    struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + scratch_skip + pi_off, ctx};
     std::vector<void *> args;
     for (unsigned q = 0; q < K; q++) {
       s_off[q] = srcs[q].a->offset;
@@ -1338,7 +1342,7 @@ class reduction_call {
     args.push_back(&d0_off);
     args.push_back(d1b);
     args.push_back(&d1_off);
-    args.push_back(scratch);
+    args.push_back(&pv_view);
     args.push_back(&pi_view);
     args.push_back(done);
     args.push_back(planbuf.data());
@@ -1359,8 +1363,8 @@ class reduction_call {
 
 int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
                   const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
-                  unsigned reduxLen, const int *reduxList, bool noalloc = false) {
-  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList, noalloc).run();
+                  unsigned reduxLen, const int *reduxList, bool noalloc = false, size_t scratch_skip = 0) {
+  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList, noalloc, scratch_skip).run();
 }
 
 }  // namespace
@@ -1511,9 +1515,17 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
     if (err != GA_NO_ERROR) return err;
     gr->fold_tc = tmp_tc;
   }
-  GpuArray tmp;
+  // The folded partial results take the start of the context's scratch
+  // buffer (which is never handed to anybody else, also not after it has been
+  // outgrown: a graph that recorded these launches may run them again); the
+  // two calls below put their own partials behind them.
   const size_t tmp_len = m * F;
-  int err = GpuArray_empty(&tmp, ctx, tmp_tc, 1, &tmp_len, GA_C_ORDER);
+  const size_t skip = (tmp_len * gpuarray_get_elsize(tmp_tc) + 255) & ~(size_t)255;
+  gpudata *scr = ga_hip_scratch(ctx, skip + 16);
+  if (scr == nullptr) return ctx->err->code;
+  GpuArray tmp;
+  const ssize_t tmp_stride = (ssize_t)gpuarray_get_elsize(tmp_tc);
+  int err = GpuArray_fromdata(&tmp, scr, 0, tmp_tc, 1, &tmp_len, &tmp_stride, 1);
   if (err != GA_NO_ERROR) return err;
   {
     // first call: (R / m, m F) over axis 0 into tmp
@@ -1522,7 +1534,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
     srcs[0].a = s0;
     srcs[0].strides = {(ssize_t)(m * rowb), (ssize_t)es};
     const int axis0 = 0;
-    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, srcs, {}, 1, &axis0);
+    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, srcs, {}, 1, &axis0, false, skip);
   }
   if (err == GA_NO_ERROR) {
     // second call: tmp as (m, kept dims...) over axis 0 into d0
@@ -1541,9 +1553,9 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
     srcs[0].a = &tmp;
     srcs[0].strides = str2;
     const int axis0 = 0;
-    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), srcs, {}, 1, &axis0);
+    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), srcs, {}, 1, &axis0, false, skip);
   }
-  GpuArray_clear(&tmp);   // the stream orders the buffer's next use after these launches
+  GpuArray_clear(&tmp);
   if (err == GA_NO_ERROR) *done = true;
   return err;
 }

@@ -36,8 +36,13 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
     a = gpuarray.zeros((n,), f32, context=ctx)
     b = gpuarray.zeros((n,), f32, context=ctx)
 
+    fold_rows = 1 << 19               # sum over a batch of rows of 10 floats: folded rows, three launches
+    wide = gpuarray.zeros((fold_rows, 10), f32, context=ctx)
+    wide_fill = ga.GpuElemwise(ctx, "w = a * 3.0f", [arg("a", f32, read=True), arg("w", f32, write=True)])
+
     def outputs():
         return dict(c=gpuarray.zeros((n,), f32, context=ctx), d=gpuarray.zeros((n,), f32, context=ctx),
+                    ws=gpuarray.zeros((10,), f32, context=ctx),
                     rs=gpuarray.zeros((rows,), f32, context=ctx), tot=gpuarray.zeros((), f32, context=ctx),
                     cs=gpuarray.zeros((cols,), f32, context=ctx),
                     mv=gpuarray.zeros((rows,), f32, context=ctx),
@@ -51,6 +56,9 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
         rsum(o["d"], [0], d0=o["tot"])          # split over many groups: two kernels, scratch partials
         rsum(d2, [0], d0=o["cs"])               # column kernel
         rmax(d2, [1], d0=o["mv"], d1=o["mi"])
+        flat = wide.reshape((fold_rows * 10,))
+        wide_fill(a[:n // 4], flat[:n // 4])        # part of `wide` follows the inputs
+        rsum(wide, [0], d0=o["ws"])
 
     eager, replayed = outputs(), outputs()
     issue(eager)                                 # compiles everything, sizes the scratch buffer
