@@ -92,7 +92,8 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
  * also the kernel that stages short contiguous rows in LDS; bit 26: the column
  * kernel of min / max scans in rising index order; bit 27: the kernel for rows
  * that one pass of a wavefront covers in place of the general row kernel
- * (64 lanes per output only). */
+ * (64 lanes per output only); bit 28: every count of the call is below 2^31
+ * (32-bit divisions). */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

@@ -86,6 +86,10 @@ def main():
             n += 1
     check("reduction 64 lanes per output, general row kernel", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4))
     check("reduction wave-per-row", gen_r(8, GA_FLOAT, GA_FLOAT, GA_LONG, 64, 4, 4 | WROWS))
+    for op, src in ((0, GA_FLOAT), (8, GA_FLOAT), (13, GA_UBYTE)):
+        check("reduction with 32-bit divisions, op %d" % op,
+              gen_r(op, src, GA_BOOL if op == 13 else GA_FLOAT, GA_LONG, 256, 4 if src == GA_FLOAT else 16, 4 | (1 << 28)))
+        n += 1
     check("reduction bytes", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1))
     check("reduction bytes, wave-per-row", gen_r(13, GA_UBYTE, GA_BOOL, GA_LONG, 64, 16, 1 | WROWS))
     # element step 2 inside a load (a [::2] view): 8 used of 16 fetched bytes

@@ -256,6 +256,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_WANT %u\n", ((vs.opts & 128u) ? 4u : (vs.opts >> 4) & 1u) | ((vs.opts >> 4) & 2u) |
                                   ((vs.opts & 256u) ? 8u : 0u));
   DEF("#define RD_RISING %u\n", (vs.opts >> 6) & 1u);
+  DEF("#define RD_IDX32 %u\n", (vs.opts >> 9) & 1u);
   DEF("#define RD_CY %u\n", vs.CY ? vs.CY : 4u);
   {
     // One-byte elements under sum / any / all with an integer accumulator:
@@ -1251,6 +1252,9 @@ class reduction_call {
     if (!use_row) vs.CY = CY;
     vs.opts |= use_row ? 16u : 32u;   // bits 4, 5: the family of kernels the text holds
     if (wrows) vs.opts |= 128u;         // bit 7: redux_wrows, not redux_row
+    // bit 9: the outputs, the reduced range and their product (the elements
+    // visited) all count below 2^31, so the kernels' divisions are 32-bit ones
+    if ((double)nrows * (double)rtotal < 2147483648.0 && groups < 0x7fffffffull) vs.opts |= 512u;
     // bit 8: the kernels of the second pass too.  Beside redux_col always: they
     // compile in a fraction of its time, and a split and an unsplit call then
     // share one text.
@@ -1258,7 +1262,7 @@ class reduction_call {
     // bit 6: redux_col meets a lane's elements in rising index order (min, max and their arg forms)
     if (!use_row && p.rising && (gr->info.kind == K_MAX || gr->info.kind == K_MIN)) vs.opts |= 64u;
     if (srows)   // one kernel, independent of the lane geometry
-      vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u, 1, 1, 1, 64, 1, 1};
+      vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u | (vs.opts & 512u), 1, 1, 1, 64, 1, 1};
     return get_variant(gr, vs, &var, !noalloc);
   }
 
@@ -1388,7 +1392,7 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
                          (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
-                         (((U >> 27) & 1u) ? 128u : 0u) | 48u | 256u, ES, 1,
+                         (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};

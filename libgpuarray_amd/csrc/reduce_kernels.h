@@ -36,6 +36,7 @@
  *   RD_U        loads in flight per lane
  *   RD_LO       redux_row: outer reduced coordinates handled side by side by
  *               the RD_G lanes when the inner reduced dim is short (1: none)
+ *   RD_IDX32    every count and flat index of the call is below 2^31: 32-bit divisions
  *   RD_RISING   redux_col: the flattened index grows along the scan and fits 31 bits
  *   RD_CV       redux_col: adjacent outputs per lane, fetched with one load
  *   RD_CY       redux_col: lane rows of a group that share the reduced range
@@ -281,6 +282,22 @@ static __device__ inline rd_acc rd_block_reduce(rd_acc a, rd_acc *lds) {
 
 /* Offsets of output `row` (flat index over the free dims, slowest first):
  * one per source, and the two destinations'. */
+/* q = a / b and the remainder, for non-negative a and positive b.  RD_IDX32:
+ * the plan says that every count and flat index of this call is below 2^31,
+ * and the division is a 32-bit one (the 64-bit one is a long sequence of
+ * instructions, slow to run and slower to compile). */
+static __device__ inline ga_long rd_divmod(ga_long a, ga_long b, ga_long *rem) {
+#if RD_IDX32
+  const ga_uint q = (ga_uint)a / (ga_uint)b;
+  *rem = (ga_long)((ga_uint)a - q * (ga_uint)b);
+  return (ga_long)q;
+#else
+  const ga_long q = a / b;
+  *rem = a - q * b;
+  return q;
+#endif
+}
+
 static __device__ inline void rd_row_offsets(const rd_plan &p, ga_long row, ga_long *so,
                                              ga_long *d0o, ga_long *d1o) {
   ga_long a = 0, b = 0;
@@ -288,7 +305,7 @@ static __device__ inline void rd_row_offsets(const rd_plan &p, ga_long row, ga_l
   for (int k = 0; k < RD_NSRC; k++) so[k] = 0;
   for (int d = p.nf - 1; d >= 0; d--) {
     ga_long c;
-    if (d > 0) { c = row % p.fdim[d]; row = row / p.fdim[d]; } else { c = row; }
+    if (d > 0) { row = rd_divmod(row, p.fdim[d], &c); } else { c = row; }
 #pragma unroll
     for (int k = 0; k < RD_NSRC; k++) so[k] += c * p.fsstr[k][d];
     a += c * p.fd0str[d];
@@ -306,7 +323,7 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
   for (int k = 0; k < RD_NSRC; k++) rb[k] = 0;
   for (int d = ri - 1; d >= 0; d--) {
     ga_long c;
-    if (d > 0) { c = ro % p.rdim[d]; ro = ro / p.rdim[d]; } else { c = ro; }
+    if (d > 0) { ro = rd_divmod(ro, p.rdim[d], &c); } else { c = ro; }
 #pragma unroll
     for (int k = 0; k < RD_NSRC; k++) rb[k] += c * p.rsstr[k][d];
     x += c * p.rmul[d];
@@ -796,7 +813,7 @@ redux_row(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__re
   /* unit -> (outer reduced coordinate ro, segment k of the inner dim): one
    * division for the first unit, then counted up */
   ga_long ro = 0, k = u0;
-  if (p.nr > 1) { ro = u0 / p.nseg; k = u0 - ro * p.nseg; }
+  if (p.nr > 1) { ro = rd_divmod(u0, p.nseg, &k); }
   ga_long rb[RD_NSRC], ib = 0;
   rd_outer_offsets(p, ri, ro, rb, &ib);
 
@@ -1156,7 +1173,7 @@ static __device__ inline void rd_col_at(const rd_plan &p, const ga_long j, ga_lo
     ga_long r = j;
     for (int d = p.nr - 1; d >= 0; d--) {
       ga_long c = r;
-      if (d > 0) { c = r % p.rdim[d]; r = r / p.rdim[d]; }
+      if (d > 0) { r = rd_divmod(r, p.rdim[d], &c); }
 #pragma unroll
       for (int k = 0; k < RD_NSRC; k++) off[k] += c * p.rsstr[k][d];
       *ix += c * p.rmul[d];
@@ -1206,8 +1223,8 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   const unsigned tx = LID_0 % RD_CX, ty = LID_0 / RD_CX;
   const ga_long split = GID_0 % (unsigned)p.nsplit;
   ga_long t = GID_0 / (unsigned)p.nsplit;
-  const ga_long bx = t % p.gx;
-  const ga_long fo = t / p.gx;   /* flat index over the outer free dims */
+  ga_long bx;
+  const ga_long fo = rd_divmod(t, p.gx, &bx);   /* flat index over the outer free dims */
   const int fi_d = p.nf - 1;
   const ga_long fin = p.fdim[fi_d];
   const ga_long fi = (bx * RD_CX + tx) * RD_CV;   /* first of the lane's outputs */
@@ -1221,7 +1238,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     ga_long r = fo;
     for (int d = fi_d - 1; d >= 0; d--) {
       ga_long c;
-      if (d > 0) { c = r % p.fdim[d]; r = r / p.fdim[d]; } else { c = r; }
+      if (d > 0) { r = rd_divmod(r, p.fdim[d], &c); } else { c = r; }
 #pragma unroll
       for (int k = 0; k < RD_NSRC; k++) so[k] += c * p.fsstr[k][d];
       d0o += c * p.fd0str[d];
