@@ -46,21 +46,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # are in profiles/hbm_traffic_all_configs.md.
 MEASURED_TRAFFIC = {
     # name: (kernel text hash, HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201245895),
-    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134364953),
-    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536632293),
-    "C3a_sum_axis1_8192x8192": ("6bb5930cba48f24d", 268796082),
-    "C4_maxandargmax_65536x1000": ("94e3fb8deeaa47db", 263492430),
-    "C5_fp16_sum_axes02": ("0710d60b15ffb320", 269738296),
-    "C5_int32_sum_axis1": ("bfbeb275e179ec1d", 538046592),
-    "C5_uint8_all_axis2": ("a288cba458843516", 134404659),
-    "C5_uint8_any_axis2": ("3ede830847c544a6", 134384141),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538650774),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538640178),
-    "F4_dot_2x2^27_fused": ("8b91825f2a4ea231", 1073828510),
-    "F4_dot_2x2^27_two_pass": ("7e9e7822441d76b0", 2146676265),
-    "elem_2^28": ("712fba8f0b8a6108", 3219404349),
-    "sum_2^28": ("7e9e7822441d76b0", 1073816039),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201251110),
+    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134363678),
+    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536644579),
+    "C3a_sum_axis1_8192x8192": ("a5ed42207d09d01e", 268766185),
+    "C4_maxandargmax_65536x1000": ("7a3409deee50fa50", 263754775),
+    "C5_fp16_sum_axes02": ("25b4f4278187082d", 269706572),
+    "C5_int32_sum_axis1": ("b06b2c493c4c87a8", 538005680),
+    "C5_uint8_all_axis2": ("75698d744ba82b47", 134384160),
+    "C5_uint8_any_axis2": ("ec550fc5d781c6f7", 134384192),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538644422),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538647224),
+    "F4_dot_2x2^27_fused": ("3489eab9d9d27d06", 1073819599),
+    "F4_dot_2x2^27_two_pass": ("3ea0e6c2086cb335", 2146698200),
+    "elem_2^28": ("712fba8f0b8a6108", 3219474723),
+    "sum_2^28": ("3ea0e6c2086cb335", 1073801732),
 }
 
 
