@@ -382,17 +382,19 @@ def test_sum_is_reproducible_run_to_run(ctx):
 # ---- the benchmark's shapes at full size -----------------------------------------------------
 
 def _record(name, **figures):
-    """Achieved errors of the benchmark's float sums, kept for the design notes
-    (gpurun_out/ comes back from a GPU run)."""
+    """Achieved errors of the benchmark's float sums: printed, and appended to
+    float_sum_errors.jsonl in the directory GPUARRAY_TEST_RECORD_DIR names, if
+    it names one."""
     import json
     import os
-    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
-    try:
-        os.makedirs(out, exist_ok=True)
-        with open(os.path.join(out, "float_sum_errors.jsonl"), "a") as f:
-            f.write(json.dumps(dict(name=name, **figures)) + "\n")
-    except OSError:
-        pass
+    out = os.environ.get("GPUARRAY_TEST_RECORD_DIR")
+    if out:
+        try:
+            os.makedirs(out, exist_ok=True)
+            with open(os.path.join(out, "float_sum_errors.jsonl"), "a") as f:
+                f.write(json.dumps(dict(name=name, **figures)) + "\n")
+        except OSError:
+            pass
     print(name, figures)
 
 
