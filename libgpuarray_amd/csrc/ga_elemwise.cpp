@@ -100,7 +100,7 @@ struct _GpuElemwise {
   std::map<unsigned, GpuKernel> k_flat_tiled;
   // the flat kernel with some read-only operands addressed through the
   // coordinates of the flat index (broadcast operands), by (mask, dims)
-  std::map<unsigned, GpuKernel> k_flat_periodic;
+  std::map<uint64_t, GpuKernel> k_flat_periodic;
   bool flat_forced = false;   // the environment fixed the flat kernel's shape
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
@@ -164,9 +164,12 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 // two divisions are multiplications by 2^k / d rounded up (n < 2^31), once
 // per chunk; a lane steps the coordinates through its chunk's elements.
 // Extra parameters, after ga_vec: d1, d2, the two multipliers and shifts,
-// then ps0, ps1, ps2 per such array.
+// then ps0, ps1, ps2 per such array.  Arrays also in pvmask have unit stride
+// along the inner dim and everything aligned to the chunk, and the caller
+// passes no head: a chunk's elements are then one chunk of the operand too,
+// fetched with one load.
 std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned unroll = 0, int tiled = -1,
-                     unsigned pmask = 0, unsigned pnd = 2) {
+                     unsigned pmask = 0, unsigned pnd = 2, unsigned pvmask = 0) {
   std::string s;
   const unsigned V = ge->vec, U = unroll ? unroll : ge->unroll;
   const bool tile = tiled < 0 ? ge->tile : tiled != 0;
@@ -179,6 +182,10 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
   auto is_p = [&](const ge_arg &a) {
     const size_t j = (size_t)(&a - ge->args.data());
     return aidx[j] >= 0 && ((pmask >> aidx[j]) & 1u);
+  };
+  auto is_pv = [&](const ge_arg &a) {
+    const size_t j = (size_t)(&a - ge->args.data());
+    return aidx[j] >= 0 && ((pmask & pvmask) >> aidx[j]) & 1u;
   };
   // lvalue of a periodic operand's element at coordinates named c0/c1/c2
   auto p_elem = [&](const ge_arg &a, const char *c0, const char *c1, const char *c2) {
@@ -264,9 +271,16 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
       char idx[64];
       snprintf(idx, sizeof(idx), "ga_head + ga_c * %uu", V);
       s += "{\n" + p_coords(idx);
+      for (const ge_arg &a : ge->args)
+        if (is_pv(a)) {
+          const size_t cb = gpuarray_get_elsize(a.typecode) * V;
+          appendf(s, "%s_u[ga_u].c = *(GLOBAL_MEM const %s *)((GLOBAL_MEM const char *)%s_p + (ga_ssize)ga_p0 * %s_ps0 + "
+                     "(ga_ssize)ga_p1 * %s_ps1 + (ga_ssize)ga_p2 * %s_ps2);\n",
+                  a.name.c_str(), chunk_type(cb), a.name.c_str(), a.name.c_str(), a.name.c_str(), a.name.c_str());
+        }
       appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
       for (const ge_arg &a : ge->args)
-        if (is_p(a))
+        if (is_p(a) && !is_pv(a))
           appendf(s, "%s_u[ga_u].e[ga_v] = %s;\n", a.name.c_str(), p_elem(a, "ga_p0", "ga_p1", "ga_p2").c_str());
       s += "if (++ga_p2 == ga_d2) { ga_p2 = 0; ";
       s += pnd == 3 ? "if (++ga_p1 == ga_d1) { ga_p1 = 0; ga_p0++; } }\n" : "ga_p1++; }\n";
@@ -1009,6 +1023,7 @@ int check_flat(GpuElemwise *ge, void **args, size_t *n_out, bool *flat) {
 // multipliers that stand in for the divisions, byte strides per array.
 struct flat_periodic {
   unsigned pmask = 0, pnd = 2;
+  unsigned pvmask = 0;   // of pmask: operands a chunk of which is one aligned load (when there is no head)
   unsigned d1 = 1, d2 = 1, k1 = 0, k2 = 0;
   uint64_t m1 = 0, m2 = 0;
   std::vector<std::array<ssize_t, 3>> ps;   // indexed by array
@@ -1086,11 +1101,12 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
     k = &it->second;
   }
   if (pi != nullptr) {
-    const unsigned key = (pi->pmask << 2) | pi->pnd;
+    const unsigned pv = (vec_ok && head == 0) ? pi->pvmask : 0u;
+    const uint64_t key = ((uint64_t)pv << 32) | (pi->pmask << 2) | pi->pnd;
     auto it = ge->k_flat_periodic.find(key);
     if (it == ge->k_flat_periodic.end()) {
       std::vector<int> ktypes;
-      std::string src = gen_flat(ge, ktypes, 0, -1, pi->pmask, pi->pnd);
+      std::string src = gen_flat(ge, ktypes, 0, -1, pi->pmask, pi->pnd, pv);
       GpuKernel nk = {nullptr, nullptr};
       if ((err = build_kernel(ge, &nk, src, ktypes)) != GA_NO_ERROR) return err;
       it = ge->k_flat_periodic.emplace(key, nk).first;
@@ -1307,14 +1323,17 @@ class strided_call {
   // Where the four-per-lane kernel can be taken it stays, except when every
   // broadcast operand is constant along the inner dim and a dense array is
   // read: (8192, 8192) * (8192, 1) 86 -> 80 us, (4096, 10, 4096) * (1, 10, 1)
-  // 220 -> 201, (64, 3, 512, 512) - (1, 3, 1, 1) 65 -> 61; with an operand
-  // that varies along the inner dim the strided kernel is the faster one
-  // ((8192, 8192) + (1, 8192) 87 against 92 us, channels last 79 against 94),
-  // and so it is when nothing dense is read (outer product 49 against 79).
+  // 220 -> 201, (64, 3, 512, 512) - (1, 3, 1, 1) 65 -> 61; an operand with
+  // unit stride along an inner extent of whole chunks is fetched a chunk per
+  // load ((8192, 8192) + (1, 8192) 89 -> 81 us).  With an operand that varies
+  // along the inner dim and cannot be fetched that way the strided kernel is
+  // the faster one (87 against 92 us, channels last 79 against 94), and so it
+  // is when nothing dense is read (outer product 49 against 79).
   bool dense_with_broadcast_operands(flat_periodic &pi) const {
     const unsigned long mode = env_ul("GPUARRAY_ELEMWISE_PERIODIC", 1);
     if (mode == 0 || tmask != 0) return false;
     bool inner_constant = true, dense_read = false;
+    const size_t V = ge->vec;
     if ((nd != 2 && nd != 3) || n >= ((size_t)1 << 31) || na > 24) return false;
     pi.ps.assign(na, std::array<ssize_t, 3>{{0, 0, 0}});
     unsigned l = 0;
@@ -1335,7 +1354,18 @@ class strided_call {
       for (unsigned j = 0; j < nd; j++) has_zero = has_zero || strs[k][j] == 0;
       const ssize_t sx = strs[k][nd - 1];
       if (ge->args[i].writes() || !has_zero || (sx != 0 && sx != (ssize_t)elsz[k])) return false;
-      inner_constant = inner_constant && sx == 0;
+      // one aligned load per chunk: unit stride along an inner extent of whole
+      // chunks, every other stride and the first element on chunk boundaries
+      bool whole_chunks = sx == (ssize_t)elsz[k] && V > 1 && dims[nd - 1] % V == 0;
+      {
+        const size_t cb = elsz[k] * V;
+        const GpuArray *v = (const GpuArray *)args[i];
+        if (((uintptr_t)v->data->devptr + offs[k]) % cb != 0) whole_chunks = false;
+        for (unsigned j = 0; j + 1 < nd; j++)
+          if (strs[k][j] % (ssize_t)cb != 0) whole_chunks = false;
+      }
+      if (whole_chunks) pi.pvmask |= 1u << k;
+      inner_constant = inner_constant && (sx == 0 || (whole_chunks && env_ul("GPUARRAY_ELEMWISE_PERIODIC_VEC", 1)));
       pi.pmask |= 1u << k;
       for (unsigned j = 0; j < nd; j++) pi.ps[k][3 - nd + j] = strs[k][j];
     }
@@ -1632,7 +1662,8 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // 8 as 4, every array that is not staged through LDS taken as constant along y
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
-  if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd).c_str());
+  // (idx64 then carries the mask of those fetched a whole chunk at a time)
+  if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu

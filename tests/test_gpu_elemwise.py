@@ -582,7 +582,7 @@ def test_dense_arrays_with_broadcast_operands(ctx, oracle, monkeypatch, mode):
         out = gpuarray.empty(shape, dt, context=ctx)
         k(*ins, out, broadcast=True)
         return np.asarray(out)
-    for R, Cn in ((1000, 3), (517, 10), (300, 1001), (64, 17), (5, 1), (1, 7), (4099, 5)):
+    for R, Cn in ((1000, 3), (517, 10), (300, 1001), (64, 17), (5, 1), (1, 7), (4099, 5), (513, 1000), (37, 64)):
         a = rng.standard_normal((R, Cn)).astype(f32)
         row = rng.standard_normal((1, Cn)).astype(f32)
         col = rng.standard_normal((R, 1)).astype(f32)
@@ -596,7 +596,7 @@ def test_dense_arrays_with_broadcast_operands(ctx, oracle, monkeypatch, mode):
         got = run(k3, [gw[1:], g(row), gm[:, 2:3]], (R, Cn))
         assert np.array_equal(got, wide[1:] * row + mat[:, 2:3]), (R, Cn)
     # three dims: per-channel operands, and one that varies along two dims
-    for shape in ((7, 3, 5), (33, 10, 257), (2, 5, 4099), (129, 3, 1)):
+    for shape in ((7, 3, 5), (33, 10, 257), (2, 5, 4099), (129, 3, 1), (9, 6, 256)):
         a = rng.standard_normal(shape).astype(f32)
         ch = rng.standard_normal((1, shape[1], 1)).astype(f32)
         nb = rng.standard_normal((shape[0], 1, shape[2])).astype(f32)
