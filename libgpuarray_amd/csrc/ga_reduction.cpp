@@ -1303,7 +1303,27 @@ class reduction_call {
     if (p.nsplit > 1 && !noalloc) {
       const size_t counters = use_row ? (size_t)nrows : groups / (size_t)p.nsplit;
       const size_t fused_max = (size_t)ncu * env_ul("GPUARRAY_REDUX_FUSED", 1);   // 0 turns it off
-      if (groups <= fused_max && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
+      // Beyond one group per compute unit the single launch pays again once a
+      // piece is long: the wait for the acknowledgement is then a small part of
+      // a group's life, and the second launch (3 to 4 us) is saved.  Measured,
+      // two launches against one: full sum of 2^24 floats (512 pieces of 128 KiB)
+      // 15.9 against 16.7 us, of 2^25 25.3 / 25.0, of 2^26 42.2 / 40.1, of 2^28
+      // 156.0 / 152.9; sum over axis 1 of (64, 2^20) 43.2 / 40.6.  The column
+      // kernel's last piece combines a tile's partials by itself, so it must
+      // not have many: over axis 0 of (4096, 16384) 44.0 / 42.0 us, of
+      // (16384, 4096) 44.3 / 43.8, of (65536, 1024) 44.0 / 51.9, of
+      // (2^20, 64) 44.3 / 73.0.
+      bool fuse = groups <= fused_max;
+      if (!fuse && fused_max > 0) {
+        const double piece_bytes = (double)nrows * (double)rtotal * (double)elsz_sum / (double)groups;
+        // (partials that carry an index cost the column kernel's last piece twice
+        // the loads: maxandargmax over axis 0 of (8192, 8192) 47.8 / 50.5)
+        const bool carries_index = info.has_d1 || (minmax && is_float_type(acc_tc));
+        fuse = use_row ? piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_PIECE", 384u << 10)
+                       : (!carries_index && p.nsplit <= (int)env_ul("GPUARRAY_REDUX_FUSED_COL_SPLITS", 16) &&
+                          piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_COL_PIECE", 128u << 10));
+      }
+      if (fuse && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
           (done = ga_hip_redux_counters(ctx)) != nullptr) {
         p.fused = 1;
         if (!use_row) p.split_major = 1;

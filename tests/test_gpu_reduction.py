@@ -740,9 +740,11 @@ def test_split_reductions_finish_in_one_launch(ctx, monkeypatch):
     cases += [((4, 1 << 20), (1,)), ((16, 1 << 18), (1,)), ((3, 5, 1 << 16), (1, 2)),     # rows in pieces
               ((4096, 256), (0,)), ((100000, 64), (0,)), ((70, 3000, 40), (1,)),          # columns in pieces
               ((20000, 1000), (0,)), ((1 << 19, 8), (0,))]
+    # long pieces: beyond one group per compute unit the single launch is taken again
+    long_pieces = [((1 << 26,), (0,)), ((64, 1 << 20), (1,)), ((2048, 32768), (0,))]
     for rep in range(2):
         for dtype in ("float32", "int32", "float64"):
-            for shape, axes in cases:
+            for shape, axes in cases + (long_pieces if rep == 0 and dtype != "float64" else []):
                 host = rng.integers(-30, 30, size=shape).astype(dtype)
                 g, _ = to_gpu_view(host, ctx)
                 if host.dtype.kind == "i":
