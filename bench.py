@@ -4,8 +4,8 @@
 One "step" is one pass of the hot path over one batch of synthetic data at the
 target shape: the fp32 elementwise c = a*b + 0.5f over 2^28 contiguous
 elements followed by the full fp32 sum of a 2^28-element array (a grid
-reduction: 512 pieces, combined by the piece that finishes last or by a second
-launch).  Inputs are resident in HBM before the timed region.
+reduction: a few hundred pieces, combined by the piece that finishes last or by
+a second launch).  Inputs are resident in HBM before the timed region.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
     python bench.py --only NAME [--steps K]     one kernel per step, for profiler runs

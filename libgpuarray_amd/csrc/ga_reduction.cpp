@@ -1032,8 +1032,25 @@ class reduction_call {
     int64_t per_cu = (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 0);
     if (per_cu == 0) {
       const int64_t inflight = (int64_t)G * U * V * ES * elsz_sum;   // bytes per group
-      per_cu = (65536 + inflight - 1) / inflight;
-      if (per_cu < 2) per_cu = 2;
+      // A kernel that does next to nothing per element - one source of floats
+      // or doubles, summed or multiplied in its own type, whole aligned loads -
+      // is best with ONE such group per unit, which also keeps it within the
+      // single launch: full fp32 sum of 2^28 153.4 -> 147.3 us (7.3 TB/s), of
+      // 2^24 16.0 -> 14.7, rows of (16, 2^22) 42.8 -> 39.6.  Everything else
+      // needs the second group to overlap its arithmetic with the loads:
+      // max of 2^26 floats 43 us with two groups against 57 with one (NaN and
+      // tie rules per element), sum of 2^27 halves 40 / 44.5 (a conversion per
+      // element), int32 into int64 39.8 / 42.7, a ragged row (masked ends)
+      // 40.2 / 48.6, the dot product of two arrays 156 / 180.
+      const int stc0 = gr->args[gr->arrays[0]].tc;
+      bool light = K == 1 && !gr->mapped && !tail && !info.has_d1 &&
+                   (info.kind == K_SUM || info.kind == K_PROD) &&
+                   (stc0 == GA_FLOAT || stc0 == GA_DOUBLE) && acc_typecode(gr, d0_tc) == stc0;
+      if (!env_ul("GPUARRAY_REDUX_LIGHT", 1)) light = false;
+      const int64_t want = (int64_t)env_ul("GPUARRAY_REDUX_INFLIGHT", light ? 32768 : 65536);
+      const int64_t least = (int64_t)env_ul("GPUARRAY_REDUX_MIN_PER_CU", light ? 1 : 2);
+      per_cu = (want + inflight - 1) / inflight;
+      if (per_cu < least) per_cu = least;
       if (per_cu > 32) per_cu = 32;
     }
     const int64_t target = ncu * per_cu;
