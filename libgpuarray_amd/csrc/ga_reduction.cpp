@@ -1231,7 +1231,16 @@ class reduction_call {
     // 16384 x 16384 54.3 -> 49.5 us, floats 65536 x 1000 48.6 -> 46.3,
     // 8192 x 8192 49.3 -> 48.1, halves 2048 x 65536 48.2 -> 46.1; two groups
     // were faster still for 2- and 4-byte elements and slower for bytes (59.5).
-    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? 3 : 8);
+    // Float sums and products (next to nothing per element), two against three:
+    // over axis 0 of (1024, 16384) 17.0 -> 14.8 us, (65536, 1024) 44.6 -> 43.6,
+    // (2^20, 64) 45.1 -> 44.0, (16384, 4096) 45.4 -> 45.0; maximum of the same
+    // 49.0 -> 51.2, sum of bytes 47.7 -> 58.0, of halves 46.0 -> 49.4.
+    const int stc0 = gr->args[gr->arrays[0]].tc;
+    const bool light = K == 1 && !gr->mapped && !info.has_d1 && (info.kind == K_SUM || info.kind == K_PROD) &&
+                       (stc0 == GA_FLOAT || stc0 == GA_DOUBLE) && acc_typecode(gr, d0_tc) == stc0 &&
+                       env_ul("GPUARRAY_REDUX_LIGHT", 1) != 0 &&
+                       scratch_skip == 0;   // folded rows measured better with three: (2^24, 3) 38.8 against 43.4 us
+    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? (light ? 2 : 3) : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
       if (nsplit > rtotal / 64) nsplit = rtotal / 64;
