@@ -92,6 +92,7 @@ struct _GpuElemwise {
   int kflags = 0;           // GA_USE_* for the compiler
   unsigned int vec = 1;     // elements per chunk in the flat kernel
   unsigned int unroll = 1;  // chunks per lane and tile in the flat kernel
+  bool narrow_side = false; // every input, or every output, is of narrower elements than the widest
   bool tile = false;        // a group's chunks are adjacent (tile) or a grid apart
   bool nontemporal = true;  // streaming hint on the flat kernel's loads and stores
   unsigned flat_nt_mask = ~0u;   // ... per array (bit k: array k)
@@ -1081,12 +1082,24 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
   // 10.0 / 8.9 / 9.9, 3 * 2^21 13.7 / 13.7 / 12.5, 2^23 17.3 / 18.0 / 16.5;
   // below (2^21: 5.8 / 6.4 / 7.8) and above (3 * 2^22: 25.0 / 26.3 / 26.9,
   // 2^24 32.6 / 34.1 / 35.3, 2^28 496 / 509 / 531) one chunk per lane is best.
+  //
+  // Arrays of narrower elements than the widest move in chunks of fewer than
+  // 16 bytes.  Where one whole side of the kernel is narrow, two chunks per
+  // lane, 256 chunks apart, are faster at every size beyond one fill (kernel
+  // time for 2^27 elements, one chunk per lane / two / four: bytes to floats
+  // 119.9 / 100.4 / 117.9 us, two byte arrays to floats 163.9 / 127.6 / 138.4,
+  // floats to bytes 112.6 / 102.1 / 106.8, floats to halves 127.5 / 120.4 /
+  // 130.2, doubles to floats 252.0 / 241.4 / 258.4, a > b to a byte 187.5 /
+  // 181.6 / 198.0); where a wide array is read and a wide one written they
+  // are slower (float + half to float 200.5 / 212.9, halves to floats 122.0 /
+  // 124.9, two floats to a half 203.0 / 206.5).
   unsigned tiled_u = 0;
   if (vec_ok && !ge->flat_forced && !ge->tile && pi == nullptr) {
     // whole chunks only: the extra unit that covers head and tail does not add a group's worth of work
     const size_t g1 = (units - 1 + GE_LANES - 1) / GE_LANES, fill = ncu * 8;
     if (g1 > fill && g1 <= 2 * fill) tiled_u = 2;
-    else if (g1 > 2 * fill && g1 <= 4 * fill) tiled_u = 4;
+    else if (g1 > 2 * fill && g1 <= 4 * fill) tiled_u = ge->narrow_side ? 2 : 4;
+    else if (g1 > 4 * fill && ge->narrow_side) tiled_u = 2;
   }
   GpuKernel *k = &ge->k_flat;
   if (tiled_u) {
@@ -1632,6 +1645,27 @@ static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, 
   // 126 -> 182 for 2^27); fewer chunks in flight when many arrays are live at once
   ge->vec = maxel >= 16 ? 1 : (unsigned)(16 / maxel);
   ge->unroll = ge->narray <= 8 ? 2 : 1;
+  {
+    // narrow inputs: every array read has elements of a quarter of the widest
+    // or less; narrow outputs: every array written is narrower than the widest
+    // and either at most one wide array is read or they are a quarter or less
+    bool in_quarter = true, out_narrow = true, out_quarter = true, any_in = false;
+    unsigned wide_in = 0;
+    for (const ge_arg &a : ge->args) {
+      if (!a.is_array()) continue;
+      const size_t es = gpuarray_get_elsize(a.typecode);
+      if (a.reads()) {
+        any_in = true;
+        if (es * 4 > maxel) in_quarter = false;
+        if (es == maxel) wide_in++;
+      }
+      if (a.writes()) {
+        if (es >= maxel) out_narrow = false;
+        if (es * 4 > maxel) out_quarter = false;
+      }
+    }
+    ge->narrow_side = ge->narray <= 8 && ((any_in && in_quarter) || (out_narrow && (wide_in <= 1 || out_quarter)));
+  }
   ge->flat_forced = getenv("GPUARRAY_ELEMWISE_UNROLL") != nullptr || getenv("GPUARRAY_ELEMWISE_TILE") != nullptr;
   ge->unroll = (unsigned)env_ul("GPUARRAY_ELEMWISE_UNROLL", ge->unroll);
   if (ge->unroll < 1) ge->unroll = 1;

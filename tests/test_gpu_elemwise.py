@@ -349,6 +349,34 @@ def test_small_types_vectorised_flat_path(ctx):
         assert np.array_equal(np.asarray(gc), (a + b).astype(dt)), dt
 
 
+@pytest.mark.parametrize("n", [(5 << 20) + 7, (1 << 24) + 5])
+def test_flat_kernel_with_a_narrow_side_takes_two_chunks_per_lane(ctx, n):
+    # bytes to floats, floats to bytes / halves, comparisons to a byte: beyond one
+    # fill of the chip these run with two chunks per lane; offsets break the alignment
+    rng = np.random.default_rng(n)
+    f = rng.uniform(-100, 100, n + 3).astype(np.float32)
+    g = rng.uniform(-100, 100, n + 3).astype(np.float32)
+    u = rng.integers(0, 256, n + 3).astype(np.uint8)
+    cases = [("o = a * 0.5f", [("a", u)], "float32", lambda a: a.astype(np.float32) * np.float32(0.5)),
+             ("o = a + b", [("a", u), ("b", u[::-1].copy())], "float32",
+              lambda a, b: a.astype(np.float32) + b.astype(np.float32)),
+             ("o = a", [("a", f)], "float16", lambda a: a.astype(np.float16)),
+             ("o = a", [("a", np.abs(f))], "uint8", lambda a: a.astype(np.uint8)),
+             ("o = a > b", [("a", f), ("b", g)], "bool", lambda a, b: a > b),
+             ("o = a", [("a", f.astype(np.float64))], "float32", lambda a: a.astype(np.float32))]
+    for expr, ins, odt, ref in cases:
+        ge = ga.GpuElemwise(ctx, expr, [arg(nm, v.dtype.name, read=True) for nm, v in ins] +
+                            [arg("o", odt, write=True)], convert_f16=True)
+        for off_in, off_out in ((0, 0), (1, 0), (0, 3), (2, 2)):
+            gins = [gpuarray.array(v, context=ctx)[off_in:off_in + n] for _, v in ins]
+            go = gpuarray.zeros((n + 3,), odt, context=ctx)
+            ge(*gins, go[off_out:off_out + n])
+            got = np.asarray(go)
+            want = ref(*[v[off_in:off_in + n] for _, v in ins])
+            assert np.array_equal(got[off_out:off_out + n], want), (expr, odt, off_in, off_out)
+            assert not got[:off_out].any() and not got[off_out + n:].any()
+
+
 def test_inplace_and_multiple_outputs(ctx):
     rng = np.random.default_rng(10)
     x = rng.normal(size=(257, 33)).astype(np.float32)
