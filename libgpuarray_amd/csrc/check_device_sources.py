@@ -125,6 +125,13 @@ def main():
         check("reduction short rows staged in LDS, op %d type %d" % (op, src),
               gen_r(op, src, d0, GA_LONG, 64, 1, 1 | (1 << 25)))
         n += 1
+    # ops: 0 sum, 4 max, 8 maxandargmax, 6 argmax (the enum of reduction.h), 13 any
+    for op, src, d0, te in ((0, GA_FLOAT, GA_FLOAT, 3), (8, GA_FLOAT, GA_FLOAT, 5), (13, GA_UBYTE, GA_BOOL, 12),
+                            (0, GA_HALF, GA_FLOAT, 6), (4, GA_DOUBLE, GA_DOUBLE, 3), (0, GA_INT, GA_LONG, 2),
+                            (0, GA_UBYTE, GA_LONG, 30)):
+        check("reduction tiny rows in registers, op %d type %d, %d elements" % (op, src, te),
+              gen_r(op, src, d0, GA_LONG, 64, te, 1 | (1 << 29)))
+        n += 1
     GA_BYTE, GA_ULONG = 1, 8
     for label, spec in (("sum of unsigned bytes", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8)),
                         ("sum of signed bytes", (0, GA_BYTE, GA_LONG, GA_LONG, 256, 16, 8)),

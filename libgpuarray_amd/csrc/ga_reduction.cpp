@@ -123,7 +123,8 @@ struct variant {
   GpuKernel row = {nullptr, nullptr}, col = {nullptr, nullptr}, fin = {nullptr, nullptr},
             fin_cols = {nullptr, nullptr},   // second pass after redux_col
             wrows = {nullptr, nullptr},   // wrows only exists in 64-lane variants
-            srows = {nullptr, nullptr};   // the only kernel of a short-rows variant (opts bit 3)
+            srows = {nullptr, nullptr},   // the only kernel of a short-rows variant (opts bit 3)
+            trows = {nullptr, nullptr};   // the only kernel of a tiny-rows variant (opts bit 10)
 };
 
 struct dimrec {
@@ -152,7 +153,7 @@ struct _GpuReduction {
   bool mapped = false;        // an expression feeds the reduction
   int acc_tc = -1;            // mapped: accumulator (= value result) type
   std::string map_expr, preamble, reduce_expr, neutral;
-  std::map<std::array<unsigned, 13>, variant> variants;   // by the fields of a variant_spec
+  std::map<std::array<unsigned, 14>, variant> variants;   // by the fields of a variant_spec
   // the same operation on the type of folded partial results (see fold_rows), made on first use
   GpuReduction *fold_op = nullptr;
   int fold_tc = -1;
@@ -184,6 +185,7 @@ struct variant_spec {
   unsigned CV;        // redux_col: adjacent outputs per lane
   unsigned LO;        // redux_row: outer reduced coordinates side by side
   unsigned CY = 4;    // redux_col: lane rows of a group (1 to 16), 256 / CY lanes along the free dim
+  unsigned TE = 0;    // redux_trows (opts bit 10): elements of a row
 };
 
 const char *load_type_name(int tc) {
@@ -252,6 +254,15 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
+  {
+    // redux_trows: a lane's run of whole rows in whole 16-byte chunks
+    const unsigned te = vs.TE ? vs.TE : 1;
+    const unsigned rowb = te * (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc);
+    unsigned g = rowb, h = 16;
+    while (h) { const unsigned t = g % h; g = h; h = t; }
+    DEF("#define RD_TROWS %u\n#define RD_TE %u\n#define RD_TC %u\n#define RD_TR %u\n", (vs.opts >> 10) & 1u,
+        te, rowb / g, 16 / g);
+  }
   // opts bits 4, 5: redux_row / redux_col; bit 7: redux_wrows in place of redux_row; bit 8: second pass
   DEF("#define RD_WANT %u\n", ((vs.opts & 128u) ? 4u : (vs.opts >> 4) & 1u) | ((vs.opts >> 4) & 2u) |
                                   ((vs.opts & 256u) ? 8u : 0u));
@@ -446,8 +457,8 @@ size_t plan_bytes(unsigned nsrc) { return sizeof(rd_plan) + (size_t)nsrc * 2 * R
 // (building one loads a code object, and that allocates device memory).
 int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out, bool may_build = true) {
   gpucontext *ctx = gr->ctx;
-  const std::array<unsigned, 13> key = {(unsigned)vs.d0_tc, (unsigned)vs.d1_tc, vs.G, vs.V, vs.U,
-                                        vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY};
+  const std::array<unsigned, 14> key = {(unsigned)vs.d0_tc, (unsigned)vs.d1_tc, vs.G, vs.V, vs.U,
+                                        vs.opts, vs.ES, vs.vecmask, vs.RB, vs.L, vs.CV, vs.LO, vs.CY, vs.TE};
   auto it = gr->variants.find(key);
   if (it != gr->variants.end()) {
     *out = &it->second;
@@ -490,6 +501,7 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out, bool ma
   int nk = 0;
   auto want = [&](const char *name, GpuKernel *k) { names[nk] = name; ks[nk++] = k; };
   if (vs.opts & 8u) want("redux_srows", &v.srows);
+  if (vs.opts & 1024u) want("redux_trows", &v.trows);
   if (vs.opts & 16u) {
     if (vs.opts & 128u) want("redux_wrows", &v.wrows);
     else want("redux_row", &v.row);
@@ -657,6 +669,7 @@ class reduction_call {
       row_geometry();
       wrows_geometry();
       srows_geometry();
+      trows_geometry();
     } else {
       col_geometry();
     }
@@ -697,7 +710,7 @@ class reduction_call {
   int64_t rin = 1, rstr = 0, fstr = 0;   // inner reduced extent and stride, inner free stride
   int64_t rin_sz = 1;               // rin plus what a shifted row can gain
   // kernel family and lane geometry
-  bool use_row = true, wrows = false, tail = false, srows = false;
+  bool use_row = true, wrows = false, tail = false, srows = false, trows = false;
   unsigned G = 256, V = 1, U = 4, ES = 1, vecmask, RB = 1, L = 64, CV = 1, LO = 1, CY = 4;
   size_t groups = 0, lds_bytes = 0;
   variant *var = nullptr;
@@ -1159,6 +1172,58 @@ class reduction_call {
     }
   }
 
+  void trows_geometry() {
+    // Rows of at most 32 bytes that follow one another in memory, the first
+    // on a 16-byte boundary: a lane takes the least run of whole rows that is
+    // whole 16-byte chunks into registers and walks its rows there
+    // (redux_trows).  redux_wrows is bound by its instructions per row on
+    // these.  Measured on MI355X, 2^26 floats in rows of 3 / 5 / 6 / 7: sum
+    // 75.4 / 62.6 / 56.9 / 51.7 us there, 50.9 / 49.6 / 48.4 / 48.5 here,
+    // argmax 86.7 / 65.9 / 64.0 / 54.4 against 58.3 / - / 51.1 / -; 2^24 rows
+    // of 6 halves 71.5 -> 36.9 us, of 12 bytes (summed into 64-bit integers)
+    // 74.9 -> 48.5.  Rows of more than 32 bytes gain nothing (10 floats 44.9
+    // there, 47.4 here; 16 floats 45 staged in LDS, 43 here).
+    const int64_t rowb = rin * elsz[0];
+    if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] && fsstr[0] == rowb &&
+        rin >= 2 && elsz[0] <= 8 && rowb <= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MAX_BYTES", 32) &&
+        nrows >= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MIN_ROWS", 16384) && env_ul("GPUARRAY_REDUX_TROWS", 1)) {
+      const GpuArray *s0 = srcs[0].a;
+      const size_t readable = ga_hip_readable_bytes(s0->data);
+      const size_t end = ((size_t)s0->offset + (size_t)(nrows * rowb) + 15) & ~(size_t)15;
+      int64_t g = rowb, h = 16;
+      while (h) { const int64_t t = g % h; g = h; h = t; }
+      const int64_t per_lane = 16 / g, chunks = rowb / g;   // a lane's rows, in as many chunks
+      // Rows of 2, 4, 8, 16 or 32 bytes need no hand-out (one or two chunks
+      // per lane), and there redux_wrows keeps up: it stays for four- and
+      // eight-byte elements (2^26 floats in rows of 2 / 4 / 8: 55.5 / 52.2 /
+      // 49.3 us against 57.1 / 54.6 / 51.6 here) and for rows of 16 bytes
+      // (2^27 bytes, any: 21.3 against 24.7 us); one- and two-byte elements
+      // in rows of 2, 4, 8 or 32 bytes come here (2^27 bytes in rows of 2 /
+      // 4 / 32, max: 104.6 / 39.9 / 28.2 us there, 29.3 / 28.4 / 21.9 here).
+      const unsigned long direct = env_ul("GPUARRAY_REDUX_TROWS_DIRECT", 1);
+      // more than two chunks per lane are handed out through LDS, 4 KiB per chunk
+      if (((uintptr_t)s0->data->devptr + (size_t)s0->offset) % 16 == 0 && end <= readable &&
+          chunks <= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MAX_CHUNKS", 7) &&
+          (chunks > 2 || direct == 2 || (direct == 1 && elsz[0] <= 2 && rowb != 16))) {
+        trows = true;
+        srows = wrows = false;
+        lds_bytes = 0;
+        p.nsplit = 1;
+        // bit 0 / 1: the values / indices of a lane's rows lie side by side
+        // in memory and start on the boundary of one store
+        auto side_by_side = [&](const GpuArray *d, int64_t stride) {
+          if (d == nullptr) return false;
+          const int64_t es = (int64_t)gpuarray_get_elsize(d->typecode);
+          const int64_t run = std::min<int64_t>(es * per_lane, 16);
+          return stride == es && ((uintptr_t)d->data->devptr + (size_t)d->offset) % (size_t)run == 0;
+        };
+        p.upb = (side_by_side(d0, p.fd0str[0]) ? 1 : 0) | (side_by_side(d1, p.fd1str[0]) ? 2 : 0);
+        const int64_t lanes = (nrows + per_lane - 1) / per_lane;
+        groups = (size_t)((lanes + 255) / 256);
+      }
+    }
+  }
+
   void col_geometry() {
     const int64_t fin = p.fdim[p.nf - 1];
     const unsigned long cy_forced = env_ul("GPUARRAY_REDUX_COL_ROWS", 0);
@@ -1289,6 +1354,10 @@ class reduction_call {
     if (!use_row && p.rising && (gr->info.kind == K_MAX || gr->info.kind == K_MIN)) vs.opts |= 64u;
     if (srows)   // one kernel, independent of the lane geometry
       vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u | (vs.opts & 512u), 1, 1, 1, 64, 1, 1};
+    if (trows) {   // one kernel per row length
+      vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 1024u | (vs.opts & 512u), 1, 1, 1, 64, 1, 1};
+      vs.TE = (unsigned)rin;
+    }
     return get_variant(gr, vs, &var, !noalloc);
   }
 
@@ -1398,7 +1467,7 @@ class reduction_call {
     args.push_back(planbuf.data());
     for (void *sc : scalars) args.push_back(sc);
     size_t ls = 256;
-    GpuKernel *k1 = srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
+    GpuKernel *k1 = trows ? &var->trows : srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
     int err;
     if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
     if (p.nsplit > 1 && !p.fused) {
@@ -1438,10 +1507,15 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
                          (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
-                         (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) | 48u | 256u, ES, 1,
+                         (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) |
+                         (((U >> 29) & 1u) ? 1024u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};
+  if ((U >> 29) & 1u) {   // redux_trows: V is the row length
+    vs.TE = V;
+    vs.V = 1;
+  }
   const int err = variant_source(gr, vs, s, ga_global_err);
   delete gr;
   return err == GA_NO_ERROR ? strdup(s.c_str()) : nullptr;
@@ -1498,6 +1572,7 @@ void GpuReduction_free(GpuReduction *gr) {
     if (kv.second.fin_cols.k != nullptr) GpuKernel_clear(&kv.second.fin_cols);
     if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
     if (kv.second.srows.k != nullptr) GpuKernel_clear(&kv.second.srows);
+    if (kv.second.trows.k != nullptr) GpuKernel_clear(&kv.second.trows);
   }
   delete gr;
 }

@@ -1140,6 +1140,235 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 }
 #endif
 
+#if RD_TROWS
+/* ---- redux_trows -----------------------------------------------------------
+ * Rows of RD_TE elements, at most 32 bytes, one after the other in memory (one
+ * source, one reduced dim, unit stride, row pitch = row length, first row on
+ * a 16-byte boundary).  There the time goes into instructions per row, not
+ * into bytes.  A lane takes the least run of whole rows that is a whole number
+ * of 16-byte chunks - RD_TR rows in RD_TC chunks, both fixed when the kernel
+ * is built - into registers and walks its rows there: every element position
+ * is a constant, no cross-lane step, no LDS. */
+#define RD_TROW_BYTES (RD_TE * RD_ELSZ0)
+typedef ga_uint rd_tchunk_t __attribute__((ext_vector_type(4)));
+
+template <int ES> struct rd_tbits;
+template <> struct rd_tbits<1> {
+  static __device__ inline ga_ulong at(const rd_tchunk_t *c, const int b) {
+    return (c[b >> 4][(b >> 2) & 3] >> ((b & 3) * 8)) & 0xffu;
+  }
+};
+template <> struct rd_tbits<2> {
+  static __device__ inline ga_ulong at(const rd_tchunk_t *c, const int b) {
+    return (c[b >> 4][(b >> 2) & 3] >> ((b & 2) * 8)) & 0xffffu;
+  }
+};
+template <> struct rd_tbits<4> {
+  static __device__ inline ga_ulong at(const rd_tchunk_t *c, const int b) { return c[b >> 4][(b >> 2) & 3]; }
+};
+template <> struct rd_tbits<8> {
+  static __device__ inline ga_ulong at(const rd_tchunk_t *c, const int b) {
+    return (ga_ulong)c[b >> 4][(b >> 2) & 3] | ((ga_ulong)c[b >> 4][((b >> 2) & 3) + 1] << 32);
+  }
+};
+
+/* element e of the lane's registers as a one-element fetch */
+static __device__ inline rd_one rd_trow_elem(const rd_tchunk_t *c, const int e) {
+  typedef decltype(rd_one::x0) elem_t;
+  const ga_ulong bits = rd_tbits<RD_ELSZ0>::at(c, e * RD_ELSZ0);
+  rd_one o;
+  __builtin_memcpy(&o.x0, &bits, sizeof(elem_t));
+  return o;
+}
+
+/* A lane's RD_TR results side by side, for the case that they lie so in
+ * memory: up to 16 bytes go out as one store per lane; a longer run is handed
+ * back through LDS so that the wavefront's stores are 16 bytes per lane side
+ * by side again (a lane storing its own 64 bytes in four pieces would leave
+ * every store instruction with 64 pieces 64 bytes apart). */
+#if RD_HAS_D0 && RD_DST_HALF
+typedef ga_half rd_tdst_t;
+#elif RD_HAS_D0
+typedef RD_DST_T rd_tdst_t;
+#else
+typedef ga_int rd_tdst_t;
+#endif
+template <typename T> struct __attribute__((aligned(sizeof(T) * RD_TR > 16 ? 16 : sizeof(T) * RD_TR))) rd_trun {
+  T e[RD_TR];
+};
+constexpr int rd_trun0 = RD_HAS_D0 ? (int)sizeof(rd_trun<rd_tdst_t>) : 0;
+constexpr int rd_trun1 = RD_HAS_D1 ? (int)sizeof(rd_trun<RD_IDX_T>) : 0;
+constexpr int rd_tmax(const int a, const int b) { return a > b ? a : b; }
+/* 16-byte chunks of LDS per lane: the loads' hand-out and the longer runs */
+constexpr int rd_tlds = rd_tmax(RD_TC > 2 ? RD_TC : 0,
+                                rd_tmax(rd_trun0 > 16 ? rd_trun0 / 16 : 0, rd_trun1 > 16 ? rd_trun1 / 16 : 0));
+
+static __device__ inline void rd_twave_sync() {
+  /* LDS operations of one wavefront run in the order they were issued; this
+   * keeps the compiler from moving them across */
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+/* `dst`: where the wavefront's first result goes; `area`: its 64 * rd_tlds chunks of LDS */
+template <typename RUN>
+static __device__ inline void rd_twave_store(char *dst, const RUN &o, rd_tchunk_t *area, const unsigned lane) {
+  ((RUN *)area)[lane] = o;
+  rd_twave_sync();
+#pragma unroll
+  for (int k = 0; k < (int)sizeof(RUN) / 16; k++) ((rd_tchunk_t *)dst)[k * 64 + lane] = area[k * 64 + lane];
+  rd_twave_sync();
+}
+
+KERNEL void __launch_bounds__(256)
+redux_trows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
+            const rd_plan p RD_SCALAR_PARAMS) {
+  (void)part_v; (void)part_i; (void)done;
+  __shared__ rd_tchunk_t rd_tstage[256 * (rd_tlds ? rd_tlds : 1)];
+  const ga_long unit = (ga_long)GID_0 * 256 + LID_0;
+  const ga_long row0 = unit * RD_TR;
+  const ga_long rml = p.rmul[0];
+  const unsigned lane = LID_0 & 63u;
+  rd_tchunk_t *area = rd_tstage + (LID_0 - lane) * rd_tlds;   /* the wavefront's own part */
+  const char *base[RD_NSRC];
+  RD_SRC_BASES(base);
+  const rd_tchunk_t *src = (const rd_tchunk_t *)base[0];
+  /* chunks that hold part of the array: the last lanes' runs may end past it */
+  const ga_long total = (p.nrows * RD_TROW_BYTES + 15) >> 4;
+  rd_tchunk_t c[RD_TC];
+#if RD_TC > 2
+  /* A lane's chunks lie RD_TC * 16 bytes from its neighbour's: fetched by the
+   * lane itself, every load of a wavefront would touch 64 separate pieces of
+   * memory.  The wavefront fetches its RD_TC * 64 chunks side by side
+   * instead and hands them out through LDS. */
+  {
+    const ga_long cw = (unit - lane) * RD_TC;   /* the wavefront's first chunk */
+    rd_tchunk_t t[RD_TC];
+#pragma unroll
+    for (int j = 0; j < RD_TC; j++) {
+      const ga_long ci = cw + j * 64 + lane;
+      if (ci < total) t[j] = RD_LOAD(src + ci);
+      else t[j] = (rd_tchunk_t)(0u);
+    }
+#pragma unroll
+    for (int j = 0; j < RD_TC; j++) area[j * 64 + lane] = t[j];
+    rd_twave_sync();
+#pragma unroll
+    for (int j = 0; j < RD_TC; j++) c[j] = area[lane * RD_TC + j];
+    rd_twave_sync();
+  }
+#else
+#pragma unroll
+  for (int j = 0; j < RD_TC; j++) {
+    if (unit * RD_TC + j < total) c[j] = RD_LOAD(src + unit * RD_TC + j);
+    else c[j] = (rd_tchunk_t)(0u);
+  }
+#endif
+  if (row0 >= p.nrows) return;
+
+  rd_acc res[RD_TR];
+#pragma unroll
+  for (int r = 0; r < RD_TR; r++) {
+    rd_acc acc = rd_neutral();
+#if RD_ARG && (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN)
+    /* value and position inside the row while walking up the row (a strict
+     * compare keeps the first of equals); the index is formed at the end */
+    RD_ACC_T bv = rd_elem(RD_ONE_VAL(rd_trow_elem(c, r * RD_TE)), 0).v;
+    ga_int bp = 0;
+#pragma unroll
+    for (int i = 1; i < RD_TE; i++) {
+      const RD_ACC_T val = rd_elem(RD_ONE_VAL(rd_trow_elem(c, r * RD_TE + i)), 0).v;
+#if RD_KIND == RD_K_MAX
+      const bool better = val > bv;
+#else
+      const bool better = val < bv;
+#endif
+      bv = better ? val : bv;
+      bp = better ? i : bp;
+    }
+    acc.v = bv;
+    acc.i = (ga_long)bp * rml;
+#else
+#pragma unroll
+    for (int i = 0; i < RD_TE; i++)
+      acc = rd_combine(acc, rd_elem(RD_ONE_VAL(rd_trow_elem(c, r * RD_TE + i)), (ga_long)i * rml));
+#endif
+    res[r] = rd_first_rule(acc, (RD_ACC_T)RD_ONE_VAL(rd_trow_elem(c, r * RD_TE)));
+  }
+
+  /* p.upb bit 0 / 1: the values / the indices of a lane's rows lie side by
+   * side in memory, the first of them on the boundary of one store.  A lane
+   * whose run is cut short by the end of the array, and for the longer runs
+   * every lane of that last wavefront, writes row by row. */
+  const bool whole = row0 + RD_TR <= p.nrows;
+  const ga_long wrow0 = (unit - lane) * RD_TR;
+  const bool wave_whole = wrow0 + 64 * RD_TR <= p.nrows;
+  (void)wave_whole; (void)area;
+  bool v_done = !RD_HAS_D0, i_done = !RD_HAS_D1;
+#if RD_HAS_D0
+  if (p.upb & 1) {
+    rd_trun<rd_tdst_t> o;
+#pragma unroll
+    for (int r = 0; r < RD_TR; r++) {
+#if RD_DST_HALF
+      o.e[r] = ga_float2half((float)res[r].v);
+#else
+      o.e[r] = (RD_DST_T)res[r].v;
+#endif
+    }
+    if constexpr (rd_trun0 > 16) {
+      if (wave_whole) {
+        rd_twave_store(d0 + d0_off + wrow0 * (ga_long)sizeof(rd_tdst_t), o, area, lane);
+        v_done = true;
+      }
+    } else if (whole) {
+      *(rd_trun<rd_tdst_t> *)(d0 + d0_off + row0 * (ga_long)sizeof(rd_tdst_t)) = o;
+      v_done = true;
+    }
+  }
+#endif
+#if RD_HAS_D1
+  if (p.upb & 2) {
+    rd_trun<RD_IDX_T> o;
+#pragma unroll
+    for (int r = 0; r < RD_TR; r++) o.e[r] = (RD_IDX_T)res[r].i;
+    if constexpr (rd_trun1 > 16) {
+      if (wave_whole) {
+        rd_twave_store(d1 + d1_off + wrow0 * (ga_long)sizeof(RD_IDX_T), o, area, lane);
+        i_done = true;
+      }
+    } else if (whole) {
+      *(rd_trun<RD_IDX_T> *)(d1 + d1_off + row0 * (ga_long)sizeof(RD_IDX_T)) = o;
+      i_done = true;
+    }
+  }
+#endif
+  if (v_done && i_done) return;
+#pragma unroll
+  for (int r = 0; r < RD_TR; r++) {
+    const ga_long row = row0 + r;
+    if (row < p.nrows) {
+      ga_long so[RD_NSRC], d0o, d1o;
+      rd_row_offsets(p, row, so, &d0o, &d1o);
+#if RD_HAS_D0
+      if (!v_done) {
+#if RD_DST_HALF
+        *(ga_half *)(d0 + d0_off + d0o) = ga_float2half((float)res[r].v);
+#else
+        *(RD_DST_T *)(d0 + d0_off + d0o) = (RD_DST_T)res[r].v;
+#endif
+      }
+#endif
+#if RD_HAS_D1
+      if (!i_done) *(RD_IDX_T *)(d1 + d1_off + d1o) = (RD_IDX_T)res[r].i;
+#endif
+    }
+  }
+}
+#endif   /* RD_TROWS */
+
 /* ---- helpers of redux_col ------------------------------------------------- */
 
 /* Position j of the flattened reduced range: byte offset in every source and

@@ -533,6 +533,79 @@ def test_short_contiguous_rows_staged_in_lds(ctx, dtype, monkeypatch):
         assert np.array_equal(np.asarray(R.all(g, axis=1)), ones.all(axis=1))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64", "int16", "int64"])
+def test_tiny_contiguous_rows_walked_in_registers(ctx, dtype, monkeypatch):
+    """Rows of at most 32 bytes lying one after the other, the first on a
+    16-byte boundary, take the kernel that keeps a lane's rows in registers
+    (here from one row on and for every row length it can take, so that the
+    cases stay small): row lengths with one, two and more chunks per lane, a
+    last lane whose run of rows is cut short, a view that starts inside its
+    buffer (on a boundary, and off one: that one falls back), every
+    operation, ties, NaN and signed zero placement."""
+    monkeypatch.setenv("GPUARRAY_REDUX_TROWS_MIN_ROWS", "1")
+    monkeypatch.setenv("GPUARRAY_REDUX_TROWS_DIRECT", "2")
+    rng = np.random.default_rng(57)
+    item = np.dtype(dtype).itemsize
+    lengths = [n for n in (2, 3, 4, 5, 6, 7, 8, 12, 14, 16, 32) if n * item <= 32]
+    per16 = 16 // item
+    for n in lengths:
+        rows = int(rng.integers(257, 900))
+        flat = rng.integers(0, 12, size=rows * n + 2 * per16 + 3).astype(dtype)      # many ties
+        for off in (0, per16, 1) if n in (3, 4) else (0, per16):
+            host = flat[off:off + rows * n].reshape(rows, n)
+            g, _ = to_gpu_view(host, ctx)
+            if dtype == "float16":
+                val, idx = R.maxandargmax(g, axis=1)
+                assert np.array_equal(np.asarray(val), host.max(axis=1)), (n, off)
+                assert np.array_equal(np.asarray(idx), host.argmax(axis=1)), (n, off)
+                got = np.asarray(R.sum(g, axis=1, dtype="float32"))
+                assert np.array_equal(got, host.astype(np.float32).sum(axis=1)), (n, off)   # small integers: exact
+                continue
+            _check_ops(ctx, host, [1])
+            if n not in (3, 4):      # every row length is a kernel of its own: the other operations on two of them
+                continue
+            ops = ["prod", "prodnz", "all", "any"] + (["and", "or", "xor"] if np.dtype(dtype).kind in "iu" else [])
+            small = host % 3 if np.dtype(dtype).kind in "iu" else host
+            gs, _ = to_gpu_view(small, ctx)
+            for op in ops:
+                odt = R._upcast(dtype) if op in ("prod", "prodnz") else np.dtype("bool") if op in ("all", "any") else np.dtype(dtype)
+                want = np_reduce(op, small, [1], odt if op in ("prod", "prodnz") else None)
+                got = np.asarray(R._reduce_named(gs, op, odt, axis=(1,)))
+                if np.dtype(dtype).kind == "f" and op in ("prod", "prodnz"):
+                    assert np.allclose(got, np_reduce(op, small.astype(np.float64), [1]), rtol=1e-4), (op, n, off)
+                else:
+                    assert np.array_equal(got, want), (op, n, off)
+            assert np.array_equal(np.asarray(R.min(g, axis=(1,))), host.min(axis=1))
+            assert np.array_equal(np.asarray(R._arg_reduce(g, "argmin", [1], False)), host.argmin(axis=1))
+            # results that do not lie side by side, or start off the boundary of a lane's store
+            for dst in (gpuarray.zeros((2 * rows,), dtype, context=ctx)[::2],
+                        gpuarray.zeros((rows + 1,), dtype, context=ctx)[1:]):
+                R._reduce_named(g, "max", np.dtype(dtype), axis=(1,), out=dst)
+                assert np.array_equal(np.asarray(dst), host.max(axis=1)), (n, off)
+    if np.dtype(dtype).kind == "f":
+        n = 32 // item - 1
+        host = rng.integers(-20, 20, size=(3001, n)).astype(dtype)
+        nan_first = rng.choice(3001, 40, replace=False)
+        host[nan_first[:20], 0] = np.nan                          # stays
+        host[nan_first[20:], rng.integers(1, n, 20)] = np.nan     # ignored
+        host[nan_first[3], :] = np.nan
+        host[7, :] = 0.0
+        host[7, 2] = -0.0              # equal to the zeros before it: index 0 stays
+        host[8, :] = -0.0
+        host[8, 1] = 0.0
+        g, _ = to_gpu_view(host, ctx)
+        for name, nanfn, argfn in (("maxandargmax", np.nanmax, np.nanargmax), ("minandargmin", np.nanmin, np.nanargmin)):
+            val, idx = getattr(R, name)(g, axis=1)
+            val, idx = np.asarray(val), np.asarray(idx)
+            for r in range(3001):
+                if np.isnan(host[r, 0]):
+                    assert np.isnan(val[r]) and idx[r] == 0, (name, r)
+                else:
+                    assert val[r] == nanfn(host[r]) and idx[r] == argfn(host[r]), (name, r)
+            assert idx[7] == 0 and not np.signbit(val[7])
+            assert idx[8] == 0 and np.signbit(val[8])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "float64", "float16"])
 @pytest.mark.parametrize("staged", [0, 1])
 def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, monkeypatch):
@@ -866,8 +939,8 @@ def test_leading_dims_with_short_kept_rows_are_folded(ctx, monkeypatch, fold):
              ((1 << 22, 1), (0,)))
     every = ("float32", "int32", "int8", "float16", "uint8")
     for ci, (shape, axes) in enumerate(cases if fold == "1" else cases[:1]):
-        # every type on the first shape, two per shape after that
-        for dt in (every if ci == 0 and fold == "1" else (every[ci % 5], every[(ci + 2) % 5])):
+        # three types on the first shape, one per shape after that
+        for dt in (every[:4:2] + every[3:4] if ci == 0 and fold == "1" else (every[ci % 5],)):
             if np.prod(shape) * np.dtype(dt).itemsize < (4 << 20):
                 continue
             host = rng.integers(-3 if np.dtype(dt).kind in "if" else 0, 4, size=shape).astype(dt)
