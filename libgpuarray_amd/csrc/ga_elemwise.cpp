@@ -606,7 +606,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
-                            unsigned tile = 64, unsigned zmask = 0) {
+                            unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
@@ -712,14 +712,14 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       }
       s += "}\n";
     }
-    // quad index q = (bx*4 + e) * TX + tx, x = 4q
-    appendf(s, "const %s ga_q0 = (ga_bx * 4u << ga_ltx) + ga_tx;\n", N);
+    // quad index q = (bx*quads + e) * TX + tx, x = 4q
+    appendf(s, "const %s ga_q0 = (ga_bx * %uu << ga_ltx) + ga_tx;\n", N, quads);
     appendf(s, "const %s ga_nq = (%s)dim%u / 4u;\n", N, N, xd);
     for (const ge_arg &a : ge->args)
       if (a.is_array())
         appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode),
                 a.name.c_str());
-    s += "#pragma unroll\nfor (int ga_e = 0; ga_e < 4; ga_e++) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
     appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
     appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
@@ -741,7 +741,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       }
     }
     s += "}\n}\n";
-    s += "#pragma unroll\nfor (int ga_e = 0; ga_e < 4; ga_e++) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
     appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
     appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
     s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
@@ -1266,7 +1266,7 @@ class strided_call {
   unsigned ntmask = 0;              // vec4: arrays touched once, streamed past the caches
   unsigned zmask = 0;               // vec4: arrays whose stride along x (bits 16..: along y) is zero
   size_t gx = 0, groups = 0;
-  unsigned ltx = 0, tile = 64;
+  unsigned ltx = 0, tile = 64, quads = 4;
   GpuKernel *kernel = nullptr;
 
   void describe_arrays() {
@@ -1504,7 +1504,28 @@ class strided_call {
       while (ltx < 8 && ((size_t)1 << ltx) < inner) ltx++;
       size_t tx = (size_t)1 << ltx, ty = 256 >> ltx;
       size_t rows = n / dims[nd - 1];
-      gx = (inner + 4 * tx - 1) / (4 * tx);
+      // Quads (of four elements) per lane, each a group's width apart along
+      // x.  One per lane when a quad of the widest type has 16 bytes, as in
+      // the flat kernel; narrower types get more, and so do grids of one to
+      // four fills of the chip.  Kernel times with 4 / 2 / 1 quads per lane,
+      // floats: outer product into 8192 x 8192 49.8 / 45.2 / 39.7 us,
+      // (8192, 8192) + (1, 8192) 87.5 / 85.6 / 80.1, (4096, 10, 4096) *
+      // (1, 10, 1) 220 / 216 / 199, a[:, ::2] + b 168.7 / 168.8 / 162.6,
+      // (4096, 4096) + (1, 4096) 23.3 / 22.4 / 20.9; halves (8192, 8192) +
+      // (1, 8192) 46.3 / 46.2 / 53.9; (64, 100000) * (64, 1), three fills at
+      // one quad per lane, 7.9 / 9.0 / 9.2.
+      if (vec4) {
+        size_t widest = 1;
+        for (unsigned k = 0; k < na; k++) widest = std::max(widest, elsz[k]);
+        quads = widest >= 4 ? 1 : (unsigned)(4 / widest);
+        const size_t fill = (size_t)ga_hip_numprocs(ctx) * 8;
+        const size_t g1 = ((inner + quads * tx - 1) / (quads * tx)) * ((rows + ty - 1) / ty);
+        if (g1 > fill && g1 <= 2 * fill) quads = std::min(4u, quads * 2);
+        else if (g1 > 2 * fill && g1 <= 4 * fill) quads = 4;
+        const unsigned long forced = env_ul("GPUARRAY_ELEMWISE_QUADS", 0);
+        if (forced == 1 || forced == 2 || forced == 4) quads = (unsigned)forced;
+      }
+      gx = (inner + quads * tx - 1) / (quads * tx);
       groups = gx * ((rows + ty - 1) / ty);
     } else {
       // Transposed tiles.  A group takes a 64 x 64 tile (256 lanes) or a
@@ -1572,14 +1593,14 @@ class strided_call {
 
   int get_kernel() {
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile);
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
