@@ -1234,8 +1234,18 @@ class reduction_call {
     // 8192 x 8192 50.9 / 49.4 / 51.4, over the middle axis of 256 x 512 x 512
     // 47.0 / 43.8 / 47.5; but 8 x 2^23 over axis 0 49.3 / 72.4 / 121 and
     // 256 x 2^18 45.8 / 48.2 / 47.2.
+    // Also 8 when successive elements of the reduced range lie 12 KiB or more
+    // apart (a middle axis over long inner rows) and there are 32 of them or
+    // more.  Sum over the middle axis, 4 / 8 lane rows: (128, 128, 4096) floats
+    // 59.7 / 41.0 us, (64, 128, 8192) 50.3 / 40.7, (128, 128, 3072) 31.5 /
+    // 29.8, (32, 128, 12288) 34.4 / 29.3, (128, 32, 16384) 48.4 / 40.0,
+    // (64, 256, 4096) 46.2 / 42.8, halves (128, 128, 8192) 60.0 / 41.7; but
+    // (256, 128, 2048), 8 KiB apart, 42.8 / 44.7 and (512, 128, 1024) 40.5 / 44.2.
+    int64_t rpitch = 0;
+    for (unsigned q = 0; q < K && p.nr > 0; q++) rpitch = std::max(rpitch, iabs(rsstr[q * RD_MAXD + p.nr - 1]));
+    const bool far_apart = rpitch >= (int64_t)env_ul("GPUARRAY_REDUX_COL_FAR", 12288) && rtotal >= 32;
     CY = (cy_forced == 1 || cy_forced == 2 || cy_forced == 4 || cy_forced == 8 || cy_forced == 16)
-             ? (unsigned)cy_forced : (rtotal >= 512 ? 8 : 4);
+             ? (unsigned)cy_forced : (rtotal >= 512 || far_apart ? 8 : 4);
     int64_t CX = 256 / CY;   // lanes along the free dim
     // Adjacent outputs per lane: as many as one 16-byte load of the widest
     // source holds, when the inner free dim is contiguous in every source and
