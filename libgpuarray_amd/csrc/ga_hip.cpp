@@ -317,6 +317,7 @@ struct hip_context : _gpucontext {
   std::string disk_cache;   // directory of the on-disk kernel cache, empty = off
   void *stage = nullptr;    // pinned host memory that small reads and writes go through
   gpukernel *copy_kernel = nullptr;   // byte copy behind buffer_move
+  gpukernel *fill_kernel = nullptr;   // byte fill behind buffer_memset
   bool stage_failed = false;
   ga_errrec errstore;
 };
@@ -591,6 +592,10 @@ void hip_deinit(gpucontext *c) {
   ga_extcopy_cache_free(c);
   ga_redux_cache_free(c);
   ga_take1_cache_free(c);
+  if (ctx->fill_kernel) {
+    hip_freekernel(ctx->fill_kernel);
+    ctx->fill_kernel = nullptr;
+  }
   if (ctx->copy_kernel) {
     hip_freekernel(ctx->copy_kernel);
     ctx->copy_kernel = nullptr;
@@ -810,6 +815,23 @@ int hip_write(gpudata *dst, size_t dstoff, const void *src, size_t sz) {
 }
 
 // Fill from dstoff to the end of the buffer with the low byte of `data`.
+// Fill of n bytes with one value: one 16-byte streaming chunk per lane, the
+// bytes before the first and after the last whole chunk one per lane.
+const char FILL_KERNEL_SRC[] =
+    "#include \"cluda.h\"\n"
+    "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n"
+    "KERNEL void __launch_bounds__(256) ga_fill(GLOBAL_MEM char *dst, const ga_size doff,\n"
+    "    const ga_size head, const ga_size nchunks, const ga_size n, const ga_uint word) {\n"
+    "  dst += doff;\n"
+    "  const ga_size t = (ga_size)GID_0 * 256 + LID_0;\n"
+    "  if (t < nchunks) {\n"
+    "    const ga_chunk16 v = {word, word, word, word};\n"
+    "    __builtin_nontemporal_store(v, (ga_chunk16 *)(dst + head) + t);\n"
+    "  }\n"
+    "  const ga_size rest = n - nchunks * 16;\n"
+    "  if (t < rest) dst[t < head ? t : t + nchunks * 16] = (char)word;\n"
+    "}\n";
+
 int hip_memset(gpudata *dst, size_t dstoff, int data) {
   hip_context *ctx = HC(dst->ctx);
   hip_data *b = HD(dst);
@@ -823,6 +845,29 @@ int hip_memset(gpudata *dst, size_t dstoff, int data) {
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     memset((char *)b->devptr + dstoff, data & 0xff, n);
     return GA_NO_ERROR;
+  }
+  // The library's own kernel whenever the stream records a graph: a memset
+  // recorded into a graph is a node of its own kind, and such nodes have
+  // replayed wrongly.  Otherwise the driver's fill, which is as fast (measured
+  // on MI355X, 30 fills back to back: 1 GiB 161.7 us against 160.1 with this
+  // kernel, 64 MiB 11.7 / 11.5, 16 MiB 5.2 / 4.7, 1 MiB 4.4 / 4.7).
+  if (ga_hip_capturing(dst->ctx) || n >= env_ul("GPUARRAY_FILL_KERNEL_MIN", ~0ul)) {
+    if (ctx->fill_kernel == nullptr) {
+      const char *strs[1] = {FILL_KERNEL_SRC};
+      const int types[6] = {GA_BUFFER, GA_SIZE, GA_SIZE, GA_SIZE, GA_SIZE, GA_UINT};
+      if ((err = hip_newkernel(&ctx->fill_kernel, ctx, 1, strs, nullptr, "ga_fill", 6, types, 0,
+                               nullptr)) != GA_NO_ERROR)
+        return err;
+    }
+    const uintptr_t da = (uintptr_t)b->devptr + dstoff;
+    size_t head = (16 - da % 16) % 16;
+    if (head > n) head = n;
+    size_t nchunks = (n - head) / 16;
+    const size_t rest = n - nchunks * 16;
+    size_t gs = (std::max(nchunks, rest) + 255) / 256, ls = 256;
+    unsigned int word = (unsigned int)(data & 0xff) * 0x01010101u;
+    void *args[6] = {dst, &dstoff, &head, &nchunks, &n, &word};
+    return hip_callkernel(ctx->fill_kernel, 1, &gs, &ls, 0, args);
   }
   HIP_TRY(ctx, hipMemsetD8Async((hipDeviceptr_t)((char *)b->devptr + dstoff),
                                 (unsigned char)(data & 0xff), n, ctx->stream));

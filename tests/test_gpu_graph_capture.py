@@ -5,7 +5,8 @@ counterpart of the reference's cuda_get_stream, src/gpuarray/ext_cuda.h) can
 put it into capture mode, issue GpuElemwise / GpuReduction calls on arrays
 that already exist, and replay the recorded launches with one graph launch.
 That only works if a call on warmed-up operators does nothing but launch
-kernels on that stream: no allocation, no memset, no synchronisation.  Each
+kernels on that stream: no allocation, no memset node (GpuArray_memset fills with a
+kernel while the stream records), no synchronisation.  Each
 replay here follows eager work (new input contents, a synchronisation) and is
 compared bit for bit with the same calls issued eagerly."""
 import ctypes as C
@@ -40,8 +41,11 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
     wide = gpuarray.zeros((fold_rows, 10), f32, context=ctx)
     wide_fill = ga.GpuElemwise(ctx, "w = a * 3.0f", [arg("a", f32, read=True), arg("w", f32, write=True)])
 
+    bump = ga.GpuElemwise(ctx, "z = z + 1", [arg("z", "uint8", read=True, write=True)])
+
     def outputs():
         return dict(c=gpuarray.zeros((n,), f32, context=ctx), d=gpuarray.zeros((n,), f32, context=ctx),
+                    z=gpuarray.zeros((100003,), "uint8", context=ctx),
                     ws=gpuarray.zeros((10,), f32, context=ctx),
                     rs=gpuarray.zeros((rows,), f32, context=ctx), tot=gpuarray.zeros((), f32, context=ctx),
                     cs=gpuarray.zeros((cols,), f32, context=ctx),
@@ -59,6 +63,8 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
         flat = wide.reshape((fold_rows * 10,))
         wide_fill(a[:n // 4], flat[:n // 4])        # part of `wide` follows the inputs
         rsum(wide, [0], d0=o["ws"])
+        o["z"].memset(5)                            # recorded as a kernel of the library, not as a memset node
+        bump(o["z"])
 
     eager, replayed = outputs(), outputs()
     issue(eager)                                 # compiles everything, sizes the scratch buffer
@@ -81,7 +87,7 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
             a.write(ha)
             b.write(hb)
             for v in replayed.values():          # stale results must not pass for fresh ones
-                v.write(np.full(v.shape, -7, v.dtype))
+                v.write(np.full(v.shape, 249 if v.dtype == np.uint8 else -7, v.dtype))
             ctx.sync()
             assert hip.hipGraphLaunch(gexec, stream) == 0
             ctx.sync()
@@ -92,6 +98,7 @@ def test_elemwise_and_reductions_replay_from_a_graph(ctx):
             c = ha * hb + np.float32(0.5)
             d = c * c - np.float32(0.25)
             assert np.array_equal(np.asarray(replayed["d"]), d)
+            assert np.all(np.asarray(replayed["z"]) == 6)
             assert np.array_equal(np.asarray(replayed["mi"]), d.reshape(rows, cols).argmax(axis=1))
     finally:
         hip.hipGraphExecDestroy(gexec)
