@@ -1,0 +1,190 @@
+"""Kernel times of common array shapes, against the bytes they must move.
+
+    python -m libgpuarray_amd.shapes_bench [--only elemwise|reductions] [--iters N]
+
+The benchmark of the repository (bench.py) prices one large contiguous
+elementwise kernel and one full sum.  This walks through the shapes that
+surround them in real use - broadcast operands, casts, transposes, views,
+reductions over every kind of axis, tiny and ragged rows - and prints, per
+case, the time its kernels run on the device (start and stop event on every
+launch, summed per call, median over the calls), the launches per call, and
+the bytes every distinct element touched once amounts to, as GB/s and as a
+share of MI355X's 8 TB/s.  Inputs are zeros; every case rotates over four
+sets of buffers so that a footprint the 256 MB Infinity Cache could hold is
+still read from memory.  One JSON line per case on stdout, a table on stderr.
+"""
+import argparse
+import json
+import sys
+
+import numpy as np
+
+PEAK_GBPS = 8000.0
+ROT = 4
+
+
+def _kernel_us(ctx, call, iters):
+    for i in range(3):
+        call(i)
+    ctx.sync()
+    ctx.kernel_timing(True)
+    for i in range(iters):
+        call(i)
+    ms = np.array(ctx.kernel_times())
+    ctx.kernel_timing(False)
+    per = max(len(ms) // iters, 1)
+    return float(np.median(ms[:per * iters].reshape(iters, per).sum(axis=1))) * 1e3, per
+
+
+def _report(kind, label, us, launches, nbytes):
+    gbps = nbytes / us / 1e3
+    print(json.dumps({"kind": kind, "case": label, "kernel_us": round(us, 2), "launches": launches,
+                      "bytes": int(nbytes), "GBps": round(gbps, 1), "of_peak": round(gbps / PEAK_GBPS, 4)}),
+          flush=True)
+    print("%-10s %-62s %8.2f us  %d launch%s  %6.0f GB/s  %5.1f %%" %
+          (kind, label, us, launches, " " if launches == 1 else "es", gbps, 100 * gbps / PEAK_GBPS),
+          file=sys.stderr, flush=True)
+
+
+def elemwise_cases():
+    """(label, expression, [(name, dtype, base shape, view or None)], output shape, output dtype)"""
+    f, h, d, u8 = "float32", "float16", "float64", "uint8"
+    N = 1 << 26
+    T = lambda *axes: (lambda b: b.transpose(*axes))
+    return [
+        ("a + b, 2^26 floats", "o = a + b", [("a", f, (N,), None), ("b", f, (N,), None)], (N,), f),
+        ("a*b + c, 2^27 halves", "o = a * b + c", [("a", h, (2 * N,), None), ("b", h, (2 * N,), None), ("c", h, (2 * N,), None)], (2 * N,), h),
+        ("a + b, 2^25 doubles", "o = a + b", [("a", d, (N // 2,), None), ("b", d, (N // 2,), None)], (N // 2,), d),
+        ("tanh, 2^26 floats", "o = tanh(a)", [("a", f, (N,), None)], (N,), f),
+        ("exp, 2^26 floats", "o = exp(a)", [("a", f, (N,), None)], (N,), f),
+        ("a > 0 ? a : 0.01 a, 2^26 floats", "o = a > 0 ? a : 0.01f * a", [("a", f, (N,), None)], (N,), f),
+        ("bytes -> floats / 255, 2^27", "o = a * (1.0f / 255.0f)", [("a", u8, (2 * N,), None)], (2 * N,), f),
+        ("floats -> halves, 2^27", "o = a", [("a", f, (2 * N,), None)], (2 * N,), h),
+        ("floats -> bytes, 2^27", "o = a", [("a", f, (2 * N,), None)], (2 * N,), u8),
+        ("a > b -> bool, 2^27 floats", "o = a > b", [("a", f, (2 * N,), None), ("b", f, (2 * N,), None)], (2 * N,), "bool"),
+        ("halves -> floats, 2^27", "o = a", [("a", h, (2 * N,), None)], (2 * N,), f),
+        ("fill, 2^26 floats", "o = 1.0f", [], (N,), f),
+        ("(8192, 8192) + (1, 8192)", "o = a + b", [("a", f, (8192, 8192), None), ("b", f, (1, 8192), None)], (8192, 8192), f),
+        ("(8192, 8192) * (8192, 1)", "o = a * b", [("a", f, (8192, 8192), None), ("b", f, (8192, 1), None)], (8192, 8192), f),
+        ("(8192, 1) * (1, 8192), outer product", "o = a * b", [("a", f, (8192, 1), None), ("b", f, (1, 8192), None)], (8192, 8192), f),
+        ("(64, 256, 64, 64): (a - m) * r per channel", "o = (a - m) * r",
+         [("a", f, (64, 256, 64, 64), None), ("m", f, (1, 256, 1, 1), None), ("r", f, (1, 256, 1, 1), None)], (64, 256, 64, 64), f),
+        ("(64, 64, 64, 256) * (1, 1, 1, 256), channels last", "o = a * b",
+         [("a", f, (64, 64, 64, 256), None), ("b", f, (1, 1, 1, 256), None)], (64, 64, 64, 256), f),
+        ("(2^24, 3) + (1, 3)", "o = a + b", [("a", f, (1 << 24, 3), None), ("b", f, (1, 3), None)], (1 << 24, 3), f),
+        ("(2^22, 10) + (1, 10)", "o = a + b", [("a", f, (1 << 22, 10), None), ("b", f, (1, 10), None)], (1 << 22, 10), f),
+        ("(2^22, 10) * (2^22, 1)", "o = a * b", [("a", f, (1 << 22, 10), None), ("b", f, (1 << 22, 1), None)], (1 << 22, 10), f),
+        ("(65536, 1001) + (1, 1001)", "o = a + b", [("a", f, (65536, 1001), None), ("b", f, (1, 1001), None)], (65536, 1001), f),
+        ("(4096, 10, 4096) * (1, 10, 1)", "o = a * b", [("a", f, (4096, 10, 4096), None), ("b", f, (1, 10, 1), None)], (4096, 10, 4096), f),
+        ("(64, 3, 512, 512) - (1, 3, 1, 1)", "o = a - b", [("a", f, (64, 3, 512, 512), None), ("b", f, (1, 3, 1, 1), None)], (64, 3, 512, 512), f),
+        ("a[:, ::2] + b, 8192 x 8192 (useful bytes)", "o = a + b",
+         [("a", f, (8192, 16384), lambda b: b[:, ::2]), ("b", f, (8192, 8192), None)], (8192, 8192), f),
+        ("a[:, 1:-1] * 2, 8192 x 8192", "o = a * 2.0f", [("a", f, (8192, 8194), lambda b: b[:, 1:-1])], (8192, 8192), f),
+        ("a[1:-1, :] * 2, 8192 x 8192", "o = a * 2.0f", [("a", f, (8194, 8192), lambda b: b[1:-1, :])], (8192, 8192), f),
+        ("a.T + b, 8192 x 8192", "o = a + b", [("a", f, (8192, 8192), T(1, 0)), ("b", f, (8192, 8192), None)], (8192, 8192), f),
+        ("transpose (0, 2, 1) of (64, 1024, 1024)", "o = a", [("a", f, (64, 1024, 1024), T(0, 2, 1))], (64, 1024, 1024), f),
+        ("transpose (1, 0, 2) of (1024, 64, 1024)", "o = a", [("a", f, (1024, 64, 1024), T(1, 0, 2))], (64, 1024, 1024), f),
+        ("transpose (2, 1, 0) of (256, 512, 512)", "o = a", [("a", f, (256, 512, 512), T(2, 1, 0))], (512, 512, 256), f),
+        ("NCHW -> NHWC, (64, 256, 64, 64)", "o = a", [("a", f, (64, 256, 64, 64), T(0, 2, 3, 1))], (64, 64, 64, 256), f),
+    ]
+
+
+def reduction_cases():
+    """(operation, dtype, shape, axes, result dtype or None, view or None, note)"""
+    f, h = "float32", "float16"
+    return [
+        ("sum", f, ((1 << 26) + 12345,), (0,), None, None, "ragged length"),
+        ("sum", h, (1 << 27,), (0,), f, None, ""),
+        ("sum", "float64", (1 << 25,), (0,), None, None, ""),
+        ("sum", "int32", (1 << 26,), (0,), "int64", None, ""),
+        ("any", "bool", (1 << 28,), (0,), "bool", None, ""),
+        ("sum", f, (65536, 1001), (1,), None, None, "rows off a 16-byte boundary"),
+        ("max", f, (65536, 1001), (1,), None, None, ""),
+        ("sum", f, (1335, 50257), (1,), None, None, ""),
+        ("sum", f, (1 << 20, 64), (1,), None, None, "short rows staged in LDS"),
+        ("max", f, (1 << 21, 32), (1,), None, None, ""),
+        ("sum", f, (1 << 22, 10), (1,), None, None, "tiny rows"),
+        ("argmax", f, (1 << 22, 10), (1,), None, None, "predicted class"),
+        ("sum", f, (22369620, 3), (1,), None, None, "rows of 12 bytes, walked in registers"),
+        ("argmax", f, (22369620, 3), (1,), None, None, ""),
+        ("sum", f, (9586980, 7), (1,), None, None, ""),
+        ("sum", h, (1 << 24, 6), (1,), f, None, ""),
+        ("sum", "uint8", (1 << 24, 12), (1,), "int64", None, ""),
+        ("max", "uint8", (1 << 25, 4), (1,), None, None, ""),
+        ("sum", f, (8192, 8192), (0,), None, None, "column kernel"),
+        ("min", "int32", (8192, 8192), (0,), None, None, ""),
+        ("sum", f, (64, 1 << 20), (0,), None, None, "few long rows"),
+        ("sum", f, (1 << 20, 64), (0,), None, None, ""),
+        ("sum", f, (1 << 22, 10), (0,), None, None, "bias gradient: folded rows"),
+        ("sum", f, (65536, 1001), (0,), None, None, "folded rows"),
+        ("sum", f, (1 << 24, 3), (0,), None, None, "folded rows"),
+        ("sum", f, (64, 256, 64, 64), (0, 2, 3), None, None, "per-channel statistics, NCHW"),
+        ("sum", f, (64, 64, 64, 256), (0, 1, 2), None, None, "per-channel statistics, NHWC"),
+        ("sum", f, (64, 256, 64, 64), (2, 3), None, None, "global pooling"),
+        ("sum", f, (64, 256, 64, 64), (1,), None, None, "over the channels"),
+        ("max", f, (64, 256, 64, 64), (1,), None, None, ""),
+        ("sum", f, (128, 128, 4096), (1,), None, None, "middle axis, 16 KiB apart"),
+        ("sum", f, (8192, 16384), (0, 1), None, lambda a: a[:, ::2], "stride-2 view (useful bytes)"),
+        ("sum", f, (8192, 8192), (1,), None, lambda a: a.T, "rows of a transposed matrix"),
+    ]
+
+
+def run_elemwise(ctx, ga, gpuarray, iters):
+    for label, expr, specs, oshape, odt in elemwise_cases():
+        args = [ga.arg(n, dt, read=True) for n, dt, _, _ in specs] + [ga.arg("o", odt, write=True)]
+        k = ga.GpuElemwise(ctx, expr, args, convert_f16=True)
+        sets = []
+        for _ in range(ROT):
+            ins = []
+            for _, dt, shape, view in specs:
+                base = gpuarray.zeros(shape, dt, context=ctx)
+                ins.append(view(base) if view else base)
+            sets.append(ins + [gpuarray.empty(oshape, odt, context=ctx)])
+        us, per = _kernel_us(ctx, lambda i: k(*sets[i % ROT], broadcast=True), iters)
+        nbytes = int(np.prod(oshape)) * np.dtype(odt).itemsize
+        for v, (_, dt, _, _) in zip(sets[0], specs):
+            nbytes += int(np.prod(v.shape)) * np.dtype(dt).itemsize
+        _report("elemwise", label, us, per, nbytes)
+        del sets
+
+
+def run_reductions(ctx, ga, gpuarray, iters):
+    for op, dt, shape, axes, odt, view, note in reduction_cases():
+        red = ga.GpuReduction(ctx, op, dt)
+        sets = []
+        for _ in range(ROT):
+            src = gpuarray.zeros(shape, dt, context=ctx)
+            if view:
+                src = view(src)
+            oshape = tuple(n for i, n in enumerate(src.shape) if i not in axes)
+            d0 = None if op in ("argmax", "argmin") else gpuarray.empty(oshape, odt or dt, context=ctx)
+            d1 = gpuarray.empty(oshape, "int64", context=ctx) if op in ("argmax", "argmin") else None
+            sets.append((src, d0, d1))
+        us, per = _kernel_us(ctx, lambda i: red(sets[i % ROT][0], list(axes), d0=sets[i % ROT][1], d1=sets[i % ROT][2]), iters)
+        src, d0, d1 = sets[0]
+        nbytes = int(np.prod(src.shape)) * np.dtype(dt).itemsize
+        for out in (d0, d1):
+            if out is not None:
+                nbytes += int(np.prod(out.shape)) * out.dtype.itemsize
+        label = "%s %s %s over %s" % (op, dt, tuple(src.shape), axes) + (" (%s)" % note if note else "")
+        _report("reduction", label, us, per, nbytes)
+        del sets
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--only", choices=["elemwise", "reductions"], default=None)
+    ap.add_argument("--iters", type=int, default=20)
+    args = ap.parse_args()
+    import libgpuarray_amd as ga
+    from libgpuarray_amd import gpuarray
+
+    ctx = ga.init("hip0")
+    if args.only in (None, "elemwise"):
+        run_elemwise(ctx, ga, gpuarray, args.iters)
+    if args.only in (None, "reductions"):
+        run_reductions(ctx, ga, gpuarray, args.iters)
+
+
+if __name__ == "__main__":
+    main()
