@@ -884,6 +884,11 @@ class reduction_call {
     use_row = p.nf == 0 || (rstr <= fstr && (rin >= 32 || p.nr <= 1)) ||
                    (rin >= 4096 && rstr <= 4 * elsz_max);
     if (rtotal == 0) use_row = true;
+    // (A handful of outputs over a small array - the sum over axis 0 of
+    // (8192, 10) floats - looks faster with lanes along the reduced run when the
+    // array is still in the cache from the call before, 7.9 -> 4.8 us; read
+    // after another kernel wrote it, as the second call of folded rows does, it
+    // is slower, 7.6 -> 10.2 us.  Not taken.)
     {
       const char *force = getenv("GPUARRAY_REDUX_FAMILY");
       if (force && strcmp(force, "row") == 0) use_row = true;
@@ -1419,11 +1424,22 @@ class reduction_call {
       // (16384, 4096) 44.3 / 43.8, of (65536, 1024) 44.0 / 51.9, of
       // (2^20, 64) 44.3 / 73.0.
       bool fuse = groups <= fused_max;
-      if (!fuse && fused_max > 0) {
+      // (partials that carry an index cost the column kernel's last piece twice
+      // the loads: maxandargmax over axis 0 of (8192, 8192) 47.8 / 50.5)
+      const bool carries_index = info.has_d1 || (minmax && is_float_type(acc_tc));
+      // The column kernel's last piece walks through a tile's partials with
+      // one lane row per 1 / RD_CY of them: many pieces are better combined by
+      // the second launch, whose every wavefront takes a share.  One launch
+      // against the kernels of two, over axis 0: sum of (8192, 10) floats, 128
+      // pieces, 5.6 / 8.0 us, of (4096, 256), 64 pieces, 7.0 / 8.2, of
+      // (16384, 64), 256 pieces, 10.5 / 7.8; maximum of floats (value and
+      // position) (4096, 256) 14.9 / 10.6, (16384, 64) 25.5 / 12.6, (1024, 1024)
+      // 11.9 / 10.4.
+      if (fuse && !use_row &&
+          p.nsplit > (int)env_ul("GPUARRAY_REDUX_FUSED_COL_FEW", carries_index ? 16 : 128))
+        fuse = false;
+      if (!fuse && fused_max > 0 && groups > fused_max) {
         const double piece_bytes = (double)nrows * (double)rtotal * (double)elsz_sum / (double)groups;
-        // (partials that carry an index cost the column kernel's last piece twice
-        // the loads: maxandargmax over axis 0 of (8192, 8192) 47.8 / 50.5)
-        const bool carries_index = info.has_d1 || (minmax && is_float_type(acc_tc));
         fuse = use_row ? piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_PIECE", 384u << 10)
                        : (!carries_index && p.nsplit <= (int)env_ul("GPUARRAY_REDUX_FUSED_COL_SPLITS", 16) &&
                           piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_COL_PIECE", 128u << 10));
@@ -1634,10 +1650,17 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   size_t g = rowb, h = 16;
   while (h) { size_t t = g % h; g = h; h = t; }      // g = gcd(rowb, 16)
   const size_t m0 = 16 / g;
+  // Folded rows of 256 KiB where the row count allows it: the first call then
+  // needs no split (or a few pieces that end in its own launch), and the second
+  // combines a few thousand partial rows.  Narrower folds for smaller arrays.
+  // Sum over axis 0, folds of 4 KiB / 256 KiB, all launches: (2^22, 10) floats
+  // 35.5 / 31.6 us (three launches / two), (2^24, 3) 38.9 / 34.1, (65536, 1001)
+  // 49.3 / 46.1, (4096, 4096, 4) over two axes 50.1 / 43.4, (2^20, 17) 20.2 / 16.9.
   size_t m = 0;
-  const size_t width = env_ul("GPUARRAY_REDUX_FOLD_BYTES", 4096);
-  for (size_t t = (width + m0 * rowb - 1) / (m0 * rowb); t * m0 <= 65536; t++)
-    if (R % (t * m0) == 0 && R / (t * m0) >= 64) { m = t * m0; break; }
+  const size_t widest = env_ul("GPUARRAY_REDUX_FOLD_BYTES", 262144);
+  for (size_t width = widest; m == 0 && width >= 4096; width /= 8)
+    for (size_t t = (width + m0 * rowb - 1) / (m0 * rowb); t * m0 <= 65536; t++)
+      if (R % (t * m0) == 0 && R / (t * m0) >= 64) { m = t * m0; break; }
   if (m <= 1) return GA_NO_ERROR;
 
   // type of the folded partial results: the accumulator's (a half result is summed in float)

@@ -1660,12 +1660,36 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     if (!last_piece) return;
     rd_before_loads();
 #pragma unroll
-    for (int c = 0; c < RD_CV; c++) {
-      rd_acc a = rd_neutral();
-      if (live)
-        for (ga_long s = ty; s < p.nsplit; s += RD_CY)
-          a = rd_combine(a, rd_fetch_partial(part_v, part_i, s * p.nrows + fo * fin + fi + c));
-      acc[c] = a;
+    for (int c = 0; c < RD_CV; c++) acc[c] = rd_neutral();
+    if (live) {
+      /* a lane row's partials four or eight splits at a time, all their loads issued
+       * before the first is combined (one at a time, the 256 partials of 64
+       * outputs took 12 of the 16 us of a sum over axis 0 of (16384, 64));
+       * combined in the order of the splits either way */
+      const ga_long at = fo * fin + fi;
+      ga_long s = ty;
+#if RD_ARG || RD_CV > 4
+#define RD_FIN_BATCH 4
+#else
+#define RD_FIN_BATCH 8
+#endif
+      for (; s + (RD_FIN_BATCH - 1) * RD_CY < p.nsplit; s += RD_FIN_BATCH * RD_CY) {
+        rd_acc t[RD_FIN_BATCH][RD_CV];
+#pragma unroll
+        for (int j = 0; j < RD_FIN_BATCH; j++)
+#pragma unroll
+          for (int c = 0; c < RD_CV; c++)
+            t[j][c] = rd_fetch_partial(part_v, part_i, (s + j * RD_CY) * p.nrows + at + c);
+#pragma unroll
+        for (int j = 0; j < RD_FIN_BATCH; j++)
+#pragma unroll
+          for (int c = 0; c < RD_CV; c++) acc[c] = rd_combine(acc[c], t[j][c]);
+      }
+#undef RD_FIN_BATCH
+      for (; s < p.nsplit; s += RD_CY)
+#pragma unroll
+        for (int c = 0; c < RD_CV; c++)
+          acc[c] = rd_combine(acc[c], rd_fetch_partial(part_v, part_i, s * p.nrows + at + c));
     }
 #if RD_CY > 1
 #pragma unroll
