@@ -47,21 +47,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # are in profiles/hbm_traffic_all_configs.md.
 MEASURED_TRAFFIC = {
     # name: (kernel text hash, HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201259246),
-    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134367705),
-    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536666880),
-    "C3a_sum_axis1_8192x8192": ("52888ba6bdb69ee9", 268766251),
-    "C4_maxandargmax_65536x1000": ("2ed07e6129037c05", 263773059),
-    "C5_fp16_sum_axes02": ("e5efd9c2b1cba640", 269706642),
-    "C5_int32_sum_axis1": ("d937fae7ff3339e7", 538005680),
-    "C5_uint8_all_axis2": ("f3623b9a39fed6b5", 134384132),
-    "C5_uint8_any_axis2": ("a527d25fdd9fe945", 134384224),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538671188),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538667901),
-    "F4_dot_2x2^27_fused": ("801b527cda3bc23d", 1073848439),
-    "F4_dot_2x2^27_two_pass": ("f1dd398ef31d30fc", 2146744643),
-    "elem_2^28": ("712fba8f0b8a6108", 3219576353),
-    "sum_2^28": ("f1dd398ef31d30fc", 1073797908),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201255162),
+    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134354659),
+    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536638854),
+    "C3a_sum_axis1_8192x8192": ("dad31caa5cba69db", 268766015),
+    "C4_maxandargmax_65536x1000": ("e07f5c491a26ec87", 263701951),
+    "C5_fp16_sum_axes02": ("1c31fb49c4b5b020", 269706750),
+    "C5_int32_sum_axis1": ("8274229b3cbbd35d", 538005647),
+    "C5_uint8_all_axis2": ("f820fbfcf8c6c517", 134384187),
+    "C5_uint8_any_axis2": ("4d7e5c2312df6b47", 134384118),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538649272),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538654594),
+    "F4_dot_2x2^27_fused": ("8b73e74aff3e53e7", 1073848190),
+    "F4_dot_2x2^27_two_pass": ("fad720c7c171b6dc", 2146728209),
+    "elem_2^28": ("712fba8f0b8a6108", 3219542703),
+    "sum_2^28": ("fad720c7c171b6dc", 1073797825),
 }
 
 
