@@ -57,4 +57,20 @@ for case in range(cases):
         g[::2] = g[::2].copy()
         picks = rng.integers(0, view.shape[0], size=int(rng.integers(1, 40)))
         assert g.take1(ga.array(picks, context=ctx)).shape == (len(picks),) + view.shape[1:]
+# fixed shapes that take the planners' special routes: rows of at most 32 bytes
+# walked in registers, leading dims over short kept rows (folded), a flat kernel
+# with a narrow side beyond one fill of the chip, an outer product
+if int(sys.argv[1]) == 0:
+    for dt, shape in (("float32", (20000, 3)), ("float16", (20011, 6)), ("uint8", (70001, 12)), ("int64", (16385, 2))):
+        g = ga.zeros(shape, dt, context=ctx)
+        assert np.asarray(R.sum(g, axis=(1,))).shape == shape[:1]
+        v, i = R.maxandargmax(g, axis=(1,))
+        assert np.asarray(i).shape == shape[:1]
+    for dt, shape, axes in (("float32", (1 << 20, 10), (0,)), ("int8", (1 << 22, 3), (0,)), ("float32", (1024, 1024, 4), (0, 1))):
+        g = ga.zeros(shape, dt, context=ctx)
+        assert np.asarray(R.sum(g, axis=axes)).shape == tuple(d for k, d in enumerate(shape) if k not in axes)
+    g = ga.zeros((3 << 20,), "uint8", context=ctx)
+    assert g.astype("float32").shape == g.shape and g.astype("float32").astype("float16").shape == g.shape
+    col, row = ga.zeros((2048, 1), "float32", context=ctx), ga.zeros((1, 2048), "float32", context=ctx)
+    assert elemwise2(col, "*", row, col, broadcast=True).shape == (2048, 2048)
 print("planner ok")
