@@ -58,6 +58,10 @@ def main():
     check("elemwise strided vec4 plain", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 2, 2, 0, 0b101 << 16))
     check("elemwise strided vec4 transposed", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 2, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 plain, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 2, 0, 0b101 << 16))
+    GA_DOUBLE_ = 12
+    dargs = (ElemwiseArg * 3)(ElemwiseArg(b"a", GA_DOUBLE_, 2), ElemwiseArg(b"b", GA_FLOAT, 2),
+                              ElemwiseArg(b"c", GA_DOUBLE_, 4))
+    check("elemwise strided, two doubles per lane", gen_e(b"", b"c = a*b + 0.5", 3, dargs, 0, 10, 2, 0, 0b101 << 16))
     check("elemwise strided vec4 transposed, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 4, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles, operand constant along x",
@@ -162,7 +166,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "20 elementwise)" % (n + 20, m, t))
+          "21 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

@@ -606,8 +606,11 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
-                            unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4) {
+                            unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4, unsigned vq = 4) {
   std::string s;
+  // elements a lane moves at a time: 4, or (plain variant only) 2 when the
+  // widest type has 8 bytes, so that the widest access stays at 16 bytes
+  const unsigned VQ = tmask ? 4 : vq;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
   emit_header(ge, s);
@@ -652,7 +655,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   auto is_y = [&](size_t j) {
     return aidx[j] >= 0 && ((zmask >> (16 + aidx[j])) & 1u) && !ge->args[j].writes();
   };
-  auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * 4); };
+  auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * VQ); };
   // 16-byte accesses of arrays whose every element is touched once carry the
   // streaming hint (ntmask); broadcast operands stay cacheable
   auto is_nt = [&](size_t j) { return aidx[j] >= 0 && ((ntmask >> aidx[j]) & 1u); };
@@ -712,15 +715,15 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       }
       s += "}\n";
     }
-    // quad index q = (bx*quads + e) * TX + tx, x = 4q
+    // quad index q = (bx*quads + e) * TX + tx, x = VQ*q
     appendf(s, "const %s ga_q0 = (ga_bx * %uu << ga_ltx) + ga_tx;\n", N, quads);
-    appendf(s, "const %s ga_nq = (%s)dim%u / 4u;\n", N, N, xd);
+    appendf(s, "const %s ga_nq = (%s)dim%u / %uu;\n", N, N, xd, VQ);
     for (const ge_arg &a : ge->args)
       if (a.is_array())
-        appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode),
+        appendf(s, "union { %s c; %s e[%u]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), VQ,
                 a.name.c_str());
     appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
-    appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
+    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, VQ, N);
     appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
@@ -729,10 +732,10 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
         s += quad_load(j, a.name + "_u[ga_e].c", quad_at(a, a.name + "_o", "ga_x"));
       } else if (is_z(j)) {
         appendf(s, "%s_u[ga_e].e[0] = %s;\n", a.name.c_str(), elem_at(a, a.name + "_o", "0").c_str());
-        for (int i = 1; i < 4; i++)
+        for (int i = 1; i < (int)VQ; i++)
           appendf(s, "%s_u[ga_e].e[%d] = %s_u[ga_e].e[0];\n", a.name.c_str(), i, a.name.c_str());
       } else {
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < (int)VQ; i++) {
           char xi[32];
           snprintf(xi, sizeof(xi), "ga_x + %du", i);
           appendf(s, "%s_u[ga_e].e[%d] = %s;\n", a.name.c_str(), i,
@@ -742,9 +745,9 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     }
     s += "}\n}\n";
     appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
-    appendf(s, "const %s ga_x = 4u * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, N);
+    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, VQ, N);
     appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
-    s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", VQ);
     for (const ge_arg &a : ge->args)
       if (a.is_array()) emit_load(ge, s, a, a.name + "_u[ga_e].e[ga_v]");
     s += ge->expr;
@@ -758,7 +761,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       if (is_u(j)) {
         s += quad_store(j, quad_at(a, a.name + "_o", "ga_x"), a.name + "_u[ga_e].c");
       } else {
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < (int)VQ; i++) {
           char xi[32];
           snprintf(xi, sizeof(xi), "ga_x + %du", i);
           appendf(s, "%s = %s_u[ga_e].e[%d];\n", elem_at(a, a.name + "_o", xi).c_str(),
@@ -1267,6 +1270,7 @@ class strided_call {
   unsigned zmask = 0;               // vec4: arrays whose stride along x (bits 16..: along y) is zero
   size_t gx = 0, groups = 0;
   unsigned ltx = 0, tile = 64, quads = 4;
+  unsigned vq = 4;                  // vec4: elements a lane moves at a time (2 for 8-byte types, plain variant)
   GpuKernel *kernel = nullptr;
 
   void describe_arrays() {
@@ -1454,12 +1458,23 @@ class strided_call {
 
   void choose_vector_access() {
     // Four elements per lane when the layout allows it (see gen_strided_vec).
-    vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % 4 == 0 &&
+    // Without transposed operands and with 8-byte elements a lane moves two
+    // elements at a time, not four: its widest access is then 16 bytes, and a
+    // wavefront's accesses lie side by side (four doubles per lane are two
+    // 16-byte accesses 32 bytes apart from the neighbour's; kernel times,
+    // four / two per lane: a[:, :4096] + b[:, 4096:] of 8192 x 8192 doubles
+    // 144.1 / 121.6 us, the same of 64-bit integers 143.6 / 122.9, (4096, 8192)
+    // + (1, 8192) doubles as a strided call 117.5 / 81.7).
+    vq = 4;
+    if (tmask == 0 && env_ul("GPUARRAY_ELEMWISE_PAIRS", 1) != 0)
+      for (unsigned k = 0; k < na; k++)
+        if (elsz[k] == 8) vq = 2;
+    vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % vq == 0 &&
                 strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
     if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
     for (unsigned k = 0; k < na && vec4; k++) {
       if (elsz[k] > 8) { vec4 = false; break; }
-      const size_t q = 4 * elsz[k];
+      const size_t q = vq * elsz[k];
       unsigned l2 = 0;
       const GpuArray *v = nullptr;
       for (size_t i = 0; i < ge->args.size(); i++)
@@ -1496,7 +1511,7 @@ class strided_call {
   int choose_grid() {
     // launch geometry
     if (tmask == 0) {
-      size_t inner = vec4 ? dims[nd - 1] / 4 : dims[nd - 1];   // lanes needed along x
+      size_t inner = vec4 ? dims[nd - 1] / vq : dims[nd - 1];   // lanes needed along x
       // as many lanes along x as the inner extent needs (a power of two), the
       // rest of the 256 along the rows: 2^24 floats in rows of 3 took 191 us
       // with a floor of 16 lanes along x, 61 us without
@@ -1517,7 +1532,7 @@ class strided_call {
       if (vec4) {
         size_t widest = 1;
         for (unsigned k = 0; k < na; k++) widest = std::max(widest, elsz[k]);
-        quads = widest >= 4 ? 1 : (unsigned)(4 / widest);
+        quads = vq * widest >= 16 ? 1 : (unsigned)(16 / (vq * widest));
         const size_t fill = (size_t)ga_hip_numprocs(ctx) * 8;
         const size_t g1 = ((inner + quads * tx - 1) / (quads * tx)) * ((rows + ty - 1) / ty);
         if (g1 > fill && g1 <= 2 * fill) quads = std::min(4u, quads * 2);
@@ -1593,14 +1608,14 @@ class strided_call {
 
   int get_kernel() {
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads);
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
@@ -1718,13 +1733,15 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // chunks per lane; 7 as 4, every array in neither mask taken as constant along x;
   // 8 as 4, every array that is not staged through LDS taken as constant along y
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
+  // 10: as 3 with one group of two elements per lane (8-byte types, no transposed operand)
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
   // (idx64 then carries the mask of those fetched a whole chunk at a time)
   if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
-                                                   : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u)
+                                                   : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u,
+                                                   strided == 10 ? 1 : 4, strided == 10 ? 2 : 4)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

@@ -381,6 +381,36 @@ def test_flat_kernel_with_a_narrow_side_takes_two_chunks_per_lane(ctx, n):
             assert not got[:off_out].any() and not got[off_out + n:].any()
 
 
+@pytest.mark.parametrize("pairs", ["1", "0"])
+def test_eight_byte_elements_in_views_move_two_per_lane(ctx, monkeypatch, pairs):
+    # doubles and 64-bit integers in views that are not dense: two elements per
+    # lane (inner extents that are a multiple of 2, not of 4, qualify), also
+    # next to narrower types; four per lane with the switch off
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_PAIRS", pairs)
+    monkeypatch.setenv("GPUARRAY_ELEMWISE_PERIODIC", "0")
+    rng = np.random.default_rng(23)
+    for rows, cols, width in ((130, 1002, 500), (67, 2052, 1026), (300, 516, 258), (33, 4100, 2048)):
+        a = rng.standard_normal((rows, cols))
+        b = rng.standard_normal((rows, cols))
+        r = rng.standard_normal((1, width)).astype(np.float32)
+        ga_, gb, gr = (gpuarray.array(v, context=ctx) for v in (a, b, r))
+        ge = ga.GpuElemwise(ctx, "o = a * b + r", [arg("a", "float64", read=True), arg("b", "float64", read=True),
+                                                   arg("r", "float32", read=True), arg("o", "float64", write=True)])
+        for lo in (0, 2, 1):                      # 16-byte boundary kept, kept, broken
+            out = gpuarray.zeros((rows, cols), "float64", context=ctx)
+            ge(ga_[:, lo:lo + width], gb[:, cols - width:], gr, out[:, lo:lo + width], broadcast=True)
+            want = np.zeros((rows, cols))
+            want[:, lo:lo + width] = a[:, lo:lo + width] * b[:, cols - width:] + r.astype(np.float64)
+            assert np.array_equal(np.asarray(out), want), (rows, cols, width, lo)
+        i = rng.integers(-2**40, 2**40, size=(rows, cols))
+        gi = gpuarray.array(i, context=ctx)
+        gk = ga.GpuElemwise(ctx, "o = a - b", [arg("a", "int64", read=True), arg("b", "int64", read=True),
+                                               arg("o", "int64", write=True)])
+        out = gpuarray.zeros((rows, width), "int64", context=ctx)
+        gk(gi[:, :width], gi[:, cols - width:], out)
+        assert np.array_equal(np.asarray(out), i[:, :width] - i[:, cols - width:])
+
+
 def test_inplace_and_multiple_outputs(ctx):
     rng = np.random.default_rng(10)
     x = rng.normal(size=(257, 33)).astype(np.float32)
