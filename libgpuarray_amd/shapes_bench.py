@@ -81,6 +81,9 @@ def elemwise_cases():
          [("a", f, (8192, 16384), lambda b: b[:, ::2]), ("b", f, (8192, 8192), None)], (8192, 8192), f),
         ("a[:, 1:-1] * 2, 8192 x 8192", "o = a * 2.0f", [("a", f, (8192, 8194), lambda b: b[:, 1:-1])], (8192, 8192), f),
         ("a[1:-1, :] * 2, 8192 x 8192", "o = a * 2.0f", [("a", f, (8194, 8192), lambda b: b[1:-1, :])], (8192, 8192), f),
+        ("a[:, :4096] + b[:, 4096:], 8192 x 8192 doubles", "o = a + b",
+         [("a", d, (8192, 8192), lambda b: b[:, :4096]), ("b", d, (8192, 8192), lambda b: b[:, 4096:])], (8192, 4096), d),
+        ("a.T + b, 4096 x 4096 doubles", "o = a + b", [("a", d, (4096, 4096), T(1, 0)), ("b", d, (4096, 4096), None)], (4096, 4096), d),
         ("a.T + b, 8192 x 8192", "o = a + b", [("a", f, (8192, 8192), T(1, 0)), ("b", f, (8192, 8192), None)], (8192, 8192), f),
         ("transpose (0, 2, 1) of (64, 1024, 1024)", "o = a", [("a", f, (64, 1024, 1024), T(0, 2, 1))], (64, 1024, 1024), f),
         ("transpose (1, 0, 2) of (1024, 64, 1024)", "o = a", [("a", f, (1024, 64, 1024), T(1, 0, 2))], (64, 1024, 1024), f),
