@@ -393,14 +393,17 @@ def test_eight_byte_elements_in_views_move_two_per_lane(ctx, monkeypatch, pairs)
         a = rng.standard_normal((rows, cols))
         b = rng.standard_normal((rows, cols))
         r = rng.standard_normal((1, width)).astype(np.float32)
-        ga_, gb, gr = (gpuarray.array(v, context=ctx) for v in (a, b, r))
-        ge = ga.GpuElemwise(ctx, "o = a * b + r", [arg("a", "float64", read=True), arg("b", "float64", read=True),
-                                                   arg("r", "float32", read=True), arg("o", "float64", write=True)])
+        c = rng.standard_normal((rows, 1))
+        ga_, gb, gr, gc = (gpuarray.array(v, context=ctx) for v in (a, b, r, c))
+        ge = ga.GpuElemwise(ctx, "o = (a * b + r) - c",
+                            [arg("a", "float64", read=True), arg("b", "float64", read=True),
+                             arg("r", "float32", read=True), arg("c", "float64", read=True),
+                             arg("o", "float64", write=True)])
         for lo in (0, 2, 1):                      # 16-byte boundary kept, kept, broken
             out = gpuarray.zeros((rows, cols), "float64", context=ctx)
-            ge(ga_[:, lo:lo + width], gb[:, cols - width:], gr, out[:, lo:lo + width], broadcast=True)
+            ge(ga_[:, lo:lo + width], gb[:, cols - width:], gr, gc, out[:, lo:lo + width], broadcast=True)
             want = np.zeros((rows, cols))
-            want[:, lo:lo + width] = a[:, lo:lo + width] * b[:, cols - width:] + r.astype(np.float64)
+            want[:, lo:lo + width] = (a[:, lo:lo + width] * b[:, cols - width:] + r.astype(np.float64)) - c
             assert np.array_equal(np.asarray(out), want), (rows, cols, width, lo)
         i = rng.integers(-2**40, 2**40, size=(rows, cols))
         gi = gpuarray.array(i, context=ctx)
