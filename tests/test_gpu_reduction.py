@@ -354,6 +354,35 @@ def test_all_value_ops_on_layouts(layout, ctx):
         assert np.array_equal(np.asarray(gi), np_maxandargmax(v, axes)[1]), dt
 
 
+@pytest.mark.parametrize("axes", [(0, 2), (1,), (2,), (0, 1, 2)])
+def test_float16_on_stepped_views(ctx, axes):
+    """float16 through the stride-2 view of the layouts above (the reference
+    refuses float16 sums, pygpu/reduction.py:156-160: NumPy on float64 is the
+    only expected value; min/max and their indices are exact)."""
+    rng = np.random.default_rng(77)
+    base = rng.uniform(-4, 4, (16, 64, 256)).astype(np.float16)
+    base[3, 5, 10] = base[3, 5, 200] = np.float16(4.5)          # a tie on a stepped row
+    for view in (lambda b: b[:, :, ::2], lambda b: b[::-1, :, ::-3]):
+        v = view(base)
+        g, _ = to_gpu_view(v, ctx)
+        x64 = v.astype(np.float64)
+        want, mag = x64.sum(axis=axes), np.abs(x64).sum(axis=axes)
+        got32 = np.asarray(R.sum(g, axis=axes, dtype="float32"))
+        assert got32.dtype == np.float32
+        assert np.allclose(got32, want, rtol=1e-2)               # the stated bound for fp16 inputs
+        assert_sum_close(got32, want, mag, cancel=1e-2)          # what fp32 accumulation achieves
+        got16 = np.asarray(R.sum(g, axis=axes))
+        assert got16.dtype == np.float16 and np.array_equal(got16, got32.astype(np.float16))
+        assert np.array_equal(np.asarray(R.max(g, axis=axes)), v.max(axis=axes))
+        assert np.array_equal(np.asarray(R.min(g, axis=axes)), v.min(axis=axes))
+        for name in ("max", "min"):
+            wm, wa = np_maxandargmax(v, list(axes), name)
+            gv, gi = R._arg_reduce(g, name + "andarg" + name, list(axes), True)
+            assert np.array_equal(np.asarray(gv), wm) and np.array_equal(np.asarray(gi), wa), name
+        assert np.array_equal(np.asarray(R.any(g, axis=axes)), v.any(axis=axes))
+        assert np.array_equal(np.asarray(R.all(g, axis=axes)), v.all(axis=axes))
+
+
 def test_integer_invariants(ctx):
     # exact in any order: permuting the data or reducing axis by axis gives
     # the same integers
@@ -438,6 +467,76 @@ def test_config3b_full_sum_2p28(ctx):
     assert float(np.asarray(R.sum(ones))) == float(n)          # exact: all partials are integers
     v, i = R.maxandargmax(g)
     assert float(np.asarray(v)) == float(x.max()) and int(np.asarray(i)) == int(x.argmax())
+
+
+def test_config4_maxandargmax_logits(ctx, oracle):
+    """BASELINE configuration 4 at its stated shape: maxandargmax over the last
+    axis of (65536, 1000) normal(0, 2) floats, 5 % of the rows with their
+    maximum copied into one to three other columns.  Through the C entry point
+    (reference tests/check_reduction.c:85-160 checks it against a CPU loop)."""
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 2, (65536, 1000)).astype(np.float32)
+    rows = rng.choice(65536, 3277, replace=False)              # 5 % of the rows get duplicated maxima
+    for r in rows:
+        cols = rng.choice(1000, int(rng.integers(1, 4)), replace=False)
+        x[r, cols] = x[r].max()
+    g = gpuarray.array(x, context=ctx)
+    gmax = gpuarray.empty((65536,), "float32", context=ctx)
+    garg = gpuarray.empty((65536,), "uint64", context=ctx)
+    arr = (C.c_uint * 1)(1)
+    assert lib.GpuArray_maxandargmax(gmax._ptr(), garg._ptr(), g._ptr(), 1, arr) == 0
+    got_m, got_a = np.asarray(gmax), np.asarray(garg).astype(np.int64)
+    assert np.array_equal(got_m, x.max(axis=1))
+    assert np.array_equal(got_a, x.argmax(axis=1))             # NumPy: first index on ties
+    # the rows really hold ties, and the first of them is what came back
+    tied = (x[rows] == x[rows].max(axis=1, keepdims=True)).sum(axis=1)
+    assert (tied >= 2).sum() >= 3200     # (a drawn column can be the maximum's own)
+    wm, wa = oracle.maxandargmax(x[rows[:512]], [1])           # the reference's scan on tied rows
+    assert np.array_equal(got_m[rows[:512]], wm) and np.array_equal(got_a[rows[:512]], wa)
+    # the Python-level entry point takes the same kernels
+    v, i = R.maxandargmax(g, axis=1)
+    assert np.array_equal(np.asarray(v), got_m) and np.array_equal(np.asarray(i), got_a)
+
+
+def test_config5_mixed_dtypes_strided(ctx, oracle):
+    """BASELINE configuration 5 at its stated shape: a (256, 512, 1024) array
+    taken with a step of 2 along the last axis; fp16 summed over axes (0, 2)
+    into fp32, int32 summed over axis 1, uint8 any / all over axis 2
+    (reference pattern: pygpu/tests/test_reduction.py:86-110)."""
+    shape = (256, 512, 1024)
+    rng = np.random.default_rng(5)
+    h = rng.uniform(-4, 4, shape).astype(np.float16)
+    gh = gpuarray.array(h, context=ctx)[:, :, ::2]
+    assert gh.shape == (256, 512, 512) and gh.strides == (1048576, 2048, 4)
+    got = np.asarray(R.sum(gh, axis=(0, 2), dtype="float32"))
+    want = h[:, :, ::2].astype(np.float64).sum(axis=(0, 2))
+    assert got.dtype == np.float32 and np.allclose(got, want, rtol=1e-2)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-2)
+    del gh, h
+
+    rng = np.random.default_rng(6)
+    i32 = rng.integers(-1000, 1001, shape, dtype=np.int32)
+    gi = gpuarray.array(i32, context=ctx)[:, :, ::2]
+    got = np.asarray(R.sum(gi, axis=1))
+    assert got.dtype == np.int64 and np.array_equal(got, i32[:, :, ::2].sum(axis=1))
+    got32 = np.asarray(R.sum(gi, axis=1, dtype="int32"))
+    assert np.array_equal(got32, i32[:, :, ::2].sum(axis=1, dtype=np.int32))
+    chk = oracle.reduk("sum", i32[:4, :, ::2], [1], "int64", ls=64)
+    assert np.array_equal(got[:4], chk)
+    del gi, i32
+
+    rng = np.random.default_rng(7)
+    u8 = (rng.random(shape) < 1e-4).astype(np.uint8)
+    gu = gpuarray.array(u8, context=ctx)[:, :, ::2]
+    any_, all_ = np.asarray(R.any(gu, axis=2)), np.asarray(R.all(gu, axis=2))
+    assert any_.dtype == np.bool_ and np.array_equal(any_, u8[:, :, ::2].any(axis=2))
+    assert np.array_equal(all_, u8[:, :, ::2].all(axis=2)) and not all_.any()
+    assert 0 < any_.sum() < any_.size                          # the test data exercises both answers
+    chk_any = oracle.reduk("any", u8[:2, :, ::2], [2], "bool", ls=64)
+    assert np.array_equal(any_[:2], chk_any.astype(bool))
+    ones = gpuarray.array(np.ones((8, 16, 64), np.uint8), context=ctx)[:, :, ::2]
+    assert np.asarray(R.all(ones, axis=2)).all()
+
 
 # ---- reduced dims with outer ones side by side, several outputs per lane ----------
 
