@@ -53,6 +53,11 @@ typedef int (*ga_hip_kernel_times_fn)(gpucontext *ctx, float *out, unsigned int 
  * the first launch): ties a measurement to the generated kernel it was made
  * on. */
 typedef unsigned long long (*ga_hip_last_launch_hash_fn)(gpucontext *ctx);
+/* "hip_reload_tuning": the planners' tuning knobs (environment variables
+ * GPUARRAY_<NAME>, numbers) are read once, when a context is made, and looked
+ * up in the context's table from then on; this reads the environment into
+ * that table again.  For tests and sweeps that change a knob between calls. */
+typedef int (*ga_hip_reload_tuning_fn)(gpucontext *ctx);
 /* "hip_take1_source": kernel text of GpuArray_take1 for result/source/index
  * typecodes and `tnd` collapsed trailing dims; chunks != 0: the variant that
  * moves dense aligned rows as 16-byte chunks. */

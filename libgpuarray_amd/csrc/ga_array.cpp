@@ -891,7 +891,7 @@ int GpuArray_take1(GpuArray *a, const GpuArray *v, const GpuArray *i, int check_
   // against this one: rows of 64 floats 139 -> 91 us, of 32 floats 344 -> 92,
   // of 16 floats 684 -> 139, of 8 floats 466 -> 225; from 128 floats on both
   // take 90 to 91 us.
-  const bool short_rows = chunks && n1e <= env_ul("GPUARRAY_TAKE1_SHORT_ROWS", 128);
+  const bool short_rows = chunks && n1e <= TUNE(ga_hip_tuning(ctx), TAKE1_SHORT_ROWS, 128);
   // lanes per row: a power of two, each lane moves up to four elements
   unsigned int lsh = 0;
   while (lsh < 8 && ((size_t)(short_rows ? 1 : 4) << lsh) < n1e) lsh++;

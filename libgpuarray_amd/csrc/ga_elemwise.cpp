@@ -1037,6 +1037,7 @@ struct flat_periodic {
 // array k's first element in its buffer.
 int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
               const flat_periodic *pi = nullptr) {
+  const ga_tuning *tn = ga_hip_tuning(ge->ctx);
   unsigned l = 0;
   int err;
   unsigned int vec_ok = (ge->vec > 1 || ge->unroll > 1) ? 1u : 0u, head = ~0u;
@@ -1064,7 +1065,7 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
   unsigned int vec_arg = vec_ok ? 1u + head : 0u;
   for (size_t q = 0; vec_ok && q < heads.size(); q++)
     if (heads[q] != head && heads[q] != ~0u) vec_arg |= 1u << (8 + q);
-  if (!env_ul("GPUARRAY_ELEMWISE_MIXED_ALIGN", 1) && (vec_arg >> 8)) vec_arg = 0;
+  if (!TUNE(tn, ELEMWISE_MIXED_ALIGN, 1) && (vec_arg >> 8)) vec_arg = 0;
   if (vec_arg == 0) vec_ok = 0;
 
   // Grid: one lane per chunk (or per element) up to a fixed number of groups
@@ -1076,7 +1077,7 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
   // unit (the eight that fit cut down by asking for local memory nobody uses)
   // are slower as well: 8 groups 495 us, 6 507, 5 589, 4 592, 3 572, 2 635.
   const size_t ncu = ga_hip_numprocs(ge->ctx);
-  const size_t per_cu = env_ul("GPUARRAY_ELEMWISE_GROUPS_PER_CU", 2048);
+  const size_t per_cu = TUNE(tn, ELEMWISE_GROUPS_PER_CU, 2048);
   size_t cap = ncu * (per_cu ? per_cu : 2048);
   size_t units = vec_ok ? (n - head) / ge->vec + 1 : n;
   // A compute unit holds eight groups of this kernel at a time.  A grid of
@@ -1231,8 +1232,8 @@ inline size_t sabs(ssize_t v) { return v < 0 ? (size_t)(-v) : (size_t)v; }
 class strided_call {
  public:
   strided_call(GpuElemwise *ge_, void **args_, size_t n_, unsigned nd_)
-      : ge(ge_), ctx(ge_->ctx), args(args_), n(n_), nd(nd_), na(ge_->narray), dims(ge_->dims),
-        strs(ge_->strs) {}
+      : ge(ge_), ctx(ge_->ctx), tn(ga_hip_tuning(ge_->ctx)), args(args_), n(n_), nd(nd_),
+        na(ge_->narray), dims(ge_->dims), strs(ge_->strs) {}
 
   int run() {
     describe_arrays();
@@ -1254,6 +1255,7 @@ class strided_call {
  private:
   GpuElemwise *ge;
   gpucontext *ctx;
+  const ga_tuning *tn;
   void **args;
   const size_t n;
   unsigned nd;
@@ -1349,7 +1351,7 @@ class strided_call {
   // the faster one (87 against 92 us, channels last 79 against 94), and so it
   // is when nothing dense is read (outer product 49 against 79).
   bool dense_with_broadcast_operands(flat_periodic &pi) const {
-    const unsigned long mode = env_ul("GPUARRAY_ELEMWISE_PERIODIC", 1);
+    const unsigned long mode = TUNE(tn, ELEMWISE_PERIODIC, 1);
     if (mode == 0 || tmask != 0) return false;
     bool inner_constant = true, dense_read = false;
     const size_t V = ge->vec;
@@ -1384,7 +1386,7 @@ class strided_call {
           if (strs[k][j] % (ssize_t)cb != 0) whole_chunks = false;
       }
       if (whole_chunks) pi.pvmask |= 1u << k;
-      inner_constant = inner_constant && (sx == 0 || (whole_chunks && env_ul("GPUARRAY_ELEMWISE_PERIODIC_VEC", 1)));
+      inner_constant = inner_constant && (sx == 0 || (whole_chunks && TUNE(tn, ELEMWISE_PERIODIC_VEC, 1)));
       pi.pmask |= 1u << k;
       for (unsigned j = 0; j < nd; j++) pi.ps[k][3 - nd + j] = strs[k][j];
     }
@@ -1466,10 +1468,10 @@ class strided_call {
     // 144.1 / 121.6 us, the same of 64-bit integers 143.6 / 122.9, (4096, 8192)
     // + (1, 8192) doubles as a strided call 117.5 / 81.7).
     vq = 4;
-    if (tmask == 0 && env_ul("GPUARRAY_ELEMWISE_PAIRS", 1) != 0)
+    if (tmask == 0 && TUNE(tn, ELEMWISE_PAIRS, 1) != 0)
       for (unsigned k = 0; k < na; k++)
         if (elsz[k] == 8) vq = 2;
-    vec4 = env_ul("GPUARRAY_ELEMWISE_VEC4", 1) != 0 && dims[nd - 1] % vq == 0 &&
+    vec4 = TUNE(tn, ELEMWISE_VEC4, 1) != 0 && dims[nd - 1] % vq == 0 &&
                 strs[outk][nd - 1] == (ssize_t)elsz[outk] && na <= 31;
     if (vec4 && tmask && dims[nd - 2] % 4 != 0) vec4 = false;
     for (unsigned k = 0; k < na && vec4; k++) {
@@ -1489,10 +1491,10 @@ class strided_call {
         if (!aligned) vec4 = false;          // a transposed operand must be vector-accessible
       } else if (aligned) {
         umask |= 1u << k;
-      } else if (strs[k][nd - 1] == 0 && env_ul("GPUARRAY_ELEMWISE_ZMASK", 1) != 0) {
+      } else if (strs[k][nd - 1] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) {
         zmask |= 1u << k;
       }
-      if (!tr && tmask && k < 16 && strs[k][nd - 2] == 0 && env_ul("GPUARRAY_ELEMWISE_ZMASK", 1) != 0)
+      if (!tr && tmask && k < 16 && strs[k][nd - 2] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0)
         zmask |= 1u << (16 + k);
     }
     if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
@@ -1504,7 +1506,7 @@ class strided_call {
           if (dims[j] > 1 && strs[k][j] == 0) once = false;
         if (once) ntmask |= 1u << k;
       }
-      ntmask &= (unsigned)env_ul("GPUARRAY_ELEMWISE_NT_MASK", 0xffffffffu);
+      ntmask &= (unsigned)TUNE(tn, ELEMWISE_NT_MASK, 0xffffffffu);
     }
   }
 
@@ -1537,7 +1539,7 @@ class strided_call {
         const size_t g1 = ((inner + quads * tx - 1) / (quads * tx)) * ((rows + ty - 1) / ty);
         if (g1 > fill && g1 <= 2 * fill) quads = std::min(4u, quads * 2);
         else if (g1 > 2 * fill && g1 <= 4 * fill) quads = 4;
-        const unsigned long forced = env_ul("GPUARRAY_ELEMWISE_QUADS", 0);
+        const unsigned long forced = TUNE(tn, ELEMWISE_QUADS, 0);
         if (forced == 1 || forced == 2 || forced == 4) quads = (unsigned)forced;
       }
       gx = (inner + quads * tx - 1) / (quads * tx);
@@ -1579,9 +1581,9 @@ class strided_call {
         // large against small tiles on smaller planes: 1536 x 1536 4.6 / 4.9 us,
         // 2048 x 2048 6.2 / 6.9, 16 planes of 512 x 512 6.0 / 6.6, 3072 x 3072
         // 15.3 / 14.8, 1024 x 1024 4.2 / 4.2
-        const size_t min128 = env_ul("GPUARRAY_ELEMWISE_TTILE_MIN", ga_hip_numprocs(ctx) / 2);
+        const size_t min128 = TUNE(tn, ELEMWISE_TTILE_MIN, ga_hip_numprocs(ctx) / 2);
         tile = (tiles128 >= min128 && lds128 <= 80 * 1024) ? 128 : 64;
-        const unsigned long ft = env_ul("GPUARRAY_ELEMWISE_TTILE", 0);
+        const unsigned long ft = TUNE(tn, ELEMWISE_TTILE, 0);
         if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
         const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
         bool aliasing = true;   // every pitch a power of two of 4 to 32 KiB
@@ -1592,8 +1594,8 @@ class strided_call {
           aliasing = (pitch & (pitch - 1)) == 0 && pitch >= 4096 && pitch <= 32768;
         }
         const unsigned long dflt = aliasing ? 0 : (tile == 128 ? 1 : (tiles >= 8192 ? 8 : 1));
-        ltx = (unsigned)env_ul("GPUARRAY_ELEMWISE_BAND", dflt) & 0xffffu;
-        if (ltx == 0) ltx |= ((unsigned)env_ul("GPUARRAY_ELEMWISE_PANEL", 0) & 0xffffu) << 16;
+        ltx = (unsigned)TUNE(tn, ELEMWISE_BAND, dflt) & 0xffffu;
+        if (ltx == 0) ltx |= ((unsigned)TUNE(tn, ELEMWISE_PANEL, 0) & 0xffffu) << 16;
       }
       gx = (dims[nd - 1] + tile - 1) / tile;
       size_t gy = (dims[nd - 2] + tile - 1) / tile;
@@ -1704,12 +1706,13 @@ static int ge_describe(GpuElemwise *ge, const char *preamble, const char *expr, 
     }
     ge->narrow_side = ge->narray <= 8 && ((any_in && in_quarter) || (out_narrow && (wide_in <= 1 || out_quarter)));
   }
-  ge->flat_forced = getenv("GPUARRAY_ELEMWISE_UNROLL") != nullptr || getenv("GPUARRAY_ELEMWISE_TILE") != nullptr;
-  ge->unroll = (unsigned)env_ul("GPUARRAY_ELEMWISE_UNROLL", ge->unroll);
+  const ga_tuning *tn = ga_hip_tuning(ge->ctx);
+  ge->flat_forced = tn->is_set(KNOB_ELEMWISE_UNROLL) || tn->is_set(KNOB_ELEMWISE_TILE);
+  ge->unroll = (unsigned)TUNE(tn, ELEMWISE_UNROLL, ge->unroll);
   if (ge->unroll < 1) ge->unroll = 1;
-  ge->tile = env_ul("GPUARRAY_ELEMWISE_TILE", 0) != 0;
-  ge->nontemporal = env_ul("GPUARRAY_ELEMWISE_NT", 1) != 0;
-  ge->flat_nt_mask = (unsigned)env_ul("GPUARRAY_ELEMWISE_FLAT_NT_MASK", 0xffffffffu);
+  ge->tile = TUNE(tn, ELEMWISE_TILE, 0) != 0;
+  ge->nontemporal = TUNE(tn, ELEMWISE_NT, 1) != 0;
+  ge->flat_nt_mask = (unsigned)TUNE(tn, ELEMWISE_FLAT_NT_MASK, 0xffffffffu);
   return GA_NO_ERROR;
 }
 

@@ -319,6 +319,7 @@ struct hip_context : _gpucontext {
   gpukernel *copy_kernel = nullptr;   // byte copy behind buffer_move
   gpukernel *fill_kernel = nullptr;   // byte fill behind buffer_memset
   bool stage_failed = false;
+  ga_tuning tuning;        // the planners' knobs, as read from the environment when the context was made
   ga_errrec errstore;
 };
 
@@ -478,6 +479,7 @@ gpucontext *hip_init(gpucontext_props *p) {
   memset(ctx->bin_id, 0, sizeof(ctx->bin_id));
   memcpy(ctx->tag, "hipctx ", 8);
   ctx->dev = dev;
+  ga_tuning_read(&ctx->tuning);
 
 #define INIT_TRY(call)                                   \
   do {                                                   \
@@ -516,7 +518,7 @@ gpucontext *hip_init(gpucontext_props *p) {
 #undef INIT_TRY
   // Every kernel is compiled for gfx950 (wave64, its DPP and LDS forms): say
   // so here rather than at the first module load on another ISA.
-  if (strcmp(ctx->bin_id, "gfx950") != 0 && env_ul("GPUARRAY_ALLOW_OTHER_ISA", 0) == 0) {
+  if (strcmp(ctx->bin_id, "gfx950") != 0 && TUNE(&ctx->tuning, ALLOW_OTHER_ISA, 0) == 0) {
     ga_err_fmt(ga_global_err, GA_DEVSUP_ERROR,
                "Device %d is %s; this library generates code for gfx950 (MI355X) only", dev, ctx->bin_id);
     ctx_destroy(ctx);
@@ -754,7 +756,7 @@ int hip_move(gpudata *dst, size_t dstoff, gpudata *src, size_t srcoff, size_t sz
   // device-to-device copy and 6.65 with the kernel above; 64 MiB 28.1 against
   // 23.8 us; 16 MiB 7.5 against 8.9 us, and below that no difference.
   const uintptr_t da = (uintptr_t)dst->devptr + dstoff, sa = (uintptr_t)src->devptr + srcoff;
-  if (sz >= env_ul("GPUARRAY_MOVE_KERNEL_MIN", 32u << 20) && (da - sa) % 16 == 0 &&
+  if (sz >= TUNE(&ctx->tuning, MOVE_KERNEL_MIN, 32u << 20) && (da - sa) % 16 == 0 &&
       !((HD(dst)->flags | HD(src)->flags) & BUF_HOSTMEM)) {
     if (ctx->copy_kernel == nullptr) {
       const char *strs[1] = {COPY_KERNEL_SRC};
@@ -851,7 +853,7 @@ int hip_memset(gpudata *dst, size_t dstoff, int data) {
   // replayed wrongly.  Otherwise the driver's fill, which is as fast (measured
   // on MI355X, 30 fills back to back: 1 GiB 161.7 us against 160.1 with this
   // kernel, 64 MiB 11.7 / 11.5, 16 MiB 5.2 / 4.7, 1 MiB 4.4 / 4.7).
-  if (ga_hip_capturing(dst->ctx) || n >= env_ul("GPUARRAY_FILL_KERNEL_MIN", ~0ul)) {
+  if (ga_hip_capturing(dst->ctx) || n >= TUNE(&ctx->tuning, FILL_KERNEL_MIN, ~0ul)) {
     if (ctx->fill_kernel == nullptr) {
       const char *strs[1] = {FILL_KERNEL_SRC};
       const int types[6] = {GA_BUFFER, GA_SIZE, GA_SIZE, GA_SIZE, GA_SIZE, GA_UINT};
@@ -1565,7 +1567,7 @@ int ext_event_record(gpucontext *c, unsigned int slot) {
   if ((err = enter(ctx)) != GA_NO_ERROR) return err;
   while (ctx->evpool.size() <= slot) {
     hipEvent_t e = nullptr;
-    HIP_TRY(ctx, hipEventCreateWithFlags(&e, (unsigned)env_ul("GPUARRAY_MARK_EVENT_FLAGS", hipEventDisableSystemFence)));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&e, (unsigned)TUNE(&ctx->tuning, MARK_EVENT_FLAGS, hipEventDisableSystemFence)));
     ctx->evpool.push_back(e);
   }
   HIP_TRY(ctx, hipEventRecord(ctx->evpool[slot], ctx->stream));
@@ -1621,6 +1623,11 @@ int ext_module_cache_stats(gpucontext *c, size_t out[4]) {
   return GA_NO_ERROR;
 }
 
+int ext_reload_tuning(gpucontext *c) {
+  ga_tuning_read(&HC(c)->tuning);
+  return GA_NO_ERROR;
+}
+
 struct ext_entry { const char *name; void *fn; };
 const ext_entry k_exts[] = {
     {"hip_get_stream", (void *)ext_get_stream},
@@ -1640,6 +1647,7 @@ const ext_entry k_exts[] = {
     {"hip_mapreduce_source", (void *)ga_mapreduce_gen_source},
     {"hip_module_cache_stats", (void *)ext_module_cache_stats},
     {"hip_take1_source", (void *)ga_take1_gen_source},
+    {"hip_reload_tuning", (void *)ext_reload_tuning},
 };
 
 }  // namespace
@@ -1716,6 +1724,33 @@ size_t ga_hip_readable_bytes(gpudata *b) {
 }
 
 unsigned int ga_hip_numprocs(gpucontext *c) { return HC(c)->numprocs; }
+const ga_tuning *ga_hip_tuning(gpucontext *c) { return c ? &HC(c)->tuning : ga_tuning_default(); }
+
+const ga_tuning *ga_tuning_default() {
+  static const ga_tuning t = [] { ga_tuning r; ga_tuning_read(&r); return r; }();
+  return &t;
+}
+
+void ga_tuning_read(ga_tuning *t) {
+  static const char *const names[GA_NKNOBS] = {
+#define X(name) "GPUARRAY_" #name,
+      GA_KNOBS(X)
+#undef X
+  };
+  for (unsigned k = 0; k < GA_NKNOBS; k++) {
+    const char *v = getenv(names[k]);
+    char *end = nullptr;
+    t->set[k] = false;
+    t->val[k] = 0;
+    if (v == nullptr || *v == 0) continue;
+    const unsigned long r = strtoul(v, &end, 10);
+    if (end == v) continue;   // not a number: as if unset
+    t->set[k] = true;
+    t->val[k] = r;
+  }
+  const char *fam = getenv("GPUARRAY_REDUX_FAMILY");
+  snprintf(t->redux_family, sizeof(t->redux_family), "%s", fam ? fam : "");
+}
 void **ga_hip_redux_cache_slot(gpucontext *c) { return &HC(c)->redux_cache; }
 void **ga_hip_take1_cache_slot(gpucontext *c) { return &HC(c)->take1_cache; }
 

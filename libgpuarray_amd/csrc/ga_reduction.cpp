@@ -213,6 +213,7 @@ bool packed_bytes(int tc, const variant_spec &vs) {
 // `gen` replaces its @RD_GENERATED@ mark.
 int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string &defs,
                      std::string &gen, ga_errrec *errrec) {
+  const ga_tuning *tn = ga_hip_tuning(gr->ctx);
   const op_info &info = gr->info;
   const rd_kind kind = info.kind;
   const bool minmax = kind == K_MIN || kind == K_MAX;
@@ -278,14 +279,14 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
     const bool bytes = K == 1 && !gr->mapped && gpuarray_get_elsize(stc) == 1 && (vs.vecmask & 1u) &&
                        (vs.V * vs.ES) % 4 == 0 && (vs.ES == 1 || vs.ES == 2 || vs.ES == 4) &&
                        (kind == K_SUM || kind == K_ANY || kind == K_ALL) && !valf &&
-                       env_ul("GPUARRAY_REDUX_FAST8", 1);
+                       TUNE(tn, REDUX_FAST8, 1);
     DEF("#define RD_FAST8 %d\n", bytes ? (stc == GA_BYTE ? 2 : 1) : 0);
     // redux_col, any / all over one-byte elements: the words of a lane's load
     // are or-ed whole (all: their zero-byte masks) and taken apart once at
     // the end.
     const unsigned cvn = vs.CV ? vs.CV : 1;
     const bool col_bytes = K == 1 && !gr->mapped && gpuarray_get_elsize(stc) == 1 && cvn % 4 == 0 &&
-                           (kind == K_ANY || kind == K_ALL) && env_ul("GPUARRAY_REDUX_FAST8", 1);
+                           (kind == K_ANY || kind == K_ALL) && TUNE(tn, REDUX_FAST8, 1);
     DEF("#define RD_COL_FAST8 %d\n", col_bytes ? 1 : 0);
   }
   {
@@ -298,7 +299,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
     // sums the same either way, the two-source dot product 162.5 / 168.7.
     bool touch = K == 1 || kind == K_MIN || kind == K_MAX || kind == K_PRODNZ ||
                  ((vs.opts >> 2) & 1u) || half_src;
-    touch = env_ul("GPUARRAY_REDUX_TOUCH", touch ? 1 : 0) != 0;
+    touch = TUNE(tn, REDUX_TOUCH, touch ? 1 : 0) != 0;
     DEF("#define RD_TOUCH_ROW %u\n", touch ? 1u : 0u);
   }
 #undef DEF
@@ -648,7 +649,7 @@ class reduction_call {
   reduction_call(GpuReduction *gr_, GpuArray *d0_, GpuArray *d1_, unsigned nd_, const size_t *dims_,
                  const std::vector<src_view> &srcs_, const std::vector<void *> &scalars_,
                  unsigned reduxLen_, const int *reduxList_, bool noalloc_ = false, size_t scratch_skip_ = 0)
-      : noalloc(noalloc_), scratch_skip(scratch_skip_), gr(gr_), ctx(gr_->ctx), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
+      : noalloc(noalloc_), scratch_skip(scratch_skip_), gr(gr_), ctx(gr_->ctx), tn(ga_hip_tuning(gr_->ctx)), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
         dims(dims_), srcs(srcs_), scalars(scalars_), reduxLen(reduxLen_), reduxList(reduxList_),
         kind(info.kind), minmax(kind == K_MIN || kind == K_MAX),
         logical(kind == K_ALL || kind == K_ANY),
@@ -686,6 +687,7 @@ class reduction_call {
   const size_t scratch_skip;
   GpuReduction *gr;
   gpucontext *ctx;
+  const ga_tuning *tn;
   const op_info &info;
   const unsigned K;                 // number of array sources
   GpuArray *d0, *d1;
@@ -890,9 +892,9 @@ class reduction_call {
     // after another kernel wrote it, as the second call of folded rows does, it
     // is slower, 7.6 -> 10.2 us.  Not taken.)
     {
-      const char *force = getenv("GPUARRAY_REDUX_FAMILY");
-      if (force && strcmp(force, "row") == 0) use_row = true;
-      if (force && strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
+      const char *force = tn->redux_family;
+      if (strcmp(force, "row") == 0) use_row = true;
+      if (strcmp(force, "col") == 0 && p.nf > 0) use_row = false;
     }
   }
 
@@ -940,7 +942,7 @@ class reduction_call {
         // for rows of 1024; element-aligned (misaligned) 16-byte loads were
         // tried first and ran slower than 4-byte loads on long rows.
         if (es == 1 && V < vmax && rin >= (int64_t)vmax && GpuArray_ISALIGNED(s0) &&
-            env_ul("GPUARRAY_REDUX_TAIL", 1)) {
+            TUNE(tn, REDUX_TAIL, 1)) {
           const size_t readable = ga_hip_readable_bytes(s0->data);
           const size_t end = ((size_t)last + (size_t)elsz[0] + 15) & ~(size_t)15;
           bool nonneg = true;   // the lowest address is the array's own start
@@ -981,17 +983,17 @@ class reduction_call {
     rin_sz = rin + (tail ? (int64_t)V - 1 : 0);
     G = (rin_sz <= (int64_t)64 * V * 8) ? 64 : 256;
     {
-      const unsigned long force = env_ul("GPUARRAY_REDUX_G", 0);
+      const unsigned long force = TUNE(tn, REDUX_G, 0);
       if (force == 64 || force == 256) G = (unsigned)force;
     }
     int64_t per_pass = (int64_t)G * V;
-    U = (unsigned)env_ul("GPUARRAY_REDUX_U", 8);
+    U = (unsigned)TUNE(tn, REDUX_U, 8);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 8;
     // Bytes a lane keeps in flight over all sources.  Measured on MI355X
     // (dot product of two 2^27-float vectors): 64 bytes per lane with 4 groups
     // per compute unit 162 us, 128 bytes with 2 groups 179 us; one source
     // keeps the 128 bytes its sweep found best.
-    const int64_t lane_bytes = (int64_t)env_ul("GPUARRAY_REDUX_LANE_BYTES", K > 1 ? 64 : 128);
+    const int64_t lane_bytes = (int64_t)TUNE(tn, REDUX_LANE_BYTES, K > 1 ? 64 : 128);
     while (U > 1 && (int64_t)U * V * ES * elsz_sum > lane_bytes) U /= 2;
     while (U > 1 && per_pass * (U / 2) >= rin_sz) U /= 2;
     int64_t outer = 1;
@@ -1005,7 +1007,7 @@ class reduction_call {
     // 5.8 / 5.5 and 6.8 / 6.0 / 5.5 us, sum 4.4 / 4.0 / 4.0 and 4.3 / 4.1 / 4.1;
     // 2^20 floats 7.4 / 7.3 / 7.9 (enough pieces as it is), 2^14 floats 4.7 / 5.0
     // / 5.5 (too short to be worth cutting at all).
-    if (env_ul("GPUARRAY_REDUX_U", 0) == 0 && rtotal >= 49152) {
+    if (TUNE(tn, REDUX_U, 0) == 0 && rtotal >= 49152) {
       const int64_t rowgroups_now = (nrows + 256 / G - 1) / (256 / G);
       auto pieces = [&](unsigned u) {
         const int64_t units_u = outer * ((rin_sz + per_pass * u - 1) / (per_pass * u));
@@ -1021,7 +1023,7 @@ class reduction_call {
     // of 512 stepped halves ran at 45.4 us with 64 lanes and two loads each,
     // 47.4 us with 32 lanes and two outer coordinates side by side.
     if (p.nr >= 2 && rtotal > 0 && G == 64 && rin_sz <= (int64_t)32 * V &&
-        env_ul("GPUARRAY_REDUX_LO", 1)) {
+        TUNE(tn, REDUX_LO, 1)) {
       const int64_t need = (rin_sz + (int64_t)V * 4 - 1) / ((int64_t)V * 4);
       unsigned LI = 1;
       while (LI < 64 && (int64_t)LI < need) LI *= 2;
@@ -1047,7 +1049,7 @@ class reduction_call {
     // loads outstanding (64 KB per unit), read at 6.9-7.1 TB/s; 16 such
     // groups per unit at 6.3, 64 at 5.8.  Narrow or strided loads carry fewer
     // bytes per lane, so they get proportionally more groups, up to 32.
-    int64_t per_cu = (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", 0);
+    int64_t per_cu = (int64_t)TUNE(tn, REDUX_GROUPS_PER_CU, 0);
     if (per_cu == 0) {
       const int64_t inflight = (int64_t)G * U * V * ES * elsz_sum;   // bytes per group
       // A kernel that does next to nothing per element - one source of floats
@@ -1064,9 +1066,9 @@ class reduction_call {
       bool light = K == 1 && !gr->mapped && !tail && !info.has_d1 &&
                    (info.kind == K_SUM || info.kind == K_PROD) &&
                    (stc0 == GA_FLOAT || stc0 == GA_DOUBLE) && acc_typecode(gr, d0_tc) == stc0;
-      if (!env_ul("GPUARRAY_REDUX_LIGHT", 1)) light = false;
-      const int64_t want = (int64_t)env_ul("GPUARRAY_REDUX_INFLIGHT", light ? 32768 : 65536);
-      const int64_t least = (int64_t)env_ul("GPUARRAY_REDUX_MIN_PER_CU", light ? 1 : 2);
+      if (!TUNE(tn, REDUX_LIGHT, 1)) light = false;
+      const int64_t want = (int64_t)TUNE(tn, REDUX_INFLIGHT, light ? 32768 : 65536);
+      const int64_t least = (int64_t)TUNE(tn, REDUX_MIN_PER_CU, light ? 1 : 2);
       per_cu = (want + inflight - 1) / inflight;
       if (per_cu < least) per_cu = least;
       if (per_cu > 32) per_cu = 32;
@@ -1074,7 +1076,7 @@ class reduction_call {
     const int64_t target = ncu * per_cu;
     if (rowgroups < target && p.units >= 8) {
       nsplit = (target + rowgroups - 1) / rowgroups;
-      const int64_t min_units = (int64_t)env_ul("GPUARRAY_REDUX_MIN_UNITS", 2);
+      const int64_t min_units = (int64_t)TUNE(tn, REDUX_MIN_UNITS, 2);
       if (nsplit > p.units / min_units) nsplit = p.units / min_units;
       if (nsplit > 65536) nsplit = 65536;
       if (nsplit < 1) nsplit = 1;
@@ -1090,7 +1092,7 @@ class reduction_call {
     // A wavefront takes RB rows at a time and issues their loads together:
     // a row that is a single load per lane would otherwise leave the
     // wavefront with one load in flight.
-    if (G == 64 && p.nsplit == 1 && p.units == 1 && p.nr <= 1 && env_ul("GPUARRAY_REDUX_WROWS", 1)) {
+    if (G == 64 && p.nsplit == 1 && p.units == 1 && p.nr <= 1 && TUNE(tn, REDUX_WROWS, 1)) {
       wrows = true;
       // Measured on MI355X: any() over 131072 rows of 512 stepped bytes 29.8 us
       // one row at a time, 24.8 us with batches of 4 and 8 rows per wavefront;
@@ -1119,7 +1121,7 @@ class reduction_call {
           while (l1 < 64 && (int64_t)l1 < need1) l1 *= 2;
           if (l1 <= 32) L = l1;
         }
-        const unsigned long force = env_ul("GPUARRAY_REDUX_L", 0);
+        const unsigned long force = TUNE(tn, REDUX_L, 0);
         if (force >= 1 && force <= 64 && (force & (force - 1)) == 0 &&
             (int64_t)force * V * 8 >= rin_sz)
           L = (unsigned)force;
@@ -1128,10 +1130,10 @@ class reduction_call {
           while (U < 8 && (int64_t)L * V * U < rin_sz) U *= 2;
         }
       }
-      RB = (unsigned)env_ul("GPUARRAY_REDUX_RB", L < 64 ? (U >= 4 ? 1 : 4 / U) : (U == 1 ? 4 : 1));
+      RB = (unsigned)TUNE(tn, REDUX_RB, L < 64 ? (U >= 4 ? 1 : 4 / U) : (U == 1 ? 4 : 1));
       if (RB != 1 && RB != 2 && RB != 4 && RB != 8) RB = 1;
       const int64_t per_batch = (int64_t)(64 / L) * RB;
-      int64_t rpw = (int64_t)env_ul("GPUARRAY_REDUX_RPW", (RB == 1 && L == 64) ? 1 : 2 * per_batch);
+      int64_t rpw = (int64_t)TUNE(tn, REDUX_RPW, (RB == 1 && L == 64) ? 1 : 2 * per_batch);
       if (rpw < 1) rpw = 1;
       p.upb = rpw;
       const int64_t waves = (nrows + rpw - 1) / rpw;
@@ -1153,11 +1155,10 @@ class reduction_call {
     // bytes, aligned) 89 / 100 against 95 / 121 us.
     if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] &&
         fsstr[0] == rin * elsz[0] && rin >= 2 &&
-        rin * elsz[0] <= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MAX_BYTES",
-                                         (rin * elsz[0]) % 16 != 0 ? 384 : (minmax ? 160 : 256)) &&
-        rin * elsz[0] > (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_BYTES", 16) &&
-        nrows >= (int64_t)env_ul("GPUARRAY_REDUX_SROWS_MIN_ROWS", 512) * ncu &&
-        GpuArray_ISALIGNED(srcs[0].a) && env_ul("GPUARRAY_REDUX_SROWS", 1)) {
+        rin * elsz[0] <= (int64_t)TUNE(tn, REDUX_SROWS_MAX_BYTES, (rin * elsz[0]) % 16 != 0 ? 384 : (minmax ? 160 : 256)) &&
+        rin * elsz[0] > (int64_t)TUNE(tn, REDUX_SROWS_MIN_BYTES, 16) &&
+        nrows >= (int64_t)TUNE(tn, REDUX_SROWS_MIN_ROWS, 512) * ncu &&
+        GpuArray_ISALIGNED(srcs[0].a) && TUNE(tn, REDUX_SROWS, 1)) {
       const GpuArray *s0 = srcs[0].a;
       const size_t readable = ga_hip_readable_bytes(s0->data);
       const size_t end = ((size_t)s0->offset + (size_t)(nrows * rin * elsz[0]) + 15) & ~(size_t)15;
@@ -1190,8 +1191,8 @@ class reduction_call {
     // there, 47.4 here; 16 floats 45 staged in LDS, 43 here).
     const int64_t rowb = rin * elsz[0];
     if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] && fsstr[0] == rowb &&
-        rin >= 2 && elsz[0] <= 8 && rowb <= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MAX_BYTES", 32) &&
-        nrows >= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MIN_ROWS", 16384) && env_ul("GPUARRAY_REDUX_TROWS", 1)) {
+        rin >= 2 && elsz[0] <= 8 && rowb <= (int64_t)TUNE(tn, REDUX_TROWS_MAX_BYTES, 32) &&
+        nrows >= (int64_t)TUNE(tn, REDUX_TROWS_MIN_ROWS, 16384) && TUNE(tn, REDUX_TROWS, 1)) {
       const GpuArray *s0 = srcs[0].a;
       const size_t readable = ga_hip_readable_bytes(s0->data);
       const size_t end = ((size_t)s0->offset + (size_t)(nrows * rowb) + 15) & ~(size_t)15;
@@ -1205,10 +1206,10 @@ class reduction_call {
       // (2^27 bytes, any: 21.3 against 24.7 us); one- and two-byte elements
       // in rows of 2, 4, 8 or 32 bytes come here (2^27 bytes in rows of 2 /
       // 4 / 32, max: 104.6 / 39.9 / 28.2 us there, 29.3 / 28.4 / 21.9 here).
-      const unsigned long direct = env_ul("GPUARRAY_REDUX_TROWS_DIRECT", 1);
+      const unsigned long direct = TUNE(tn, REDUX_TROWS_DIRECT, 1);
       // more than two chunks per lane are handed out through LDS, 4 KiB per chunk
       if (((uintptr_t)s0->data->devptr + (size_t)s0->offset) % 16 == 0 && end <= readable &&
-          chunks <= (int64_t)env_ul("GPUARRAY_REDUX_TROWS_MAX_CHUNKS", 7) &&
+          chunks <= (int64_t)TUNE(tn, REDUX_TROWS_MAX_CHUNKS, 7) &&
           (chunks > 2 || direct == 2 || (direct == 1 && elsz[0] <= 2 && rowb != 16))) {
         trows = true;
         srows = wrows = false;
@@ -1231,7 +1232,7 @@ class reduction_call {
 
   void col_geometry() {
     const int64_t fin = p.fdim[p.nf - 1];
-    const unsigned long cy_forced = env_ul("GPUARRAY_REDUX_COL_ROWS", 0);
+    const unsigned long cy_forced = TUNE(tn, REDUX_COL_ROWS, 0);
     // Lane rows of a group: 8 (32 lanes along the free dim) when the reduced
     // range is long, else 4.  Measured on MI355X with 4 / 8 / 16: per-channel
     // sum of (64, 56, 56, 256) floats 45.2 / 40.9 / 39.7 us, max over the
@@ -1248,7 +1249,7 @@ class reduction_call {
     // (256, 128, 2048), 8 KiB apart, 42.8 / 44.7 and (512, 128, 1024) 40.5 / 44.2.
     int64_t rpitch = 0;
     for (unsigned q = 0; q < K && p.nr > 0; q++) rpitch = std::max(rpitch, iabs(rsstr[q * RD_MAXD + p.nr - 1]));
-    const bool far_apart = rpitch >= (int64_t)env_ul("GPUARRAY_REDUX_COL_FAR", 12288) && rtotal >= 32;
+    const bool far_apart = rpitch >= (int64_t)TUNE(tn, REDUX_COL_FAR, 12288) && rtotal >= 32;
     CY = (cy_forced == 1 || cy_forced == 2 || cy_forced == 4 || cy_forced == 8 || cy_forced == 16)
              ? (unsigned)cy_forced : (rtotal >= 512 || far_apart ? 8 : 4);
     int64_t CX = 256 / CY;   // lanes along the free dim
@@ -1258,7 +1259,7 @@ class reduction_call {
     {
       unsigned cv = (unsigned)(16 / elsz_max);
       if (info.has_d1 && cv > 8) cv = 8;   // (value, index) pairs meet in LDS: 32 KiB per group at 8
-      if (cv > (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16)) cv = (unsigned)env_ul("GPUARRAY_REDUX_COL_CVMAX", 16);
+      if (cv > (unsigned)TUNE(tn, REDUX_COL_CVMAX, 16)) cv = (unsigned)TUNE(tn, REDUX_COL_CVMAX, 16);
       for (unsigned q = 0; q < K; q++)
         if (fsstr[q * RD_MAXD + p.nf - 1] != elsz[q]) cv = 1;
       while (cv > 1) {
@@ -1273,7 +1274,7 @@ class reduction_call {
         if (ok) break;
         cv /= 2;
       }
-      if (!env_ul("GPUARRAY_REDUX_COLVEC", 1)) cv = 1;
+      if (!TUNE(tn, REDUX_COLVEC, 1)) cv = 1;
       // Splitting the reduced range costs a second pass (sum over the middle
       // axis of 256x512x512 floats: 54 us unsplit with one output per lane,
       // 64 us split in two with four), so when the widest load leaves too
@@ -1318,9 +1319,9 @@ class reduction_call {
     const int stc0 = gr->args[gr->arrays[0]].tc;
     const bool light = K == 1 && !gr->mapped && !info.has_d1 && (info.kind == K_SUM || info.kind == K_PROD) &&
                        (stc0 == GA_FLOAT || stc0 == GA_DOUBLE) && acc_typecode(gr, d0_tc) == stc0 &&
-                       env_ul("GPUARRAY_REDUX_LIGHT", 1) != 0 &&
+                       TUNE(tn, REDUX_LIGHT, 1) != 0 &&
                        scratch_skip == 0;   // folded rows measured better with three: (2^24, 3) 38.8 against 43.4 us
-    const int64_t target = ncu * (int64_t)env_ul("GPUARRAY_REDUX_GROUPS_PER_CU", CV > 1 ? (light ? 2 : 3) : 8);
+    const int64_t target = ncu * (int64_t)TUNE(tn, REDUX_GROUPS_PER_CU, CV > 1 ? (light ? 2 : 3) : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
       if (nsplit > rtotal / 64) nsplit = rtotal / 64;
@@ -1337,10 +1338,10 @@ class reduction_call {
     // outputs that second pass would have too few lanes (1000 outputs over
     // 256 splits: 51.6 -> 65.9 us), and they stay output-major for the
     // wavefront-per-output pass.
-    const int64_t many = (int64_t)env_ul("GPUARRAY_REDUX_SPLIT_MAJOR_MIN", 4096);
+    const int64_t many = (int64_t)TUNE(tn, REDUX_SPLIT_MAJOR_MIN, 4096);
     p.split_major = (nsplit > 1 && nrows >= many) ? 1 : 0;
     groups = (size_t)(base_groups * nsplit);
-    U = (unsigned)env_ul("GPUARRAY_REDUX_COL_U", 4);
+    U = (unsigned)TUNE(tn, REDUX_COL_U, 4);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 4;
   }
 
@@ -1349,8 +1350,8 @@ class reduction_call {
       return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Reduction needs more groups than one launch has");
 
     // bit 0: streaming loads; bit 1: interleaved splits (single reduced dim only)
-    unsigned opts = env_ul("GPUARRAY_REDUX_NT", 1) ? 1u : 0u;
-    if (use_row && p.nr == 1 && p.nsplit > 1 && env_ul("GPUARRAY_REDUX_INTERLEAVE", 1)) opts |= 2u;
+    unsigned opts = TUNE(tn, REDUX_NT, 1) ? 1u : 0u;
+    if (use_row && p.nr == 1 && p.nsplit > 1 && TUNE(tn, REDUX_INTERLEAVE, 1)) opts |= 2u;
     if (use_row && tail) opts |= 4u;   // bit 2: element-aligned vector loads with a ragged end
     variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
                        use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
@@ -1412,7 +1413,7 @@ class reduction_call {
     gpudata *done = nullptr;
     if (p.nsplit > 1 && !noalloc) {
       const size_t counters = use_row ? (size_t)nrows : groups / (size_t)p.nsplit;
-      const size_t fused_max = (size_t)ncu * env_ul("GPUARRAY_REDUX_FUSED", 1);   // 0 turns it off
+      const size_t fused_max = (size_t)ncu * TUNE(tn, REDUX_FUSED, 1);   // 0 turns it off
       // Beyond one group per compute unit the single launch pays again once a
       // piece is long: the wait for the acknowledgement is then a small part of
       // a group's life, and the second launch (3 to 4 us) is saved.  Measured,
@@ -1436,13 +1437,13 @@ class reduction_call {
       // position) (4096, 256) 14.9 / 10.6, (16384, 64) 25.5 / 12.6, (1024, 1024)
       // 11.9 / 10.4.
       if (fuse && !use_row &&
-          p.nsplit > (int)env_ul("GPUARRAY_REDUX_FUSED_COL_FEW", carries_index ? 16 : 128))
+          p.nsplit > (int)TUNE(tn, REDUX_FUSED_COL_FEW, carries_index ? 16 : 128))
         fuse = false;
       if (!fuse && fused_max > 0 && groups > fused_max) {
         const double piece_bytes = (double)nrows * (double)rtotal * (double)elsz_sum / (double)groups;
-        fuse = use_row ? piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_PIECE", 384u << 10)
-                       : (!carries_index && p.nsplit <= (int)env_ul("GPUARRAY_REDUX_FUSED_COL_SPLITS", 16) &&
-                          piece_bytes >= (double)env_ul("GPUARRAY_REDUX_FUSED_COL_PIECE", 128u << 10));
+        fuse = use_row ? piece_bytes >= (double)TUNE(tn, REDUX_FUSED_PIECE, 384u << 10)
+                       : (!carries_index && p.nsplit <= (int)TUNE(tn, REDUX_FUSED_COL_SPLITS, 16) &&
+                          piece_bytes >= (double)TUNE(tn, REDUX_FUSED_COL_PIECE, 128u << 10));
       }
       if (fuse && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
           (done = ga_hip_redux_counters(ctx)) != nullptr) {
@@ -1622,7 +1623,8 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
                      const int *reduxList, bool *done) {
   *done = false;
   gpucontext *ctx = gr->ctx;
-  if (env_ul("GPUARRAY_REDUX_FOLD", 1) == 0 || gr->mapped || d0 == nullptr || reduxLen == 0 ||
+  const ga_tuning *tn = ga_hip_tuning(ctx);
+  if (TUNE(tn, REDUX_FOLD, 1) == 0 || gr->mapped || d0 == nullptr || reduxLen == 0 ||
       reduxLen >= s0->nd || !GpuArray_IS_C_CONTIGUOUS(s0) || GpuArray_context(d0) != ctx)
     return GA_NO_ERROR;
   const rd_kind kind = gr->info.kind;
@@ -1640,7 +1642,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   size_t R = 1, F = 1;
   for (unsigned j = 0; j < s0->nd; j++) (j < reduxLen ? R : F) *= s0->dimensions[j];
   const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
-  if (R * rowb < env_ul("GPUARRAY_REDUX_FOLD_MIN_BYTES", 4u << 20) || F == 0) return GA_NO_ERROR;
+  if (R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20) || F == 0) return GA_NO_ERROR;
   if (rowb % 16 == 0 && rowb >= 256) return GA_NO_ERROR;
   // d0 must have the kept dims' shape (the launch below checks the rest)
   if (d0->nd != s0->nd - reduxLen) return GA_NO_ERROR;
@@ -1657,7 +1659,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   // 35.5 / 31.6 us (three launches / two), (2^24, 3) 38.9 / 34.1, (65536, 1001)
   // 49.3 / 46.1, (4096, 4096, 4) over two axes 50.1 / 43.4, (2^20, 17) 20.2 / 16.9.
   size_t m = 0;
-  const size_t widest = env_ul("GPUARRAY_REDUX_FOLD_BYTES", 262144);
+  const size_t widest = TUNE(tn, REDUX_FOLD_BYTES, 262144);
   for (size_t width = widest; m == 0 && width >= 4096; width /= 8)
     for (size_t t = (width + m0 * rowb - 1) / (m0 * rowb); t * m0 <= 65536; t++)
       if (R % (t * m0) == 0 && R / (t * m0) >= 64) { m = t * m0; break; }

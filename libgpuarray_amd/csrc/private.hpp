@@ -24,6 +24,10 @@
 #include <gpuarray/types.h>
 #include <gpuarray/util.h>
 
+#include "ga_tuning.hpp"
+// A knob of the context's tuning table `t`, `dflt` when it is not set.
+#define TUNE(t, NAME, dflt) ((t)->get(KNOB_##NAME, (unsigned long)(dflt)))
+
 // ---- error record (reference src/util/error.h:10-22) ----------------------
 #define GA_ERROR_MSGBUF_LEN 1020
 struct ga_errrec {
@@ -135,15 +139,6 @@ extern const char ga_reduce_kernels_src[];
 // Grow-only scratch buffer owned by the context (partials of two-pass
 // reductions).  Work on a context is in stream order, so one buffer is
 // shared by consecutive calls.
-// A tuning knob from the environment: its value as a number, `dflt` when unset or not one.
-inline unsigned long env_ul(const char *name, unsigned long dflt) {
-  const char *v = getenv(name);
-  if (v == nullptr || *v == 0) return dflt;
-  char *end = nullptr;
-  unsigned long r = strtoul(v, &end, 10);
-  return end == v ? dflt : r;
-}
-
 gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
 // Counters of split reductions that finish in one launch: a buffer of
 // ga_hip_redux_counters_max 32-bit zeros, made on first use; every kernel

@@ -220,6 +220,12 @@ class GpuContext(object):
             raise GpuArrayException("kernel timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
         return list(buf[:min(n, limit)])
 
+    def reload_tuning(self):
+        """Read the GPUARRAY_* tuning knobs from the environment again (a
+        context reads them once, when it is made)."""
+        fn = _lib.extension("hip_reload_tuning", C.c_int, [C.c_void_p])
+        check(fn(self.ctx), self.ctx)
+
     def sync(self):
         # any buffer of the context syncs the one stream; use the error buffer
         eb = C.c_void_p()

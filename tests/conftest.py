@@ -27,3 +27,30 @@ def ctx():
 def oracle():
     from oracle import oracle as O
     return O
+
+
+@pytest.fixture
+def knobs(ctx):
+    """Sets tuning knobs for one test: knobs(REDUX_FUSED=0) puts
+    GPUARRAY_REDUX_FUSED=0 into the environment and has the context read its
+    tuning table again (a context reads the environment once, when it is made);
+    None removes a knob.  Everything is put back, and read back, afterwards."""
+    saved = {}
+
+    def set_knobs(**values):
+        for short, value in values.items():
+            name = "GPUARRAY_" + short
+            saved.setdefault(name, os.environ.get(name))
+            if value is None:
+                os.environ.pop(name, None)
+            else:
+                os.environ[name] = str(value)
+        ctx.reload_tuning()
+
+    yield set_knobs
+    for name, old in saved.items():
+        if old is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = old
+    ctx.reload_tuning()

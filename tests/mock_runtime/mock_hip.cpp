@@ -12,6 +12,8 @@
 extern "C" {
 // calls that allocate or free memory on the device or pinned host side, or load code onto the device
 unsigned long mock_allocating_calls = 0;
+// kernel launches so far (a planner's choice between one launch and two shows here)
+unsigned long mock_kernel_launches = 0;
 hipError_t hipGetDeviceCount(int *n) { *n = 1; return hipSuccess; }
 hipError_t hipSetDevice(int) { return hipSuccess; }
 hipError_t hipGetDevice(int *d) { *d = 0; return hipSuccess; }
@@ -51,7 +53,7 @@ hipError_t hipModuleLoadData(hipModule_t *m, const void *) { mock_allocating_cal
 hipError_t hipModuleUnload(hipModule_t m) { free(m); return hipSuccess; }
 hipError_t hipModuleGetFunction(hipFunction_t *f, hipModule_t, const char *) { *f = (hipFunction_t)0x30; return hipSuccess; }
 hipError_t hipFuncGetAttribute(int *v, hipFunction_attribute, hipFunction_t) { *v = 1024; return hipSuccess; }
-hipError_t hipExtModuleLaunchKernel(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, size_t, hipStream_t, void **, void **, hipEvent_t, hipEvent_t, uint32_t) { return hipSuccess; }
+hipError_t hipExtModuleLaunchKernel(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, size_t, hipStream_t, void **, void **, hipEvent_t, hipEvent_t, uint32_t) { mock_kernel_launches++; return hipSuccess; }
 hipError_t hipModuleLaunchKernel(hipFunction_t, unsigned gx, unsigned, unsigned, unsigned bx, unsigned, unsigned, unsigned, hipStream_t, void **params, void **) {
-  (void)gx; (void)bx; (void)params; return hipSuccess; }
+  (void)gx; (void)bx; (void)params; mock_kernel_launches++; return hipSuccess; }
 }

@@ -95,12 +95,12 @@ def test_buffer_read_write_move(ctx):           # check_buffer.c:95-177
         lib.gpudata_release(b)
 
 
-def test_large_moves_take_the_copy_kernel(ctx, monkeypatch):
+def test_large_moves_take_the_copy_kernel(ctx, knobs):
     """buffer_move copies large ranges with the library's own kernel when source
     and destination sit equally far from a 16-byte boundary (here from the
     first byte on), with the driver's copy otherwise: same bytes either way,
     nothing outside the range, and a cleared array struct is refused."""
-    monkeypatch.setenv("GPUARRAY_MOVE_KERNEL_MIN", "1")
+    knobs(MOVE_KERNEL_MIN=1)
     rng = np.random.default_rng(31)
     total = (1 << 20) + 200
     h = rng.integers(0, 256, total).astype(np.uint8)

@@ -382,12 +382,11 @@ def test_flat_kernel_with_a_narrow_side_takes_two_chunks_per_lane(ctx, n):
 
 
 @pytest.mark.parametrize("pairs", ["1", "0"])
-def test_eight_byte_elements_in_views_move_two_per_lane(ctx, monkeypatch, pairs):
+def test_eight_byte_elements_in_views_move_two_per_lane(ctx, knobs, pairs):
     # doubles and 64-bit integers in views that are not dense: two elements per
     # lane (inner extents that are a multiple of 2, not of 4, qualify), also
     # next to narrower types; four per lane with the switch off
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_PAIRS", pairs)
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_PERIODIC", "0")
+    knobs(ELEMWISE_PAIRS=pairs, ELEMWISE_PERIODIC=0)
     rng = np.random.default_rng(23)
     for rows, cols, width in ((130, 1002, 500), (67, 2052, 1026), (300, 516, 258), (33, 4100, 2048)):
         a = rng.standard_normal((rows, cols))
@@ -518,15 +517,13 @@ def test_linearity_at_full_size(ctx):
 
 @pytest.mark.parametrize("tile,band,panel", [(64, 0, 0), (64, 0, 3), (64, 1, 0), (64, 3, 0), (64, 8, 0),
                                              (128, 0, 0), (128, 0, 2), (128, 1, 0), (128, 2, 0), (128, 5, 0)])
-def test_transposed_tiles_and_bands(ctx, monkeypatch, tile, band, panel):
+def test_transposed_tiles_and_bands(ctx, knobs, tile, band, panel):
     """Every tile size and tile order of the transposed kernels (bands of
     `band` tile rows; 0: diagonals, within panels of `panel` tile columns), on
     extents that leave ragged tiles, a partial last band and a narrower last
     panel, with one and with two transposed operands, a transposed result,
     several planes and 8-byte elements: bit-exact against NumPy."""
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_TTILE", str(tile))
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_BAND", str(band))
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_PANEL", str(panel))
+    knobs(ELEMWISE_TTILE=tile, ELEMWISE_BAND=band, ELEMWISE_PANEL=panel)
     rng = np.random.default_rng(40 + tile + band)
     f32 = "float32"
     k2 = ga.GpuElemwise(ctx, "out = a + b*c", [arg("a", f32, read=True), arg("b", f32, read=True),
@@ -630,7 +627,7 @@ def test_math_library_functions_match_numpy(ctx):
 
 
 @pytest.mark.parametrize("mode", ["1", "2", "0"])
-def test_dense_arrays_with_broadcast_operands(ctx, oracle, monkeypatch, mode):
+def test_dense_arrays_with_broadcast_operands(ctx, oracle, knobs, mode):
     """Dense arrays combined with operands broadcast along some dims take the
     flat kernel, which reads the broadcast operands through the coordinates of
     the flat index (mode 1: where four elements per lane are not possible;
@@ -638,7 +635,7 @@ def test_dense_arrays_with_broadcast_operands(ctx, oracle, monkeypatch, mode):
     multiples of 4, a misaligned first element, a strided column, several
     broadcast operands, mixed types, 8- and 1-byte elements; bit for bit
     against NumPy."""
-    monkeypatch.setenv("GPUARRAY_ELEMWISE_PERIODIC", mode)
+    knobs(ELEMWISE_PERIODIC=mode)
     rng = np.random.default_rng(91)
     f32 = "float32"
     k3 = ga.GpuElemwise(ctx, "o = a * b + c", [arg("a", f32, read=True), arg("b", f32, read=True),

@@ -73,7 +73,7 @@ def test_random_elementwise_matches_numpy(ctx, seed):
 
 
 @pytest.mark.parametrize("seed", range(3))
-def test_large_planes_and_flat_size_classes_match_numpy(ctx, monkeypatch, seed):
+def test_large_planes_and_flat_size_classes_match_numpy(ctx, knobs, seed):
     """The paths whose launch shape depends on size: transposed operands over
     planes of up to 14 x 14 large tiles with ragged edges (tile size, band
     height, diagonal order and panel width drawn per case, or left to the
@@ -95,16 +95,14 @@ def test_large_planes_and_flat_size_classes_match_numpy(ctx, monkeypatch, seed):
         return rng.integers(0, 11, size=shape).astype(dt)
 
     for case in range(10):
-        for knob in ("GPUARRAY_ELEMWISE_TTILE", "GPUARRAY_ELEMWISE_BAND", "GPUARRAY_ELEMWISE_PANEL"):
-            monkeypatch.delenv(knob, raising=False)
+        knobs(ELEMWISE_TTILE=None, ELEMWISE_BAND=None, ELEMWISE_PANEL=None)
         dt = str(rng.choice(["float32", "float32", "float64", "int16"]))
         mode = int(rng.integers(0, 4))
         if mode <= 1:
             if rng.random() < 0.5:
-                monkeypatch.setenv("GPUARRAY_ELEMWISE_TTILE", str(rng.choice([64, 128])))
+                knobs(ELEMWISE_TTILE=rng.choice([64, 128]))
             if rng.random() < 0.6:
-                monkeypatch.setenv("GPUARRAY_ELEMWISE_BAND", str(rng.choice([0, 0, 1, 2, 8])))
-                monkeypatch.setenv("GPUARRAY_ELEMWISE_PANEL", str(rng.choice([0, 0, 1, 3, 16])))
+                knobs(ELEMWISE_BAND=rng.choice([0, 0, 1, 2, 8]), ELEMWISE_PANEL=rng.choice([0, 0, 1, 3, 16]))
             ny = int(rng.integers(1, 14)) * 128 + int(rng.choice([0, 0, 4, 8, 60, 100]))
             nx = int(rng.integers(1, 14)) * 128 + int(rng.choice([0, 0, 4, 12, 64, 124]))
             planes = int(rng.choice([1, 1, 1, 2, 5]))

@@ -139,10 +139,12 @@ def test_scratch_that_a_graph_recorded_is_never_handed_out_again(monkeypatch):
         # an eager split reduction whose partials outgrow that buffer: 8 pieces
         # for each of 65536 columns, 6 MiB
         monkeypatch.setenv("GPUARRAY_REDUX_GROUPS_PER_CU", "256")
+        ctx.reload_tuning()
         wide = gpuarray.zeros((512, 65536), f32, context=ctx)
         cols = gpuarray.empty((65536,), f32, context=ctx)
         rsum(wide, [0], d0=cols)
         monkeypatch.delenv("GPUARRAY_REDUX_GROUPS_PER_CU")
+        ctx.reload_tuning()
         ctx.sync()
         # arrays made now take whatever blocks the cache has free
         fresh = [gpuarray.array(np.full(1 << 16, 5.0, np.float32), context=ctx) for _ in range(32)]

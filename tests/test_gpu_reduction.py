@@ -576,12 +576,12 @@ def test_short_rows_share_a_wavefront(ctx, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64", "int16"])
-def test_short_contiguous_rows_staged_in_lds(ctx, dtype, monkeypatch):
+def test_short_contiguous_rows_staged_in_lds(ctx, dtype, knobs):
     """Many short rows lying one after the other take the kernel that stages a
     group's rows in LDS (here from 1000 rows on, so that the case stays
     small): every row length up to the limit, starts off the 16-byte boundary,
     a last group that is not full, ties, and NaN / signed zero placement."""
-    monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")
+    knobs(REDUX_SROWS_MIN_ROWS=1)
     rng = np.random.default_rng(54)
     item = np.dtype(dtype).itemsize
     # up to 256 bytes per row, 384 where the row length is no multiple of 16 bytes
@@ -633,7 +633,7 @@ def test_short_contiguous_rows_staged_in_lds(ctx, dtype, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64", "int16", "int64"])
-def test_tiny_contiguous_rows_walked_in_registers(ctx, dtype, monkeypatch):
+def test_tiny_contiguous_rows_walked_in_registers(ctx, dtype, knobs):
     """Rows of at most 32 bytes lying one after the other, the first on a
     16-byte boundary, take the kernel that keeps a lane's rows in registers
     (here from one row on and for every row length it can take, so that the
@@ -641,8 +641,7 @@ def test_tiny_contiguous_rows_walked_in_registers(ctx, dtype, monkeypatch):
     last lane whose run of rows is cut short, a view that starts inside its
     buffer (on a boundary, and off one: that one falls back), every
     operation, ties, NaN and signed zero placement."""
-    monkeypatch.setenv("GPUARRAY_REDUX_TROWS_MIN_ROWS", "1")
-    monkeypatch.setenv("GPUARRAY_REDUX_TROWS_DIRECT", "2")
+    knobs(REDUX_TROWS_MIN_ROWS=1, REDUX_TROWS_DIRECT=2)
     rng = np.random.default_rng(57)
     item = np.dtype(dtype).itemsize
     lengths = [n for n in (2, 3, 4, 5, 6, 7, 8, 12, 14, 16, 32) if n * item <= 32]
@@ -707,13 +706,12 @@ def test_tiny_contiguous_rows_walked_in_registers(ctx, dtype, monkeypatch):
 
 @pytest.mark.parametrize("dtype", ["float32", "float64", "float16"])
 @pytest.mark.parametrize("staged", [0, 1])
-def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, monkeypatch):
+def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, knobs):
     """The NaN rule of the sequential scan (a NaN stays only when it is the
     first element) in the kernels that take it from their own registers: rows
     sharing a wavefront in every lane geometry, rows shifted to a load
     boundary, one row per wavefront, rows staged in LDS."""
-    monkeypatch.setenv("GPUARRAY_REDUX_SROWS", str(staged))
-    monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")
+    knobs(REDUX_SROWS=staged, REDUX_SROWS_MIN_ROWS=1)
     rng = np.random.default_rng(55)
     for n in (2, 3, 4, 8, 15, 16, 33, 64, 100, 129, 250, 513, 1000, 1001):
         rows = 131
@@ -902,7 +900,7 @@ def test_column_scans_keep_the_first_of_equals(ctx, dtype):
                     assert np.array_equal(plain.view(bits), want_v.astype(dt).view(bits)), (name[:3], shape)
 
 
-def test_split_reductions_finish_in_one_launch(ctx, monkeypatch):
+def test_split_reductions_finish_in_one_launch(ctx, knobs):
     """A reduction whose outputs are cut into pieces: the piece that finishes
     last combines the partials in the same launch (a counter per output, or per
     tile of outputs of the column kernel, that the launch leaves at zero).
@@ -953,9 +951,9 @@ def test_split_reductions_finish_in_one_launch(ctx, monkeypatch):
     g, _ = to_gpu_view(host, ctx)
     gf, _ = to_gpu_view(flat, ctx)
     one = (np.asarray(R.sum(g, axis=0, dtype="int64")), np.asarray(R.maxandargmax(gf)[1]))
-    monkeypatch.setenv("GPUARRAY_REDUX_FUSED", "0")
+    knobs(REDUX_FUSED=0)
     two = (np.asarray(R.sum(g, axis=0, dtype="int64")), np.asarray(R.maxandargmax(gf)[1]))
-    monkeypatch.delenv("GPUARRAY_REDUX_FUSED")
+    knobs(REDUX_FUSED=None)
     assert np.array_equal(one[0], two[0]) and np.array_equal(one[0], host.sum(axis=0, dtype=np.int64))
     assert one[1] == two[1] == flat.argmax()
     # NaN in the first position of a cut row stays; later NaNs are passed over
@@ -1030,14 +1028,14 @@ def test_stepped_eight_byte_rows_are_planned(ctx):
 
 
 @pytest.mark.parametrize("fold", ["1", "0"])
-def test_leading_dims_with_short_kept_rows_are_folded(ctx, monkeypatch, fold):
+def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, fold):
     """Reducing the leading dims of a dense array whose kept rows are short or
     off a 16-byte boundary goes through folded rows (every m rows taken as one,
     then the m copies of each output combined): every operation that may be
     regrouped, integer and floating types, one and two leading dims, row
     counts with and without a usable divisor, a strided destination; against
     NumPy, and with folding switched off."""
-    monkeypatch.setenv("GPUARRAY_REDUX_FOLD", fold)
+    knobs(REDUX_FOLD=fold)
     rng = np.random.default_rng(71)
     cases = (((1 << 20, 10), (0,)), ((1 << 21, 3), (0,)), ((16384, 1001), (0,)),
              ((1024, 1024, 4), (0, 1)), ((1048573, 5), (0,)), ((3 * (1 << 18), 6, 2), (0,)),

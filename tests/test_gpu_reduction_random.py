@@ -45,8 +45,8 @@ def draw(rng):
 
 
 @pytest.mark.parametrize("seed", range(6))
-def test_random_reductions_match_numpy(ctx, seed, monkeypatch):
-    monkeypatch.setenv("GPUARRAY_REDUX_SROWS_MIN_ROWS", "1")    # staged rows at test sizes too
+def test_random_reductions_match_numpy(ctx, seed, knobs):
+    knobs(REDUX_SROWS_MIN_ROWS=1)    # staged rows at test sizes too
     rng = np.random.default_rng(1000 + seed)
     for case in range(10):
         dt, view, axes = draw(rng)

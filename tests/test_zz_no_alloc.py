@@ -87,7 +87,7 @@ def test_noalloc_matches_call_on_two_calls_in_a_row(ctx, case):
             assert np.array_equal(g, h.max(axis=ax)) and np.array_equal(gi, h.argmax(axis=ax)), (name, k)
 
 
-def test_noalloc_refuses_what_it_would_have_to_allocate_for(ctx, monkeypatch):
+def test_noalloc_refuses_what_it_would_have_to_allocate_for(ctx, knobs):
     # kernels not built yet: building loads a code object, which allocates
     op = ga.GpuReduction(ctx, "prod", "float64")
     x = ga.zeros((1000, 37), "float64", context=ctx)
@@ -104,12 +104,12 @@ def test_noalloc_refuses_what_it_would_have_to_allocate_for(ctx, monkeypatch):
     op = ga.GpuReduction(ctx, "sum", "float32")
     big = ga.zeros((512, 65536), "float32", context=ctx)
     res = ga.empty((65536,), "float32", context=ctx)
-    monkeypatch.setenv("GPUARRAY_REDUX_GROUPS_PER_CU", "256")
+    knobs(REDUX_GROUPS_PER_CU=256)
     op(big, [0], d0=res)
     with pytest.raises(_lib.GpuArrayException, match="static scratch array holds") as e:
         op(big, [0], d0=res, noalloc=True)
     assert e.value.code == _lib.GA_XLARGE_ERROR
-    monkeypatch.delenv("GPUARRAY_REDUX_GROUPS_PER_CU")
+    knobs(REDUX_GROUPS_PER_CU=None)
     op(big, [0], d0=res)
     op(big, [0], d0=res, noalloc=True)      # the default split fits
     assert not np.asarray(res).any()
