@@ -40,13 +40,16 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 # HBM bytes per call measured with the profiler's byte counters (two runs per
 # configuration, FETCH_SIZE then WRITE_SIZE, each scaled by what the same
 # counter reads for a copy kernel of known size).  Counters cannot be read
-# from inside this process, so the figures are carried here, each with the
-# hash of the kernel text it was measured on (hip_last_launch_hash): when the
-# kernel being timed is generated differently, the figure does not describe
-# it any more and the line says "traffic": null.  The runs and the arithmetic
-# are in profiles/hbm_traffic_all_configs.md.
+# from inside this process, so the figures are carried here (they are NOT
+# measured by the run that prints them: "traffic_source" says so), each with
+# the hashes of the texts of all the kernels of one call, in launch order
+# (hip_kernel_hashes): when any kernel being timed is generated differently,
+# the figure does not describe the call any more and the line says
+# "traffic": null.  The runs and the arithmetic are in
+# profiles/hbm_traffic_all_configs.md.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_all_configs.md (earlier rocprofv3 --pmc runs, matched by kernel text hash)"
 MEASURED_TRAFFIC = {
-    # name: (kernel text hash, HBM bytes per call)
+    # name: (kernel text hashes of one call joined by "+", HBM bytes per call)
     "C1_elemwise_2^24": ("712fba8f0b8a6108", 201255162),
     "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134354659),
     "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536638854),
@@ -65,13 +68,14 @@ MEASURED_TRAFFIC = {
 }
 
 
-def traffic_for(name, kernel_hash):
+def traffic_for(name, kernel_hashes):
+    """kernel_hashes: the text hashes of one call's launches, in order."""
     rec = MEASURED_TRAFFIC.get(name)
     if rec is None:
         return None, "no counter run recorded for this configuration"
-    if rec[0] != kernel_hash:
-        return None, ("the counter run was made on kernel text %s; the kernel timed here is %s"
-                      % (rec[0], kernel_hash))
+    now = "+".join(kernel_hashes)
+    if rec[0] != now:
+        return None, "the counter run was made on kernel texts %s; the kernels timed here are %s" % (rec[0], now)
     return rec[1], None
 
 
@@ -93,7 +97,8 @@ def time_calls(ctx, fn, iters=30, warm=5):
 def time_kernels(ctx, fn, iters=30, warm=3):
     """Median microseconds one call's kernels run on the device: every launch
     carries its own start and stop event, the durations of the launches of one
-    call are added up.  Returns (us, launches per call)."""
+    call are added up.  Returns (us, launches per call, text hashes of one
+    call's kernels in launch order)."""
     for _ in range(warm):
         fn(0)
     ctx.sync()
@@ -101,10 +106,11 @@ def time_kernels(ctx, fn, iters=30, warm=3):
     for i in range(iters):
         fn(i)
     ms = np.array(ctx.kernel_times())
+    hashes = ctx.kernel_hashes()
     ctx.kernel_timing(False)
     per = max(len(ms) // iters, 1)
     per_call = ms[:per * iters].reshape(iters, per).sum(axis=1)
-    return float(np.median(per_call)) * 1e3, per
+    return float(np.median(per_call)) * 1e3, per, hashes[-per:]
 
 
 def time_stream(ctx, fn, iters=40, warm=5):
@@ -202,16 +208,22 @@ def cfg_c3a(ctx, ga, R):
 
 
 def cfg_c4(ctx, ga, R):
-    L = np.random.default_rng(4).normal(0, 2, (65536, 1000)).astype(np.float32)
+    rng = np.random.default_rng(4)
+    L = rng.normal(0, 2, (65536, 1000)).astype(np.float32)
+    tied_rows = rng.choice(65536, 3277, replace=False)      # 5 % of the rows: the maximum copied
+    for r in tied_rows:                                     # into one to three other columns
+        L[r, rng.choice(1000, int(rng.integers(1, 4)), replace=False)] = L[r].max()
     op4 = ga.GpuReduction(ctx, "maxandargmax", f32)
     sets = [(ga.array(L, context=ctx), ga.empty((65536,), f32, context=ctx),
              ga.empty((65536,), "int64", context=ctx)) for _ in range(ROT)]
 
     def check():
-        wm, wa = L.max(axis=1), L.argmax(axis=1)
-        return all(np.array_equal(np.asarray(s[1]), wm) and np.array_equal(np.asarray(s[2]), wa)
-                   for s in sets)
+        wm, wa = L.max(axis=1), L.argmax(axis=1)              # NumPy: first index on ties
+        ties = int(((L[tied_rows] == wm[tied_rows, None]).sum(axis=1) >= 2).sum())
+        return ties >= 3200 and all(np.array_equal(np.asarray(s[1]), wm) and
+                                    np.array_equal(np.asarray(s[2]), wa) for s in sets)
     return {"bytes": 65536 * 1000 * 4 + 65536 * 12, "sets": ROT, "check": check,
+            "note": "3277 rows hold their maximum two to four times; the first index is the answer",
             "call": lambda i: op4(sets[i % ROT][0], [1], d0=sets[i % ROT][1], d1=sets[i % ROT][2]),
             "numpy": lambda: (L.max(axis=1), L.argmax(axis=1))}
 
@@ -230,7 +242,8 @@ def cfg_c5_f16(ctx, ga, R):
 
     def check():
         want = H[:, :, ::2].astype(np.float64).sum(axis=(0, 2))
-        return bool(np.all(np.abs(np.asarray(o5) - want) <= 1e-2 * np.abs(want) + 1e-2 * 4 * 256))
+        # the bound of the GPU test of this configuration (tests/test_gpu_reduction.py)
+        return bool(np.allclose(np.asarray(o5), want, rtol=1e-5, atol=1e-2))
     return {"bytes": 256 * 512 * 512 * 2 + 2048, "call": lambda i: oph(gh, [0, 2], d0=o5), "sets": 1,
             "check": check, "numpy": lambda: H[:, :, ::2].sum(axis=(0, 2), dtype=np.float32),
             "numpy_reps": 1, "note": C5_NOTE}
@@ -336,15 +349,14 @@ STEP_MODES = ("step", "elem", "sum", "copy")
 def measure_config(ctx, name, cfg):
     nbytes, call, sets = cfg["bytes"], cfg["call"], cfg["sets"]
     call(0)
-    khash = ctx.last_launch_hash()
     cold = time_calls(ctx, call)
-    kern, launches = time_kernels(ctx, call)
+    kern, launches, khashes = time_kernels(ctx, call)
     e = {"algorithmic_bytes": nbytes,
          "us_per_call_cold": round(cold, 2), "GBps_cold": round(nbytes / cold / 1e3, 1),
          "frac_cold": round(nbytes / cold / 1e3 / HBM_PEAK_GBS, 4),
          "kernel_us_cold": round(kern, 2), "GBps_kernel_cold": round(nbytes / kern / 1e3, 1),
          "frac_kernel_cold": round(nbytes / kern / 1e3 / HBM_PEAK_GBS, 4),
-         "launches_per_call": launches, "kernel_text_hash": khash}
+         "launches_per_call": launches, "kernel_text_hashes": "+".join(khashes)}
     if sets > 1:
         warm = time_calls(ctx, lambda i: call(0))
         e["us_per_call_warm"] = round(warm, 2)
@@ -352,10 +364,11 @@ def measure_config(ctx, name, cfg):
     b2b = time_stream(ctx, call)
     e["us_per_call_back_to_back"] = round(b2b, 2)
     e["GBps_back_to_back"] = round(nbytes / b2b / 1e3, 1)
-    traffic, why = traffic_for(name, khash)
+    traffic, why = traffic_for(name, khashes)
     e["traffic"] = traffic
     if traffic is not None:
         e["traffic_over_algorithmic"] = round(traffic / nbytes, 4)
+        e["traffic_source"] = TRAFFIC_SOURCE
     else:
         e["traffic_note"] = why
     if "check" in cfg:
@@ -523,17 +536,27 @@ def run_reference_kernels(device_type, cases):
                    "GpuKernel_sched's geometry by oracle/opencl_runner.py; wall time per launch over "
                    "several launches between two clFinish"}
     try:
-        r = subprocess.run([sys.executable, "-m", "oracle.opencl_runner", "--device-type", device_type] + cases,
-                           cwd=ROOT, capture_output=True, text=True, timeout=240)
+        # a session of its own, so that at the time limit the whole group goes
+        # (the child and anything it started), not only the direct child
+        proc = subprocess.Popen([sys.executable, "-m", "oracle.opencl_runner", "--device-type", device_type] + cases,
+                                cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                                start_new_session=True)
+        try:
+            stdout, stderr = proc.communicate(timeout=240)
+        except subprocess.TimeoutExpired:
+            import signal
+            os.killpg(proc.pid, signal.SIGKILL)
+            stdout, stderr = proc.communicate()
+            res["error"] = "time limit (240 s): the child's process group was killed"
         rows = []
-        for line in r.stdout.splitlines():
+        for line in stdout.splitlines():
             try:
                 rows.append(json.loads(line))
             except ValueError:
                 pass
         res["cases"] = rows
-        if r.returncode != 0:
-            res["error"] = (r.stderr or "")[-400:]
+        if proc.returncode != 0 and "error" not in res:
+            res["error"] = (stderr or "")[-400:]
     except Exception as e:
         res["error"] = repr(e)
     return res
@@ -576,16 +599,15 @@ def main():
         for i in range(W):
             cfg["call"](i)
         ctx.sync()
-        khash = ctx.last_launch_hash()
         ctx.mark(0)
         for i in range(K):
             cfg["call"](i)
         ctx.mark(1)
         us = ctx.elapsed(0, 1) * 1e3 / K
-        kern, launches = time_kernels(ctx, cfg["call"], iters=K, warm=0)
+        kern, launches, khashes = time_kernels(ctx, cfg["call"], iters=K, warm=0)
         print(json.dumps({"only": args.only, "calls": K, "warmup_calls": W, "us_per_call_back_to_back": round(us, 2),
                           "kernel_us": round(kern, 2), "launches_per_call": launches,
-                          "algorithmic_bytes_per_call": cfg["bytes"], "kernel_text_hash": khash,
+                          "algorithmic_bytes_per_call": cfg["bytes"], "kernel_text_hashes": "+".join(khashes),
                           "GBps": round(cfg["bytes"] / us / 1e3, 1),
                           "GBps_kernel": round(cfg["bytes"] / kern / 1e3, 1)}))
         return
@@ -623,7 +645,6 @@ def main():
             ctx.mark(3 * i)
         if only in ("step", "elem"):
             elem(a_, b_, c_)
-            hashes["elem"] = ctx.last_launch_hash()
         elif only == "copy":
             copy(a_, c_)
         if i is not None:
@@ -654,11 +675,11 @@ def main():
         # profiler run: report the one kernel that was launched and stop
         ms = elem_ms if only in ("elem", "copy") else sum_ms
         nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
-        kern, launches = time_kernels(ctx, lambda i: step(), iters=K, warm=0)
+        kern, launches, khashes = time_kernels(ctx, lambda i: step(), iters=K, warm=0)
         print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
                           "kernel_us": round(kern, 2), "launches_per_call": launches,
                           "bytes_per_launch": nbytes, "buffer_sets": len(sets),
-                          "kernel_text_hash": ctx.last_launch_hash(),
+                          "kernel_text_hashes": "+".join(khashes),
                           "GBps": round(nbytes / (float(ms.mean()) * 1e-3) / 1e9, 1),
                           "GBps_kernel": round(nbytes / kern / 1e3, 1)}))
         return
@@ -670,14 +691,42 @@ def main():
     for _ in range(KT):
         elem(a, b, c)
     elem_kernel_ms = np.array(ctx.kernel_times())
-    ctx.kernel_timing(True)
-    for _ in range(KT):
-        summ(x, [0], d0=s)
-    sum_kernel_ms = np.array(ctx.kernel_times())
+    hashes["elem"] = ctx.kernel_hashes()[-1:]
+
+    def timed_sums():
+        ctx.kernel_timing(True)
+        for _ in range(KT):
+            summ(x, [0], d0=s)
+        ms = np.array(ctx.kernel_times())
+        per = max(len(ms) // KT, 1)
+        return ms[:per * KT].reshape(KT, per).sum(axis=1), per, ctx.kernel_hashes()[-per:]
+    sum_kernel_ms, sum_launches, hashes["sum"] = timed_sums()
     ctx.kernel_timing(False)
-    sum_launches = max(len(sum_kernel_ms) // KT, 1)
-    sum_kernel_ms = sum_kernel_ms[:sum_launches * KT].reshape(KT, sum_launches).sum(axis=1)
-    hashes["sum"] = ctx.last_launch_hash()
+    sum_result = float(np.asarray(s))
+
+    # The same full sum finished by a second launch (GPUARRAY_REDUX_FUSED=0):
+    # the form that rests on nothing but stream order between two kernels.
+    old_fused = os.environ.get("GPUARRAY_REDUX_FUSED")
+    os.environ["GPUARRAY_REDUX_FUSED"] = "0"
+    ctx.reload_tuning()
+    try:
+        for _ in range(3):
+            summ(x, [0], d0=s)
+        ctx.sync()
+        for i in range(KT):
+            ctx.mark(2 * i)
+            summ(x, [0], d0=s)
+            ctx.mark(2 * i + 1)
+        two_marks_ms = np.array([ctx.elapsed(2 * i, 2 * i + 1) for i in range(KT)])
+        two_kernel_ms, two_launches, _ = timed_sums()
+        ctx.kernel_timing(False)
+        two_result = float(np.asarray(s))
+    finally:
+        if old_fused is None:
+            del os.environ["GPUARRAY_REDUX_FUSED"]
+        else:
+            os.environ["GPUARRAY_REDUX_FUSED"] = old_fused
+        ctx.reload_tuning()
 
     # parity of what was just timed: the whole output, outside the timed region
     got = np.asarray(c)
@@ -686,8 +735,9 @@ def main():
         int(np.count_nonzero(got != want)), n)
     del got, want
     ref_sum = float(x_h.sum(dtype=np.float64))
-    sum_rel_err = abs(float(np.asarray(s)) - ref_sum) / abs(ref_sum)
+    sum_rel_err = abs(sum_result - ref_sum) / abs(ref_sum)
     assert sum_rel_err <= 1e-5, "sum result wrong (relative error %.3g)" % sum_rel_err
+    assert abs(two_result - ref_sum) <= 1e-5 * abs(ref_sum), "two-launch sum wrong"
 
     elem_avg = float(elem_ms.mean())
     achieved = elem_bytes / (elem_avg * 1e-3) / 1e9
@@ -700,11 +750,17 @@ def main():
                 "avg_launch_us": round(elem_avg * 1e3, 2),
                 "median_launch_us": round(float(np.median(elem_ms)) * 1e3, 2),
                 "kernel_us": round(float(elem_kernel_ms.mean()) * 1e3, 2),
-                "kernel_text_hash": hashes["elem"],
+                "kernel_text_hash": "+".join(hashes["elem"]),
+                "frac_clock": "avg_launch_us: two events on the library's stream around each call in the timed "
+                              "region (kernel_us, from events on the dispatch itself, is what a kernel trace "
+                              "reports; frac_kernel is priced on it)",
+                "frac_kernel": round(elem_bytes / (float(elem_kernel_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "parity": "all 2^%d outputs equal NumPy's" % args.log2n,
                 "algorithmic_bytes_per_launch": elem_bytes}
     if traffic is None:
         roofline["traffic_note"] = why
+    else:
+        roofline["traffic_source"] = TRAFFIC_SOURCE
     sum_avg = float(sum_ms.mean())
     sum_gbs = sum_bytes / (sum_avg * 1e-3) / 1e9
     traffic_s, why_s = traffic_for("sum_2^%d" % args.log2n, hashes["sum"])
@@ -717,11 +773,21 @@ def main():
               "traffic": traffic_s,
               "avg_launch_us": round(sum_avg * 1e3, 2),
               "kernel_us": round(float(sum_kernel_ms.mean()) * 1e3, 2),
-              "kernel_text_hash": hashes["sum"],
+              "kernel_text_hash": "+".join(hashes["sum"]),
               "relative_error": float("%.3g" % sum_rel_err),
-              "algorithmic_bytes_per_launch": sum_bytes}
+              "algorithmic_bytes_per_launch": sum_bytes,
+              # finished by a second launch instead (GPUARRAY_REDUX_FUSED=0)
+              "two_launch_us": round(float(two_marks_ms.mean()) * 1e3, 2),
+              "two_launch_kernel_us": round(float(two_kernel_ms.mean()) * 1e3, 2),
+              "two_launch_launches": int(two_launches),
+              "two_launch_frac": round(sum_bytes / (float(two_marks_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     if traffic_s is None:
         second["traffic_note"] = why_s
+    else:
+        second["traffic_source"] = TRAFFIC_SOURCE
+    # the sum's figures once more inside "roofline" (readers that keep only the named objects)
+    roofline["sum"] = {k: second[k] for k in ("achieved", "frac", "avg_launch_us", "kernel_us", "launches_per_call",
+                                              "two_launch_us", "two_launch_kernel_us", "two_launch_frac")}
 
     # A second yardstick next to the published peak: what the driver's own
     # device-to-device copy (hipMemcpyDtoDAsync on the library's stream)
@@ -765,6 +831,16 @@ def main():
             del cfg
         res["latency"] = latency_table(ctx, ga)
         out["per_config"] = res
+        # the same table in short inside "config":
+        # name -> [fraction of peak between marks, by the kernel's own time,
+        #          counted HBM bytes / algorithmic bytes (null: no counter run
+        #          on these kernel texts), result equal to NumPy's]
+        out["config"]["per_config"] = {
+            name: [e["frac_cold"], e["frac_kernel_cold"], e.get("traffic_over_algorithmic"), e.get("parity_ok")]
+            for name, e in res.items() if name != "latency"}
+        out["config"]["per_config_columns"] = "frac_marks, frac_kernel, traffic/algorithmic, parity_ok"
+        out["config"]["latency_us"] = {k: v.get("device_us", v.get("wall_us_per_call"))
+                                       for k, v in res["latency"].items()}
     print(json.dumps(out))
 
 

@@ -48,6 +48,11 @@ typedef float (*ga_hip_event_elapsed_fn)(gpucontext *ctx, unsigned int a, unsign
  * returns the number of launches recorded, < 0 on error. */
 typedef int (*ga_hip_kernel_timing_fn)(gpucontext *ctx, int on);
 typedef int (*ga_hip_kernel_times_fn)(gpucontext *ctx, float *out, unsigned int max);
+/* "hip_kernel_hashes": the text hashes (as "hip_last_launch_hash" gives for the
+ * last launch) of the launches recorded since hip_kernel_timing was turned
+ * on, in launch order, to out[0..max); returns the number recorded.  A call
+ * made of several kernels is identified by all of them. */
+typedef int (*ga_hip_kernel_hashes_fn)(gpucontext *ctx, unsigned long long *out, unsigned int max);
 /* "hip_last_launch_hash": 64-bit FNV-1a hash of the source text, followed by
  * the entry point's name, of the kernel the context launched last (0 before
  * the first launch): ties a measurement to the generated kernel it was made

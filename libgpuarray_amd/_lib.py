@@ -7,7 +7,9 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libgpuarray.so")
+# GPUARRAY_LIBRARY names another build of the same library (the DEBUG and
+# sanitizer variants of csrc/Makefile); there is no other implementation.
+LIB_PATH = os.environ.get("GPUARRAY_LIBRARY") or os.path.join(_HERE, "libgpuarray.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(

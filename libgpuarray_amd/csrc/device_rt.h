@@ -8,7 +8,9 @@
  *   - __global__ / __device__ / __shared__ / __launch_bounds__,
  *     threadIdx / blockIdx / blockDim / gridDim, __syncthreads();
  *   - atomicAdd / atomicSub / atomicExch / atomicCAS / atomicMin / atomicMax /
- *     atomicAnd / atomicOr / atomicXor (relaxed, device scope);
+ *     atomicAnd / atomicOr / atomicXor (relaxed, device scope) on int, unsigned
+ *     int, unsigned long and unsigned long long (add and exchange on float, add
+ *     on double, min and max on long long as well);
  *   - the C math library for float and double under its C names (expf, exp,
  *     ...), its C++ overloads on the unsuffixed names (exp(float) is the float
  *     function; integers promote to double; mixed arguments to the wider type),
@@ -65,6 +67,7 @@ GA_RT_FN void __threadfence_block() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "
 #define GA_RT_ATOMIC_INTS(name, builtin) \
   GA_RT_ATOMIC(name, builtin, int)       \
   GA_RT_ATOMIC(name, builtin, unsigned int) \
+  GA_RT_ATOMIC(name, builtin, unsigned long) \
   GA_RT_ATOMIC(name, builtin, unsigned long long)
 GA_RT_ATOMIC_INTS(atomicAdd, __hip_atomic_fetch_add)
 GA_RT_ATOMIC(atomicAdd, __hip_atomic_fetch_add, float)
@@ -73,7 +76,9 @@ GA_RT_ATOMIC_INTS(atomicSub, __hip_atomic_fetch_sub)
 GA_RT_ATOMIC_INTS(atomicExch, __hip_atomic_exchange)
 GA_RT_ATOMIC(atomicExch, __hip_atomic_exchange, float)
 GA_RT_ATOMIC_INTS(atomicMin, __hip_atomic_fetch_min)
+GA_RT_ATOMIC(atomicMin, __hip_atomic_fetch_min, long long)
 GA_RT_ATOMIC_INTS(atomicMax, __hip_atomic_fetch_max)
+GA_RT_ATOMIC(atomicMax, __hip_atomic_fetch_max, long long)
 GA_RT_ATOMIC_INTS(atomicAnd, __hip_atomic_fetch_and)
 GA_RT_ATOMIC_INTS(atomicOr, __hip_atomic_fetch_or)
 GA_RT_ATOMIC_INTS(atomicXor, __hip_atomic_fetch_xor)
@@ -85,6 +90,7 @@ GA_RT_ATOMIC_INTS(atomicXor, __hip_atomic_fetch_xor)
   }
 GA_RT_CAS(int)
 GA_RT_CAS(unsigned int)
+GA_RT_CAS(unsigned long)
 GA_RT_CAS(unsigned long long)
 
 /* ---- integer helpers -------------------------------------------------------- */

@@ -146,12 +146,23 @@ int GpuArray_empty(GpuArray *a, gpucontext *ctx, int typecode, unsigned int nd,
                         "Total array size greater than addressable space");
     bytes *= dims[i];
   }
+  // A DEBUG build puts 64 bytes in front of every array, as the reference
+  // does (src/gpuarray_array.c:124-137): code that forgets an array's offset
+  // then reads or writes the wrong elements in every test instead of only on
+  // views.
+#ifdef DEBUG
+  const size_t lead = 64;
+  if (bytes > SIZE_MAX - lead)
+    return ga_err_set(ctx->err, GA_XLARGE_ERROR, "Total array size greater than addressable space");
+#else
+  const size_t lead = 0;
+#endif
   memset(a, 0, sizeof(*a));
   int res = GA_NO_ERROR;
-  a->data = gpudata_alloc(ctx, bytes, nullptr, 0, &res);
+  a->data = gpudata_alloc(ctx, bytes + lead, nullptr, 0, &res);
   if (a->data == nullptr) return ctx->err->code;
   a->nd = nd;
-  a->offset = 0;
+  a->offset = lead;
   a->typecode = typecode;
   a->dimensions = (size_t *)calloc(nd ? nd : 1, sizeof(size_t));
   a->strides = (ssize_t *)calloc(nd ? nd : 1, sizeof(ssize_t));
@@ -661,7 +672,7 @@ int GpuArray_fdump(FILE *fd, const GpuArray *a) {
     return ga_err_fmt(ctx->err, GA_UNSUPPORTED_ERROR, "Unsupported data type for dump: %d",
                       a->typecode);
   }
-  std::vector<char> buf(count * el ? count * el : 1);
+  std::vector<char> buf(count * el != 0 ? count * el : 1);
   int err = GpuArray_read(buf.data(), count * el, a);
   if (err != GA_NO_ERROR) return err;
   for (size_t k = 0; k < count; k++) {

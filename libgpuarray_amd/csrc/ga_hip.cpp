@@ -11,9 +11,14 @@
 // orders all work, so there are no per-buffer events.
 #include "private.hpp"
 
+#ifdef DEBUG
+#include <cassert>
+#endif
+
 #include <hip/hip_runtime_api.h>
 #include <amd_comgr/amd_comgr.h>
 
+#include <dlfcn.h>
 #include <fcntl.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -310,6 +315,7 @@ struct hip_context : _gpucontext {
   bool ktime_on = false;
   std::vector<hipEvent_t> ktime_ev;
   size_t ktime_n = 0;
+  std::vector<uint64_t> ktime_hash;   // text_hash of each recorded launch
   uint64_t last_launch_hash = 0;   // text_hash of the kernel launched last
   void *redux_cache = nullptr;
   void *take1_cache = nullptr;
@@ -345,11 +351,39 @@ void *stage_of(hip_context *ctx) {
 #define BUF_INTERNAL 0x20000   /* does not keep the context alive */
 #define BUF_HOSTMEM 0x40000    /* devptr is pinned host memory that kernels can write */
 
+// The reference's debugging aid (src/private_cuda.h:12-40): in a DEBUG build
+// contexts, buffers and kernels carry an 8-byte tag, set when the object is made
+// and wiped when it is freed, and every entry of the backend asserts the tag of
+// what it was handed: a stale or foreign pointer stops at the door instead of
+// corrupting something later.  (A context carries its tag in every build: it is
+// part of the struct's public head.)
+#define CTX_TAG "hipctx "
+#ifdef DEBUG
+#define BUF_TAG "hipbuf  "
+#define KER_TAG "hipkern "
+#define TAG_BUF(b) memcpy((b)->tag, BUF_TAG, 8)
+#define TAG_KER(k) memcpy((k)->tag, KER_TAG, 8)
+#define ASSERT_CTX(c) assert(memcmp((c)->tag, CTX_TAG, 8) == 0)
+#define ASSERT_BUF(b) assert(memcmp((b)->tag, BUF_TAG, 8) == 0)
+#define ASSERT_KER(k) assert(memcmp((k)->tag, KER_TAG, 8) == 0)
+#define CLEAR_TAG(o) memset((o)->tag, 0, 8)
+#else
+#define TAG_BUF(b)
+#define TAG_KER(k)
+#define ASSERT_CTX(c)
+#define ASSERT_BUF(b)
+#define ASSERT_KER(k)
+#define CLEAR_TAG(o)
+#endif
+
 struct hip_data : _gpudata {
   size_t sz;
   unsigned int refcnt;
   int flags;
   mem_block *block;   // cache block behind devptr; NULL when taken straight from the driver
+#ifdef DEBUG
+  char tag[8];
+#endif
 };
 
 struct hip_kernel : _gpukernel {
@@ -363,11 +397,24 @@ struct hip_kernel : _gpukernel {
   void **args;           // what setarg recorded: gpudata* or pointer into argstore
   size_t maxlsize;
   uint64_t text_hash;    // FNV-1a of the source text followed by the entry point's name
+#ifdef DEBUG
+  char tag[8];
+#endif
 };
 
-inline hip_context *HC(gpucontext *c) { return static_cast<hip_context *>(c); }
-inline hip_data *HD(gpudata *b) { return static_cast<hip_data *>(b); }
-inline hip_kernel *HK(gpukernel *k) { return static_cast<hip_kernel *>(k); }
+// (a NULL passes: the callers that allow one test for it themselves)
+inline hip_context *HC(gpucontext *c) {
+  if (c != nullptr) { ASSERT_CTX(c); }
+  return static_cast<hip_context *>(c);
+}
+inline hip_data *HD(gpudata *b) {
+  if (b != nullptr) { ASSERT_BUF(static_cast<hip_data *>(b)); }
+  return static_cast<hip_data *>(b);
+}
+inline hip_kernel *HK(gpukernel *k) {
+  if (k != nullptr) { ASSERT_KER(static_cast<hip_kernel *>(k)); }
+  return static_cast<hip_kernel *>(k);
+}
 
 int hip_fail(ga_errrec *e, const char *what, hipError_t err) {
   return ga_err_fmt(e, GA_IMPL_ERROR, "%s: %s (%d)", what, hipGetErrorString(err),
@@ -437,6 +484,7 @@ void ctx_destroy(hip_context *ctx) {
   if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
+  memset(ctx->tag, 0, 8);   // (in every build: a freed context no longer looks like one)
   delete ctx;
 }
 
@@ -477,7 +525,7 @@ gpucontext *hip_init(gpucontext_props *p) {
   ctx->errbuf = nullptr;
   ctx->extcopy_cache = nullptr;
   memset(ctx->bin_id, 0, sizeof(ctx->bin_id));
-  memcpy(ctx->tag, "hipctx ", 8);
+  memcpy(ctx->tag, CTX_TAG, 8);
   ctx->dev = dev;
   ga_tuning_read(&ctx->tuning);
 
@@ -568,6 +616,7 @@ gpucontext *hip_init(gpucontext_props *p) {
     hip_data *b = (hip_data *)calloc(1, sizeof(hip_data));
     if (b != nullptr && hipHostMalloc(&flag, 64, hipHostMallocCoherent) == hipSuccess) {
       memset(flag, 0, 64);
+      TAG_BUF(b);
       b->devptr = flag;
       b->ctx = ctx;
       b->sz = 8;
@@ -628,6 +677,7 @@ gpudata *hip_alloc(gpucontext *c, size_t sz, void *data, int flags) {
     ga_err_sys(ctx->err, "calloc");
     return nullptr;
   }
+  TAG_BUF(b);
   size_t asz = sz ? sz : 1;   // a zero-byte request still yields a valid buffer
   if (ctx->mem.max != 0) {
     int why = 0;
@@ -695,6 +745,7 @@ void hip_release(gpudata *bb) {
     (void)hipFree(b->devptr);
   }
   bool counted = !(b->flags & BUF_INTERNAL);
+  CLEAR_TAG(b);
   free(b);
   if (counted) ctx_unref(ctx);
 }
@@ -1044,6 +1095,109 @@ int rtc_compile(const std::string &src, std::vector<char> &code, std::string &lo
   return GA_NO_ERROR;
 }
 
+// The same through hipRTC, with the toolchain's HIP headers in front of the
+// text instead of device_rt.h.  Kernel text handed to GpuKernel_init may be
+// written against those headers (hip_fp16.h types, __shfl and __ballot,
+// float4 / make_float4, printf, clock64, cooperative groups); the contract is
+// "any source the backend's compiler accepts" (reference
+// src/gpuarray/kernel.h:54-70, whose CUDA backend compiles with NVRTC and its
+// full device vocabulary).  Used only as a second try for text that fails
+// against device_rt.h on something a header would supply: it costs the
+// quarter of a second per kernel that the first path is there to save.
+// libhiprtc is loaded when the first such kernel arrives.
+struct hiprtc_api {
+  void *lib = nullptr;
+  int (*create)(void **, const char *, const char *, int, const char *const *, const char *const *) = nullptr;
+  int (*compile)(void *, int, const char *const *) = nullptr;
+  int (*log_size)(void *, size_t *) = nullptr;
+  int (*get_log)(void *, char *) = nullptr;
+  int (*code_size)(void *, size_t *) = nullptr;
+  int (*get_code)(void *, char *) = nullptr;
+  int (*destroy)(void **) = nullptr;
+  bool ok = false;
+};
+
+const hiprtc_api &hiprtc() {
+  static const hiprtc_api api = [] {
+    hiprtc_api a;
+    for (const char *name : {"libhiprtc.so", "libhiprtc.so.7"}) {
+      a.lib = dlopen(name, RTLD_NOW | RTLD_LOCAL);
+      if (a.lib != nullptr) break;
+    }
+    if (a.lib == nullptr) return a;
+    a.create = (decltype(a.create))dlsym(a.lib, "hiprtcCreateProgram");
+    a.compile = (decltype(a.compile))dlsym(a.lib, "hiprtcCompileProgram");
+    a.log_size = (decltype(a.log_size))dlsym(a.lib, "hiprtcGetProgramLogSize");
+    a.get_log = (decltype(a.get_log))dlsym(a.lib, "hiprtcGetProgramLog");
+    a.code_size = (decltype(a.code_size))dlsym(a.lib, "hiprtcGetCodeSize");
+    a.get_code = (decltype(a.get_code))dlsym(a.lib, "hiprtcGetCode");
+    a.destroy = (decltype(a.destroy))dlsym(a.lib, "hiprtcDestroyProgram");
+    a.ok = a.create && a.compile && a.log_size && a.get_log && a.code_size && a.get_code && a.destroy;
+    return a;
+  }();
+  return api;
+}
+
+// Does a failed compile against device_rt.h look like text that wants the
+// toolchain's headers (rather than text that is simply wrong)?
+bool wants_toolchain_headers(const std::string &log) {
+  for (const char *sign : {"file not found", "undeclared identifier", "unknown type name",
+                           "no matching function", "no member named", "use of undeclared"})
+    if (log.find(sign) != std::string::npos) return true;
+  return false;
+}
+
+int hiprtc_compile(const std::string &src, std::vector<char> &code, std::string &log) {
+  const hiprtc_api &rt = hiprtc();
+  if (!rt.ok) {
+    log += "\n(libhiprtc could not be loaded for a second try with the toolchain's headers)";
+    return GA_IMPL_ERROR;
+  }
+  static std::mutex compiler_lock;
+  std::lock_guard<std::mutex> guard(compiler_lock);
+  void *prog = nullptr;
+  const char *headers[1] = {ga_cluda_hip_src};
+  const char *names[1] = {"cluda.h"};
+  if (rt.create(&prog, src.c_str(), "ga_kernel.hip", 1, headers, names) != 0) return GA_IMPL_ERROR;
+  // headers beyond the ones hipRTC carries inside itself come from the installation
+  const char *root = getenv("ROCM_PATH");
+  const std::string inc = std::string("-I") + ((root && *root) ? root : "/opt/rocm") + "/include";
+  const char *const opts[] = {"--offload-arch=gfx950", "-O2", "-ffp-contract=off",
+                              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                              "-Wno-unused-value", inc.c_str()};
+  const int rc = rt.compile(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+  size_t n = 0;
+  std::string second;
+  if (rt.log_size(prog, &n) == 0 && n > 1) {
+    second.resize(n);
+    if (rt.get_log(prog, &second[0]) != 0) second.clear();
+    while (!second.empty() && second.back() == '\0') second.pop_back();
+  }
+  int err = GA_IMPL_ERROR;
+  if (rc == 0 && rt.code_size(prog, &n) == 0 && n > 0) {
+    code.resize(n);
+    if (rt.get_code(prog, code.data()) == 0) err = GA_NO_ERROR;
+  }
+  if (err != GA_NO_ERROR) {
+    code.clear();
+    log += "\n--- second try, with the toolchain's HIP headers (hipRTC) ---\n" + second;
+  }
+  rt.destroy(&prog);
+  return err;
+}
+
+// Compile kernel text: against device_rt.h first; text that fails there on
+// something the toolchain's headers would supply gets one more try through hipRTC.
+int compile_kernel_text(const std::string &src, std::vector<char> &code, std::string &log) {
+  int err = rtc_compile(src, code, log);
+  if (err != GA_NO_ERROR && wants_toolchain_headers(log)) err = hiprtc_compile(src, code, log);
+#ifdef DEBUG
+  // (the reference's DEBUG builds print the compiler's log, src/gpuarray_elemwise.c:682-690)
+  if (err != GA_NO_ERROR) fprintf(stderr, "%s\n", log.c_str());
+#endif
+  return err;
+}
+
 // ---- on-disk cache of compiled kernels ------------------------------------------
 // A compile costs 0.3-0.5 s; a process that builds a few hundred operators
 // spends minutes in the compiler.  With a cache directory (property
@@ -1203,7 +1357,7 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
       from_disk = disk_load(ctx->disk_cache, dkey, code);
     }
     if (!from_disk) {
-      err = rtc_compile(src, code, log);
+      err = compile_kernel_text(src, code, log);
       if (err != GA_NO_ERROR) {
         if (err_str) *err_str = strdup(log.c_str());
         return ga_err_fmt(ctx->err, GA_IMPL_ERROR, "Kernel compilation failed: %.900s", log.c_str());
@@ -1215,7 +1369,7 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
     if (e != hipSuccess && from_disk) {
       // a damaged cache entry: compile afresh and replace it
       (void)hipGetLastError();
-      err = rtc_compile(src, code, log);
+      err = compile_kernel_text(src, code, log);
       if (err != GA_NO_ERROR) {
         delete m;
         if (err_str) *err_str = strdup(log.c_str());
@@ -1247,6 +1401,7 @@ int hip_newkernel(gpukernel **out, gpucontext *c, unsigned int count, const char
 
   hip_kernel *k = (hip_kernel *)calloc(1, sizeof(hip_kernel));
   if (k == nullptr) return ga_err_sys(ctx->err, "calloc");
+  TAG_KER(k);
   k->ctx = ctx;
   k->fn = fn;
   k->mod = m;
@@ -1296,6 +1451,7 @@ void hip_freekernel(gpukernel *kk) {
   free(k->argoff);
   free(k->args);
   free(k->argstore);
+  CLEAR_TAG(k);
   free(k);
   ctx_unref(ctx);
 }
@@ -1376,6 +1532,8 @@ int hip_callkernel(gpukernel *kk, unsigned int n, const size_t *gs, const size_t
                                           shared, ctx->stream, params, nullptr,
                                           ctx->ktime_ev[2 * ctx->ktime_n],
                                           ctx->ktime_ev[2 * ctx->ktime_n + 1], 0));
+    if (ctx->ktime_hash.size() <= ctx->ktime_n) ctx->ktime_hash.resize(ctx->ktime_n + 1);
+    ctx->ktime_hash[ctx->ktime_n] = k->text_hash;
     ctx->ktime_n++;
     return GA_NO_ERROR;
   }
@@ -1502,6 +1660,7 @@ gpudata *ext_make_buf(gpucontext *c, void *devptr, size_t sz) {
     ga_err_sys(ctx->err, "calloc");
     return nullptr;
   }
+  TAG_BUF(b);
   b->devptr = devptr;
   b->ctx = ctx;
   b->sz = sz;
@@ -1514,7 +1673,7 @@ gpudata *ext_make_buf(gpucontext *c, void *devptr, size_t sz) {
 int ext_compile_only(unsigned int count, const char **strs, const size_t *lens, char **log) {
   std::vector<char> code;
   std::string l;
-  int err = rtc_compile(join_sources(count, strs, lens), code, l);
+  int err = compile_kernel_text(join_sources(count, strs, lens), code, l);
   if (log) *log = l.empty() ? nullptr : strdup(l.c_str());
   if (err != GA_NO_ERROR) ga_err_fmt(ga_global_err, err, "Kernel compilation failed: %.900s", l.c_str());
   return err;
@@ -1609,6 +1768,16 @@ int ext_kernel_times(gpucontext *c, float *out, unsigned int max) {
   return (int)n;
 }
 
+// The text hashes (see ext_last_launch_hash) of the launches recorded since
+// timing was turned on, in launch order, into out[0..max).  Returns how many
+// were recorded.
+int ext_kernel_hashes(gpucontext *c, unsigned long long *out, unsigned int max) {
+  hip_context *ctx = HC(c);
+  const size_t n = ctx->ktime_n;
+  for (size_t i = 0; i < n && i < max; i++) out[i] = ctx->ktime_hash[i];
+  return (int)n;
+}
+
 // Identifies the text of the kernel the context launched last: a 64-bit hash
 // of its source followed by its entry point's name.  Lets a measurement say
 // which generated kernel it belongs to.
@@ -1641,6 +1810,7 @@ const ext_entry k_exts[] = {
     {"hip_event_elapsed", (void *)ext_event_elapsed},
     {"hip_kernel_timing", (void *)ext_kernel_timing},
     {"hip_kernel_times", (void *)ext_kernel_times},
+    {"hip_kernel_hashes", (void *)ext_kernel_hashes},
     {"hip_last_launch_hash", (void *)ext_last_launch_hash},
     {"hip_elemwise_source", (void *)ga_elemwise_gen_source},
     {"hip_reduction_source", (void *)ga_reduction_gen_source},

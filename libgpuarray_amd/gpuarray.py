@@ -220,6 +220,13 @@ class GpuContext(object):
             raise GpuArrayException("kernel timing failed: " + self.error(), _lib.GA_IMPL_ERROR)
         return list(buf[:min(n, limit)])
 
+    def kernel_hashes(self, limit=65536):
+        """Text hash (hex) of each launch recorded since kernel_timing(True)."""
+        fn = _lib.extension("hip_kernel_hashes", C.c_int, [C.c_void_p, C.POINTER(C.c_ulonglong), C.c_uint])
+        buf = (C.c_ulonglong * limit)()
+        n = fn(self.ctx, buf, limit)
+        return ["%016x" % v for v in buf[:min(n, limit)]]
+
     def reload_tuning(self):
         """Read the GPUARRAY_* tuning knobs from the environment again (a
         context reads them once, when it is made)."""

@@ -195,3 +195,25 @@ def test_reduction_plan_struct_matches_the_kernel_side():
     src = take_string(gen_reduction(0, _lib.GA_FLOAT, _lib.GA_FLOAT, _lib.GA_LONG, 64, 1, 1)).decode()
     body = re.search(r"struct rd_plan \{(.*?)\};", src, re.S).group(1)
     assert body.count("[RD_MAXD]") == 7 and "#define RD_MAXD 8" in src
+
+
+def test_text_that_needs_the_toolchain_headers_gets_a_second_compile():
+    """The library's device runtime covers what its own generators use; a
+    caller's kernel may use more of HIP.  What fails on a missing header or
+    identifier is compiled once more through hipRTC (needs no device)."""
+    plain = b'#include "cluda.h"\nKERNEL void k(GLOBAL_MEM float *a) { a[LID_0] = 1.0f; }'
+    err, log = compile_src(plain)
+    assert err == 0 and "second try" not in log
+    rich = (b'#include <hip/hip_fp16.h>\n'
+            b'extern "C" __global__ void k(__half *a, float4 *b) {\n'
+            b'  a[threadIdx.x] = __float2half(1.0f); b[0] = make_float4(1, 2, 3, 4);\n'
+            b'  a[1] = __float2half((float)__shfl(5, 0)); printf("%d", (int)clock64()); }')
+    err, log = compile_src(rich)
+    assert err == 0, log[-800:]
+    # the atomics callers most often reach for on 64-bit words are in the small runtime itself
+    words = (b'#include "cluda.h"\nKERNEL void k(GLOBAL_MEM unsigned long *a, GLOBAL_MEM long long *b) {\n'
+             b'  atomicAdd(a, 1ul); atomicMax(b, 3ll); atomicCAS(a, 1ul, 2ul); }')
+    err, log = compile_src(words)
+    assert err == 0 and log == "", log[-400:]
+    err, log = compile_src(b'extern "C" __global__ void k(int *p) { p[0] = no_such_thing(3); }')
+    assert err != 0 and "no_such_thing" in log and "second try" in log

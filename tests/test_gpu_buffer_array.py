@@ -120,6 +120,53 @@ def test_large_moves_take_the_copy_kernel(ctx, knobs):
     assert lib.GpuArray_read(h.ctypes.data, 4, C.byref(cleared)) == _lib.GA_INVALID_ERROR
 
 
+def test_user_kernel_written_against_the_toolchain_headers(ctx):
+    """Kernel text that leans on the toolchain's HIP headers (half types,
+    cross-lane shuffles, float4, the cooperative-groups header) fails against
+    the library's own small device runtime and gets a second compile through
+    hipRTC: GpuKernel_init accepts any source the backend's compiler accepts
+    (reference src/gpuarray/kernel.h:54-70)."""
+    src = b"""#include <hip/hip_fp16.h>
+#include <hip/hip_cooperative_groups.h>
+extern "C" __global__ void lanes(float *out, __half *h, float4 *q, unsigned int n) {
+  auto block = cooperative_groups::this_thread_block();
+  unsigned int i = blockIdx.x * blockDim.x + block.thread_rank();
+  if (i >= n) return;
+  float from_left = __shfl_up((float)i, 1);          // lane 0 of a wavefront keeps its own
+  out[i] = from_left;
+  h[i] = __float2half(0.5f * (float)(i % 7));
+  if (i < n / 4) q[i] = make_float4(i, i + 1.0f, i + 2.0f, i + 3.0f);
+}"""
+    n = 1024
+    out = gpuarray.zeros((n,), "float32", context=ctx)
+    h = gpuarray.zeros((n,), "float16", context=ctx)
+    q = gpuarray.zeros((n,), "float32", context=ctx)
+    k = _lib.GpuKernelStruct()
+    types = (C.c_int * 4)(_lib.GA_BUFFER, _lib.GA_BUFFER, _lib.GA_BUFFER, _lib.GA_UINT)
+    strs = (C.c_char_p * 1)(src)
+    log = C.c_char_p()
+    rc = lib.GpuKernel_init(C.byref(k), ctx.ctx, 1, strs, None, b"lanes", 4, types, _lib.GA_USE_HALF, C.byref(log))
+    assert rc == 0, (log.value or b"").decode(errors="replace")[-800:]
+    nn = C.c_uint(n)
+    for i, a in enumerate((out.ga.data, h.ga.data, q.ga.data, C.byref(nn))):
+        assert lib.GpuKernel_setarg(C.byref(k), i, a) == 0
+    gs, ls = C.c_size_t(n // 256), C.c_size_t(256)
+    assert lib.GpuKernel_call(C.byref(k), 1, C.byref(gs), C.byref(ls), 0, None) == 0
+    idx = np.arange(n)
+    want = np.where(idx % 64 == 0, idx, idx - 1).astype(np.float32)
+    assert np.array_equal(np.asarray(out), want)
+    assert np.array_equal(np.asarray(h), (0.5 * (idx % 7)).astype(np.float16))
+    wq = np.zeros(n, np.float32)
+    wq[:n] = (np.arange(n // 4)[:, None] + np.arange(4)[None, :]).reshape(-1)[:n]
+    assert np.array_equal(np.asarray(q), wq)
+    lib.GpuKernel_clear(C.byref(k))
+    # text that is simply wrong still fails, and the log holds both tries
+    bad = (C.c_char_p * 1)(b'extern "C" __global__ void k(int *p) { p[0] = no_such_thing(3); }')
+    assert lib.GpuKernel_init(C.byref(k), ctx.ctx, 1, bad, None, b"k", 1, types, 0, C.byref(log)) == _lib.GA_IMPL_ERROR
+    text = (log.value or b"").decode(errors="replace")
+    assert "no_such_thing" in text and "second try" in text
+
+
 def test_user_kernel_through_gpukernel(ctx):
     # a kernel in the reference's dialect, launched with explicit geometry and
     # with GpuKernel_sched's geometry

@@ -969,6 +969,94 @@ def test_split_reductions_finish_in_one_launch(ctx, knobs):
     assert np.asarray(v) == np.nanmax(x) and int(np.asarray(i)) == int(np.nanargmax(x))
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_single_launch_finish_equals_two_launches_bit_for_bit(ctx, knobs, seed):
+    """Every family of split reduction that can end in its own launch (row and
+    column kernels, 4- and 8-byte accumulators, integer, float, with and
+    without an index) against the same call finished by a second launch
+    (REDUX_FUSED=0), bit for bit, over sixty drawn shapes per seed; the first
+    mismatch stops the test.  The single launch orders its partials with
+    device-scope atomics and a counter; the two launches with nothing but
+    stream order.  Float data are small integers, so that every sum is exact
+    and the two forms, which group the partials differently, must agree in
+    every bit (specification of the result: reference pygpu/reduction.py:85-132);
+    values change from call to call, so a partial left over from an earlier
+    call, or one read before it arrived, shows."""
+    rng = np.random.default_rng(9100 + seed)
+    ops = [("sum", "float32", "float32"), ("sum", "float64", "float64"), ("sum", "int32", "int64"),
+           ("sum", "int32", "int32"), ("sum", "int16", "int64"), ("max", "float32", None),
+           ("min", "float64", None), ("max", "int32", None), ("maxandargmax", "float32", None),
+           ("minandargmin", "float64", None), ("maxandargmax", "int32", None), ("argmax", "float32", None),
+           ("prod", "int32", "int64"), ("any", "uint8", None), ("all", "int32", None), ("xor", "uint32", None)]
+
+    def draw_shape():
+        kind = int(rng.integers(0, 6))
+        if kind == 0:      # one long row
+            return (int(rng.integers(1 << 15, 1 << 22)),), (0,)
+        if kind == 1:      # a few long rows
+            return (int(rng.integers(2, 40)), int(rng.integers(1 << 14, 1 << 18))), (1,)
+        if kind == 2:      # long columns, few to many outputs
+            return (int(rng.integers(1 << 11, 1 << 15)), int(rng.choice([8, 64, 100, 256, 1000, 4096]))), (0,)
+        if kind == 3:      # reduced dims around a kept one
+            return (int(rng.integers(8, 200)), int(rng.integers(2, 30)), int(rng.integers(256, 8192))), (0, 2)
+        if kind == 4:      # a middle axis over long columns
+            return (int(rng.integers(2, 8)), int(rng.integers(1 << 10, 1 << 13)), int(rng.choice([32, 128, 512]))), (1,)
+        return (int(rng.integers(1 << 16, 1 << 20)), int(rng.choice([1, 2, 3, 8]))), (0,)
+
+    def run_all(cases):
+        out, launches = [], []
+        for g, name, odt, axes in cases:
+            ctx.kernel_timing(True)
+            if name in ("maxandargmax", "minandargmin"):
+                r = R._arg_reduce(g, name, list(axes), True)
+            elif name == "argmax":
+                r = (R._arg_reduce(g, name, list(axes), False),)
+            else:
+                r = (R._reduce_named(g, name, np.dtype(odt) if odt else
+                                     (np.dtype("bool") if name in ("any", "all") else g.dtype), axis=axes),)
+            launches.append(len(ctx.kernel_times()))
+            ctx.kernel_timing(False)
+            out.append([np.asarray(x) for x in r])
+        return out, launches
+
+    single_launch_taken = 0
+    for batch in range(4):
+        cases, hosts = [], []
+        for _ in range(15):
+            name, dt, odt = ops[int(rng.integers(0, len(ops)))]
+            shape, axes = draw_shape()
+            if name == "prod":
+                host = rng.choice(np.array([1, 1, 1, -1], dt), size=shape)     # +-2^k: exact in int64
+                host.reshape(-1)[rng.integers(0, host.size, 20)] = 2
+            elif name in ("any", "all"):
+                host = (rng.random(shape) < (0.0005 if name == "any" else 0.9995)).astype(dt)
+            elif np.dtype(dt).kind == "u":
+                host = rng.integers(0, 1 << 16, size=shape).astype(dt)
+            else:
+                host = rng.integers(-40, 41, size=shape).astype(dt)
+            g, _ = to_gpu_view(host, ctx)
+            cases.append((g, name, odt, axes))
+            hosts.append(host)
+        one, n_one = run_all(cases)
+        knobs(REDUX_FUSED=0)
+        two, n_two = run_all(cases)
+        knobs(REDUX_FUSED=None)
+        for k, (a, b) in enumerate(zip(one, two)):
+            what = (seed, batch, k, cases[k][1], hosts[k].dtype.name, hosts[k].shape, cases[k][3],
+                    n_one[k], n_two[k])
+            assert len(a) == len(b)
+            for x, y in zip(a, b):
+                assert x.dtype == y.dtype and x.shape == y.shape, what
+                assert x.tobytes() == y.tobytes(), what
+            single_launch_taken += n_one[k] < n_two[k]
+        # and against NumPy for the plain sums (exact data)
+        for k, (g, name, odt, axes) in enumerate(cases):
+            if name == "sum":
+                assert np.array_equal(one[k][0], hosts[k].sum(axis=axes, dtype=odt)), (seed, batch, k)
+    # the draw must really exercise the single launch
+    assert single_launch_taken >= 15, single_launch_taken
+
+
 @pytest.mark.parametrize("dtype", ["uint8", "int8", "bool"])
 def test_any_all_over_columns_of_bytes(ctx, dtype):
     """any / all with lanes along the free dim over one-byte elements: the

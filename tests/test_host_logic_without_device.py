@@ -5,7 +5,13 @@ errors, read/write checks) run here against tests/mock_runtime/mock_hip.cpp,
 a preloaded stand-in for the HIP runtime whose buffers are host memory and
 whose kernel launches do nothing.  The C client runs through context
 teardown the same way (its numeric checks fail, by construction; it must not
-crash).  On a GPU box the same tests run for real under `-m gpu`."""
+crash).  On a GPU box the same tests run for real under `-m gpu`.
+
+Each test runs against three builds of the library (csrc/Makefile): the
+shipped one, the DEBUG one (the reference's debugging aids: 64 bytes in front
+of every array, tagged structs with asserts) and one whose host code is
+compiled with GCC's address and undefined-behaviour sanitizers, where any
+report fails the test."""
 import os
 import subprocess
 import sys
@@ -33,9 +39,29 @@ HOST_ONLY = [
 ]
 
 
-def preload(lib):
-    """LD_PRELOAD with `lib` in front of whatever is preloaded already."""
-    return " ".join(x for x in (lib, os.environ.get("LD_PRELOAD", "")) if x)
+CSRC = os.path.join(ROOT, "libgpuarray_amd", "csrc")
+
+
+@pytest.fixture(scope="module", params=["shipped", "debug", "asan"])
+def build(request, mock_runtime):
+    """Environment of a child process that runs the named build of the library
+    on the stand-in runtime."""
+    variant = request.param
+    env = dict(os.environ)
+    pre = [mock_runtime]
+    if variant != "shipped":
+        subprocess.check_call(["make", "-s", "-C", CSRC, "-j8", variant], stdout=subprocess.DEVNULL)
+        env["GPUARRAY_LIBRARY"] = os.path.join(CSRC, "build", variant, "libgpuarray.so")
+    if variant == "asan":
+        # the sanitizer runtimes come first; leaks are not asked for (the
+        # interpreter itself never frees everything); the first report ends the process
+        for name in ("libubsan.so", "libasan.so"):
+            pre.insert(0, subprocess.check_output(["gcc", "-print-file-name=" + name], text=True).strip())
+        env["ASAN_OPTIONS"] = "detect_leaks=0:halt_on_error=1:abort_on_error=1"
+        env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
+    env["LD_PRELOAD"] = " ".join(pre + [x for x in (os.environ.get("LD_PRELOAD", ""),) if x])
+    env["GA_TEST_MOCK_RUNTIME"] = mock_runtime
+    return variant, env
 
 
 @pytest.fixture(scope="module")
@@ -47,22 +73,22 @@ def mock_runtime(tmp_path_factory):
     return str(out)
 
 
-def test_host_only_tests_pass_without_a_device(mock_runtime):
-    env = dict(os.environ, LD_PRELOAD=preload(mock_runtime))
+def test_host_only_tests_pass_without_a_device(build):
+    variant, env = build
     r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-m", "gpu", "-p", "no:cacheprovider",
                         "--timeout", "300"] + HOST_ONLY, cwd=ROOT, env=env, capture_output=True,
                        text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
 
 
-def test_c_client_survives_teardown_without_a_device(mock_runtime, tmp_path):
-    libdir = os.path.join(ROOT, "libgpuarray_amd")
+def test_c_client_survives_teardown_without_a_device(build, tmp_path):
+    variant, env = build
+    libdir = os.path.dirname(env.get("GPUARRAY_LIBRARY", os.path.join(ROOT, "libgpuarray_amd", "libgpuarray.so")))
     exe = tmp_path / "client"
     subprocess.check_call(["gcc", "-std=gnu99", "-O1", "-I", os.path.join(ROOT, "include"),
                            os.path.join(ROOT, "tests", "c_client", "client.c"), "-o", str(exe),
                            "-L", libdir, "-l:libgpuarray.so", "-Wl,-rpath," + libdir])
-    r = subprocess.run([str(exe)], env=dict(os.environ, LD_PRELOAD=preload(mock_runtime)),
-                       capture_output=True, text=True, timeout=300)
+    r = subprocess.run([str(exe)], env=env, capture_output=True, text=True, timeout=300)
     # kernels do nothing here, so the numeric checks fail (status 1); what is
     # asked is that every host path, context teardown included, runs through
     assert r.returncode in (0, 1), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
@@ -70,22 +96,26 @@ def test_c_client_survives_teardown_without_a_device(mock_runtime, tmp_path):
 
 
 @pytest.mark.parametrize("seed", [0, 1])
-def test_planners_survive_random_layouts(mock_runtime, seed):
+def test_planners_survive_random_layouts(build, seed):
     """Random element types, shapes, steps (1 to 4), offsets, transposes and
     axis sets through the reduction and elementwise planners (an 8-byte type
     stepping by four once gave the row planner a vector width of zero)."""
-    r = subprocess.run([sys.executable, os.path.join("tests", "planner_random_layouts.py"), str(seed), "100"],
-                       cwd=ROOT, env=dict(os.environ, LD_PRELOAD=preload(mock_runtime)), capture_output=True,
-                       text=True, timeout=900)
+    variant, env = build
+    if variant == "asan" and seed != 0:
+        pytest.skip("one seed under the sanitizers (kernel compiles take ten times as long there)")
+    count = "12" if variant == "asan" else "100"
+    r = subprocess.run([sys.executable, os.path.join("tests", "planner_random_layouts.py"), str(seed), count],
+                       cwd=ROOT, env=env, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "planner ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
 
 
-def test_views_follow_numpy_on_random_chains(mock_runtime):
+def test_views_follow_numpy_on_random_chains(build):
     """Chains of indexing, transposition and reshaping: shape, strides, byte
     offset and contiguity flags against NumPy's at every step."""
-    r = subprocess.run([sys.executable, os.path.join("tests", "views_random_walk.py"), "0", "3000"],
-                       cwd=ROOT, env=dict(os.environ, LD_PRELOAD=preload(mock_runtime)), capture_output=True,
-                       text=True, timeout=600)
+    variant, env = build
+    r = subprocess.run([sys.executable, os.path.join("tests", "views_random_walk.py"), "0",
+                        "600" if variant == "asan" else "3000"],
+                       cwd=ROOT, env=env, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0 and "views ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
 
 
@@ -95,7 +125,7 @@ import numpy as np
 sys.path.insert(0, os.getcwd())
 import libgpuarray_amd as ga
 from libgpuarray_amd import _lib
-mock = C.CDLL(os.environ["LD_PRELOAD"].split()[0])
+mock = C.CDLL(os.environ["GA_TEST_MOCK_RUNTIME"])
 calls = C.c_ulong.in_dll(mock, "mock_allocating_calls")
 ctx = ga.init("hip0")
 for dtype, shape, axes, d1 in (("float32", (1 << 22,), [0], False), ("int32", (6, 1 << 18), [1], False),
@@ -115,13 +145,13 @@ print("noalloc ok")
 """
 
 
-def test_noalloc_entry_point_calls_nothing_that_allocates(mock_runtime):
+def test_noalloc_entry_point_calls_nothing_that_allocates(build):
     """GpuReduction_call_noalloc between two counts of the stand-in runtime's
     allocating calls (hipMalloc, hipFree, hipHostMalloc, hipHostFree,
     hipModuleLoadData, hipEventCreate): none may happen, for split and unsplit
     reductions, with and without an index result."""
-    r = subprocess.run([sys.executable, "-c", NOALLOC_SCRIPT], cwd=ROOT,
-                       env=dict(os.environ, LD_PRELOAD=preload(mock_runtime)), capture_output=True, text=True,
+    variant, env = build
+    r = subprocess.run([sys.executable, "-c", NOALLOC_SCRIPT], cwd=ROOT, env=env, capture_output=True, text=True,
                        timeout=300)
     assert r.returncode == 0 and "noalloc ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])
 
@@ -130,7 +160,7 @@ TUNING_SCRIPT = r"""
 import ctypes as C, os, sys
 sys.path.insert(0, os.getcwd())
 import libgpuarray_amd as ga
-mock = C.CDLL(os.environ["LD_PRELOAD"].split()[0])
+mock = C.CDLL(os.environ["GA_TEST_MOCK_RUNTIME"])
 launches = C.c_ulong.in_dll(mock, "mock_kernel_launches")
 ctx = ga.init("hip0")
 op = ga.GpuReduction(ctx, "sum", "float32")
@@ -158,11 +188,11 @@ print("tuning ok")
 """
 
 
-def test_tuning_knobs_are_read_when_a_context_is_made_not_per_call(mock_runtime):
+def test_tuning_knobs_are_read_when_a_context_is_made_not_per_call(build):
     """The GPUARRAY_* knobs live in a table of the context, filled from the
     environment at gpucontext_init and by the hip_reload_tuning hook; a call
     reads the table only."""
-    r = subprocess.run([sys.executable, "-c", TUNING_SCRIPT], cwd=ROOT,
-                       env=dict(os.environ, LD_PRELOAD=preload(mock_runtime)), capture_output=True, text=True,
+    variant, env = build
+    r = subprocess.run([sys.executable, "-c", TUNING_SCRIPT], cwd=ROOT, env=env, capture_output=True, text=True,
                        timeout=300)
     assert r.returncode == 0 and "tuning ok" in r.stdout, (r.returncode, r.stdout[-600:], r.stderr[-1500:])

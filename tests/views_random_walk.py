@@ -56,7 +56,8 @@ for chain in range(chains):
     h0 = np.zeros(shape, dt, order=order)
     g = ga.zeros(shape, dt, order=order, context=ctx)
     h = h0
-    base_ptr = h0.__array_interface__["data"][0]
+    # (a fresh array starts at offset 0, or at 64 in a DEBUG build of the library)
+    base_ptr = h0.__array_interface__["data"][0] - g.offset
     trail = [(shape, dt, order)]
     same(g, h, base_ptr, trail)
     for step in range(int(rng.integers(1, 6))):
