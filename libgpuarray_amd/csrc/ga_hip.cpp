@@ -307,6 +307,7 @@ struct hip_context : _gpucontext {
   std::vector<gpudata *> retired_scratch;   // outgrown scratch buffers, kept until teardown
   void *static_scratch = nullptr;           // this device's copy of the static scratch array
   int static_scratch_err = 0;               // HIP error code of its lookup
+  gpudata *static_buf = nullptr;            // that array as a buffer of the context (not owned, not counted)
   gpudata *redux_counters = nullptr;   // zeroed counters of single-launch split reductions
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::vector<hipEvent_t> evpool;   // timing marks for callers (hip_event_* hooks)
@@ -465,6 +466,7 @@ void ctx_destroy(hip_context *ctx) {
   // internal buffers do not count as owners, so they are still here
   if (ctx->errbuf) { hip_release(ctx->errbuf); ctx->errbuf = nullptr; }
   if (ctx->scratch) { hip_release(ctx->scratch); ctx->scratch = nullptr; }
+  if (ctx->static_buf) { hip_release(ctx->static_buf); ctx->static_buf = nullptr; }
   for (gpudata *b : ctx->retired_scratch) hip_release(b);
   ctx->retired_scratch.clear();
   if (ctx->redux_counters) { hip_release(ctx->redux_counters); ctx->redux_counters = nullptr; }
@@ -576,6 +578,19 @@ gpucontext *hip_init(gpucontext_props *p) {
   // of GpuReduction_call_noalloc).  A failed lookup only disables that entry
   // point, which then reports the code kept here.
   ctx->static_scratch_err = ga_static_scratch_setup(dev, &ctx->static_scratch);
+  if (ctx->static_scratch != nullptr) {
+    // made here, so that the entry point that may not allocate finds it ready
+    hip_data *b = (hip_data *)calloc(1, sizeof(hip_data));
+    if (b != nullptr) {
+      TAG_BUF(b);
+      b->devptr = ctx->static_scratch;
+      b->ctx = ctx;
+      b->sz = ga_static_scratch_bytes;
+      b->refcnt = 1;
+      b->flags = BUF_INTERNAL;   // not owned (release leaves the memory alone), does not keep the context alive
+      ctx->static_buf = b;
+    }
+  }
 
   {
     const char *dc = p->kernel_cache_path ? p->kernel_cache_path : getenv("GPUARRAY_CACHE_PATH");
@@ -1846,6 +1861,14 @@ gpudata *ga_hip_scratch(gpucontext *c, size_t bytes) {
   ctx->scratch = grown;
   ctx->scratch_sz = want;
   return ctx->scratch;
+}
+
+gpudata *ga_hip_static_scratch_buf(gpucontext *c, const char **why) {
+  hip_context *ctx = HC(c);
+  if (why != nullptr)
+    *why = ctx->static_scratch != nullptr ? (ctx->static_buf ? "" : "out of host memory")
+                                          : hipGetErrorString((hipError_t)ctx->static_scratch_err);
+  return ctx->static_buf;
 }
 
 void *ga_hip_static_scratch(gpucontext *c, const char **why) {

@@ -157,6 +157,8 @@ struct _GpuReduction {
   // the same operation on the type of folded partial results (see fold_rows), made on first use
   GpuReduction *fold_op = nullptr;
   int fold_tc = -1;
+  // (row count, row bytes, widest fold) -> rows per folded row, 0 = no fold
+  std::map<std::array<size_t, 3>, size_t> fold_memo;
   int src_tc() const { return args[arrays[0]].tc; }
   unsigned nsrc() const { return (unsigned)arrays.size(); }
 };
@@ -1382,18 +1384,15 @@ class reduction_call {
     // values first, indices after, both 8-byte aligned
     const int acc_tc = acc_typecode(gr, d0_tc);
     const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
-    // A view of the static scratch array, for calls that may not allocate: a
-    // gpudata is only read through its leading {device pointer, context}.
-    struct { void *devptr; gpucontext *ctx; } static_view = {nullptr, ctx};
     gpudata *scratch = nullptr;
     if (noalloc) {
+      // the static scratch array, for calls that may not allocate
       const char *why = "";
-      static_view.devptr = ga_hip_static_scratch(ctx, &why);
-      if (static_view.devptr == nullptr)
+      scratch = ga_hip_static_scratch_buf(ctx, &why);
+      if (scratch == nullptr)
         return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
                           "GpuReduction_call_noalloc: the static scratch array was not found on "
                           "this device when the context was made (%s)", why);
-      scratch = reinterpret_cast<gpudata *>(&static_view);
     } else {
       scratch = ga_hip_scratch(ctx, scratch_skip + 16);
     }
@@ -1456,11 +1455,11 @@ class reduction_call {
       pi_off = (slots * accsz + 255) & ~(size_t)255;
       const size_t need = pi_off + slots * 8;
       if (noalloc) {
-        if (need > ga_static_scratch_bytes)
+        if (scratch_skip + need > ga_static_scratch_bytes)
           return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
                             "GpuReduction_call_noalloc: this reduction is split into %zu partial "
                             "results that take %zu bytes; the static scratch array holds %zu",
-                            slots, need, (size_t)ga_static_scratch_bytes);
+                            slots, scratch_skip + need, (size_t)ga_static_scratch_bytes);
       } else {
         scratch = ga_hip_scratch(ctx, scratch_skip + need);
       }
@@ -1620,7 +1619,7 @@ void GpuReduction_free(GpuReduction *gr) {
 // folded rows hardly matters (2 KiB to 64 KiB: within 3 us of each other).
 // Returns GA_NO_ERROR with *done = true when the reduction was carried out.
 static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigned reduxLen,
-                     const int *reduxList, bool *done) {
+                     const int *reduxList, bool *done, bool noalloc = false) {
   *done = false;
   gpucontext *ctx = gr->ctx;
   const ga_tuning *tn = ga_hip_tuning(ctx);
@@ -1658,16 +1657,37 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   // Sum over axis 0, folds of 4 KiB / 256 KiB, all launches: (2^22, 10) floats
   // 35.5 / 31.6 us (three launches / two), (2^24, 3) 38.9 / 34.1, (65536, 1001)
   // 49.3 / 46.1, (4096, 4096, 4) over two axes 50.1 / 43.4, (2^20, 17) 20.2 / 16.9.
+  // The search is remembered per (row count, row bytes, widest fold), "no
+  // fold" included: a row count that no candidate divides (a prime one, say)
+  // walks through every candidate, tens of thousands of them, which takes
+  // longer than the kernels that follow; that is paid once per shape, not per
+  // call.  (m0 must divide the row count for any candidate to.)
   size_t m = 0;
   const size_t widest = TUNE(tn, REDUX_FOLD_BYTES, 262144);
-  for (size_t width = widest; m == 0 && width >= 4096; width /= 8)
-    for (size_t t = (width + m0 * rowb - 1) / (m0 * rowb); t * m0 <= 65536; t++)
-      if (R % (t * m0) == 0 && R / (t * m0) >= 64) { m = t * m0; break; }
+  const std::array<size_t, 3> memo_key = {R, rowb, widest};
+  auto memo = gr->fold_memo.find(memo_key);
+  if (memo != gr->fold_memo.end()) {
+    m = memo->second;
+  } else {
+    if (R % m0 == 0)
+      for (size_t width = widest; m == 0 && width >= 4096; width /= 8) {
+        const size_t t0 = (width + m0 * rowb - 1) / (m0 * rowb);
+        for (size_t t = t0; t * m0 <= 65536; t++)
+          if (R % (t * m0) == 0 && R / (t * m0) >= 64) { m = t * m0; break; }
+      }
+    if (gr->fold_memo.size() >= 256) gr->fold_memo.clear();
+    gr->fold_memo[memo_key] = m;
+  }
   if (m <= 1) return GA_NO_ERROR;
 
   // type of the folded partial results: the accumulator's (a half result is summed in float)
   int tmp_tc = acc_typecode(gr, d0->typecode);
   if (tmp_tc == GA_HALF) tmp_tc = GA_FLOAT;
+  if (noalloc && (gr->fold_op == nullptr || gr->fold_tc != tmp_tc))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR,
+                      "GpuReduction_call_noalloc: the kernels for arrays of this layout are not "
+                      "built yet, and building them allocates; run GpuReduction_call once on "
+                      "arrays of this layout first");
   if (gr->fold_op == nullptr || gr->fold_tc != tmp_tc) {
     GpuReduction_free(gr->fold_op);
     gr->fold_op = nullptr;
@@ -1681,7 +1701,22 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   // two calls below put their own partials behind them.
   const size_t tmp_len = m * F;
   const size_t skip = (tmp_len * gpuarray_get_elsize(tmp_tc) + 255) & ~(size_t)255;
-  gpudata *scr = ga_hip_scratch(ctx, skip + 16);
+  gpudata *scr = nullptr;
+  if (noalloc) {
+    const char *why = "";
+    scr = ga_hip_static_scratch_buf(ctx, &why);
+    if (scr == nullptr)
+      return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
+                        "GpuReduction_call_noalloc: the static scratch array was not found on "
+                        "this device when the context was made (%s)", why);
+    if (skip + 16 > ga_static_scratch_bytes)
+      return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
+                        "GpuReduction_call_noalloc: the folded partial results of this reduction "
+                        "take %zu bytes; the static scratch array holds %zu",
+                        skip, (size_t)ga_static_scratch_bytes);
+  } else {
+    scr = ga_hip_scratch(ctx, skip + 16);
+  }
   if (scr == nullptr) return ctx->err->code;
   GpuArray tmp;
   const ssize_t tmp_stride = (ssize_t)gpuarray_get_elsize(tmp_tc);
@@ -1694,7 +1729,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
     srcs[0].a = s0;
     srcs[0].strides = {(ssize_t)(m * rowb), (ssize_t)es};
     const int axis0 = 0;
-    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, srcs, {}, 1, &axis0, false, skip);
+    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, srcs, {}, 1, &axis0, noalloc, skip);
   }
   if (err == GA_NO_ERROR) {
     // second call: tmp as (m, kept dims...) over axis 0 into d0
@@ -1713,7 +1748,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
     srcs[0].a = &tmp;
     srcs[0].strides = str2;
     const int axis0 = 0;
-    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), srcs, {}, 1, &axis0, false, skip);
+    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), srcs, {}, 1, &axis0, noalloc, skip);
   }
   GpuArray_clear(&tmp);
   if (err == GA_NO_ERROR) *done = true;
@@ -1748,6 +1783,13 @@ int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d
   if (gr->nsrc() != 1 || !gr->scalars.empty())
     return ga_err_set(gr->ctx->err, GA_INVALID_ERROR,
                       "GpuReduction_call_noalloc takes operators made by GpuReduction_new");
+  {
+    // the same route as GpuReduction_call, so that the kernels its warm-up
+    // call built are the ones asked for here
+    bool done = false;
+    const int err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done, true);
+    if (err != GA_NO_ERROR || done) return err;
+  }
   std::vector<src_view> srcs(1);
   srcs[0].a = s0;
   srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);

@@ -156,6 +156,9 @@ int ga_static_scratch_setup(int dev, void **ptr);
 // The address found for the context's device when the context was made, NULL
 // when the lookup failed (the reason is then in *why, if not NULL).
 void *ga_hip_static_scratch(gpucontext *ctx, const char **why);
+// The same array as a buffer of the context (made with the context; releasing
+// it never frees anything), NULL when the lookup failed.
+gpudata *ga_hip_static_scratch_buf(gpucontext *ctx, const char **why);
 // Bytes from a buffer's start that lie inside the memory behind it (at least
 // its size; more when the allocation was rounded up).
 size_t ga_hip_readable_bytes(gpudata *b);

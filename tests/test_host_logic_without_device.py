@@ -129,7 +129,8 @@ mock = C.CDLL(os.environ["GA_TEST_MOCK_RUNTIME"])
 calls = C.c_ulong.in_dll(mock, "mock_allocating_calls")
 ctx = ga.init("hip0")
 for dtype, shape, axes, d1 in (("float32", (1 << 22,), [0], False), ("int32", (6, 1 << 18), [1], False),
-                               ("float32", (1 << 14, 256), [0], True), ("float32", (4096, 100), [1], False)):
+                               ("float32", (1 << 14, 256), [0], True), ("float32", (4096, 100), [1], False),
+                               ("float32", (1 << 20, 10), [0], False)):          # folded rows
     op = ga.GpuReduction(ctx, "maxandargmax" if d1 else "sum", dtype)
     src = ga.zeros(shape, dtype, context=ctx)
     oshape = tuple(d for k, d in enumerate(shape) if k not in axes)
@@ -141,6 +142,17 @@ for dtype, shape, axes, d1 in (("float32", (1 << 22,), [0], False), ("int32", (6
         op(src, axes, d0=d0, d1=di, noalloc=True)
     assert calls.value == before, (dtype, shape, calls.value - before)
     op(src, axes, d0=d0, d1=di)
+# a prime row count: no fold divides it; the search for one runs once per shape
+import time
+op = ga.GpuReduction(ctx, "sum", "float32")
+src = ga.zeros((4194319, 10), "float32", context=ctx)
+d0 = ga.empty((10,), "float32", context=ctx)
+op(src, [0], d0=d0)
+t0 = time.perf_counter()
+for _ in range(200):
+    op(src, [0], d0=d0)
+per_call = (time.perf_counter() - t0) / 200
+assert per_call < 100e-6, per_call      # 366 us per call when every call searched again
 print("noalloc ok")
 """
 
