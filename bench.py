@@ -343,7 +343,7 @@ CONFIGS = [
     ("F2_take1_65536x1024_rows", _cfg_take1(True)),
     ("F2_take1_65536x1024_rows_unchecked", _cfg_take1(False)),
 ]
-STEP_MODES = ("step", "elem", "sum", "copy")
+STEP_MODES = ("step", "elem", "sum", "copy", "fill")
 
 
 def measure_config(ctx, name, cfg):
@@ -573,9 +573,10 @@ def main():
     ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count")
     ap.add_argument("--list", action="store_true", help="print the names --only takes")
     ap.add_argument("--only", default="step",
-                    help="launch only one kernel per step (for profiler runs): 'elem', 'sum', or 'copy' "
+                    help="launch only one kernel per step (for profiler runs): 'elem', 'sum', 'copy' "
                          "(a plain copy dst = src of 2^log2n floats whose traffic is known, 4*n read + "
-                         "4*n written, to scale byte counters by), or the name of a per-config entry")
+                         "4*n written, to scale byte counters by), 'fill' (dst = 1.0f: writes only), "
+                         "or the name of a per-config entry")
     args = ap.parse_args()
     names = [n for n, _ in CONFIGS]
     if args.list:
@@ -627,6 +628,7 @@ def main():
     summ = ga.GpuReduction(ctx, "sum", "float32")
     copy = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", "float32", read=True),
                                              ga.arg("dst", "float32", write=True)])
+    fill = ga.GpuElemwise(ctx, "dst = 1.0f", [ga.arg("dst", "float32", write=True)])
     only = args.only
     hashes = {}
     # Below the target size the one-kernel modes rotate over four copies of the
@@ -647,6 +649,8 @@ def main():
             elem(a_, b_, c_)
         elif only == "copy":
             copy(a_, c_)
+        elif only == "fill":
+            fill(c_)
         if i is not None:
             ctx.mark(3 * i + 1)
         if only in ("step", "sum"):
@@ -673,8 +677,8 @@ def main():
 
     if only != "step":
         # profiler run: report the one kernel that was launched and stop
-        ms = elem_ms if only in ("elem", "copy") else sum_ms
-        nbytes = {"elem": elem_bytes, "copy": 8 * n, "sum": sum_bytes}[only]
+        ms = elem_ms if only in ("elem", "copy", "fill") else sum_ms
+        nbytes = {"elem": elem_bytes, "copy": 8 * n, "fill": 4 * n, "sum": sum_bytes}[only]
         kern, launches, khashes = time_kernels(ctx, lambda i: step(), iters=K, warm=0)
         print(json.dumps({"only": only, "launches": K, "avg_launch_us": round(float(ms.mean()) * 1e3, 2),
                           "kernel_us": round(kern, 2), "launches_per_call": launches,
@@ -751,9 +755,7 @@ def main():
                 "median_launch_us": round(float(np.median(elem_ms)) * 1e3, 2),
                 "kernel_us": round(float(elem_kernel_ms.mean()) * 1e3, 2),
                 "kernel_text_hash": "+".join(hashes["elem"]),
-                "frac_clock": "avg_launch_us: two events on the library's stream around each call in the timed "
-                              "region (kernel_us, from events on the dispatch itself, is what a kernel trace "
-                              "reports; frac_kernel is priced on it)",
+                "frac_clock": "avg_launch_us (events around each call; frac_kernel: on kernel_us, a trace's figure)",
                 "frac_kernel": round(elem_bytes / (float(elem_kernel_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "parity": "all 2^%d outputs equal NumPy's" % args.log2n,
                 "algorithmic_bytes_per_launch": elem_bytes}

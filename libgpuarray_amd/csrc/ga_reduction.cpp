@@ -641,18 +641,19 @@ int make_plain_operator(GpuReduction **grp, gpucontext *ctx, ga_errrec *errrec, 
 // extents `dims`; `scalars` point at host values of the declared types.
 struct src_view {
   const GpuArray *a;
-  std::vector<int64_t> strides;
+  const int64_t *strides;   // nd byte strides (an array's own, or 0 where it is broadcast)
 };
+static_assert(sizeof(ssize_t) == sizeof(int64_t), "strides are read through int64_t pointers");
 
 // One call of an operator: argument checks, the dim lists and the plan the
 // kernels read, the choice of kernel family and lane geometry, the launch.
 class reduction_call {
  public:
   reduction_call(GpuReduction *gr_, GpuArray *d0_, GpuArray *d1_, unsigned nd_, const size_t *dims_,
-                 const std::vector<src_view> &srcs_, const std::vector<void *> &scalars_,
+                 const src_view *srcs_, void *const *scalars_, unsigned nscalars_,
                  unsigned reduxLen_, const int *reduxList_, bool noalloc_ = false, size_t scratch_skip_ = 0)
       : noalloc(noalloc_), scratch_skip(scratch_skip_), gr(gr_), ctx(gr_->ctx), tn(ga_hip_tuning(gr_->ctx)), info(gr_->info), K(gr_->nsrc()), d0(d0_), d1(d1_), nd(nd_),
-        dims(dims_), srcs(srcs_), scalars(scalars_), reduxLen(reduxLen_), reduxList(reduxList_),
+        dims(dims_), srcs(srcs_), scalars(scalars_), nscalars(nscalars_), reduxLen(reduxLen_), reduxList(reduxList_),
         kind(info.kind), minmax(kind == K_MIN || kind == K_MAX),
         logical(kind == K_ALL || kind == K_ANY),
         planbuf(plan_bytes(K) / sizeof(int64_t), 0),
@@ -695,8 +696,9 @@ class reduction_call {
   GpuArray *d0, *d1;
   const unsigned nd;
   const size_t *dims;
-  const std::vector<src_view> &srcs;
-  const std::vector<void *> &scalars;
+  const src_view *srcs;             // K of them
+  void *const *scalars;             // nscalars host values, in the operator's order
+  const unsigned nscalars;
   const unsigned reduxLen;
   const int *reduxList;
   const rd_kind kind;
@@ -1379,24 +1381,11 @@ class reduction_call {
     return get_variant(gr, vs, &var, !noalloc);
   }
 
-  int launch() {
-    // partials of a split reduction live in the context's scratch buffer:
-    // values first, indices after, both 8-byte aligned
+  // What is left of the plan once the kernels are chosen: which kernels, how
+  // many groups, how the partials of a split reduction are laid out.
+  int prepare_launch() {
     const int acc_tc = acc_typecode(gr, d0_tc);
     const size_t accsz = logical ? 4 : acc_size_for(acc_tc);
-    gpudata *scratch = nullptr;
-    if (noalloc) {
-      // the static scratch array, for calls that may not allocate
-      const char *why = "";
-      scratch = ga_hip_static_scratch_buf(ctx, &why);
-      if (scratch == nullptr)
-        return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
-                          "GpuReduction_call_noalloc: the static scratch array was not found on "
-                          "this device when the context was made (%s)", why);
-    } else {
-      scratch = ga_hip_scratch(ctx, scratch_skip + 16);
-    }
-    size_t pi_off = 0;
     // A split reduction of moderate size ends in the launch that started it:
     // its outputs (row kernel) or tiles of outputs (column kernel) have a
     // counter each, and the piece that counts in last combines the partials.
@@ -1409,7 +1398,7 @@ class reduction_call {
     // Calls on the static scratch array always take two launches: the second
     // reads only what the first has written, so nothing there has to start
     // at zero.
-    gpudata *done = nullptr;
+    rec.fused = false;
     if (p.nsplit > 1 && !noalloc) {
       const size_t counters = use_row ? (size_t)nrows : groups / (size_t)p.nsplit;
       const size_t fused_max = (size_t)ncu * TUNE(tn, REDUX_FUSED, 1);   // 0 turns it off
@@ -1444,72 +1433,110 @@ class reduction_call {
                        : (!carries_index && p.nsplit <= (int)TUNE(tn, REDUX_FUSED_COL_SPLITS, 16) &&
                           piece_bytes >= (double)TUNE(tn, REDUX_FUSED_COL_PIECE, 128u << 10));
       }
-      if (fuse && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8) &&
-          (done = ga_hip_redux_counters(ctx)) != nullptr) {
-        p.fused = 1;
-        if (!use_row) p.split_major = 1;
+      if (fuse && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8)) {
+        if (ga_hip_redux_counters(ctx) != nullptr) {
+          rec.fused = true;
+          p.fused = 1;
+          if (!use_row) p.split_major = 1;
+        } else {
+          // (no counters while the stream records a graph: two launches now,
+          // and a later call should ask again rather than remember this plan)
+          rec.remember = false;
+        }
       }
     }
+    rec.pi_off = rec.need = 0;
     if (p.nsplit > 1) {
       const size_t slots = (size_t)nrows * (size_t)p.nsplit;
-      pi_off = (slots * accsz + 255) & ~(size_t)255;
-      const size_t need = pi_off + slots * 8;
-      if (noalloc) {
-        if (scratch_skip + need > ga_static_scratch_bytes)
-          return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
-                            "GpuReduction_call_noalloc: this reduction is split into %zu partial "
-                            "results that take %zu bytes; the static scratch array holds %zu",
-                            slots, scratch_skip + need, (size_t)ga_static_scratch_bytes);
-      } else {
-        scratch = ga_hip_scratch(ctx, scratch_skip + need);
-      }
+      rec.pi_off = (slots * accsz + 255) & ~(size_t)255;
+      rec.need = rec.pi_off + slots * 8;
+      if (noalloc && scratch_skip + rec.need > ga_static_scratch_bytes)
+        return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
+                          "GpuReduction_call_noalloc: this reduction is split into %zu partial "
+                          "results that take %zu bytes; the static scratch array holds %zu",
+                          slots, scratch_skip + rec.need, (size_t)ga_static_scratch_bytes);
     }
-    if (scratch == nullptr) return ctx->err->code;
-    if (!p.fused) done = scratch;   // not used then, but the kernels take a pointer
-
-    // A destination the operation does not write still needs a valid pointer.
-    gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
-    size_t d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
-    std::vector<size_t> s_off(K);
-
-    // The two scratch views are passed as (buffer) arguments; the index part
-    // starts pi_off bytes in, which the kernels receive through a second
-    // gpudata wrapping the same memory.
-    struct { void *devptr; gpucontext *ctx; } pv_view = {(char *)scratch->devptr + scratch_skip, ctx};
-    struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + scratch_skip + pi_off, ctx};
-    std::vector<void *> args;
-    for (unsigned q = 0; q < K; q++) {
-      s_off[q] = srcs[q].a->offset;
-      args.push_back(srcs[q].a->data);
-      args.push_back(&s_off[q]);
-    }
-    args.push_back(d0b);
-    args.push_back(&d0_off);
-    args.push_back(d1b);
-    args.push_back(&d1_off);
-    args.push_back(&pv_view);
-    args.push_back(&pi_view);
-    args.push_back(done);
-    args.push_back(planbuf.data());
-    for (void *sc : scalars) args.push_back(sc);
-    size_t ls = 256;
-    GpuKernel *k1 = trows ? &var->trows : srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
-    int err;
-    if ((err = GpuKernel_call(k1, 1, &groups, &ls, lds_bytes, args.data())) != GA_NO_ERROR) return err;
-    if (p.nsplit > 1 && !p.fused) {
-      size_t fg = (size_t)(p.split_major ? (nrows + 63) / 64 : (nrows + 3) / 4);
-      if ((err = GpuKernel_call(p.split_major ? &var->fin_cols : &var->fin, 1, &fg, &ls, 0,
-                                args.data())) != GA_NO_ERROR)
-        return err;
+    rec.k1 = trows ? &var->trows : srows ? &var->srows : use_row ? (wrows ? &var->wrows : &var->row) : &var->col;
+    rec.k2 = nullptr;
+    rec.groups = groups;
+    rec.lds_bytes = lds_bytes;
+    rec.fin_groups = 0;
+    if (p.nsplit > 1 && !rec.fused) {
+      rec.k2 = p.split_major ? &var->fin_cols : &var->fin;
+      rec.fin_groups = (size_t)(p.split_major ? (nrows + 63) / 64 : (nrows + 3) / 4);
     }
     return GA_NO_ERROR;
   }
 };
 
+// The launches of a planned call.  `plan` is the kernels' by-value plan
+// argument; partials of a split reduction live in the context's scratch buffer
+// (in the device's static scratch array for a call that may not allocate):
+// values first, indices after, both 8-byte aligned, `scratch_skip` bytes in.
+int issue_launches(gpucontext *ctx, const launch_rec &rec, const void *plan, unsigned K, const src_view *srcs,
+                   GpuArray *d0, GpuArray *d1, void *const *scalars, unsigned nscalars, bool noalloc,
+                   size_t scratch_skip) {
+  gpudata *scratch = nullptr;
+  if (noalloc) {
+    const char *why = "";
+    scratch = ga_hip_static_scratch_buf(ctx, &why);
+    if (scratch == nullptr)
+      return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
+                        "GpuReduction_call_noalloc: the static scratch array was not found on "
+                        "this device when the context was made (%s)", why);
+  } else {
+    scratch = ga_hip_scratch(ctx, scratch_skip + (rec.need > 16 ? rec.need : 16));
+  }
+  if (scratch == nullptr) return ctx->err->code;
+  // the counters of a launch that finishes itself; a pointer the kernels take but do not use otherwise
+  gpudata *done = rec.fused ? ga_hip_redux_counters(ctx) : scratch;
+  if (done == nullptr) return ctx->err->code;
+
+  // A destination the operation does not write still needs a valid pointer.
+  gpudata *d0b = d0 ? d0->data : scratch, *d1b = d1 ? d1->data : scratch;
+  size_t d0_off = d0 ? d0->offset : 0, d1_off = d1 ? d1->offset : 0;
+  size_t s_off[RD_MAXSRC];
+  // The two scratch views are passed as (buffer) arguments; the index part
+  // starts pi_off bytes in, which the kernels receive through a second
+  // gpudata wrapping the same memory (a kernel argument is only read through
+  // the leading {device pointer, context} of a gpudata).
+  struct { void *devptr; gpucontext *ctx; } pv_view = {(char *)scratch->devptr + scratch_skip, ctx};
+  struct { void *devptr; gpucontext *ctx; } pi_view = {(char *)scratch->devptr + scratch_skip + rec.pi_off, ctx};
+  constexpr unsigned MAXSCALARS = 32;
+  void *fixed[2 * RD_MAXSRC + 8 + MAXSCALARS];
+  std::vector<void *> many;
+  void **args = fixed;
+  if (nscalars > MAXSCALARS) {
+    many.resize(2 * RD_MAXSRC + 8 + nscalars);
+    args = many.data();
+  }
+  unsigned n = 0;
+  for (unsigned q = 0; q < K; q++) {
+    s_off[q] = srcs[q].a->offset;
+    args[n++] = srcs[q].a->data;
+    args[n++] = &s_off[q];
+  }
+  args[n++] = d0b;
+  args[n++] = &d0_off;
+  args[n++] = d1b;
+  args[n++] = &d1_off;
+  args[n++] = &pv_view;
+  args[n++] = &pi_view;
+  args[n++] = done;
+  args[n++] = const_cast<void *>(plan);
+  for (unsigned i = 0; i < nscalars; i++) args[n++] = scalars[i];
+  size_t ls = 256, g1 = rec.groups, g2 = rec.fin_groups;
+  int err;
+  if ((err = GpuKernel_call(rec.k1, 1, &g1, &ls, rec.lds_bytes, args)) != GA_NO_ERROR) return err;
+  if (rec.k2 != nullptr && (err = GpuKernel_call(rec.k2, 1, &g2, &ls, 0, args)) != GA_NO_ERROR) return err;
+  return GA_NO_ERROR;
+}
+
 int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
-                  const std::vector<src_view> &srcs, const std::vector<void *> &scalars,
+                  const src_view *srcs, void *const *scalars, unsigned nscalars,
                   unsigned reduxLen, const int *reduxList, bool noalloc = false, size_t scratch_skip = 0) {
-  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, reduxLen, reduxList, noalloc, scratch_skip).run();
+  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, nscalars, reduxLen, reduxList, noalloc,
+                        scratch_skip).run();
 }
 
 }  // namespace
@@ -1725,30 +1752,28 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   {
     // first call: (R / m, m F) over axis 0 into tmp
     const size_t dims1[2] = {R / m, m * F};
-    std::vector<src_view> srcs(1);
-    srcs[0].a = s0;
-    srcs[0].strides = {(ssize_t)(m * rowb), (ssize_t)es};
+    const int64_t str1[2] = {(int64_t)(m * rowb), (int64_t)es};
+    const src_view src = {s0, str1};
     const int axis0 = 0;
-    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, srcs, {}, 1, &axis0, noalloc, skip);
+    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, &src, nullptr, 0, 1, &axis0, noalloc, skip);
   }
   if (err == GA_NO_ERROR) {
     // second call: tmp as (m, kept dims...) over axis 0 into d0
     std::vector<size_t> dims2(1 + d0->nd);
-    std::vector<ssize_t> str2(1 + d0->nd);
+    std::vector<int64_t> str2(1 + d0->nd);
     const size_t tes = gpuarray_get_elsize(tmp_tc);
     dims2[0] = m;
     size_t run = tes;
     for (unsigned j = d0->nd; j-- > 0;) {
       dims2[1 + j] = d0->dimensions[j];
-      str2[1 + j] = (ssize_t)run;
+      str2[1 + j] = (int64_t)run;
       run *= d0->dimensions[j];
     }
-    str2[0] = (ssize_t)run;
-    std::vector<src_view> srcs(1);
-    srcs[0].a = &tmp;
-    srcs[0].strides = str2;
+    str2[0] = (int64_t)run;
+    const src_view src = {&tmp, str2.data()};
     const int axis0 = 0;
-    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), srcs, {}, 1, &axis0, noalloc, skip);
+    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), &src, nullptr, 0, 1, &axis0,
+                        noalloc, skip);
   }
   GpuArray_clear(&tmp);
   if (err == GA_NO_ERROR) *done = true;
@@ -1768,10 +1793,8 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     const int err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done);
     if (err != GA_NO_ERROR || done) return err;
   }
-  std::vector<src_view> srcs(1);
-  srcs[0].a = s0;
-  srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);
-  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, srcs, {}, reduxLen, reduxList);
+  const src_view src = {s0, (const int64_t *)s0->strides};
+  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, &src, nullptr, 0, reduxLen, reduxList);
 }
 
 int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1,
@@ -1790,10 +1813,8 @@ int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d
     const int err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done, true);
     if (err != GA_NO_ERROR || done) return err;
   }
-  std::vector<src_view> srcs(1);
-  srcs[0].a = s0;
-  srcs[0].strides.assign(s0->strides, s0->strides + s0->nd);
-  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, srcs, {}, reduxLen, reduxList, true);
+  const src_view src = {s0, (const int64_t *)s0->strides};
+  return reduce_launch(gr, d0, d1, s0->nd, s0->dimensions, &src, nullptr, 0, reduxLen, reduxList, true);
 }
 
 int GpuReduction_call_map(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, void **args,
@@ -1834,13 +1855,16 @@ int GpuReduction_call_map(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, v
     }
     dims[ax] = d;
   }
+  std::vector<int64_t> strides((size_t)K * (nd ? nd : 1));
   for (unsigned q = 0; q < K; q++) {
     const GpuArray *a = srcs[q].a;
-    srcs[q].strides.resize(nd);
+    int64_t *st = strides.data() + (size_t)q * nd;
     for (unsigned ax = 0; ax < nd; ax++)
-      srcs[q].strides[ax] = a->dimensions[ax] == dims[ax] ? (int64_t)a->strides[ax] : 0;
+      st[ax] = a->dimensions[ax] == dims[ax] ? (int64_t)a->strides[ax] : 0;
+    srcs[q].strides = st;
   }
-  return reduce_launch(gr, d0, d1, nd, dims.data(), srcs, scalars, reduxLen, reduxList);
+  return reduce_launch(gr, d0, d1, nd, dims.data(), srcs.data(), scalars.data(), (unsigned)scalars.size(),
+                       reduxLen, reduxList);
 }
 
 // Reference entry point (src/gpuarray_reduction.c:100-124).  The operator is
