@@ -8,11 +8,13 @@ the part of the reference's Python layer that drives this path:
   reduction  sum/prod/all/any/min/max/arg* (pygpu/reduction.py, pygpu/_array.py)
   _array     ndgpuarray: NumPy operators   (pygpu/_array.py)
   dtypes     C spellings, promotion        (pygpu/dtypes.py)
+  operations split / stack family          (pygpu/operations.py)
+  basic      triu / tril via GpuKernel     (pygpu/basic.py)
   tools      argument descriptors, check_args, lru_cache (pygpu/tools.py)
 """
 from . import _lib
 from ._lib import GpuArrayException, UnsupportedException, LIB_PATH
-from . import gpuarray, elemwise, reduction, tools
+from . import gpuarray, elemwise, reduction, operations, basic, tools
 from .gpuarray import (GpuContext, GpuArray, GpuKernel, init, array, asarray, empty, zeros, zeros_like,
                        empty_like, ascontiguousarray, asfortranarray, may_share_memory,
                        set_default_context, get_default_context, count_devices, count_platforms,

@@ -83,6 +83,38 @@ const char *chunk_type(size_t bytes) {
 
 }  // namespace
 
+// One planned launch: the kernel, its geometry and where each of its
+// arguments comes from - a value fixed by the plan, the buffer of an array
+// argument of the call, or a scalar argument of the call.
+struct ew_slot {
+  enum : unsigned char { VALUE, ARRAY, SCALAR } kind;
+  unsigned char arg;   // ARRAY / SCALAR: position among the call's arguments
+  int64_t value;       // VALUE: the bytes of a 4- or 8-byte kernel argument
+};
+struct ew_launch {
+  GpuKernel *k = nullptr;
+  size_t gs = 0, ls = 0;
+  std::vector<ew_slot> slots;
+  bool valid = false;
+  void value(const void *p, size_t bytes) {
+    ew_slot s = {ew_slot::VALUE, 0, 0};
+    memcpy(&s.value, p, bytes);
+    slots.push_back(s);
+  }
+  template <class T> void value(const T &v) { static_assert(sizeof(T) <= 8, ""); value(&v, sizeof(T)); }
+  void array(size_t arg) { slots.push_back(ew_slot{ew_slot::ARRAY, (unsigned char)arg, 0}); }
+  void scalar(size_t arg) { slots.push_back(ew_slot{ew_slot::SCALAR, (unsigned char)arg, 0}); }
+};
+// A planned call kept with its operator.  The key lists every input of the
+// planners: the call's flags, the tuning table's generation and, per array,
+// rank, extents, strides, offset, flags and the alignment of the buffer's base.
+constexpr unsigned EW_KEYMAX = 176, EW_ENTRIES = 4;
+struct ew_memo {
+  unsigned nkey = 0;
+  int64_t key[EW_KEYMAX];
+  ew_launch launch;
+};
+
 struct _GpuElemwise {
   gpucontext *ctx = nullptr;
   std::string expr, preamble;
@@ -109,6 +141,9 @@ struct _GpuElemwise {
   std::vector<size_t> dims;
   std::vector<std::vector<ssize_t>> strs;
   std::vector<ssize_t *> strp;
+  ew_launch pending;             // what the planners leave for GpuElemwise_call to launch
+  std::vector<ew_memo> memo;     // planned calls
+  unsigned memo_next = 0;        // the entry the next new plan replaces once all are taken
 };
 
 namespace {
@@ -1135,37 +1170,39 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
   const bool tile = tiled_u ? true : ge->tile;
   const unsigned unroll = tiled_u ? tiled_u : ge->unroll;
 
-  unsigned p = 0;
+  if (ge->args.size() > 255)
+    return ga_err_set(ge->ctx->err, GA_UNSUPPORTED_ERROR, "More than 255 arguments");
+  ew_launch &L = ge->pending;
+  L.slots.clear();
   l = 0;
-  if ((err = GpuKernel_setarg(k, p++, &n)) != GA_NO_ERROR) return err;
+  L.value(n);
   for (size_t i = 0; i < ge->args.size(); i++) {
     if (ge->args[i].is_array()) {
-      GpuArray *a = (GpuArray *)args[i];
-      size_t off = offs[l++];
-      if ((err = GpuKernel_setarg(k, p++, a->data)) != GA_NO_ERROR) return err;
-      if ((err = GpuKernel_setarg(k, p++, &off)) != GA_NO_ERROR) return err;
+      L.array(i);
+      L.value(offs[l++]);
     } else {
-      if ((err = GpuKernel_setarg(k, p++, args[i])) != GA_NO_ERROR) return err;
+      L.scalar(i);
     }
   }
-  if ((err = GpuKernel_setarg(k, p++, &vec_arg)) != GA_NO_ERROR) return err;
+  L.value(vec_arg);
   if (pi != nullptr) {
-    GpuKernel_setarg(k, p++, (void *)&pi->d1);
-    GpuKernel_setarg(k, p++, (void *)&pi->d2);
-    GpuKernel_setarg(k, p++, (void *)&pi->m1);
-    GpuKernel_setarg(k, p++, (void *)&pi->k1);
-    GpuKernel_setarg(k, p++, (void *)&pi->m2);
-    GpuKernel_setarg(k, p++, (void *)&pi->k2);
+    L.value(pi->d1);
+    L.value(pi->d2);
+    L.value(pi->m1);
+    L.value(pi->k1);
+    L.value(pi->m2);
+    L.value(pi->k2);
     for (size_t q = 0; q < pi->ps.size(); q++)
       if ((pi->pmask >> q) & 1u)
-        for (int j = 0; j < 3; j++)
-          if ((err = GpuKernel_setarg(k, p++, (void *)&pi->ps[q][j])) != GA_NO_ERROR) return err;
+        for (int j = 0; j < 3; j++) L.value(pi->ps[q][j]);
   }
   size_t per_group = GE_LANES * (size_t)((vec_ok && tile) ? unroll : 1);
   size_t want = (units + per_group - 1) / per_group;
-  size_t gs = want < 1 ? 1 : (want > cap ? cap : want);
-  size_t ls = GE_LANES;
-  return GpuKernel_call(k, 1, &gs, &ls, 0, nullptr);
+  L.k = k;
+  L.gs = want < 1 ? 1 : (want > cap ? cap : want);
+  L.ls = GE_LANES;
+  L.valid = true;
+  return GA_NO_ERROR;
 }
 
 // ---- general path ---------------------------------------------------------------
@@ -1627,28 +1664,33 @@ class strided_call {
     return GA_NO_ERROR;
   }
 
+  // (leaves the launch to GpuElemwise_call, see ew_launch)
   int launch() {
-    unsigned p = 0, l = 0;
-    int err;
-    for (unsigned j = 0; j < nd; j++)
-      if ((err = GpuKernel_setarg(kernel, p++, &dims[j])) != GA_NO_ERROR) return err;
+    if (ge->args.size() > 255)
+      return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR, "More than 255 arguments");
+    ew_launch &L = ge->pending;
+    L.slots.clear();
+    unsigned l = 0;
+    for (unsigned j = 0; j < nd; j++) L.value(dims[j]);
     for (size_t i = 0; i < ge->args.size(); i++) {
       if (ge->args[i].is_array()) {
-        GpuArray *v = (GpuArray *)args[i];
-        if ((err = GpuKernel_setarg(kernel, p++, v->data)) != GA_NO_ERROR) return err;
-        if ((err = GpuKernel_setarg(kernel, p++, &v->offset)) != GA_NO_ERROR) return err;
-        for (unsigned j = 0; j < nd; j++)
-          if ((err = GpuKernel_setarg(kernel, p++, &strs[l][j])) != GA_NO_ERROR) return err;
+        const GpuArray *v = (const GpuArray *)args[i];
+        L.array(i);
+        L.value(v->offset);
+        for (unsigned j = 0; j < nd; j++) L.value(strs[l][j]);
         l++;
       } else {
-        if ((err = GpuKernel_setarg(kernel, p++, args[i])) != GA_NO_ERROR) return err;
+        L.scalar(i);
       }
     }
-    unsigned int gx32 = (unsigned int)gx;
-    if ((err = GpuKernel_setarg(kernel, p++, &gx32)) != GA_NO_ERROR) return err;
-    if ((err = GpuKernel_setarg(kernel, p++, &ltx)) != GA_NO_ERROR) return err;
-    size_t ls = (vec4 && tmask) ? (size_t)tile * tile / 16 : 256;
-    return GpuKernel_call(kernel, 1, &groups, &ls, 0, nullptr);
+    const unsigned int gx32 = (unsigned int)gx;
+    L.value(gx32);
+    L.value(ltx);
+    L.k = kernel;
+    L.gs = groups;
+    L.ls = (vec4 && tmask) ? (size_t)tile * tile / 16 : 256;
+    L.valid = true;
+    return GA_NO_ERROR;
   }
 };
 
@@ -1786,7 +1828,46 @@ void GpuElemwise_free(GpuElemwise *ge) {
   delete ge;
 }
 
-int GpuElemwise_call(GpuElemwise *ge, void **args, int flags) {
+namespace {
+
+int ew_issue(const ew_launch &L, void **args) {
+  void *fixed[96];
+  std::vector<void *> many;
+  void **argv = fixed;
+  if (L.slots.size() > 96) {
+    many.resize(L.slots.size());
+    argv = many.data();
+  }
+  for (size_t i = 0; i < L.slots.size(); i++) {
+    const ew_slot &s = L.slots[i];
+    argv[i] = s.kind == ew_slot::VALUE ? (void *)&s.value
+              : s.kind == ew_slot::ARRAY ? (void *)((GpuArray *)args[s.arg])->data : args[s.arg];
+  }
+  return GpuKernel_call(L.k, 1, &L.gs, &L.ls, 0, argv);
+}
+
+// The key of a call (see ew_memo); 0 when the call is not one to remember.
+unsigned ew_key(const GpuElemwise *ge, void **args, int flags, int64_t *key) {
+  if (ge->narray > 8 || ge->args.size() > 255) return 0;
+  unsigned n = 0;
+  key[n++] = flags;
+  key[n++] = (int64_t)ga_hip_tuning(ge->ctx)->generation;
+  for (size_t i = 0; i < ge->args.size(); i++) {
+    if (!ge->args[i].is_array()) continue;
+    const GpuArray *v = (const GpuArray *)args[i];
+    if (v == nullptr || v->data == nullptr || v->nd > 8) return 0;
+    key[n++] = (int64_t)v->nd | ((int64_t)(unsigned)v->flags << 8) | ((int64_t)v->typecode << 40);
+    for (unsigned j = 0; j < v->nd; j++) {
+      key[n++] = (int64_t)v->dimensions[j];
+      key[n++] = (int64_t)v->strides[j];
+    }
+    key[n++] = (int64_t)v->offset;
+    key[n++] = (int64_t)((uintptr_t)v->data->devptr & 255u);
+  }
+  return n;   // at most 2 + 8 * (3 + 16) = 154
+}
+
+int ew_plan(GpuElemwise *ge, void **args, int flags) {
   size_t n = 0;
   bool flat = false;
   if (check_flat(ge, args, &n, &flat) == GA_NO_ERROR && flat) {
@@ -1802,6 +1883,58 @@ int GpuElemwise_call(GpuElemwise *ge, void **args, int flags) {
   if (err != GA_NO_ERROR) return err;
   if (n == 0) return GA_NO_ERROR;
   return call_general(ge, args, n, nd);
+}
+
+}  // namespace
+
+int GpuElemwise_call(GpuElemwise *ge, void **args, int flags) {
+  // ELEMWISE_MEMO: 0 plans every call anew; 2 plans every call anew and
+  // compares with the kept plan where there is one (a difference is a planner
+  // input missing from the key: the process stops)
+  const unsigned long mode = TUNE(ga_hip_tuning(ge->ctx), ELEMWISE_MEMO, 1);
+  int64_t key[EW_KEYMAX];
+  const unsigned nkey = mode ? ew_key(ge, args, flags, key) : 0;
+  ew_memo *hit = nullptr;
+  if (nkey != 0) {
+    for (size_t i = 0; i < ge->memo.size(); i++) {
+      ew_memo &m = ge->memo[i];
+      if (m.nkey == nkey && memcmp(m.key, key, nkey * sizeof(int64_t)) == 0) {
+        hit = &m;
+        break;
+      }
+    }
+  }
+  if (hit != nullptr && mode != 2) return ew_issue(hit->launch, args);
+  ge->pending.valid = false;
+  const int err = ew_plan(ge, args, flags);
+  if (err != GA_NO_ERROR || !ge->pending.valid) {   // (an empty iteration space launches nothing)
+    if (hit != nullptr) {
+      fprintf(stderr, "libgpuarray: a remembered elementwise plan exists for a call that planning refuses (%d)\n", err);
+      abort();
+    }
+    return err;
+  }
+  const ew_launch &L = ge->pending;
+  if (hit != nullptr) {
+    const ew_launch &H = hit->launch;
+    bool same = H.k == L.k && H.gs == L.gs && H.ls == L.ls && H.slots.size() == L.slots.size();
+    for (size_t i = 0; same && i < L.slots.size(); i++)
+      same = H.slots[i].kind == L.slots[i].kind && H.slots[i].arg == L.slots[i].arg &&
+             H.slots[i].value == L.slots[i].value;
+    if (!same) {
+      fprintf(stderr, "libgpuarray: a remembered elementwise plan differs from the plan made anew\n");
+      abort();
+    }
+  } else if (nkey != 0) {
+    // a few entries, replaced in turn once all are taken
+    const bool room = ge->memo.size() < EW_ENTRIES;
+    if (room) ge->memo.emplace_back();
+    ew_memo &m = room ? ge->memo.back() : ge->memo[ge->memo_next++ % EW_ENTRIES];
+    m.nkey = nkey;
+    memcpy(m.key, key, nkey * sizeof(int64_t));
+    m.launch = L;
+  }
+  return ew_issue(L, args);
 }
 
 }  // extern "C"

@@ -1916,6 +1916,13 @@ size_t ga_hip_readable_bytes(gpudata *b) {
   return (d->sz + 15) & ~(size_t)15;             // straight from the driver
 }
 
+void ga_hip_buf_info(gpudata *b, uintptr_t *devptr, size_t *size, size_t *readable) {
+  hip_data *d = HD(b);
+  *devptr = (uintptr_t)d->devptr;
+  *size = d->sz;
+  *readable = d->block != nullptr ? d->block->size : !(d->flags & BUF_OWNED) ? d->sz : ((d->sz + 15) & ~(size_t)15);
+}
+
 unsigned int ga_hip_numprocs(gpucontext *c) { return HC(c)->numprocs; }
 const ga_tuning *ga_hip_tuning(gpucontext *c) { return c ? &HC(c)->tuning : ga_tuning_default(); }
 
@@ -1925,6 +1932,8 @@ const ga_tuning *ga_tuning_default() {
 }
 
 void ga_tuning_read(ga_tuning *t) {
+  static std::atomic<unsigned long> generations{0};
+  t->generation = ++generations;
   static const char *const names[GA_NKNOBS] = {
 #define X(name) "GPUARRAY_" #name,
       GA_KNOBS(X)

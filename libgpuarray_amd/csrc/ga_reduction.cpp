@@ -132,6 +132,28 @@ struct dimrec {
   int64_t smax;                      // largest |source stride|: the sort key
 };
 
+// What the launches of a planned call need besides the plan itself.
+struct launch_rec {
+  GpuKernel *k1 = nullptr, *k2 = nullptr;   // first launch; second pass of a split reduction, or NULL
+  size_t groups = 0, fin_groups = 0, lds_bytes = 0;
+  size_t pi_off = 0, need = 0;   // partials of a split reduction: offset of the indices, bytes in all
+  bool fused = false;            // the first launch finishes the reduction itself (counters)
+  bool remember = true;          // false: planned under a passing condition, plan again next time
+};
+
+// A planned call kept with its operator.  The key lists every input of the
+// planners: extents, axes, the layout of every array (strides, offset,
+// alignment of the base address, flags, type), the sizes of the sources'
+// buffers, the tuning table's generation, the scratch arrangement.  A call
+// whose key equals a kept one launches with the kept plan.
+constexpr unsigned MEMO_KEYMAX = 160, MEMO_ENTRIES = 4;
+struct call_memo {
+  unsigned nkey = 0;
+  int64_t key[MEMO_KEYMAX];
+  std::vector<int64_t> plan;
+  launch_rec rec;
+};
+
 struct rd_arg {
   std::string name;
   int tc;
@@ -159,6 +181,9 @@ struct _GpuReduction {
   int fold_tc = -1;
   // (row count, row bytes, widest fold) -> rows per folded row, 0 = no fold
   std::map<std::array<size_t, 3>, size_t> fold_memo;
+  // planned calls, and the entry the next new plan replaces once all are taken
+  std::vector<call_memo> memo;
+  unsigned memo_next = 0;
   int src_tc() const { return args[arrays[0]].tc; }
   unsigned nsrc() const { return (unsigned)arrays.size(); }
 };
@@ -645,6 +670,10 @@ struct src_view {
 };
 static_assert(sizeof(ssize_t) == sizeof(int64_t), "strides are read through int64_t pointers");
 
+int issue_launches(gpucontext *ctx, const launch_rec &rec, const void *plan, unsigned K, const src_view *srcs,
+                   GpuArray *d0, GpuArray *d1, void *const *scalars, unsigned nscalars, bool noalloc,
+                   size_t scratch_skip);
+
 // One call of an operator: argument checks, the dim lists and the plan the
 // kernels read, the choice of kernel family and lane geometry, the launch.
 class reduction_call {
@@ -678,8 +707,16 @@ class reduction_call {
       col_geometry();
     }
     if ((err = pick_variant()) != GA_NO_ERROR) return err;
-    return launch();
+    if ((err = prepare_launch()) != GA_NO_ERROR) return err;
+    planned = true;
+    if (plan_only) return GA_NO_ERROR;
+    return issue_launches(ctx, rec, planbuf.data(), K, srcs, d0, d1, scalars, nscalars, noalloc, scratch_skip);
   }
+
+  // what the planning left (valid when `planned`: arguments fine, something to launch)
+  bool plan_only = false, planned = false;
+  launch_rec rec;
+  const std::vector<int64_t> &plan() const { return planbuf; }
 
  private:
   // true: partials go to the device's static scratch array, kernels must be
@@ -1532,11 +1569,109 @@ int issue_launches(gpucontext *ctx, const launch_rec &rec, const void *plan, uns
   return GA_NO_ERROR;
 }
 
+// The key of a call (see call_memo); 0 when the call is not one to remember:
+// more dims or sources than the key has room for, or an argument that the
+// checks of the planned path must report.
+unsigned memo_key(GpuReduction *gr, const GpuArray *d0, const GpuArray *d1, unsigned nd, const size_t *dims,
+                  const src_view *srcs, unsigned reduxLen, const int *reduxList, bool noalloc,
+                  size_t scratch_skip, int64_t *key) {
+  const unsigned K = gr->nsrc();
+  if (nd == 0 || nd > 8 || K > 4 || reduxLen == 0 || reduxLen > nd || reduxList == nullptr) return 0;
+  gpucontext *ctx = gr->ctx;
+  unsigned n = 0;
+  key[n++] = (int64_t)nd | ((int64_t)reduxLen << 8) | ((int64_t)K << 16) | ((int64_t)(noalloc ? 1 : 0) << 24) |
+             ((int64_t)(d0 ? 1 : 0) << 25) | ((int64_t)(d1 ? 1 : 0) << 26);
+  key[n++] = (int64_t)scratch_skip;
+  key[n++] = (int64_t)ga_hip_tuning(ctx)->generation;
+  for (unsigned i = 0; i < nd; i++) key[n++] = (int64_t)dims[i];
+  for (unsigned i = 0; i < reduxLen; i++) key[n++] = reduxList[i];
+  for (unsigned q = 0; q < K; q++) {
+    const GpuArray *a = srcs[q].a;
+    if (a == nullptr || a->data == nullptr || gpudata_context(a->data) != ctx) return 0;
+    for (unsigned i = 0; i < nd; i++) key[n++] = srcs[q].strides[i];
+    size_t sz = 0, readable = 0;
+    uintptr_t base = 0;
+    ga_hip_buf_info(a->data, &base, &sz, &readable);
+    key[n++] = (int64_t)a->offset;
+    key[n++] = (int64_t)(unsigned)a->flags | ((int64_t)a->typecode << 32);
+    key[n++] = (int64_t)(base & 255u);
+    key[n++] = (int64_t)sz;
+    key[n++] = (int64_t)readable;
+  }
+  for (const GpuArray *d : {d0, d1}) {
+    if (d == nullptr) continue;
+    if (d->data == nullptr || gpudata_context(d->data) != ctx || d->nd > 8) return 0;
+    key[n++] = (int64_t)d->nd | ((int64_t)d->typecode << 32);
+    key[n++] = (int64_t)(unsigned)d->flags;
+    for (unsigned i = 0; i < d->nd; i++) {
+      key[n++] = (int64_t)d->dimensions[i];
+      key[n++] = (int64_t)d->strides[i];
+    }
+    size_t sz = 0, readable = 0;
+    uintptr_t base = 0;
+    ga_hip_buf_info(d->data, &base, &sz, &readable);
+    key[n++] = (int64_t)d->offset;
+    key[n++] = (int64_t)(base & 255u);
+  }
+  return n;   // at most 3 + 8 + 8 + 4 * (8 + 5) + 2 * (2 + 16 + 2) = 111
+}
+
 int reduce_launch(GpuReduction *gr, GpuArray *d0, GpuArray *d1, unsigned nd, const size_t *dims,
                   const src_view *srcs, void *const *scalars, unsigned nscalars,
                   unsigned reduxLen, const int *reduxList, bool noalloc = false, size_t scratch_skip = 0) {
-  return reduction_call(gr, d0, d1, nd, dims, srcs, scalars, nscalars, reduxLen, reduxList, noalloc,
-                        scratch_skip).run();
+  gpucontext *ctx = gr->ctx;
+  // REDUX_MEMO: 0 plans every call anew; 2 plans every call anew and compares
+  // with the kept plan where there is one (a difference is a planner input
+  // missing from the key: the process stops)
+  const unsigned long mode = TUNE(ga_hip_tuning(ctx), REDUX_MEMO, 1);
+  if (!gr->info.has_d0) d0 = nullptr;
+  if (!gr->info.has_d1) d1 = nullptr;
+  int64_t key[MEMO_KEYMAX];
+  const unsigned nkey = mode ? memo_key(gr, d0, d1, nd, dims, srcs, reduxLen, reduxList, noalloc,
+                                        scratch_skip, key) : 0;
+  call_memo *hit = nullptr;
+  if (nkey != 0) {
+    for (size_t i = 0; i < gr->memo.size(); i++) {
+      call_memo &m = gr->memo[i];
+      if (m.nkey == nkey && memcmp(m.key, key, nkey * sizeof(int64_t)) == 0) {
+        hit = &m;
+        break;
+      }
+    }
+  }
+  if (hit != nullptr && mode != 2)
+    return issue_launches(ctx, hit->rec, hit->plan.data(), gr->nsrc(), srcs, d0, d1, scalars, nscalars,
+                          noalloc, scratch_skip);
+  reduction_call call(gr, d0, d1, nd, dims, srcs, scalars, nscalars, reduxLen, reduxList, noalloc, scratch_skip);
+  call.plan_only = true;
+  int err = call.run();
+  if (err != GA_NO_ERROR || !call.planned) {
+    if (hit != nullptr) {
+      fprintf(stderr, "libgpuarray: a remembered reduction plan exists for a call that planning refuses (%d)\n", err);
+      abort();
+    }
+    return err;
+  }
+  if (hit != nullptr) {
+    const launch_rec &a = hit->rec, &b = call.rec;
+    if (hit->plan != call.plan() || a.k1 != b.k1 || a.k2 != b.k2 || a.groups != b.groups ||
+        a.fin_groups != b.fin_groups || a.lds_bytes != b.lds_bytes || a.pi_off != b.pi_off ||
+        a.need != b.need || a.fused != b.fused) {
+      fprintf(stderr, "libgpuarray: a remembered reduction plan differs from the plan made anew\n");
+      abort();
+    }
+  } else if (nkey != 0 && call.rec.remember) {
+    // a few entries, replaced in turn once all are taken
+    const bool room = gr->memo.size() < MEMO_ENTRIES;
+    if (room) gr->memo.emplace_back();
+    call_memo &m = room ? gr->memo.back() : gr->memo[gr->memo_next++ % MEMO_ENTRIES];
+    m.nkey = nkey;
+    memcpy(m.key, key, nkey * sizeof(int64_t));
+    m.plan = call.plan();
+    m.rec = call.rec;
+  }
+  return issue_launches(ctx, call.rec, call.plan().data(), gr->nsrc(), srcs, d0, d1, scalars, nscalars,
+                        noalloc, scratch_skip);
 }
 
 }  // namespace

@@ -162,6 +162,8 @@ gpudata *ga_hip_static_scratch_buf(gpucontext *ctx, const char **why);
 // Bytes from a buffer's start that lie inside the memory behind it (at least
 // its size; more when the allocation was rounded up).
 size_t ga_hip_readable_bytes(gpudata *b);
+// Device address, size and readable bytes (as above) of a buffer, in one call.
+void ga_hip_buf_info(gpudata *b, uintptr_t *devptr, size_t *size, size_t *readable);
 // Number of compute units of the context's device.
 unsigned int ga_hip_numprocs(gpucontext *ctx);
 // Frees the strided-copy operator cache of a context (array.cpp).

@@ -1,6 +1,6 @@
 """Kernel times of common array shapes, against the bytes they must move.
 
-    python -m libgpuarray_amd.shapes_bench [--only elemwise|reductions] [--iters N]
+    python shapes_bench.py [--only elemwise|reductions] [--iters N]
 
 The benchmark of the repository (bench.py) prices one large contiguous
 elementwise kernel and one full sum.  This walks through the shapes that

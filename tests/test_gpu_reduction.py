@@ -803,8 +803,6 @@ def test_several_outputs_per_lane(ctx, dtype):
     # take 8 or 16 lane rows)
     shapes = ((300, 1000), (8, 4096), (1000, 256), (37, 20), (513, 772), (4, 64, 260), (2000, 8192),
               (5, 300, 4096), (3000, 64), (7, 1500, 32), (1201, 16), (900, 8), (4000, 100))
-    if dtype not in ("float32", "uint8"):      # every shape on two types, every other one on the rest
-        shapes = shapes[::2] if dtype in ("int32", "int16", "float16") else shapes[1::2] + shapes[6:7]
     for shape in shapes:
         host = rng.integers(0, 40, size=shape).astype(dtype)
         if dtype == "float16":
@@ -1093,13 +1091,10 @@ def test_stepped_inner_dim_of_every_width(ctx, dtype):
     rng = np.random.default_rng(93)
     for shape in ((16, 4), (300, 4000), (5, 70001), (2000, 64)):
         base = rng.integers(0, 50, size=shape).astype(dtype)
-        _check_ops(ctx, base[:, :1], [1])
-        _check_ops(ctx, base[:, :1], [0, 1])
         for step in (2, 3, 4):
-            for view in (base[:, ::step], base[:, 1::step], base[::step, ::step]):
+            for view in (base[:, ::step], base[:, 1::step], base[:, :1], base[::step, ::step]):
                 _check_ops(ctx, view, [1])
-            _check_ops(ctx, base[:, ::step], [0, 1])
-            _check_ops(ctx, base[::step, ::step], [0, 1])
+                _check_ops(ctx, view, [0, 1])
 
 
 def test_stepped_eight_byte_rows_are_planned(ctx):
