@@ -128,7 +128,7 @@ def test_a_tuning_knob_read_again_is_a_new_plan(ctx, knobs):
     assert launches() == 1
     # and the elementwise side: the transposed-tile size is part of the plan's geometry
     a = np.random.default_rng(8).integers(0, 50, size=(700, 900)).astype(np.float32)
-    k = ga.GpuElemwise(ctx, "o = i", [ga.arg("i", "float32", read=True), ga.arg("o", "float32", write=True)])
+    k = ga.GpuElemwise(ctx, "dst = src", [ga.arg("src", "float32", read=True), ga.arg("dst", "float32", write=True)])
     gi = gpuarray.array(a, context=ctx)
     for tile in (64, 128, None, 64):
         knobs(ELEMWISE_TTILE=tile)
