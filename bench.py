@@ -55,14 +55,14 @@ MEASURED_TRAFFIC = {
     "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536638854),
     "C3a_sum_axis1_8192x8192": ("dad31caa5cba69db", 268766015),
     "C4_maxandargmax_65536x1000": ("e07f5c491a26ec87", 263701951),
-    "C5_fp16_sum_axes02": ("1c31fb49c4b5b020", 269706750),
+    "C5_fp16_sum_axes02": ("d21d92d81160c1dc+1c31fb49c4b5b020", 269706750),
     "C5_int32_sum_axis1": ("8274229b3cbbd35d", 538005647),
     "C5_uint8_all_axis2": ("f820fbfcf8c6c517", 134384187),
     "C5_uint8_any_axis2": ("4d7e5c2312df6b47", 134384118),
     "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538649272),
     "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538654594),
     "F4_dot_2x2^27_fused": ("8b73e74aff3e53e7", 1073848190),
-    "F4_dot_2x2^27_two_pass": ("fad720c7c171b6dc", 2146728209),
+    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+fad720c7c171b6dc", 2146728209),
     "elem_2^28": ("712fba8f0b8a6108", 3219542703),
     "sum_2^28": ("fad720c7c171b6dc", 1073797825),
 }

@@ -1,6 +1,6 @@
 """Kernel times of common array shapes, against the bytes they must move.
 
-    python shapes_bench.py [--only elemwise|reductions] [--iters N]
+    python shapes_bench.py [--only elemwise|reductions|floor] [--iters N]
 
 The benchmark of the repository (bench.py) prices one large contiguous
 elementwise kernel and one full sum.  This walks through the shapes that
@@ -174,9 +174,39 @@ def run_reductions(ctx, ga, gpuarray, iters):
         del sets
 
 
+def run_floor(ctx, ga, gpuarray, iters):
+    """What the clock used here reads for a kernel that does nothing (the time
+    of a dispatch by itself), and the same four kernels - full sum, full max,
+    c = a*b + 0.5f, fill - over contiguous floats from 2^18 to 2^28 elements:
+    how much of a kernel's time does not depend on its size."""
+    from libgpuarray_amd import reduction as R
+    nop = ga.GpuKernel('#include "cluda.h"\nKERNEL void nop(GLOBAL_MEM float *a) { }', "nop",
+                       [gpuarray.GpuArray], context=ctx)
+    one = gpuarray.zeros((16,), "float32", context=ctx)
+    for groups in (1, 256, 2048, 65536):
+        us, per = _kernel_us(ctx, lambda i: nop(one, gs=groups, ls=256), iters)
+        _report("floor", "empty kernel, %d groups of 256 lanes" % groups, us, per, 0)
+    f32 = "float32"
+    elem = ga.GpuElemwise(ctx, "c = a*b + 0.5f", [ga.arg("a", f32, read=True), ga.arg("b", f32, read=True),
+                                                   ga.arg("c", f32, write=True)])
+    fill = ga.GpuElemwise(ctx, "c = 1.0f", [ga.arg("c", f32, write=True)])
+    for log2n in range(18, 29):
+        n = 1 << log2n
+        rot = max(1, min(8, (1 << 30) // (16 * n)))
+        xs, ys, zs = ([gpuarray.zeros((n,), f32, context=ctx) for _ in range(rot)] for _ in range(3))
+        for label, call, nbytes in (
+                ("sum of 2^%d floats" % log2n, lambda i: R.sum(xs[i % rot]), 4 * n),
+                ("max of 2^%d floats" % log2n, lambda i: R.max(xs[i % rot]), 4 * n),
+                ("c = a*b + 0.5f, 2^%d floats" % log2n, lambda i: elem(xs[i % rot], ys[i % rot], zs[i % rot]), 12 * n),
+                ("fill, 2^%d floats" % log2n, lambda i: fill(zs[i % rot]), 4 * n)):
+            us, per = _kernel_us(ctx, call, iters)
+            _report("floor", label, us, per, nbytes)
+        del xs, ys, zs
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("--only", choices=["elemwise", "reductions"], default=None)
+    ap.add_argument("--only", choices=["elemwise", "reductions", "floor"], default=None)
     ap.add_argument("--iters", type=int, default=20)
     args = ap.parse_args()
     import libgpuarray_amd as ga
@@ -187,6 +217,8 @@ def main():
         run_elemwise(ctx, ga, gpuarray, args.iters)
     if args.only in (None, "reductions"):
         run_reductions(ctx, ga, gpuarray, args.iters)
+    if args.only == "floor":
+        run_floor(ctx, ga, gpuarray, args.iters)
 
 
 if __name__ == "__main__":
