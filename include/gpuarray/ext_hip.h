@@ -106,7 +106,9 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
  * that one pass of a wavefront covers in place of the general row kernel
  * (64 lanes per output only); bit 28: every count of the call is below 2^31
  * (32-bit divisions); bit 29: also the kernel that walks rows of at most 32
- * bytes in registers, with bits 0..7 of vec as the row length in elements. */
+ * bytes in registers, with bits 0..7 of vec as the row length in elements;
+ * bit 30: also the kernel that reduces the leading dims of a dense array over
+ * short kept rows in one launch. */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

@@ -136,6 +136,11 @@ def main():
         check("reduction tiny rows in registers, op %d type %d, %d elements" % (op, src, te),
               gen_r(op, src, d0, GA_LONG, 64, te, 1 | (1 << 29)))
         n += 1
+    for op, src, d0 in ((0, GA_FLOAT, GA_FLOAT), (0, GA_HALF, GA_FLOAT), (0, GA_INT, GA_LONG), (4, GA_INT, GA_INT),
+                        (1, GA_DOUBLE, GA_DOUBLE), (13, GA_INT, GA_BOOL), (0, GA_HALF, GA_HALF)):
+        check("reduction over leading dims with short kept rows in one launch, op %d type %d" % (op, src),
+              gen_r(op, src, d0, GA_LONG, 64, 1, 8 | (1 << 30)))
+        n += 1
     GA_BYTE, GA_ULONG = 1, 8
     for label, spec in (("sum of unsigned bytes", (0, GA_UBYTE, GA_ULONG, GA_LONG, 256, 16, 8)),
                         ("sum of signed bytes", (0, GA_BYTE, GA_LONG, GA_LONG, 256, 16, 8)),

@@ -1890,6 +1890,8 @@ bool ga_hip_capturing(gpucontext *c) {
   return cap != hipStreamCaptureStatusNone;
 }
 
+bool ga_hip_redux_counters_made(gpucontext *c) { return HC(c)->redux_counters != nullptr; }
+
 gpudata *ga_hip_redux_counters(gpucontext *c) {
   hip_context *ctx = HC(c);
   if (ctx->redux_counters != nullptr) return ctx->redux_counters;

@@ -124,7 +124,8 @@ struct variant {
             fin_cols = {nullptr, nullptr},   // second pass after redux_col
             wrows = {nullptr, nullptr},   // wrows only exists in 64-lane variants
             srows = {nullptr, nullptr},   // the only kernel of a short-rows variant (opts bit 3)
-            trows = {nullptr, nullptr};   // the only kernel of a tiny-rows variant (opts bit 10)
+            trows = {nullptr, nullptr},   // the only kernel of a tiny-rows variant (opts bit 10)
+            pcols = {nullptr, nullptr};   // the only kernel of a short-kept-rows variant (opts bit 11)
 };
 
 struct dimrec {
@@ -282,6 +283,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_TAIL %u\n#define RD_ELSZ0 %u\n", (vs.opts >> 2) & 1u,
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
+  DEF("#define RD_PCOLS %u\n", (vs.opts >> 11) & 1u);
   {
     // redux_trows: a lane's run of whole rows in whole 16-byte chunks
     const unsigned te = vs.TE ? vs.TE : 1;
@@ -530,6 +532,7 @@ int get_variant(GpuReduction *gr, const variant_spec &vs, variant **out, bool ma
   auto want = [&](const char *name, GpuKernel *k) { names[nk] = name; ks[nk++] = k; };
   if (vs.opts & 8u) want("redux_srows", &v.srows);
   if (vs.opts & 1024u) want("redux_trows", &v.trows);
+  if (vs.opts & 2048u) want("redux_pcols", &v.pcols);
   if (vs.opts & 16u) {
     if (vs.opts & 128u) want("redux_wrows", &v.wrows);
     else want("redux_row", &v.row);
@@ -1696,7 +1699,7 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
                          (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
                          (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) |
-                         (((U >> 29) & 1u) ? 1024u : 0u) | 48u | 256u, ES, 1,
+                         (((U >> 29) & 1u) ? 1024u : 0u) | (((U >> 30) & 1u) ? 2048u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};
@@ -1761,8 +1764,143 @@ void GpuReduction_free(GpuReduction *gr) {
     if (kv.second.wrows.k != nullptr) GpuKernel_clear(&kv.second.wrows);
     if (kv.second.srows.k != nullptr) GpuKernel_clear(&kv.second.srows);
     if (kv.second.trows.k != nullptr) GpuKernel_clear(&kv.second.trows);
+    if (kv.second.pcols.k != nullptr) GpuKernel_clear(&kv.second.pcols);
   }
   delete gr;
+}
+
+// Reducing the leading dims of a dense array over short kept rows in one
+// launch (redux_pcols): the array is walked as one run of 16-byte chunks by
+// groups of L lanes, L chunks being a whole number of kept rows, so that a
+// lane meets the same outputs at the same places of every chunk it loads; the
+// groups' partial rows (a few hundred times F values) are combined by the
+// group that finishes last.  Taken when such an L exists (F / gcd(F, elements
+// per chunk) <= 256), the first element sits on a 16-byte boundary, the
+// counters of single-launch reductions can be had and the caller may allocate;
+// everything else is left to fold_rows below.  Measured on MI355X, kernel
+// time, folded rows (two or three launches) against this, sums over axis 0:
+// (2^22, 10) floats 31.0 -> 29.6 us, (2^24, 3) 35.7 -> 36.3, (2^20, 17) 17.6 ->
+// 17.3, (2^20, 63) 47.3 -> 43.9, (2^22, 32) 81.5 -> 77.5 (87 % of peak),
+// (2^24, 6) halves 40.0 -> 36.0, integer maximum of (2^22, 10) 30.6 -> 29.7;
+// two groups per compute unit measured slower (31.7 us for the first shape).
+static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigned reduxLen,
+                      const int *reduxList, bool *done, bool noalloc = false) {
+  *done = false;
+  gpucontext *ctx = gr->ctx;
+  const ga_tuning *tn = ga_hip_tuning(ctx);
+  // (REDUX_FUSED = 0 asks for reductions that do not end in their own launch)
+  if (TUNE(tn, REDUX_PCOLS, 1) == 0 || TUNE(tn, REDUX_FUSED, 1) == 0 || gr->mapped || d0 == nullptr || s0->data == nullptr ||
+      d0->data == nullptr || reduxLen == 0 || reduxLen >= s0->nd || !GpuArray_IS_C_CONTIGUOUS(s0) ||
+      GpuArray_context(d0) != ctx || GpuArray_context(s0) != ctx || s0->typecode != gr->src_tc() ||
+      !GpuArray_ISWRITEABLE(d0))
+    return GA_NO_ERROR;
+  const rd_kind kind = gr->info.kind;
+  const int stc = s0->typecode;
+  const bool regroupable = !gr->info.has_d1 &&
+      (kind == K_SUM || kind == K_PROD || kind == K_AND || kind == K_OR || kind == K_XOR ||
+       kind == K_ALL || kind == K_ANY || ((kind == K_MIN || kind == K_MAX) && is_int_type(stc)));
+  if (!regroupable) return GA_NO_ERROR;
+  std::array<char, 64> seen{};
+  if (reduxLen > seen.size()) return GA_NO_ERROR;
+  for (unsigned i = 0; i < reduxLen; i++) {
+    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= reduxLen || seen[reduxList[i]]) return GA_NO_ERROR;
+    seen[reduxList[i]] = 1;
+  }
+  size_t R = 1, F = 1;
+  for (unsigned j = 0; j < s0->nd; j++) (j < reduxLen ? R : F) *= s0->dimensions[j];
+  const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
+  // (one kept element is a full reduction of a dense array: the planned path's ground)
+  if (F < 2 || R < 2 || R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20)) return GA_NO_ERROR;
+  if (rowb % 16 == 0 && rowb >= 256) return GA_NO_ERROR;   // the column kernel's own ground
+  if (es > 8 || 16 % es != 0 || d0->nd != s0->nd - reduxLen || d0->nd > (unsigned)RD_MAXD) return GA_NO_ERROR;
+  for (unsigned j = 0; j < d0->nd; j++)
+    if (d0->dimensions[j] != s0->dimensions[reduxLen + j]) return GA_NO_ERROR;
+  // the result's type must be one the operation accepts (the planned path reports what is wrong)
+  const int d0_tc = d0->typecode;
+  const bool logical = kind == K_ALL || kind == K_ANY, minmax = kind == K_MIN || kind == K_MAX;
+  if ((minmax && d0_tc != stc) || ((kind == K_AND || kind == K_OR || kind == K_XOR || logical) && !is_int_type(d0_tc)) ||
+      (!is_int_type(d0_tc) && !is_float_type(d0_tc)))
+    return GA_NO_ERROR;
+  const size_t accsz = logical ? 4 : acc_size_for(acc_typecode(gr, d0_tc));
+  if (accsz != 4 && accsz != 8) return GA_NO_ERROR;
+  // A lane keeps one accumulator per element of a chunk.  Up to 32 bytes of
+  // them (four floats or doubles, four 64-bit sums of int32, eight float sums
+  // of halves) this kernel wins; beyond, the elements are narrow and each is
+  // taken out of its word and widened on its own, and the folded rows, whose
+  // kernels take bytes four per instruction, are faster: 2^24 rows of 12 bytes
+  // summed into 64-bit integers 68 us here against 43, of 6 int16 47 against 41.
+  if (16 / es * accsz > 32) return GA_NO_ERROR;
+  // L: the most lanes of 256 whose chunks are a whole number of kept rows
+  const size_t pv = 16 / es;
+  size_t g = F, h = pv;
+  while (h) { const size_t t = g % h; g = h; h = t; }
+  const size_t q = F / g;
+  if (q > 256 || F > 65536) return GA_NO_ERROR;
+  const size_t L = 256 / q * q;
+  uintptr_t base = 0;
+  size_t bufsz = 0, readable = 0;
+  ga_hip_buf_info(s0->data, &base, &bufsz, &readable);
+  const size_t bytes = R * rowb, chunks = (bytes + 15) / 16;
+  if ((base + s0->offset) % 16 != 0 || s0->offset + chunks * 16 > readable) return GA_NO_ERROR;
+  // (the counters are not to be had while the stream records a graph; a call
+  // that may not allocate takes them only if an earlier call has made them)
+  if (noalloc ? !ga_hip_redux_counters_made(ctx) : ga_hip_redux_counters(ctx) == nullptr) {
+    if (noalloc)
+      return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR,
+                        "GpuReduction_call_noalloc: the kernels for arrays of this layout are not "
+                        "built yet, and building them allocates; run GpuReduction_call once on "
+                        "arrays of this layout first");
+    return GA_NO_ERROR;
+  }
+  // groups: one per compute unit, each lane eight loads per batch
+  const size_t ncu = ga_hip_numprocs(ctx), U = 8;
+  size_t G = ncu * TUNE(tn, REDUX_PCOLS_PER_CU, 1);
+  // The group that finishes last combines G partial rows by itself: that pays
+  // while they are a few thousand values.
+  // (256 groups, floats, one launch against folded rows in two: kept rows of 63,
+  // 16 128 partial values, 43.9 against 47.3 us; of 250, 64 000 values, 52.8 against 46.7)
+  if (G * F > TUNE(tn, REDUX_PCOLS_MAX_PARTIALS, 20000)) return GA_NO_ERROR;
+  size_t J = (chunks + G * L - 1) / (G * L);
+  J = (J + U - 1) / U * U;
+  G = (chunks + L * J - 1) / (L * J);
+  if (G < 1) G = 1;
+
+  unsigned opts = TUNE(tn, REDUX_NT, 1) ? 1u : 0u;
+  variant_spec vs = {d0_tc, GA_LONG, 64, 1, (unsigned)U, opts | 2048u, 1, 1, 1, 64, 1, 1};
+  variant *var = nullptr;
+  int err = get_variant(gr, vs, &var, !noalloc);
+  if (err != GA_NO_ERROR) return err;
+  std::vector<int64_t> planbuf(plan_bytes(1) / sizeof(int64_t), 0);
+  rd_plan &p = *reinterpret_cast<rd_plan *>(planbuf.data());
+  p.nf = (int)d0->nd;
+  for (unsigned j = 0; j < d0->nd; j++) {
+    p.fdim[j] = (int64_t)d0->dimensions[j];
+    p.fd0str[j] = (int64_t)d0->strides[j];
+  }
+  if (p.nf == 0) {   // a 0-d result: one output
+    p.nf = 1;
+    p.fdim[0] = 1;
+  }
+  p.nrows = (int64_t)F;
+  p.rtotal = (int64_t)R;
+  p.upb = (int64_t)L;
+  p.units = (int64_t)J;
+  p.nsplit = (int)G;
+  p.fused = 1;
+  launch_rec rec;
+  rec.k1 = &var->pcols;
+  rec.groups = G;
+  rec.fused = true;
+  rec.pi_off = (G * F * accsz + 255) & ~(size_t)255;
+  rec.need = rec.pi_off + 16;
+  const src_view src = {s0, (const int64_t *)s0->strides};
+  if (noalloc && rec.need > ga_static_scratch_bytes)
+    return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
+                      "GpuReduction_call_noalloc: the partial results of this reduction take %zu "
+                      "bytes; the static scratch array holds %zu", rec.need, (size_t)ga_static_scratch_bytes);
+  err = issue_launches(ctx, rec, planbuf.data(), 1, &src, d0, nullptr, nullptr, 0, noalloc, 0);
+  if (err == GA_NO_ERROR) *done = true;
+  return err;
 }
 
 // Reducing the leading dims of a dense array whose trailing (kept) dims are
@@ -1925,7 +2063,9 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
                       "This operator takes several arguments: use GpuReduction_call_map");
   {
     bool done = false;
-    const int err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done);
+    int err = pcols_call(gr, d0, s0, reduxLen, reduxList, &done);
+    if (err != GA_NO_ERROR || done) return err;
+    err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done);
     if (err != GA_NO_ERROR || done) return err;
   }
   const src_view src = {s0, (const int64_t *)s0->strides};
@@ -1945,7 +2085,9 @@ int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d
     // the same route as GpuReduction_call, so that the kernels its warm-up
     // call built are the ones asked for here
     bool done = false;
-    const int err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done, true);
+    int err = pcols_call(gr, d0, s0, reduxLen, reduxList, &done, true);
+    if (err != GA_NO_ERROR || done) return err;
+    err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done, true);
     if (err != GA_NO_ERROR || done) return err;
   }
   const src_view src = {s0, (const int64_t *)s0->strides};

@@ -145,6 +145,8 @@ gpudata *ga_hip_scratch(gpucontext *ctx, size_t bytes);
 // that counts on it leaves it zeroed.  NULL (error set) when it cannot be made.
 constexpr size_t ga_hip_redux_counters_max = 16384;
 gpudata *ga_hip_redux_counters(gpucontext *ctx);
+// Have they been made already?  (For callers that may not allocate.)
+bool ga_hip_redux_counters_made(gpucontext *ctx);
 bool ga_hip_capturing(gpucontext *ctx);
 // The scratch of GpuReduction_call_noalloc: a file-scope device array of
 // ga_static_scratch_bytes bytes in ga_static_scratch.hip, one copy per GPU.

@@ -25,6 +25,8 @@
  *               all; 1: unsigned bytes, 2: signed), 0: off
  *   RD_COL_FAST8  redux_col: any / all over one-byte elements work on whole words
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
+ *   RD_PCOLS    emit redux_pcols (leading dims of a dense array reduced over
+ *               short kept rows, the array walked as one run of chunks)
  *   RD_WANT     which kernels the text holds: bit 0 redux_row, bit 1 redux_col,
  *               bit 2 redux_wrows, bit 3 the second pass (redux_final, and
  *               redux_final_cols beside redux_col)
@@ -1149,7 +1151,9 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
  * of 16-byte chunks - RD_TR rows in RD_TC chunks, both fixed when the kernel
  * is built - into registers and walks its rows there: every element position
  * is a constant, no cross-lane step, no LDS. */
-#define RD_TROW_BYTES (RD_TE * RD_ELSZ0)
+#endif   /* RD_TROWS */
+#if RD_TROWS || RD_PCOLS
+/* elements out of 16-byte chunks held in registers (redux_trows, redux_pcols) */
 typedef ga_uint rd_tchunk_t __attribute__((ext_vector_type(4)));
 
 template <int ES> struct rd_tbits;
@@ -1180,6 +1184,10 @@ static __device__ inline rd_one rd_trow_elem(const rd_tchunk_t *c, const int e) 
   __builtin_memcpy(&o.x0, &bits, sizeof(elem_t));
   return o;
 }
+
+#endif   /* RD_TROWS || RD_PCOLS */
+#if RD_TROWS
+#define RD_TROW_BYTES (RD_TE * RD_ELSZ0)
 
 /* A lane's RD_TR results side by side, for the case that they lie so in
  * memory: up to 16 bytes go out as one store per lane; a longer run is handed
@@ -1368,6 +1376,140 @@ redux_trows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
   }
 }
 #endif   /* RD_TROWS */
+
+#if RD_PCOLS
+/* ---- redux_pcols -----------------------------------------------------------
+ * Reducing the leading dims of a dense array whose kept rows are short - the
+ * sum over a batch of rows of 10 floats: p.nrows outputs (the kept row, F
+ * elements), p.rtotal rows, all F * rtotal elements one after the other in
+ * memory, the first on a 16-byte boundary (one source).  The array is walked
+ * as one run of 16-byte chunks, like a full reduction; which output an
+ * element belongs to is its position modulo F.  L = p.upb lanes of a group
+ * are active, L chosen so that L chunks hold a whole number of kept rows:
+ * the lane's next chunk, L further on, then holds the same outputs at the
+ * same places, and a lane keeps one accumulator per element of a chunk
+ * without ever computing a position.  Group g owns the chunks from g L J on
+ * (J = p.units chunks per lane).  At the end the L * 16 / size accumulators
+ * of a group meet in LDS, F of them come out per group, and the group that
+ * counts in last (p.nsplit groups, one counter) combines the groups'
+ * partials and writes the outputs: one launch.  For operations whose result
+ * does not depend on how the elements are grouped. */
+#define RD_PVN (16 / RD_ELSZ0)
+static __device__ inline rd_acc rd_pacc(const RD_ACC_T v) {
+  rd_acc a = rd_neutral();
+  a.v = v;
+  return a;
+}
+
+/* The L * RD_PVN (or nsplit * F) values at stage[i * F + k] combined per
+ * column k: lane t < S F takes column t mod F and every S-th copy, S = 256 / F
+ * lane subsets, which then meet; with more than 256 columns a lane walks its
+ * columns alone.  `out(k, a)` receives each column once. */
+template <typename FETCH, typename OUT>
+static __device__ inline void rd_pcols_fold(const unsigned F, const unsigned copies, RD_ACC_T *meet,
+                                            FETCH fetch, OUT out) {
+  if (F <= 256u) {
+    const unsigned S = 256u / F, s = LID_0 / F, k = LID_0 - s * F;
+    rd_acc a = rd_neutral();
+    if (s < S) {
+      /* eight fetches go out before the first is combined: one at a time each
+       * would wait for the one before it */
+      unsigned i = s;
+      for (; i + 7 * S < copies; i += 8 * S) {
+        RD_ACC_T t[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = fetch((i + j * S) * F + k);
+#pragma unroll
+        for (int j = 0; j < 8; j++) a = rd_combine(a, rd_pacc(t[j]));
+      }
+      for (; i < copies; i += S) a = rd_combine(a, rd_pacc(fetch(i * F + k)));
+    }
+    meet[LID_0] = a.v;
+    local_barrier();
+    if (LID_0 < F) {
+      for (unsigned q = 1; q < S; q++) a = rd_combine(a, rd_pacc(meet[q * F + LID_0]));
+      out(LID_0, a);
+    }
+  } else {
+    for (unsigned k = LID_0; k < F; k += 256u) {
+      rd_acc a = rd_neutral();
+      for (unsigned i = 0; i < copies; i++) a = rd_combine(a, rd_pacc(fetch(i * F + k)));
+      out(k, a);
+    }
+  }
+}
+
+KERNEL void __launch_bounds__(256)
+redux_pcols(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__restrict__ d1,
+            const ga_size d1_off, RD_ACC_T *__restrict__ part_v, ga_long *__restrict__ part_i, ga_uint *done,
+            const rd_plan p RD_SCALAR_PARAMS) {
+  __shared__ RD_ACC_T stage[256 * RD_PVN];
+  __shared__ RD_ACC_T meet[256];
+  __shared__ ga_uint last_piece;
+  const unsigned F = (unsigned)p.nrows, L = (unsigned)p.upb, G = (unsigned)p.nsplit;
+  const ga_long J = p.units;
+  const ga_long bytes = p.nrows * p.rtotal * RD_ELSZ0;
+  const ga_long full = bytes >> 4;                          /* whole chunks */
+  const int rem = (int)((bytes & 15) / RD_ELSZ0);           /* elements of a last, partial chunk */
+  const char *base[RD_NSRC];
+  RD_SRC_BASES(base);
+  const rd_tchunk_t *src = (const rd_tchunk_t *)base[0];
+
+  rd_acc acc[RD_PVN];
+#pragma unroll
+  for (int v = 0; v < RD_PVN; v++) acc[v] = rd_neutral();
+  if (LID_0 < L) {
+    const ga_long c0 = (ga_long)GID_0 * L * J + LID_0;
+    for (ga_long j = 0; j < J; j += RD_U) {
+      rd_tchunk_t c[RD_U];
+      if (j + RD_U <= J && c0 + (j + RD_U - 1) * L < full) {
+        /* all of the batch inside the array: the loads go out together */
+#pragma unroll
+        for (int u = 0; u < RD_U; u++) c[u] = RD_LOAD(src + c0 + (j + u) * L);
+#pragma unroll
+        for (int u = 0; u < RD_U; u++)
+#pragma unroll
+          for (int v = 0; v < RD_PVN; v++)
+            acc[v] = rd_combine(acc[v], rd_elem(RD_ONE_VAL(rd_trow_elem(&c[u], v)), 0));
+      } else {
+#pragma unroll
+        for (int u = 0; u < RD_U; u++) {
+          const ga_long ci = c0 + (j + u) * L;
+          const bool in = j + u < J && (ci < full || (ci == full && rem > 0));
+          c[u] = (rd_tchunk_t)(0u);
+          if (in) c[u] = RD_LOAD(src + ci);
+#pragma unroll
+          for (int v = 0; v < RD_PVN; v++)
+            if (in && (ci < full || v < rem))
+              acc[v] = rd_combine(acc[v], rd_elem(RD_ONE_VAL(rd_trow_elem(&c[u], v)), 0));
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < RD_PVN; v++) stage[LID_0 * RD_PVN + v] = acc[v].v;   /* idle lanes: neutral */
+  local_barrier();
+  /* a group's chunks start at a multiple of L chunks, a whole number of kept
+   * rows: accumulator v of lane l belongs to output (l RD_PVN + v) mod F */
+  rd_pcols_fold(F, L * RD_PVN / F, meet,
+                [&](const unsigned at) { return stage[at]; },
+                [&](const unsigned k, const rd_acc a) { rd_publish_partial(a, part_v, part_i, (ga_long)GID_0 * F + k); });
+  rd_stores_done();   /* every lane that left partials */
+  local_barrier();
+  if (LID_0 == 0) last_piece = rd_count_in(done, G) ? 1u : 0u;
+  local_barrier();
+  if (!last_piece) return;
+  rd_before_loads();
+  rd_pcols_fold(F, G, meet,
+                [&](const unsigned at) { return rd_fetch_partial(part_v, part_i, (ga_long)at).v; },
+                [&](const unsigned k, const rd_acc a) {
+                  ga_long so[RD_NSRC], d0o, d1o;
+                  rd_row_offsets(p, (ga_long)k, so, &d0o, &d1o);
+                  rd_write(a, d0 + d0_off, d0o, d1 + d1_off, d1o);
+                });
+  if (LID_0 == 0) rd_count_reset(done);
+}
+#endif   /* RD_PCOLS */
 
 /* ---- helpers of redux_col ------------------------------------------------- */
 

@@ -118,9 +118,10 @@ def reduction_cases():
         ("min", "int32", (8192, 8192), (0,), None, None, ""),
         ("sum", f, (64, 1 << 20), (0,), None, None, "few long rows"),
         ("sum", f, (1 << 20, 64), (0,), None, None, ""),
-        ("sum", f, (1 << 22, 10), (0,), None, None, "bias gradient: folded rows"),
+        ("sum", f, (1 << 22, 10), (0,), None, None, "bias gradient: short kept rows, one launch"),
+        ("sum", f, (1 << 22, 32), (0,), None, None, "short kept rows, one launch"),
         ("sum", f, (65536, 1001), (0,), None, None, "folded rows"),
-        ("sum", f, (1 << 24, 3), (0,), None, None, "folded rows"),
+        ("sum", f, (1 << 24, 3), (0,), None, None, "short kept rows, one launch"),
         ("sum", f, (64, 256, 64, 64), (0, 2, 3), None, None, "per-channel statistics, NCHW"),
         ("sum", f, (64, 64, 64, 256), (0, 1, 2), None, None, "per-channel statistics, NHWC"),
         ("sum", f, (64, 256, 64, 64), (2, 3), None, None, "global pooling"),

@@ -383,6 +383,68 @@ def test_float16_on_stepped_views(ctx, axes):
         assert np.array_equal(np.asarray(R.all(g, axis=axes)), v.all(axis=axes))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint8", "float16", "float64", "int16"])
+def test_short_kept_rows_in_one_launch(ctx, dtype):
+    """redux_pcols: kept rows of 1 to 1000 elements (row bytes below 256, or
+    not a multiple of 16), totals that end inside a 16-byte chunk, several
+    leading and several kept dims, a result with its own strides, a half
+    result; sum, product, any / all, integer min / max and the bitwise ones,
+    against NumPy (values small enough for every sum to be exact)."""
+    rng = np.random.default_rng(1234)
+    es = np.dtype(dtype).itemsize
+    kept_lengths = [1, 2, 3, 5, 7, 10, 12, 17, 33, 63, 100, 250, 255, 1000]
+    launches = []
+    for F in kept_lengths:
+        rowb = F * es
+        if rowb % 16 == 0 and rowb >= 256:
+            continue
+        R0 = ((6 << 20) // rowb) | 1            # an odd row count: the total ends inside a chunk for most F
+        for shape, axes in (((R0, F), (0,)), ((3, R0 // 3 + 1, F), (0, 1))):
+            if F == 12:
+                shape, axes = (shape[0],) * 1 + shape[1:-1] + (3, 4), axes        # two kept dims
+            lo, hi = (0, 3) if np.dtype(dtype).kind == "u" else (-2, 3)
+            host = rng.integers(lo, hi, size=shape).astype(dtype)
+            g = gpuarray.array(host, context=ctx)
+            ctx.kernel_timing(True)
+            if np.dtype(dtype).kind == "f":
+                got = np.asarray(R.sum(g, axis=axes, dtype="float32"))
+                n = len(ctx.kernel_times())
+                assert np.array_equal(got, host.sum(axis=axes, dtype=np.float64).astype(np.float32)), (shape, "sum")
+            else:
+                got = np.asarray(R.sum(g, axis=axes, dtype="int64"))
+                n = len(ctx.kernel_times())
+                assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64)), (shape, "sum")
+            ctx.kernel_timing(False)
+            launches.append((F, n))
+            for name, npf in (("all", np.all), ("any", np.any)):
+                got = np.asarray(R._reduce_named(g, name, np.dtype("bool"), axis=axes))
+                assert np.array_equal(got, npf(host, axis=axes)), (shape, name)
+            if np.dtype(dtype).kind in "iu":
+                for name, npf in (("max", np.max), ("min", np.min)):
+                    assert np.array_equal(np.asarray(getattr(R, name)(g, axis=axes)), npf(host, axis=axes)), (shape, name)
+                got = np.asarray(R._reduce_named(g, "xor", np.dtype(dtype), axis=axes))
+                assert np.array_equal(got, np.bitwise_xor.reduce(host, axis=axes if len(axes) == 1 else None)
+                                      if len(axes) == 1 else
+                                      np.bitwise_xor.reduce(np.bitwise_xor.reduce(host, axis=0), axis=0)), (shape, "xor")
+    # kept rows of 2 to 63 elements of a type whose accumulators fit the lane went out as one launch
+    if dtype in ("float32", "float64", "int32", "float16"):
+        assert all(n == 1 for F, n in launches if 2 <= F <= 63), launches
+    # a result with strides of its own, a half result, a product of +-1
+    host = rng.integers(-2, 3, size=(1 << 20, 10)).astype(dtype)
+    g = gpuarray.array(host, context=ctx)
+    wide = gpuarray.zeros((10, 3), "int64" if np.dtype(dtype).kind in "iu" else "float32", context=ctx)
+    ga.GpuReduction(ctx, "sum", dtype)(g, [0], d0=wide[:, 1])
+    assert np.array_equal(np.asarray(wide)[:, 1], host.sum(axis=0, dtype=np.float64).astype(np.asarray(wide).dtype))
+    assert not np.asarray(wide)[:, 0].any() and not np.asarray(wide)[:, 2].any()
+    if dtype == "float16":
+        got = np.asarray(R.sum(g, axis=0))
+        assert got.dtype == np.float16
+        assert np.array_equal(got, host.sum(axis=0, dtype=np.float64).astype(np.float32).astype(np.float16))
+    signs = rng.choice(np.array([1, -1]).astype(dtype) if np.dtype(dtype).kind != "u" else np.array([1, 1], dtype), size=(1 << 20, 6))
+    got = np.asarray(R._reduce_named(gpuarray.array(signs, context=ctx), "prod", np.dtype(dtype), axis=(0,)))
+    assert np.array_equal(got, np.prod(signs.astype(np.float64), axis=0).astype(dtype))
+
+
 def test_integer_invariants(ctx):
     # exact in any order: permuting the data or reducing axis by axis gives
     # the same integers
@@ -1110,15 +1172,18 @@ def test_stepped_eight_byte_rows_are_planned(ctx):
     assert np.asarray(R.sum(g, axis=1)).shape == (64,)
 
 
-@pytest.mark.parametrize("fold", ["1", "0"])
-def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, fold):
+@pytest.mark.parametrize("route", ["one launch", "folded", "neither"])
+def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, route):
     """Reducing the leading dims of a dense array whose kept rows are short or
-    off a 16-byte boundary goes through folded rows (every m rows taken as one,
-    then the m copies of each output combined): every operation that may be
-    regrouped, integer and floating types, one and two leading dims, row
-    counts with and without a usable divisor, a strided destination; against
-    NumPy, and with folding switched off."""
-    knobs(REDUX_FOLD=fold)
+    off a 16-byte boundary: in one launch that walks the array as one run of
+    chunks (redux_pcols) where the row length allows it, else through folded
+    rows (every m rows taken as one, then the m copies of each output
+    combined): every operation that may be regrouped, integer and floating
+    types, one and two leading dims, row counts with and without a usable
+    divisor, a strided destination; against NumPy, by each of the two routes
+    and with both switched off."""
+    fold = "0" if route == "neither" else "1"
+    knobs(REDUX_FOLD=fold, REDUX_PCOLS=1 if route == "one launch" else 0)
     rng = np.random.default_rng(71)
     cases = (((1 << 20, 10), (0,)), ((1 << 21, 3), (0,)), ((16384, 1001), (0,)),
              ((1024, 1024, 4), (0, 1)), ((1048573, 5), (0,)), ((3 * (1 << 18), 6, 2), (0,)),

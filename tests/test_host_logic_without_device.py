@@ -130,7 +130,8 @@ calls = C.c_ulong.in_dll(mock, "mock_allocating_calls")
 ctx = ga.init("hip0")
 for dtype, shape, axes, d1 in (("float32", (1 << 22,), [0], False), ("int32", (6, 1 << 18), [1], False),
                                ("float32", (1 << 14, 256), [0], True), ("float32", (4096, 100), [1], False),
-                               ("float32", (1 << 20, 10), [0], False)):          # folded rows
+                               ("float32", (1 << 20, 10), [0], False),           # short kept rows, one launch
+                               ("float32", (1 << 14, 250), [0], False)):         # folded rows
     op = ga.GpuReduction(ctx, "maxandargmax" if d1 else "sum", dtype)
     src = ga.zeros(shape, dtype, context=ctx)
     oshape = tuple(d for k, d in enumerate(shape) if k not in axes)

@@ -28,10 +28,13 @@ CASES = [
     ("columns, split", "sum", "int32", (1 << 14, 512), (5000, 384), (0,), "int32", False),
     ("columns, split, arg", "maxandargmax", "float32", (1 << 14, 256), (4097, 200), (0,), "float32", True),
     ("not split", "sum", "float32", (8192, 1024), (100, 33), (1,), "float32", False),
-    # leading dims over short kept rows: every m rows taken as one long row, then
+    # leading dims over short kept rows, in one launch (the array walked as one run
+    # of chunks, the groups' partial rows in the static array) ...
+    ("short kept rows", "sum", "float32", (1 << 20, 10), (1 << 19, 6), (0,), "float32", False),
+    ("short kept rows, int", "sum", "int32", (1 << 18, 3, 5), (1 << 18, 3, 3), (0,), "int64", False),
+    # ... and longer ones through folded rows: every m rows taken as one long row, then
     # the m copies of each output combined; all intermediate results in the static array
-    ("folded rows", "sum", "float32", (1 << 20, 10), (1 << 19, 6), (0,), "float32", False),
-    ("folded rows, int", "sum", "int32", (1 << 18, 3, 5), (1 << 18, 3, 3), (0,), "int64", False),
+    ("folded rows", "sum", "float32", (1 << 14, 250), (5000, 250), (0,), "float32", False),
 ]
 
 
