@@ -86,7 +86,11 @@ GPUARRAY_PUBLIC int GpuReduction_call(const GpuReduction *gr, GpuArray *d0,
  * entry point keeps them in a device array that is part of the library
  * itself, GA_REDUCTION_NOALLOC_SCRATCH bytes on every GPU the library runs
  * on, looked up once when the context is made; it calls no allocating
- * routine, and a split reduction always ends in a second launch.
+ * routine, and a split reduction always ends in a second launch (the one
+ * exception: the leading dims of a dense array over short kept rows keep
+ * their single launch, whose counter an earlier GpuReduction_call has made).
+ * Every layout takes the route GpuReduction_call takes for it, so that one
+ * such call is the warm-up this entry point needs.
  *   GA_UNSUPPORTED_ERROR  the kernels for this layout are not built yet
  *                         (building loads a code object, which allocates):
  *                         call GpuReduction_call once on arrays of the same
