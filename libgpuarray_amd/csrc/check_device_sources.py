@@ -64,6 +64,10 @@ def main():
     check("elemwise strided, two doubles per lane", gen_e(b"", b"c = a*b + 0.5", 3, dargs, 0, 10, 2, 0, 0b101 << 16))
     check("elemwise strided vec4 transposed, streaming", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 4, 3, 1, 0b001 | (0b110 << 16)))
+    check("elemwise strided vec4 transposed, 8-byte elements (quads as two pairs)",
+          gen_e(b"", b"c = a*b + 0.5", 3, dargs, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
+    check("elemwise strided vec4, 8-byte result written through a transposed tile",
+          gen_e(b"", b"c = a*b + 0.5", 3, dargs, 0, 3, 2, 0, 0b100 | (0b011 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles, operand constant along x",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 7, 2, 0, 0b001 | (0b100 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles, operands constant along y",

@@ -641,7 +641,8 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 // gather 4 consecutive y from the tile and store them with one access.
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
-                            unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4, unsigned vq = 4) {
+                            unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4, unsigned vq = 4,
+                            bool pairs_ok = true) {
   std::string s;
   // elements a lane moves at a time: 4, or (plain variant only) 2 when the
   // widest type has 8 bytes, so that the widest access stays at 16 bytes
@@ -812,6 +813,22 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   const unsigned yd = nd - 2;
   const unsigned T = tile, Q = tile / 4;
   const std::string TP = std::to_string(T + 1) + "u";
+  // A lane's four elements along an axis (its "quad").  With elements of up
+  // to four bytes they are adjacent, one access of up to 16 bytes.  With
+  // eight-byte elements in the kernel they are two pairs, half a tile apart:
+  // four adjacent doubles per lane are two 16-byte accesses that lie 32 bytes
+  // from the neighbouring lane's, so every access instruction of a wavefront
+  // touches twice the lines it uses; as pairs, the 16 lanes of a line cover
+  // two runs of 256 contiguous bytes.  Measured on MI355X, kernel time, quads /
+  // pairs: out = in.T of 4096 x 4096 doubles 47.3 / 44.6 us (71 -> 75 % of
+  // peak), a.T + b on the same 70.1 / 66.3; kernels of narrower elements are
+  // the same text as before (out = in.T of 8192 x 8192 floats 81.6 us).
+  size_t widest = 1;
+  for (const ge_arg &a : ge->args)
+    if (a.is_array()) widest = std::max(widest, gpuarray_get_elsize(a.typecode));
+  const bool halves = widest == 8 && pairs_ok;
+  const unsigned NH = halves ? 2 : 1, VE = 4 / NH;   // accesses per quad, elements per access
+  auto vec_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * VE); };
   for (size_t j = 0; j < ge->args.size(); j++)
     if (is_t(j))
       appendf(s, "LOCAL_MEM %s %s_t[%u * %u];\n", ctype(ge->args[j].typecode),
@@ -827,6 +844,9 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // measured no faster at 4096 x 4096 and 4 to 10 % slower at 8192 x 8192 and
   // 16384 x 16384: the kernel waits on memory, not on LDS.
   appendf(s, "const %s ga_lo = LID_0 & %uu;\nconst %s ga_hi = LID_0 / %uu;\n", N, Q - 1, N, Q);
+  // position of element i of the lane's quad along the quad's axis
+  if (halves) appendf(s, "#define GA_QP(i) (2u * ga_lo + ((i) & 1u) + ((i) >> 1) * %uu)\n", T / 2);
+  else s += "#define GA_QP(i) (4u * ga_lo + (i))\n";
   appendf(s, "const %s ga_gy = ((%s)dim%u + %uu) / %uu;\n", N, N, yd, T - 1, T);
   // Tiles of one plane are handed out in bands of ga_ltx tile rows, walking
   // down a band's rows first: groups that run together then read runs that
@@ -885,62 +905,86 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     if (ge->args[j].reads()) any_tr = true;
     if (ge->args[j].writes()) any_tw = true;
   }
+  // access h of the quad of array j (h < NH): along y at column `x` (phase 1
+  // and 3), or along x at row `y` (the direct operands and results of phase 2)
+  auto vec_ptr = [&](const ge_arg &a, bool along_y, unsigned h, const char *other) {
+    char q[64];
+    snprintf(q, sizeof(q), "%s + GA_QP(%uu)", along_y ? "ga_y0" : "ga_x0", h * VE);
+    std::string pe;
+    appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", vec_t(a), a.name.c_str(),
+            (along_y ? off_yx(a, q, other) : off_yx(a, other, q)).c_str());
+    return pe;
+  };
+  // is access h of the quad, whose other coordinate is in range, in range itself?
+  auto in_range = [&](bool along_y, unsigned h) {
+    std::string c;
+    appendf(c, "%s + GA_QP(%uu) < (%s)dim%u", along_y ? "ga_y0" : "ga_x0", h * VE, N, along_y ? yd : xd);
+    return c;
+  };
   // loads of the operands that phase 2 reads straight from memory
   auto emit_direct_loads = [&]() {
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (a.is_array() && !is_t(j))
-        appendf(s, "union { %s c; %s e[4]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), a.name.c_str());
+        appendf(s, "union { %s p[%u]; %s e[4]; } %s_u[4];\n", vec_t(a), NH, ctype(a.typecode), a.name.c_str());
     }
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    appendf(s, "const %s ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u) {\n", N, yd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || is_t(j) || !a.reads()) continue;
       if (is_y(j)) s += "if (ga_k == 0) {\n";
       if (is_u(j)) {
-        std::string pe;
-        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
-                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
-        s += quad_load(j, a.name + "_u[ga_k].c", pe);
+        for (unsigned h = 0; h < NH; h++) {
+          appendf(s, "if (%s) ", in_range(false, h).c_str());
+          char dst[64];
+          snprintf(dst, sizeof(dst), "%s_u[ga_k].p[%u]", a.name.c_str(), h);
+          s += quad_load(j, dst, vec_ptr(a, false, h, "ga_y0 + ga_ly"));
+        }
       } else if (is_z(j)) {
-        appendf(s, "%s_u[ga_k].e[0] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(),
-                ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "0").c_str());
+        appendf(s, "if (%s) {\n%s_u[ga_k].e[0] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", in_range(false, 0).c_str(),
+                a.name.c_str(), ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "0").c_str());
         for (int i = 1; i < 4; i++)
           appendf(s, "%s_u[ga_k].e[%d] = %s_u[ga_k].e[0];\n", a.name.c_str(), i, a.name.c_str());
+        s += "}\n";
       } else {
         for (int i = 0; i < 4; i++) {
           char xi[48];
-          snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
-          appendf(s, "%s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", a.name.c_str(), i,
-                  ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
+          snprintf(xi, sizeof(xi), "ga_x0 + GA_QP(%du)", i);
+          appendf(s, "if (%s < (%s)dim%u) %s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", xi, N, xd,
+                  a.name.c_str(), i, ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
         }
       }
       // a lane's row 0 is in range whenever one of its later rows is
-      if (is_y(j)) appendf(s, "} else {\n%s_u[ga_k].c = %s_u[0].c;\n}\n", a.name.c_str(), a.name.c_str());
+      if (is_y(j)) {
+        s += "} else {\n";
+        for (unsigned h = 0; h < NH; h++)
+          appendf(s, "%s_u[ga_k].p[%u] = %s_u[0].p[%u];\n", a.name.c_str(), h, a.name.c_str(), h);
+        s += "}\n";
+      }
     }
     s += "}\n}\n";
   };
-  // phase 1: transposed reads.  lane: y quad ga_lo (y = 4*ga_lo..+3), x column ga_hi + 16k
+  // phase 1: transposed reads.  lane: y quad of ga_lo, x column ga_hi + Q k
   if (any_tr) {
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (is_t(j) && a.reads())
-        appendf(s, "union { %s c; %s e[4]; } %s_in[4];\n", quad_t(a), ctype(a.typecode),
+        appendf(s, "union { %s p[%u]; %s e[4]; } %s_in[4];\n", vec_t(a), NH, ctype(a.typecode),
                 a.name.c_str());
     }
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    appendf(s, "const %s ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+    appendf(s, "if (ga_x0 + ga_lx < (%s)dim%u) {\n", N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
-      {
-        std::string pe;
-        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
-                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
-        s += quad_load(j, a.name + "_in[ga_k].c", pe);
+      for (unsigned h = 0; h < NH; h++) {
+        appendf(s, "if (%s) ", in_range(true, h).c_str());
+        char dst[64];
+        snprintf(dst, sizeof(dst), "%s_in[ga_k].p[%u]", a.name.c_str(), h);
+        s += quad_load(j, dst, vec_ptr(a, true, h, "ga_x0 + ga_lx"));
       }
     }
     s += "}\n}\n";
@@ -948,27 +992,27 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     // loads and before the barrier, so that their latency is not paid after it
     emit_direct_loads();
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    appendf(s, "const %s ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+    appendf(s, "if (ga_x0 + ga_lx < (%s)dim%u) {\n", N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
       appendf(s, "#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
-                 "%s_t[(ga_ly + ga_i) * %uu + ga_lx] = %s_in[ga_k].e[ga_i];\n",
-              a.name.c_str(), T + 1, a.name.c_str());
+                 "if (ga_y0 + GA_QP(ga_i) < (%s)dim%u) %s_t[GA_QP(ga_i) * %uu + ga_lx] = %s_in[ga_k].e[ga_i];\n",
+              N, yd, a.name.c_str(), T + 1, a.name.c_str());
     }
     s += "}\n}\nlocal_barrier();\n";
   }
-  // phase 2: the expression.  lane: x quad ga_lo (x = 4*ga_lo..+3), y row ga_hi + 16k
+  // phase 2: the expression.  lane: x quad of ga_lo, y row ga_hi + Q k
   if (!any_tr) emit_direct_loads();
   s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-  appendf(s, "const %s ga_lx = 4u * ga_lo, ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
-  s += "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) {\n";
+  appendf(s, "const %s ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+  appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u) {\n", N, yd);
+  appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) if (ga_x0 + GA_QP(ga_v) < (%s)dim%u) {\n", N, xd);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * " + TP + " + ga_lx + ga_v]");
+    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * " + TP + " + GA_QP(ga_v)]");
     else emit_load(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += ge->expr;
@@ -976,7 +1020,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * " + TP + " + ga_lx + ga_v]");
+    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * " + TP + " + GA_QP(ga_v)]");
     else emit_store(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += "}\n";
@@ -984,16 +1028,18 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     const ge_arg &a = ge->args[j];
     if (!a.is_array() || is_t(j) || !a.writes()) continue;
     if (is_u(j)) {
-      std::string pe;
-      appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
-              off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
-      s += quad_store(j, pe, a.name + "_u[ga_k].c");
+      for (unsigned h = 0; h < NH; h++) {
+        appendf(s, "if (%s) ", in_range(false, h).c_str());
+        char val[64];
+        snprintf(val, sizeof(val), "%s_u[ga_k].p[%u]", a.name.c_str(), h);
+        s += quad_store(j, vec_ptr(a, false, h, "ga_y0 + ga_ly"), val);
+      }
     } else {
       for (int i = 0; i < 4; i++) {
         char xi[48];
-        snprintf(xi, sizeof(xi), "ga_x0 + ga_lx + %du", i);
-        appendf(s, "*(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].e[%d];\n", ctype(a.typecode),
-                a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str(), a.name.c_str(), i);
+        snprintf(xi, sizeof(xi), "ga_x0 + GA_QP(%du)", i);
+        appendf(s, "if (%s < (%s)dim%u) *(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].e[%d];\n", xi, N, xd,
+                ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str(), a.name.c_str(), i);
       }
     }
   }
@@ -1001,25 +1047,25 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // phase 3: transposed writes, mirror of phase 1
   if (any_tw) {
     s += "local_barrier();\n#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
-    appendf(s, "const %s ga_ly = 4u * ga_lo, ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u && ga_x0 + ga_lx < (%s)dim%u) {\n", N, yd, N, xd);
+    appendf(s, "const %s ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
+    appendf(s, "if (ga_x0 + ga_lx < (%s)dim%u) {\n", N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.writes()) continue;
-      appendf(s, "{ union { %s c; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
-                 "ga_o.e[ga_i] = %s_t[(ga_ly + ga_i) * %uu + ga_lx];\n",
-              quad_t(a), ctype(a.typecode), a.name.c_str(), T + 1);
-      {
-        std::string pe;
-        appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", quad_t(a), a.name.c_str(),
-                off_yx(a, "ga_y0 + ga_ly", "ga_x0 + ga_lx").c_str());
-        s += quad_store(j, pe, "ga_o.c");
-        s += "}\n";
+      appendf(s, "{ union { %s p[%u]; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
+                 "ga_o.e[ga_i] = %s_t[GA_QP(ga_i) * %uu + ga_lx];\n",
+              vec_t(a), NH, ctype(a.typecode), a.name.c_str(), T + 1);
+      for (unsigned h = 0; h < NH; h++) {
+        appendf(s, "if (%s) ", in_range(true, h).c_str());
+        char val[32];
+        snprintf(val, sizeof(val), "ga_o.p[%u]", h);
+        s += quad_store(j, vec_ptr(a, true, h, "ga_x0 + ga_lx"), val);
       }
+      s += "}\n";
     }
     s += "}\n}\n";
   }
-  s += "}\n";
+  s += "#undef GA_QP\n}\n";
   return s;
 }
 
@@ -1646,15 +1692,17 @@ class strided_call {
   }
 
   int get_kernel() {
+    // (0: a lane's four 8-byte elements along a transposed tile's axes stay adjacent)
+    const bool tpairs = TUNE(tn, ELEMWISE_TPAIRS, 1) != 0;
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq);
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u:%d", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq, tpairs ? 1 : 0);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq, tpairs)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
