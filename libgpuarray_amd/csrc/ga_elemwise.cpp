@@ -821,8 +821,8 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // touches twice the lines it uses; as pairs, the 16 lanes of a line cover
   // two runs of 256 contiguous bytes.  Measured on MI355X, kernel time, quads /
   // pairs: out = in.T of 4096 x 4096 doubles 47.3 / 44.6 us (71 -> 75 % of
-  // peak), a.T + b on the same 70.1 / 66.3; kernels of narrower elements are
-  // the same text as before (out = in.T of 8192 x 8192 floats 81.6 us).
+  // peak), a.T + b on the same 70.1 / 66.3; kernels of narrower elements
+  // keep their adjacent quads (out = in.T of 8192 x 8192 floats 81.6 us either way).
   size_t widest = 1;
   for (const ge_arg &a : ge->args)
     if (a.is_array()) widest = std::max(widest, gpuarray_get_elsize(a.typecode));
