@@ -50,21 +50,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_configs.md (earlier rocprofv3 --pmc runs, matched by kernel text hash)"
 MEASURED_TRAFFIC = {
     # name: (kernel text hashes of one call joined by "+", HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201255162),
-    "C2_transposed_broadcast_4096": ("fb8ac38966f6e0e0", 134354659),
-    "X_transpose_8192x8192": ("6a36dae9d3bfd9c4", 536638854),
-    "C3a_sum_axis1_8192x8192": ("dad31caa5cba69db", 268766015),
-    "C4_maxandargmax_65536x1000": ("e07f5c491a26ec87", 263701951),
-    "C5_fp16_sum_axes02": ("d21d92d81160c1dc+1c31fb49c4b5b020", 269706750),
-    "C5_int32_sum_axis1": ("8274229b3cbbd35d", 538005647),
-    "C5_uint8_all_axis2": ("f820fbfcf8c6c517", 134384187),
-    "C5_uint8_any_axis2": ("4d7e5c2312df6b47", 134384118),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538649272),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538654594),
-    "F4_dot_2x2^27_fused": ("8b73e74aff3e53e7", 1073848190),
-    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+fad720c7c171b6dc", 2146728209),
-    "elem_2^28": ("712fba8f0b8a6108", 3219542703),
-    "sum_2^28": ("fad720c7c171b6dc", 1073797825),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201253635),
+    "C2_transposed_broadcast_4096": ("d188ff564c901e86", 134376140),
+    "X_transpose_8192x8192": ("a8d106ba259ef190", 536629163),
+    "C3a_sum_axis1_8192x8192": ("7b1e5b3d393b65cf", 268766354),
+    "C4_maxandargmax_65536x1000": ("2b61e61df66fc82d", 263731413),
+    "C5_fp16_sum_axes02": ("4296e62da8ed8910+8be870fa9892586c", 269706664),
+    "C5_int32_sum_axis1": ("0d1aff898d530c09", 538005643),
+    "C5_uint8_all_axis2": ("2195f3f51c85c279", 134384275),
+    "C5_uint8_any_axis2": ("867a1aaf40f33d29", 134384235),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538658597),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538656615),
+    "F4_dot_2x2^27_fused": ("f13108789ad1ada9", 1073848072),
+    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+b3b28b94a7047bb8", 2146736177),
+    "elem_2^28": ("712fba8f0b8a6108", 3219556758),
+    "sum_2^28": ("b3b28b94a7047bb8", 1073797880),
 }
 
 
