@@ -1158,11 +1158,21 @@ class reduction_call {
         // lanes, 67 with 8).
         // (vector loads only: rows of 3 floats, element loads, 60 us with one
         // lane per row and 74 with four).
+        // Below 8 lanes a row of four-byte or wider elements does better
+        // with one load per lane again (maximum over rows of 32 floats: 50.3 us
+        // with 4 lanes x 2 loads, 44.3 with 8 x 1; of 24: 53.1 / 50.9).
         if (V > 1) {
-          const int64_t per_lane = (int64_t)V * (minmax ? 2 : 1);
-          const int64_t need1 = (rin_sz + per_lane - 1) / per_lane;
-          unsigned l1 = 1;
-          while (l1 < 64 && (int64_t)l1 < need1) l1 *= 2;
+          const auto lanes_for = [&](int64_t per_lane) {
+            const int64_t n = (rin_sz + per_lane - 1) / per_lane;
+            unsigned l = 1;
+            while (l < 64 && (int64_t)l < n) l *= 2;
+            return l;
+          };
+          unsigned l1 = lanes_for((int64_t)V * (minmax ? 2 : 1));
+          if (minmax && elsz[0] >= 4 && l1 < 8) {
+            const unsigned single = lanes_for((int64_t)V);
+            l1 = single < 8 ? single : 8;
+          }
           if (l1 <= 32) L = l1;
         }
         const unsigned long force = TUNE(tn, REDUX_L, 0);
@@ -1196,10 +1206,20 @@ class reduction_call {
     // whose pitch is no multiple of 16 bytes cost redux_wrows a shifted,
     // masked load pattern per row and stay here longer: 33 doubles (264
     // bytes) sum / max 118 / 145 us there, 91 / 91 us staged; 40 doubles (320
-    // bytes, aligned) 89 / 100 against 95 / 121 us.
+    // bytes, aligned) 89 / 100 against 95 / 121 us.  Rows of whole 16-byte
+    // pieces leave at 128 bytes (96 for min/max): 2^26 floats in rows of 24 /
+    // 32 / 48 / 64, staged against redux_wrows: sum 44.0 / 43.3 / 42.9 / 43.0
+    // against 44.4 / 42.7 / 41.0 / 40.5 us, maximum 44.7 / 48.9 / 57.8 / 63.9
+    // against 50.9 / 44.3 / 44.0 / 41.7; maximum of 2^26 halves in rows of 48 /
+    // 64: 30.6 / 35.4 against 26.6 / 25.8.  Bytes that are summed or tested
+    // (four to an operation in redux_wrows, one by one in a staged walk) leave
+    // at 32: 2^28 bytes in rows of 48 / 64 / 96 / 128, sum 60.3 / 58.1 / 54.7 /
+    // 68.0 against 50.9 / 48.8 / 48.2 / 47.5 us, any 53.1 / 48.6 / 49.9 / 70.4
+    // against 41.6 / 41.2 / 40.0 / 40.6; their maximum stays to 96 (47.8 / 46.5 /
+    // 43.5 against 76.0 / 65.5 / 74.7).
     if (K == 1 && p.nr == 1 && p.nf == 1 && rtotal > 0 && rsstr[0] == elsz[0] &&
         fsstr[0] == rin * elsz[0] && rin >= 2 &&
-        rin * elsz[0] <= (int64_t)TUNE(tn, REDUX_SROWS_MAX_BYTES, (rin * elsz[0]) % 16 != 0 ? 384 : (minmax ? 160 : 256)) &&
+        rin * elsz[0] <= (int64_t)TUNE(tn, REDUX_SROWS_MAX_BYTES, (rin * elsz[0]) % 16 != 0 ? 384 : (minmax ? 96 : (elsz[0] == 1 ? 32 : 128))) &&
         rin * elsz[0] > (int64_t)TUNE(tn, REDUX_SROWS_MIN_BYTES, 16) &&
         nrows >= (int64_t)TUNE(tn, REDUX_SROWS_MIN_ROWS, 512) * ncu &&
         GpuArray_ISALIGNED(srcs[0].a) && TUNE(tn, REDUX_SROWS, 1)) {

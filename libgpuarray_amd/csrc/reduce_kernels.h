@@ -201,6 +201,19 @@ static __device__ inline rd_acc rd_elem(const T x, ga_long idx) {
   return a;
 }
 
+/* An element's value for a strict compare against a running best that is not
+ * a NaN (the first element of the scan went through rd_elem, or the scan
+ * started from the neutral value): a NaN loses every such compare by itself,
+ * so it needs no mapping. */
+template <typename T>
+static __device__ inline RD_ACC_T rd_later(const T x) {
+#if (RD_KIND == RD_K_MAX || RD_KIND == RD_K_MIN) && RD_FLT
+  return (RD_ACC_T)x;
+#else
+  return rd_elem(x, 0).v;
+#endif
+}
+
 /* ---- cross-lane network --------------------------------------------------
  * Data-parallel-primitive moves on 32-bit words; an accumulator is moved
  * word by word.  Steps: swap with the neighbour (quad_perm 1,0,3,2), with the
@@ -620,7 +633,7 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
     for (int v = 0; v < RD_VEC; v++) {
       if (j == 0 && v < RD_NCH) continue;
       const int c = v % RD_NCH;
-      const RD_ACC_T val = rd_elem(RD_UNIT_VAL(x, j, v), 0).v;
+      const RD_ACC_T val = rd_later(RD_UNIT_VAL(x, j, v));
 #if RD_KIND == RD_K_MAX
       const bool better = in && val > cv[c];
 #else
@@ -1100,7 +1113,7 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
 #pragma unroll 4
       for (ga_int i = 1; i < n; i++) {
         o.x0 = e[i];
-        const RD_ACC_T val = rd_elem(RD_ONE_VAL(o), 0).v;
+        const RD_ACC_T val = rd_later(RD_ONE_VAL(o));
         const bool better = RD_SR_BETTER(val, bv);
         bv = better ? val : bv;
         bp = better ? i : bp;
@@ -1113,7 +1126,7 @@ redux_srows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
       for (ga_int i = 0; i < n; i++) {
         rd_one o;
         o.x0 = e[pos];
-        const RD_ACC_T val = rd_elem(RD_ONE_VAL(o), 0).v;
+        const RD_ACC_T val = rd_later(RD_ONE_VAL(o));
         const bool better = RD_SR_BETTER(val, bv) || (val == bv && pos < bp);
         bv = better ? val : bv;
         bp = better ? pos : bp;
@@ -1287,7 +1300,7 @@ redux_trows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
     ga_int bp = 0;
 #pragma unroll
     for (int i = 1; i < RD_TE; i++) {
-      const RD_ACC_T val = rd_elem(RD_ONE_VAL(rd_trow_elem(c, r * RD_TE + i)), 0).v;
+      const RD_ACC_T val = rd_later(RD_ONE_VAL(rd_trow_elem(c, r * RD_TE + i)));
 #if RD_KIND == RD_K_MAX
       const bool better = val > bv;
 #else
@@ -1649,7 +1662,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       for (int q = 0; q < RD_U; q++) {
 #pragma unroll
         for (int c = 0; c < RD_CV; c++) {
-          const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x[q], c), 0).v;
+          const RD_ACC_T val = rd_later(RD_CVEC_VAL(x[q], c));
           const bool better = RD_COL_BETTER(val, bv[c]);
           bv[c] = better ? val : bv[c];
           bj[c] = better ? (ga_int)(j0 + RD_CY * q) : bj[c];
@@ -1666,7 +1679,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
         if (j0 + RD_CY * q < r1) {
 #pragma unroll
           for (int c = 0; c < RD_CV; c++) {
-            const RD_ACC_T val = rd_elem(RD_CVEC_VAL(x[q], c), 0).v;
+            const RD_ACC_T val = rd_later(RD_CVEC_VAL(x[q], c));
             const bool better = RD_COL_BETTER(val, bv[c]);
             bv[c] = better ? val : bv[c];
             bj[c] = better ? (ga_int)(j0 + RD_CY * q) : bj[c];

@@ -796,6 +796,47 @@ def test_nan_in_first_position_of_short_rows(ctx, dtype, staged, knobs):
                         assert val[r] == nanfn(view[r]) and idx[r] == argfn(view[r]), (name, n, r)
 
 
+def _strict_scan(row, better):
+    """The reference's scan (src/gpuarray_reduction.c:545-607): the first
+    element, then every later one that compares strictly better."""
+    bv, bi = row[0], 0
+    for i in range(1, len(row)):
+        if better(row[i], bv):
+            bv, bi = row[i], i
+    return bv, bi
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "float16"])
+@pytest.mark.parametrize("staged", [0, 1])
+def test_nans_among_values_equal_to_the_neutral_element(ctx, dtype, staged, knobs):
+    """Rows of NaN, -inf and +inf only (few finite values): a NaN loses every
+    compare, a value equal to the scan's starting value never replaces it, so
+    the answer is the row's first element unless a later one beats it, and
+    the first of the equals among those.  Over rows (every short-row kernel)
+    and over columns."""
+    knobs(REDUX_SROWS=staged, REDUX_SROWS_MIN_ROWS=1, REDUX_TROWS_MIN_ROWS=1)
+    rng = np.random.default_rng(66)
+    pool = np.array([np.nan, np.nan, -np.inf, -np.inf, np.inf, 1.0], dtype)
+    for n in (2, 3, 4, 6, 8, 15, 16, 24, 32, 33, 64, 100, 250, 1001):
+        rows = 97
+        for lo_only in (True, False):
+            host = pool[rng.integers(0, 4 if lo_only else 6, size=(rows, n))]
+            host[:8, 0] = np.nan
+            host[8:16, 0] = -np.inf
+            for axis, view in ((1, host), (0, np.ascontiguousarray(host.T))):
+                g, _ = to_gpu_view(view, ctx)
+                seq = host
+                for name, better in (("maxandargmax", lambda a, b: a > b), ("minandargmin", lambda a, b: a < b)):
+                    data = seq if name == "maxandargmax" else -seq
+                    gd = g if name == "maxandargmax" else to_gpu_view(-view, ctx)[0]
+                    val, idx = getattr(R, name)(gd, axis=axis)
+                    val, idx = np.asarray(val), np.asarray(idx)
+                    for r in range(rows):
+                        wv, wi = _strict_scan(data[r], better)
+                        assert idx[r] == wi and (val[r] == wv or (np.isnan(wv) and np.isnan(val[r]))), \
+                            (name, n, axis, r, lo_only, data[r][:8])
+
+
 @pytest.mark.parametrize("dtype", ["uint8", "int8", "bool"])
 def test_one_byte_elements_four_per_operation(ctx, dtype):
     """sum / any / all over one-byte elements (combined a 32-bit word at a
