@@ -1125,6 +1125,32 @@ class reduction_call {
       if (nsplit > 65536) nsplit = 65536;
       if (nsplit < 1) nsplit = 1;
     }
+    // Groups that all fit on the chip at once start together, and the compute
+    // units that hold one more than the others finish last, alone: 300 rows
+    // leave 212 units with one group and 44 with two.  More pieces even that
+    // out.  Measured on MI355X, sum over axis 1 of (300, 223696) floats: 51.0
+    // us whole rows, 45.2 in pieces (two launches); (130, 500000) 50.6 -> 43.5,
+    // (520, 129000) 50.8 -> 45.8, int32 (290, 230000) 50.8 -> 48.0.  Only for a
+    // large excess: the pieces need a finish of their own, often a second
+    // launch ((640, 104857), a fifth too many on some units, 46.5 whole and
+    // 47.3 in pieces; (1000, 65536), 3.9 groups per unit, 40.4 whole).
+    if (TUNE(tn, REDUX_BALANCE, 1) && p.units >= 8 && rowgroups > 0) {
+      const auto excess = [&](int64_t ns) {
+        const int64_t g = rowgroups * ns;
+        return (double)((g + ncu - 1) / ncu * ncu) / (double)g;
+      };
+      const int64_t resident = ncu * 8;
+      int64_t cap = p.units / (int64_t)TUNE(tn, REDUX_MIN_UNITS, 2);
+      if (cap > 65536) cap = 65536;
+      if (rowgroups * nsplit < resident && excess(nsplit) > 1.25) {
+        int64_t best = nsplit;
+        for (int64_t ns = nsplit + 1; ns <= cap && rowgroups * ns <= 2 * resident; ns++) {
+          if (excess(ns) < excess(best) - 0.02) best = ns;
+          if (excess(best) <= 1.03) break;
+        }
+        nsplit = best;
+      }
+    }
     p.upb = p.units > 0 ? (p.units + nsplit - 1) / nsplit : 0;
     if (p.upb > 0) nsplit = (p.units + p.upb - 1) / p.upb;
     p.nsplit = (int)nsplit;

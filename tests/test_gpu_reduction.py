@@ -1070,6 +1070,34 @@ def test_split_reductions_finish_in_one_launch(ctx, knobs):
     assert np.asarray(v) == np.nanmax(x) and int(np.asarray(i)) == int(np.nanargmax(x))
 
 
+@pytest.mark.parametrize("rows,cols", [(300, 70001), (130, 150000), (520, 66000), (41, 300000)])
+def test_rows_cut_to_even_out_the_compute_units(ctx, knobs, rows, cols):
+    """A few hundred long rows, one group each, would leave some compute units
+    with one group more than the others: such rows are cut into pieces
+    (REDUX_BALANCE).  Whole and cut rows must agree bit for bit on data whose
+    sums are exact, and with NumPy; the cut is there when the plan allows it
+    (more than one launch, or a finish inside the first)."""
+    rng = np.random.default_rng(rows)
+    host = rng.integers(-30, 31, size=(rows, cols)).astype(np.float32)
+    host[rng.integers(0, rows, 40), rng.integers(1, cols, 40)] = np.nan
+    g = gpuarray.array(host, context=ctx)
+    clean = np.nan_to_num(host)
+    gi = gpuarray.array(clean.astype(np.int32), context=ctx)
+    gc = gpuarray.array(clean, context=ctx)
+    got = {}
+    for balance in (0, 1):
+        knobs(REDUX_BALANCE=balance)
+        v, i = R.maxandargmax(g, axis=1)
+        got[balance] = (np.asarray(R.sum(gc, axis=1)), np.asarray(R.sum(gi, axis=1, dtype="int64")),
+                        np.asarray(v), np.asarray(i), np.asarray(R.min(gc, axis=1)))
+    for a, b in zip(got[0], got[1]):
+        assert np.array_equal(a, b)
+    assert np.array_equal(got[1][0], clean.sum(axis=1, dtype=np.float64).astype(np.float32))
+    assert np.array_equal(got[1][1], clean.astype(np.int64).sum(axis=1))
+    assert np.array_equal(got[1][2], np.nanmax(host, axis=1)) and np.array_equal(got[1][3], np.nanargmax(host, axis=1))
+    assert np.array_equal(got[1][4], clean.min(axis=1))
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_single_launch_finish_equals_two_launches_bit_for_bit(ctx, knobs, seed):
     """Every family of split reduction that can end in its own launch (row and
