@@ -1,6 +1,6 @@
 """Kernel times of common array shapes, against the bytes they must move.
 
-    python shapes_bench.py [--only elemwise|reductions|floor] [--iters N]
+    python shapes_bench.py [--only elemwise|reductions|floor] [--iters N] [--list] [--case K]
 
 The benchmark of the repository (bench.py) prices one large contiguous
 elementwise kernel and one full sum.  This walks through the shapes that
@@ -89,6 +89,8 @@ def elemwise_cases():
         ("transpose (1, 0, 2) of (1024, 64, 1024)", "o = a", [("a", f, (1024, 64, 1024), T(1, 0, 2))], (64, 1024, 1024), f),
         ("transpose (2, 1, 0) of (256, 512, 512)", "o = a", [("a", f, (256, 512, 512), T(2, 1, 0))], (512, 512, 256), f),
         ("NCHW -> NHWC, (64, 256, 64, 64)", "o = a", [("a", f, (64, 256, 64, 64), T(0, 2, 3, 1))], (64, 64, 64, 256), f),
+        ("copy, 2^28 floats (1 GiB read, 1 GiB written: the yardstick of the traffic counters)", "o = a",
+         [("a", f, (1 << 28,), None)], (1 << 28,), f),
     ]
 
 
@@ -104,6 +106,7 @@ def reduction_cases():
         ("sum", f, (65536, 1001), (1,), None, None, "rows off a 16-byte boundary"),
         ("max", f, (65536, 1001), (1,), None, None, ""),
         ("sum", f, (1335, 50257), (1,), None, None, ""),
+        ("sum", f, (300, 223696), (1,), None, None, "300 long rows, cut to even out the compute units"),
         ("sum", f, (1 << 20, 64), (1,), None, None, "short rows staged in LDS"),
         ("max", f, (1 << 21, 32), (1,), None, None, ""),
         ("sum", f, (1 << 22, 10), (1,), None, None, "tiny rows"),
@@ -133,8 +136,10 @@ def reduction_cases():
     ]
 
 
-def run_elemwise(ctx, ga, gpuarray, iters):
-    for label, expr, specs, oshape, odt in elemwise_cases():
+def run_elemwise(ctx, ga, gpuarray, iters, case=None):
+    for number, (label, expr, specs, oshape, odt) in enumerate(elemwise_cases()):
+        if case is not None and number != case:
+            continue
         args = [ga.arg(n, dt, read=True) for n, dt, _, _ in specs] + [ga.arg("o", odt, write=True)]
         k = ga.GpuElemwise(ctx, expr, args, convert_f16=True)
         sets = []
@@ -152,8 +157,10 @@ def run_elemwise(ctx, ga, gpuarray, iters):
         del sets
 
 
-def run_reductions(ctx, ga, gpuarray, iters):
-    for op, dt, shape, axes, odt, view, note in reduction_cases():
+def run_reductions(ctx, ga, gpuarray, iters, case=None):
+    for number, (op, dt, shape, axes, odt, view, note) in enumerate(reduction_cases()):
+        if case is not None and number != case:
+            continue
         red = ga.GpuReduction(ctx, op, dt)
         sets = []
         for _ in range(ROT):
@@ -209,15 +216,26 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--only", choices=["elemwise", "reductions", "floor"], default=None)
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--list", action="store_true", help="number and name the cases, run nothing")
+    ap.add_argument("--case", type=int, default=None,
+                    help="with --only elemwise / reductions: run the case of this number alone")
     args = ap.parse_args()
+    if args.list:
+        for number, c in enumerate(elemwise_cases()):
+            print("elemwise %d: %s" % (number, c[0]))
+        for number, (op, dt, shape, axes, odt, view, note) in enumerate(reduction_cases()):
+            print("reductions %d: %s %s %s over %s%s" % (number, op, dt, shape, axes, " (%s)" % note if note else ""))
+        return
+    if args.case is not None and args.only not in ("elemwise", "reductions"):
+        ap.error("--case needs --only elemwise or --only reductions")
     import libgpuarray_amd as ga
     from libgpuarray_amd import gpuarray
 
     ctx = ga.init("hip0")
     if args.only in (None, "elemwise"):
-        run_elemwise(ctx, ga, gpuarray, args.iters)
+        run_elemwise(ctx, ga, gpuarray, args.iters, args.case)
     if args.only in (None, "reductions"):
-        run_reductions(ctx, ga, gpuarray, args.iters)
+        run_reductions(ctx, ga, gpuarray, args.iters, args.case)
     if args.only == "floor":
         run_floor(ctx, ga, gpuarray, args.iters)
 
