@@ -642,7 +642,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
                             unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4, unsigned vq = 4,
-                            bool pairs_ok = true) {
+                            bool pairs_ok = true, unsigned skew = 0) {
   std::string s;
   // elements a lane moves at a time: 4, or (plain variant only) 2 when the
   // widest type has 8 bytes, so that the widest access stays at 16 bytes
@@ -689,7 +689,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // the same along y (bits 16.. of zmask; transposed variant only): one load
   // serves the four rows a lane works on
   auto is_y = [&](size_t j) {
-    return aidx[j] >= 0 && ((zmask >> (16 + aidx[j])) & 1u) && !ge->args[j].writes();
+    return skew == 0 && aidx[j] >= 0 && ((zmask >> (16 + aidx[j])) & 1u) && !ge->args[j].writes();
   };
   auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * VQ); };
   // 16-byte accesses of arrays whose every element is touched once carry the
@@ -812,7 +812,35 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // ---- transposed, nd >= 2 ----
   const unsigned yd = nd - 2;
   const unsigned T = tile, Q = tile / 4;
-  const std::string TP = std::to_string(T + 1) + "u";
+  // Rows of the array `skew` names (its number among the arrays, plus one; a
+  // direct result of four-byte elements) that do not start on 64-byte
+  // boundaries: a tile's window on row y is moved left by the ga_sy elements
+  // (0, 4, 8 or 12) that put its first element on such a boundary, so that a
+  // group stores whole 64-byte blocks only; the blocks a rectangular tile
+  // would share with its neighbours reach memory as two partial writes
+  // (out = in.T of 8192 x 8192 floats, rows 32 bytes into a line: 136 us
+  // against 89 on whole lines).  The staged tiles then hold SK more columns,
+  // fetched by one more pass of the group, and the grid has tiles for SK more
+  // columns than the rows have.
+  const unsigned SK = skew ? 12u : 0u, W = T + SK, LP = W + 1;
+  const unsigned NP = (W + Q - 1) / Q;      // passes of Q columns over a staged tile
+  const std::string TP = std::to_string(LP) + "u";
+  const char *skew_name = nullptr;
+  for (size_t j = 0; j < ge->args.size(); j++)
+    if (skew && aidx[j] == (int)skew - 1) skew_name = ge->args[j].name.c_str();
+  const char *XB = skew ? "ga_xs" : "ga_x0";   // where a row's window starts
+  // (inside a loop over the lane's rows: the window of row ga_y0 + ga_ly)
+  auto emit_row_window = [&]() {
+    if (!skew) return;
+    appendf(s, "const %s ga_sy = (%s)((((ga_size)%s_b + (ga_size)(ga_ssize)(%s_o + (%s)(ga_y0 + ga_ly) * (%s)%s_str_%u)) & 63u) >> 2);\n",
+            N, N, skew_name, skew_name, I, I, skew_name, yd);
+    appendf(s, "const %s ga_xs = ga_x0 - ga_sy;\n", N);
+  };
+  // column of the staged tile that holds element GA_QP(v) of the row's window
+  const std::string TCOL = skew ? std::to_string(SK) + "u - ga_sy + " : "";
+  // x of column ga_lx of the staged tile (below 0 wraps to a huge value and fails the extent test)
+  const std::string TX = skew ? "ga_x0 + ga_lx - " + std::to_string(SK) + "u" : "ga_x0 + ga_lx";
+  const std::string LXOK = NP * Q > W ? "ga_lx < " + std::to_string(W) + "u && " : "";
   // A lane's four elements along an axis (its "quad").  With elements of up
   // to four bytes they are adjacent, one access of up to 16 bytes.  With
   // eight-byte elements in the kernel they are two pairs, half a tile apart:
@@ -832,7 +860,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   for (size_t j = 0; j < ge->args.size(); j++)
     if (is_t(j))
       appendf(s, "LOCAL_MEM %s %s_t[%u * %u];\n", ctype(ge->args[j].typecode),
-              ge->args[j].name.c_str(), T, T + 1);
+              ge->args[j].name.c_str(), T, LP);
   // T x T tile, T*T/16 lanes: ga_lo picks a quad along one axis, ga_hi a line
   // along the other; four passes of T/4 lines cover the tile
   // Lane -> (quad ga_lo, line ga_hi): the quad from the low bits, so that 16
@@ -909,7 +937,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // and 3), or along x at row `y` (the direct operands and results of phase 2)
   auto vec_ptr = [&](const ge_arg &a, bool along_y, unsigned h, const char *other) {
     char q[64];
-    snprintf(q, sizeof(q), "%s + GA_QP(%uu)", along_y ? "ga_y0" : "ga_x0", h * VE);
+    snprintf(q, sizeof(q), "%s + GA_QP(%uu)", along_y ? "ga_y0" : XB, h * VE);
     std::string pe;
     appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", vec_t(a), a.name.c_str(),
             (along_y ? off_yx(a, q, other) : off_yx(a, other, q)).c_str());
@@ -918,7 +946,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // is access h of the quad, whose other coordinate is in range, in range itself?
   auto in_range = [&](bool along_y, unsigned h) {
     std::string c;
-    appendf(c, "%s + GA_QP(%uu) < (%s)dim%u", along_y ? "ga_y0" : "ga_x0", h * VE, N, along_y ? yd : xd);
+    appendf(c, "%s + GA_QP(%uu) < (%s)dim%u", along_y ? "ga_y0" : XB, h * VE, N, along_y ? yd : xd);
     return c;
   };
   // loads of the operands that phase 2 reads straight from memory
@@ -931,6 +959,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
     appendf(s, "const %s ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
     appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u) {\n", N, yd);
+    emit_row_window();
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || is_t(j) || !a.reads()) continue;
@@ -951,7 +980,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       } else {
         for (int i = 0; i < 4; i++) {
           char xi[48];
-          snprintf(xi, sizeof(xi), "ga_x0 + GA_QP(%du)", i);
+          snprintf(xi, sizeof(xi), "%s + GA_QP(%du)", XB, i);
           appendf(s, "if (%s < (%s)dim%u) %s_u[ga_k].e[%d] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", xi, N, xd,
                   a.name.c_str(), i, ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str());
         }
@@ -971,12 +1000,12 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (is_t(j) && a.reads())
-        appendf(s, "union { %s p[%u]; %s e[4]; } %s_in[4];\n", vec_t(a), NH, ctype(a.typecode),
-                a.name.c_str());
+        appendf(s, "union { %s p[%u]; %s e[4]; } %s_in[%u];\n", vec_t(a), NH, ctype(a.typecode),
+                a.name.c_str(), NP);
     }
-    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_k = 0; ga_k < %u; ga_k++) {\n", NP);
     appendf(s, "const %s ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_x0 + ga_lx < (%s)dim%u) {\n", N, xd);
+    appendf(s, "if (%s%s < (%s)dim%u) {\n", LXOK.c_str(), TX.c_str(), N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
@@ -984,22 +1013,22 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
         appendf(s, "if (%s) ", in_range(true, h).c_str());
         char dst[64];
         snprintf(dst, sizeof(dst), "%s_in[ga_k].p[%u]", a.name.c_str(), h);
-        s += quad_load(j, dst, vec_ptr(a, true, h, "ga_x0 + ga_lx"));
+        s += quad_load(j, dst, vec_ptr(a, true, h, TX.c_str()));
       }
     }
     s += "}\n}\n";
     // the direct operands of phase 2 are asked for here, behind the tile's
     // loads and before the barrier, so that their latency is not paid after it
     emit_direct_loads();
-    s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
+    appendf(s, "#pragma unroll\nfor (int ga_k = 0; ga_k < %u; ga_k++) {\n", NP);
     appendf(s, "const %s ga_lx = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
-    appendf(s, "if (ga_x0 + ga_lx < (%s)dim%u) {\n", N, xd);
+    appendf(s, "if (%s%s < (%s)dim%u) {\n", LXOK.c_str(), TX.c_str(), N, xd);
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!is_t(j) || !a.reads()) continue;
       appendf(s, "#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
                  "if (ga_y0 + GA_QP(ga_i) < (%s)dim%u) %s_t[GA_QP(ga_i) * %uu + ga_lx] = %s_in[ga_k].e[ga_i];\n",
-              N, yd, a.name.c_str(), T + 1, a.name.c_str());
+              N, yd, a.name.c_str(), LP, a.name.c_str());
     }
     s += "}\n}\nlocal_barrier();\n";
   }
@@ -1008,11 +1037,12 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   s += "#pragma unroll\nfor (int ga_k = 0; ga_k < 4; ga_k++) {\n";
   appendf(s, "const %s ga_ly = ga_hi + %uu * (%s)ga_k;\n", N, Q, N);
   appendf(s, "if (ga_y0 + ga_ly < (%s)dim%u) {\n", N, yd);
-  appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) if (ga_x0 + GA_QP(ga_v) < (%s)dim%u) {\n", N, xd);
+  emit_row_window();
+  appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < 4; ga_v++) if (%s + GA_QP(ga_v) < (%s)dim%u) {\n", XB, N, xd);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * " + TP + " + GA_QP(ga_v)]");
+    if (is_t(j)) emit_load(ge, s, a, a.name + "_t[ga_ly * " + TP + " + " + TCOL + "GA_QP(ga_v)]");
     else emit_load(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += ge->expr;
@@ -1020,7 +1050,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * " + TP + " + GA_QP(ga_v)]");
+    if (is_t(j)) emit_store(ge, s, a, a.name + "_t[ga_ly * " + TP + " + " + TCOL + "GA_QP(ga_v)]");
     else emit_store(ge, s, a, a.name + "_u[ga_k].e[ga_v]");
   }
   s += "}\n";
@@ -1037,7 +1067,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     } else {
       for (int i = 0; i < 4; i++) {
         char xi[48];
-        snprintf(xi, sizeof(xi), "ga_x0 + GA_QP(%du)", i);
+        snprintf(xi, sizeof(xi), "%s + GA_QP(%du)", XB, i);
         appendf(s, "if (%s < (%s)dim%u) *(GLOBAL_MEM %s *)(%s_b + %s) = %s_u[ga_k].e[%d];\n", xi, N, xd,
                 ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", xi).c_str(), a.name.c_str(), i);
       }
@@ -1054,7 +1084,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
       if (!is_t(j) || !a.writes()) continue;
       appendf(s, "{ union { %s p[%u]; %s e[4]; } ga_o;\n#pragma unroll\nfor (int ga_i = 0; ga_i < 4; ga_i++) "
                  "ga_o.e[ga_i] = %s_t[GA_QP(ga_i) * %uu + ga_lx];\n",
-              vec_t(a), NH, ctype(a.typecode), a.name.c_str(), T + 1);
+              vec_t(a), NH, ctype(a.typecode), a.name.c_str(), LP);
       for (unsigned h = 0; h < NH; h++) {
         appendf(s, "if (%s) ", in_range(true, h).c_str());
         char val[32];
@@ -1356,6 +1386,7 @@ class strided_call {
   size_t gx = 0, groups = 0;
   unsigned ltx = 0, tile = 64, quads = 4;
   unsigned vq = 4;                  // vec4: elements a lane moves at a time (2 for 8-byte types, plain variant)
+  unsigned skew = 0;                // transposed tiles: 1 + the array whose rows the tiles' windows follow
   GpuKernel *kernel = nullptr;
 
   void describe_arrays() {
@@ -1655,11 +1686,31 @@ class strided_call {
       // in.T + b*c 24.0 -> 24.5 us, 8192 x 8192 82.0 -> 83.5): two resident
       // groups per compute unit already overlap one's loads with the other's
       // stores.
+      skew = 0;
       if (vec4) {
+        // Rows of the result off the 64-byte blocks of memory: the tiles' windows
+        // follow the rows (see the generator).  Measured on MI355X, out = in.T
+        // of 8192 x 8192 floats, rectangular against skewed tiles: result rows
+        // 32 bytes into a block 135.8 / 92.6 us, a pitch of 8328 floats (the
+        // rows walk through the four phases) 114.1 / 95.5, both pitches 8200
+        // floats 114.5 / 102.4; (5000, 3000) -> (3000, 5000) 27.2 / 25.9.
+        if (outk >= 0 && !((tmask >> outk) & 1u) && elsz[outk] == 4 && TUNE(tn, ELEMWISE_SKEW, 1) != 0) {
+          bool wide = false;
+          for (unsigned k = 0; k < na; k++) wide = wide || elsz[k] > 4;
+          const GpuArray *ov = nullptr;
+          unsigned l2 = 0;
+          for (size_t i = 0; i < ge->args.size(); i++)
+            if (ge->args[i].is_array() && l2++ == (unsigned)outk) { ov = (const GpuArray *)args[i]; break; }
+          bool whole = ((uintptr_t)ov->data->devptr + ov->offset) % 64 == 0;
+          for (unsigned j = 0; j + 1 < nd && whole; j++)
+            if (dims[j] > 1 && strs[outk][j] % 64 != 0) whole = false;
+          if (!wide && !whole) skew = (unsigned)outk + 1;
+        }
+        const size_t cols = skew ? 12 : 0;
         size_t lds128 = 0;
         for (unsigned k = 0; k < na; k++)
-          if ((tmask >> k) & 1u) lds128 += (size_t)128 * 129 * elsz[k];
-        const size_t tiles128 = ((dims[nd - 1] + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
+          if ((tmask >> k) & 1u) lds128 += (size_t)128 * (129 + cols) * elsz[k];
+        const size_t tiles128 = ((dims[nd - 1] + cols + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
                                 (n / dims[nd - 1] / dims[nd - 2]);
         // large against small tiles on smaller planes: 1536 x 1536 4.6 / 4.9 us,
         // 2048 x 2048 6.2 / 6.9, 16 planes of 512 x 512 6.0 / 6.6, 3072 x 3072
@@ -1668,7 +1719,7 @@ class strided_call {
         tile = (tiles128 >= min128 && lds128 <= 80 * 1024) ? 128 : 64;
         const unsigned long ft = TUNE(tn, ELEMWISE_TTILE, 0);
         if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
-        const size_t tiles = ((dims[nd - 1] + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
+        const size_t tiles = ((dims[nd - 1] + cols + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);
         bool aliasing = true;   // every pitch a power of two of 4 to 32 KiB
         for (unsigned k = 0; k < na && aliasing; k++) {
           // operands that are broadcast along x or y are a row or a column, not a plane
@@ -1680,7 +1731,7 @@ class strided_call {
         ltx = (unsigned)TUNE(tn, ELEMWISE_BAND, dflt) & 0xffffu;
         if (ltx == 0) ltx |= ((unsigned)TUNE(tn, ELEMWISE_PANEL, 0) & 0xffffu) << 16;
       }
-      gx = (dims[nd - 1] + tile - 1) / tile;
+      gx = (dims[nd - 1] + (skew ? 12 : 0) + tile - 1) / tile;
       size_t gy = (dims[nd - 2] + tile - 1) / tile;
       size_t outer = n / dims[nd - 1] / dims[nd - 2];
       groups = gx * gy * outer;
@@ -1695,14 +1746,14 @@ class strided_call {
     // (0: a lane's four 8-byte elements along a transposed tile's axes stay adjacent)
     const bool tpairs = TUNE(tn, ELEMWISE_TPAIRS, 1) != 0;
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u:%d", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
-             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq, tpairs ? 1 : 0);
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u:%d:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+             vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq, tpairs ? 1 : 0, vec4 ? skew : 0u);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq, tpairs)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq, tpairs, skew)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
@@ -1827,6 +1878,7 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // 8 as 4, every array that is not staged through LDS taken as constant along y
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
   // 10: as 3 with one group of two elements per lane (8-byte types, no transposed operand)
+  // 11: as 4, the tiles' windows on a row starting on the 64-byte blocks of the last array's rows
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
   // (idx64 then carries the mask of those fetched a whole chunk at a time)
   if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
@@ -1834,7 +1886,8 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
                                                    : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u,
-                                                   strided == 10 ? 1 : 4, strided == 10 ? 2 : 4)
+                                                   strided == 10 ? 1 : 4, strided == 10 ? 2 : 4, true,
+                                                   strided == 11 ? ge.narray : 0)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

@@ -85,6 +85,10 @@ def elemwise_cases():
          [("a", d, (8192, 8192), lambda b: b[:, :4096]), ("b", d, (8192, 8192), lambda b: b[:, 4096:])], (8192, 4096), d),
         ("a.T + b, 4096 x 4096 doubles", "o = a + b", [("a", d, (4096, 4096), T(1, 0)), ("b", d, (4096, 4096), None)], (4096, 4096), d),
         ("a.T + b, 8192 x 8192", "o = a + b", [("a", f, (8192, 8192), T(1, 0)), ("b", f, (8192, 8192), None)], (8192, 8192), f),
+        ("a.T, 8000 x 8000 (pitches of 32000 bytes)", "o = a", [("a", f, (8000, 8000), T(1, 0))], (8000, 8000), f),
+        ("a.T, (5000, 3000) -> (3000, 5000) (rows of 20000 bytes: off the 128-byte lines)", "o = a",
+         [("a", f, (5000, 3000), T(1, 0))], (3000, 5000), f),
+        ("a.T, (50000, 1000) -> (1000, 50000)", "o = a", [("a", f, (50000, 1000), T(1, 0))], (1000, 50000), f),
         ("transpose (0, 2, 1) of (64, 1024, 1024)", "o = a", [("a", f, (64, 1024, 1024), T(0, 2, 1))], (64, 1024, 1024), f),
         ("transpose (1, 0, 2) of (1024, 64, 1024)", "o = a", [("a", f, (1024, 64, 1024), T(1, 0, 2))], (64, 1024, 1024), f),
         ("transpose (2, 1, 0) of (256, 512, 512)", "o = a", [("a", f, (256, 512, 512), T(2, 1, 0))], (512, 512, 256), f),

@@ -558,6 +558,46 @@ def test_transposed_tiles_and_bands(ctx, knobs, tile, band, panel):
     assert np.array_equal(np.asarray(o), p.transpose(0, 2, 1) * 2.0)
 
 
+@pytest.mark.parametrize("skew", [1, 0])
+@pytest.mark.parametrize("tile", [64, 128])
+def test_tile_windows_follow_result_rows_off_the_64_byte_blocks(ctx, knobs, tile, skew):
+    """A result whose rows do not start on 64-byte blocks of memory: the
+    transposed kernels move a tile's window on every row to the block
+    boundary before it (ELEMWISE_SKEW).  Every phase of the first row (base 0
+    to 12 floats into a block), pitches that walk through the phases from row
+    to row, extents around a tile's width and around the extra columns the
+    windows need, a row operand (its window moves with the row), several
+    planes; with the rectangular tiles as well.  The whole buffer of the result
+    is compared, so a store outside the view shows."""
+    knobs(ELEMWISE_TTILE=tile, ELEMWISE_SKEW=skew)
+    rng = np.random.default_rng(700 + tile)
+    k = ga.GpuElemwise(ctx, "o = a * r + c", [arg("a", "float32", read=True), arg("r", "float32", read=True),
+                                              arg("c", "float32", read=True), arg("o", "float32", write=True)])
+    cases = [(ny, nx, pad, lead) for ny in (36, 132) for nx in (4, 52, 116, 120, 124, 128, 132, 244, 252, 260)
+             for pad, lead in ((4, 0), (8, 4), (12, 8), (20, 12), (16, 0), (0, 4))]
+    for ny, nx, pad, lead in cases[::3] if tile == 64 else cases[1::3] + cases[2::3]:
+        a = rng.integers(-9, 10, size=(nx, ny)).astype(np.float32)              # read as a.T
+        r = rng.integers(-9, 10, size=(1, nx)).astype(np.float32)
+        c = rng.integers(-9, 10, size=(ny, nx + 8)).astype(np.float32)[:, 4:4 + nx]   # its own phase
+        root = rng.integers(-9, 10, size=(ny + 2, lead + nx + pad)).astype(np.float32)
+        view = root[1:1 + ny, lead:lead + nx]
+        go, groot = to_gpu_view(view, ctx)
+        gc, _ = to_gpu_view(c, ctx)
+        k(gpuarray.array(a, context=ctx).T, gpuarray.array(r, context=ctx), gc, go, broadcast=True)
+        want = root.copy()
+        want[1:1 + ny, lead:lead + nx] = a.T * r + c
+        assert np.array_equal(read_root(groot, root), want), (ny, nx, pad, lead)
+    # planes: the phase of a row depends on the plane too
+    p = rng.integers(-9, 10, size=(3, 140, 76)).astype(np.float32)
+    root = np.zeros((3, 76, 140 + 4), np.float32)
+    go, groot = to_gpu_view(root[:, :, :140], ctx)
+    kc = ga.GpuElemwise(ctx, "o = p", [arg("p", "float32", read=True), arg("o", "float32", write=True)])
+    kc(gpuarray.array(p, context=ctx).transpose(0, 2, 1), go)
+    want = root.copy()
+    want[:, :, :140] = p.transpose(0, 2, 1)
+    assert np.array_equal(read_root(groot, root), want)
+
+
 def test_math_library_functions_match_numpy(ctx):
     """The C math library as kernels see it (the library's own device runtime
     maps it to compiler builtins and the device library): every function on
