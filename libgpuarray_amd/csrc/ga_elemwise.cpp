@@ -173,6 +173,7 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
   s += "#include \"cluda.h\"\n";
   s += "typedef ga_uint __attribute__((ext_vector_type(2))) ga_chunk8;\n"
        "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n"
+       "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n"
        "typedef ga_uint __attribute__((ext_vector_type(8))) ga_chunk32;\n";
   s += ge->preamble;
   s += "\n";
@@ -642,7 +643,7 @@ std::string gen_strided(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned
 std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned tmask,
                             unsigned umask, std::vector<int> &ktypes, unsigned ntmask = 0,
                             unsigned tile = 64, unsigned zmask = 0, unsigned quads = 4, unsigned vq = 4,
-                            bool pairs_ok = true, unsigned skew = 0) {
+                            bool pairs_ok = true, unsigned skew = 0, bool loose = false) {
   std::string s;
   // elements a lane moves at a time: 4, or (plain variant only) 2 when the
   // widest type has 8 bytes, so that the widest access stays at 16 bytes
@@ -822,7 +823,12 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   // against 89 on whole lines).  The staged tiles then hold SK more columns,
   // fetched by one more pass of the group, and the grid has tiles for SK more
   // columns than the rows have.
-  const unsigned SK = skew ? 12u : 0u, W = T + SK, LP = W + 1;
+  // `loose` (every array of four-byte elements): nothing is asked of bases,
+  // pitches and extents.  A lane's four elements are then one access that is
+  // only known to lie on a four-byte boundary (the windows still put the
+  // result's on 16), rows can start at any of the 16 elements of a block, and
+  // the quads that an extent cuts are moved element by element.
+  const unsigned SK = skew ? (loose ? 15u : 12u) : 0u, W = T + SK, LP = W | 1u;   // (an odd pitch of the staged tile, for its banks)
   const unsigned NP = (W + Q - 1) / Q;      // passes of Q columns over a staged tile
   const std::string TP = std::to_string(LP) + "u";
   const char *skew_name = nullptr;
@@ -856,7 +862,9 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     if (a.is_array()) widest = std::max(widest, gpuarray_get_elsize(a.typecode));
   const bool halves = widest == 8 && pairs_ok;
   const unsigned NH = halves ? 2 : 1, VE = 4 / NH;   // accesses per quad, elements per access
-  auto vec_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * VE); };
+  auto vec_t = [&](const ge_arg &a) {
+    return loose ? "ga_chunk16u" : chunk_type(gpuarray_get_elsize(a.typecode) * VE);
+  };
   for (size_t j = 0; j < ge->args.size(); j++)
     if (is_t(j))
       appendf(s, "LOCAL_MEM %s %s_t[%u * %u];\n", ctype(ge->args[j].typecode),
@@ -947,7 +955,26 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   auto in_range = [&](bool along_y, unsigned h) {
     std::string c;
     appendf(c, "%s + GA_QP(%uu) < (%s)dim%u", along_y ? "ga_y0" : XB, h * VE, N, along_y ? yd : xd);
+    if (loose)   // the whole quad (a window can start below 0: its first positions wrap to huge values)
+      appendf(c, " && %s + GA_QP(%uu) + 3u < (%s)dim%u", along_y ? "ga_y0" : XB, h * VE, N, along_y ? yd : xd);
     return c;
+  };
+  // loose: the elements of a quad that the extent cuts, one by one
+  // (`reg` names the lane's copy of the quad; element i of it is reg.e[i])
+  auto emit_cut_quad = [&](const ge_arg &a, bool along_y, const char *other, const std::string &reg, bool store) {
+    if (!loose) return;
+    s += "else {\n";
+    for (int i = 0; i < 4; i++) {
+      char q[64];
+      snprintf(q, sizeof(q), "%s + GA_QP(%du)", along_y ? "ga_y0" : XB, i);
+      std::string pe;
+      appendf(pe, "*(GLOBAL_MEM %s *)(%s_b + %s)", ctype(a.typecode), a.name.c_str(),
+              (along_y ? off_yx(a, q, other) : off_yx(a, other, q)).c_str());
+      appendf(s, "if (%s < (%s)dim%u) ", q, N, along_y ? yd : xd);
+      if (store) appendf(s, "%s = %s.e[%d];\n", pe.c_str(), reg.c_str(), i);
+      else appendf(s, "%s.e[%d] = %s;\n", reg.c_str(), i, pe.c_str());
+    }
+    s += "}\n";
   };
   // loads of the operands that phase 2 reads straight from memory
   auto emit_direct_loads = [&]() {
@@ -970,9 +997,11 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
           char dst[64];
           snprintf(dst, sizeof(dst), "%s_u[ga_k].p[%u]", a.name.c_str(), h);
           s += quad_load(j, dst, vec_ptr(a, false, h, "ga_y0 + ga_ly"));
+          emit_cut_quad(a, false, "ga_y0 + ga_ly", a.name + "_u[ga_k]", false);
         }
       } else if (is_z(j)) {
-        appendf(s, "if (%s) {\n%s_u[ga_k].e[0] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", in_range(false, 0).c_str(),
+        // (loose: some element of a cut quad may be in range, and the row's element 0 always exists)
+        appendf(s, "if (%s) {\n%s_u[ga_k].e[0] = *(GLOBAL_MEM %s *)(%s_b + %s);\n", loose ? "true" : in_range(false, 0).c_str(),
                 a.name.c_str(), ctype(a.typecode), a.name.c_str(), off_yx(a, "ga_y0 + ga_ly", "0").c_str());
         for (int i = 1; i < 4; i++)
           appendf(s, "%s_u[ga_k].e[%d] = %s_u[ga_k].e[0];\n", a.name.c_str(), i, a.name.c_str());
@@ -1014,6 +1043,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
         char dst[64];
         snprintf(dst, sizeof(dst), "%s_in[ga_k].p[%u]", a.name.c_str(), h);
         s += quad_load(j, dst, vec_ptr(a, true, h, TX.c_str()));
+        emit_cut_quad(a, true, TX.c_str(), a.name + "_in[ga_k]", false);
       }
     }
     s += "}\n}\n";
@@ -1063,6 +1093,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
         char val[64];
         snprintf(val, sizeof(val), "%s_u[ga_k].p[%u]", a.name.c_str(), h);
         s += quad_store(j, vec_ptr(a, false, h, "ga_y0 + ga_ly"), val);
+        emit_cut_quad(a, false, "ga_y0 + ga_ly", a.name + "_u[ga_k]", true);
       }
     } else {
       for (int i = 0; i < 4; i++) {
@@ -1387,6 +1418,7 @@ class strided_call {
   unsigned ltx = 0, tile = 64, quads = 4;
   unsigned vq = 4;                  // vec4: elements a lane moves at a time (2 for 8-byte types, plain variant)
   unsigned skew = 0;                // transposed tiles: 1 + the array whose rows the tiles' windows follow
+  bool loose = false;               // transposed tiles of four-byte elements on any bases, pitches and extents
   GpuKernel *kernel = nullptr;
 
   void describe_arrays() {
@@ -1562,6 +1594,13 @@ class strided_call {
     }
   }
 
+  bool array_writes(unsigned k) const {
+    unsigned l = 0;
+    for (size_t i = 0; i < ge->args.size(); i++)
+      if (ge->args[i].is_array() && l++ == k) return ge->args[i].writes();
+    return false;
+  }
+
   void choose_offset_width() {
     // 32-bit offsets when every reachable byte offset fits
     idx64 = n >= (size_t)GA_SADDR32_MAX;
@@ -1612,6 +1651,36 @@ class strided_call {
         zmask |= 1u << (16 + k);
     }
     if (vec4 && !((umask >> outk) & 1u)) vec4 = false;
+    // Transposed operands whose layout fails the above - an extent that is no
+    // multiple of four, rows that start off the 16-byte boundaries - still
+    // move four elements per lane when every array has four-byte elements:
+    // accesses that only assume a four-byte boundary, and the quads that an
+    // extent cuts element by element (see the generator).  Measured on
+    // MI355X, out = in.T of floats, one element per lane against this:
+    // 8190 x 8190 154.9 / 110.6 us, 8191 x 8193 150.1 / 106.2; 8192 x 8192
+    // inside wider buffers, the result's pitch 8318 floats 154.1 / 96.3, the
+    // operand's 8319 floats 117.2 / 101.4, extents 8190 on pitches of 8320
+    // floats 102.9 / 93.1; out = in.T + b of 8190 x 8190 207.4 / 158.4.
+    loose = false;
+    if (!vec4 && tmask && !((tmask >> outk) & 1u) && TUNE(tn, ELEMWISE_VEC4, 1) != 0 &&
+        TUNE(tn, ELEMWISE_LOOSE, 1) != 0 && na <= 31 && strs[outk][nd - 1] == 4) {
+      bool ok = true;
+      unsigned um = 0, zm = 0;
+      for (unsigned k = 0; k < na && ok; k++) {
+        const bool tr = (tmask >> k) & 1u;
+        if (elsz[k] != 4) ok = false;
+        else if (tr) ok = strs[k][nd - 2] == 4 && !array_writes(k);
+        else if (strs[k][nd - 1] == 4) um |= 1u << k;
+        else if (strs[k][nd - 1] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) zm |= 1u << k;
+        if (!tr && k < 16 && strs[k][nd - 2] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) zm |= 1u << (16 + k);
+      }
+      if (ok) {
+        loose = vec4 = true;
+        vq = 4;
+        umask = um;
+        zmask = zm;
+      }
+    }
     // arrays read or written exactly once per element stream past the caches
     if (vec4 && ge->nontemporal) {
       for (unsigned k = 0; k < na; k++) {
@@ -1706,10 +1775,10 @@ class strided_call {
             if (dims[j] > 1 && strs[outk][j] % 64 != 0) whole = false;
           if (!wide && !whole) skew = (unsigned)outk + 1;
         }
-        const size_t cols = skew ? 12 : 0;
+        const size_t cols = skew ? (loose ? 15 : 12) : 0;
         size_t lds128 = 0;
         for (unsigned k = 0; k < na; k++)
-          if ((tmask >> k) & 1u) lds128 += (size_t)128 * (129 + cols) * elsz[k];
+          if ((tmask >> k) & 1u) lds128 += (size_t)128 * ((128 + cols) | 1) * elsz[k];
         const size_t tiles128 = ((dims[nd - 1] + cols + 127) / 128) * ((dims[nd - 2] + 127) / 128) *
                                 (n / dims[nd - 1] / dims[nd - 2]);
         // large against small tiles on smaller planes: 1536 x 1536 4.6 / 4.9 us,
@@ -1731,7 +1800,7 @@ class strided_call {
         ltx = (unsigned)TUNE(tn, ELEMWISE_BAND, dflt) & 0xffffu;
         if (ltx == 0) ltx |= ((unsigned)TUNE(tn, ELEMWISE_PANEL, 0) & 0xffffu) << 16;
       }
-      gx = (dims[nd - 1] + (skew ? 12 : 0) + tile - 1) / tile;
+      gx = (dims[nd - 1] + (skew ? (loose ? 15 : 12) : 0) + tile - 1) / tile;
       size_t gy = (dims[nd - 2] + tile - 1) / tile;
       size_t outer = n / dims[nd - 1] / dims[nd - 2];
       groups = gx * gy * outer;
@@ -1746,14 +1815,14 @@ class strided_call {
     // (0: a lane's four 8-byte elements along a transposed tile's axes stay adjacent)
     const bool tpairs = TUNE(tn, ELEMWISE_TPAIRS, 1) != 0;
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u:%d:%u", vec4 ? "v" : "s", nd, idx64 ? 1 : 0, tmask,
+    snprintf(key, sizeof(key), "%s%u:%d:%x:%x:%x:%x:%u:%u:%u:%d:%u", vec4 ? (loose ? "l" : "v") : "s", nd, idx64 ? 1 : 0, tmask,
              vec4 ? umask : 0u, ntmask, vec4 ? zmask : 0u, tile, quads, vq, tpairs ? 1 : 0, vec4 ? skew : 0u);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq, tpairs, skew)
+      std::string src = vec4 ? gen_strided_vec(ge, nd, idx64, tmask, umask, ktypes, ntmask, tile, zmask, quads, vq, tpairs, skew, loose)
                              : gen_strided(ge, nd, idx64, tmask, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       int err = build_kernel(ge, &nk, src, ktypes);
@@ -1879,6 +1948,7 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   if (strided == 5 || strided == 6) return strdup(gen_flat(&ge, ktypes, strided == 5 ? 2 : 4, 1).c_str());
   // 10: as 3 with one group of two elements per lane (8-byte types, no transposed operand)
   // 11: as 4, the tiles' windows on a row starting on the 64-byte blocks of the last array's rows
+  // 12: as 11 for four-byte elements on any bases, pitches and extents
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
   // (idx64 then carries the mask of those fetched a whole chunk at a time)
   if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
@@ -1887,7 +1957,7 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
                                                    : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u,
                                                    strided == 10 ? 1 : 4, strided == 10 ? 2 : 4, true,
-                                                   strided == 11 ? ge.narray : 0)
+                                                   strided == 11 || strided == 12 ? ge.narray : 0, strided == 12)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

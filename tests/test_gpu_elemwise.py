@@ -598,6 +598,51 @@ def test_tile_windows_follow_result_rows_off_the_64_byte_blocks(ctx, knobs, tile
     assert np.array_equal(read_root(groot, root), want)
 
 
+@pytest.mark.parametrize("loose", [1, 0])
+@pytest.mark.parametrize("dtype", ["float32", "int32"])
+def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
+    """Transposed operands whose bases, pitches and extents are no multiples of
+    four elements (ELEMWISE_LOOSE: four elements per lane through accesses that
+    assume four-byte boundaries only, cut quads element by element; 0: one
+    element per lane).  Odd extents around the tile sizes, every phase of the
+    operand's and the result's first element, a row and a column operand, a
+    second transposed operand, planes; the result's whole buffer is compared."""
+    knobs(ELEMWISE_LOOSE=loose)
+    rng = np.random.default_rng(810 + loose)
+    k = ga.GpuElemwise(ctx, "o = a * r + c", [arg("a", dtype, read=True), arg("r", dtype, read=True),
+                                              arg("c", dtype, read=True), arg("o", dtype, write=True)])
+    k2 = ga.GpuElemwise(ctx, "o = a - b", [arg("a", dtype, read=True), arg("b", dtype, read=True),
+                                           arg("o", dtype, write=True)])
+    draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
+    for ny, nx in ((17, 19), (63, 130), (129, 127), (131, 257), (250, 66), (61, 391), (257, 129)):
+        for la, lo_, pad in ((0, 0, 0), (1, 0, 3), (2, 3, 1), (3, 1, 2), (0, 2, 5)):
+            aroot = draw((nx + 1, la + ny + pad))
+            a = aroot[1:, la:la + ny]                        # read as a.T: rows start at any element
+            r = draw((1, nx))
+            c = draw((ny, 1))
+            root = draw((ny + 2, lo_ + nx + pad))
+            view = root[1:1 + ny, lo_:lo_ + nx]
+            go, groot = to_gpu_view(view, ctx)
+            gat, _ = to_gpu_view(a.T, ctx)
+            k(gat, gpuarray.array(r, context=ctx), gpuarray.array(c, context=ctx), go, broadcast=True)
+            want = root.copy()
+            want[1:1 + ny, lo_:lo_ + nx] = a.T * r + c
+            assert np.array_equal(read_root(groot, root), want), (ny, nx, la, lo_, pad)
+            b = draw((nx, ny + 1))[:, 1:]
+            gbt, _ = to_gpu_view(b.T, ctx)
+            k2(gat, gbt, go)
+            want[1:1 + ny, lo_:lo_ + nx] = a.T - b.T
+            assert np.array_equal(read_root(groot, root), want), (ny, nx, la, lo_, pad)
+    p = draw((3, 133, 77))
+    root = np.zeros((3, 77, 133 + 3), dtype)
+    go, groot = to_gpu_view(root[:, :, 2:135], ctx)
+    kc = ga.GpuElemwise(ctx, "o = p", [arg("p", dtype, read=True), arg("o", dtype, write=True)])
+    kc(gpuarray.array(p, context=ctx).transpose(0, 2, 1), go)
+    want = root.copy()
+    want[:, :, 2:135] = p.transpose(0, 2, 1)
+    assert np.array_equal(read_root(groot, root), want)
+
+
 def test_math_library_functions_match_numpy(ctx):
     """The C math library as kernels see it (the library's own device runtime
     maps it to compiler builtins and the device library): every function on
