@@ -72,6 +72,10 @@ def main():
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 12, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4 transposed, 128-tiles, four-byte elements on any layout, 32-bit offsets",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 12, 2, 0, 0b001 | (0b100 << 16)))
+    check("elemwise strided vec4 plain, four-byte elements on any layout",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 13, 2, 0, 0b101 << 16))
+    check("elemwise strided vec4 plain, four-byte elements on any layout, 64-bit offsets, one operand element by element",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 13, 3, 1, 0b100 << 16))
     check("elemwise strided vec4 transposed, 8-byte elements (quads as two pairs)",
           gen_e(b"", b"c = a*b + 0.5", 3, dargs, 0, 3, 3, 1, 0b001 | (0b110 << 16)))
     check("elemwise strided vec4, 8-byte result written through a transposed tile",
@@ -183,7 +187,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "25 elementwise)" % (n + 20, m, t))
+          "27 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

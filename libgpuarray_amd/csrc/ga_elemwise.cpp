@@ -173,7 +173,6 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
   s += "#include \"cluda.h\"\n";
   s += "typedef ga_uint __attribute__((ext_vector_type(2))) ga_chunk8;\n"
        "typedef ga_uint __attribute__((ext_vector_type(4))) ga_chunk16;\n"
-       "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n"
        "typedef ga_uint __attribute__((ext_vector_type(8))) ga_chunk32;\n";
   s += ge->preamble;
   s += "\n";
@@ -651,6 +650,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
   emit_header(ge, s);
+  if (loose) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
   appendf(s, "KERNEL void __launch_bounds__(%u) elem(", tmask ? tile * tile / 16 : 256u);
   for (unsigned d = 0; d < nd; d++) {
     appendf(s, "%sconst ga_size dim%u", d ? ", " : "", d);
@@ -692,7 +692,9 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
   auto is_y = [&](size_t j) {
     return skew == 0 && aidx[j] >= 0 && ((zmask >> (16 + aidx[j])) & 1u) && !ge->args[j].writes();
   };
-  auto quad_t = [&](const ge_arg &a) { return chunk_type(gpuarray_get_elsize(a.typecode) * VQ); };
+  auto quad_t = [&](const ge_arg &a) {
+    return loose ? "ga_chunk16u" : chunk_type(gpuarray_get_elsize(a.typecode) * VQ);
+  };
   // 16-byte accesses of arrays whose every element is touched once carry the
   // streaming hint (ntmask); broadcast operands stay cacheable
   auto is_nt = [&](size_t j) { return aidx[j] >= 0 && ((ntmask >> aidx[j]) & 1u); };
@@ -755,13 +757,41 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     // quad index q = (bx*quads + e) * TX + tx, x = VQ*q
     appendf(s, "const %s ga_q0 = (ga_bx * %uu << ga_ltx) + ga_tx;\n", N, quads);
     appendf(s, "const %s ga_nq = (%s)dim%u / %uu;\n", N, N, xd, VQ);
+    // loose (four-byte elements on any layout, `skew` names the result): the
+    // quads of a row start ga_sy elements before it, so that the result's lie
+    // on 16-byte boundaries; a quad that an end of the row cuts is moved
+    // element by element (positions before the row wrap to huge values)
+    const char *skew_name = nullptr;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (loose && skew && aidx[j] == (int)skew - 1) skew_name = ge->args[j].name.c_str();
+    if (loose)
+      appendf(s, "const %s ga_sy = (%s)((((ga_size)%s_b + (ga_size)(ga_ssize)%s_o) & 15u) >> 2);\n", N, N,
+              skew_name, skew_name);
+    const std::string XQ = loose ? " - ga_sy" : "";
+    const std::string WHOLE = loose ? " && ga_x + 3u < (" + std::string(N) + ")dim" + std::to_string(xd) : "";
+    auto emit_cut = [&](bool store) {
+      if (!loose) return;
+      s += "else {\n";
+      for (size_t j = 0; j < ge->args.size(); j++) {
+        const ge_arg &a = ge->args[j];
+        if (!a.is_array() || !(store ? a.writes() : a.reads())) continue;
+        for (int i = 0; i < 4; i++) {
+          char xi[32];
+          snprintf(xi, sizeof(xi), "ga_x + %du", i);
+          const std::string at = elem_at(a, a.name + "_o", (!store && is_z(j)) ? "0" : xi);
+          if (store) appendf(s, "if (%s < (%s)dim%u) %s = %s_u[ga_e].e[%d];\n", xi, N, xd, at.c_str(), a.name.c_str(), i);
+          else appendf(s, "if (%s < (%s)dim%u) %s_u[ga_e].e[%d] = %s;\n", xi, N, xd, a.name.c_str(), i, at.c_str());
+        }
+      }
+      s += "}\n";
+    };
     for (const ge_arg &a : ge->args)
       if (a.is_array())
         appendf(s, "union { %s c; %s e[%u]; } %s_u[4];\n", quad_t(a), ctype(a.typecode), VQ,
                 a.name.c_str());
     appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
-    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, VQ, N);
-    appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
+    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx))%s;\n", N, VQ, N, XQ.c_str());
+    appendf(s, "if (ga_x < (%s)dim%u%s) {\n", N, xd, WHOLE.c_str());
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || !a.reads()) continue;
@@ -780,11 +810,19 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
         }
       }
     }
-    s += "}\n}\n";
+    s += "}\n";
+    emit_cut(false);
+    s += "}\n";
     appendf(s, "#pragma unroll\nfor (int ga_e = 0; ga_e < %u; ga_e++) {\n", quads);
-    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx));\n", N, VQ, N);
-    appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
-    appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", VQ);
+    appendf(s, "const %s ga_x = %uu * (ga_q0 + ((%s)ga_e << ga_ltx))%s;\n", N, VQ, N, XQ.c_str());
+    if (loose) {
+      // some element of the quad in the row (a quad that starts before the row has wrapped)
+      appendf(s, "if (ga_x < (%s)dim%u || ga_x + 3u < 3u) {\n", N, xd);
+      appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) if (ga_x + ga_v < (%s)dim%u) {\n", VQ, N, xd);
+    } else {
+      appendf(s, "if (ga_x < (%s)dim%u) {\n", N, xd);
+      appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", VQ);
+    }
     for (const ge_arg &a : ge->args)
       if (a.is_array()) emit_load(ge, s, a, a.name + "_u[ga_e].e[ga_v]");
     s += ge->expr;
@@ -792,6 +830,7 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
     for (const ge_arg &a : ge->args)
       if (a.is_array()) emit_store(ge, s, a, a.name + "_u[ga_e].e[ga_v]");
     s += "}\n";
+    if (loose) appendf(s, "if (ga_x < (%s)dim%u%s) {\n", N, xd, WHOLE.c_str());
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || !a.writes()) continue;
@@ -805,6 +844,10 @@ std::string gen_strided_vec(const GpuElemwise *ge, unsigned nd, bool idx64, unsi
                   a.name.c_str(), i);
         }
       }
+    }
+    if (loose) {
+      s += "}\n";
+      emit_cut(true);
     }
     s += "}\n}\n}\n";
     return s;
@@ -1661,8 +1704,13 @@ class strided_call {
     // inside wider buffers, the result's pitch 8318 floats 154.1 / 96.3, the
     // operand's 8319 floats 117.2 / 101.4, extents 8190 on pitches of 8320
     // floats 102.9 / 93.1; out = in.T + b of 8190 x 8190 207.4 / 158.4.
+    // The same without transposed operands (a row's quads then start on the
+    // result's 16-byte boundaries): o = a + b on 8192 rows of 8191 floats
+    // inside pitches of 8320 137.9 / 122.5 us (73 -> 82 % of peak), rows of
+    // 8192 that start one element in 144.0 / 121.9, pitches of 8319 floats
+    // 141.8 / 125.6, 65536 rows of 1001 in pitches of 1003 141.9 / 122.2.
     loose = false;
-    if (!vec4 && tmask && !((tmask >> outk) & 1u) && TUNE(tn, ELEMWISE_VEC4, 1) != 0 &&
+    if (!vec4 && !((tmask >> outk) & 1u) && TUNE(tn, ELEMWISE_VEC4, 1) != 0 &&
         TUNE(tn, ELEMWISE_LOOSE, 1) != 0 && na <= 31 && strs[outk][nd - 1] == 4) {
       bool ok = true;
       unsigned um = 0, zm = 0;
@@ -1672,7 +1720,7 @@ class strided_call {
         else if (tr) ok = strs[k][nd - 2] == 4 && !array_writes(k);
         else if (strs[k][nd - 1] == 4) um |= 1u << k;
         else if (strs[k][nd - 1] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) zm |= 1u << k;
-        if (!tr && k < 16 && strs[k][nd - 2] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) zm |= 1u << (16 + k);
+        if (!tr && tmask && k < 16 && strs[k][nd - 2] == 0 && TUNE(tn, ELEMWISE_ZMASK, 1) != 0) zm |= 1u << (16 + k);
       }
       if (ok) {
         loose = vec4 = true;
@@ -1697,6 +1745,9 @@ class strided_call {
     // launch geometry
     if (tmask == 0) {
       size_t inner = vec4 ? dims[nd - 1] / vq : dims[nd - 1];   // lanes needed along x
+      // (loose: a row's quads start up to three elements before it)
+      skew = 0;
+      if (vec4 && loose) { inner = (dims[nd - 1] + 6) / 4; skew = (unsigned)outk + 1; }
       // as many lanes along x as the inner extent needs (a power of two), the
       // rest of the 256 along the rows: 2^24 floats in rows of 3 took 191 us
       // with a floor of 16 lanes along x, 61 us without
@@ -1949,15 +2000,17 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // 10: as 3 with one group of two elements per lane (8-byte types, no transposed operand)
   // 11: as 4, the tiles' windows on a row starting on the 64-byte blocks of the last array's rows
   // 12: as 11 for four-byte elements on any bases, pitches and extents
+  // 13: as 3 for the same
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
   // (idx64 then carries the mask of those fetched a whole chunk at a time)
   if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
-                                                   strided >= 3 ? 0xffffffffu : 0u, strided >= 4 ? 128 : 64,
+                                                   strided >= 3 ? 0xffffffffu : 0u, strided >= 4 && strided != 13 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu
                                                    : strided == 8 ? (~tmask & 0xffffu) << 16 : 0u,
                                                    strided == 10 ? 1 : 4, strided == 10 ? 2 : 4, true,
-                                                   strided == 11 || strided == 12 ? ge.narray : 0, strided == 12)
+                                                   strided >= 11 && strided <= 13 ? ge.narray : 0,
+                                                   strided == 12 || strided == 13)
                     : strided  ? gen_strided(&ge, nd, idx64 != 0, tmask, ktypes)
                                : gen_flat(&ge, ktypes);
   return strdup(src.c_str());

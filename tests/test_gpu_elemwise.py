@@ -643,6 +643,45 @@ def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dty
     assert np.array_equal(read_root(groot, root), want)
 
 
+@pytest.mark.parametrize("loose", [1, 0])
+def test_row_views_of_four_byte_elements_on_any_layout(ctx, knobs, loose):
+    """Views without transposed operands whose rows start at any element and
+    have any length: the quads of a row start on the result's 16-byte
+    boundaries, before the row if need be, and the quads that an end of the
+    row cuts move element by element (ELEMWISE_LOOSE; 0: one element per
+    lane).  Rows of 1 to 9 elements in every phase (a cut quad can hold the
+    whole row), longer odd rows, operands in other phases than the result,
+    a stepped and a constant operand; the result's whole buffer is compared."""
+    knobs(ELEMWISE_LOOSE=loose)
+    rng = np.random.default_rng(830 + loose)
+    k = ga.GpuElemwise(ctx, "o = a * s + c", [arg("a", "float32", read=True), arg("s", "float32", read=True),
+                                              arg("c", "float32", read=True), arg("o", "float32", write=True)])
+    draw = lambda shape: rng.integers(-9, 10, size=shape).astype(np.float32)
+    for rows in (1, 7, 300):
+        for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 31, 130, 1001):
+            for lo_, la, pad in ((0, 1, 1), (1, 0, 2), (2, 3, 1), (3, 2, 3)):
+                root = draw((rows + 1, lo_ + n + pad))
+                view = root[1:, lo_:lo_ + n]
+                a = draw((rows, la + n + 2))[:, la:la + n]
+                st = draw((rows, 2 * n + 1))[:, 1::2]                  # stepped along the row
+                c = draw((rows, 1))                                    # constant along the row
+                go, groot = to_gpu_view(view, ctx)
+                k(to_gpu_view(a, ctx)[0], to_gpu_view(st, ctx)[0], gpuarray.array(c, context=ctx), go, broadcast=True)
+                want = root.copy()
+                want[1:, lo_:lo_ + n] = a * st + c
+                assert np.array_equal(read_root(groot, root), want), (rows, n, lo_, la, pad)
+    # rows that run backwards through memory, next to each other
+    root = draw((40, 6))
+    view = root[::-1, 1:4]
+    a = draw((40, 3))
+    go, groot = to_gpu_view(view, ctx)
+    k(gpuarray.array(a, context=ctx), gpuarray.array(a, context=ctx), gpuarray.array(draw((40, 1)) * 0, context=ctx), go,
+      broadcast=True)
+    want = root.copy()
+    want[::-1, 1:4] = a * a
+    assert np.array_equal(read_root(groot, root), want)
+
+
 def test_math_library_functions_match_numpy(ctx):
     """The C math library as kernels see it (the library's own device runtime
     maps it to compiler builtins and the device library): every function on
