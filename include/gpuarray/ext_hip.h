@@ -108,7 +108,9 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
  * (32-bit divisions); bit 29: also the kernel that walks rows of at most 32
  * bytes in registers, with bits 0..7 of vec as the row length in elements;
  * bit 30: also the kernel that reduces the leading dims of a dense array over
- * short kept rows in one launch. */
+ * short kept rows in one launch; bit 31: the column kernel's loads assume the
+ * elements' own alignment only, and the inner free dim need not be a multiple
+ * of the outputs per lane. */
 typedef char *(*ga_hip_reduction_source_fn)(int op, int src_typecode, int d0_typecode,
                                             int d1_typecode, unsigned int lanes_per_output,
                                             unsigned int vec, unsigned int unroll);

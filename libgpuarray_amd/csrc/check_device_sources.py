@@ -129,6 +129,11 @@ def main():
         check("column min / max in rising index order, op %d type %d" % (op, src),
               gen_r(op, src, src, GA_LONG, 256, 1 | (4 << 16), 4 | (1 << 26)))
         n += 1
+    for op, src, cv in ((0, GA_FLOAT, 4), (8, GA_FLOAT, 4), (6, GA_INT, 4), (0, GA_INT, 2)):
+        check("column reduction on any alignment and extent, op %d type %d, %d outputs per lane" % (op, src, cv),
+              gen_r(op, src, GA_LONG if (op == 0 and src == GA_INT) else src, GA_LONG, 256, 1 | (cv << 16),
+                    4 | (1 << 31) | ((1 << 26) if op in (6, 8) else 0)))
+        n += 1
     for op, cv in ((13, 16), (12, 4), (13, 8)):
         check("column any / all over bytes, op %d, %d outputs per lane" % (op, cv),
               gen_r(op, GA_UBYTE, GA_BOOL, GA_LONG, 256, 1 | (cv << 16), 4))

@@ -284,6 +284,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
       (unsigned)gpuarray_get_elsize(gr->args[gr->arrays[0]].tc));
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
   DEF("#define RD_PCOLS %u\n", (vs.opts >> 11) & 1u);
+  DEF("#define RD_CLOOSE %u\n", (vs.opts >> 12) & 1u);
   {
     // redux_trows: a lane's run of whole rows in whole 16-byte chunks
     const unsigned te = vs.TE ? vs.TE : 1;
@@ -437,13 +438,29 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
     if ((es == 1 || es == 2) && (cvn * es) % 4 == 0) words[k] = cvn * es / 4;
     if (words[k] == 1) GEN("typedef ga_uint rd_cv%u_t;\n", k);
     else if (words[k] > 1) GEN("typedef ga_uint rd_cv%u_t __attribute__((ext_vector_type(%u)));\n", k, words[k]);
+    else if ((vs.opts >> 12) & 1u)
+      GEN("typedef %s rd_cv%u_t __attribute__((ext_vector_type(RD_CV), aligned(%u)));\n", load_type_name(tc), k, es);
     else GEN("typedef %s rd_cv%u_t __attribute__((ext_vector_type(RD_CV)));\n", load_type_name(tc), k);
   }
   gen += "struct rd_cvec {";
   for (unsigned k = 0; k < K; k++) GEN(" rd_cv%u_t x%u;", k, k);
-  gen += " };\nstatic __device__ inline void rd_cvec_load(rd_cvec &o, const char *const *p) {\n";
-  for (unsigned k = 0; k < K; k++)
-    GEN("  o.x%u = RD_LOAD((const rd_cv%u_t *)p[%u]);\n", k, k, k);
+  gen += " };\nstatic __device__ inline void rd_cvec_load(rd_cvec &o, const char *const *p, const int nv) {\n";
+  if ((vs.opts >> 12) & 1u) {
+    // (the lane at the end of the inner free dim: only its nv first elements exist)
+    gen += "  if (nv == RD_CV) {\n";
+    for (unsigned k = 0; k < K; k++)
+      GEN("    o.x%u = RD_LOAD((const rd_cv%u_t *)p[%u]);\n", k, k, k);
+    gen += "  } else {\n#pragma unroll\n    for (int c = 0; c < RD_CV; c++) {\n";
+    for (unsigned k = 0; k < K; k++) {
+      const char *t = load_type_name(gr->args[gr->arrays[k]].tc);
+      GEN("      o.x%u[c] = c < nv ? RD_LOAD((const %s *)p[%u] + c) : (%s)0;\n", k, t, k, t);
+    }
+    gen += "    }\n  }\n";
+  } else {
+    gen += "  (void)nv;\n";
+    for (unsigned k = 0; k < K; k++)
+      GEN("  o.x%u = RD_LOAD((const rd_cv%u_t *)p[%u]);\n", k, k, k);
+  }
   gen += "}\n#define RD_CVEC_VAL(o, c) rd_map(";
   for (unsigned k = 0; k < K; k++) {
     const int tc = gr->args[gr->arrays[k]].tc;
@@ -758,6 +775,7 @@ class reduction_call {
   // kernel family and lane geometry
   bool use_row = true, wrows = false, tail = false, srows = false, trows = false;
   unsigned G = 256, V = 1, U = 4, ES = 1, vecmask, RB = 1, L = 64, CV = 1, LO = 1, CY = 4;
+  bool cloose = false;   // redux_col: four outputs per lane on any alignment and extent (four-byte elements)
   size_t groups = 0, lds_bytes = 0;
   variant *var = nullptr;
 
@@ -1364,7 +1382,28 @@ class reduction_call {
         if (ok) break;
         cv /= 2;
       }
-      if (!TUNE(tn, REDUX_COLVEC, 1)) cv = 1;
+      // Four-byte elements that fail the above - an inner free dim that is no
+      // multiple of four, rows that start off the 16-byte boundaries - still
+      // go four to a lane: a load that assumes four-byte boundaries only, and
+      // the lane at the end of the dim fetches what exists of its four one by
+      // one.  Measured on MI355X, sums, one output per lane against this:
+      // over axis 0 of (8192, 8192)[:, 1:] floats 75.6 / 51.3 us (44 -> 65 % of
+      // peak), of (8192, 8192)[:, :8191] 53.2 / 49.0, of (8192, 8190) 63.4 /
+      // 50.5, over the middle axis of (64, 1001, 1001) 77.9 / 56.8.  Such loads
+      // run at about six sevenths of the rate of aligned ones ((8192, 8188):
+      // 44.2 us), and folded rows, where they apply, stay ahead ((20000, 3001)
+      // 40.2 us folded, 57.0 this way).  Not for scans that carry a position:
+      // maximum over axis 0 of (8192, 8191) 57.0 / 63.8.
+      cloose = false;
+      const bool carries_position = info.has_d1 || (minmax && is_float_type(acc_typecode(gr, d0_tc)));
+      if (cv < 4 && elsz_max == 4 && !carries_position && TUNE(tn, REDUX_COL_LOOSE, 1) != 0 && fin >= 4) {
+        bool ok = true;
+        for (unsigned q = 0; ok && q < K; q++) {
+          ok = elsz[q] == 4 && fsstr[q * RD_MAXD + p.nf - 1] == 4 && GpuArray_ISALIGNED(srcs[q].a);
+        }
+        if (ok) { cv = 4; cloose = true; }
+      }
+      if (!TUNE(tn, REDUX_COLVEC, 1)) { cv = 1; cloose = false; }
       // Splitting the reduced range costs a second pass (sum over the middle
       // axis of 256x512x512 floats: 54 us unsplit with one output per lane,
       // 64 us split in two with four), so when the widest load leaves too
@@ -1458,6 +1497,7 @@ class reduction_call {
     if (p.nsplit > 1 || !use_row) vs.opts |= 256u;
     // bit 6: redux_col meets a lane's elements in rising index order (min, max and their arg forms)
     if (!use_row && p.rising && (gr->info.kind == K_MAX || gr->info.kind == K_MIN)) vs.opts |= 64u;
+    if (!use_row && cloose && CV > 1) vs.opts |= 4096u;   // bit 12: redux_col's loads assume the elements' alignment only
     if (srows)   // one kernel, independent of the lane geometry
       vs = {d0_tc, d1_tc, 64, 1, 1, (opts & 1u) | 8u | (vs.opts & 512u), 1, 1, 1, 64, 1, 1};
     if (trows) {   // one kernel per row length
@@ -1745,7 +1785,8 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
                      ((U >> 16) & 0xffu ? 1u : 3u) | (((U >> 24) & 1u) ? 4u : 0u) |
                          (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
                          (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) |
-                         (((U >> 29) & 1u) ? 1024u : 0u) | (((U >> 30) & 1u) ? 2048u : 0u) | 48u | 256u, ES, 1,
+                         (((U >> 29) & 1u) ? 1024u : 0u) | (((U >> 30) & 1u) ? 2048u : 0u) |
+                         (((U >> 31) & 1u) ? 4096u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};

@@ -24,6 +24,10 @@
  *   RD_FAST8    one-byte elements combined four per 32-bit operation (sum, any,
  *               all; 1: unsigned bytes, 2: signed), 0: off
  *   RD_COL_FAST8  redux_col: any / all over one-byte elements work on whole words
+ *   RD_CLOOSE   redux_col: a lane's RD_CV adjacent elements are fetched with a
+ *               load that only assumes the elements' own alignment, and the
+ *               inner free dim need not be a multiple of RD_CV (the lane that
+ *               holds its end fetches its elements one by one)
  *   RD_SROWS    also emit redux_srows (short contiguous rows staged in LDS)
  *   RD_PCOLS    emit redux_pcols (leading dims of a dense array reduced over
  *               short kept rows, the array walked as one run of chunks)
@@ -362,7 +366,7 @@ static __device__ inline void rd_outer_offsets(const rd_plan &p, int ri, ga_long
  *   RD_UNIT_VAL(u, j, v)     the reduced value of element v of load j
  *   struct rd_one, rd_one_load(o, ptrs), RD_ONE_VAL(o)   the same for one
  *                            element addressed by one pointer per source
- *   struct rd_cvec, rd_cvec_load(o, ptrs), RD_CVEC_VAL(o, c)   the same for
+ *   struct rd_cvec, rd_cvec_load(o, ptrs, nv), RD_CVEC_VAL(o, c)   the same for
  *                            RD_CV adjacent elements (redux_col)
  * RD_PV (elements per vector load) and RD_LOAD are defined first because the
  * emitted text uses them. */
@@ -1585,13 +1589,13 @@ static __device__ inline ga_long rd_col_index(const rd_plan &p, const ga_long j)
 
 /* A lane's RD_CV adjacent elements at position j of the reduced range. */
 static __device__ inline void rd_col_fetch(const rd_plan &p, const char *const *srow, const ga_long j,
-                                           rd_cvec &x) {
+                                           rd_cvec &x, const int nv) {
   ga_long off[RD_NSRC], ix;
   rd_col_at(p, j, off, &ix);
   const char *ep[RD_NSRC];
 #pragma unroll
   for (int k = 0; k < RD_NSRC; k++) ep[k] = srow[k] + off[k];
-  rd_cvec_load(x, ep);
+  rd_cvec_load(x, ep, nv);
 }
 
 /* Arg-min/max and floating min/max scan a lane's elements in rising order
@@ -1625,6 +1629,13 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   const ga_long fin = p.fdim[fi_d];
   const ga_long fi = (bx * RD_CX + tx) * RD_CV;   /* first of the lane's outputs */
   const bool live = fi < fin;
+  /* how many of the lane's RD_CV outputs exist (RD_CLOOSE: the inner free
+   * dim need not be a multiple of RD_CV; else all of them do) */
+#if RD_CLOOSE
+  const int nv = fin - fi >= RD_CV ? RD_CV : (int)(fin - fi);
+#else
+  const int nv = RD_CV;
+#endif
 
   /* offsets of this lane's first output */
   ga_long so[RD_NSRC], d0o = 0, d1o = 0;
@@ -1669,7 +1680,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
 #pragma unroll
-      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
 #pragma unroll
@@ -1685,7 +1696,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       rd_cvec x[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
-        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
         if (j0 + RD_CY * q < r1) {
@@ -1726,7 +1737,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     for (; j0 + RD_CY * (RD_U - 1) < r1; j0 += RD_CY * RD_U) {
       rd_cvec x[RD_U];
 #pragma unroll
-      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+      for (int q = 0; q < RD_U; q++) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
 #pragma unroll
       for (int q = 0; q < RD_U; q++) { RD_COL_BYTES_SEEN(x[q]) }
     }
@@ -1734,7 +1745,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       rd_cvec x[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
-        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+        if (j0 + RD_CY * q < r1) rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
         if (j0 + RD_CY * q < r1) { RD_COL_BYTES_SEEN(x[q]) }
@@ -1755,7 +1766,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       ga_long idx[RD_U];
 #pragma unroll
       for (int q = 0; q < RD_U; q++) {
-        rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+        rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
         idx[q] = RD_ARG ? rd_col_index(p, j0 + RD_CY * q) : 0;
       }
 #pragma unroll
@@ -1771,7 +1782,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
 #pragma unroll
       for (int q = 0; q < RD_U; q++)
         if (j0 + RD_CY * q < r1) {
-          rd_col_fetch(p, srow, j0 + RD_CY * q, x[q]);
+          rd_col_fetch(p, srow, j0 + RD_CY * q, x[q], nv);
           idx[q] = RD_ARG ? rd_col_index(p, j0 + RD_CY * q) : 0;
         }
 #pragma unroll
@@ -1794,6 +1805,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
   if (ty == 0 && live) {
 #pragma unroll
     for (int c = 0; c < RD_CV; c++) {
+      if (RD_CLOOSE && c >= nv) break;
       rd_acc a = acc[c];
 #pragma unroll
       for (int y = 1; y < RD_CY; y++) a = rd_combine(a, lds[y][c][tx]);
@@ -1846,7 +1858,8 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
         for (int j = 0; j < RD_FIN_BATCH; j++)
 #pragma unroll
           for (int c = 0; c < RD_CV; c++)
-            t[j][c] = rd_fetch_partial(part_v, part_i, (s + j * RD_CY) * p.nrows + at + c);
+            t[j][c] = (RD_CLOOSE && c >= nv) ? rd_neutral()
+                                              : rd_fetch_partial(part_v, part_i, (s + j * RD_CY) * p.nrows + at + c);
 #pragma unroll
         for (int j = 0; j < RD_FIN_BATCH; j++)
 #pragma unroll
@@ -1856,7 +1869,8 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
       for (; s < p.nsplit; s += RD_CY)
 #pragma unroll
         for (int c = 0; c < RD_CV; c++)
-          acc[c] = rd_combine(acc[c], rd_fetch_partial(part_v, part_i, s * p.nrows + at + c));
+          if (!RD_CLOOSE || c < nv)
+            acc[c] = rd_combine(acc[c], rd_fetch_partial(part_v, part_i, s * p.nrows + at + c));
     }
 #if RD_CY > 1
 #pragma unroll
@@ -1866,6 +1880,7 @@ redux_col(RD_SRC_PARAMS, char *d0, const ga_size d0_off, char *d1, const ga_size
     if (ty == 0 && live) {
 #pragma unroll
       for (int c = 0; c < RD_CV; c++) {
+        if (RD_CLOOSE && c >= nv) break;
         rd_acc a = acc[c];
 #pragma unroll
         for (int y = 1; y < RD_CY; y++) a = rd_combine(a, lds[y][c][tx]);

@@ -1070,6 +1070,44 @@ def test_split_reductions_finish_in_one_launch(ctx, knobs):
     assert np.asarray(v) == np.nanmax(x) and int(np.asarray(i)) == int(np.nanargmax(x))
 
 
+@pytest.mark.parametrize("loose", [1, 0])
+@pytest.mark.parametrize("dtype", ["float32", "int32", "uint32"])
+def test_column_reductions_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
+    """Reductions over leading or middle axes whose kept rows start at any
+    element and have any length (REDUX_COL_LOOSE: a lane still takes four
+    adjacent outputs, with loads that assume four-byte boundaries only; the
+    lane at the end of a row takes what exists of its four one by one).
+    Kept rows of 4 to 1001 elements inside wider buffers, every phase of the
+    first element, one and several pieces of the reduced range (with the
+    finish in the same launch and in a second one), folded rows switched off
+    so that dense arrays come here too; results against NumPy, exact."""
+    knobs(REDUX_COL_LOOSE=loose, REDUX_FOLD=0, REDUX_PCOLS=0)
+    rng = np.random.default_rng(870 + loose)
+    draw = lambda shape: rng.integers(0 if dtype == "uint32" else -20, 21, size=shape).astype(dtype)
+    ops = [("sum", lambda g, ax: R.sum(g, axis=ax),
+            lambda v, ax: v.sum(axis=ax, dtype=np.float64 if dtype == "float32" else np.int64))]
+    if dtype != "float32":
+        ops += [("max", lambda g, ax: R.max(g, axis=ax), lambda v, ax: v.max(axis=ax)),
+                ("min", lambda g, ax: R.min(g, axis=ax), lambda v, ax: v.min(axis=ax))]
+    if dtype == "uint32":
+        ops += [("xor", lambda g, ax: R._reduce_named(g, "xor", g.dtype, axis=ax),
+                 lambda v, ax: np.bitwise_xor.reduce(v, axis=ax))]
+    for rows, n, lead, pad in ((33, 4, 1, 0), (700, 5, 0, 0), (70, 7, 3, 2), (1500, 131, 2, 1), (64, 1001, 0, 0),
+                               (5000, 66, 1, 1), (9, 1001, 3, 0), (40000, 9, 0, 2), (2100, 259, 1, 0)):
+        root = draw((rows, lead + n + pad))
+        view = root[:, lead:lead + n]
+        g, _ = to_gpu_view(view, ctx)
+        for name, call, want in ops:
+            assert np.array_equal(np.asarray(call(g, 0)), want(view, 0)), (name, rows, n, lead, pad)
+    # a middle axis, and the two outer axes of three
+    root = draw((6, 300, 70 + 3))
+    view = root[:, :, 2:72 - 1]
+    g, _ = to_gpu_view(view, ctx)
+    for name, call, want in ops:
+        assert np.array_equal(np.asarray(call(g, 1)), want(view, 1)), name
+    assert np.array_equal(np.asarray(R.sum(g, axis=(0, 1))), ops[0][2](view, (0, 1)))
+
+
 @pytest.mark.parametrize("rows,cols", [(300, 70001), (130, 150000), (520, 66000), (41, 300000)])
 def test_rows_cut_to_even_out_the_compute_units(ctx, knobs, rows, cols):
     """A few hundred long rows, one group each, would leave some compute units
