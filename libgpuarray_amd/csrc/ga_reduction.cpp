@@ -2019,21 +2019,31 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
       (kind == K_SUM || kind == K_PROD || kind == K_AND || kind == K_OR || kind == K_XOR ||
        kind == K_ALL || kind == K_ANY || ((kind == K_MIN || kind == K_MAX) && is_int_type(stc)));
   if (!regroupable) return GA_NO_ERROR;
-  // the reduced axes are exactly the leading ones
+  // the reduced axes are one run of adjacent ones, [a0, a0 + reduxLen), and
+  // dims are kept behind it: O slabs (the dims in front of the run) of R rows
+  // of F elements each
+  unsigned a0 = s0->nd;
+  for (unsigned i = 0; i < reduxLen; i++) {
+    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= s0->nd) return GA_NO_ERROR;
+    if ((unsigned)reduxList[i] < a0) a0 = (unsigned)reduxList[i];
+  }
+  if (a0 + reduxLen >= s0->nd) return GA_NO_ERROR;
   std::vector<char> seen(reduxLen, 0);
   for (unsigned i = 0; i < reduxLen; i++) {
-    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= reduxLen || seen[reduxList[i]]) return GA_NO_ERROR;
-    seen[reduxList[i]] = 1;
+    const unsigned at = (unsigned)reduxList[i] - a0;
+    if (at >= reduxLen || seen[at]) return GA_NO_ERROR;
+    seen[at] = 1;
   }
-  size_t R = 1, F = 1;
-  for (unsigned j = 0; j < s0->nd; j++) (j < reduxLen ? R : F) *= s0->dimensions[j];
+  size_t O = 1, R = 1, F = 1;
+  for (unsigned j = 0; j < s0->nd; j++) (j < a0 ? O : j < a0 + reduxLen ? R : F) *= s0->dimensions[j];
+  if (a0 > 0 && TUNE(tn, REDUX_FOLD, 1) == 2) return GA_NO_ERROR;   // (2: leading axes only)
   const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
-  if (R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20) || F == 0) return GA_NO_ERROR;
+  if (O * R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20) || F == 0 || O == 0) return GA_NO_ERROR;
   if (rowb % 16 == 0 && rowb >= 256) return GA_NO_ERROR;
   // d0 must have the kept dims' shape (the launch below checks the rest)
   if (d0->nd != s0->nd - reduxLen) return GA_NO_ERROR;
   for (unsigned j = 0; j < d0->nd; j++)
-    if (d0->dimensions[j] != s0->dimensions[reduxLen + j]) return GA_NO_ERROR;
+    if (d0->dimensions[j] != s0->dimensions[j < a0 ? j : reduxLen + j]) return GA_NO_ERROR;
   // m: rows per folded row
   size_t g = rowb, h = 16;
   while (h) { size_t t = g % h; g = h; h = t; }      // g = gcd(rowb, 16)
@@ -2086,7 +2096,7 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   // buffer (which is never handed to anybody else, also not after it has been
   // outgrown: a graph that recorded these launches may run them again); the
   // two calls below put their own partials behind them.
-  const size_t tmp_len = m * F;
+  const size_t tmp_len = O * m * F;
   const size_t skip = (tmp_len * gpuarray_get_elsize(tmp_tc) + 255) & ~(size_t)255;
   gpudata *scr = nullptr;
   if (noalloc) {
@@ -2109,30 +2119,41 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   const ssize_t tmp_stride = (ssize_t)gpuarray_get_elsize(tmp_tc);
   int err = GpuArray_fromdata(&tmp, scr, 0, tmp_tc, 1, &tmp_len, &tmp_stride, 1);
   if (err != GA_NO_ERROR) return err;
-  {
+  if (O == 1) {
     // first call: (R / m, m F) over axis 0 into tmp
     const size_t dims1[2] = {R / m, m * F};
     const int64_t str1[2] = {(int64_t)(m * rowb), (int64_t)es};
     const src_view src = {s0, str1};
     const int axis0 = 0;
     err = reduce_launch(gr, &tmp, nullptr, 2, dims1, &src, nullptr, 0, 1, &axis0, noalloc, skip);
+  } else {
+    // the same per slab: (O, R / m, m F) over axis 1 into tmp as (O, m F)
+    GpuArray_clear(&tmp);
+    const size_t tdims[2] = {O, m * F};
+    const ssize_t tstr[2] = {(ssize_t)(m * F) * tmp_stride, tmp_stride};
+    err = GpuArray_fromdata(&tmp, scr, 0, tmp_tc, 2, tdims, tstr, 1);
+    if (err != GA_NO_ERROR) return err;
+    const size_t dims1[3] = {O, R / m, m * F};
+    const int64_t str1[3] = {(int64_t)(R * rowb), (int64_t)(m * rowb), (int64_t)es};
+    const src_view src = {s0, str1};
+    const int axis1 = 1;
+    err = reduce_launch(gr, &tmp, nullptr, 3, dims1, &src, nullptr, 0, 1, &axis1, noalloc, skip);
   }
   if (err == GA_NO_ERROR) {
-    // second call: tmp as (m, kept dims...) over axis 0 into d0
+    // second call: tmp as (slab dims..., m, dims kept behind the run...) over
+    // the axis of the m copies into d0
     std::vector<size_t> dims2(1 + d0->nd);
     std::vector<int64_t> str2(1 + d0->nd);
     const size_t tes = gpuarray_get_elsize(tmp_tc);
-    dims2[0] = m;
     size_t run = tes;
-    for (unsigned j = d0->nd; j-- > 0;) {
-      dims2[1 + j] = d0->dimensions[j];
-      str2[1 + j] = (int64_t)run;
-      run *= d0->dimensions[j];
+    for (unsigned j = d0->nd + 1; j-- > 0;) {
+      dims2[j] = j < a0 ? d0->dimensions[j] : j == a0 ? m : d0->dimensions[j - 1];
+      str2[j] = (int64_t)run;
+      run *= dims2[j];
     }
-    str2[0] = (int64_t)run;
     const src_view src = {&tmp, str2.data()};
-    const int axis0 = 0;
-    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), &src, nullptr, 0, 1, &axis0,
+    const int axis = (int)a0;
+    err = reduce_launch(gr->fold_op, d0, nullptr, 1 + d0->nd, dims2.data(), &src, nullptr, 0, 1, &axis,
                         noalloc, skip);
   }
   GpuArray_clear(&tmp);

@@ -1279,6 +1279,41 @@ def test_stepped_eight_byte_rows_are_planned(ctx):
     assert np.asarray(R.sum(g, axis=1)).shape == (64,)
 
 
+@pytest.mark.parametrize("fold", [1, 2, 0])
+def test_a_run_of_middle_axes_over_short_kept_rows_is_folded_per_slab(ctx, knobs, fold):
+    """The same folding under leading dims that are kept: (O, R, F) over the
+    middle run of axes is O slabs, each folded like a dense array (REDUX_FOLD:
+    1 slabs too, 2 leading axes only, 0 never).  One and two kept dims in
+    front, one and two reduced axes (in either order), kept rows of 1 to 250
+    elements, row counts with and without a divisor, a strided destination;
+    integer results exact, against NumPy."""
+    knobs(REDUX_FOLD=fold)
+    rng = np.random.default_rng(72)
+    cases = (((64, 1000, 250), (1,), "float32"), ((8, 65536, 33), (1,), "int32"), ((16, 64, 64, 62), (1, 2), "int32"),
+             ((16, 64, 64, 62), (2, 1), "float32"), ((3, 5, 4096, 30), (2,), "uint8"), ((40, 4099, 10), (1,), "int32"),
+             ((128, 16384, 1), (1,), "float32"), ((6, 262144, 3), (1,), "float16"))
+    for shape, axes, dt in cases:
+        host = rng.integers(-3 if np.dtype(dt).kind in "if" else 0, 4, size=shape).astype(dt)
+        g = gpuarray.array(host, context=ctx)
+        odt = "int64" if np.dtype(dt).kind in "iu" else "float32"
+        got = np.asarray(R.sum(g, axis=axes, dtype=odt))
+        assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64).astype(odt)), (shape, axes, dt)
+        got = np.asarray(R._reduce_named(g, "any", np.dtype("bool"), axis=axes))
+        assert np.array_equal(got, host.any(axis=axes)), (shape, axes, dt)
+        if np.dtype(dt).kind in "iu":
+            assert np.array_equal(np.asarray(R.max(g, axis=axes)), host.max(axis=axes)), (shape, axes, dt)
+        else:
+            val, idx = R.maxandargmax(g, axis=axes[:1])      # keeps the order of the scan: not folded
+            assert np.array_equal(np.asarray(val), host.max(axis=axes[0]))
+            assert np.array_equal(np.asarray(idx), host.argmax(axis=axes[0]))
+    host = rng.integers(-3, 4, size=(64, 1000, 250)).astype(np.float32)
+    g = gpuarray.array(host, context=ctx)
+    wide = gpuarray.zeros((64, 250, 3), "float32", context=ctx)
+    ga.GpuReduction(ctx, "sum", "float32")(g, [1], d0=wide[:, :, 1])
+    assert np.array_equal(np.asarray(wide)[:, :, 1], host.sum(axis=1))
+    assert not np.asarray(wide)[:, :, [0, 2]].any()
+
+
 @pytest.mark.parametrize("route", ["one launch", "folded", "neither"])
 def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, route):
     """Reducing the leading dims of a dense array whose kept rows are short or
