@@ -50,21 +50,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_configs.md (earlier rocprofv3 --pmc runs, matched by kernel text hash)"
 MEASURED_TRAFFIC = {
     # name: (kernel text hashes of one call joined by "+", HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201253635),
-    "C2_transposed_broadcast_4096": ("d188ff564c901e86", 134376140),
-    "X_transpose_8192x8192": ("a8d106ba259ef190", 536629163),
-    "C3a_sum_axis1_8192x8192": ("7b1e5b3d393b65cf", 268766354),
-    "C4_maxandargmax_65536x1000": ("2b61e61df66fc82d", 263731413),
-    "C5_fp16_sum_axes02": ("4296e62da8ed8910+8be870fa9892586c", 269706664),
-    "C5_int32_sum_axis1": ("0d1aff898d530c09", 538005643),
-    "C5_uint8_all_axis2": ("2195f3f51c85c279", 134384275),
-    "C5_uint8_any_axis2": ("867a1aaf40f33d29", 134384235),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538658597),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538656615),
-    "F4_dot_2x2^27_fused": ("f13108789ad1ada9", 1073848072),
-    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+b3b28b94a7047bb8", 2146736177),
-    "elem_2^28": ("712fba8f0b8a6108", 3219556758),
-    "sum_2^28": ("b3b28b94a7047bb8", 1073797880),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201255189),
+    "C2_transposed_broadcast_4096": ("d188ff564c901e86", 134381523),
+    "X_transpose_8192x8192": ("a8d106ba259ef190", 536641947),
+    "C3a_sum_axis1_8192x8192": ("436023b8d83373f6", 268765949),
+    "C4_maxandargmax_65536x1000": ("20cdd8d3a74eb928", 263831093),
+    "C5_fp16_sum_axes02": ("7b4594a69af14d77+2a6e9b910df1348b", 269706608),
+    "C5_int32_sum_axis1": ("ca6ab9f45a27cdba", 538005699),
+    "C5_uint8_all_axis2": ("d8b08ecb35fcbf32", 134384191),
+    "C5_uint8_any_axis2": ("082f1e86bbc7e9e2", 134384171),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538661074),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538660526),
+    "F4_dot_2x2^27_fused": ("ab6309c02f4df4f6", 1073848082),
+    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+437dabd09ccf439b", 2146732451),
+    "elem_2^28": ("712fba8f0b8a6108", 3219551715),
+    "sum_2^28": ("437dabd09ccf439b", 1073797844),
 }
 
 

@@ -1580,7 +1580,9 @@ class strided_call {
       for (unsigned j = 0; j < nd; j++) pi.ps[k][3 - nd + j] = strs[k][j];
     }
     if (pi.pmask == 0) return false;
-    if (vec4 && mode != 2 && !(inner_constant && dense_read)) return false;
+    // (four per lane on any layout, `loose`, does not count here: rows of a few
+    // elements are all cut quads - (2^24, 3) + (1, 3) 154 us that way, 60 us flat)
+    if (vec4 && !loose && mode != 2 && !(inner_constant && dense_read)) return false;
     pi.pnd = nd;
     auto magic = [](unsigned d, uint64_t &m, unsigned &k) {
       unsigned c = 0;
@@ -1709,8 +1711,23 @@ class strided_call {
     // inside pitches of 8320 137.9 / 122.5 us (73 -> 82 % of peak), rows of
     // 8192 that start one element in 144.0 / 121.9, pitches of 8319 floats
     // 141.8 / 125.6, 65536 rows of 1001 in pitches of 1003 141.9 / 122.2.
+    // Only for arrays that cannot all sit in the 256 MB of the last-level cache:
+    // on data that does, the kernel with one element per lane (fewer
+    // instructions, no cut quads) is the faster one.  Side of a square
+    // float array, transposed copy and o = a + b on row views, one element per
+    // lane against this, the same buffers every call / rotating through more
+    // buffers than the cache holds: 2047 +53 % / +9 % and +5 % / -2 %, 4095
+    // +39 % / -15 % and +22 % / -16 %, 8190 -29 % / -29 % and -12 % / -11 %.
     loose = false;
+    size_t footprint = 0;
+    for (unsigned k = 0; k < na; k++) {
+      bool once = true;
+      for (unsigned j = 0; j < nd && once; j++)
+        if (dims[j] > 1 && strs[k][j] == 0) once = false;
+      if (once) footprint += n * elsz[k];
+    }
     if (!vec4 && !((tmask >> outk) & 1u) && TUNE(tn, ELEMWISE_VEC4, 1) != 0 &&
+        footprint >= (size_t)TUNE(tn, ELEMWISE_LOOSE_MIN_BYTES, 256u << 20) &&
         TUNE(tn, ELEMWISE_LOOSE, 1) != 0 && na <= 31 && strs[outk][nd - 1] == 4) {
       bool ok = true;
       unsigned um = 0, zm = 0;
@@ -1814,7 +1831,12 @@ class strided_call {
         // 32 bytes into a block 135.8 / 92.6 us, a pitch of 8328 floats (the
         // rows walk through the four phases) 114.1 / 95.5, both pitches 8200
         // floats 114.5 / 102.4; (5000, 3000) -> (3000, 5000) 27.2 / 25.9.
-        if (outk >= 0 && !((tmask >> outk) & 1u) && elsz[outk] == 4 && TUNE(tn, ELEMWISE_SKEW, 1) != 0) {
+        // (large arrays only, like `loose`: 2047 x 2047 floats ran 12 to 19 % slower this way)
+        size_t moved = 0;
+        for (unsigned k = 0; k < na; k++)
+          if (strs[k][nd - 1] != 0 && strs[k][nd - 2] != 0) moved += n * elsz[k];
+        if (outk >= 0 && !((tmask >> outk) & 1u) && elsz[outk] == 4 && TUNE(tn, ELEMWISE_SKEW, 1) != 0 &&
+            moved >= (size_t)TUNE(tn, ELEMWISE_LOOSE_MIN_BYTES, 256u << 20)) {
           bool wide = false;
           for (unsigned k = 0; k < na; k++) wide = wide || elsz[k] > 4;
           const GpuArray *ov = nullptr;

@@ -1213,7 +1213,7 @@ class reduction_call {
             return l;
           };
           unsigned l1 = lanes_for((int64_t)V * (minmax ? 2 : 1));
-          if (minmax && elsz[0] >= 4 && l1 < 8) {
+          if (minmax && elsz[0] >= 4 && l1 < 8 && nrows >= 65536) {   // (a thousand rows of 17: 4.6 us with 4 lanes, 7.3 with 8)
             const unsigned single = lanes_for((int64_t)V);
             l1 = single < 8 ? single : 8;
           }
@@ -1396,7 +1396,12 @@ class reduction_call {
       // maximum over axis 0 of (8192, 8191) 57.0 / 63.8.
       cloose = false;
       const bool carries_position = info.has_d1 || (minmax && is_float_type(acc_typecode(gr, d0_tc)));
-      if (cv < 4 && elsz_max == 4 && !carries_position && TUNE(tn, REDUX_COL_LOOSE, 1) != 0 && fin >= 4) {
+      // (nor for small inputs, which want lanes, not wide loads: the (128, 1001)
+      // partial rows of a folded (65536, 1001) took 2.5 us longer this way, sums
+      // over axis 0 of 16 MB, (4097, 1023) and (513, 8191), 13 and 23 % longer;
+      // 36 MB, (3000, 3001), 20 % shorter)
+      if (cv < 4 && elsz_max == 4 && !carries_position && TUNE(tn, REDUX_COL_LOOSE, 1) != 0 && fin >= 4 &&
+          (double)nrows * (double)rtotal * 4.0 >= (double)TUNE(tn, REDUX_COL_LOOSE_MIN_BYTES, 32u << 20)) {
         bool ok = true;
         for (unsigned q = 0; ok && q < K; q++) {
           ok = elsz[q] == 4 && fsstr[q * RD_MAXD + p.nf - 1] == 4 && GpuArray_ISALIGNED(srcs[q].a);
@@ -2037,6 +2042,10 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   size_t O = 1, R = 1, F = 1;
   for (unsigned j = 0; j < s0->nd; j++) (j < a0 ? O : j < a0 + reduxLen ? R : F) *= s0->dimensions[j];
   if (a0 > 0 && TUNE(tn, REDUX_FOLD, 1) == 2) return GA_NO_ERROR;   // (2: leading axes only)
+  // (slabs from 32 MiB on: (16, 16384, 42) floats, 42 MB, 18.6 -> 15.0 us, (8, 65536, 33) 25.7 -> 19.1;
+  // below, (256, 1024, 30), 30 MB, 14.0 -> 14.3, (8, 8192, 33), 8 MB, 9.4 -> 12.0)
+  if (a0 > 0 && O * R * F * gpuarray_get_elsize(stc) < TUNE(tn, REDUX_FOLD_SLAB_MIN_BYTES, 32u << 20))
+    return GA_NO_ERROR;
   const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
   if (O * R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20) || F == 0 || O == 0) return GA_NO_ERROR;
   if (rowb % 16 == 0 && rowb >= 256) return GA_NO_ERROR;

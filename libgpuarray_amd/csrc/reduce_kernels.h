@@ -726,31 +726,22 @@ static __device__ inline rd_acc rd_unit_combine(const rd_unit &x, ga_long e0, ga
   return r;
 #else
   rd_acc t[RD_U];
-#if RD_TAIL
-  /* A lane whose loads of this unit all lie inside the row (every lane of
-   * every unit but a row's first and last) combines them as they are; the
-   * others put every element under a select.  Both sides use every loaded
-   * register (see above), and both combine in the same order. */
-  const bool inside = e0 >= sh && e0 + (ga_long)(RD_U - 1) * LN * RD_VEC + RD_VEC <= rin;
-#endif
 #pragma unroll
   for (int j = 0; j < RD_U; j++) {
     const ga_long e = e0 + (ga_long)j * LN * RD_VEC;
     t[j] = rd_neutral();
 #if RD_TAIL
-    if (inside) {
+    /* every element under a select, no branch (see above; a branch that sends
+     * the lanes whose loads lie inside the row past the selects saved half a
+     * microsecond of 46 on rows of 50257 floats and cost a few hundred rows of
+     * a hundred floats as much of 4) */
+    const ga_long dl = sh - e, dh = rin - e;
+    const int lo = dl > RD_VEC ? RD_VEC : (int)dl;
+    const int hi = dh < 0 ? 0 : (dh > RD_VEC ? RD_VEC : (int)dh);
 #pragma unroll
-      for (int v = 0; v < RD_VEC; v++)
-        t[j] = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v - sh) * rml));
-    } else {
-      const ga_long dl = sh - e, dh = rin - e;
-      const int lo = dl > RD_VEC ? RD_VEC : (int)dl;
-      const int hi = dh < 0 ? 0 : (dh > RD_VEC ? RD_VEC : (int)dh);
-#pragma unroll
-      for (int v = 0; v < RD_VEC; v++) {
-        const rd_acc c = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v - sh) * rml));
-        t[j] = (v >= lo && v < hi) ? c : t[j];
-      }
+    for (int v = 0; v < RD_VEC; v++) {
+      const rd_acc c = rd_combine(t[j], rd_elem(RD_UNIT_VAL(x, j, v), ib + (e + v - sh) * rml));
+      t[j] = (v >= lo && v < hi) ? c : t[j];
     }
 #else
     if (e < rin) {

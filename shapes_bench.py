@@ -93,6 +93,11 @@ def elemwise_cases():
         ("transpose (1, 0, 2) of (1024, 64, 1024)", "o = a", [("a", f, (1024, 64, 1024), T(1, 0, 2))], (64, 1024, 1024), f),
         ("transpose (2, 1, 0) of (256, 512, 512)", "o = a", [("a", f, (256, 512, 512), T(2, 1, 0))], (512, 512, 256), f),
         ("NCHW -> NHWC, (64, 256, 64, 64)", "o = a", [("a", f, (64, 256, 64, 64), T(0, 2, 3, 1))], (64, 64, 64, 256), f),
+        ("a.T, 8190 x 8190 (extents and pitches off the multiples of four)", "o = a", [("a", f, (8190, 8190), T(1, 0))], (8190, 8190), f),
+        ("a + b, 8192 rows of 8191 floats inside pitches of 8320", "o = a + b",
+         [("a", f, (8192, 8320), lambda b: b[:, :8191]), ("b", f, (8192, 8320), lambda b: b[:, :8191])], (8192, 8191), f),
+        ("a[:, 1:] + b[:, :-1], 8192 x 8193 (rows that start one element in)", "o = a + b",
+         [("a", f, (8192, 8193), lambda b: b[:, 1:]), ("b", f, (8192, 8193), lambda b: b[:, :-1])], (8192, 8192), f),
         ("copy, 2^28 floats (1 GiB read, 1 GiB written: the yardstick of the traffic counters)", "o = a",
          [("a", f, (1 << 28,), None)], (1 << 28,), f),
     ]
@@ -137,6 +142,9 @@ def reduction_cases():
         ("sum", f, (128, 128, 4096), (1,), None, None, "middle axis, 16 KiB apart"),
         ("sum", f, (8192, 16384), (0, 1), None, lambda a: a[:, ::2], "stride-2 view (useful bytes)"),
         ("sum", f, (8192, 8192), (1,), None, lambda a: a.T, "rows of a transposed matrix"),
+        ("sum", f, (8192, 8192), (0,), None, lambda a: a[:, 1:], "columns of a view that starts one element in"),
+        ("sum", f, (64, 1000, 1000), (1,), None, None, "middle axis, rows of 4000 bytes"),
+        ("sum", f, (64, 4096, 250), (1,), None, None, "middle axis over short kept rows: folded per slab"),
     ]
 
 

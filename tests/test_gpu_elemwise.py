@@ -569,7 +569,7 @@ def test_tile_windows_follow_result_rows_off_the_64_byte_blocks(ctx, knobs, tile
     windows need, a row operand (its window moves with the row), several
     planes; with the rectangular tiles as well.  The whole buffer of the result
     is compared, so a store outside the view shows."""
-    knobs(ELEMWISE_TTILE=tile, ELEMWISE_SKEW=skew)
+    knobs(ELEMWISE_TTILE=tile, ELEMWISE_SKEW=skew, ELEMWISE_LOOSE_MIN_BYTES=1)
     rng = np.random.default_rng(700 + tile)
     k = ga.GpuElemwise(ctx, "o = a * r + c", [arg("a", "float32", read=True), arg("r", "float32", read=True),
                                               arg("c", "float32", read=True), arg("o", "float32", write=True)])
@@ -607,7 +607,7 @@ def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dty
     element per lane).  Odd extents around the tile sizes, every phase of the
     operand's and the result's first element, a row and a column operand, a
     second transposed operand, planes; the result's whole buffer is compared."""
-    knobs(ELEMWISE_LOOSE=loose)
+    knobs(ELEMWISE_LOOSE=loose, ELEMWISE_LOOSE_MIN_BYTES=1)
     rng = np.random.default_rng(810 + loose)
     k = ga.GpuElemwise(ctx, "o = a * r + c", [arg("a", dtype, read=True), arg("r", dtype, read=True),
                                               arg("c", dtype, read=True), arg("o", dtype, write=True)])
@@ -652,7 +652,7 @@ def test_row_views_of_four_byte_elements_on_any_layout(ctx, knobs, loose):
     lane).  Rows of 1 to 9 elements in every phase (a cut quad can hold the
     whole row), longer odd rows, operands in other phases than the result,
     a stepped and a constant operand; the result's whole buffer is compared."""
-    knobs(ELEMWISE_LOOSE=loose)
+    knobs(ELEMWISE_LOOSE=loose, ELEMWISE_LOOSE_MIN_BYTES=1)
     rng = np.random.default_rng(830 + loose)
     k = ga.GpuElemwise(ctx, "o = a * s + c", [arg("a", "float32", read=True), arg("s", "float32", read=True),
                                               arg("c", "float32", read=True), arg("o", "float32", write=True)])

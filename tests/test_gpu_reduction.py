@@ -1081,7 +1081,7 @@ def test_column_reductions_of_four_byte_elements_on_any_layout(ctx, knobs, dtype
     first element, one and several pieces of the reduced range (with the
     finish in the same launch and in a second one), folded rows switched off
     so that dense arrays come here too; results against NumPy, exact."""
-    knobs(REDUX_COL_LOOSE=loose, REDUX_FOLD=0, REDUX_PCOLS=0)
+    knobs(REDUX_COL_LOOSE=loose, REDUX_COL_LOOSE_MIN_BYTES=1, REDUX_FOLD=0, REDUX_PCOLS=0)
     rng = np.random.default_rng(870 + loose)
     draw = lambda shape: rng.integers(0 if dtype == "uint32" else -20, 21, size=shape).astype(dtype)
     ops = [("sum", lambda g, ax: R.sum(g, axis=ax),
@@ -1287,7 +1287,7 @@ def test_a_run_of_middle_axes_over_short_kept_rows_is_folded_per_slab(ctx, knobs
     front, one and two reduced axes (in either order), kept rows of 1 to 250
     elements, row counts with and without a divisor, a strided destination;
     integer results exact, against NumPy."""
-    knobs(REDUX_FOLD=fold)
+    knobs(REDUX_FOLD=fold, REDUX_FOLD_SLAB_MIN_BYTES=1)
     rng = np.random.default_rng(72)
     cases = (((64, 1000, 250), (1,), "float32"), ((8, 65536, 33), (1,), "int32"), ((16, 64, 64, 62), (1, 2), "int32"),
              ((16, 64, 64, 62), (2, 1), "float32"), ((3, 5, 4096, 30), (2,), "uint8"), ((40, 4099, 10), (1,), "int32"),
