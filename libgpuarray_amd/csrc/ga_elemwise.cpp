@@ -1752,6 +1752,24 @@ class strided_call {
         bool once = true;
         for (unsigned j = 0; j < nd && once; j++)
           if (dims[j] > 1 && strs[k][j] == 0) once = false;
+        // A transposed operand whose rows do not start on 128-byte lines: a
+        // tile's 512-byte pieces of them share their first and last line with
+        // the neighbouring tiles', and a streamed line is fetched again by the
+        // neighbour (out = in.T of 8190 x 8190 floats read 1.38 times the array).
+        // Such an operand stays cacheable: (5000, 3000) -> (3000, 5000) 27.1 ->
+        // 21.2 us (55 -> 71 % of peak), 8190 x 8190 110.8 -> 97.7, (50000, 1000) ->
+        // (1000, 50000) 80.8 -> 76.4; on whole lines streaming is ahead (a.T + b
+        // of 8192 x 8192 121.6 us streamed, 128.0 cacheable).
+        if (once && ((tmask >> k) & 1u) && TUNE(tn, ELEMWISE_NT_LINES, 1) != 0) {
+          unsigned l2 = 0;
+          const GpuArray *v = nullptr;
+          for (size_t i = 0; i < ge->args.size(); i++)
+            if (ge->args[i].is_array() && l2++ == k) { v = (const GpuArray *)args[i]; break; }
+          bool lines = ((uintptr_t)v->data->devptr + v->offset) % 128 == 0;
+          for (unsigned j = 0; j < nd && lines; j++)
+            if (j != nd - 2 && dims[j] > 1 && strs[k][j] % 128 != 0) lines = false;
+          if (!lines) once = false;
+        }
         if (once) ntmask |= 1u << k;
       }
       ntmask &= (unsigned)TUNE(tn, ELEMWISE_NT_MASK, 0xffffffffu);

@@ -1487,6 +1487,22 @@ class reduction_call {
     unsigned opts = TUNE(tn, REDUX_NT, 1) ? 1u : 0u;
     if (use_row && p.nr == 1 && p.nsplit > 1 && TUNE(tn, REDUX_INTERLEAVE, 1)) opts |= 2u;
     if (use_row && tail) opts |= 4u;   // bit 2: element-aligned vector loads with a ragged end
+    // The column kernel's loads that assume four-byte boundaries only (cloose)
+    // share lines with the neighbouring groups' when rows do not start on
+    // 128-byte lines, and a streamed line is fetched again by the neighbour
+    // (sum over axis 0 of (8192, 8191) floats read 1.11 times the array): such
+    // loads stay cacheable, (8192, 8192)[:, 1:] 51.6 -> 48.7 us.  Aligned loads
+    // keep the hint on any pitch: (65536, 1000) over axis 0 72.8 % of peak
+    // streamed, 66.9 cacheable, (8, 10000, 1000) over the middle axis 79.5 / 72.2.
+    if (!use_row && cloose && CV > 1 && (opts & 1u) && TUNE(tn, REDUX_NT_LINES, 1) != 0) {
+      bool lines = true;
+      for (unsigned q = 0; q < K && lines; q++) {
+        lines = ((uintptr_t)srcs[q].a->data->devptr + srcs[q].a->offset) % 128 == 0;
+        for (int i = 0; lines && i + 1 < p.nf; i++) lines = fsstr[q * RD_MAXD + i] % 128 == 0;
+        for (int i = 0; lines && i < p.nr; i++) lines = rsstr[q * RD_MAXD + i] % 128 == 0;
+      }
+      if (!lines) opts &= ~1u;
+    }
     variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
                        use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
                        (use_row && !wrows) ? LO : 1};
