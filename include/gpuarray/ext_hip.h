@@ -94,7 +94,8 @@ typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *exp
                                            unsigned int tmask);
 /* vec: elements used per load in bits 0..7, element step of the inner
  * reduced dim (1, 2 or 4; 0 means 1) in bits 8..15, adjacent outputs per lane
- * of the column kernel in bits 16 and up (0 means 1).
+ * of the column kernel in bits 16..23 (0 means 1); bit 24: the column kernel
+ * numbers its groups so that neighbours along the inner kept dim run on one die.
  * lanes_per_output: 64 or 256 in bits 0..15; lanes per row of the short-row
  * kernel in bits 16 and up (0 means 64).
  * unroll: loads in flight per lane in bits 0..7; rows per batch of the

@@ -134,6 +134,11 @@ def main():
               gen_r(op, src, GA_LONG if (op == 0 and src == GA_INT) else src, GA_LONG, 256, 1 | (cv << 16),
                     4 | (1 << 31) | ((1 << 26) if op in (6, 8) else 0)))
         n += 1
+    for op, src, cv, loose in ((0, GA_FLOAT, 4, 1), (6, GA_INT, 4, 0), (0, GA_DOUBLE, 2, 0), (0, GA_HALF, 1, 0)):
+        check("column reduction with neighbouring groups on one die, op %d type %d, %d outputs per lane" % (op, src, cv),
+              gen_r(op, src, src, GA_LONG, 256, 1 | (cv << 16) | (1 << 24),
+                    4 | ((1 << 31) if loose else 0) | ((1 << 26) if op in (6, 8) else 0)))
+        n += 1
     for op, cv in ((13, 16), (12, 4), (13, 8)):
         check("column any / all over bytes, op %d, %d outputs per lane" % (op, cv),
               gen_r(op, GA_UBYTE, GA_BOOL, GA_LONG, 256, 1 | (cv << 16), 4))

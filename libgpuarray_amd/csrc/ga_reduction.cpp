@@ -285,6 +285,7 @@ int gen_variant_text(const GpuReduction *gr, const variant_spec &vs, std::string
   DEF("#define RD_SROWS %u\n", (vs.opts >> 3) & 1u);
   DEF("#define RD_PCOLS %u\n", (vs.opts >> 11) & 1u);
   DEF("#define RD_CLOOSE %u\n", (vs.opts >> 12) & 1u);
+  DEF("#define RD_XCD %u\n", (vs.opts >> 13) & 1u);
   {
     // redux_trows: a lane's run of whole rows in whole 16-byte chunks
     const unsigned te = vs.TE ? vs.TE : 1;
@@ -1475,6 +1476,7 @@ class reduction_call {
     const int64_t many = (int64_t)TUNE(tn, REDUX_SPLIT_MAJOR_MIN, 4096);
     p.split_major = (nsplit > 1 && nrows >= many) ? 1 : 0;
     groups = (size_t)(base_groups * nsplit);
+    p.units = (int64_t)(groups / 8 * 8);   // for the order that keeps neighbours on one die
     U = (unsigned)TUNE(tn, REDUX_COL_U, 4);
     if (U != 1 && U != 2 && U != 4 && U != 8) U = 4;
   }
@@ -1487,21 +1489,35 @@ class reduction_call {
     unsigned opts = TUNE(tn, REDUX_NT, 1) ? 1u : 0u;
     if (use_row && p.nr == 1 && p.nsplit > 1 && TUNE(tn, REDUX_INTERLEAVE, 1)) opts |= 2u;
     if (use_row && tail) opts |= 4u;   // bit 2: element-aligned vector loads with a ragged end
-    // The column kernel's loads that assume four-byte boundaries only (cloose)
-    // share lines with the neighbouring groups' when rows do not start on
-    // 128-byte lines, and a streamed line is fetched again by the neighbour
-    // (sum over axis 0 of (8192, 8191) floats read 1.11 times the array): such
-    // loads stay cacheable, (8192, 8192)[:, 1:] 51.6 -> 48.7 us.  Aligned loads
-    // keep the hint on any pitch: (65536, 1000) over axis 0 72.8 % of peak
-    // streamed, 66.9 cacheable, (8, 10000, 1000) over the middle axis 79.5 / 72.2.
-    if (!use_row && cloose && CV > 1 && (opts & 1u) && TUNE(tn, REDUX_NT_LINES, 1) != 0) {
+    // Column kernel on rows that do not start on 128-byte lines: the pieces of a
+    // row that neighbouring groups fetch share the lines they straddle.
+    //  - Groups that follow one another in launch order run on different dies,
+    //    each with its own cache, so such a line came from memory once per die:
+    //    sum over the middle axis of (64, 1000, 1000) floats read 1.38 times the
+    //    array.  bit 13: neighbours along the inner free dim follow one another
+    //    on ONE die (see the kernel).  Measured on MI355X, sums of floats, plain
+    //    order / this one: middle axis of (64, 1000, 1000) 52.5 -> 39.2 us (61 ->
+    //    82 % of peak), of (64, 1001, 1001) 56.1 -> 43.1 us, of (64, 1000, 1008)
+    //    66 -> 83 %, of (16, 2000, 2000) 69 -> 79 %, int32 maxima of the first
+    //    61 -> 82 %, axis 0 of (1000, 50257) 42.7 -> 38.6 us, of (8192, 8191)
+    //    54.2 -> 46.8 us.  On whole lines nothing is shared and the plain order
+    //    stays: (256, 512, 512) over the middle axis 84.5 % plain, 79.1 this way.
+    //  - A streamed line is fetched again by the neighbour, so the loads that
+    //    assume four-byte boundaries only (cloose) stay cacheable there:
+    //    (8192, 8192)[:, 1:] over axis 0 51.6 -> 48.7 us.  Aligned loads keep the
+    //    hint on any pitch: (65536, 1000) over axis 0 72.8 % of peak streamed,
+    //    66.9 cacheable, (8, 10000, 1000) over the middle axis 79.5 / 72.2.
+    if (!use_row) {
       bool lines = true;
       for (unsigned q = 0; q < K && lines; q++) {
         lines = ((uintptr_t)srcs[q].a->data->devptr + srcs[q].a->offset) % 128 == 0;
         for (int i = 0; lines && i + 1 < p.nf; i++) lines = fsstr[q * RD_MAXD + i] % 128 == 0;
         for (int i = 0; lines && i < p.nr; i++) lines = rsstr[q * RD_MAXD + i] % 128 == 0;
       }
-      if (!lines) opts &= ~1u;
+      const unsigned long xcd = TUNE(tn, REDUX_XCD, 1);
+      // (fewer than 16 groups: the order would be the plain one, or nearly)
+      if (xcd == 2 || (xcd == 1 && !lines && groups >= 16)) opts |= 8192u;
+      if (!lines && cloose && CV > 1 && TUNE(tn, REDUX_NT_LINES, 1) != 0) opts &= ~1u;
     }
     variant_spec vs = {d0_tc, d1_tc, use_row ? G : 256, use_row ? V : 1, U, opts, use_row ? ES : 1,
                        use_row ? vecmask : (1u << K) - 1, wrows ? RB : 1, wrows ? L : 64, use_row ? 1 : CV,
@@ -1797,9 +1813,11 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
     return nullptr;
   // bits 8.. of V carry the element step of strided loads (0 means 1), bits
   // 8.. of U the rows per batch of redux_wrows (0 means 1), bits 16.. of G its
-  // lanes per row (0 means 64), bits 16.. of V the outputs per lane of redux_col
+  // lanes per row (0 means 64), bits 16..23 of V the outputs per lane of
+  // redux_col, bit 24 of V its order of groups that keeps neighbours on one die
   const unsigned ES = ((V >> 8) & 0xffu) ? ((V >> 8) & 0xffu) : 1;
-  const unsigned cv_bits = V >> 16;
+  const unsigned cv_bits = (V >> 16) & 0xffu;
+  const unsigned xcd_bit = (V >> 24) & 1u;
   V &= 0xffu;
   std::string s;
   variant_spec vs = {d0_tc, d1_tc, G & 0xffffu, V, U & 0xffu,
@@ -1807,7 +1825,7 @@ GPUARRAY_PUBLIC char *ga_reduction_gen_source(int op, int src_tc, int d0_tc, int
                          (((U >> 25) & 1u) ? 8u : 0u) | (((U >> 26) & 1u) ? 64u : 0u) |
                          (((U >> 27) & 1u) ? 128u : 0u) | (((U >> 28) & 1u) ? 512u : 0u) |
                          (((U >> 29) & 1u) ? 1024u : 0u) | (((U >> 30) & 1u) ? 2048u : 0u) |
-                         (((U >> 31) & 1u) ? 4096u : 0u) | 48u | 256u, ES, 1,
+                         (((U >> 31) & 1u) ? 4096u : 0u) | (xcd_bit ? 8192u : 0u) | 48u | 256u, ES, 1,
                      ((U >> 8) & 0xffu) ? ((U >> 8) & 0xffu) : 1,
                      (G >> 16) ? (G >> 16) : 64, cv_bits ? cv_bits : 1,
                      ((U >> 16) & 0xffu) ? ((U >> 16) & 0xffu) : 1};

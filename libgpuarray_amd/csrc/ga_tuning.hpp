@@ -25,7 +25,7 @@
   X(REDUX_MIN_UNITS) X(REDUX_NT) X(REDUX_NT_LINES) X(REDUX_RB) X(REDUX_RPW) X(REDUX_SPLIT_MAJOR_MIN) \
   X(REDUX_SROWS) X(REDUX_SROWS_MAX_BYTES) X(REDUX_SROWS_MIN_BYTES) X(REDUX_SROWS_MIN_ROWS) \
   X(REDUX_TAIL) X(REDUX_TOUCH) X(REDUX_TROWS) X(REDUX_TROWS_DIRECT) X(REDUX_TROWS_MAX_BYTES) \
-  X(REDUX_TROWS_MAX_CHUNKS) X(REDUX_TROWS_MIN_ROWS) X(REDUX_U) X(REDUX_WROWS) \
+  X(REDUX_TROWS_MAX_CHUNKS) X(REDUX_TROWS_MIN_ROWS) X(REDUX_U) X(REDUX_WROWS) X(REDUX_XCD) \
   X(TAKE1_SHORT_ROWS)
 
 enum ga_knob : unsigned {

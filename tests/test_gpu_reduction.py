@@ -1108,6 +1108,40 @@ def test_column_reductions_of_four_byte_elements_on_any_layout(ctx, knobs, dtype
     assert np.array_equal(np.asarray(R.sum(g, axis=(0, 1))), ops[0][2](view, (0, 1)))
 
 
+@pytest.mark.parametrize("order", [0, 1, 2])
+def test_column_kernel_groups_numbered_to_keep_neighbours_on_one_die(ctx, knobs, order):
+    """The column kernel may number its groups so that the neighbours along the
+    inner kept dim run one after another on the same die (REDUX_XCD: 0 never,
+    1 when kept rows start off the 128-byte lines, 2 always).  The numbering
+    must reach every tile of outputs and every piece of the reduced range
+    exactly once: leading, middle and several axes, group counts that are and
+    are not multiples of 8 (also fewer than 8), one and several pieces per
+    output with the finish inside the launch, sums, extrema with positions and
+    any / all, against NumPy, exact."""
+    knobs(REDUX_XCD=order, REDUX_FOLD=0, REDUX_PCOLS=0)
+    rng = np.random.default_rng(4100 + order)
+    for shape, ax in (((700, 1000), 0), ((64, 130, 250), 1), ((3, 20000, 37), 1), ((9, 40, 1001), (0, 1)),
+                      ((40000, 9), 0), ((5, 7, 300, 129), (0, 2)), ((2, 100000, 4), 1), ((333, 8191), 0),
+                      ((17, 1200, 513), 1), ((4100, 2050), 0)):
+        host = rng.integers(-20, 21, size=shape).astype(np.float32)
+        g = gpuarray.array(host, context=ctx)
+        assert np.array_equal(np.asarray(R.sum(g, axis=ax)), host.sum(axis=ax, dtype=np.float64).astype(np.float32)), shape
+        assert np.array_equal(np.asarray(R.min(g, axis=ax)), host.min(axis=ax)), shape
+        gi = gpuarray.array(host.astype(np.int32), context=ctx)
+        assert np.array_equal(np.asarray(R.sum(gi, axis=ax, dtype="int64")), host.astype(np.int64).sum(axis=ax)), shape
+        if isinstance(ax, int):
+            v, i = R.maxandargmax(g, axis=ax)
+            assert np.array_equal(np.asarray(v), host.max(axis=ax)) and np.array_equal(np.asarray(i), host.argmax(axis=ax)), shape
+        gb = gpuarray.array((host > -20).astype(np.bool_), context=ctx)
+        assert np.array_equal(np.asarray(R.all(gb, axis=ax)), (host > -20).all(axis=ax)), shape
+    # kept rows that start off the 128-byte lines inside a wider buffer
+    root = rng.integers(-20, 21, size=(1200, 777)).astype(np.float32)
+    view = root[:, 5:774]
+    g, _ = to_gpu_view(view, ctx)
+    assert np.array_equal(np.asarray(R.sum(g, axis=0)), view.sum(axis=0, dtype=np.float64).astype(np.float32))
+    assert np.array_equal(np.asarray(R.max(g, axis=0)), view.max(axis=0))
+
+
 @pytest.mark.parametrize("rows,cols", [(300, 70001), (130, 150000), (520, 66000), (41, 300000)])
 def test_rows_cut_to_even_out_the_compute_units(ctx, knobs, rows, cols):
     """A few hundred long rows, one group each, would leave some compute units
