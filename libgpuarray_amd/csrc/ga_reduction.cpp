@@ -1574,7 +1574,10 @@ class reduction_call {
       // kernel's last piece combines a tile's partials by itself, so it must
       // not have many: over axis 0 of (4096, 16384) 44.0 / 42.0 us, of
       // (16384, 4096) 44.3 / 43.8, of (65536, 1024) 44.0 / 51.9, of
-      // (2^20, 64) 44.3 / 73.0.
+      // (2^20, 64) 44.3 / 73.0.  With up to 16 pieces per tile they may be as
+      // short as 32 KiB: sum over the middle axis of (128, 500, 128) floats,
+      // two launches / one, 12.6 / 9.7 us, of (32, 2000, 256) 17.0 / 14.7, over
+      // axis 0 of (4000, 4000) 16.3 / 15.4.
       bool fuse = groups <= fused_max;
       // (partials that carry an index cost the column kernel's last piece twice
       // the loads: maxandargmax over axis 0 of (8192, 8192) 47.8 / 50.5)
@@ -1594,7 +1597,7 @@ class reduction_call {
         const double piece_bytes = (double)nrows * (double)rtotal * (double)elsz_sum / (double)groups;
         fuse = use_row ? piece_bytes >= (double)TUNE(tn, REDUX_FUSED_PIECE, 384u << 10)
                        : (!carries_index && p.nsplit <= (int)TUNE(tn, REDUX_FUSED_COL_SPLITS, 16) &&
-                          piece_bytes >= (double)TUNE(tn, REDUX_FUSED_COL_PIECE, 128u << 10));
+                          piece_bytes >= (double)TUNE(tn, REDUX_FUSED_COL_PIECE, 32u << 10));
       }
       if (fuse && counters <= ga_hip_redux_counters_max && (accsz == 4 || accsz == 8)) {
         if (ga_hip_redux_counters(ctx) != nullptr) {
