@@ -86,7 +86,9 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * load for a lane's four rows), 9 the flat kernel with the arrays in tmask
  * (read-only, broadcast against the dense ones) read through the coordinates
  * of the flat index in nd = 2 or 3 dims (idx64 then carries the mask of those
- * among them that are fetched a whole aligned chunk at a time), 10 as 3 with
+ * among them that are fetched a whole aligned chunk at a time in bits 0..15,
+ * and in bits 16.. the mask of those whose chunks inside one row of the inner
+ * dim are fetched with one load on four-byte boundaries), 10 as 3 with
  * one group of two elements per lane (8-byte types, no transposed operand). */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
                                            unsigned int n, void *args, int flags,

@@ -90,6 +90,10 @@ def main():
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 2, 0, 0b010))
     check("elemwise flat, one operand read a chunk at a time through the flat index's coordinates",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 2, 0b010, 0b010))
+    check("elemwise flat, an operand's chunks inside one row fetched with one load on four-byte boundaries",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 2, 0b010 << 16, 0b010))
+    check("elemwise flat, the same for two operands, 3 dims",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 3, 0b011 << 16, 0b011))
     check("elemwise flat, two operands read through the flat index's coordinates, 3 dims",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 3, 0, 0b011))
     check("elemwise flat, 2 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 5, 0, 0, 0))
@@ -197,7 +201,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "27 elementwise)" % (n + 20, m, t))
+          "29 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

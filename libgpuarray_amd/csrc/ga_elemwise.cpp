@@ -133,7 +133,7 @@ struct _GpuElemwise {
   std::map<unsigned, GpuKernel> k_flat_tiled;
   // the flat kernel with some read-only operands addressed through the
   // coordinates of the flat index (broadcast operands), by (mask, dims)
-  std::map<uint64_t, GpuKernel> k_flat_periodic;
+  std::map<std::array<uint32_t, 4>, GpuKernel> k_flat_periodic;
   bool flat_forced = false;   // the environment fixed the flat kernel's shape
   // strided kernels by variant key: "<nd>:<idx64>:<transposed mask>"
   std::map<std::string, GpuKernel> k_strided;
@@ -203,9 +203,13 @@ void emit_header(const GpuElemwise *ge, std::string &s) {
 // then ps0, ps1, ps2 per such array.  Arrays also in pvmask have unit stride
 // along the inner dim and everything aligned to the chunk, and the caller
 // passes no head: a chunk's elements are then one chunk of the operand too,
-// fetched with one load.
+// fetched with one load.  Arrays in pumask (four-byte elements, four to a
+// chunk, not in pvmask) fetch a chunk that lies inside one row of the inner
+// dim with one load that assumes four-byte boundaries only, when their stride
+// along that dim is the element's size; the chunks that straddle two rows
+// stay element by element.
 std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned unroll = 0, int tiled = -1,
-                     unsigned pmask = 0, unsigned pnd = 2, unsigned pvmask = 0) {
+                     unsigned pmask = 0, unsigned pnd = 2, unsigned pvmask = 0, unsigned pumask = 0) {
   std::string s;
   const unsigned V = ge->vec, U = unroll ? unroll : ge->unroll;
   const bool tile = tiled < 0 ? ge->tile : tiled != 0;
@@ -222,6 +226,11 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
   auto is_pv = [&](const ge_arg &a) {
     const size_t j = (size_t)(&a - ge->args.data());
     return aidx[j] >= 0 && ((pmask & pvmask) >> aidx[j]) & 1u;
+  };
+  auto is_pu = [&](const ge_arg &a) {
+    const size_t j = (size_t)(&a - ge->args.data());
+    return aidx[j] >= 0 && ((pmask & ~pvmask & pumask) >> aidx[j]) & 1u && V == 4 &&
+           gpuarray_get_elsize(a.typecode) == 4;
   };
   // lvalue of a periodic operand's element at coordinates named c0/c1/c2
   auto p_elem = [&](const ge_arg &a, const char *c0, const char *c1, const char *c2) {
@@ -244,6 +253,11 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     return e;
   };
   emit_header(ge, s);
+  {
+    bool any_pu = false;
+    for (const ge_arg &a : ge->args) any_pu = any_pu || is_pu(a);
+    if (any_pu) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  }
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size n";
   ktypes.push_back(GA_SIZE);
   for (const ge_arg &a : ge->args) {
@@ -297,8 +311,8 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
     for (const ge_arg &a : ge->args) {
       if (!a.is_array()) continue;
       size_t cb = gpuarray_get_elsize(a.typecode) * V;
-      appendf(s, "union { %s c; %s e[%u]; } %s_u[%u];\n", chunk_type(cb), ctype(a.typecode), V,
-              a.name.c_str(), U);
+      appendf(s, "union { %s c; %s e[%u];%s } %s_u[%u];\n", chunk_type(cb), ctype(a.typecode), V,
+              is_pu(a) ? " ga_chunk16u w;" : "", a.name.c_str(), U);
     }
     appendf(s, "#pragma unroll\nfor (int ga_u = 0; ga_u < %u; ga_u++) {\n", U);
     s += "const ga_size ga_c = ga_c0 + (ga_size)ga_u * ga_ustep;\nif (ga_c < ga_nchunks) {\n";
@@ -314,10 +328,19 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
                      "(ga_ssize)ga_p1 * %s_ps1 + (ga_ssize)ga_p2 * %s_ps2);\n",
                   a.name.c_str(), chunk_type(cb), a.name.c_str(), a.name.c_str(), a.name.c_str(), a.name.c_str());
         }
+      for (const ge_arg &a : ge->args)
+        if (is_pu(a))
+          appendf(s, "const bool %s_w = %s_ps2 == 4 && ga_p2 + %uu <= ga_d2;\n"
+                     "if (%s_w) %s_u[ga_u].w = *(GLOBAL_MEM const ga_chunk16u *)((GLOBAL_MEM const char *)%s_p + "
+                     "(ga_ssize)ga_p0 * %s_ps0 + (ga_ssize)ga_p1 * %s_ps1 + (ga_ssize)ga_p2 * 4);\n",
+                  a.name.c_str(), a.name.c_str(), V, a.name.c_str(), a.name.c_str(), a.name.c_str(),
+                  a.name.c_str(), a.name.c_str());
       appendf(s, "#pragma unroll\nfor (int ga_v = 0; ga_v < %u; ga_v++) {\n", V);
       for (const ge_arg &a : ge->args)
-        if (is_p(a) && !is_pv(a))
+        if (is_p(a) && !is_pv(a)) {
+          if (is_pu(a)) appendf(s, "if (!%s_w) ", a.name.c_str());
           appendf(s, "%s_u[ga_u].e[ga_v] = %s;\n", a.name.c_str(), p_elem(a, "ga_p0", "ga_p1", "ga_p2").c_str());
+        }
       s += "if (++ga_p2 == ga_d2) { ga_p2 = 0; ";
       s += pnd == 3 ? "if (++ga_p1 == ga_d1) { ga_p1 = 0; ga_p0++; } }\n" : "ga_p1++; }\n";
       s += "}\n}\n";
@@ -1213,6 +1236,7 @@ int check_flat(GpuElemwise *ge, void **args, size_t *n_out, bool *flat) {
 struct flat_periodic {
   unsigned pmask = 0, pnd = 2;
   unsigned pvmask = 0;   // of pmask: operands a chunk of which is one aligned load (when there is no head)
+  unsigned pumask = 0;   // of pmask: a chunk inside one row is one load on four-byte boundaries
   unsigned d1 = 1, d2 = 1, k1 = 0, k2 = 0;
   uint64_t m1 = 0, m2 = 0;
   std::vector<std::array<ssize_t, 3>> ps;   // indexed by array
@@ -1306,11 +1330,12 @@ int call_flat(GpuElemwise *ge, void **args, size_t n, const size_t *offs,
   }
   if (pi != nullptr) {
     const unsigned pv = (vec_ok && head == 0) ? pi->pvmask : 0u;
-    const uint64_t key = ((uint64_t)pv << 32) | (pi->pmask << 2) | pi->pnd;
+    const unsigned pu = vec_ok ? pi->pumask & ~pv : 0u;
+    const std::array<uint32_t, 4> key = {{pi->pmask, pi->pnd, pv, pu}};
     auto it = ge->k_flat_periodic.find(key);
     if (it == ge->k_flat_periodic.end()) {
       std::vector<int> ktypes;
-      std::string src = gen_flat(ge, ktypes, 0, -1, pi->pmask, pi->pnd, pv);
+      std::string src = gen_flat(ge, ktypes, 0, -1, pi->pmask, pi->pnd, pv, pu);
       GpuKernel nk = {nullptr, nullptr};
       if ((err = build_kernel(ge, &nk, src, ktypes)) != GA_NO_ERROR) return err;
       it = ge->k_flat_periodic.emplace(key, nk).first;
@@ -1575,6 +1600,21 @@ class strided_call {
           if (strs[k][j] % (ssize_t)cb != 0) whole_chunks = false;
       }
       if (whole_chunks) pi.pvmask |= 1u << k;
+      // one load on four-byte boundaries for the chunks inside a row: the
+      // operand's own base and outer strides only need the element's alignment.
+      // A wavefront with a chunk that straddles two rows runs both ways, so
+      // this is for long rows.  Measured on MI355X, o = a + b with b one row,
+      // element by element / this way: rows of 50257 floats 91.2 -> 86.4 us
+      // (73.6 -> 77.7 % of peak), of 2050 91.1 -> 84.6, (512, 64, 2050) +
+      // (512, 1, 2050) 93.9 -> 88.4, rows of 1001 87.7 -> 85.8 (but 16 MB of
+      // them 8.0 -> 8.3); rows of 17 90.3 -> 116.9, of 10 54.1 -> 70.0.
+      if (sx == 4 && elsz[k] == 4 && V == 4 &&
+          dims[nd - 1] >= (size_t)TUNE(tn, ELEMWISE_PERIODIC_ROWLOAD, 1024) && TUNE(tn, ELEMWISE_PERIODIC_ROWLOAD, 1024) != 0) {
+        const GpuArray *v = (const GpuArray *)args[i];
+        bool ok = ((uintptr_t)v->data->devptr + offs[k]) % 4 == 0;
+        for (unsigned j = 0; j + 1 < nd; j++) ok = ok && strs[k][j] % 4 == 0;
+        if (ok) pi.pumask |= 1u << k;
+      }
       inner_constant = inner_constant && (sx == 0 || (whole_chunks && TUNE(tn, ELEMWISE_PERIODIC_VEC, 1)));
       pi.pmask |= 1u << k;
       for (unsigned j = 0; j < nd; j++) pi.ps[k][3 - nd + j] = strs[k][j];
@@ -2043,7 +2083,9 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // 13: as 3 for the same
   // 9: the flat kernel with the arrays in tmask read through the coordinates of the flat index (nd = 2 or 3)
   // (idx64 then carries the mask of those fetched a whole chunk at a time)
-  if (strided == 9) return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64).c_str());
+  // (and its bits 16.. the mask of those that fetch a chunk inside one row with one load on four-byte boundaries)
+  if (strided == 9)
+    return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64 & 0xffffu, (unsigned)idx64 >> 16).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 && strided != 13 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu

@@ -748,6 +748,53 @@ def test_math_library_functions_match_numpy(ctx):
     assert np.allclose(np.asarray(out), np.sqrt(ia.astype(np.float64)) + ia.astype(np.float64) ** 2, rtol=1e-15)
 
 
+@pytest.mark.parametrize("rowload", [8, 0])
+def test_broadcast_rows_of_four_byte_elements_fetched_a_chunk_at_a_time(ctx, knobs, rowload):
+    """A row operand broadcast against a dense array whose rows are no whole
+    number of 16-byte chunks, or that does not start on a 16-byte boundary:
+    the flat kernel fetches the chunks that lie inside one row with one load
+    that assumes four-byte boundaries only, and the chunks that straddle two
+    rows element by element (ELEMWISE_PERIODIC_ROWLOAD: the shortest row that
+    is read this way, 1024 elements unless set; 0: none).  Row lengths around
+    the multiples of four, every phase of the operand's first element, a
+    dense array that starts off a chunk (a head of one to three elements), two
+    and three dims, int32 as well; bit for bit against NumPy."""
+    knobs(ELEMWISE_PERIODIC=2, ELEMWISE_PERIODIC_ROWLOAD=rowload)
+    rng = np.random.default_rng(93 + rowload)
+    for dt in ("float32", "int32"):
+        k2 = ga.GpuElemwise(ctx, "o = a * b + c", [arg("a", dt, read=True), arg("b", dt, read=True),
+                                                    arg("c", dt, read=True), arg("o", dt, write=True)])
+        draw = lambda shape: rng.integers(-50, 51, size=shape).astype(dt)
+        for R, Cn in ((300, 1001), (517, 10), (64, 17), (1000, 8), (77, 9), (4099, 11), (33, 1000), (129, 254), (5, 6)):
+            for lead in (0, 1, 2, 3):
+                a = draw((R, Cn))
+                wide = draw((1, Cn + 4))
+                row = wide[:, lead:lead + Cn]
+                col = draw((R, 1))
+                ga_, gw, gc = (gpuarray.array(x, context=ctx) for x in (a, wide, col))
+                out = gpuarray.empty((R, Cn), dt, context=ctx)
+                k2(ga_, gw[:, lead:lead + Cn], gc, out, broadcast=True)
+                assert np.array_equal(np.asarray(out), a * row + col), (dt, R, Cn, lead)
+            # the dense array starts one to three elements into its buffer
+            for head in (1, 3):
+                flat = draw((R * Cn + 4,))
+                gf = gpuarray.array(flat, context=ctx)
+                a = flat[head:head + R * Cn].reshape(R, Cn)
+                row, col = draw((1, Cn)), draw((R, 1))
+                out = gpuarray.empty((R, Cn), dt, context=ctx)
+                k2(gf[head:head + R * Cn].reshape((R, Cn)), gpuarray.array(row, context=ctx),
+                   gpuarray.array(col, context=ctx), out, broadcast=True)
+                assert np.array_equal(np.asarray(out), a * row + col), (dt, R, Cn, "head", head)
+        # three dims: an operand that varies along the outer and the inner dim, and a row of the inner dim
+        for shape in ((33, 10, 257), (2, 5, 4099), (9, 6, 250), (7, 3, 9)):
+            a = draw(shape)
+            nb = draw((shape[0], 1, shape[2]))
+            rw = draw((1, 1, shape[2]))
+            out = gpuarray.empty(shape, dt, context=ctx)
+            k2(gpuarray.array(a, context=ctx), gpuarray.array(nb, context=ctx), gpuarray.array(rw, context=ctx), out, broadcast=True)
+            assert np.array_equal(np.asarray(out), a * nb + rw), (dt, shape)
+
+
 @pytest.mark.parametrize("mode", ["1", "2", "0"])
 def test_dense_arrays_with_broadcast_operands(ctx, oracle, knobs, mode):
     """Dense arrays combined with operands broadcast along some dims take the
