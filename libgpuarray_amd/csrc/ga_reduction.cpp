@@ -1940,7 +1940,13 @@ static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsign
   const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
   // (one kept element is a full reduction of a dense array: the planned path's ground)
   if (F < 2 || R < 2 || R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20)) return GA_NO_ERROR;
-  if (rowb % 16 == 0 && rowb >= 256) return GA_NO_ERROR;   // the column kernel's own ground
+  // The column kernel's own ground: kept rows of whole 16-byte pieces from 256
+  // bytes on.  Between 256 and 512 bytes its second tile of 256 bytes is mostly
+  // idle and this kernel is ahead (sums over axis 0, column kernel in two
+  // launches / this one: (2^20, 72) floats 62.3 -> 52.0 us, 61 -> 73 % of peak,
+  // (2^20, 36) doubles 62.0 -> 50.0, (2^18, 68) floats 20.9 -> 19.7; 19 MB of
+  // rows of 72 floats 11.2 -> 11.7); rows of 256 bytes exactly are a tie.
+  if (rowb % 16 == 0 && (rowb == 256 || rowb >= TUNE(tn, REDUX_PCOLS_COL_BYTES, 512))) return GA_NO_ERROR;
   if (es > 8 || 16 % es != 0 || d0->nd != s0->nd - reduxLen || d0->nd > (unsigned)RD_MAXD) return GA_NO_ERROR;
   for (unsigned j = 0; j < d0->nd; j++)
     if (d0->dimensions[j] != s0->dimensions[reduxLen + j]) return GA_NO_ERROR;

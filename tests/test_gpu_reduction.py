@@ -1391,6 +1391,16 @@ def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, route):
                 moved = host.reshape(-1, int(np.prod(kept)))
                 assert np.array_equal(np.asarray(val).ravel(), moved.max(axis=0))
                 assert np.array_equal(np.asarray(idx).ravel(), moved.argmax(axis=0))
+    # kept rows of whole 16-byte pieces between 256 and 512 bytes (one launch too: the
+    # column kernel's second tile of 256 bytes would be mostly idle), and 256 bytes exactly
+    for shape, dt in (((1 << 16, 72), "float32"), ((1 << 15, 36), "float64"), ((1 << 16, 68), "int32"),
+                      ((40000, 124), "float32"), ((1 << 16, 64), "float32")):
+        host = rng.integers(-3, 4, size=shape).astype(dt)
+        g = gpuarray.array(host, context=ctx)
+        got = np.asarray(R.sum(g, axis=0, dtype="int64" if dt == "int32" else dt))
+        assert np.array_equal(got, host.sum(axis=0, dtype=np.int64 if dt == "int32" else np.float64).astype(got.dtype)), (shape, dt)
+        if dt == "int32":
+            assert np.array_equal(np.asarray(R.max(g, axis=0)), host.max(axis=0)), (shape, dt)
     # products (of +-1, so that nothing overflows), float sums to tolerance, a strided destination
     host = rng.choice(np.array([1.0, -1.0], dtype=np.float32), size=(1 << 20, 6))
     g = gpuarray.array(host, context=ctx)
