@@ -24,6 +24,7 @@
 #include <algorithm>
 #include <array>
 #include <cctype>
+#include <cmath>
 #include <map>
 #include <mutex>
 #include <string>
@@ -1456,9 +1457,48 @@ class reduction_call {
                        (stc0 == GA_FLOAT || stc0 == GA_DOUBLE) && acc_typecode(gr, d0_tc) == stc0 &&
                        TUNE(tn, REDUX_LIGHT, 1) != 0 &&
                        scratch_skip == 0;   // folded rows measured better with three: (2^24, 3) 38.8 against 43.4 us
-    const int64_t target = ncu * (int64_t)TUNE(tn, REDUX_GROUPS_PER_CU, CV > 1 ? (light ? 2 : 3) : 8);
+    // Lanes past the end of the inner free dim idle (160 kept floats under tiles
+    // of 256: 5 lanes of 8), and a group then has fewer bytes in flight: such
+    // float sums get the third group per unit as well.  Sums over axis 0, two /
+    // three groups: (419430, 160) floats 51.6 -> 44.6 us (65 -> 75 % of peak),
+    // (209715, 320) 47.6 -> 44.1, (174762, 384) 48.4 -> 44.9; over the middle
+    // axis of (64, 4096, 320) 58.6 -> 52.0 (71 -> 81 %), of (64, 4096, 160)
+    // 39.4 -> 29.1, of (64, 8192, 72) 32.0 -> 28.4.
+    const double lanes_used = (double)fin / (double)(p.gx * (int64_t)(CX * CV));
+    const bool idle_lanes = light && CV > 1 && lanes_used <= 0.8 && TUNE(tn, REDUX_COL_IDLE, 1) != 0;
+    const int64_t target = ncu * (int64_t)TUNE(tn, REDUX_GROUPS_PER_CU, CV > 1 ? (light && !idle_lanes ? 2 : 3) : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
+      // Groups are dealt out to the compute units in turn: a few more than a
+      // whole number per unit leave some units with one group more than the
+      // rest (3 tiles of outputs in 171 pieces: 513 groups on 256 units; 192
+      // tiles in 3 pieces: 576).  Of the piece counts from the target down to
+      // one group per unit less and up to one more, the nearest one that fills
+      // the units more evenly is taken.  Sums of floats, before / after: over
+      // axis 0 of (87381, 768) 51.4 -> 45.7 us (65 -> 74 % of peak), of
+      // (104857, 640) 50.7 -> 45.6, of (20000, 3000) 61 -> 71 %, of (4096, 12000)
+      // 70 -> 77 %; whole powers of two divide the target and are not touched.
+      if (TUNE(tn, REDUX_COL_BALANCE, 1) != 0) {
+        auto excess = [&](int64_t ns) {
+          const double per = (double)(base_groups * ns) / (double)ncu;
+          return std::ceil(per) / per;
+        };
+        int64_t cap = rtotal / 64 < 4096 ? rtotal / 64 : 4096;
+        if (cap < 1) cap = 1;
+        const int64_t lo = std::max<int64_t>(1, (target - ncu) / base_groups);
+        const int64_t hi = std::min<int64_t>(cap, (target + ncu + base_groups - 1) / base_groups);
+        if (nsplit <= cap && base_groups * nsplit >= ncu) {
+          int64_t best = nsplit;
+          double be = excess(nsplit);
+          for (int64_t d = 1; nsplit - d >= lo || nsplit + d <= hi; d++)
+            for (const int64_t ns : {nsplit - d, nsplit + d})
+              if (ns >= lo && ns <= hi && base_groups * ns >= ncu && excess(ns) + 0.02 < be) {
+                best = ns;
+                be = excess(ns);
+              }
+          nsplit = best;
+        }
+      }
       if (nsplit > rtotal / 64) nsplit = rtotal / 64;
       if (nsplit > 4096) nsplit = 4096;
       if (nsplit < 1) nsplit = 1;

@@ -17,7 +17,7 @@
   X(ELEMWISE_PANEL) X(ELEMWISE_PERIODIC) X(ELEMWISE_PERIODIC_ROWLOAD) X(ELEMWISE_PERIODIC_VEC) X(ELEMWISE_LOOSE) X(ELEMWISE_LOOSE_MIN_BYTES) X(ELEMWISE_QUADS) X(ELEMWISE_SKEW) \
   X(ELEMWISE_TILE) X(ELEMWISE_TTILE) X(ELEMWISE_TTILE_MIN) X(ELEMWISE_UNROLL) X(ELEMWISE_VEC4) \
   X(ELEMWISE_ZMASK) X(FILL_KERNEL_MIN) X(MARK_EVENT_FLAGS) X(MOVE_KERNEL_MIN) X(REDUX_BALANCE) X(REDUX_COLVEC) \
-  X(REDUX_COL_CVMAX) X(REDUX_COL_FAR) X(REDUX_COL_LOOSE) X(REDUX_COL_LOOSE_MIN_BYTES) X(REDUX_COL_ROWS) X(REDUX_COL_U) X(REDUX_FAST8) \
+  X(REDUX_COL_BALANCE) X(REDUX_COL_CVMAX) X(REDUX_COL_FAR) X(REDUX_COL_IDLE) X(REDUX_COL_LOOSE) X(REDUX_COL_LOOSE_MIN_BYTES) X(REDUX_COL_ROWS) X(REDUX_COL_U) X(REDUX_FAST8) \
   X(REDUX_FOLD) X(REDUX_FOLD_BYTES) X(REDUX_FOLD_MIN_BYTES) X(REDUX_FOLD_SLAB_MIN_BYTES) X(REDUX_FUSED) \
   X(REDUX_FUSED_COL_FEW) X(REDUX_FUSED_COL_PIECE) X(REDUX_FUSED_COL_SPLITS) \
   X(REDUX_FUSED_PIECE) X(REDUX_G) X(REDUX_GROUPS_PER_CU) X(REDUX_INFLIGHT) X(REDUX_INTERLEAVE) \

@@ -1108,6 +1108,30 @@ def test_column_reductions_of_four_byte_elements_on_any_layout(ctx, knobs, dtype
     assert np.array_equal(np.asarray(R.sum(g, axis=(0, 1))), ops[0][2](view, (0, 1)))
 
 
+@pytest.mark.parametrize("even", [1, 0])
+def test_column_pieces_counted_to_fill_the_compute_units_evenly(ctx, knobs, even):
+    """The column kernel cuts the reduced range into the number of pieces that
+    leaves every compute unit with the same number of groups where one exists
+    near its target (REDUX_COL_BALANCE), and gives float sums a third group
+    per unit where the inner kept dim leaves lanes idle (REDUX_COL_IDLE).
+    Tiles of outputs that do not divide the unit count (3, 5, 12, 192 of them),
+    kept rows of 160 and 72 elements, leading and middle axes; sums, integer
+    and float extrema with positions, against NumPy, exact, whichever count
+    of pieces the plan takes."""
+    knobs(REDUX_COL_BALANCE=even, REDUX_COL_IDLE=even, REDUX_FOLD=0, REDUX_PCOLS=0)
+    rng = np.random.default_rng(4300 + even)
+    for shape, ax in (((6000, 768), 0), ((5000, 640), 0), ((9000, 160), 0), ((2500, 3000), 0), ((1100, 1280), 0),
+                      ((64, 600, 320), 1), ((64, 700, 160), 1), ((32, 1500, 72), 1), ((3, 4000, 257), 1)):
+        host = rng.integers(-20, 21, size=shape).astype(np.float32)
+        g = gpuarray.array(host, context=ctx)
+        assert np.array_equal(np.asarray(R.sum(g, axis=ax)), host.sum(axis=ax, dtype=np.float64).astype(np.float32)), shape
+        v, i = R.maxandargmax(g, axis=ax)
+        assert np.array_equal(np.asarray(v), host.max(axis=ax)) and np.array_equal(np.asarray(i), host.argmax(axis=ax)), shape
+        gi = gpuarray.array(host.astype(np.int32), context=ctx)
+        assert np.array_equal(np.asarray(R.sum(gi, axis=ax, dtype="int64")), host.astype(np.int64).sum(axis=ax)), shape
+        assert np.array_equal(np.asarray(R.min(gi, axis=ax)), host.astype(np.int32).min(axis=ax)), shape
+
+
 @pytest.mark.parametrize("order", [0, 1, 2])
 def test_column_kernel_groups_numbered_to_keep_neighbours_on_one_die(ctx, knobs, order):
     """The column kernel may number its groups so that the neighbours along the
