@@ -1166,11 +1166,12 @@ def test_column_kernel_groups_numbered_to_keep_neighbours_on_one_die(ctx, knobs,
     assert np.array_equal(np.asarray(R.max(g, axis=0)), view.max(axis=0))
 
 
-@pytest.mark.parametrize("rows,cols", [(300, 70001), (130, 150000), (520, 66000), (41, 300000)])
+@pytest.mark.parametrize("rows,cols", [(300, 70001), (130, 150000), (520, 66000), (41, 300000), (10, 700001), (48, 140003), (3, 2000000)])
 def test_rows_cut_to_even_out_the_compute_units(ctx, knobs, rows, cols):
     """A few hundred long rows, one group each, would leave some compute units
-    with one group more than the others: such rows are cut into pieces
-    (REDUX_BALANCE).  Whole and cut rows must agree bit for bit on data whose
+    with one group more than the others: such rows are cut into pieces, and
+    rows that are in pieces anyway into the nearest number of pieces that
+    fills the units evenly (REDUX_BALANCE).  Whole and cut rows must agree bit for bit on data whose
     sums are exact, and with NumPy; the cut is there when the plan allows it
     (more than one launch, or a finish inside the first)."""
     rng = np.random.default_rng(rows)
