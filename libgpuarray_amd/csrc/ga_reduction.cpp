@@ -1166,9 +1166,11 @@ class reduction_call {
         // Rows already in pieces: another count costs nothing, so the nearest
         // one that fills the units more evenly is taken, below the target as
         // well as above (10 rows in 52 pieces are 520 groups on 256 units, in
-        // 51 pieces 510).  Sum over axis 1, floats: (10, 6710886) 47.3 -> 41.9 us,
-        // (24, 2796202) 47.8 -> 42.0, (48, 1398101) 48.8 -> 42.3, (3, 22369621)
-        // 46.4 -> 42.9, maximum of int32 (10, 6710886) 45.9 -> 42.5.
+        // 51 pieces 510).  Sum over axis 1, floats: (10, 6710886) 47.3 -> 43.7 us,
+        // (24, 2796202) 47.8 -> 43.3, (48, 1398101) 48.8 -> 42.9 (two launches ->
+        // one), (3, 22369621) 46.4 -> 42.7, maximum of int32 (10, 6710886) 45.9 ->
+        // 43.7.  The search stops at the first count within 7 % of even: one further
+        // away may cut the pieces too short to end in the same launch.
         const int64_t lo = std::max<int64_t>(1, (target - ncu) / rowgroups);
         int64_t best = nsplit;
         double be = excess(nsplit);
