@@ -1655,7 +1655,17 @@ class reduction_call {
         fuse = false;
       if (!fuse && fused_max > 0 && groups > fused_max) {
         const double piece_bytes = (double)nrows * (double)rtotal * (double)elsz_sum / (double)groups;
-        fuse = use_row ? piece_bytes >= (double)TUNE(tn, REDUX_FUSED_PIECE, 384u << 10)
+        // (rows in a few pieces each spread the counting over many counters and
+        // the combining over many groups, and below 160 MB the second launch is
+        // a larger share: there pieces from 64 KiB on.  Two launches / one:
+        // maximum over axis 1 of (64, 262144) floats 18.8 / 16.5 us, of int32
+        // (100, 100000) 13.1 / 10.0, sum of halves (50, 400000) 13.0 / 10.2, of
+        // (100, 671088) 26.8 / 24.1, of floats (40, 200000) 11.7 / 8.8; one row
+        // in 512 pieces stays with two: maximum of 2^24 floats 17.5 / 18.5, of
+        // 2^23 13.0 / 14.6; 268 MB of 130 to 520 rows 43.4 / 44.7, 45.8 / 47.7)
+        const bool few = p.nsplit <= (int)TUNE(tn, REDUX_FUSED_FEW, 64) &&
+                         (double)nrows * (double)rtotal * (double)elsz_sum < 160.0 * 1048576.0;
+        fuse = use_row ? piece_bytes >= (double)TUNE(tn, REDUX_FUSED_PIECE, few ? 64u << 10 : 384u << 10)
                        : (!carries_index && p.nsplit <= (int)TUNE(tn, REDUX_FUSED_COL_SPLITS, 16) &&
                           piece_bytes >= (double)TUNE(tn, REDUX_FUSED_COL_PIECE, 32u << 10));
       }
