@@ -100,6 +100,8 @@ def elemwise_cases():
          [("a", f, (8192, 8193), lambda b: b[:, 1:]), ("b", f, (8192, 8193), lambda b: b[:, :-1])], (8192, 8192), f),
         ("copy, 2^28 floats (1 GiB read, 1 GiB written: the yardstick of the traffic counters)", "o = a",
          [("a", f, (1 << 28,), None)], (1 << 28,), f),
+        ("(1335, 50257) + (1, 50257), a bias row off the 16-byte chunks", "o = a + b",
+         [("a", f, (1335, 50257), None), ("b", f, (1, 50257), None)], (1335, 50257), f),
     ]
 
 
@@ -145,6 +147,12 @@ def reduction_cases():
         ("sum", f, (8192, 8192), (0,), None, lambda a: a[:, 1:], "columns of a view that starts one element in"),
         ("sum", f, (64, 1000, 1000), (1,), None, None, "middle axis, rows of 4000 bytes"),
         ("sum", f, (64, 4096, 250), (1,), None, None, "middle axis over short kept rows: folded per slab"),
+        ("sum", f, (87381, 768), (0,), None, None, "bias gradient, 3 tiles of outputs: pieces counted to fill the units evenly"),
+        ("sum", f, (419430, 160), (0,), None, None, "bias gradient, kept rows that leave lanes idle"),
+        ("sum", f, (1 << 20, 72), (0,), None, None, "kept rows of 288 bytes, one launch"),
+        ("sum", f, (64, 4096, 320), (1,), None, None, "middle axis, 192 tiles of outputs"),
+        ("sum", f, (10, 6710886), (1,), None, None, "ten long rows"),
+        ("max", f, (64, 262144), (1,), None, None, "64 MB of rows in a few pieces each, one launch"),
     ]
 
 
