@@ -2283,6 +2283,126 @@ static int fold_rows(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigne
   return err;
 }
 
+// Reducing leading AND trailing dims of a dense array around kept ones when
+// the trailing reduced run is short - per-channel sums over (batch, channel,
+// a small height x width): the bias gradient of a convolution.  One kernel
+// would walk reduced rows of a few dozen elements that lie a whole slab
+// apart.  Done in two calls instead: the leading dims of (A, K B) go first,
+// with the column kernel at full load width, into K B partial results, and
+// the short trailing run of those (1 / A of the input) second.  For the
+// operations that may be regrouped, on 4 MiB and more, when the trailing run
+// has at most 4 KiB.  Measured on MI355X, sums of floats, kernel time of all
+// launches, one call / two: (64, 52428, 20) over axes (0, 2) 215.5 -> 46.1 us
+// (16 -> 73 % of peak), (64, 87381, 12) 147.6 -> 48.5, (256, 2048, 49) 34.6 ->
+// 23.5, (64, 1024, 196) 21.1 -> 13.8, (64, 8065, 130) 75.7 -> 52.4, (64, 5242,
+// 200) 53.7 -> 45.6, (64, 3495, 300) 52.3 -> 46.7, (16, 65536, 33) 40.4 ->
+// 30.2; from 400 floats on the two are within 2 us of each other up to 8 KiB.
+// Returns GA_NO_ERROR with *done = true when the reduction was carried out.
+static int outer_then_inner(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsigned reduxLen,
+                            const int *reduxList, bool *done, bool noalloc = false) {
+  *done = false;
+  gpucontext *ctx = gr->ctx;
+  const ga_tuning *tn = ga_hip_tuning(ctx);
+  const size_t max_inner = TUNE(tn, REDUX_OUTER_FIRST, 4096);
+  if (max_inner == 0 || gr->mapped || d0 == nullptr || reduxLen < 2 || reduxLen >= s0->nd ||
+      s0->nd > 16 || !GpuArray_IS_C_CONTIGUOUS(s0) || GpuArray_context(d0) != ctx)
+    return GA_NO_ERROR;
+  const rd_kind kind = gr->info.kind;
+  const int stc = s0->typecode;
+  const bool regroupable = !gr->info.has_d1 &&
+      (kind == K_SUM || kind == K_PROD || kind == K_AND || kind == K_OR || kind == K_XOR ||
+       kind == K_ALL || kind == K_ANY || ((kind == K_MIN || kind == K_MAX) && is_int_type(stc)));
+  if (!regroupable) return GA_NO_ERROR;
+  // the reduced axes are a leading run [0, a) and a trailing run [b, nd), both non-empty
+  bool reduced[16] = {};
+  for (unsigned i = 0; i < reduxLen; i++) {
+    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= s0->nd || reduced[reduxList[i]]) return GA_NO_ERROR;
+    reduced[reduxList[i]] = true;
+  }
+  unsigned a = 0, b = s0->nd;
+  while (a < s0->nd && reduced[a]) a++;
+  while (b > a && reduced[b - 1]) b--;
+  if (a == 0 || b == s0->nd || a >= b || a + (s0->nd - b) != reduxLen) return GA_NO_ERROR;
+  size_t A = 1, K = 1, B = 1;
+  for (unsigned j = 0; j < s0->nd; j++) (j < a ? A : j < b ? K : B) *= s0->dimensions[j];
+  const size_t es = gpuarray_get_elsize(stc);
+  if (A < 2 || B < 2 || K == 0 || B * es > max_inner ||
+      A * K * B * es < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20))
+    return GA_NO_ERROR;
+  // d0 must have the kept dims' shape (the launch below checks the rest)
+  if (d0->nd != b - a) return GA_NO_ERROR;
+  for (unsigned j = 0; j < d0->nd; j++)
+    if (d0->dimensions[j] != s0->dimensions[a + j]) return GA_NO_ERROR;
+
+  // type of the partial results: the accumulator's (a half result is summed in float)
+  int tmp_tc = acc_typecode(gr, d0->typecode);
+  if (tmp_tc == GA_HALF) tmp_tc = GA_FLOAT;
+  if (noalloc && (gr->fold_op == nullptr || gr->fold_tc != tmp_tc))
+    return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR,
+                      "GpuReduction_call_noalloc: the kernels for arrays of this layout are not "
+                      "built yet, and building them allocates; run GpuReduction_call once on "
+                      "arrays of this layout first");
+  if (gr->fold_op == nullptr || gr->fold_tc != tmp_tc) {
+    GpuReduction_free(gr->fold_op);
+    gr->fold_op = nullptr;
+    int err = make_plain_operator(&gr->fold_op, ctx, ctx->err, gr->op, tmp_tc);
+    if (err != GA_NO_ERROR) return err;
+    gr->fold_tc = tmp_tc;
+  }
+  // The partial results take the start of the context's scratch buffer (see
+  // fold_rows); the two calls below put their own partials behind them.
+  const size_t tes = gpuarray_get_elsize(tmp_tc);
+  const size_t tmp_len = K * B;
+  const size_t skip = (tmp_len * tes + 255) & ~(size_t)255;
+  gpudata *scr = nullptr;
+  if (noalloc) {
+    const char *why = "";
+    scr = ga_hip_static_scratch_buf(ctx, &why);
+    if (scr == nullptr)
+      return ga_err_fmt(ctx->err, GA_IMPL_ERROR,
+                        "GpuReduction_call_noalloc: the static scratch array was not found on "
+                        "this device when the context was made (%s)", why);
+    if (skip + 16 > ga_static_scratch_bytes)
+      return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,
+                        "GpuReduction_call_noalloc: the partial results of this reduction take "
+                        "%zu bytes; the static scratch array holds %zu",
+                        skip, (size_t)ga_static_scratch_bytes);
+  } else {
+    scr = ga_hip_scratch(ctx, skip + 16);
+  }
+  if (scr == nullptr) return ctx->err->code;
+  GpuArray tmp;
+  const ssize_t tmp_stride = (ssize_t)tes;
+  int err = GpuArray_fromdata(&tmp, scr, 0, tmp_tc, 1, &tmp_len, &tmp_stride, 1);
+  if (err != GA_NO_ERROR) return err;
+  {
+    // first call: (A, K B) over axis 0 into tmp
+    const size_t dims1[2] = {A, K * B};
+    const int64_t str1[2] = {(int64_t)(K * B * es), (int64_t)es};
+    const src_view src = {s0, str1};
+    const int axis0 = 0;
+    err = reduce_launch(gr, &tmp, nullptr, 2, dims1, &src, nullptr, 0, 1, &axis0, noalloc, skip);
+  }
+  if (err == GA_NO_ERROR) {
+    // second call: tmp as (kept dims..., B) over its last axis into d0
+    std::vector<size_t> dims2(d0->nd + 1);
+    std::vector<int64_t> str2(d0->nd + 1);
+    size_t run = tes;
+    for (unsigned j = d0->nd + 1; j-- > 0;) {
+      dims2[j] = j == d0->nd ? B : d0->dimensions[j];
+      str2[j] = (int64_t)run;
+      run *= dims2[j];
+    }
+    const src_view src = {&tmp, str2.data()};
+    const int axis = (int)d0->nd;
+    err = reduce_launch(gr->fold_op, d0, nullptr, d0->nd + 1, dims2.data(), &src, nullptr, 0, 1, &axis,
+                        noalloc, skip);
+  }
+  GpuArray_clear(&tmp);
+  if (err == GA_NO_ERROR) *done = true;
+  return err;
+}
+
 int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const GpuArray *s0,
                       unsigned reduxLen, const int *reduxList, int flags) {
   (void)flags;
@@ -2296,6 +2416,8 @@ int GpuReduction_call(const GpuReduction *cgr, GpuArray *d0, GpuArray *d1, const
     int err = pcols_call(gr, d0, s0, reduxLen, reduxList, &done);
     if (err != GA_NO_ERROR || done) return err;
     err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done);
+    if (err != GA_NO_ERROR || done) return err;
+    err = outer_then_inner(gr, d0, s0, reduxLen, reduxList, &done);
     if (err != GA_NO_ERROR || done) return err;
   }
   const src_view src = {s0, (const int64_t *)s0->strides};
@@ -2318,6 +2440,8 @@ int GpuReduction_call_noalloc(const GpuReduction *cgr, GpuArray *d0, GpuArray *d
     int err = pcols_call(gr, d0, s0, reduxLen, reduxList, &done, true);
     if (err != GA_NO_ERROR || done) return err;
     err = fold_rows(gr, d0, s0, reduxLen, reduxList, &done, true);
+    if (err != GA_NO_ERROR || done) return err;
+    err = outer_then_inner(gr, d0, s0, reduxLen, reduxList, &done, true);
     if (err != GA_NO_ERROR || done) return err;
   }
   const src_view src = {s0, (const int64_t *)s0->strides};

@@ -153,6 +153,8 @@ def reduction_cases():
         ("sum", f, (64, 4096, 320), (1,), None, None, "middle axis, 192 tiles of outputs"),
         ("sum", f, (10, 6710886), (1,), None, None, "ten long rows"),
         ("max", f, (64, 262144), (1,), None, None, "64 MB of rows in a few pieces each, one launch"),
+        ("sum", f, (256, 2048, 7, 7), (0, 2, 3), None, None, "bias gradient of a convolution, 7 x 7 maps: leading dims first"),
+        ("sum", f, (64, 16384, 8, 8), (0, 2, 3), None, None, "the same on 256 MiB"),
     ]
 
 

@@ -1373,6 +1373,58 @@ def test_a_run_of_middle_axes_over_short_kept_rows_is_folded_per_slab(ctx, knobs
     assert not np.asarray(wide)[:, :, [0, 2]].any()
 
 
+@pytest.mark.parametrize("two_calls", [1, 0])
+def test_leading_and_short_trailing_axes_around_kept_ones(ctx, knobs, two_calls):
+    """Per-channel reductions over (batch, channel, a small height x width):
+    leading and trailing dims reduced around kept ones.  With a trailing run of
+    at most REDUX_OUTER_FIRST bytes the leading dims are reduced first, at full
+    load width, and the short trailing run of the partial results second (0:
+    one call).  Every operation that may be regrouped, integer and floating
+    types, three to five dims, a strided destination, results against NumPy;
+    arg-reductions and floating extrema keep the single call and stay right."""
+    knobs(REDUX_OUTER_FIRST=4096 if two_calls else 0, REDUX_FOLD_MIN_BYTES=1)
+    rng = np.random.default_rng(5100 + two_calls)
+    cases = (((64, 400, 49), (0, 2)), ((16, 3000, 33), (0, 2)), ((8, 4, 500, 7, 7), (0, 1, 3, 4)), ((128, 100, 4, 4), (0, 2, 3)),
+             ((6, 5, 70, 3, 16), (0, 1, 4)), ((2, 100000, 12), (0, 2)), ((32, 64, 256), (0, 2)), ((32, 64, 257), (0, 2)))
+    every = ("float32", "int32", "int8", "float16", "uint8", "float64")
+    for ci, (shape, axes) in enumerate(cases):
+        for dt in (every[:2] if ci else every):
+            host = rng.integers(-3 if np.dtype(dt).kind in "if" else 0, 4, size=shape).astype(dt)
+            g = gpuarray.array(host, context=ctx)
+            kept = tuple(d for i, d in enumerate(shape) if i not in axes)
+            got = np.asarray(R.sum(g, axis=axes, dtype="int64" if np.dtype(dt).kind in "iu" else
+                                   ("float64" if dt == "float64" else "float32")))
+            assert got.shape == kept
+            assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64).astype(got.dtype)), (shape, dt, "sum")
+            for name, npf in (("all", np.all), ("any", np.any)):
+                got = np.asarray(R._reduce_named(g, name, np.dtype("bool"), axis=axes))
+                assert np.array_equal(got, npf(host, axis=axes)), (shape, dt, name)
+            if np.dtype(dt).kind in "iu":
+                for name, npf in (("max", np.max), ("min", np.min)):
+                    assert np.array_equal(np.asarray(getattr(R, name)(g, axis=axes)), npf(host, axis=axes)), (shape, dt, name)
+                got = np.asarray(R._reduce_named(g, "xor", np.dtype(dt), axis=axes))
+                assert np.array_equal(got, np.bitwise_xor.reduce(host, axis=axes)), (shape, dt, "xor")
+            else:
+                # floating extrema follow the order of the scan: one call, still right
+                assert np.array_equal(np.asarray(R.max(g, axis=axes)), host.max(axis=axes)), (shape, dt, "max")
+    # products of +-1, float sums to tolerance, a strided destination
+    host = rng.choice(np.array([1.0, -1.0], dtype=np.float32), size=(64, 300, 20))
+    g = gpuarray.array(host, context=ctx)
+    got = np.asarray(R._reduce_named(g, "prod", np.dtype("float32"), axis=(0, 2)))
+    assert np.array_equal(got, np.prod(host.astype(np.float64), axis=(0, 2)).astype(np.float32))
+    host = rng.standard_normal((64, 500, 49)).astype(np.float32) + np.float32(0.5)
+    g = gpuarray.array(host, context=ctx)
+    wide = gpuarray.zeros((500, 3), "float32", context=ctx)
+    ga.GpuReduction(ctx, "sum", "float32")(g, [0, 2], d0=wide[:, 1])
+    x64 = host.astype(np.float64)
+    assert_sum_close(np.asarray(wide)[:, 1], x64.sum(axis=(0, 2)), np.abs(x64).sum(axis=(0, 2)))
+    assert not np.asarray(wide)[:, [0, 2]].any()
+    # reduxList in any order
+    out = gpuarray.empty((500,), "float32", context=ctx)
+    ga.GpuReduction(ctx, "sum", "float32")(g, [2, 0], d0=out)
+    assert_sum_close(np.asarray(out), x64.sum(axis=(0, 2)), np.abs(x64).sum(axis=(0, 2)))
+
+
 @pytest.mark.parametrize("route", ["one launch", "folded", "neither"])
 def test_leading_dims_with_short_kept_rows_are_folded(ctx, knobs, route):
     """Reducing the leading dims of a dense array whose kept rows are short or

@@ -35,6 +35,10 @@ CASES = [
     # ... and longer ones through folded rows: every m rows taken as one long row, then
     # the m copies of each output combined; all intermediate results in the static array
     ("folded rows", "sum", "float32", (1 << 14, 250), (5000, 250), (0,), "float32", False),
+    # leading and a short trailing run of dims around kept ones: the leading dims first,
+    # their partial results in the static array, then the trailing run of those
+    ("leading dims first", "sum", "float32", (64, 512, 49), (32, 700, 49), (0, 2), "float32", False),
+    ("leading dims first, int", "sum", "int32", (16, 4, 300, 7, 7), (64, 2, 100, 4, 4), (0, 1, 3, 4), "int64", False),
 ]
 
 
