@@ -1999,27 +1999,58 @@ static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsign
       (kind == K_SUM || kind == K_PROD || kind == K_AND || kind == K_OR || kind == K_XOR ||
        kind == K_ALL || kind == K_ANY || ((kind == K_MIN || kind == K_MAX) && is_int_type(stc)));
   if (!regroupable) return GA_NO_ERROR;
+  // the reduced axes are one run of adjacent ones, [a0, a0 + reduxLen): the
+  // leading dims (a0 = 0), or a middle run under O kept slabs
   std::array<char, 64> seen{};
   if (reduxLen > seen.size()) return GA_NO_ERROR;
+  unsigned a0 = s0->nd;
   for (unsigned i = 0; i < reduxLen; i++) {
-    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= reduxLen || seen[reduxList[i]]) return GA_NO_ERROR;
-    seen[reduxList[i]] = 1;
+    if (reduxList[i] < 0 || (unsigned)reduxList[i] >= s0->nd) return GA_NO_ERROR;
+    if ((unsigned)reduxList[i] < a0) a0 = (unsigned)reduxList[i];
   }
-  size_t R = 1, F = 1;
-  for (unsigned j = 0; j < s0->nd; j++) (j < reduxLen ? R : F) *= s0->dimensions[j];
+  if (a0 + reduxLen >= s0->nd) return GA_NO_ERROR;
+  for (unsigned i = 0; i < reduxLen; i++) {
+    const unsigned at = (unsigned)reduxList[i] - a0;
+    if (at >= reduxLen || seen[at]) return GA_NO_ERROR;
+    seen[at] = 1;
+  }
+  size_t O = 1, R = 1, F = 1;
+  for (unsigned j = 0; j < s0->nd; j++) (j < a0 ? O : j < a0 + reduxLen ? R : F) *= s0->dimensions[j];
   const size_t es = gpuarray_get_elsize(stc), rowb = F * es;
   // (one kept element is a full reduction of a dense array: the planned path's ground)
-  if (F < 2 || R < 2 || R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20)) return GA_NO_ERROR;
+  if (F < 2 || R < 2 || O == 0 || O * R * rowb < TUNE(tn, REDUX_FOLD_MIN_BYTES, 4u << 20)) return GA_NO_ERROR;
+  // Slabs: one group each walks its slab as one run of chunks and writes the
+  // slab's outputs itself - no partial results, no counter.  For slabs of whole
+  // chunks that keep a group's lanes busy (4 KiB and more, up to 1 MiB), one
+  // per compute unit and more - but not a few more than a whole number per
+  // unit while that number is small: the stragglers then run alone ((524, 512,
+  // 250) 67 % of peak this way, 69 with the column kernel; (262, 512, 500) 59 /
+  // 69).  Measured on MI355X, sum over the middle axis of floats, column
+  // kernel / this one: (10922, 512, 12) 67.1 -> 44.5 us (50 -> 75 % of peak),
+  // (6553, 512, 20) 70 -> 80 %, (3971, 512, 33) 68 -> 80 %, (1008, 512, 130)
+  // 67 -> 79 %, (655, 512, 200) 60 -> 77 %, (436, 512, 300) 65 -> 78 %,
+  // (327, 512, 400) 68 -> 75 %.
+  const size_t slabb = R * rowb;
+  if (O > 1) {
+    const size_t ncu = ga_hip_numprocs(ctx);
+    const size_t rounds = O / ncu, over = O % ncu;
+    if (TUNE(tn, REDUX_PSLABS, 1) == 0 || slabb % 16 != 0 || slabb < 4096 ||
+        slabb > TUNE(tn, REDUX_PSLABS_MAX_BYTES, 1u << 20) ||
+        O < TUNE(tn, REDUX_PSLABS_MIN_SLABS, ncu) || O > 0x7fffffffull ||
+        (rounds <= 3 && over != 0 && over * 10 < ncu))
+      return GA_NO_ERROR;
+  }
   // The column kernel's own ground: kept rows of whole 16-byte pieces from 256
   // bytes on.  Between 256 and 512 bytes its second tile of 256 bytes is mostly
   // idle and this kernel is ahead (sums over axis 0, column kernel in two
   // launches / this one: (2^20, 72) floats 62.3 -> 52.0 us, 61 -> 73 % of peak,
   // (2^20, 36) doubles 62.0 -> 50.0, (2^18, 68) floats 20.9 -> 19.7; 19 MB of
   // rows of 72 floats 11.2 -> 11.7); rows of 256 bytes exactly are a tie.
-  if (rowb % 16 == 0 && (rowb == 256 || rowb >= TUNE(tn, REDUX_PCOLS_COL_BYTES, 512))) return GA_NO_ERROR;
+  // (under slabs it has no second tile to spare: there every row length is taken)
+  if (O == 1 && rowb % 16 == 0 && (rowb == 256 || rowb >= TUNE(tn, REDUX_PCOLS_COL_BYTES, 512))) return GA_NO_ERROR;
   if (es > 8 || 16 % es != 0 || d0->nd != s0->nd - reduxLen || d0->nd > (unsigned)RD_MAXD) return GA_NO_ERROR;
   for (unsigned j = 0; j < d0->nd; j++)
-    if (d0->dimensions[j] != s0->dimensions[reduxLen + j]) return GA_NO_ERROR;
+    if (d0->dimensions[j] != s0->dimensions[j < a0 ? j : reduxLen + j]) return GA_NO_ERROR;
   // the result's type must be one the operation accepts (the planned path reports what is wrong)
   const int d0_tc = d0->typecode;
   const bool logical = kind == K_ALL || kind == K_ANY, minmax = kind == K_MIN || kind == K_MAX;
@@ -2045,11 +2076,11 @@ static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsign
   uintptr_t base = 0;
   size_t bufsz = 0, readable = 0;
   ga_hip_buf_info(s0->data, &base, &bufsz, &readable);
-  const size_t bytes = R * rowb, chunks = (bytes + 15) / 16;
-  if ((base + s0->offset) % 16 != 0 || s0->offset + chunks * 16 > readable) return GA_NO_ERROR;
+  const size_t bytes = R * rowb, chunks = (bytes + 15) / 16;   // of one slab
+  if ((base + s0->offset) % 16 != 0 || s0->offset + O * chunks * 16 > readable) return GA_NO_ERROR;
   // (the counters are not to be had while the stream records a graph; a call
   // that may not allocate takes them only if an earlier call has made them)
-  if (noalloc ? !ga_hip_redux_counters_made(ctx) : ga_hip_redux_counters(ctx) == nullptr) {
+  if (O == 1 && (noalloc ? !ga_hip_redux_counters_made(ctx) : ga_hip_redux_counters(ctx) == nullptr)) {
     if (noalloc)
       return ga_err_set(ctx->err, GA_UNSUPPORTED_ERROR,
                         "GpuReduction_call_noalloc: the kernels for arrays of this layout are not "
@@ -2064,10 +2095,11 @@ static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsign
   // while they are a few thousand values.
   // (256 groups, floats, one launch against folded rows in two: kept rows of 63,
   // 16 128 partial values, 43.9 against 47.3 us; of 250, 64 000 values, 52.8 against 46.7)
+  if (O > 1) G = 1;   // a group per slab
   if (G * F > TUNE(tn, REDUX_PCOLS_MAX_PARTIALS, 20000)) return GA_NO_ERROR;
   size_t J = (chunks + G * L - 1) / (G * L);
   J = (J + U - 1) / U * U;
-  G = (chunks + L * J - 1) / (L * J);
+  if (O == 1) G = (chunks + L * J - 1) / (L * J);
   if (G < 1) G = 1;
 
   unsigned opts = TUNE(tn, REDUX_NT, 1) ? 1u : 0u;
@@ -2092,12 +2124,13 @@ static int pcols_call(GpuReduction *gr, GpuArray *d0, const GpuArray *s0, unsign
   p.units = (int64_t)J;
   p.nsplit = (int)G;
   p.fused = 1;
+  p.router = (int64_t)O;
   launch_rec rec;
   rec.k1 = &var->pcols;
-  rec.groups = G;
-  rec.fused = true;
-  rec.pi_off = (G * F * accsz + 255) & ~(size_t)255;
-  rec.need = rec.pi_off + 16;
+  rec.groups = O * G;
+  rec.fused = O == 1;
+  rec.pi_off = O == 1 ? (G * F * accsz + 255) & ~(size_t)255 : 0;
+  rec.need = O == 1 ? rec.pi_off + 16 : 0;
   const src_view src = {s0, (const int64_t *)s0->strides};
   if (noalloc && rec.need > ga_static_scratch_bytes)
     return ga_err_fmt(ctx->err, GA_XLARGE_ERROR,

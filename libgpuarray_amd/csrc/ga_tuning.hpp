@@ -21,7 +21,7 @@
   X(REDUX_FOLD) X(REDUX_FOLD_BYTES) X(REDUX_FOLD_MIN_BYTES) X(REDUX_FOLD_SLAB_MIN_BYTES) X(REDUX_FUSED) \
   X(REDUX_FUSED_COL_FEW) X(REDUX_FUSED_COL_PIECE) X(REDUX_FUSED_COL_SPLITS) \
   X(REDUX_FUSED_FEW) X(REDUX_FUSED_PIECE) X(REDUX_G) X(REDUX_GROUPS_PER_CU) X(REDUX_INFLIGHT) X(REDUX_INTERLEAVE) \
-  X(REDUX_L) X(REDUX_LANE_BYTES) X(REDUX_LIGHT) X(REDUX_LO) X(REDUX_MIN_PER_CU) X(REDUX_MEMO) X(REDUX_PCOLS) X(REDUX_PCOLS_PER_CU) X(REDUX_PCOLS_COL_BYTES) X(REDUX_PCOLS_MAX_PARTIALS) X(ELEMWISE_MEMO) X(ELEMWISE_TPAIRS) \
+  X(REDUX_L) X(REDUX_LANE_BYTES) X(REDUX_LIGHT) X(REDUX_LO) X(REDUX_MIN_PER_CU) X(REDUX_MEMO) X(REDUX_PCOLS) X(REDUX_PCOLS_PER_CU) X(REDUX_PSLABS) X(REDUX_PSLABS_MAX_BYTES) X(REDUX_PSLABS_MIN_SLABS) X(REDUX_PCOLS_COL_BYTES) X(REDUX_PCOLS_MAX_PARTIALS) X(ELEMWISE_MEMO) X(ELEMWISE_TPAIRS) \
   X(REDUX_MIN_UNITS) X(REDUX_NT) X(REDUX_NT_LINES) X(REDUX_OUTER_FIRST) X(REDUX_RB) X(REDUX_RPW) X(REDUX_SPLIT_MAJOR_MIN) \
   X(REDUX_SROWS) X(REDUX_SROWS_MAX_BYTES) X(REDUX_SROWS_MIN_BYTES) X(REDUX_SROWS_MIN_ROWS) \
   X(REDUX_TAIL) X(REDUX_TOUCH) X(REDUX_TROWS) X(REDUX_TROWS_DIRECT) X(REDUX_TROWS_MAX_BYTES) \

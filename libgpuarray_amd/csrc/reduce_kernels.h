@@ -123,7 +123,8 @@ struct rd_plan {
                     * launch's groups, rounded down to a multiple of 8 */
   ga_long upb;     /* work per split: units (row) or elements (col) */
   ga_long gx;      /* redux_col: groups along the inner free dim */
-  ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates */
+  ga_long router;  /* redux_row with RD_LO > 1: count of outer reduced coordinates;
+                    * redux_pcols: the number of slabs when more than one */
   ga_int nf, nr, nsplit, split_major;   /* split_major: layout of redux_col's partials */
   ga_int rising, fused;   /* rising: the flattened index grows with the position in the
                            * reduced range, and the range has fewer than 2^31 positions;
@@ -1415,7 +1416,11 @@ redux_trows(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
  * of a group meet in LDS, F of them come out per group, and the group that
  * counts in last (p.nsplit groups, one counter) combines the groups'
  * partials and writes the outputs: one launch.  For operations whose result
- * does not depend on how the elements are grouped. */
+ * does not depend on how the elements are grouped.
+ * With p.router > 1 the source is that many such arrays one behind the other
+ * (slabs: a middle run of reduced dims under kept ones), whole chunks each;
+ * with one group per slab (p.nsplit == 1) a group's F values are the slab's
+ * outputs, and nothing is left or counted. */
 #define RD_PVN (16 / RD_ELSZ0)
 static __device__ inline rd_acc rd_pacc(const RD_ACC_T v) {
   rd_acc a = rd_neutral();
@@ -1475,13 +1480,18 @@ redux_pcols(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
   const int rem = (int)((bytes & 15) / RD_ELSZ0);           /* elements of a last, partial chunk */
   const char *base[RD_NSRC];
   RD_SRC_BASES(base);
-  const rd_tchunk_t *src = (const rd_tchunk_t *)base[0];
+  /* p.router > 1: that many dense arrays (slabs) of p.rtotal rows one behind
+   * the other, whole chunks each, G groups per slab; the outputs of slab s are
+   * the rows s F ... s F + F - 1 of the result */
+  const ga_long slab = p.router > 1 ? (ga_long)(GID_0 / G) : 0;
+  const unsigned gi = (unsigned)((ga_long)GID_0 - slab * G);
+  const rd_tchunk_t *src = (const rd_tchunk_t *)base[0] + slab * full;
 
   rd_acc acc[RD_PVN];
 #pragma unroll
   for (int v = 0; v < RD_PVN; v++) acc[v] = rd_neutral();
   if (LID_0 < L) {
-    const ga_long c0 = (ga_long)GID_0 * L * J + LID_0;
+    const ga_long c0 = (ga_long)gi * L * J + LID_0;
     for (ga_long j = 0; j < J; j += RD_U) {
       rd_tchunk_t c[RD_U];
       if (j + RD_U <= J && c0 + (j + RD_U - 1) * L < full) {
@@ -1513,23 +1523,34 @@ redux_pcols(RD_SRC_PARAMS, char *__restrict__ d0, const ga_size d0_off, char *__
   local_barrier();
   /* a group's chunks start at a multiple of L chunks, a whole number of kept
    * rows: accumulator v of lane l belongs to output (l RD_PVN + v) mod F */
+  if (G == 1u) {
+    /* one group per slab: its F values are the slab's outputs (no partials, no counter) */
+    rd_pcols_fold(F, L * RD_PVN / F, meet,
+                  [&](const unsigned at) { return stage[at]; },
+                  [&](const unsigned k, const rd_acc a) {
+                    ga_long so[RD_NSRC], d0o, d1o;
+                    rd_row_offsets(p, slab * F + k, so, &d0o, &d1o);
+                    rd_write(a, d0 + d0_off, d0o, d1 + d1_off, d1o);
+                  });
+    return;
+  }
   rd_pcols_fold(F, L * RD_PVN / F, meet,
                 [&](const unsigned at) { return stage[at]; },
                 [&](const unsigned k, const rd_acc a) { rd_publish_partial(a, part_v, part_i, (ga_long)GID_0 * F + k); });
   rd_stores_done();   /* every lane that left partials */
   local_barrier();
-  if (LID_0 == 0) last_piece = rd_count_in(done, G) ? 1u : 0u;
+  if (LID_0 == 0) last_piece = rd_count_in(done + slab, G) ? 1u : 0u;
   local_barrier();
   if (!last_piece) return;
   rd_before_loads();
   rd_pcols_fold(F, G, meet,
-                [&](const unsigned at) { return rd_fetch_partial(part_v, part_i, (ga_long)at).v; },
+                [&](const unsigned at) { return rd_fetch_partial(part_v, part_i, slab * G * F + (ga_long)at).v; },
                 [&](const unsigned k, const rd_acc a) {
                   ga_long so[RD_NSRC], d0o, d1o;
-                  rd_row_offsets(p, (ga_long)k, so, &d0o, &d1o);
+                  rd_row_offsets(p, slab * F + k, so, &d0o, &d1o);
                   rd_write(a, d0 + d0_off, d0o, d1 + d1_off, d1o);
                 });
-  if (LID_0 == 0) rd_count_reset(done);
+  if (LID_0 == 0) rd_count_reset(done + slab);
 }
 #endif   /* RD_PCOLS */
 

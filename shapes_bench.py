@@ -155,6 +155,8 @@ def reduction_cases():
         ("max", f, (64, 262144), (1,), None, None, "64 MB of rows in a few pieces each, one launch"),
         ("sum", f, (256, 2048, 7, 7), (0, 2, 3), None, None, "bias gradient of a convolution, 7 x 7 maps: leading dims first"),
         ("sum", f, (64, 16384, 8, 8), (0, 2, 3), None, None, "the same on 256 MiB"),
+        ("sum", f, (10922, 512, 12), (1,), None, None, "middle axis under many small slabs: a group per slab"),
+        ("sum", f, (655, 512, 200), (1,), None, None, "the same, slabs of 400 KiB"),
     ]
 
 

@@ -1373,6 +1373,52 @@ def test_a_run_of_middle_axes_over_short_kept_rows_is_folded_per_slab(ctx, knobs
     assert not np.asarray(wide)[:, :, [0, 2]].any()
 
 
+@pytest.mark.parametrize("slabs", [1, 0])
+def test_a_middle_run_of_axes_under_many_small_slabs(ctx, knobs, slabs):
+    """(O, R, F) reduced over its middle run with many slabs of a few KiB to a
+    few hundred and short kept rows: one group walks a whole slab as one run
+    of 16-byte chunks and writes the slab's F outputs itself (REDUX_PSLABS; 0:
+    the column kernel).  Kept rows of 3 to 100 elements, 4- and 8-byte and
+    half elements, slabs whose chunk count is and is not a multiple of the
+    active lanes, two reduced dims, a strided destination; every operation
+    that may be regrouped, against NumPy."""
+    knobs(REDUX_PSLABS=slabs, REDUX_FOLD_MIN_BYTES=1)
+    rng = np.random.default_rng(5300 + slabs)
+    cases = (((600, 512, 12), (1,)), ((1000, 256, 30), (1,)), ((520, 100, 33), (1,)), ((512, 7, 64, 20), (1, 2)),
+             ((700, 64, 100), (1,)), ((2048, 344, 3), (1,)), ((513, 1024, 5), (1,)), ((16, 40, 300, 4, 6), (2,)))
+    every = ("float32", "int32", "float16", "float64")
+    for ci, (shape, axes) in enumerate(cases):
+        for dt in (every if ci < 2 else every[ci % 2::2]):
+            host = rng.integers(-3, 4, size=shape).astype(dt)
+            g = gpuarray.array(host, context=ctx)
+            kept = tuple(d for i, d in enumerate(shape) if i not in axes)
+            odt = "int64" if dt == "int32" else ("float32" if dt == "float16" else dt)
+            got = np.asarray(R.sum(g, axis=axes, dtype=odt))
+            assert got.shape == kept
+            assert np.array_equal(got, host.sum(axis=axes, dtype=np.int64).astype(got.dtype)), (shape, dt, "sum")
+            for name, npf in (("all", np.all), ("any", np.any)):
+                got = np.asarray(R._reduce_named(g, name, np.dtype("bool"), axis=axes))
+                assert np.array_equal(got, npf(host, axis=axes)), (shape, dt, name)
+            if dt == "int32":
+                for name, npf in (("max", np.max), ("min", np.min)):
+                    assert np.array_equal(np.asarray(getattr(R, name)(g, axis=axes)), npf(host, axis=axes)), (shape, dt, name)
+                got = np.asarray(R._reduce_named(g, "xor", np.dtype(dt), axis=axes))
+                assert np.array_equal(got, np.bitwise_xor.reduce(host, axis=axes)), (shape, dt, "xor")
+            else:
+                v, i = R.maxandargmax(g, axis=axes[:1]) if len(axes) == 1 else (None, None)
+                if v is not None:   # keeps the order of the scan: the planned path, still right
+                    assert np.array_equal(np.asarray(v), host.max(axis=axes[0]))
+                    assert np.array_equal(np.asarray(i), host.argmax(axis=axes[0]))
+    # float sums to tolerance, a strided destination
+    host = rng.standard_normal((800, 300, 20)).astype(np.float32) + np.float32(0.5)
+    g = gpuarray.array(host, context=ctx)
+    wide = gpuarray.zeros((800, 20, 3), "float32", context=ctx)
+    ga.GpuReduction(ctx, "sum", "float32")(g, [1], d0=wide[:, :, 1])
+    x64 = host.astype(np.float64)
+    assert_sum_close(np.asarray(wide)[:, :, 1], x64.sum(axis=1), np.abs(x64).sum(axis=1))
+    assert not np.asarray(wide)[:, :, [0, 2]].any()
+
+
 @pytest.mark.parametrize("two_calls", [1, 0])
 def test_leading_and_short_trailing_axes_around_kept_ones(ctx, knobs, two_calls):
     """Per-channel reductions over (batch, channel, a small height x width):
