@@ -50,21 +50,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_configs.md (earlier rocprofv3 --pmc runs, matched by kernel text hash)"
 MEASURED_TRAFFIC = {
     # name: (kernel text hashes of one call joined by "+", HBM bytes per call)
-    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201253305),
-    "C2_transposed_broadcast_4096": ("d188ff564c901e86", 134371643),
-    "X_transpose_8192x8192": ("a8d106ba259ef190", 536631458),
-    "C3a_sum_axis1_8192x8192": ("c849fb35fcfbcaf5", 268766152),
-    "C4_maxandargmax_65536x1000": ("1df395b36785e211", 263825976),
-    "C5_fp16_sum_axes02": ("dbf534ae4bcff368+ee8b025d3b851384", 269706681),
-    "C5_int32_sum_axis1": ("2a54fab5cf973555", 538005639),
-    "C5_uint8_all_axis2": ("b5b1d85faeed0adf", 134384282),
-    "C5_uint8_any_axis2": ("51ab57408948c70f", 134384216),
-    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538665007),
-    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538658699),
-    "F4_dot_2x2^27_fused": ("45af0a52784be32b", 1073847945),
-    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+9b3865c7d7aef2c6", 2146742579),
-    "elem_2^28": ("712fba8f0b8a6108", 3219572181),
-    "sum_2^28": ("9b3865c7d7aef2c6", 1073797889),
+    "C1_elemwise_2^24": ("712fba8f0b8a6108", 201252087),
+    "C2_transposed_broadcast_4096": ("d188ff564c901e86", 134378715),
+    "X_transpose_8192x8192": ("a8d106ba259ef190", 536642099),
+    "C3a_sum_axis1_8192x8192": ("e5f7f26dacba7629", 268765987),
+    "C4_maxandargmax_65536x1000": ("89789767af7d992d", 263859662),
+    "C5_fp16_sum_axes02": ("23389c3ca6d59214+acb367d638b58138", 269706636),
+    "C5_int32_sum_axis1": ("dc897e80b02e8b67", 538005539),
+    "C5_uint8_all_axis2": ("6cc909296d81cd49", 134384345),
+    "C5_uint8_any_axis2": ("8de2df4cbd2103d9", 134384275),
+    "F2_take1_65536x1024_rows": ("387e1f6257b6354e", 538655430),
+    "F2_take1_65536x1024_rows_unchecked": ("387e1f6257b6354e", 538651678),
+    "F4_dot_2x2^27_fused": ("e3c066d4d32a9eed", 1073848145),
+    "F4_dot_2x2^27_two_pass": ("4e9896a5dfc469a8+dae530aa9febdb16", 2146727490),
+    "elem_2^28": ("712fba8f0b8a6108", 3219540124),
+    "sum_2^28": ("dae530aa9febdb16", 1073797990),
 }
 
 
