@@ -1483,11 +1483,12 @@ class reduction_call {
     // three groups: (419430, 160) floats 51.6 -> 44.6 us (65 -> 75 % of peak),
     // (209715, 320) 47.6 -> 44.1, (174762, 384) 48.4 -> 44.9; over the middle
     // axis of (64, 4096, 320) 58.6 -> 52.0 (71 -> 81 %), of (64, 4096, 160)
-    // 39.4 -> 29.1, of (64, 8192, 72) 32.0 -> 28.4.  Up to 70 % of the lanes
-    // busy: with 200 kept floats of 256 two groups are ahead, 67.7 against 62.3 %
-    // of peak over axis 0 of (335544, 200); with 192 the two are even.
+    // 39.4 -> 29.1, of (64, 8192, 72) 32.0 -> 28.4.  Up to 80 % of the lanes
+    // busy; at 78 % the shapes disagree: over axis 0 of (223696, 300), 300 kept
+    // floats of 384, three groups 74 % of peak and two 66, of (335544, 200), 200
+    // of 256, three 62 and two 68; with 192 of 256 the two are even.
     const double lanes_used = (double)fin / (double)(p.gx * (int64_t)(CX * CV));
-    const bool idle_lanes = light && CV > 1 && lanes_used <= 0.7 && TUNE(tn, REDUX_COL_IDLE, 1) != 0;
+    const bool idle_lanes = light && CV > 1 && lanes_used <= 0.8 && TUNE(tn, REDUX_COL_IDLE, 1) != 0;
     const int64_t target = ncu * (int64_t)TUNE(tn, REDUX_GROUPS_PER_CU, CV > 1 ? (light && !idle_lanes ? 2 : 3) : 8);
     if (base_groups < target && rtotal >= 256) {
       nsplit = (target + base_groups - 1) / base_groups;
