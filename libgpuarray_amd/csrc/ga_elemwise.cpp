@@ -1639,6 +1639,9 @@ class strided_call {
 
   void find_transposed_operands() {
     // Transposed operands: small stride on some outer dim, large on x.
+    // (from 12 elements along that dim on: out = in.T of (N, 13) floats 470 us with
+    // single elements per lane, 222 through tiles, of (N, 15) 539 / 200; of (N, 11)
+    // 395 / 436, of (N, 8) 299 / 341)
     if (nd >= 2 && dims[nd - 1] >= 16) {
       // candidate y axis: the outer dim on which most arrays have their
       // smallest non-zero stride
@@ -1651,7 +1654,7 @@ class strided_call {
         size_t bs = sx;
         for (unsigned j = 0; j + 1 < nd; j++) {
           size_t sj = sabs(strs[k][j]);
-          if (sj != 0 && sj < bs && sj <= 4 * elsz[k] && dims[j] >= 16) { bs = sj; b = (int)j; }
+          if (sj != 0 && sj < bs && sj <= 4 * elsz[k] && dims[j] >= (size_t)TUNE(tn, ELEMWISE_TMIN, 12)) { bs = sj; b = (int)j; }
         }
         best[k] = b;
         if (b >= 0) votes[b]++;
@@ -1917,6 +1920,20 @@ class strided_call {
         // 15.3 / 14.8, 1024 x 1024 4.2 / 4.2
         const size_t min128 = TUNE(tn, ELEMWISE_TTILE_MIN, ga_hip_numprocs(ctx) / 2);
         tile = (tiles128 >= min128 && lds128 <= 80 * 1024) ? 128 : 64;
+        // A narrow plane - (N, 48) taken as its transpose - leaves most of a large
+        // tile empty: the small one where it is filled better by a tenth and more.
+        // out = in.T of 256 MiB of floats, large / small tiles: rows of 20
+        // 232 / 147 us (29 / 46 % of peak), of 33 171 / 116, of 48 125 / 103, of 49
+        // 138 / 105, of 130 117 / 104; of 100 101 / 118 and of 196 107 / 114 fill
+        // both alike and keep the large one.
+        if (tile == 128 && TUNE(tn, ELEMWISE_TTILE_FILL, 1) != 0) {
+          auto fill = [&](size_t t) {
+            const double fx = (double)dims[nd - 1] / (double)((dims[nd - 1] + t - 1) / t * t);
+            const double fy = (double)dims[nd - 2] / (double)((dims[nd - 2] + t - 1) / t * t);
+            return fx * fy;
+          };
+          if (fill(64) > fill(128) + 0.1) tile = 64;
+        }
         const unsigned long ft = TUNE(tn, ELEMWISE_TTILE, 0);
         if (ft == 64 || (ft == 128 && lds128 <= 160 * 1024)) tile = (unsigned)ft;
         const size_t tiles = ((dims[nd - 1] + cols + tile - 1) / tile) * ((dims[nd - 2] + tile - 1) / tile);

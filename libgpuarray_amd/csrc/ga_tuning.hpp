@@ -15,7 +15,7 @@
   X(ALLOW_OTHER_ISA) X(ELEMWISE_BAND) X(ELEMWISE_FLAT_NT_MASK) X(ELEMWISE_GROUPS_PER_CU) \
   X(ELEMWISE_MIXED_ALIGN) X(ELEMWISE_NT) X(ELEMWISE_NT_LINES) X(ELEMWISE_NT_MASK) X(ELEMWISE_PAIRS) \
   X(ELEMWISE_PANEL) X(ELEMWISE_PERIODIC) X(ELEMWISE_PERIODIC_ROWLOAD) X(ELEMWISE_PERIODIC_VEC) X(ELEMWISE_LOOSE) X(ELEMWISE_LOOSE_MIN_BYTES) X(ELEMWISE_QUADS) X(ELEMWISE_SKEW) \
-  X(ELEMWISE_TILE) X(ELEMWISE_TTILE) X(ELEMWISE_TTILE_MIN) X(ELEMWISE_UNROLL) X(ELEMWISE_VEC4) \
+  X(ELEMWISE_TILE) X(ELEMWISE_TMIN) X(ELEMWISE_TTILE) X(ELEMWISE_TTILE_FILL) X(ELEMWISE_TTILE_MIN) X(ELEMWISE_UNROLL) X(ELEMWISE_VEC4) \
   X(ELEMWISE_ZMASK) X(FILL_KERNEL_MIN) X(MARK_EVENT_FLAGS) X(MOVE_KERNEL_MIN) X(REDUX_BALANCE) X(REDUX_COLVEC) \
   X(REDUX_COL_BALANCE) X(REDUX_COL_CVMAX) X(REDUX_COL_FAR) X(REDUX_COL_IDLE) X(REDUX_COL_LOOSE) X(REDUX_COL_LOOSE_MIN_BYTES) X(REDUX_COL_ROWS) X(REDUX_COL_U) X(REDUX_FAST8) \
   X(REDUX_FOLD) X(REDUX_FOLD_BYTES) X(REDUX_FOLD_MIN_BYTES) X(REDUX_FOLD_SLAB_MIN_BYTES) X(REDUX_FUSED) \

@@ -598,6 +598,34 @@ def test_tile_windows_follow_result_rows_off_the_64_byte_blocks(ctx, knobs, tile
     assert np.array_equal(read_root(groot, root), want)
 
 
+@pytest.mark.parametrize("fill,tmin", [(1, 12), (0, 16), (1, 2)])
+def test_transposed_operands_of_narrow_planes(ctx, knobs, fill, tmin):
+    """(N, f) taken as its transpose with f from 3 to 130: the small tile where
+    it is filled better than the large one (ELEMWISE_TTILE_FILL), tiles at all
+    from ELEMWISE_TMIN elements along the narrow dim on (below, single elements
+    per lane); also the other way round, a narrow result of a wide transposed
+    operand.  Floats and doubles, with a row operand; against NumPy, exact."""
+    knobs(ELEMWISE_TTILE_FILL=fill, ELEMWISE_TMIN=tmin, ELEMWISE_TTILE_MIN=1)
+    rng = np.random.default_rng(830 + tmin)
+    for dtype in ("float32", "float64"):
+        k = ga.GpuElemwise(ctx, "o = a + r", [arg("a", dtype, read=True), arg("r", dtype, read=True),
+                                               arg("o", dtype, write=True)])
+        draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
+        for n, f in ((5000, 3), (4096, 8), (3001, 12), (2500, 13), (6000, 15), (4000, 16), (3333, 20),
+                     (2048, 33), (2500, 48), (1999, 49), (1500, 100), (1111, 130)):
+            a = draw((n, f))
+            ga_ = gpuarray.array(a, context=ctx)
+            r = draw((1, n))
+            out = gpuarray.empty((f, n), dtype, context=ctx)
+            k(ga_.transpose(1, 0), gpuarray.array(r, context=ctx), out, broadcast=True)
+            assert np.array_equal(np.asarray(out), a.T + r), (dtype, n, f)
+            b = draw((f, n))
+            r2 = draw((1, f))
+            out2 = gpuarray.empty((n, f), dtype, context=ctx)
+            k(gpuarray.array(b, context=ctx).transpose(1, 0), gpuarray.array(r2, context=ctx), out2, broadcast=True)
+            assert np.array_equal(np.asarray(out2), b.T + r2), (dtype, n, f, "wide")
+
+
 @pytest.mark.parametrize("loose", [1, 0])
 @pytest.mark.parametrize("dtype", ["float32", "int32"])
 def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
