@@ -96,6 +96,18 @@ def main():
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 3, 0b011 << 16, 0b011))
     check("elemwise flat, two operands read through the flat index's coordinates, 3 dims",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 9, 3, 0, 0b011))
+    # narrow planes in registers: short extent in nd, the short dim in bit 1 of idx64, streaming in bit 2
+    check("elemwise narrow plane of 3 in registers: one operand with the short dim innermost, the rest chunked",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 14, 3, 0b100, 0b001 | (0b110 << 16)))
+    check("elemwise narrow plane of 11 in registers: the result with the short dim innermost, 64-bit offsets",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 14, 11, 0b011, 0b100 | (0b001 << 16)))
+    check("elemwise narrow plane of 8 in registers: operand through the LDS, result chunked on four-byte boundaries",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 14, 8, 0b11100, 0b001 | (0b110 << 16)))
+    check("elemwise narrow plane of 5 in registers: the result through the LDS, 64-bit offsets",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 14, 5, 0b01011, 0b100 | (0b011 << 16)))
+    iargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_FLOAT, 6))
+    check("elemwise narrow plane of 4 in registers: an array read and written through the LDS",
+          gen_e(b"", b"c = a + c", 2, iargs, 0, 14, 4, 0b01000, 0b10 | (0b01 << 16)))
     check("elemwise flat, 2 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 5, 0, 0, 0))
     check("elemwise flat, 4 adjacent chunks per lane", gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 6, 0, 0, 0))
     hargs = (ElemwiseArg * 2)(ElemwiseArg(b"src", GA_HALF, 2), ElemwiseArg(b"dst", GA_DOUBLE, 4))
@@ -201,7 +213,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "29 elementwise)" % (n + 20, m, t))
+          "34 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

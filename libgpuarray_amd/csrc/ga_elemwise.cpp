@@ -420,6 +420,258 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
   return s;
 }
 
+// ---- narrow planes in registers -------------------------------------------------
+// Same parameters as the strided kernel with two dims.  One of the two dims is
+// short (S, extent F <= 16, fixed in the text), the other long (L).  A lane
+// owns four adjacent positions along L and all F along S; a group 1024
+// positions along L.
+//  * The arrays in bmask have the short dim innermost: a lane's 4 F elements,
+//    and a group's 4096 F, lie one after the other in memory (stride of S one
+//    element, of L F elements: an (N, F) array taken as its transpose), on a
+//    16-byte boundary.  Those also in smask pass through the LDS: the group
+//    moves its piece of the array in 16-byte chunks, consecutive lanes on
+//    consecutive chunks, and a lane exchanges its own F chunks with the LDS
+//    (slots swizzled when F is a power of two: a lane's chunks are then a
+//    multiple of 8 slots from its neighbours').  The others are fetched or
+//    stored as the lane's own F chunks.
+//  * The arrays in cmask run along L with unit stride and move as one 16-byte
+//    chunk per position of S, side by side with the neighbouring lanes'; those
+//    also in umask through accesses that assume four-byte boundaries only.
+//  * Every other array one element at a time.
+// All arrays have four-byte elements.  The last lane of a row takes what exists
+// of its four positions one by one.
+std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsigned sd, unsigned bmask,
+                             unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask = 0,
+                             unsigned smask = 0) {
+  std::string s;
+  const char *I = idx64 ? "ga_ssize" : "ga_int";
+  const char *N = idx64 ? "ga_size" : "ga_uint";
+  const unsigned ld = 1 - sd;
+  const bool swz = (F & (F - 1)) == 0;
+  emit_header(ge, s);
+  if (umask) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  if (smask) s += swz ? "#define GA_SLOT(q) ((q) ^ (((q) >> 3) & 7u))\n" : "#define GA_SLOT(q) (q)\n";
+  s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0, const ga_size dim1";
+  ktypes.push_back(GA_SIZE);
+  ktypes.push_back(GA_SIZE);
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto in = [&](unsigned mask, size_t j) { return aidx[j] >= 0 && ((mask >> aidx[j]) & 1u); };
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset, const ga_ssize %s_str_0, const ga_ssize %s_str_1",
+              ctype(a.typecode), a.name.c_str(), a.name.c_str(), a.name.c_str(), a.name.c_str());
+      for (int t : {GA_BUFFER, GA_SIZE, GA_SSIZE, GA_SSIZE}) ktypes.push_back(t);
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n(void)ga_gx; (void)ga_ltx; (void)dim0; (void)dim1;\n";
+  ktypes.push_back(GA_UINT);
+  ktypes.push_back(GA_UINT);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n", a.name.c_str(), a.name.c_str(),
+            a.name.c_str());
+    if (in(smask, j)) appendf(s, "LOCAL_MEM ga_chunk16 %s_s[%u];\n", a.name.c_str(), 256 * F);
+  }
+  appendf(s, "const %s ga_l0 = (%s)GID_0 * 1024u;\n", N, N);
+  appendf(s, "const %s ga_l4 = ga_l0 + LID_0 * 4u;\n", N);
+  if (!smask) appendf(s, "if (ga_l4 >= (%s)dim%u) return;\n", N, ld);
+  appendf(s, "const bool ga_full = ga_l4 + 3u < (%s)dim%u;\n", N, ld);
+  // the four-byte words of a staged array that the group's piece holds
+  if (smask)
+    appendf(s, "const ga_uint ga_cnt = (ga_uint)((%s)dim%u - ga_l0 < 1024u ? (%s)dim%u - ga_l0 : 1024u) * %uu;\n", N, ld,
+            N, ld, F);
+  // registers of the block arrays (element e * F + y: position e along L, y along S)
+  // and of the chunked ones (element e of chunk y)
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (in(bmask, j)) appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r;\n", F, ctype(a.typecode), 4 * F, a.name.c_str());
+    else if (in(cmask, j)) appendf(s, "union { ga_chunk16 c; %s e[4]; } %s_r[%u];\n", ctype(a.typecode), a.name.c_str(), F);
+  }
+  auto elem_at = [&](const ge_arg &a, const std::string &y, const std::string &l) {
+    std::string e;
+    appendf(e, "*(GLOBAL_MEM %s *)(%s_b + ((%s)(%s) * (%s)%s_str_%u + (%s)(%s) * (%s)%s_str_%u))", ctype(a.typecode),
+            a.name.c_str(), I, y.c_str(), I, a.name.c_str(), sd, I, l.c_str(), I, a.name.c_str(), ld);
+    return e;
+  };
+  // byte address of the group's piece of a staged array, plus an expression in bytes
+  auto piece_at = [&](const ge_arg &a, const char *cast, const std::string &bytes) {
+    std::string e;
+    appendf(e, "(GLOBAL_MEM %s *)(%s_b + (%s)ga_l0 * (%s)%s_str_%u + (%s))", cast, a.name.c_str(), I, I,
+            a.name.c_str(), ld, bytes.c_str());
+    return e;
+  };
+  // loads
+  bool staged_in = false, staged_inout = false;
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array() || !a.reads()) continue;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    if (in(smask, j)) {
+      staged_in = true;
+      if (a.writes()) staged_inout = true;
+      for (unsigned h = 0; h < F; h++) {
+        appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
+        const std::string ptr = piece_at(a, "const ga_chunk16", "ga_q * 16u");
+        appendf(s, "if (ga_q * 4u + 3u < ga_cnt) %s_s[GA_SLOT(ga_q)] = %s(%s);\n", a.name.c_str(),
+                nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) "
+                   "((%s *)%s_s)[GA_SLOT(ga_q) * 4u + ga_e] = *(%s);\n",
+                ctype(a.typecode), a.name.c_str(), piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str());
+        s += "}\n";
+      }
+    } else if (in(bmask, j)) {
+      s += "if (ga_full) {\n";
+      for (unsigned h = 0; h < F; h++) {
+        std::string ptr;
+        appendf(ptr, "(GLOBAL_MEM const ga_chunk16 *)(%s_b + (%s)ga_l4 * (%s)%s_str_%u) + %u", a.name.c_str(), I, I,
+                a.name.c_str(), ld, h);
+        appendf(s, "%s_r.c[%u] = %s(%s);\n", a.name.c_str(), h, nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
+      }
+      s += "} else {\n";
+      for (unsigned e = 0; e < 4; e++)
+        for (unsigned y = 0; y < F; y++) {
+          char l[32], yy[16];
+          snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+          snprintf(yy, sizeof(yy), "%uu", y);
+          appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s_r.e[%u] = %s;\n", e, N, ld, a.name.c_str(), e * F + y,
+                  elem_at(a, yy, l).c_str());
+        }
+      s += "}\n";
+    } else if (in(cmask, j)) {
+      const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+      for (unsigned y = 0; y < F; y++) {
+        char yy[16];
+        snprintf(yy, sizeof(yy), "%uu", y);
+        std::string ptr;
+        appendf(ptr, "(GLOBAL_MEM const %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
+        appendf(s, "if (ga_full) %s_r[%u].c = %s(%s); else {\n", a.name.c_str(), y,
+                nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
+        for (unsigned e = 0; e < 4; e++) {
+          char l[32];
+          snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+          appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s_r[%u].e[%u] = %s;\n", e, N, ld, a.name.c_str(), y, e,
+                  elem_at(a, yy, l).c_str());
+        }
+        s += "}\n";
+      }
+    }
+  }
+  if (staged_in) {
+    s += "local_barrier();\n";
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!a.is_array() || !a.reads() || !in(smask, j)) continue;
+      for (unsigned h = 0; h < F; h++)
+        appendf(s, "%s_r.c[%u] = %s_s[GA_SLOT(LID_0 * %uu + %uu)];\n", a.name.c_str(), h, a.name.c_str(), F, h);
+    }
+  }
+  // the expression, position by position
+  for (unsigned y = 0; y < F; y++)
+    for (unsigned e = 0; e < 4; e++) {
+      char l[32], yy[16];
+      snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+      snprintf(yy, sizeof(yy), "%uu", y);
+      appendf(s, "if (ga_l4 + %uu < (%s)dim%u) {\n", e, N, ld);
+      for (size_t j = 0; j < ge->args.size(); j++) {
+        const ge_arg &a = ge->args[j];
+        if (!a.is_array()) continue;
+        std::string src;
+        if (in(bmask, j)) appendf(src, "%s_r.e[%u]", a.name.c_str(), e * F + y);
+        else if (in(cmask, j)) appendf(src, "%s_r[%u].e[%u]", a.name.c_str(), y, e);
+        else src = elem_at(a, yy, l);
+        emit_load(ge, s, a, src);
+      }
+      s += ge->expr;
+      s += ";\n";
+      for (size_t j = 0; j < ge->args.size(); j++) {
+        const ge_arg &a = ge->args[j];
+        if (!a.is_array() || !a.writes()) continue;
+        std::string dst;
+        if (in(bmask, j)) appendf(dst, "%s_r.e[%u]", a.name.c_str(), e * F + y);
+        else if (in(cmask, j)) appendf(dst, "%s_r[%u].e[%u]", a.name.c_str(), y, e);
+        else dst = elem_at(a, yy, l);
+        emit_store(ge, s, a, dst);
+      }
+      s += "}\n";
+    }
+  // stores of the results kept in registers
+  if (staged_inout) s += "local_barrier();\n";   // every lane has taken its chunks before the slots are written again
+  bool staged_out = false;
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array() || !a.writes() || !in(smask, j)) continue;
+    staged_out = true;
+    for (unsigned h = 0; h < F; h++)
+      appendf(s, "%s_s[GA_SLOT(LID_0 * %uu + %uu)] = %s_r.c[%u];\n", a.name.c_str(), F, h, a.name.c_str(), h);
+  }
+  if (staged_out) s += "local_barrier();\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array() || !a.writes()) continue;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    if (in(smask, j)) {
+      for (unsigned h = 0; h < F; h++) {
+        appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
+        const std::string ptr = piece_at(a, "ga_chunk16", "ga_q * 16u");
+        if (nt) appendf(s, "if (ga_q * 4u + 3u < ga_cnt) __builtin_nontemporal_store(%s_s[GA_SLOT(ga_q)], %s);\n",
+                        a.name.c_str(), ptr.c_str());
+        else appendf(s, "if (ga_q * 4u + 3u < ga_cnt) *(%s) = %s_s[GA_SLOT(ga_q)];\n", ptr.c_str(), a.name.c_str());
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) "
+                   "*(%s) = ((%s *)%s_s)[GA_SLOT(ga_q) * 4u + ga_e];\n",
+                piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str(), ctype(a.typecode), a.name.c_str());
+        s += "}\n";
+      }
+    } else if (in(bmask, j)) {
+      s += "if (ga_full) {\n";
+      for (unsigned h = 0; h < F; h++) {
+        std::string ptr;
+        appendf(ptr, "(GLOBAL_MEM ga_chunk16 *)(%s_b + (%s)ga_l4 * (%s)%s_str_%u) + %u", a.name.c_str(), I, I,
+                a.name.c_str(), ld, h);
+        if (nt) appendf(s, "__builtin_nontemporal_store(%s_r.c[%u], %s);\n", a.name.c_str(), h, ptr.c_str());
+        else appendf(s, "*(%s) = %s_r.c[%u];\n", ptr.c_str(), a.name.c_str(), h);
+      }
+      s += "} else {\n";
+      for (unsigned e = 0; e < 4; e++)
+        for (unsigned y = 0; y < F; y++) {
+          char l[32], yy[16];
+          snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+          snprintf(yy, sizeof(yy), "%uu", y);
+          appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s = %s_r.e[%u];\n", e, N, ld, elem_at(a, yy, l).c_str(),
+                  a.name.c_str(), e * F + y);
+        }
+      s += "}\n";
+    } else if (in(cmask, j)) {
+      const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+      for (unsigned y = 0; y < F; y++) {
+        char yy[16];
+        snprintf(yy, sizeof(yy), "%uu", y);
+        std::string ptr;
+        appendf(ptr, "(GLOBAL_MEM %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
+        if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store((%s)%s_r[%u].c, %s); else {\n", ct, a.name.c_str(), y, ptr.c_str());
+        else appendf(s, "if (ga_full) *(%s) = %s_r[%u].c; else {\n", ptr.c_str(), a.name.c_str(), y);
+        for (unsigned e = 0; e < 4; e++) {
+          char l[32];
+          snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+          appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s = %s_r[%u].e[%u];\n", e, N, ld, elem_at(a, yy, l).c_str(),
+                  a.name.c_str(), y, e);
+        }
+        s += "}\n";
+      }
+    }
+  }
+  s += "}\n";
+  return s;
+}
+
 // ---- strided kernel -------------------------------------------------------------
 // elem(dim0..dim{nd-1}, {data, byte offset, str_0..str_{nd-1} | scalar}...,
 //      ga_gx, ga_ltx)
@@ -1451,6 +1703,10 @@ class strided_call {
     describe_arrays();
     normalise_layout();
     if (is_one_dense_run()) return call_flat(ge, args, n, offs.data());
+    {
+      int err = GA_NO_ERROR;
+      if (narrow_plane_in_registers(err)) return err;
+    }
     find_transposed_operands();
     choose_offset_width();
     choose_vector_access();
@@ -1533,6 +1789,88 @@ class strided_call {
     ge->strp.resize(na);
     for (unsigned k = 0; k < na; k++) ge->strp[k] = strs[k].data();
     gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
+  }
+
+  // A plane with one short extent F (2 to 15) of four-byte elements where some
+  // array has the short dim innermost and another the long one - (N, F) taken as
+  // its transpose, or written as one: too narrow for tiles through the LDS, which
+  // F of 64 or 128 columns fill.  A lane takes four positions along the long dim
+  // and all F of the short one in registers (gen_narrow_block).  out = in.T of
+  // 256 MiB of floats, (N, F) -> (F, N), before / now in % of 8 TB/s: F = 2
+  // 54 / 73, 3 47 / 67, 4 37 / 70, 5 30 / 66, 7 25 / 67, 8 22 / 70, 11 17 / 63,
+  // 12 19 / 63, 13 30 / 63, 15 33 / 61; (F, N) -> (N, F): 2 29 / 81, 3 29 / 78,
+  // 5 37 / 74, 7 34 / 76, 9 32 / 74, 11 39 / 69, 13 32 / 69, 15 34 / 58.  16 and
+  // more fill a quarter of a small tile's rows and stay with the tiles (73 and
+  // 77 % against 62 and 77).  From 4096 positions on: below, either kernel takes
+  // the 4 us of a launch.
+  bool narrow_plane_in_registers(int &err) {
+    const unsigned long fmax = TUNE(tn, ELEMWISE_NARROW, 15);
+    if (fmax == 0 || nd != 2 || na > 31) return false;
+    const unsigned sd = dims[0] <= dims[1] ? 0 : 1, ld = 1 - sd;
+    const size_t F = dims[sd], L = dims[ld];
+    if (F < 2 || F > fmax || F > 16 || L < TUNE(tn, ELEMWISE_NARROW_MIN, 4096)) return false;
+    if (ge->flags & GE_CONVERT_F16) return false;
+    // a short extent of whole quads innermost in the result: four elements per
+    // lane of the strided kernel are a chunk of the result and coalesced single
+    // elements of the operands (out = in.T of (4, N) 78 against 75 % of peak, of
+    // (8, N) 79 against 74)
+    if (sd == 1 && F % 4 == 0 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
+    unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0;
+    bool crossed = false;   // some array runs along the long dim and moves along the short one
+    const unsigned long stage = TUNE(tn, ELEMWISE_NARROW_LDS, 2);   // 1: staged when read, 2: when written
+    size_t lds = 0;
+    {
+      unsigned k = 0;
+      for (size_t i = 0; i < ge->args.size(); i++) {
+        if (!ge->args[i].is_array()) continue;
+        if (elsz[k] != 4 || offs[k] % 4 != 0) return false;
+        const bool base16 = offs[k] % 16 == 0;
+        if (base16 && strs[k][sd] == 4 && strs[k][ld] == (ssize_t)(4 * F)) {
+          bmask |= 1u << k;
+          const bool want = (ge->args[i].reads() ? (stage & 1) : 0) || (ge->args[i].writes() ? (stage & 2) : 0);
+          if (want && lds + 4096 * F <= 64 * 1024) {
+            smask |= 1u << k;
+            lds += 4096 * F;
+          }
+        } else if (strs[k][ld] == 4 && strs[k][sd] % 4 == 0) {
+          cmask |= 1u << k;
+          if (strs[k][sd] != 0) crossed = true;
+          if (!base16 || strs[k][sd] % 16 != 0) umask |= 1u << k;
+        }
+        k++;
+      }
+    }
+    if (bmask == 0 || !crossed) return false;
+    // arrays that take part once, whole, are streamed (the rest, broadcast or
+    // overlapping, stays cacheable)
+    {
+      const unsigned long m = TUNE(tn, ELEMWISE_NARROW_NT, 3);
+      if (m & 1) nt |= cmask;
+      if (m & 2) nt |= smask;
+      if (m & 4) nt |= bmask;
+      for (unsigned k = 0; k < na; k++)
+        if (strs[k][sd] == 0) nt &= ~(1u << k);
+    }
+    choose_offset_width();
+    gx = (L + 1023) / 1024;
+    groups = gx;
+    ltx = 0;
+    if (groups > 0x7fffffffull) return false;
+    char key[64];
+    snprintf(key, sizeof(key), "n%zu:%u:%d:%x:%x:%x:%x:%x", F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask, smask);
+    auto it = ge->k_strided.find(key);
+    if (it != ge->k_strided.end()) {
+      kernel = &it->second;
+    } else {
+      std::vector<int> ktypes;
+      std::string src = gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask);
+      GpuKernel nk = {nullptr, nullptr};
+      err = build_kernel(ge, &nk, src, ktypes);
+      if (err != GA_NO_ERROR) return true;
+      kernel = &ge->k_strided.emplace(key, nk).first->second;
+    }
+    err = launch();
+    return true;
   }
 
   bool is_one_dense_run() const {
@@ -2103,6 +2441,13 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // (and its bits 16.. the mask of those that fetch a chunk inside one row with one load on four-byte boundaries)
   if (strided == 9)
     return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64 & 0xffffu, (unsigned)idx64 >> 16).c_str());
+  // 14: a narrow plane in registers: nd carries the short extent, idx64 bit 0 the offsets' width, bit 1 the
+  // short dim, bit 2 streaming accesses, bit 3 the first kind of arrays through the LDS, bit 4 the second kind
+  // on four-byte boundaries; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
+  if (strided == 14)
+    return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd, ((unsigned)idx64 >> 1) & 1u, tmask & 0xffffu, tmask >> 16,
+                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
+                                   (idx64 & 8) ? tmask & 0xffffu : 0u).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 && strided != 13 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu

@@ -102,6 +102,11 @@ def elemwise_cases():
          [("a", f, (1 << 28,), None)], (1 << 28,), f),
         ("(1335, 50257) + (1, 50257), a bias row off the 16-byte chunks", "o = a + b",
          [("a", f, (1335, 50257), None), ("b", f, (1, 50257), None)], (1335, 50257), f),
+        ("a.T, (22369621, 3) -> (3, 22369621) (interleaved channels to planes)", "o = a",
+         [("a", f, (22369621, 3), T(1, 0))], (3, 22369621), f),
+        ("a.T, (3, 22369621) -> (22369621, 3) (planes to interleaved channels)", "o = a",
+         [("a", f, (3, 22369621), T(1, 0))], (22369621, 3), f),
+        ("a.T, (6710886, 10) -> (10, 6710886)", "o = a", [("a", f, (6710886, 10), T(1, 0))], (10, 6710886), f),
     ]
 
 

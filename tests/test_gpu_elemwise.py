@@ -603,9 +603,10 @@ def test_transposed_operands_of_narrow_planes(ctx, knobs, fill, tmin):
     """(N, f) taken as its transpose with f from 3 to 130: the small tile where
     it is filled better than the large one (ELEMWISE_TTILE_FILL), tiles at all
     from ELEMWISE_TMIN elements along the narrow dim on (below, single elements
-    per lane); also the other way round, a narrow result of a wide transposed
+    per lane), with the kernel that holds very narrow planes in registers
+    switched off; also the other way round, a narrow result of a wide transposed
     operand.  Floats and doubles, with a row operand; against NumPy, exact."""
-    knobs(ELEMWISE_TTILE_FILL=fill, ELEMWISE_TMIN=tmin, ELEMWISE_TTILE_MIN=1)
+    knobs(ELEMWISE_TTILE_FILL=fill, ELEMWISE_TMIN=tmin, ELEMWISE_TTILE_MIN=1, ELEMWISE_NARROW=0)
     rng = np.random.default_rng(830 + tmin)
     for dtype in ("float32", "float64"):
         k = ga.GpuElemwise(ctx, "o = a + r", [arg("a", dtype, read=True), arg("r", dtype, read=True),
@@ -624,6 +625,57 @@ def test_transposed_operands_of_narrow_planes(ctx, knobs, fill, tmin):
             out2 = gpuarray.empty((n, f), dtype, context=ctx)
             k(gpuarray.array(b, context=ctx).transpose(1, 0), gpuarray.array(r2, context=ctx), out2, broadcast=True)
             assert np.array_equal(np.asarray(out2), b.T + r2), (dtype, n, f, "wide")
+
+
+@pytest.mark.parametrize("lds,nt,quads", [(2, 3, 0), (3, 0, 1), (0, 7, 1), (1, 1, 0)])
+def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads):
+    """(N, f) with f from 2 to 15 taken as its transpose, and written as one: a
+    lane holds four positions of the long dim by all f of the short one
+    (ELEMWISE_NARROW; the arrays with the short dim innermost directly or through
+    the LDS, ELEMWISE_NARROW_LDS; the others as 16-byte chunks, on four-byte
+    boundaries when N is no multiple of four).  Long extents of whole and cut
+    groups and lanes, a row operand, an array read and written, a result inside a
+    larger buffer whose rows start off the 16-byte boundaries; floats and 32-bit
+    integers against NumPy, exact."""
+    knobs(ELEMWISE_NARROW_LDS=lds, ELEMWISE_NARROW_NT=nt, ELEMWISE_NARROW_QUADS=quads, ELEMWISE_NARROW_MIN=1024)
+    rng = np.random.default_rng(900 + lds)
+    for dtype in ("float32", "int32"):
+        k = ga.GpuElemwise(ctx, "o = a + r", [arg("a", dtype, read=True), arg("r", dtype, read=True),
+                                               arg("o", dtype, write=True)])
+        kio = ga.GpuElemwise(ctx, "o = o - a", [arg("a", dtype, read=True), arg("o", dtype, read=True, write=True)])
+        draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
+        for f in range(2, 16):
+            for n in ((1024, 4099, 100001) if f % 3 else (2048, 5003, 8190)):
+                a = draw((n, f))
+                r = draw((1, n))
+                out = gpuarray.empty((f, n), dtype, context=ctx)
+                k(gpuarray.array(a, context=ctx).transpose(1, 0), gpuarray.array(r, context=ctx), out, broadcast=True)
+                assert np.array_equal(np.asarray(out), a.T + r), (dtype, n, f)
+                b = draw((f, n))
+                r2 = draw((1, f))
+                out2 = gpuarray.empty((n, f), dtype, context=ctx)
+                k(gpuarray.array(b, context=ctx).transpose(1, 0), gpuarray.array(r2, context=ctx), out2, broadcast=True)
+                assert np.array_equal(np.asarray(out2), b.T + r2), (dtype, n, f, "narrow result")
+                o3 = draw((n, f))
+                g3 = gpuarray.array(o3, context=ctx)
+                kio(gpuarray.array(b, context=ctx).transpose(1, 0), g3)
+                assert np.array_equal(np.asarray(g3), o3 - b.T), (dtype, n, f, "read and written")
+        # the wide result inside a larger buffer: rows one element into pitches of n + 3
+        n, f = 6001, 5
+        a = draw((n, f))
+        root = np.zeros((f, n + 3), dtype)
+        go, groot = to_gpu_view(root[:, 1:n + 1], ctx)
+        kc = ga.GpuElemwise(ctx, "o = a", [arg("a", dtype, read=True), arg("o", dtype, write=True)])
+        kc(gpuarray.array(a, context=ctx).transpose(1, 0), go)
+        want = root.copy()
+        want[:, 1:n + 1] = a.T
+        assert np.array_equal(read_root(groot, root), want), dtype
+        # the narrow operand as a view that starts off the 16-byte boundaries: the other kernels
+        aroot = draw((n + 1, f))
+        gv, _ = to_gpu_view(aroot[1:], ctx)
+        out = gpuarray.empty((f, n), dtype, context=ctx)
+        kc(gv.transpose(1, 0), out)
+        assert np.array_equal(np.asarray(out), aroot[1:].T), dtype
 
 
 @pytest.mark.parametrize("loose", [1, 0])
