@@ -92,7 +92,8 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * one group of two elements per lane (8-byte types, no transposed operand),
  * 11 to 13 variants of 4 and 3 for rows off the 64-byte blocks and for
  * four-byte elements on any layout, 14 a plane of two dims with a short
- * extent held in registers: nd carries the short extent (2 to 16), idx64 the
+ * extent held in registers: nd carries the short extent (2 to 16; plus 256
+ * for three dims, planes one after the other), idx64 the
  * width of the offsets in bit 0, which of the two dims is the short one in bit
  * 1, the streaming hint in bit 2, the LDS for the first kind of arrays in bit
  * 3 and four-byte boundaries for the second kind in bit 4; tmask bits 0..15

@@ -421,7 +421,8 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 }
 
 // ---- narrow planes in registers -------------------------------------------------
-// Same parameters as the strided kernel with two dims.  One of the two dims is
+// Same parameters as the strided kernel with two or three dims (with three, the
+// first counts planes, ga_gx groups each).  One of the last two dims is
 // short (S, extent F <= 16, fixed in the text), the other long (L).  A lane
 // owns four adjacent positions along L and all F along S; a group 1024
 // positions along L.
@@ -442,18 +443,21 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 // of its four positions one by one.
 std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsigned sd, unsigned bmask,
                              unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask = 0,
-                             unsigned smask = 0) {
+                             unsigned smask = 0, unsigned nd = 2) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
-  const unsigned ld = 1 - sd;
+  const unsigned ld = sd == nd - 1 ? nd - 2 : nd - 1;
   const bool swz = (F & (F - 1)) == 0;
   emit_header(ge, s);
   if (umask) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
   if (smask) s += swz ? "#define GA_SLOT(q) ((q) ^ (((q) >> 3) & 7u))\n" : "#define GA_SLOT(q) (q)\n";
-  s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0, const ga_size dim1";
+  s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
   ktypes.push_back(GA_SIZE);
-  ktypes.push_back(GA_SIZE);
+  for (unsigned d = 1; d < nd; d++) {
+    appendf(s, ", const ga_size dim%u", d);
+    ktypes.push_back(GA_SIZE);
+  }
   std::vector<int> aidx(ge->args.size(), -1);
   {
     int k = 0;
@@ -463,9 +467,13 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
   auto in = [&](unsigned mask, size_t j) { return aidx[j] >= 0 && ((mask >> aidx[j]) & 1u); };
   for (const ge_arg &a : ge->args) {
     if (a.is_array()) {
-      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset, const ga_ssize %s_str_0, const ga_ssize %s_str_1",
-              ctype(a.typecode), a.name.c_str(), a.name.c_str(), a.name.c_str(), a.name.c_str());
-      for (int t : {GA_BUFFER, GA_SIZE, GA_SSIZE, GA_SSIZE}) ktypes.push_back(t);
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset", ctype(a.typecode), a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+      for (unsigned d = 0; d < nd; d++) {
+        appendf(s, ", const ga_ssize %s_str_%u", a.name.c_str(), d);
+        ktypes.push_back(GA_SSIZE);
+      }
     } else {
       appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
       ktypes.push_back(a.typecode);
@@ -474,14 +482,18 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
   s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n(void)ga_gx; (void)ga_ltx; (void)dim0; (void)dim1;\n";
   ktypes.push_back(GA_UINT);
   ktypes.push_back(GA_UINT);
+  // three dims: planes one after the other, ga_gx groups each
+  if (nd == 3) s += "const ga_uint ga_o = GID_0 / ga_gx;\nconst ga_uint ga_pc = GID_0 - ga_o * ga_gx;\n";
+  else s += "const ga_uint ga_pc = GID_0;\n";
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
     appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n", a.name.c_str(), a.name.c_str(),
             a.name.c_str());
+    if (nd == 3) appendf(s, "%s_b += (%s)ga_o * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
     if (in(smask, j)) appendf(s, "LOCAL_MEM ga_chunk16 %s_s[%u];\n", a.name.c_str(), 256 * F);
   }
-  appendf(s, "const %s ga_l0 = (%s)GID_0 * 1024u;\n", N, N);
+  appendf(s, "const %s ga_l0 = (%s)ga_pc * 1024u;\n", N, N);
   appendf(s, "const %s ga_l4 = ga_l0 + LID_0 * 4u;\n", N);
   if (!smask) appendf(s, "if (ga_l4 >= (%s)dim%u) return;\n", N, ld);
   appendf(s, "const bool ga_full = ga_l4 + 3u < (%s)dim%u;\n", N, ld);
@@ -1802,19 +1814,24 @@ class strided_call {
   // 5 37 / 74, 7 34 / 76, 9 32 / 74, 11 39 / 69, 13 32 / 69, 15 34 / 58.  16 and
   // more fill a quarter of a small tile's rows and stay with the tiles (73 and
   // 77 % against 62 and 77).  From 4096 positions on: below, either kernel takes
-  // the 4 us of a launch.
+  // the 4 us of a launch.  With three dims the first counts planes, each cut into
+  // groups of its own - images between channels last and channels first, (B, H,
+  // W, C) <-> (B, C, H, W) with H and W fused: (16, 1024, 1024, 3) 75 -> 66 us
+  // and back 175 -> 63, (256, 56, 56, 8) 28.6 -> 8.2 - from planes of 256
+  // positions on (shorter ones leave most of a group idle: (65536, 4, 4, 3) 4.8
+  // us with the strided kernel, 17 this way).
   bool narrow_plane_in_registers(int &err) {
     const unsigned long fmax = TUNE(tn, ELEMWISE_NARROW, 15);
-    if (fmax == 0 || nd != 2 || na > 31) return false;
-    const unsigned sd = dims[0] <= dims[1] ? 0 : 1, ld = 1 - sd;
+    if (fmax == 0 || (nd != 2 && nd != 3) || na > 31) return false;
+    const unsigned sd = dims[nd - 2] <= dims[nd - 1] ? nd - 2 : nd - 1, ld = sd == nd - 1 ? nd - 2 : nd - 1;
     const size_t F = dims[sd], L = dims[ld];
-    if (F < 2 || F > fmax || F > 16 || L < TUNE(tn, ELEMWISE_NARROW_MIN, 4096)) return false;
-    if (ge->flags & GE_CONVERT_F16) return false;
+    if (F < 2 || F > fmax || F > 16 || n / F < TUNE(tn, ELEMWISE_NARROW_MIN, 4096)) return false;
+    if (L < TUNE(tn, ELEMWISE_NARROW_MIN_PLANE, 256)) return false;
     // a short extent of whole quads innermost in the result: four elements per
     // lane of the strided kernel are a chunk of the result and coalesced single
     // elements of the operands (out = in.T of (4, N) 78 against 75 % of peak, of
     // (8, N) 79 against 74)
-    if (sd == 1 && F % 4 == 0 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
+    if (sd == nd - 1 && F % 4 == 0 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
     unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0;
     bool crossed = false;   // some array runs along the long dim and moves along the short one
     const unsigned long stage = TUNE(tn, ELEMWISE_NARROW_LDS, 2);   // 1: staged when read, 2: when written
@@ -1824,7 +1841,8 @@ class strided_call {
       for (size_t i = 0; i < ge->args.size(); i++) {
         if (!ge->args[i].is_array()) continue;
         if (elsz[k] != 4 || offs[k] % 4 != 0) return false;
-        const bool base16 = offs[k] % 16 == 0;
+        const bool base16 = offs[k] % 16 == 0 && (nd == 2 || strs[k][0] % 16 == 0);
+        if (nd == 3 && strs[k][0] % 4 != 0) return false;
         if (base16 && strs[k][sd] == 4 && strs[k][ld] == (ssize_t)(4 * F)) {
           bmask |= 1u << k;
           const bool want = (ge->args[i].reads() ? (stage & 1) : 0) || (ge->args[i].writes() ? (stage & 2) : 0);
@@ -1853,17 +1871,17 @@ class strided_call {
     }
     choose_offset_width();
     gx = (L + 1023) / 1024;
-    groups = gx;
+    groups = gx * (nd == 3 ? dims[0] : 1);
     ltx = 0;
-    if (groups > 0x7fffffffull) return false;
+    if (groups > 0x7fffffffull || gx > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "n%zu:%u:%d:%x:%x:%x:%x:%x", F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask, smask);
+    snprintf(key, sizeof(key), "n%u:%zu:%u:%d:%x:%x:%x:%x:%x", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask, smask);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask);
+      std::string src = gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2441,13 +2459,13 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // (and its bits 16.. the mask of those that fetch a chunk inside one row with one load on four-byte boundaries)
   if (strided == 9)
     return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64 & 0xffffu, (unsigned)idx64 >> 16).c_str());
-  // 14: a narrow plane in registers: nd carries the short extent, idx64 bit 0 the offsets' width, bit 1 the
+  // 14: a narrow plane in registers: nd carries the short extent (plus 256: planes, three dims), idx64 bit 0 the offsets' width, bit 1 the
   // short dim, bit 2 streaming accesses, bit 3 the first kind of arrays through the LDS, bit 4 the second kind
   // on four-byte boundaries; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
   if (strided == 14)
-    return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd, ((unsigned)idx64 >> 1) & 1u, tmask & 0xffffu, tmask >> 16,
-                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
-                                   (idx64 & 8) ? tmask & 0xffffu : 0u).c_str());
+    return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
+                                   tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
+                                   (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8)).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 && strided != 13 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu

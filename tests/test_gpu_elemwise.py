@@ -635,8 +635,9 @@ def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads):
     the LDS, ELEMWISE_NARROW_LDS; the others as 16-byte chunks, on four-byte
     boundaries when N is no multiple of four).  Long extents of whole and cut
     groups and lanes, a row operand, an array read and written, a result inside a
-    larger buffer whose rows start off the 16-byte boundaries; floats and 32-bit
-    integers against NumPy, exact."""
+    larger buffer whose rows start off the 16-byte boundaries, batches of planes
+    (channels last to channels first and back); floats and 32-bit integers against
+    NumPy, exact."""
     knobs(ELEMWISE_NARROW_LDS=lds, ELEMWISE_NARROW_NT=nt, ELEMWISE_NARROW_QUADS=quads, ELEMWISE_NARROW_MIN=1024)
     rng = np.random.default_rng(900 + lds)
     for dtype in ("float32", "int32"):
@@ -670,6 +671,25 @@ def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads):
         want = root.copy()
         want[:, 1:n + 1] = a.T
         assert np.array_equal(read_root(groot, root), want), dtype
+        # planes: channels last to channels first and back, (B, H, W, C) <-> (B, C, H, W); whole planes
+        # of 1024 positions, cut ones, short ones, and planes inside a larger buffer
+        for bsz, h, w, c in ((3, 32, 32, 3), (5, 17, 31, 7), (2, 40, 50, 4), (4, 16, 16, 5)):
+            x = draw((bsz, h, w, c))
+            out = gpuarray.empty((bsz, c, h, w), dtype, context=ctx)
+            kc(gpuarray.array(x, context=ctx).transpose(0, 3, 1, 2), out)
+            assert np.array_equal(np.asarray(out), x.transpose(0, 3, 1, 2)), (dtype, bsz, h, w, c)
+            y = draw((bsz, c, h, w))
+            out = gpuarray.empty((bsz, h, w, c), dtype, context=ctx)
+            kc(gpuarray.array(y, context=ctx).transpose(0, 2, 3, 1), out)
+            assert np.array_equal(np.asarray(out), y.transpose(0, 2, 3, 1)), (dtype, bsz, h, w, c, "back")
+        xroot = draw((3, 1000 + 2, 6))
+        gx_, _ = to_gpu_view(xroot[:, 2:], ctx)
+        oroot = np.zeros((3, 6 + 1, 1000), dtype)
+        go, groot = to_gpu_view(oroot[:, :6], ctx)
+        kc(gx_.transpose(0, 2, 1), go)
+        want = oroot.copy()
+        want[:, :6] = xroot[:, 2:].transpose(0, 2, 1)
+        assert np.array_equal(read_root(groot, oroot), want), dtype
         # the narrow operand as a view that starts off the 16-byte boundaries: the other kernels
         aroot = draw((n + 1, f))
         gv, _ = to_gpu_view(aroot[1:], ctx)
