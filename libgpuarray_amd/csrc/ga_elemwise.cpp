@@ -684,6 +684,187 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
   return s;
 }
 
+// ---- narrow planes through the LDS ----------------------------------------------
+// The same planes and parameters as gen_narrow_block for short extents F too
+// large for a lane's registers (16 to 64).  A group owns 256 positions along L:
+// the arrays in bmask (short dim innermost, the group's piece one contiguous
+// run of 256 F elements on a 16-byte boundary) pass through the LDS whole, as
+// consecutive 16-byte chunks on consecutive lanes; lane (lx, ly) = (LID_0 % 64,
+// LID_0 / 64) then takes positions 4 lx .. 4 lx + 3 of the short dim's rows ly,
+// ly + 4, ...: four words of the LDS per such array, one 16-byte chunk of the
+// arrays in cmask (on four-byte boundaries for those in umask), single elements
+// of the others.  In the LDS position l of the group and row y sit at word
+// ((l % 4) * 65 + l / 4) * (F | 1) + y: the 64 lanes of a wavefront, on 64
+// positions four apart and one row, then fall on 64 consecutive multiples of
+// an odd pitch (no two on one bank beyond the two a bank serves anyway), and
+// the words of the chunks that move between memory and the LDS, four rows
+// apart on consecutive lanes, spread over the banks through the 65.
+std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, unsigned sd, unsigned bmask,
+                              unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask,
+                              unsigned nd) {
+  std::string s;
+  const char *I = idx64 ? "ga_ssize" : "ga_int";
+  const char *N = idx64 ? "ga_size" : "ga_uint";
+  const unsigned ld = sd == nd - 1 ? nd - 2 : nd - 1;
+  const unsigned chunks = 64 * F;            // 16-byte chunks of a group's piece
+  const unsigned Fp = F | 1;
+  emit_header(ge, s);
+  appendf(s, "#define GA_AT(l, y) ((((l) & 3u) * 65u + ((l) >> 2)) * %uu + (y))\n", Fp);
+  if (umask) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
+  ktypes.push_back(GA_SIZE);
+  for (unsigned d = 1; d < nd; d++) {
+    appendf(s, ", const ga_size dim%u", d);
+    ktypes.push_back(GA_SIZE);
+  }
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto in = [&](unsigned mask, size_t j) { return aidx[j] >= 0 && ((mask >> aidx[j]) & 1u); };
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset", ctype(a.typecode), a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+      for (unsigned d = 0; d < nd; d++) {
+        appendf(s, ", const ga_ssize %s_str_%u", a.name.c_str(), d);
+        ktypes.push_back(GA_SSIZE);
+      }
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n(void)ga_gx; (void)ga_ltx; (void)dim0; (void)dim1;\n";
+  ktypes.push_back(GA_UINT);
+  ktypes.push_back(GA_UINT);
+  if (nd == 3) s += "const ga_uint ga_o = GID_0 / ga_gx;\nconst ga_uint ga_pc = GID_0 - ga_o * ga_gx;\n";
+  else s += "const ga_uint ga_pc = GID_0;\n";
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n", a.name.c_str(), a.name.c_str(),
+            a.name.c_str());
+    if (nd == 3) appendf(s, "%s_b += (%s)ga_o * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
+    if (in(bmask, j)) appendf(s, "LOCAL_MEM %s %s_s[%u];\n", ctype(a.typecode), a.name.c_str(), 260 * Fp);
+  }
+  appendf(s, "const %s ga_l0 = (%s)ga_pc * 256u;\n", N, N);
+  s += "const ga_uint ga_lx = LID_0 & 63u, ga_ly = LID_0 >> 6;\n";
+  appendf(s, "const %s ga_l4 = ga_l0 + ga_lx * 4u;\n", N);
+  appendf(s, "const bool ga_full = ga_l4 + 3u < (%s)dim%u;\n", N, ld);
+  appendf(s, "const ga_uint ga_cnt = (ga_uint)((%s)dim%u - ga_l0 < 256u ? (%s)dim%u - ga_l0 : 256u) * %uu;\n", N, ld, N, ld, F);
+  auto elem_at = [&](const ge_arg &a, const std::string &y, const std::string &l) {
+    std::string e;
+    appendf(e, "*(GLOBAL_MEM %s *)(%s_b + ((%s)(%s) * (%s)%s_str_%u + (%s)(%s) * (%s)%s_str_%u))", ctype(a.typecode),
+            a.name.c_str(), I, y.c_str(), I, a.name.c_str(), sd, I, l.c_str(), I, a.name.c_str(), ld);
+    return e;
+  };
+  auto piece_at = [&](const ge_arg &a, const char *cast, const std::string &bytes) {
+    std::string e;
+    appendf(e, "(GLOBAL_MEM %s *)(%s_b + (%s)ga_l0 * (%s)%s_str_%u + (%s))", cast, a.name.c_str(), I, I,
+            a.name.c_str(), ld, bytes.c_str());
+    return e;
+  };
+  bool staged_in = false, staged_out = false;
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(bmask, j)) continue;
+    if (a.writes()) staged_out = true;
+    if (!a.reads()) continue;
+    staged_in = true;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    appendf(s, "for (ga_uint ga_q = LID_0; ga_q < %uu; ga_q += 256u) {\n", chunks);
+    appendf(s, "union { ga_chunk16 c; %s e[4]; } ga_v;\n", ctype(a.typecode));
+    appendf(s, "if (ga_q * 4u + 3u < ga_cnt) ga_v.c = %s(%s);\n", nt ? "__builtin_nontemporal_load" : "*",
+            piece_at(a, "const ga_chunk16", "ga_q * 16u").c_str());
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) ga_v.e[ga_e] = *(%s);\n",
+            piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str());
+    appendf(s, "for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) { const ga_uint ga_w = ga_q * 4u + ga_e, ga_l = ga_w / %uu; "
+               "%s_s[GA_AT(ga_l, ga_w - ga_l * %uu)] = ga_v.e[ga_e]; }\n", F, a.name.c_str(), F);
+    s += "}\n";
+  }
+  if (staged_in) s += "local_barrier();\n";
+  appendf(s, "for (ga_uint ga_y = ga_ly; ga_y < %uu; ga_y += 4u) {\n", F);
+  // a lane's four values of the chunked arrays for this row
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(cmask, j)) continue;
+    const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    appendf(s, "union { ga_chunk16 c; %s e[4]; } %s_r;\n", ctype(a.typecode), a.name.c_str());
+    if (!a.reads()) continue;
+    std::string ptr;
+    appendf(ptr, "(GLOBAL_MEM const %s *)&%s", ct, elem_at(a, "ga_y", "ga_l4").c_str());
+    appendf(s, "if (ga_full) %s_r.c = %s(%s); else {\n", a.name.c_str(), nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
+    for (unsigned e = 0; e < 4; e++) {
+      char l[32];
+      snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+      appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s_r.e[%u] = %s;\n", e, N, ld, a.name.c_str(), e, elem_at(a, "ga_y", l).c_str());
+    }
+    s += "}\n";
+  }
+  for (unsigned e = 0; e < 4; e++) {
+    char l[32];
+    snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+    appendf(s, "if (ga_l4 + %uu < (%s)dim%u) {\n", e, N, ld);
+    auto place = [&](size_t j) {
+      const ge_arg &a = ge->args[j];
+      std::string x;
+      if (in(bmask, j)) appendf(x, "%s_s[(%uu + ga_lx) * %uu + ga_y]", a.name.c_str(), e * 65, Fp);
+      else if (in(cmask, j)) appendf(x, "%s_r.e[%u]", a.name.c_str(), e);
+      else x = elem_at(a, "ga_y", l);
+      return x;
+    };
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) emit_load(ge, s, ge->args[j], place(j));
+    s += ge->expr;
+    s += ";\n";
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array() && ge->args[j].writes()) emit_store(ge, s, ge->args[j], place(j));
+    s += "}\n";
+  }
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(cmask, j) || !a.writes()) continue;
+    const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    std::string ptr;
+    appendf(ptr, "(GLOBAL_MEM %s *)&%s", ct, elem_at(a, "ga_y", "ga_l4").c_str());
+    if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store((%s)%s_r.c, %s); else {\n", ct, a.name.c_str(), ptr.c_str());
+    else appendf(s, "if (ga_full) *(%s) = %s_r.c; else {\n", ptr.c_str(), a.name.c_str());
+    for (unsigned e = 0; e < 4; e++) {
+      char l[32];
+      snprintf(l, sizeof(l), "ga_l4 + %uu", e);
+      appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s = %s_r.e[%u];\n", e, N, ld, elem_at(a, "ga_y", l).c_str(), a.name.c_str(), e);
+    }
+    s += "}\n";
+  }
+  s += "}\n";
+  if (staged_out) {
+    s += "local_barrier();\n";
+    for (size_t j = 0; j < ge->args.size(); j++) {
+      const ge_arg &a = ge->args[j];
+      if (!in(bmask, j) || !a.writes()) continue;
+      const bool nt = (ntmask >> aidx[j]) & 1u;
+      appendf(s, "for (ga_uint ga_q = LID_0; ga_q < %uu; ga_q += 256u) {\n", chunks);
+      appendf(s, "union { ga_chunk16 c; %s e[4]; } ga_v;\n", ctype(a.typecode));
+      appendf(s, "for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) { const ga_uint ga_w = ga_q * 4u + ga_e, ga_l = ga_w / %uu; "
+                 "ga_v.e[ga_e] = %s_s[GA_AT(ga_l, ga_w - ga_l * %uu)]; }\n", F, a.name.c_str(), F);
+      const std::string ptr = piece_at(a, "ga_chunk16", "ga_q * 16u");
+      if (nt) appendf(s, "if (ga_q * 4u + 3u < ga_cnt) __builtin_nontemporal_store(ga_v.c, %s);\n", ptr.c_str());
+      else appendf(s, "if (ga_q * 4u + 3u < ga_cnt) *(%s) = ga_v.c;\n", ptr.c_str());
+      appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) *(%s) = ga_v.e[ga_e];\n",
+              piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str());
+      s += "}\n";
+    }
+  }
+  s += "}\n";
+  return s;
+}
+
 // ---- strided kernel -------------------------------------------------------------
 // elem(dim0..dim{nd-1}, {data, byte offset, str_0..str_{nd-1} | scalar}...,
 //      ga_gx, ga_ltx)
@@ -1825,7 +2006,16 @@ class strided_call {
     if (fmax == 0 || (nd != 2 && nd != 3) || na > 31) return false;
     const unsigned sd = dims[nd - 2] <= dims[nd - 1] ? nd - 2 : nd - 1, ld = sd == nd - 1 ? nd - 2 : nd - 1;
     const size_t F = dims[sd], L = dims[ld];
-    if (F < 2 || F > fmax || F > 16 || n / F < TUNE(tn, ELEMWISE_NARROW_MIN, 4096)) return false;
+    // Wider ones whole through the LDS (gen_narrow_staged), where the tiles are
+    // filled badly.  out = in.T of 256 MiB of floats, tiles / this kernel in % of
+    // 8 TB/s: (N, F) -> (F, N) F = 17 37 / 58, 19 39 / 59, 22 45 / 60, 25 51 / 59,
+    // 27 51 / 58, 31 56 / 59, then level (34 57 / 58) and behind (40 64 / 56, 56
+    // 71 / 47: the result's rows leave a group in pieces of 1 KiB); (F, N) -> (N,
+    // F), F no multiple of four: 17 41 / 71, 23 47 / 73, 29 43 / 67, 35 50 / 65, 41
+    // 53 / 57, 50 37 / 59, 57 36 / 43, 63 41 / 46.
+    const unsigned long smax = sd == nd - 1 ? TUNE(tn, ELEMWISE_NARROW_STAGED, 64) : TUNE(tn, ELEMWISE_NARROW_STAGED_WIDE, 31);
+    const bool wide = F > 16;
+    if (F < 2 || F > (wide ? smax : fmax) || F > 64 || n / F < TUNE(tn, ELEMWISE_NARROW_MIN, 4096)) return false;
     if (L < TUNE(tn, ELEMWISE_NARROW_MIN_PLANE, 256)) return false;
     // a short extent of whole quads innermost in the result: four elements per
     // lane of the strided kernel are a chunk of the result and coalesced single
@@ -1846,7 +2036,10 @@ class strided_call {
         if (base16 && strs[k][sd] == 4 && strs[k][ld] == (ssize_t)(4 * F)) {
           bmask |= 1u << k;
           const bool want = (ge->args[i].reads() ? (stage & 1) : 0) || (ge->args[i].writes() ? (stage & 2) : 0);
-          if (want && lds + 4096 * F <= 64 * 1024) {
+          if (wide) {
+            lds += 260 * 4 * (F | 1);
+            if (lds > 72 * 1024) return false;
+          } else if (want && lds + 4096 * F <= 64 * 1024) {
             smask |= 1u << k;
             lds += 4096 * F;
           }
@@ -1864,24 +2057,26 @@ class strided_call {
     {
       const unsigned long m = TUNE(tn, ELEMWISE_NARROW_NT, 3);
       if (m & 1) nt |= cmask;
-      if (m & 2) nt |= smask;
+      if (m & 2) nt |= wide ? bmask : smask;
       if (m & 4) nt |= bmask;
       for (unsigned k = 0; k < na; k++)
         if (strs[k][sd] == 0) nt &= ~(1u << k);
     }
     choose_offset_width();
-    gx = (L + 1023) / 1024;
+    gx = wide ? (L + 255) / 256 : (L + 1023) / 1024;
     groups = gx * (nd == 3 ? dims[0] : 1);
     ltx = 0;
     if (groups > 0x7fffffffull || gx > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "n%u:%zu:%u:%d:%x:%x:%x:%x:%x", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask, smask);
+    snprintf(key, sizeof(key), "%s%u:%zu:%u:%d:%x:%x:%x:%x:%x", wide ? "w" : "n", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask,
+             smask);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd);
+      std::string src = wide ? gen_narrow_staged(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, nd)
+                             : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2466,6 +2661,11 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
     return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
                                    tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
                                    (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8)).c_str());
+  // 15: the same arguments for a wider short extent, whole through the LDS
+  if (strided == 15)
+    return strdup(gen_narrow_staged(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
+                                    tmask >> 16, (idx64 & 4) ? 0xffffu : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
+                                    2 + (nd >> 8)).c_str());
   std::string src = strided >= 2 ? gen_strided_vec(&ge, nd, idx64 != 0, tmask & 0xffffu, tmask >> 16, ktypes,
                                                    strided >= 3 ? 0xffffffffu : 0u, strided >= 4 && strided != 13 ? 128 : 64,
                                                    strided == 7 ? ~(tmask | (tmask >> 16)) & 0xffffu

@@ -627,25 +627,28 @@ def test_transposed_operands_of_narrow_planes(ctx, knobs, fill, tmin):
             assert np.array_equal(np.asarray(out2), b.T + r2), (dtype, n, f, "wide")
 
 
-@pytest.mark.parametrize("lds,nt,quads", [(2, 3, 0), (3, 0, 1), (0, 7, 1), (1, 1, 0)])
-def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads):
+@pytest.mark.parametrize("lds,nt,quads,wide", [(2, 3, 0, None), (3, 0, 1, 64), (0, 7, 1, None), (1, 1, 0, 64)])
+def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads, wide):
     """(N, f) with f from 2 to 15 taken as its transpose, and written as one: a
     lane holds four positions of the long dim by all f of the short one
     (ELEMWISE_NARROW; the arrays with the short dim innermost directly or through
     the LDS, ELEMWISE_NARROW_LDS; the others as 16-byte chunks, on four-byte
-    boundaries when N is no multiple of four).  Long extents of whole and cut
+    boundaries when N is no multiple of four).  f from 17 to 64: a group's piece
+    of the arrays with the short dim innermost whole through the LDS
+    (ELEMWISE_NARROW_STAGED for narrow results, _STAGED_WIDE for wide ones).  Long extents of whole and cut
     groups and lanes, a row operand, an array read and written, a result inside a
     larger buffer whose rows start off the 16-byte boundaries, batches of planes
     (channels last to channels first and back); floats and 32-bit integers against
     NumPy, exact."""
-    knobs(ELEMWISE_NARROW_LDS=lds, ELEMWISE_NARROW_NT=nt, ELEMWISE_NARROW_QUADS=quads, ELEMWISE_NARROW_MIN=1024)
+    knobs(ELEMWISE_NARROW_LDS=lds, ELEMWISE_NARROW_NT=nt, ELEMWISE_NARROW_QUADS=quads, ELEMWISE_NARROW_MIN=1024,
+          ELEMWISE_NARROW_STAGED_WIDE=wide)
     rng = np.random.default_rng(900 + lds)
     for dtype in ("float32", "int32"):
         k = ga.GpuElemwise(ctx, "o = a + r", [arg("a", dtype, read=True), arg("r", dtype, read=True),
                                                arg("o", dtype, write=True)])
         kio = ga.GpuElemwise(ctx, "o = o - a", [arg("a", dtype, read=True), arg("o", dtype, read=True, write=True)])
         draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
-        for f in range(2, 16):
+        for f in list(range(2, 16)) + [17, 20, 23, 31, 32, 33, 50, 63, 64]:
             for n in ((1024, 4099, 100001) if f % 3 else (2048, 5003, 8190)):
                 a = draw((n, f))
                 r = draw((1, n))
@@ -673,7 +676,7 @@ def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads):
         assert np.array_equal(read_root(groot, root), want), dtype
         # planes: channels last to channels first and back, (B, H, W, C) <-> (B, C, H, W); whole planes
         # of 1024 positions, cut ones, short ones, and planes inside a larger buffer
-        for bsz, h, w, c in ((3, 32, 32, 3), (5, 17, 31, 7), (2, 40, 50, 4), (4, 16, 16, 5)):
+        for bsz, h, w, c in ((3, 32, 32, 3), (5, 17, 31, 7), (2, 40, 50, 4), (4, 16, 16, 5), (3, 20, 21, 18), (2, 16, 16, 35)):
             x = draw((bsz, h, w, c))
             out = gpuarray.empty((bsz, c, h, w), dtype, context=ctx)
             kc(gpuarray.array(x, context=ctx).transpose(0, 3, 1, 2), out)
