@@ -113,6 +113,12 @@ def main():
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 15, 33, 0b00100, 0b001 | (0b110 << 16)))
     check("elemwise narrow planes of 20 through the LDS, three dims: the result staged, chunks on four-byte boundaries",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 15, 20 | 256, 0b10111, 0b100 | (0b011 << 16)))
+    check("elemwise narrow plane of 3 doubles in registers: the result through the LDS",
+          gen_e(b"", b"c = a + c", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_DOUBLE, 2), ElemwiseArg(b"c", GA_DOUBLE, 6)),
+                0, 14, 3, 0b01110, 0b10 | (0b01 << 16)))
+    check("elemwise narrow plane of 7 halves in registers, computed in floats",
+          gen_e(b"", b"c = a + 1", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_HALF, 2), ElemwiseArg(b"c", GA_HALF, 4)),
+                2, 14, 7, 0b00100, 0b01 | (0b10 << 16)))
     iargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_FLOAT, 6))
     check("elemwise narrow plane of 4 in registers: an array read and written through the LDS",
           gen_e(b"", b"c = a + c", 2, iargs, 0, 14, 4, 0b01000, 0b10 | (0b01 << 16)))
@@ -221,7 +227,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "38 elementwise)" % (n + 20, m, t))
+          "40 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

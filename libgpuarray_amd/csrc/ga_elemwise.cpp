@@ -423,9 +423,10 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 // ---- narrow planes in registers -------------------------------------------------
 // Same parameters as the strided kernel with two or three dims (with three, the
 // first counts planes, ga_gx groups each).  One of the last two dims is
-// short (S, extent F <= 16, fixed in the text), the other long (L).  A lane
-// owns four adjacent positions along L and all F along S; a group 1024
-// positions along L.
+// short (S, extent F <= 16, fixed in the text), the other long (L).  Every
+// array has elements of es = 2, 4 or 8 bytes, E = 16 / es to a chunk (the text
+// below says four).  A lane owns E adjacent positions along L and all F along S;
+// a group 256 E positions along L.
 //  * The arrays in bmask have the short dim innermost: a lane's 4 F elements,
 //    and a group's 4096 F, lie one after the other in memory (stride of S one
 //    element, of L F elements: an (N, F) array taken as its transpose), on a
@@ -437,21 +438,23 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 //    stored as the lane's own F chunks.
 //  * The arrays in cmask run along L with unit stride and move as one 16-byte
 //    chunk per position of S, side by side with the neighbouring lanes'; those
-//    also in umask through accesses that assume four-byte boundaries only.
+//    also in umask through accesses that assume four-byte boundaries only (the
+//    element's own with two-byte elements).
 //  * Every other array one element at a time.
-// All arrays have four-byte elements.  The last lane of a row takes what exists
-// of its four positions one by one.
+// The last lane of a row takes what exists of its positions one by one.
 std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsigned sd, unsigned bmask,
                              unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask = 0,
-                             unsigned smask = 0, unsigned nd = 2) {
+                             unsigned smask = 0, unsigned nd = 2, unsigned es = 4) {
   std::string s;
+  const unsigned E = 16 / es;   // elements of a chunk = positions of a lane
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
   const unsigned ld = sd == nd - 1 ? nd - 2 : nd - 1;
   const bool swz = (F & (F - 1)) == 0;
   emit_header(ge, s);
-  if (umask) s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  if (umask) appendf(s, "typedef ga_uint __attribute__((ext_vector_type(4), aligned(%u))) ga_chunk16u;\n", es < 4 ? es : 4);
   if (smask) s += swz ? "#define GA_SLOT(q) ((q) ^ (((q) >> 3) & 7u))\n" : "#define GA_SLOT(q) (q)\n";
+  appendf(s, "#define GA_E %uu\n#define GA_ES %uu\n", E, es);
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
   ktypes.push_back(GA_SIZE);
   for (unsigned d = 1; d < nd; d++) {
@@ -493,20 +496,20 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     if (nd == 3) appendf(s, "%s_b += (%s)ga_o * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
     if (in(smask, j)) appendf(s, "LOCAL_MEM ga_chunk16 %s_s[%u];\n", a.name.c_str(), 256 * F);
   }
-  appendf(s, "const %s ga_l0 = (%s)ga_pc * 1024u;\n", N, N);
-  appendf(s, "const %s ga_l4 = ga_l0 + LID_0 * 4u;\n", N);
+  appendf(s, "const %s ga_l0 = (%s)ga_pc * %uu;\n", N, N, 256 * E);
+  appendf(s, "const %s ga_l4 = ga_l0 + LID_0 * %uu;\n", N, E);
   if (!smask) appendf(s, "if (ga_l4 >= (%s)dim%u) return;\n", N, ld);
-  appendf(s, "const bool ga_full = ga_l4 + 3u < (%s)dim%u;\n", N, ld);
+  appendf(s, "const bool ga_full = ga_l4 + %uu < (%s)dim%u;\n", E - 1, N, ld);
   // the four-byte words of a staged array that the group's piece holds
   if (smask)
-    appendf(s, "const ga_uint ga_cnt = (ga_uint)((%s)dim%u - ga_l0 < 1024u ? (%s)dim%u - ga_l0 : 1024u) * %uu;\n", N, ld,
-            N, ld, F);
+    appendf(s, "const ga_uint ga_cnt = (ga_uint)((%s)dim%u - ga_l0 < %uu ? (%s)dim%u - ga_l0 : %uu) * %uu;\n", N, ld, 256 * E,
+            N, ld, 256 * E, F);
   // registers of the block arrays (element e * F + y: position e along L, y along S)
   // and of the chunked ones (element e of chunk y)
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
-    if (in(bmask, j)) appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r;\n", F, ctype(a.typecode), 4 * F, a.name.c_str());
-    else if (in(cmask, j)) appendf(s, "union { ga_chunk16 c; %s e[4]; } %s_r[%u];\n", ctype(a.typecode), a.name.c_str(), F);
+    if (in(bmask, j)) appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r;\n", F, ctype(a.typecode), E * F, a.name.c_str());
+    else if (in(cmask, j)) appendf(s, "union { ga_chunk16 c; %s e[%u]; } %s_r[%u];\n", ctype(a.typecode), E, a.name.c_str(), F);
   }
   auto elem_at = [&](const ge_arg &a, const std::string &y, const std::string &l) {
     std::string e;
@@ -533,11 +536,11 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
       for (unsigned h = 0; h < F; h++) {
         appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
         const std::string ptr = piece_at(a, "const ga_chunk16", "ga_q * 16u");
-        appendf(s, "if (ga_q * 4u + 3u < ga_cnt) %s_s[GA_SLOT(ga_q)] = %s(%s);\n", a.name.c_str(),
+        appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) %s_s[GA_SLOT(ga_q)] = %s(%s);\n", a.name.c_str(),
                 nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
-        appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) "
-                   "((%s *)%s_s)[GA_SLOT(ga_q) * 4u + ga_e] = *(%s);\n",
-                ctype(a.typecode), a.name.c_str(), piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str());
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < GA_E; ga_e++) if (ga_q * GA_E + ga_e < ga_cnt) "
+                   "((%s *)%s_s)[GA_SLOT(ga_q) * GA_E + ga_e] = *(%s);\n",
+                ctype(a.typecode), a.name.c_str(), piece_at(a, ctype(a.typecode), "(ga_q * GA_E + ga_e) * GA_ES").c_str());
         s += "}\n";
       }
     } else if (in(bmask, j)) {
@@ -549,7 +552,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         appendf(s, "%s_r.c[%u] = %s(%s);\n", a.name.c_str(), h, nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
       }
       s += "} else {\n";
-      for (unsigned e = 0; e < 4; e++)
+      for (unsigned e = 0; e < E; e++)
         for (unsigned y = 0; y < F; y++) {
           char l[32], yy[16];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
@@ -567,7 +570,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         appendf(ptr, "(GLOBAL_MEM const %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
         appendf(s, "if (ga_full) %s_r[%u].c = %s(%s); else {\n", a.name.c_str(), y,
                 nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
-        for (unsigned e = 0; e < 4; e++) {
+        for (unsigned e = 0; e < E; e++) {
           char l[32];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
           appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s_r[%u].e[%u] = %s;\n", e, N, ld, a.name.c_str(), y, e,
@@ -588,7 +591,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
   }
   // the expression, position by position
   for (unsigned y = 0; y < F; y++)
-    for (unsigned e = 0; e < 4; e++) {
+    for (unsigned e = 0; e < E; e++) {
       char l[32], yy[16];
       snprintf(l, sizeof(l), "ga_l4 + %uu", e);
       snprintf(yy, sizeof(yy), "%uu", y);
@@ -634,12 +637,12 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
       for (unsigned h = 0; h < F; h++) {
         appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
         const std::string ptr = piece_at(a, "ga_chunk16", "ga_q * 16u");
-        if (nt) appendf(s, "if (ga_q * 4u + 3u < ga_cnt) __builtin_nontemporal_store(%s_s[GA_SLOT(ga_q)], %s);\n",
+        if (nt) appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) __builtin_nontemporal_store(%s_s[GA_SLOT(ga_q)], %s);\n",
                         a.name.c_str(), ptr.c_str());
-        else appendf(s, "if (ga_q * 4u + 3u < ga_cnt) *(%s) = %s_s[GA_SLOT(ga_q)];\n", ptr.c_str(), a.name.c_str());
-        appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_q * 4u + ga_e < ga_cnt) "
-                   "*(%s) = ((%s *)%s_s)[GA_SLOT(ga_q) * 4u + ga_e];\n",
-                piece_at(a, ctype(a.typecode), "(ga_q * 4u + ga_e) * 4u").c_str(), ctype(a.typecode), a.name.c_str());
+        else appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) *(%s) = %s_s[GA_SLOT(ga_q)];\n", ptr.c_str(), a.name.c_str());
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < GA_E; ga_e++) if (ga_q * GA_E + ga_e < ga_cnt) "
+                   "*(%s) = ((%s *)%s_s)[GA_SLOT(ga_q) * GA_E + ga_e];\n",
+                piece_at(a, ctype(a.typecode), "(ga_q * GA_E + ga_e) * GA_ES").c_str(), ctype(a.typecode), a.name.c_str());
         s += "}\n";
       }
     } else if (in(bmask, j)) {
@@ -652,7 +655,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         else appendf(s, "*(%s) = %s_r.c[%u];\n", ptr.c_str(), a.name.c_str(), h);
       }
       s += "} else {\n";
-      for (unsigned e = 0; e < 4; e++)
+      for (unsigned e = 0; e < E; e++)
         for (unsigned y = 0; y < F; y++) {
           char l[32], yy[16];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
@@ -670,7 +673,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         appendf(ptr, "(GLOBAL_MEM %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
         if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store((%s)%s_r[%u].c, %s); else {\n", ct, a.name.c_str(), y, ptr.c_str());
         else appendf(s, "if (ga_full) *(%s) = %s_r[%u].c; else {\n", ptr.c_str(), a.name.c_str(), y);
-        for (unsigned e = 0; e < 4; e++) {
+        for (unsigned e = 0; e < E; e++) {
           char l[32];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
           appendf(s, "if (ga_l4 + %uu < (%s)dim%u) %s = %s_r[%u].e[%u];\n", e, N, ld, elem_at(a, yy, l).c_str(),
@@ -1984,7 +1987,8 @@ class strided_call {
     gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
   }
 
-  // A plane with one short extent F (2 to 15) of four-byte elements where some
+  // A plane with one short extent F (2 to 15) of two-, four- or eight-byte
+  // elements (all arrays alike; the figures are for four-byte ones) where some
   // array has the short dim innermost and another the long one - (N, F) taken as
   // its transpose, or written as one: too narrow for tiles through the LDS, which
   // F of 64 or 128 columns fill.  A lane takes four positions along the long dim
@@ -2021,7 +2025,10 @@ class strided_call {
     // lane of the strided kernel are a chunk of the result and coalesced single
     // elements of the operands (out = in.T of (4, N) 78 against 75 % of peak, of
     // (8, N) 79 against 74)
-    if (sd == nd - 1 && F % 4 == 0 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
+    const size_t es = elsz[0], E = 16 / (es ? es : 1);
+    if ((es != 2 && es != 4 && es != 8) || (wide && es != 4)) return false;
+    // (two-byte elements: (8, N) -> (N, 8) of halves 54 % there, 73 % here)
+    if (sd == nd - 1 && F % E == 0 && es >= 4 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
     unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0;
     bool crossed = false;   // some array runs along the long dim and moves along the short one
     const unsigned long stage = TUNE(tn, ELEMWISE_NARROW_LDS, 2);   // 1: staged when read, 2: when written
@@ -2030,10 +2037,10 @@ class strided_call {
       unsigned k = 0;
       for (size_t i = 0; i < ge->args.size(); i++) {
         if (!ge->args[i].is_array()) continue;
-        if (elsz[k] != 4 || offs[k] % 4 != 0) return false;
+        if (elsz[k] != es || offs[k] % es != 0) return false;
         const bool base16 = offs[k] % 16 == 0 && (nd == 2 || strs[k][0] % 16 == 0);
-        if (nd == 3 && strs[k][0] % 4 != 0) return false;
-        if (base16 && strs[k][sd] == 4 && strs[k][ld] == (ssize_t)(4 * F)) {
+        if (nd == 3 && strs[k][0] % (ssize_t)es != 0) return false;
+        if (base16 && strs[k][sd] == (ssize_t)es && strs[k][ld] == (ssize_t)(es * F)) {
           bmask |= 1u << k;
           const bool want = (ge->args[i].reads() ? (stage & 1) : 0) || (ge->args[i].writes() ? (stage & 2) : 0);
           if (wide) {
@@ -2043,10 +2050,11 @@ class strided_call {
             smask |= 1u << k;
             lds += 4096 * F;
           }
-        } else if (strs[k][ld] == 4 && strs[k][sd] % 4 == 0) {
+        } else if (strs[k][ld] == (ssize_t)es && strs[k][sd] % (ssize_t)es == 0) {
+          const bool whole = base16 && strs[k][sd] % 16 == 0;
           cmask |= 1u << k;
           if (strs[k][sd] != 0) crossed = true;
-          if (!base16 || strs[k][sd] % 16 != 0) umask |= 1u << k;
+          if (!whole) umask |= 1u << k;
         }
         k++;
       }
@@ -2063,20 +2071,20 @@ class strided_call {
         if (strs[k][sd] == 0) nt &= ~(1u << k);
     }
     choose_offset_width();
-    gx = wide ? (L + 255) / 256 : (L + 1023) / 1024;
+    gx = wide ? (L + 255) / 256 : (L + 256 * E - 1) / (256 * E);
     groups = gx * (nd == 3 ? dims[0] : 1);
     ltx = 0;
     if (groups > 0x7fffffffull || gx > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%zu:%u:%d:%x:%x:%x:%x:%x", wide ? "w" : "n", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask,
-             smask);
+    snprintf(key, sizeof(key), "%s%u:%zu:%u:%d:%x:%x:%x:%x:%x:%zu", wide ? "w" : "n", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask,
+             smask, es);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
       std::string src = wide ? gen_narrow_staged(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, nd)
-                             : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd);
+                             : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd, (unsigned)es);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2657,10 +2665,17 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // 14: a narrow plane in registers: nd carries the short extent (plus 256: planes, three dims), idx64 bit 0 the offsets' width, bit 1 the
   // short dim, bit 2 streaming accesses, bit 3 the first kind of arrays through the LDS, bit 4 the second kind
   // on four-byte boundaries; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
-  if (strided == 14)
+  if (strided == 14) {
+    unsigned es = 4;   // the element size of every array: the first one's
+    for (const ge_arg &a : ge.args)
+      if (a.is_array()) {
+        es = (unsigned)gpuarray_get_elsize(a.typecode);
+        break;
+      }
     return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
                                    tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
-                                   (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8)).c_str());
+                                   (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8), es).c_str());
+  }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)
     return strdup(gen_narrow_staged(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,

@@ -107,6 +107,8 @@ def elemwise_cases():
         ("a.T, (3, 22369621) -> (22369621, 3) (planes to interleaved channels)", "o = a",
          [("a", f, (3, 22369621), T(1, 0))], (22369621, 3), f),
         ("a.T, (6710886, 10) -> (10, 6710886)", "o = a", [("a", f, (6710886, 10), T(1, 0))], (10, 6710886), f),
+        ("a.T, (11184810, 3) -> (3, 11184810) doubles (points to coordinate rows)", "o = a",
+         [("a", d, (11184810, 3), T(1, 0))], (3, 11184810), d),
         ("NHWC -> NCHW, (16, 1024, 1024, 3) (images, channels last to planes)", "o = a",
          [("a", f, (16, 1024, 1024, 3), T(0, 3, 1, 2))], (16, 3, 1024, 1024), f),
         ("NCHW -> NHWC, (16, 3, 1024, 1024)", "o = a", [("a", f, (16, 3, 1024, 1024), T(0, 2, 3, 1))], (16, 1024, 1024, 3), f),

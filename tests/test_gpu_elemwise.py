@@ -701,6 +701,48 @@ def test_very_narrow_planes_held_in_registers(ctx, knobs, lds, nt, quads, wide):
         assert np.array_equal(np.asarray(out), aroot[1:].T), dtype
 
 
+@pytest.mark.parametrize("dtype", ["float64", "int64", "float16", "int16"])
+def test_very_narrow_planes_of_two_and_eight_byte_elements(ctx, knobs, dtype):
+    """The kernel that holds narrow planes in registers with two and eight elements
+    to a 16-byte chunk: (N, f) as its transpose and written as one, f from 2 to 15, N
+    with and without whole chunks (rows of the wide side off the 16-byte
+    boundaries), an array read and written, planes; halves computed as floats.
+    Against NumPy, exact (small integers)."""
+    knobs(ELEMWISE_NARROW_MIN=1024, ELEMWISE_NARROW_QUADS=1)
+    rng = np.random.default_rng(917)
+    k = ga.GpuElemwise(ctx, "o = a + r", [arg("a", dtype, read=True), arg("r", dtype, read=True),
+                                           arg("o", dtype, write=True)], convert_f16=True)
+    kio = ga.GpuElemwise(ctx, "o = o - a", [arg("a", dtype, read=True), arg("o", dtype, read=True, write=True)],
+                         convert_f16=True)
+    draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
+    for f in (2, 3, 4, 5, 8, 11, 15):
+        for n in (2048, 4099, 65537):
+            a = draw((n, f))
+            r = draw((1, n))
+            out = gpuarray.empty((f, n), dtype, context=ctx)
+            k(gpuarray.array(a, context=ctx).transpose(1, 0), gpuarray.array(r, context=ctx), out, broadcast=True)
+            assert np.array_equal(np.asarray(out), a.T + r), (n, f)
+            b = draw((f, n))
+            r2 = draw((1, f))
+            out2 = gpuarray.empty((n, f), dtype, context=ctx)
+            k(gpuarray.array(b, context=ctx).transpose(1, 0), gpuarray.array(r2, context=ctx), out2, broadcast=True)
+            assert np.array_equal(np.asarray(out2), b.T + r2), (n, f, "narrow result")
+            o3 = draw((n, f))
+            g3 = gpuarray.array(o3, context=ctx)
+            kio(gpuarray.array(b, context=ctx).transpose(1, 0), g3)
+            assert np.array_equal(np.asarray(g3), o3 - b.T), (n, f, "read and written")
+    kc = ga.GpuElemwise(ctx, "o = a", [arg("a", dtype, read=True), arg("o", dtype, write=True)], convert_f16=True)
+    for bsz, h, w, c in ((3, 32, 32, 3), (5, 17, 31, 7), (2, 40, 52, 2)):
+        x = draw((bsz, h, w, c))
+        out = gpuarray.empty((bsz, c, h, w), dtype, context=ctx)
+        kc(gpuarray.array(x, context=ctx).transpose(0, 3, 1, 2), out)
+        assert np.array_equal(np.asarray(out), x.transpose(0, 3, 1, 2)), (bsz, h, w, c)
+        y = draw((bsz, c, h, w))
+        out = gpuarray.empty((bsz, h, w, c), dtype, context=ctx)
+        kc(gpuarray.array(y, context=ctx).transpose(0, 2, 3, 1), out)
+        assert np.array_equal(np.asarray(out), y.transpose(0, 2, 3, 1)), (bsz, h, w, c, "back")
+
+
 @pytest.mark.parametrize("loose", [1, 0])
 @pytest.mark.parametrize("dtype", ["float32", "int32"])
 def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
