@@ -119,6 +119,15 @@ def main():
     check("elemwise narrow plane of 7 halves in registers, computed in floats",
           gen_e(b"", b"c = a + 1", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_HALF, 2), ElemwiseArg(b"c", GA_HALF, 4)),
                 2, 14, 7, 0b00100, 0b01 | (0b10 << 16)))
+    check("elemwise narrow plane of 3 in registers: bytes with the short dim innermost to floats in planes",
+          gen_e(b"", b"c = a * 0.5f", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_UBYTE, 2), ElemwiseArg(b"c", GA_FLOAT, 4)),
+                0, 14, 3, 0b10100, 0b01 | (0b10 << 16)))
+    check("elemwise narrow plane of 3 in registers: floats in planes to bytes with the short dim innermost, staged",
+          gen_e(b"", b"c = a", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_UBYTE, 4)),
+                0, 14, 3, 0b01110, 0b10 | (0b01 << 16)))
+    check("elemwise narrow plane of 4 in registers: bytes in planes to floats with the short dim innermost, staged",
+          gen_e(b"", b"c = a", 2, (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_UBYTE, 2), ElemwiseArg(b"c", GA_FLOAT, 4)),
+                0, 14, 4, 0b01110, 0b10 | (0b01 << 16)))
     iargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_FLOAT, 6))
     check("elemwise narrow plane of 4 in registers: an array read and written through the LDS",
           gen_e(b"", b"c = a + c", 2, iargs, 0, 14, 4, 0b01000, 0b10 | (0b01 << 16)))
@@ -227,7 +236,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "40 elementwise)" % (n + 20, m, t))
+          "43 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

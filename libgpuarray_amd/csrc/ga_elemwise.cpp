@@ -423,10 +423,12 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 // ---- narrow planes in registers -------------------------------------------------
 // Same parameters as the strided kernel with two or three dims (with three, the
 // first counts planes, ga_gx groups each).  One of the last two dims is
-// short (S, extent F <= 16, fixed in the text), the other long (L).  Every
-// array has elements of es = 2, 4 or 8 bytes, E = 16 / es to a chunk (the text
-// below says four).  A lane owns E adjacent positions along L and all F along S;
-// a group 256 E positions along L.
+// short (S, extent F <= 16, fixed in the text), the other long (L).  The
+// arrays have elements of 1, 2, 4 or 8 bytes; es is the smallest size among
+// them and E = 16 / es the elements of a chunk of that type (the text below
+// says four).  A lane owns E adjacent positions along L and all F along S, a
+// group 256 E positions along L; of an array of wider elements a lane's E
+// positions of a row are several chunks, one after the other.
 //  * The arrays in bmask have the short dim innermost: a lane's 4 F elements,
 //    and a group's 4096 F, lie one after the other in memory (stride of S one
 //    element, of L F elements: an (N, F) array taken as its transpose), on a
@@ -446,15 +448,25 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
                              unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask = 0,
                              unsigned smask = 0, unsigned nd = 2, unsigned es = 4) {
   std::string s;
-  const unsigned E = 16 / es;   // elements of a chunk = positions of a lane
+  const unsigned E = 16 / es;   // positions of a lane: the elements of a chunk of the smallest type (es bytes)
+  // chunks that a lane's E positions of one row take in an array, and elements of a chunk of it
+  auto cpr = [&](const ge_arg &a) { return (unsigned)(E * gpuarray_get_elsize(a.typecode) / 16); };
+  auto epc = [&](const ge_arg &a) { return (unsigned)(16 / gpuarray_get_elsize(a.typecode)); };
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const char *N = idx64 ? "ga_size" : "ga_uint";
   const unsigned ld = sd == nd - 1 ? nd - 2 : nd - 1;
-  const bool swz = (F & (F - 1)) == 0;
   emit_header(ge, s);
-  if (umask) appendf(s, "typedef ga_uint __attribute__((ext_vector_type(4), aligned(%u))) ga_chunk16u;\n", es < 4 ? es : 4);
-  if (smask) s += swz ? "#define GA_SLOT(q) ((q) ^ (((q) >> 3) & 7u))\n" : "#define GA_SLOT(q) (q)\n";
-  appendf(s, "#define GA_E %uu\n#define GA_ES %uu\n", E, es);
+  if (umask)
+    s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n"
+         "typedef ga_uint __attribute__((ext_vector_type(4), aligned(2))) ga_chunk16u2;\n"
+         "typedef ga_uint __attribute__((ext_vector_type(4), aligned(1))) ga_chunk16u1;\n";
+  auto loose_type = [&](const ge_arg &a) {
+    const size_t z = gpuarray_get_elsize(a.typecode);
+    return z >= 4 ? "ga_chunk16u" : z == 2 ? "ga_chunk16u2" : "ga_chunk16u1";
+  };
+  if (smask) s += "#define GA_SLOTX(q) ((q) ^ (((q) >> 3) & 7u))\n#define GA_SLOTP(q) (q)\n";
+  // (slots swizzled where a lane's chunks of the array are a power of two)
+  auto slot = [&](const ge_arg &a) { const unsigned m = F * cpr(a); return (m & (m - 1)) == 0 ? "GA_SLOTX" : "GA_SLOTP"; };
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
   ktypes.push_back(GA_SIZE);
   for (unsigned d = 1; d < nd; d++) {
@@ -494,7 +506,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset;\n", a.name.c_str(), a.name.c_str(),
             a.name.c_str());
     if (nd == 3) appendf(s, "%s_b += (%s)ga_o * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
-    if (in(smask, j)) appendf(s, "LOCAL_MEM ga_chunk16 %s_s[%u];\n", a.name.c_str(), 256 * F);
+    if (in(smask, j)) appendf(s, "LOCAL_MEM ga_chunk16 %s_s[%u];\n", a.name.c_str(), 256 * F * cpr(a));
   }
   appendf(s, "const %s ga_l0 = (%s)ga_pc * %uu;\n", N, N, 256 * E);
   appendf(s, "const %s ga_l4 = ga_l0 + LID_0 * %uu;\n", N, E);
@@ -508,8 +520,10 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
   // and of the chunked ones (element e of chunk y)
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
-    if (in(bmask, j)) appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r;\n", F, ctype(a.typecode), E * F, a.name.c_str());
-    else if (in(cmask, j)) appendf(s, "union { ga_chunk16 c; %s e[%u]; } %s_r[%u];\n", ctype(a.typecode), E, a.name.c_str(), F);
+    if (in(bmask, j))
+      appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r;\n", F * cpr(a), ctype(a.typecode), E * F, a.name.c_str());
+    else if (in(cmask, j))
+      appendf(s, "union { ga_chunk16 c[%u]; %s e[%u]; } %s_r[%u];\n", cpr(a), ctype(a.typecode), E, a.name.c_str(), F);
   }
   auto elem_at = [&](const ge_arg &a, const std::string &y, const std::string &l) {
     std::string e;
@@ -533,19 +547,21 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     if (in(smask, j)) {
       staged_in = true;
       if (a.writes()) staged_inout = true;
-      for (unsigned h = 0; h < F; h++) {
+      char eb[64];
+      snprintf(eb, sizeof(eb), "(ga_q * %uu + ga_e) * %uu", epc(a), 16 / epc(a));
+      for (unsigned h = 0; h < F * cpr(a); h++) {
         appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
         const std::string ptr = piece_at(a, "const ga_chunk16", "ga_q * 16u");
-        appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) %s_s[GA_SLOT(ga_q)] = %s(%s);\n", a.name.c_str(),
+        appendf(s, "if (ga_q * %uu + %uu < ga_cnt) %s_s[%s(ga_q)] = %s(%s);\n", epc(a), epc(a) - 1, a.name.c_str(), slot(a),
                 nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
-        appendf(s, "else for (ga_uint ga_e = 0; ga_e < GA_E; ga_e++) if (ga_q * GA_E + ga_e < ga_cnt) "
-                   "((%s *)%s_s)[GA_SLOT(ga_q) * GA_E + ga_e] = *(%s);\n",
-                ctype(a.typecode), a.name.c_str(), piece_at(a, ctype(a.typecode), "(ga_q * GA_E + ga_e) * GA_ES").c_str());
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < %uu; ga_e++) if (ga_q * %uu + ga_e < ga_cnt) "
+                   "((%s *)%s_s)[%s(ga_q) * %uu + ga_e] = *(%s);\n",
+                epc(a), epc(a), ctype(a.typecode), a.name.c_str(), slot(a), epc(a), piece_at(a, ctype(a.typecode), eb).c_str());
         s += "}\n";
       }
     } else if (in(bmask, j)) {
       s += "if (ga_full) {\n";
-      for (unsigned h = 0; h < F; h++) {
+      for (unsigned h = 0; h < F * cpr(a); h++) {
         std::string ptr;
         appendf(ptr, "(GLOBAL_MEM const ga_chunk16 *)(%s_b + (%s)ga_l4 * (%s)%s_str_%u) + %u", a.name.c_str(), I, I,
                 a.name.c_str(), ld, h);
@@ -562,14 +578,17 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         }
       s += "}\n";
     } else if (in(cmask, j)) {
-      const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+      const char *ct = in(umask, j) ? loose_type(a) : "ga_chunk16";
       for (unsigned y = 0; y < F; y++) {
         char yy[16];
         snprintf(yy, sizeof(yy), "%uu", y);
         std::string ptr;
         appendf(ptr, "(GLOBAL_MEM const %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
-        appendf(s, "if (ga_full) %s_r[%u].c = %s(%s); else {\n", a.name.c_str(), y,
-                nt ? "__builtin_nontemporal_load" : "*", ptr.c_str());
+        s += "if (ga_full) {";
+        for (unsigned c = 0; c < cpr(a); c++)
+          appendf(s, " %s_r[%u].c[%u] = %s((%s) + %u);", a.name.c_str(), y, c, nt ? "__builtin_nontemporal_load" : "*",
+                  ptr.c_str(), c);
+        s += " } else {\n";
         for (unsigned e = 0; e < E; e++) {
           char l[32];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
@@ -585,8 +604,8 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     for (size_t j = 0; j < ge->args.size(); j++) {
       const ge_arg &a = ge->args[j];
       if (!a.is_array() || !a.reads() || !in(smask, j)) continue;
-      for (unsigned h = 0; h < F; h++)
-        appendf(s, "%s_r.c[%u] = %s_s[GA_SLOT(LID_0 * %uu + %uu)];\n", a.name.c_str(), h, a.name.c_str(), F, h);
+      for (unsigned h = 0; h < F * cpr(a); h++)
+        appendf(s, "%s_r.c[%u] = %s_s[%s(LID_0 * %uu + %uu)];\n", a.name.c_str(), h, a.name.c_str(), slot(a), F * cpr(a), h);
     }
   }
   // the expression, position by position
@@ -625,8 +644,8 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     const ge_arg &a = ge->args[j];
     if (!a.is_array() || !a.writes() || !in(smask, j)) continue;
     staged_out = true;
-    for (unsigned h = 0; h < F; h++)
-      appendf(s, "%s_s[GA_SLOT(LID_0 * %uu + %uu)] = %s_r.c[%u];\n", a.name.c_str(), F, h, a.name.c_str(), h);
+    for (unsigned h = 0; h < F * cpr(a); h++)
+      appendf(s, "%s_s[%s(LID_0 * %uu + %uu)] = %s_r.c[%u];\n", a.name.c_str(), slot(a), F * cpr(a), h, a.name.c_str(), h);
   }
   if (staged_out) s += "local_barrier();\n";
   for (size_t j = 0; j < ge->args.size(); j++) {
@@ -634,20 +653,23 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
     if (!a.is_array() || !a.writes()) continue;
     const bool nt = (ntmask >> aidx[j]) & 1u;
     if (in(smask, j)) {
-      for (unsigned h = 0; h < F; h++) {
+      char eb[64];
+      snprintf(eb, sizeof(eb), "(ga_q * %uu + ga_e) * %uu", epc(a), 16 / epc(a));
+      for (unsigned h = 0; h < F * cpr(a); h++) {
         appendf(s, "{ const ga_uint ga_q = %uu + LID_0;\n", h * 256);
         const std::string ptr = piece_at(a, "ga_chunk16", "ga_q * 16u");
-        if (nt) appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) __builtin_nontemporal_store(%s_s[GA_SLOT(ga_q)], %s);\n",
-                        a.name.c_str(), ptr.c_str());
-        else appendf(s, "if (ga_q * GA_E + GA_E - 1u < ga_cnt) *(%s) = %s_s[GA_SLOT(ga_q)];\n", ptr.c_str(), a.name.c_str());
-        appendf(s, "else for (ga_uint ga_e = 0; ga_e < GA_E; ga_e++) if (ga_q * GA_E + ga_e < ga_cnt) "
-                   "*(%s) = ((%s *)%s_s)[GA_SLOT(ga_q) * GA_E + ga_e];\n",
-                piece_at(a, ctype(a.typecode), "(ga_q * GA_E + ga_e) * GA_ES").c_str(), ctype(a.typecode), a.name.c_str());
+        if (nt) appendf(s, "if (ga_q * %uu + %uu < ga_cnt) __builtin_nontemporal_store(%s_s[%s(ga_q)], %s);\n", epc(a),
+                        epc(a) - 1, a.name.c_str(), slot(a), ptr.c_str());
+        else appendf(s, "if (ga_q * %uu + %uu < ga_cnt) *(%s) = %s_s[%s(ga_q)];\n", epc(a), epc(a) - 1, ptr.c_str(),
+                     a.name.c_str(), slot(a));
+        appendf(s, "else for (ga_uint ga_e = 0; ga_e < %uu; ga_e++) if (ga_q * %uu + ga_e < ga_cnt) "
+                   "*(%s) = ((%s *)%s_s)[%s(ga_q) * %uu + ga_e];\n",
+                epc(a), epc(a), piece_at(a, ctype(a.typecode), eb).c_str(), ctype(a.typecode), a.name.c_str(), slot(a), epc(a));
         s += "}\n";
       }
     } else if (in(bmask, j)) {
       s += "if (ga_full) {\n";
-      for (unsigned h = 0; h < F; h++) {
+      for (unsigned h = 0; h < F * cpr(a); h++) {
         std::string ptr;
         appendf(ptr, "(GLOBAL_MEM ga_chunk16 *)(%s_b + (%s)ga_l4 * (%s)%s_str_%u) + %u", a.name.c_str(), I, I,
                 a.name.c_str(), ld, h);
@@ -665,14 +687,18 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         }
       s += "}\n";
     } else if (in(cmask, j)) {
-      const char *ct = in(umask, j) ? "ga_chunk16u" : "ga_chunk16";
+      const char *ct = in(umask, j) ? loose_type(a) : "ga_chunk16";
       for (unsigned y = 0; y < F; y++) {
         char yy[16];
         snprintf(yy, sizeof(yy), "%uu", y);
         std::string ptr;
         appendf(ptr, "(GLOBAL_MEM %s *)&%s", ct, elem_at(a, yy, "ga_l4").c_str());
-        if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store((%s)%s_r[%u].c, %s); else {\n", ct, a.name.c_str(), y, ptr.c_str());
-        else appendf(s, "if (ga_full) *(%s) = %s_r[%u].c; else {\n", ptr.c_str(), a.name.c_str(), y);
+        s += "if (ga_full) {";
+        for (unsigned c = 0; c < cpr(a); c++) {
+          if (nt) appendf(s, " __builtin_nontemporal_store((%s)%s_r[%u].c[%u], (%s) + %u);", ct, a.name.c_str(), y, c, ptr.c_str(), c);
+          else appendf(s, " *((%s) + %u) = %s_r[%u].c[%u];", ptr.c_str(), c, a.name.c_str(), y, c);
+        }
+        s += " } else {\n";
         for (unsigned e = 0; e < E; e++) {
           char l[32];
           snprintf(l, sizeof(l), "ga_l4 + %uu", e);
@@ -1987,8 +2013,8 @@ class strided_call {
     gpuarray_elemwise_collapse(na, &nd, dims.data(), ge->strp.data());
   }
 
-  // A plane with one short extent F (2 to 15) of two-, four- or eight-byte
-  // elements (all arrays alike; the figures are for four-byte ones) where some
+  // A plane with one short extent F (2 to 15) of elements of one to eight bytes
+  // (the figures are for four-byte ones) where some
   // array has the short dim innermost and another the long one - (N, F) taken as
   // its transpose, or written as one: too narrow for tiles through the LDS, which
   // F of 64 or 128 columns fill.  A lane takes four positions along the long dim
@@ -2025,10 +2051,19 @@ class strided_call {
     // lane of the strided kernel are a chunk of the result and coalesced single
     // elements of the operands (out = in.T of (4, N) 78 against 75 % of peak, of
     // (8, N) 79 against 74)
-    const size_t es = elsz[0], E = 16 / (es ? es : 1);
-    if ((es != 2 && es != 4 && es != 8) || (wide && es != 4)) return false;
+    // positions per lane: the elements of a chunk of the smallest type
+    size_t es = 16;
+    bool same = true;
+    for (unsigned k = 0; k < na; k++) {
+      if (elsz[k] != 1 && elsz[k] != 2 && elsz[k] != 4 && elsz[k] != 8) return false;
+      es = std::min(es, elsz[k]);
+      same = same && elsz[k] == elsz[0];
+    }
+    const size_t E = 16 / es;
+    if (wide && !(same && es == 4)) return false;
     // (two-byte elements: (8, N) -> (N, 8) of halves 54 % there, 73 % here)
-    if (sd == nd - 1 && F % E == 0 && es >= 4 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
+    if (sd == nd - 1 && F % E == 0 && same && es >= 4 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
+    size_t held = 0;   // 16-byte chunks in a lane's registers
     unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0;
     bool crossed = false;   // some array runs along the long dim and moves along the short one
     const unsigned long stage = TUNE(tn, ELEMWISE_NARROW_LDS, 2);   // 1: staged when read, 2: when written
@@ -2037,29 +2072,36 @@ class strided_call {
       unsigned k = 0;
       for (size_t i = 0; i < ge->args.size(); i++) {
         if (!ge->args[i].is_array()) continue;
-        if (elsz[k] != es || offs[k] % es != 0) return false;
+        const size_t ek = elsz[k], cprk = E * ek / 16;
+        if (offs[k] % ek != 0) return false;
         const bool base16 = offs[k] % 16 == 0 && (nd == 2 || strs[k][0] % 16 == 0);
-        if (nd == 3 && strs[k][0] % (ssize_t)es != 0) return false;
-        if (base16 && strs[k][sd] == (ssize_t)es && strs[k][ld] == (ssize_t)(es * F)) {
+        if (nd == 3 && strs[k][0] % (ssize_t)ek != 0) return false;
+        if (base16 && strs[k][sd] == (ssize_t)ek && strs[k][ld] == (ssize_t)(ek * F)) {
           bmask |= 1u << k;
+          held += F * cprk;
           const bool want = (ge->args[i].reads() ? (stage & 1) : 0) || (ge->args[i].writes() ? (stage & 2) : 0);
           if (wide) {
             lds += 260 * 4 * (F | 1);
             if (lds > 72 * 1024) return false;
-          } else if (want && lds + 4096 * F <= 64 * 1024) {
+          } else if (want && lds + 4096 * F * cprk <= 64 * 1024) {
             smask |= 1u << k;
-            lds += 4096 * F;
+            lds += 4096 * F * cprk;
           }
-        } else if (strs[k][ld] == (ssize_t)es && strs[k][sd] % (ssize_t)es == 0) {
+        } else if (strs[k][ld] == (ssize_t)ek && strs[k][sd] % (ssize_t)ek == 0) {
           const bool whole = base16 && strs[k][sd] % 16 == 0;
+          // a lane's positions of a row of wider elements are several chunks: written, they would
+          // reach memory as pieces of lines (bytes with the short dim innermost to floats in planes
+          // 157 us that way, 34 with single bytes fetched and whole chunks stored by the strided kernel)
+          if (cprk > 1 && ge->args[i].writes()) return false;
           cmask |= 1u << k;
+          held += F * cprk;
           if (strs[k][sd] != 0) crossed = true;
           if (!whole) umask |= 1u << k;
         }
         k++;
       }
     }
-    if (bmask == 0 || !crossed) return false;
+    if (bmask == 0 || !crossed || (!wide && held > TUNE(tn, ELEMWISE_NARROW_CHUNKS, 32))) return false;
     // arrays that take part once, whole, are streamed (the rest, broadcast or
     // overlapping, stays cacheable)
     {
@@ -2666,12 +2708,9 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // short dim, bit 2 streaming accesses, bit 3 the first kind of arrays through the LDS, bit 4 the second kind
   // on four-byte boundaries; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
   if (strided == 14) {
-    unsigned es = 4;   // the element size of every array: the first one's
+    unsigned es = 8;   // the smallest element size among the arrays
     for (const ge_arg &a : ge.args)
-      if (a.is_array()) {
-        es = (unsigned)gpuarray_get_elsize(a.typecode);
-        break;
-      }
+      if (a.is_array()) es = std::min(es, (unsigned)gpuarray_get_elsize(a.typecode));
     return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
                                    tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
                                    (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8), es).c_str());

@@ -112,6 +112,8 @@ def elemwise_cases():
         ("NHWC -> NCHW, (16, 1024, 1024, 3) (images, channels last to planes)", "o = a",
          [("a", f, (16, 1024, 1024, 3), T(0, 3, 1, 2))], (16, 3, 1024, 1024), f),
         ("NCHW -> NHWC, (16, 3, 1024, 1024)", "o = a", [("a", f, (16, 3, 1024, 1024), T(0, 2, 3, 1))], (16, 1024, 1024, 3), f),
+        ("NHWC -> NCHW of bytes, (16, 1024, 1024, 3)", "o = a", [("a", "uint8", (16, 1024, 1024, 3), T(0, 3, 1, 2))], (16, 3, 1024, 1024), "uint8"),
+        ("NCHW floats -> NHWC bytes, (16, 3, 1024, 1024)", "o = a", [("a", f, (16, 3, 1024, 1024), T(0, 2, 3, 1))], (16, 1024, 1024, 3), "uint8"),
         ("NHWC -> NCHW, (256, 56, 56, 8)", "o = a", [("a", f, (256, 56, 56, 8), T(0, 3, 1, 2))], (256, 8, 56, 56), f),
     ]
 

@@ -743,6 +743,38 @@ def test_very_narrow_planes_of_two_and_eight_byte_elements(ctx, knobs, dtype):
         assert np.array_equal(np.asarray(out), y.transpose(0, 2, 3, 1)), (bsz, h, w, c, "back")
 
 
+def test_very_narrow_planes_between_element_sizes(ctx, knobs):
+    """Narrow planes in registers with arrays of different element sizes (images of
+    bytes, halves and floats between channels last and channels first, also with one
+    byte per element throughout): a lane's positions are a chunk of the smallest
+    type, and of the wider arrays several chunks.  A wide result of wider elements
+    than the operand's is the strided kernel's (its rows would be stored in pieces);
+    checked all the same.  Against NumPy, exact (small integers)."""
+    knobs(ELEMWISE_NARROW_MIN=1024)
+    rng = np.random.default_rng(931)
+    for di, do in (("uint8", "uint8"), ("uint8", "float32"), ("float32", "uint8"), ("float16", "float32"),
+                   ("float32", "float16"), ("int16", "int64"), ("float64", "uint8")):
+        kc = ga.GpuElemwise(ctx, "o = a + 1", [arg("a", di, read=True), arg("o", do, write=True)], convert_f16=True)
+        for bsz, h, w, c in ((2, 40, 52, 3), (3, 33, 31, 4), (1, 70, 70, 7), (2, 64, 64, 1 + 14 * (di == do))):
+            x = rng.integers(0, 10, size=(bsz, h, w, c)).astype(di)
+            out = gpuarray.empty((bsz, c, h, w), do, context=ctx)
+            kc(gpuarray.array(x, context=ctx).transpose(0, 3, 1, 2), out)
+            assert np.array_equal(np.asarray(out), (x.transpose(0, 3, 1, 2) + 1).astype(do)), (di, do, bsz, h, w, c)
+            y = rng.integers(0, 10, size=(bsz, c, h, w)).astype(di)
+            out = gpuarray.empty((bsz, h, w, c), do, context=ctx)
+            kc(gpuarray.array(y, context=ctx).transpose(0, 2, 3, 1), out)
+            assert np.array_equal(np.asarray(out), (y.transpose(0, 2, 3, 1) + 1).astype(do)), (di, do, bsz, h, w, c, "back")
+        for n, f in ((4099, 3), (70001, 5)):
+            a = rng.integers(0, 10, size=(n, f)).astype(di)
+            out = gpuarray.empty((f, n), do, context=ctx)
+            kc(gpuarray.array(a, context=ctx).transpose(1, 0), out)
+            assert np.array_equal(np.asarray(out), (a.T + 1).astype(do)), (di, do, n, f)
+            b = rng.integers(0, 10, size=(f, n)).astype(di)
+            out = gpuarray.empty((n, f), do, context=ctx)
+            kc(gpuarray.array(b, context=ctx).transpose(1, 0), out)
+            assert np.array_equal(np.asarray(out), (b.T + 1).astype(do)), (di, do, n, f, "narrow result")
+
+
 @pytest.mark.parametrize("loose", [1, 0])
 @pytest.mark.parametrize("dtype", ["float32", "int32"])
 def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
