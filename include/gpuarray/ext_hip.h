@@ -96,7 +96,8 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * for three dims, planes one after the other), idx64 the
  * width of the offsets in bit 0, which of the two dims is the short one in bit
  * 1, the streaming hint in bit 2, the LDS for the first kind of arrays in bit
- * 3 and four-byte boundaries for the second kind in bit 4; tmask bits 0..15
+ * 3, four-byte boundaries for the second kind in bit 4 and the arrays of
+ * neither kind taken as constant along the long dim in bit 5; tmask bits 0..15
  * the arrays with the short dim innermost, bits 16.. those with the long one;
  * 15 the same arguments for a short extent of 17 to 64, whole through the LDS. */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,

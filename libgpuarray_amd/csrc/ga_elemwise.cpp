@@ -442,11 +442,12 @@ std::string gen_flat(const GpuElemwise *ge, std::vector<int> &ktypes, unsigned u
 //    chunk per position of S, side by side with the neighbouring lanes'; those
 //    also in umask through accesses that assume four-byte boundaries only (the
 //    element's own with two-byte elements).
+//  * Operands constant along L (zmask): one element per position of S, once.
 //  * Every other array one element at a time.
 // The last lane of a row takes what exists of its positions one by one.
 std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsigned sd, unsigned bmask,
                              unsigned cmask, unsigned ntmask, std::vector<int> &ktypes, unsigned umask = 0,
-                             unsigned smask = 0, unsigned nd = 2, unsigned es = 4) {
+                             unsigned smask = 0, unsigned nd = 2, unsigned es = 4, unsigned zmask = 0) {
   std::string s;
   const unsigned E = 16 / es;   // positions of a lane: the elements of a chunk of the smallest type (es bytes)
   // chunks that a lane's E positions of one row take in an array, and elements of a chunk of it
@@ -608,6 +609,17 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         appendf(s, "%s_r.c[%u] = %s_s[%s(LID_0 * %uu + %uu)];\n", a.name.c_str(), h, a.name.c_str(), slot(a), F * cpr(a), h);
     }
   }
+  // operands constant along L (in zmask, read only): one element per position of S, fetched once
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(zmask, j)) continue;
+    appendf(s, "%s %s_z[%u];\n", ctype(a.typecode), a.name.c_str(), F);
+    for (unsigned y = 0; y < F; y++) {
+      char yy[16];
+      snprintf(yy, sizeof(yy), "%uu", y);
+      appendf(s, "%s_z[%u] = %s;\n", a.name.c_str(), y, elem_at(a, yy, "0u").c_str());
+    }
+  }
   // the expression, position by position
   for (unsigned y = 0; y < F; y++)
     for (unsigned e = 0; e < E; e++) {
@@ -621,6 +633,7 @@ std::string gen_narrow_block(const GpuElemwise *ge, bool idx64, unsigned F, unsi
         std::string src;
         if (in(bmask, j)) appendf(src, "%s_r.e[%u]", a.name.c_str(), e * F + y);
         else if (in(cmask, j)) appendf(src, "%s_r[%u].e[%u]", a.name.c_str(), y, e);
+        else if (in(zmask, j)) appendf(src, "%s_z[%u]", a.name.c_str(), y);
         else src = elem_at(a, yy, l);
         emit_load(ge, s, a, src);
       }
@@ -2064,7 +2077,7 @@ class strided_call {
     // (two-byte elements: (8, N) -> (N, 8) of halves 54 % there, 73 % here)
     if (sd == nd - 1 && F % E == 0 && same && es >= 4 && TUNE(tn, ELEMWISE_NARROW_QUADS, 0) == 0) return false;
     size_t held = 0;   // 16-byte chunks in a lane's registers
-    unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0;
+    unsigned bmask = 0, cmask = 0, umask = 0, smask = 0, nt = 0, zmask_l = 0;
     bool crossed = false;   // some array runs along the long dim and moves along the short one
     const unsigned long stage = TUNE(tn, ELEMWISE_NARROW_LDS, 2);   // 1: staged when read, 2: when written
     size_t lds = 0;
@@ -2097,6 +2110,8 @@ class strided_call {
           held += F * cprk;
           if (strs[k][sd] != 0) crossed = true;
           if (!whole) umask |= 1u << k;
+        } else if (strs[k][ld] == 0 && !ge->args[i].writes()) {
+          zmask_l |= 1u << k;
         }
         k++;
       }
@@ -2118,15 +2133,15 @@ class strided_call {
     ltx = 0;
     if (groups > 0x7fffffffull || gx > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "%s%u:%zu:%u:%d:%x:%x:%x:%x:%x:%zu", wide ? "w" : "n", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask,
-             smask, es);
+    snprintf(key, sizeof(key), "%s%u:%zu:%u:%d:%x:%x:%x:%x:%x:%zu:%x", wide ? "w" : "n", nd, F, sd, idx64 ? 1 : 0, bmask, cmask, nt, umask,
+             smask, es, wide ? 0u : zmask_l);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
       std::string src = wide ? gen_narrow_staged(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, nd)
-                             : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd, (unsigned)es);
+                             : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd, (unsigned)es, zmask_l);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2706,14 +2721,15 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
     return strdup(gen_flat(&ge, ktypes, 0, -1, tmask, nd, (unsigned)idx64 & 0xffffu, (unsigned)idx64 >> 16).c_str());
   // 14: a narrow plane in registers: nd carries the short extent (plus 256: planes, three dims), idx64 bit 0 the offsets' width, bit 1 the
   // short dim, bit 2 streaming accesses, bit 3 the first kind of arrays through the LDS, bit 4 the second kind
-  // on four-byte boundaries; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
+  // on four-byte boundaries, bit 5 the arrays of neither kind constant along the long dim; tmask the arrays with the short dim innermost, its bits 16.. those with the long one
   if (strided == 14) {
     unsigned es = 8;   // the smallest element size among the arrays
     for (const ge_arg &a : ge.args)
       if (a.is_array()) es = std::min(es, (unsigned)gpuarray_get_elsize(a.typecode));
     return strdup(gen_narrow_block(&ge, (idx64 & 1) != 0, nd & 0xffu, (((unsigned)idx64 >> 1) & 1u) + (nd >> 8), tmask & 0xffffu,
                                    tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
-                                   (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8), es).c_str());
+                                   (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8), es,
+                                   (idx64 & 32) ? ~(tmask | (tmask >> 16)) & ((1u << ge.narray) - 1u) : 0u).c_str());
   }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)

@@ -764,6 +764,25 @@ def test_very_narrow_planes_between_element_sizes(ctx, knobs):
             out = gpuarray.empty((bsz, h, w, c), do, context=ctx)
             kc(gpuarray.array(y, context=ctx).transpose(0, 2, 3, 1), out)
             assert np.array_equal(np.asarray(out), (y.transpose(0, 2, 3, 1) + 1).astype(do)), (di, do, bsz, h, w, c, "back")
+        # a per-channel shift and factor fused into the change of layout (fetched once per channel)
+        kn = ga.GpuElemwise(ctx, "o = (a - m) * s", [arg("a", di, read=True), arg("m", do, read=True), arg("s", do, read=True),
+                                                      arg("o", do, write=True)], convert_f16=True)
+        for bsz, h, w, c in ((2, 40, 52, 3), (3, 33, 31, 5)):
+            x = rng.integers(4, 10, size=(bsz, h, w, c)).astype(di)
+            m = rng.integers(0, 4, size=(1, c, 1, 1)).astype(do)
+            f_ = rng.integers(1, 4, size=(1, c, 1, 1)).astype(do)
+            out = gpuarray.empty((bsz, c, h, w), do, context=ctx)
+            kn(gpuarray.array(x, context=ctx).transpose(0, 3, 1, 2), gpuarray.array(m, context=ctx),
+               gpuarray.array(f_, context=ctx), out, broadcast=True)
+            want = ((x.transpose(0, 3, 1, 2).astype(np.float64) - m) * f_).astype(do)
+            assert np.array_equal(np.asarray(out), want), (di, do, bsz, h, w, c, "normalised")
+            y = rng.integers(4, 10, size=(bsz, c, h, w)).astype(di)
+            ml, fl = m.reshape(1, 1, 1, c), f_.reshape(1, 1, 1, c)
+            out = gpuarray.empty((bsz, h, w, c), do, context=ctx)
+            kn(gpuarray.array(y, context=ctx).transpose(0, 2, 3, 1), gpuarray.array(ml, context=ctx),
+               gpuarray.array(fl, context=ctx), out, broadcast=True)
+            want = ((y.transpose(0, 2, 3, 1).astype(np.float64) - ml) * fl).astype(do)
+            assert np.array_equal(np.asarray(out), want), (di, do, bsz, h, w, c, "normalised, back")
         for n, f in ((4099, 3), (70001, 5)):
             a = rng.integers(0, 10, size=(n, f)).astype(di)
             out = gpuarray.empty((f, n), do, context=ctx)
