@@ -65,6 +65,27 @@ def test_strided_elementwise_with_64bit_offsets(ctx, big):
         assert np.array_equal(np.asarray(out[lo:hi]), hr[lo:hi] ^ np.uint8(0x5a)), (lo, hi)
 
 
+def test_narrow_planes_past_2p31_positions(ctx, big):
+    """The array taken as (N / 3, 3) bytes and moved to three planes and back: the
+    kernel that holds narrow planes in registers with 64-bit positions and offsets."""
+    host, dev = big
+    rows = N // 3
+    src = dev.reshape((rows, 3))
+    planes = gpuarray.empty((3, rows), "uint8", context=ctx)
+    k = ga.GpuElemwise(ctx, "c = a", [ga.arg("a", "uint8", read=True), ga.arg("c", "uint8", write=True)])
+    k(src.transpose(1, 0), planes)
+    h2 = host.reshape(rows, 3)
+    for lo, hi in windows(rows):
+        for c in range(3):
+            assert np.array_equal(np.asarray(planes[c][lo:hi]), h2[lo:hi, c]), (c, lo, hi)
+    back = gpuarray.empty((rows, 3), "uint8", context=ctx)
+    k(planes.transpose(1, 0), back)
+    flat = back.reshape((N,))
+    for lo, hi in windows(N):
+        assert np.array_equal(np.asarray(flat[lo:hi]), host[lo:hi]), (lo, hi)
+    assert int(np.asarray(R.sum(flat, dtype="uint64"))) == int(host.sum(dtype=np.uint64))
+
+
 def test_reductions_past_2p32(ctx, big):
     host, dev = big
     assert int(np.asarray(R.sum(dev, dtype="uint64"))) == int(host.sum(dtype=np.uint64))
