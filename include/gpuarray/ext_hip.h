@@ -99,7 +99,11 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * 3, four-byte boundaries for the second kind in bit 4 and the arrays of
  * neither kind taken as constant along the long dim in bit 5; tmask bits 0..15
  * the arrays with the short dim innermost, bits 16.. those with the long one;
- * 15 the same arguments for a short extent of 17 to 64, whole through the LDS. */
+ * 15 the same arguments for a short extent of 17 to 64, whole through the LDS;
+ * 16 tiles of short records: nd carries the record's elements (plus 256 for
+ * four dims), idx64 the width of the offsets in bit 0 and the streaming hint
+ * in bit 2, tmask bits 0..15 the arrays whose records follow one another
+ * along Y, bits 16.. those laid out like the result. */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,
                                            unsigned int n, void *args, int flags,
                                            int strided, unsigned int nd, int idx64,

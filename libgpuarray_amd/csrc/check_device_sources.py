@@ -130,6 +130,10 @@ def main():
                 0, 14, 4, 0b01110, 0b10 | (0b01 << 16)))
     check("elemwise narrow planes of 3 in registers, three dims: a per-channel operand fetched once per channel",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 14, 3 | 256, 0b101100, 0b001 | (0b100 << 16)))
+    check("elemwise tiles of records of 3: one operand's records along Y, the other's and the result's along X",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 16, 3, 0b100, 0b001 | (0b110 << 16)))
+    check("elemwise tiles of records of 20, four dims, 64-bit offsets, one operand element by element",
+          gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 16, 20 | 256, 0b001, 0b001 | (0b100 << 16)))
     iargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_FLOAT, 6))
     check("elemwise narrow plane of 4 in registers: an array read and written through the LDS",
           gen_e(b"", b"c = a + c", 2, iargs, 0, 14, 4, 0b01000, 0b10 | (0b01 << 16)))
@@ -238,7 +242,7 @@ def main():
               gen_t(chunks, a_tc, v_tc, i_tc, tnd))
         t += 1
     print("device sources compile for gfx950 (%d reduction variants, %d map-reduce, %d take1, "
-          "44 elementwise)" % (n + 20, m, t))
+          "46 elementwise)" % (n + 20, m, t))
 
 
 if __name__ == "__main__":

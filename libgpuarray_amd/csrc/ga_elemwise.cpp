@@ -907,6 +907,139 @@ std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, uns
   return s;
 }
 
+// ---- tiles of short records -------------------------------------------------------
+// Same parameters as the strided kernel with three or four dims: (planes,) Y, X
+// and a short inner dim of F four-byte elements with unit stride in every array
+// that has it - a record.  The result and the arrays laid out like it have their
+// records one after the other along X (stride of X = F elements); the arrays in
+// tmask, read only, along Y (stride of Y = F elements): matrices of records taken
+// as their transposes, (H, W, C) images turned, batch-major sequences of short
+// feature vectors made time-major.  A group owns T x T records: of each array in
+// tmask the T runs of T F contiguous elements (one per position of X) go to the
+// LDS, four elements per lane through accesses that assume four-byte boundaries;
+// then the lanes walk the T runs of the result (one per position of Y), four
+// elements each, take the transposed arrays' elements out of the LDS and move
+// the others directly.  ga_gx counts the tiles along X, ga_ltx those along Y.
+std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned F, unsigned T, unsigned tmask,
+                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes) {
+  std::string s;
+  const char *I = idx64 ? "ga_ssize" : "ga_int";
+  const unsigned R = T * F;          // elements of a run
+  const unsigned pitch = R + 4;      // of a run in the LDS
+  const unsigned dy = nd - 3, dx = nd - 2, dc = nd - 1;
+  emit_header(ge, s);
+  s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
+  ktypes.push_back(GA_SIZE);
+  for (unsigned d = 1; d < nd; d++) {
+    appendf(s, ", const ga_size dim%u", d);
+    ktypes.push_back(GA_SIZE);
+  }
+  std::vector<int> aidx(ge->args.size(), -1);
+  {
+    int k = 0;
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) aidx[j] = k++;
+  }
+  auto in = [&](unsigned mask, size_t j) { return aidx[j] >= 0 && ((mask >> aidx[j]) & 1u); };
+  for (const ge_arg &a : ge->args) {
+    if (a.is_array()) {
+      appendf(s, ", GLOBAL_MEM %s *%s_data, const ga_size %s_offset", ctype(a.typecode), a.name.c_str(), a.name.c_str());
+      ktypes.push_back(GA_BUFFER);
+      ktypes.push_back(GA_SIZE);
+      for (unsigned d = 0; d < nd; d++) {
+        appendf(s, ", const ga_ssize %s_str_%u", a.name.c_str(), d);
+        ktypes.push_back(GA_SSIZE);
+      }
+    } else {
+      appendf(s, ", %s %s", ctype(a.typecode), a.name.c_str());
+      ktypes.push_back(a.typecode);
+    }
+  }
+  s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n";
+  ktypes.push_back(GA_UINT);
+  ktypes.push_back(GA_UINT);
+  s += "ga_uint ga_g = GID_0;\nconst ga_uint ga_bx = ga_g % ga_gx; ga_g /= ga_gx;\nconst ga_uint ga_by = ga_g % ga_ltx; ga_g /= ga_ltx;\n";
+  appendf(s, "const ga_uint ga_x0 = ga_bx * %uu, ga_y0 = ga_by * %uu;\n", T, T);
+  appendf(s, "const ga_uint ga_nx = (ga_uint)dim%u - ga_x0 < %uu ? (ga_uint)dim%u - ga_x0 : %uu;\n", dx, T, dx, T);
+  appendf(s, "const ga_uint ga_ny = (ga_uint)dim%u - ga_y0 < %uu ? (ga_uint)dim%u - ga_y0 : %uu;\n", dy, T, dy, T);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!a.is_array()) continue;
+    appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset + (%s)ga_y0 * (%s)%s_str_%u + (%s)ga_x0 * (%s)%s_str_%u;\n",
+            a.name.c_str(), a.name.c_str(), a.name.c_str(), I, I, a.name.c_str(), dy, I, I, a.name.c_str(), dx);
+    if (nd == 4) appendf(s, "%s_b += (%s)ga_g * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
+    if (in(tmask, j)) appendf(s, "LOCAL_MEM %s %s_s[%u] __attribute__((aligned(16)));\n", ctype(a.typecode), a.name.c_str(), T * pitch);
+  }
+  // the transposed arrays' runs into the LDS: run r (position x0 + r of X), elements k .. k + 3 of it
+  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", T * R);
+  appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
+  appendf(s, "if (ga_r < ga_nx) {\n");
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(tmask, j)) continue;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    appendf(s, "{ GLOBAL_MEM const %s *ga_p = (GLOBAL_MEM const %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u) + ga_k;\n",
+            ctype(a.typecode), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dx);
+    appendf(s, "union { ga_chunk16u c; %s e[4]; } ga_v;\n", ctype(a.typecode));
+    appendf(s, "if (ga_k + 3u < ga_ny * %uu) ga_v.c = %s((GLOBAL_MEM const ga_chunk16u *)ga_p);\n", F,
+            nt ? "__builtin_nontemporal_load" : "*");
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_ny * %uu) ga_v.e[ga_e] = ga_p[ga_e];\n", F);
+    appendf(s, "*(ga_chunk16u *)&%s_s[ga_r * %uu + ga_k] = ga_v.c; }\n", a.name.c_str(), pitch);
+  }
+  s += "}\n}\nlocal_barrier();\n";
+  // the result's runs: run r (position y0 + r of Y), elements k .. k + 3 of it (record k / F, element k % F)
+  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", T * R);
+  appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
+  appendf(s, "if (ga_r >= ga_ny || ga_k >= ga_nx * %uu) continue;\n", F);
+  appendf(s, "const bool ga_full = ga_k + 3u < ga_nx * %uu;\n", F);
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(pmask, j)) continue;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    appendf(s, "GLOBAL_MEM %s *%s_p = (GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u) + ga_k;\n", ctype(a.typecode),
+            a.name.c_str(), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dy);
+    appendf(s, "union { ga_chunk16u c; %s e[4]; } %s_v;\n", ctype(a.typecode), a.name.c_str());
+    if (a.reads()) {
+      appendf(s, "if (ga_full) %s_v.c = %s((GLOBAL_MEM const ga_chunk16u *)%s_p);\n", a.name.c_str(),
+              nt ? "__builtin_nontemporal_load" : "*", a.name.c_str());
+      appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_nx * %uu) %s_v.e[ga_e] = %s_p[ga_e];\n", F,
+              a.name.c_str(), a.name.c_str());
+    }
+  }
+  for (unsigned e = 0; e < 4; e++) {
+    appendf(s, "if (ga_k + %uu < ga_nx * %uu) {\n", e, F);
+    appendf(s, "const ga_uint ga_x = (ga_k + %uu) / %uu, ga_c = ga_k + %uu - ga_x * %uu;\n", e, F, e, F);
+    auto place = [&](size_t j) {
+      const ge_arg &a = ge->args[j];
+      std::string x;
+      if (in(tmask, j)) appendf(x, "%s_s[ga_x * %uu + ga_r * %uu + ga_c]", a.name.c_str(), pitch, F);
+      else if (in(pmask, j)) appendf(x, "%s_v.e[%u]", a.name.c_str(), e);
+      else appendf(x, "*(GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u + (%s)ga_x * (%s)%s_str_%u + (%s)ga_c * (%s)%s_str_%u)",
+                   ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dy, I, I, a.name.c_str(), dx, I, I, a.name.c_str(), dc);
+      return x;
+    };
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array()) emit_load(ge, s, ge->args[j], place(j));
+    s += ge->expr;
+    s += ";\n";
+    for (size_t j = 0; j < ge->args.size(); j++)
+      if (ge->args[j].is_array() && ge->args[j].writes()) emit_store(ge, s, ge->args[j], place(j));
+    s += "}\n";
+  }
+  for (size_t j = 0; j < ge->args.size(); j++) {
+    const ge_arg &a = ge->args[j];
+    if (!in(pmask, j) || !a.writes()) continue;
+    const bool nt = (ntmask >> aidx[j]) & 1u;
+    if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store(%s_v.c, (GLOBAL_MEM ga_chunk16u *)%s_p);\n", a.name.c_str(), a.name.c_str());
+    else appendf(s, "if (ga_full) *(GLOBAL_MEM ga_chunk16u *)%s_p = %s_v.c;\n", a.name.c_str(), a.name.c_str());
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_nx * %uu) %s_p[ga_e] = %s_v.e[ga_e];\n", F,
+            a.name.c_str(), a.name.c_str());
+  }
+  s += "}\n}\n";
+  return s;
+}
+
 // ---- strided kernel -------------------------------------------------------------
 // elem(dim0..dim{nd-1}, {data, byte offset, str_0..str_{nd-1} | scalar}...,
 //      ga_gx, ga_ltx)
@@ -1942,6 +2075,10 @@ class strided_call {
       int err = GA_NO_ERROR;
       if (narrow_plane_in_registers(err)) return err;
     }
+    {
+      int err = GA_NO_ERROR;
+      if (tiles_of_short_records(err)) return err;
+    }
     find_transposed_operands();
     choose_offset_width();
     choose_vector_access();
@@ -2142,6 +2279,72 @@ class strided_call {
       std::vector<int> ktypes;
       std::string src = wide ? gen_narrow_staged(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, nd)
                              : gen_narrow_block(ge, idx64, (unsigned)F, sd, bmask, cmask, nt, ktypes, umask, smask, nd, (unsigned)es, zmask_l);
+      GpuKernel nk = {nullptr, nullptr};
+      err = build_kernel(ge, &nk, src, ktypes);
+      if (err != GA_NO_ERROR) return true;
+      kernel = &ge->k_strided.emplace(key, nk).first->second;
+    }
+    err = launch();
+    return true;
+  }
+
+  // Matrices of short records taken as their transposes (gen_record_tiles): three
+  // dims (four with planes), the inner one of 2 to 64 four-byte elements with unit
+  // stride; the result's records follow one another along X, a read-only
+  // operand's along Y.  Neither counts as a transposed operand for the tiles (both
+  // have their smallest stride on the inner dim), and a lane of the strided
+  // kernels walks the short inner dim.
+  // (side of a tile in records; records of 8 floats 69 / 76 % of peak with 32 / 16, of 32 69 / 75 % with 16 / 8,
+  // of 2 67 / 74 / 59 % with 64 / 32 / 16)
+  static unsigned record_tile_side(size_t F) { return F <= 7 ? 32 : F <= 31 ? 16 : 8; }
+  bool tiles_of_short_records(int &err) {
+    const unsigned long fmax = TUNE(tn, ELEMWISE_RECORDS, 64);
+    if (fmax == 0 || (nd != 3 && nd != 4) || na > 31) return false;
+    const size_t F = dims[nd - 1], X = dims[nd - 2], Y = dims[nd - 3];
+    if (F < 2 || F > fmax || F > 64 || X < 32 || Y < 32 || X > 0x7fffffffull || Y > 0x7fffffffull ||
+        n < TUNE(tn, ELEMWISE_RECORDS_MIN, 65536))
+      return false;
+    unsigned tm = 0, pm = 0;
+    {
+      unsigned k = 0;
+      for (size_t i = 0; i < ge->args.size(); i++) {
+        if (!ge->args[i].is_array()) continue;
+        if (elsz[k] != 4 || offs[k] % 4 != 0) return false;
+        for (unsigned j = 0; j < nd; j++)
+          if (strs[k][j] % 4 != 0) return false;
+        const bool unit = strs[k][nd - 1] == 4;
+        if (unit && strs[k][nd - 2] == (ssize_t)(4 * F)) pm |= 1u << k;
+        else if (unit && strs[k][nd - 3] == (ssize_t)(4 * F) && !ge->args[i].writes()) tm |= 1u << k;
+        else if (ge->args[i].writes()) return false;
+        k++;
+      }
+    }
+    if (tm == 0 || !((pm >> outk) & 1u)) return false;
+    unsigned T = record_tile_side(F);
+    {
+      const unsigned long ft = TUNE(tn, ELEMWISE_RECORDS_TILE, 0);
+      if (ft == 8 || ft == 16 || ft == 32 || ft == 64) T = (unsigned)ft;
+    }
+    size_t lds = 0;
+    for (unsigned k = 0; k < na; k++)
+      if ((tm >> k) & 1u) lds += (size_t)T * (T * F + 4) * 4;
+    if (lds > 80 * 1024) return false;
+    choose_offset_width();
+    const unsigned long ntm = TUNE(tn, ELEMWISE_RECORDS_NT, 3);
+    const unsigned nt = ((ntm & 1) ? pm : 0u) | ((ntm & 2) ? tm : 0u);
+    gx = (X + T - 1) / T;
+    const size_t gy = (Y + T - 1) / T;
+    ltx = (unsigned)gy;
+    groups = gx * gy * (nd == 4 ? dims[0] : 1);
+    if (groups > 0x7fffffffull) return false;
+    char key[64];
+    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x", nd, F, T, idx64 ? 1 : 0, tm, pm, nt);
+    auto it = ge->k_strided.find(key);
+    if (it != ge->k_strided.end()) {
+      kernel = &it->second;
+    } else {
+      std::vector<int> ktypes;
+      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2730,6 +2933,14 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
                                    tmask >> 16, (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 16) ? tmask >> 16 : 0u,
                                    (idx64 & 8) ? tmask & 0xffffu : 0u, 2 + (nd >> 8), es,
                                    (idx64 & 32) ? ~(tmask | (tmask >> 16)) & ((1u << ge.narray) - 1u) : 0u).c_str());
+  }
+  // 16: tiles of short records: nd carries the record's elements (plus 256: planes, four dims), idx64 bit 0 the
+  // offsets' width, bit 2 streaming accesses; tmask the arrays whose records follow one another along Y, its bits
+  // 16.. those laid out like the result
+  if (strided == 16) {
+    const unsigned F = nd & 0xffu, T = F <= 7 ? 32 : F <= 31 ? 16 : 8;
+    return strdup(gen_record_tiles(&ge, 3 + (nd >> 8), (idx64 & 1) != 0, F, T, tmask & 0xffffu, tmask >> 16,
+                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes).c_str());
   }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)

@@ -114,6 +114,10 @@ def elemwise_cases():
         ("NCHW -> NHWC, (16, 3, 1024, 1024)", "o = a", [("a", f, (16, 3, 1024, 1024), T(0, 2, 3, 1))], (16, 1024, 1024, 3), f),
         ("NHWC -> NCHW of bytes, (16, 1024, 1024, 3)", "o = a", [("a", "uint8", (16, 1024, 1024, 3), T(0, 3, 1, 2))], (16, 3, 1024, 1024), "uint8"),
         ("NCHW floats -> NHWC bytes, (16, 3, 1024, 1024)", "o = a", [("a", f, (16, 3, 1024, 1024), T(0, 2, 3, 1))], (16, 1024, 1024, 3), "uint8"),
+        ("(4096, 4096, 4) -> transpose (1, 0, 2) (a matrix of records of four floats)", "o = a",
+         [("a", f, (4096, 4096, 4), T(1, 0, 2))], (4096, 4096, 4), f),
+        ("(4729, 4729, 3) -> transpose (1, 0, 2) (an image turned; rows that are no whole lines)", "o = a",
+         [("a", f, (4729, 4729, 3), T(1, 0, 2))], (4729, 4729, 3), f),
         ("NHWC -> NCHW, (256, 56, 56, 8)", "o = a", [("a", f, (256, 56, 56, 8), T(0, 3, 1, 2))], (256, 8, 56, 56), f),
     ]
 

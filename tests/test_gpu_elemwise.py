@@ -794,6 +794,39 @@ def test_very_narrow_planes_between_element_sizes(ctx, knobs):
             assert np.array_equal(np.asarray(out), (b.T + 1).astype(do)), (di, do, n, f, "narrow result")
 
 
+@pytest.mark.parametrize("tile,nt", [(0, 3), (8, 0), (64, 1), (16, 2)])
+def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, nt):
+    """(X, Y, f) with a short inner dim taken as (Y, X, f): images turned, sequences
+    of short feature vectors between batch-major and time-major.  Tiles of records
+    through the LDS (ELEMWISE_RECORDS; side of a tile ELEMWISE_RECORDS_TILE): whole
+    and cut tiles, a second operand laid out like the result, a broadcast operand,
+    planes, and an operand whose records start inside a larger buffer.  Floats and
+    32-bit integers against NumPy, exact."""
+    knobs(ELEMWISE_RECORDS_TILE=tile, ELEMWISE_RECORDS_NT=nt, ELEMWISE_RECORDS_MIN=1)
+    rng = np.random.default_rng(950 + tile)
+    for dtype in ("float32", "int32"):
+        k = ga.GpuElemwise(ctx, "o = a + b * r", [arg("a", dtype, read=True), arg("b", dtype, read=True),
+                                                   arg("r", dtype, read=True), arg("o", dtype, write=True)])
+        kc = ga.GpuElemwise(ctx, "o = a", [arg("a", dtype, read=True), arg("o", dtype, write=True)])
+        draw = lambda shape: rng.integers(-9, 10, size=shape).astype(dtype)
+        for f in (2, 3, 5, 8, 13, 16, 33, 64):
+            if tile == 64 and f > 4:
+                continue          # (more LDS than a group has)
+            for ny, nx in ((32, 32), (100, 257), (333, 64), (65, 1000)):
+                a = draw((nx, ny, f))
+                b = draw((ny, nx, f))
+                r = draw((1, nx, 1))
+                out = gpuarray.empty((ny, nx, f), dtype, context=ctx)
+                k(gpuarray.array(a, context=ctx).transpose(1, 0, 2), gpuarray.array(b, context=ctx),
+                  gpuarray.array(r, context=ctx), out, broadcast=True)
+                assert np.array_equal(np.asarray(out), a.transpose(1, 0, 2) + b * r), (dtype, f, ny, nx)
+                aroot = draw((3, nx, ny + 2, f))
+                gv, _ = to_gpu_view(aroot[:, :, 1:ny + 1, :], ctx)
+                out2 = gpuarray.empty((3, ny, nx, f), dtype, context=ctx)
+                kc(gv.transpose(0, 2, 1, 3), out2)
+                assert np.array_equal(np.asarray(out2), aroot[:, :, 1:ny + 1, :].transpose(0, 2, 1, 3)), (dtype, f, ny, nx, "planes")
+
+
 @pytest.mark.parametrize("loose", [1, 0])
 @pytest.mark.parametrize("dtype", ["float32", "int32"])
 def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
