@@ -920,12 +920,20 @@ std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, uns
 // then the lanes walk the T runs of the result (one per position of Y), four
 // elements each, take the transposed arrays' elements out of the LDS and move
 // the others directly.  ga_gx counts the tiles along X, ga_ltx those along Y.
+// skew >= 0 (an array laid out like the result, normally the result): the window
+// of a tile on a row is moved left by the 0 to 15 elements that put its first
+// element on a 64-byte block of that array's row, so that a group stores whole
+// blocks also where rows are no whole blocks long; the staged runs cover the
+// records such a window can reach, and the grid has tiles for 15 more elements
+// (T F must then be a multiple of 16: the windows of neighbouring tiles meet).
 std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned F, unsigned T, unsigned tmask,
-                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes) {
+                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes, int skew = -1) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const unsigned R = T * F;          // elements of a run
   const unsigned pitch = R + 4;      // of a run in the LDS
+  const unsigned extra = skew >= 0 ? (15 + F - 1) / F + 1 : 0;   // records that a moved window can reach beyond the tile's
+  const unsigned TS = T + extra;     // runs staged per transposed array
   const unsigned dy = nd - 3, dx = nd - 2, dc = nd - 1;
   emit_header(ge, s);
   s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
@@ -936,10 +944,14 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
     ktypes.push_back(GA_SIZE);
   }
   std::vector<int> aidx(ge->args.size(), -1);
+  int skew_j = -1;
   {
     int k = 0;
     for (size_t j = 0; j < ge->args.size(); j++)
-      if (ge->args[j].is_array()) aidx[j] = k++;
+      if (ge->args[j].is_array()) {
+        if (k == skew) skew_j = (int)j;
+        aidx[j] = k++;
+      }
   }
   auto in = [&](unsigned mask, size_t j) { return aidx[j] >= 0 && ((mask >> aidx[j]) & 1u); };
   for (const ge_arg &a : ge->args) {
@@ -960,26 +972,30 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
   ktypes.push_back(GA_UINT);
   ktypes.push_back(GA_UINT);
   s += "ga_uint ga_g = GID_0;\nconst ga_uint ga_bx = ga_g % ga_gx; ga_g /= ga_gx;\nconst ga_uint ga_by = ga_g % ga_ltx; ga_g /= ga_ltx;\n";
-  appendf(s, "const ga_uint ga_x0 = ga_bx * %uu, ga_y0 = ga_by * %uu;\n", T, T);
-  appendf(s, "const ga_uint ga_nx = (ga_uint)dim%u - ga_x0 < %uu ? (ga_uint)dim%u - ga_x0 : %uu;\n", dx, T, dx, T);
+  // the tile: elements k0 .. k0 + R - 1 of the result's rows y0 .. y0 + T - 1; the transposed
+  // arrays' records from xs on are staged
+  appendf(s, "const ga_uint ga_k0 = ga_bx * %uu, ga_y0 = ga_by * %uu, ga_xf = (ga_uint)dim%u * %uu;\n", R, T, dx, F);
+  if (skew >= 0) appendf(s, "const ga_uint ga_xs = ga_k0 >= 15u ? (ga_k0 - 15u) / %uu : 0u;\n", F);
+  else appendf(s, "const ga_uint ga_xs = ga_bx * %uu;\n", T);
   appendf(s, "const ga_uint ga_ny = (ga_uint)dim%u - ga_y0 < %uu ? (ga_uint)dim%u - ga_y0 : %uu;\n", dy, T, dy, T);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!a.is_array()) continue;
-    appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset + (%s)ga_y0 * (%s)%s_str_%u + (%s)ga_x0 * (%s)%s_str_%u;\n",
-            a.name.c_str(), a.name.c_str(), a.name.c_str(), I, I, a.name.c_str(), dy, I, I, a.name.c_str(), dx);
+    appendf(s, "GLOBAL_MEM char *%s_b = (GLOBAL_MEM char *)%s_data + %s_offset + (%s)ga_y0 * (%s)%s_str_%u;\n", a.name.c_str(),
+            a.name.c_str(), a.name.c_str(), I, I, a.name.c_str(), dy);
     if (nd == 4) appendf(s, "%s_b += (%s)ga_g * (%s)%s_str_0;\n", a.name.c_str(), I, I, a.name.c_str());
-    if (in(tmask, j)) appendf(s, "LOCAL_MEM %s %s_s[%u] __attribute__((aligned(16)));\n", ctype(a.typecode), a.name.c_str(), T * pitch);
+    if (in(tmask, j))
+      appendf(s, "LOCAL_MEM %s %s_s[%u] __attribute__((aligned(16)));\n", ctype(a.typecode), a.name.c_str(), TS * pitch);
   }
-  // the transposed arrays' runs into the LDS: run r (position x0 + r of X), elements k .. k + 3 of it
-  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", T * R);
+  // the transposed arrays' runs into the LDS: run r (record xs + r along X), elements k .. k + 3 of it
+  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", TS * R);
   appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
-  appendf(s, "if (ga_r < ga_nx) {\n");
+  appendf(s, "if (ga_xs + ga_r < (ga_uint)dim%u) {\n", dx);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!in(tmask, j)) continue;
     const bool nt = (ntmask >> aidx[j]) & 1u;
-    appendf(s, "{ GLOBAL_MEM const %s *ga_p = (GLOBAL_MEM const %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u) + ga_k;\n",
+    appendf(s, "{ GLOBAL_MEM const %s *ga_p = (GLOBAL_MEM const %s *)(%s_b + (%s)(ga_xs + ga_r) * (%s)%s_str_%u) + ga_k;\n",
             ctype(a.typecode), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dx);
     appendf(s, "union { ga_chunk16u c; %s e[4]; } ga_v;\n", ctype(a.typecode));
     appendf(s, "if (ga_k + 3u < ga_ny * %uu) ga_v.c = %s((GLOBAL_MEM const ga_chunk16u *)ga_p);\n", F,
@@ -988,32 +1004,43 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
     appendf(s, "*(ga_chunk16u *)&%s_s[ga_r * %uu + ga_k] = ga_v.c; }\n", a.name.c_str(), pitch);
   }
   s += "}\n}\nlocal_barrier();\n";
-  // the result's runs: run r (position y0 + r of Y), elements k .. k + 3 of it (record k / F, element k % F)
+  // the result's rows: row r (position y0 + r of Y), elements kk .. kk + 3 (record kk / F, element kk % F);
+  // with moved windows a row's first element is the one on a 64-byte block of the array in skew at
+  // or below element k0, and elements before the row wrap to huge indices that fail the extent test
   appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", T * R);
   appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
-  appendf(s, "if (ga_r >= ga_ny || ga_k >= ga_nx * %uu) continue;\n", F);
-  appendf(s, "const bool ga_full = ga_k + 3u < ga_nx * %uu;\n", F);
+  s += "if (ga_r >= ga_ny) continue;\n";
+  if (skew_j >= 0) {
+    const ge_arg &a = ge->args[skew_j];
+    appendf(s, "const ga_uint ga_sh = (ga_uint)(((ga_size)(%s_b + (%s)ga_r * (%s)%s_str_%u) >> 2) + ga_k0) & 15u;\n",
+            a.name.c_str(), I, I, a.name.c_str(), dy);
+    s += "const ga_uint ga_kk = ga_k0 - ga_sh + ga_k;\n";
+  } else {
+    s += "const ga_uint ga_kk = ga_k0 + ga_k;\n";
+  }
+  s += "if (ga_kk >= ga_xf && ga_kk + 3u >= ga_xf) continue;\n";
+  s += "const bool ga_full = ga_kk < ga_xf && ga_kk + 3u < ga_xf;\n";
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!in(pmask, j)) continue;
     const bool nt = (ntmask >> aidx[j]) & 1u;
-    appendf(s, "GLOBAL_MEM %s *%s_p = (GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u) + ga_k;\n", ctype(a.typecode),
+    appendf(s, "GLOBAL_MEM %s *%s_p = (GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u);\n", ctype(a.typecode),
             a.name.c_str(), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dy);
     appendf(s, "union { ga_chunk16u c; %s e[4]; } %s_v;\n", ctype(a.typecode), a.name.c_str());
     if (a.reads()) {
-      appendf(s, "if (ga_full) %s_v.c = %s((GLOBAL_MEM const ga_chunk16u *)%s_p);\n", a.name.c_str(),
+      appendf(s, "if (ga_full) %s_v.c = %s((GLOBAL_MEM const ga_chunk16u *)(%s_p + ga_kk));\n", a.name.c_str(),
               nt ? "__builtin_nontemporal_load" : "*", a.name.c_str());
-      appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_nx * %uu) %s_v.e[ga_e] = %s_p[ga_e];\n", F,
+      appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_v.e[ga_e] = %s_p[(ga_uint)(ga_kk + ga_e)];\n",
               a.name.c_str(), a.name.c_str());
     }
   }
   for (unsigned e = 0; e < 4; e++) {
-    appendf(s, "if (ga_k + %uu < ga_nx * %uu) {\n", e, F);
-    appendf(s, "const ga_uint ga_x = (ga_k + %uu) / %uu, ga_c = ga_k + %uu - ga_x * %uu;\n", e, F, e, F);
+    appendf(s, "if ((ga_uint)(ga_kk + %uu) < ga_xf) {\n", e);
+    appendf(s, "const ga_uint ga_x = (ga_uint)(ga_kk + %uu) / %uu, ga_c = (ga_uint)(ga_kk + %uu) - ga_x * %uu;\n", e, F, e, F);
     auto place = [&](size_t j) {
       const ge_arg &a = ge->args[j];
       std::string x;
-      if (in(tmask, j)) appendf(x, "%s_s[ga_x * %uu + ga_r * %uu + ga_c]", a.name.c_str(), pitch, F);
+      if (in(tmask, j)) appendf(x, "%s_s[(ga_x - ga_xs) * %uu + ga_r * %uu + ga_c]", a.name.c_str(), pitch, F);
       else if (in(pmask, j)) appendf(x, "%s_v.e[%u]", a.name.c_str(), e);
       else appendf(x, "*(GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u + (%s)ga_x * (%s)%s_str_%u + (%s)ga_c * (%s)%s_str_%u)",
                    ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dy, I, I, a.name.c_str(), dx, I, I, a.name.c_str(), dc);
@@ -1031,9 +1058,9 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
     const ge_arg &a = ge->args[j];
     if (!in(pmask, j) || !a.writes()) continue;
     const bool nt = (ntmask >> aidx[j]) & 1u;
-    if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store(%s_v.c, (GLOBAL_MEM ga_chunk16u *)%s_p);\n", a.name.c_str(), a.name.c_str());
-    else appendf(s, "if (ga_full) *(GLOBAL_MEM ga_chunk16u *)%s_p = %s_v.c;\n", a.name.c_str(), a.name.c_str());
-    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_nx * %uu) %s_p[ga_e] = %s_v.e[ga_e];\n", F,
+    if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store(%s_v.c, (GLOBAL_MEM ga_chunk16u *)(%s_p + ga_kk));\n", a.name.c_str(), a.name.c_str());
+    else appendf(s, "if (ga_full) *(GLOBAL_MEM ga_chunk16u *)(%s_p + ga_kk) = %s_v.c;\n", a.name.c_str(), a.name.c_str());
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_p[(ga_uint)(ga_kk + ga_e)] = %s_v.e[ga_e];\n",
             a.name.c_str(), a.name.c_str());
   }
   s += "}\n}\n";
@@ -2325,26 +2352,41 @@ class strided_call {
       const unsigned long ft = TUNE(tn, ELEMWISE_RECORDS_TILE, 0);
       if (ft == 8 || ft == 16 || ft == 32 || ft == 64) T = (unsigned)ft;
     }
+    // Windows moved onto the result's 64-byte blocks where its rows, or the tiles' pieces of them,
+    // do not start on such blocks by themselves: (4729, 4729, 3) floats transposed (1, 0, 2) 41 ->
+    // 54 % of peak, (3663, 3663, 5) 47 -> 59 %, (2590, 2590, 10) 54 -> 61 % ((4736, 4736, 3), whole
+    // lines, runs at 73 %); moved windows on rows of whole blocks cost 6 to 10 points.
+    if (X * F + 15 + (size_t)T * F >= 0x7fffffffull) return false;
+    bool skewed = offs[outk] % 64 != 0 || ((size_t)T * F * 4) % 64 != 0;
+    for (unsigned j = 0; j + 2 < nd; j++) skewed = skewed || strs[outk][j] % 64 != 0;
+    {
+      const unsigned long sk = TUNE(tn, ELEMWISE_RECORDS_SKEW, 1);
+      // (records of 33 and 50 floats on such rows: 59 and 60 % rectangular, 59 and 58 % moved)
+      skewed = sk == 2 || (sk == 1 && skewed && F <= 31);
+    }
+    // (the windows of neighbouring tiles meet only if a tile's piece of a row is whole blocks)
+    if (skewed && ((size_t)T * F) % 16 != 0) T = 16;
+    const unsigned extra = skewed ? (unsigned)((15 + F - 1) / F + 1) : 0;
     size_t lds = 0;
     for (unsigned k = 0; k < na; k++)
-      if ((tm >> k) & 1u) lds += (size_t)T * (T * F + 4) * 4;
+      if ((tm >> k) & 1u) lds += (size_t)(T + extra) * (T * F + 4) * 4;
     if (lds > 80 * 1024) return false;
     choose_offset_width();
     const unsigned long ntm = TUNE(tn, ELEMWISE_RECORDS_NT, 3);
     const unsigned nt = ((ntm & 1) ? pm : 0u) | ((ntm & 2) ? tm : 0u);
-    gx = (X + T - 1) / T;
+    gx = (X * F + (skewed ? 15 : 0) + (size_t)T * F - 1) / ((size_t)T * F);
     const size_t gy = (Y + T - 1) / T;
     ltx = (unsigned)gy;
     groups = gx * gy * (nd == 4 ? dims[0] : 1);
     if (groups > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x", nd, F, T, idx64 ? 1 : 0, tm, pm, nt);
+    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x:%d", nd, F, T, idx64 ? 1 : 0, tm, pm, nt, skewed ? outk : -1);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes);
+      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes, skewed ? outk : -1);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2935,12 +2977,12 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
                                    (idx64 & 32) ? ~(tmask | (tmask >> 16)) & ((1u << ge.narray) - 1u) : 0u).c_str());
   }
   // 16: tiles of short records: nd carries the record's elements (plus 256: planes, four dims), idx64 bit 0 the
-  // offsets' width, bit 2 streaming accesses; tmask the arrays whose records follow one another along Y, its bits
-  // 16.. those laid out like the result
+  // offsets' width, bit 2 streaming accesses, bit 3 windows moved onto the last array's 64-byte blocks; tmask the
+  // arrays whose records follow one another along Y, its bits 16.. those laid out like the result
   if (strided == 16) {
     const unsigned F = nd & 0xffu, T = F <= 7 ? 32 : F <= 31 ? 16 : 8;
     return strdup(gen_record_tiles(&ge, 3 + (nd >> 8), (idx64 & 1) != 0, F, T, tmask & 0xffffu, tmask >> 16,
-                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes).c_str());
+                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 8) ? (int)ge.narray - 1 : -1).c_str());
   }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)

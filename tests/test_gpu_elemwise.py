@@ -794,15 +794,18 @@ def test_very_narrow_planes_between_element_sizes(ctx, knobs):
             assert np.array_equal(np.asarray(out), (b.T + 1).astype(do)), (di, do, n, f, "narrow result")
 
 
-@pytest.mark.parametrize("tile,nt", [(0, 3), (8, 0), (64, 1), (16, 2)])
-def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, nt):
+@pytest.mark.parametrize("tile,nt,skew", [(0, 3, 1), (8, 0, 2), (64, 1, 0), (16, 2, 2), (0, 3, 0)])
+def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, nt, skew):
     """(X, Y, f) with a short inner dim taken as (Y, X, f): images turned, sequences
     of short feature vectors between batch-major and time-major.  Tiles of records
     through the LDS (ELEMWISE_RECORDS; side of a tile ELEMWISE_RECORDS_TILE): whole
     and cut tiles, a second operand laid out like the result, a broadcast operand,
-    planes, and an operand whose records start inside a larger buffer.  Floats and
+    planes, and an operand whose records start inside a larger buffer; rectangular
+    tiles and windows moved onto the result's 64-byte blocks (ELEMWISE_RECORDS_SKEW:
+    0 never, 1 where the result's rows start off them, 2 always), also with the
+    result inside a larger buffer.  Floats and
     32-bit integers against NumPy, exact."""
-    knobs(ELEMWISE_RECORDS_TILE=tile, ELEMWISE_RECORDS_NT=nt, ELEMWISE_RECORDS_MIN=1)
+    knobs(ELEMWISE_RECORDS_TILE=tile, ELEMWISE_RECORDS_NT=nt, ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew)
     rng = np.random.default_rng(950 + tile)
     for dtype in ("float32", "int32"):
         k = ga.GpuElemwise(ctx, "o = a + b * r", [arg("a", dtype, read=True), arg("b", dtype, read=True),
@@ -825,6 +828,16 @@ def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, n
                 out2 = gpuarray.empty((3, ny, nx, f), dtype, context=ctx)
                 kc(gv.transpose(0, 2, 1, 3), out2)
                 assert np.array_equal(np.asarray(out2), aroot[:, :, 1:ny + 1, :].transpose(0, 2, 1, 3)), (dtype, f, ny, nx, "planes")
+            # the result inside a larger buffer: rows that start 1 + 2 f elements into pitches of (nx + 3) f
+            ny, nx = 70, 130
+            a = draw((nx, ny, f))
+            oroot = np.zeros((ny, nx + 3, f), dtype)
+            oroot.reshape(-1)[0] = 0
+            go, groot = to_gpu_view(oroot[:, 2:nx + 2, :], ctx)
+            kc(gpuarray.array(a, context=ctx).transpose(1, 0, 2), go)
+            want = oroot.copy()
+            want[:, 2:nx + 2, :] = a.transpose(1, 0, 2)
+            assert np.array_equal(read_root(groot, oroot), want), (dtype, f, "result inside a larger buffer")
 
 
 @pytest.mark.parametrize("loose", [1, 0])
