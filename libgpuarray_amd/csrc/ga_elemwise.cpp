@@ -909,8 +909,9 @@ std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, uns
 
 // ---- tiles of short records -------------------------------------------------------
 // Same parameters as the strided kernel with three or four dims: (planes,) Y, X
-// and a short inner dim of F four-byte elements with unit stride in every array
-// that has it - a record.  The result and the arrays laid out like it have their
+// and a short inner dim of F elements with unit stride in every array that has
+// it - a record.  Every array has elements of es bytes (four in what follows;
+// with others a lane's step is 16 / es elements and a block 64 / es).  The result and the arrays laid out like it have their
 // records one after the other along X (stride of X = F elements); the arrays in
 // tmask, read only, along Y (stride of Y = F elements): matrices of records taken
 // as their transposes, (H, W, C) images turned, batch-major sequences of short
@@ -927,16 +928,19 @@ std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, uns
 // records such a window can reach, and the grid has tiles for 15 more elements
 // (T F must then be a multiple of 16: the windows of neighbouring tiles meet).
 std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned F, unsigned T, unsigned tmask,
-                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes, int skew = -1) {
+                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes, int skew = -1, unsigned es = 4) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const unsigned R = T * F;          // elements of a run
-  const unsigned pitch = R + 4;      // of a run in the LDS
-  const unsigned extra = skew >= 0 ? (15 + F - 1) / F + 1 : 0;   // records that a moved window can reach beyond the tile's
+  const unsigned V = 16 / es;        // elements per lane and step: a 16-byte chunk
+  const unsigned B = 64 / es;        // elements of a 64-byte block
+  const unsigned lg = es == 1 ? 0 : es == 2 ? 1 : es == 4 ? 2 : 3;
+  const unsigned pitch = R + V;      // of a run in the LDS
+  const unsigned extra = skew >= 0 ? (B - 1 + F - 1) / F + 1 : 0;   // records that a moved window can reach beyond the tile's
   const unsigned TS = T + extra;     // runs staged per transposed array
   const unsigned dy = nd - 3, dx = nd - 2, dc = nd - 1;
   emit_header(ge, s);
-  s += "typedef ga_uint __attribute__((ext_vector_type(4), aligned(4))) ga_chunk16u;\n";
+  appendf(s, "typedef ga_uint __attribute__((ext_vector_type(4), aligned(%u))) ga_chunk16u;\n", es < 4 ? es : 4);
   s += "KERNEL void __launch_bounds__(256) elem(const ga_size dim0";
   ktypes.push_back(GA_SIZE);
   for (unsigned d = 1; d < nd; d++) {
@@ -975,7 +979,7 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
   // the tile: elements k0 .. k0 + R - 1 of the result's rows y0 .. y0 + T - 1; the transposed
   // arrays' records from xs on are staged
   appendf(s, "const ga_uint ga_k0 = ga_bx * %uu, ga_y0 = ga_by * %uu, ga_xf = (ga_uint)dim%u * %uu;\n", R, T, dx, F);
-  if (skew >= 0) appendf(s, "const ga_uint ga_xs = ga_k0 >= 15u ? (ga_k0 - 15u) / %uu : 0u;\n", F);
+  if (skew >= 0) appendf(s, "const ga_uint ga_xs = ga_k0 >= %uu ? (ga_k0 - %uu) / %uu : 0u;\n", B - 1, B - 1, F);
   else appendf(s, "const ga_uint ga_xs = ga_bx * %uu;\n", T);
   appendf(s, "const ga_uint ga_ny = (ga_uint)dim%u - ga_y0 < %uu ? (ga_uint)dim%u - ga_y0 : %uu;\n", dy, T, dy, T);
   for (size_t j = 0; j < ge->args.size(); j++) {
@@ -988,7 +992,7 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
       appendf(s, "LOCAL_MEM %s %s_s[%u] __attribute__((aligned(16)));\n", ctype(a.typecode), a.name.c_str(), TS * pitch);
   }
   // the transposed arrays' runs into the LDS: run r (record xs + r along X), elements k .. k + 3 of it
-  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", TS * R);
+  appendf(s, "for (ga_uint ga_i = LID_0 * %uu; ga_i < %uu; ga_i += %uu) {\n", V, TS * R, 256 * V);
   appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
   appendf(s, "if (ga_xs + ga_r < (ga_uint)dim%u) {\n", dx);
   for (size_t j = 0; j < ge->args.size(); j++) {
@@ -997,44 +1001,44 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
     const bool nt = (ntmask >> aidx[j]) & 1u;
     appendf(s, "{ GLOBAL_MEM const %s *ga_p = (GLOBAL_MEM const %s *)(%s_b + (%s)(ga_xs + ga_r) * (%s)%s_str_%u) + ga_k;\n",
             ctype(a.typecode), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dx);
-    appendf(s, "union { ga_chunk16u c; %s e[4]; } ga_v;\n", ctype(a.typecode));
-    appendf(s, "if (ga_k + 3u < ga_ny * %uu) ga_v.c = %s((GLOBAL_MEM const ga_chunk16u *)ga_p);\n", F,
+    appendf(s, "union { ga_chunk16u c; %s e[%u]; } ga_v;\n", ctype(a.typecode), V);
+    appendf(s, "if (ga_k + %uu < ga_ny * %uu) ga_v.c = %s((GLOBAL_MEM const ga_chunk16u *)ga_p);\n", V - 1, F,
             nt ? "__builtin_nontemporal_load" : "*");
-    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if (ga_k + ga_e < ga_ny * %uu) ga_v.e[ga_e] = ga_p[ga_e];\n", F);
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < %uu; ga_e++) if (ga_k + ga_e < ga_ny * %uu) ga_v.e[ga_e] = ga_p[ga_e];\n", V, F);
     appendf(s, "*(ga_chunk16u *)&%s_s[ga_r * %uu + ga_k] = ga_v.c; }\n", a.name.c_str(), pitch);
   }
   s += "}\n}\nlocal_barrier();\n";
   // the result's rows: row r (position y0 + r of Y), elements kk .. kk + 3 (record kk / F, element kk % F);
   // with moved windows a row's first element is the one on a 64-byte block of the array in skew at
   // or below element k0, and elements before the row wrap to huge indices that fail the extent test
-  appendf(s, "for (ga_uint ga_i = LID_0 * 4u; ga_i < %uu; ga_i += 1024u) {\n", T * R);
+  appendf(s, "for (ga_uint ga_i = LID_0 * %uu; ga_i < %uu; ga_i += %uu) {\n", V, T * R, 256 * V);
   appendf(s, "const ga_uint ga_r = ga_i / %uu, ga_k = ga_i - ga_r * %uu;\n", R, R);
   s += "if (ga_r >= ga_ny) continue;\n";
   if (skew_j >= 0) {
     const ge_arg &a = ge->args[skew_j];
-    appendf(s, "const ga_uint ga_sh = (ga_uint)(((ga_size)(%s_b + (%s)ga_r * (%s)%s_str_%u) >> 2) + ga_k0) & 15u;\n",
-            a.name.c_str(), I, I, a.name.c_str(), dy);
+    appendf(s, "const ga_uint ga_sh = (ga_uint)(((ga_size)(%s_b + (%s)ga_r * (%s)%s_str_%u) >> %u) + ga_k0) & %uu;\n",
+            a.name.c_str(), I, I, a.name.c_str(), dy, lg, B - 1);
     s += "const ga_uint ga_kk = ga_k0 - ga_sh + ga_k;\n";
   } else {
     s += "const ga_uint ga_kk = ga_k0 + ga_k;\n";
   }
-  s += "if (ga_kk >= ga_xf && ga_kk + 3u >= ga_xf) continue;\n";
-  s += "const bool ga_full = ga_kk < ga_xf && ga_kk + 3u < ga_xf;\n";
+  appendf(s, "if (ga_kk >= ga_xf && ga_kk + %uu >= ga_xf) continue;\n", V - 1);
+  appendf(s, "const bool ga_full = ga_kk < ga_xf && ga_kk + %uu < ga_xf;\n", V - 1);
   for (size_t j = 0; j < ge->args.size(); j++) {
     const ge_arg &a = ge->args[j];
     if (!in(pmask, j)) continue;
     const bool nt = (ntmask >> aidx[j]) & 1u;
     appendf(s, "GLOBAL_MEM %s *%s_p = (GLOBAL_MEM %s *)(%s_b + (%s)ga_r * (%s)%s_str_%u);\n", ctype(a.typecode),
             a.name.c_str(), ctype(a.typecode), a.name.c_str(), I, I, a.name.c_str(), dy);
-    appendf(s, "union { ga_chunk16u c; %s e[4]; } %s_v;\n", ctype(a.typecode), a.name.c_str());
+    appendf(s, "union { ga_chunk16u c; %s e[%u]; } %s_v;\n", ctype(a.typecode), V, a.name.c_str());
     if (a.reads()) {
       appendf(s, "if (ga_full) %s_v.c = %s((GLOBAL_MEM const ga_chunk16u *)(%s_p + ga_kk));\n", a.name.c_str(),
               nt ? "__builtin_nontemporal_load" : "*", a.name.c_str());
-      appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_v.e[ga_e] = %s_p[(ga_uint)(ga_kk + ga_e)];\n",
-              a.name.c_str(), a.name.c_str());
+      appendf(s, "else for (ga_uint ga_e = 0; ga_e < %uu; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_v.e[ga_e] = %s_p[(ga_uint)(ga_kk + ga_e)];\n",
+              V, a.name.c_str(), a.name.c_str());
     }
   }
-  for (unsigned e = 0; e < 4; e++) {
+  for (unsigned e = 0; e < V; e++) {
     appendf(s, "if ((ga_uint)(ga_kk + %uu) < ga_xf) {\n", e);
     appendf(s, "const ga_uint ga_x = (ga_uint)(ga_kk + %uu) / %uu, ga_c = (ga_uint)(ga_kk + %uu) - ga_x * %uu;\n", e, F, e, F);
     auto place = [&](size_t j) {
@@ -1060,8 +1064,8 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
     const bool nt = (ntmask >> aidx[j]) & 1u;
     if (nt) appendf(s, "if (ga_full) __builtin_nontemporal_store(%s_v.c, (GLOBAL_MEM ga_chunk16u *)(%s_p + ga_kk));\n", a.name.c_str(), a.name.c_str());
     else appendf(s, "if (ga_full) *(GLOBAL_MEM ga_chunk16u *)(%s_p + ga_kk) = %s_v.c;\n", a.name.c_str(), a.name.c_str());
-    appendf(s, "else for (ga_uint ga_e = 0; ga_e < 4u; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_p[(ga_uint)(ga_kk + ga_e)] = %s_v.e[ga_e];\n",
-            a.name.c_str(), a.name.c_str());
+    appendf(s, "else for (ga_uint ga_e = 0; ga_e < %uu; ga_e++) if ((ga_uint)(ga_kk + ga_e) < ga_xf) %s_p[(ga_uint)(ga_kk + ga_e)] = %s_v.e[ga_e];\n",
+            V, a.name.c_str(), a.name.c_str());
   }
   s += "}\n}\n";
   return s;
@@ -2316,14 +2320,15 @@ class strided_call {
   }
 
   // Matrices of short records taken as their transposes (gen_record_tiles): three
-  // dims (four with planes), the inner one of 2 to 64 four-byte elements with unit
-  // stride; the result's records follow one another along X, a read-only
+  // dims (four with planes), the inner one of 2 to 64 elements (up to 256 bytes;
+  // all arrays of one element size) with unit stride; the result's records follow one another along X, a read-only
   // operand's along Y.  Neither counts as a transposed operand for the tiles (both
   // have their smallest stride on the inner dim), and a lane of the strided
   // kernels walks the short inner dim.
   // (side of a tile in records; records of 8 floats 69 / 76 % of peak with 32 / 16, of 32 69 / 75 % with 16 / 8,
   // of 2 67 / 74 / 59 % with 64 / 32 / 16)
-  static unsigned record_tile_side(size_t F) { return F <= 7 ? 32 : F <= 31 ? 16 : 8; }
+  // (by the record's bytes; records of up to 6 bytes get runs of 128 bytes and more from a side of 64)
+  static unsigned record_tile_side(size_t fb) { return fb <= 6 ? 64 : fb <= 28 ? 32 : fb <= 124 ? 16 : 8; }
   bool tiles_of_short_records(int &err) {
     const unsigned long fmax = TUNE(tn, ELEMWISE_RECORDS, 64);
     if (fmax == 0 || (nd != 3 && nd != 4) || na > 31) return false;
@@ -2332,61 +2337,67 @@ class strided_call {
         n < TUNE(tn, ELEMWISE_RECORDS_MIN, 65536))
       return false;
     unsigned tm = 0, pm = 0;
+    const size_t es = elsz[0];
+    if ((es != 1 && es != 2 && es != 4 && es != 8) || F * es > 256) return false;
     {
       unsigned k = 0;
       for (size_t i = 0; i < ge->args.size(); i++) {
         if (!ge->args[i].is_array()) continue;
-        if (elsz[k] != 4 || offs[k] % 4 != 0) return false;
+        if (elsz[k] != es || offs[k] % es != 0) return false;
         for (unsigned j = 0; j < nd; j++)
-          if (strs[k][j] % 4 != 0) return false;
-        const bool unit = strs[k][nd - 1] == 4;
-        if (unit && strs[k][nd - 2] == (ssize_t)(4 * F)) pm |= 1u << k;
-        else if (unit && strs[k][nd - 3] == (ssize_t)(4 * F) && !ge->args[i].writes()) tm |= 1u << k;
+          if (strs[k][j] % (ssize_t)es != 0) return false;
+        const bool unit = strs[k][nd - 1] == (ssize_t)es;
+        if (unit && strs[k][nd - 2] == (ssize_t)(es * F)) pm |= 1u << k;
+        else if (unit && strs[k][nd - 3] == (ssize_t)(es * F) && !ge->args[i].writes()) tm |= 1u << k;
         else if (ge->args[i].writes()) return false;
         k++;
       }
     }
     if (tm == 0 || !((pm >> outk) & 1u)) return false;
-    unsigned T = record_tile_side(F);
+    unsigned T = record_tile_side(F * es);
     {
       const unsigned long ft = TUNE(tn, ELEMWISE_RECORDS_TILE, 0);
       if (ft == 8 || ft == 16 || ft == 32 || ft == 64) T = (unsigned)ft;
     }
+    const size_t V = 16 / es, B = 64 / es;
+    while (((size_t)T * F) % V != 0 && T < 64) T *= 2;   // a run of whole chunks
+    if (((size_t)T * F) % V != 0) return false;
     // Windows moved onto the result's 64-byte blocks where its rows, or the tiles' pieces of them,
     // do not start on such blocks by themselves: (4729, 4729, 3) floats transposed (1, 0, 2) 41 ->
     // 54 % of peak, (3663, 3663, 5) 47 -> 59 %, (2590, 2590, 10) 54 -> 61 % ((4736, 4736, 3), whole
     // lines, runs at 73 %); moved windows on rows of whole blocks cost 6 to 10 points.
-    if (X * F + 15 + (size_t)T * F >= 0x7fffffffull) return false;
-    bool skewed = offs[outk] % 64 != 0 || ((size_t)T * F * 4) % 64 != 0;
+    if (X * F + 64 + (size_t)64 * F >= 0x7fffffffull) return false;
+    bool skewed = offs[outk] % 64 != 0 || ((size_t)T * F * es) % 64 != 0;
     for (unsigned j = 0; j + 2 < nd; j++) skewed = skewed || strs[outk][j] % 64 != 0;
     {
       const unsigned long sk = TUNE(tn, ELEMWISE_RECORDS_SKEW, 1);
       // (records of 33 and 50 floats on such rows: 59 and 60 % rectangular, 59 and 58 % moved)
-      skewed = sk == 2 || (sk == 1 && skewed && F <= 31);
+      skewed = sk == 2 || (sk == 1 && skewed && F * es <= 124);
     }
     // (the windows of neighbouring tiles meet only if a tile's piece of a row is whole blocks)
-    if (skewed && ((size_t)T * F) % 16 != 0) T = 16;
-    const unsigned extra = skewed ? (unsigned)((15 + F - 1) / F + 1) : 0;
+    while (skewed && ((size_t)T * F) % B != 0 && T < 64) T *= 2;
+    if (skewed && ((size_t)T * F) % B != 0) skewed = false;
+    const unsigned extra = skewed ? (unsigned)((B - 1 + F - 1) / F + 1) : 0;
     size_t lds = 0;
     for (unsigned k = 0; k < na; k++)
-      if ((tm >> k) & 1u) lds += (size_t)(T + extra) * (T * F + 4) * 4;
+      if ((tm >> k) & 1u) lds += (size_t)(T + extra) * (T * F + V) * es;
     if (lds > 80 * 1024) return false;
     choose_offset_width();
     const unsigned long ntm = TUNE(tn, ELEMWISE_RECORDS_NT, 3);
     const unsigned nt = ((ntm & 1) ? pm : 0u) | ((ntm & 2) ? tm : 0u);
-    gx = (X * F + (skewed ? 15 : 0) + (size_t)T * F - 1) / ((size_t)T * F);
+    gx = (X * F + (skewed ? B - 1 : 0) + (size_t)T * F - 1) / ((size_t)T * F);
     const size_t gy = (Y + T - 1) / T;
     ltx = (unsigned)gy;
     groups = gx * gy * (nd == 4 ? dims[0] : 1);
     if (groups > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x:%d", nd, F, T, idx64 ? 1 : 0, tm, pm, nt, skewed ? outk : -1);
+    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x:%d:%zu", nd, F, T, idx64 ? 1 : 0, tm, pm, nt, skewed ? outk : -1, es);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes, skewed ? outk : -1);
+      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes, skewed ? outk : -1, (unsigned)es);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2980,9 +2991,17 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
   // offsets' width, bit 2 streaming accesses, bit 3 windows moved onto the last array's 64-byte blocks; tmask the
   // arrays whose records follow one another along Y, its bits 16.. those laid out like the result
   if (strided == 16) {
-    const unsigned F = nd & 0xffu, T = F <= 7 ? 32 : F <= 31 ? 16 : 8;
+    unsigned es = 4;   // the element size of every array: the first one's
+    for (const ge_arg &a : ge.args)
+      if (a.is_array()) {
+        es = (unsigned)gpuarray_get_elsize(a.typecode);
+        break;
+      }
+    const unsigned F = nd & 0xffu, fb = F * es;
+    unsigned T = fb <= 6 ? 64 : fb <= 28 ? 32 : fb <= 124 ? 16 : 8;
+    while ((T * F) % (((idx64 & 8) ? 64 : 16) / es) != 0 && T < 64) T *= 2;
     return strdup(gen_record_tiles(&ge, 3 + (nd >> 8), (idx64 & 1) != 0, F, T, tmask & 0xffffu, tmask >> 16,
-                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 8) ? (int)ge.narray - 1 : -1).c_str());
+                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 8) ? (int)ge.narray - 1 : -1, es).c_str());
   }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)

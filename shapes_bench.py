@@ -118,6 +118,8 @@ def elemwise_cases():
          [("a", f, (4096, 4096, 4), T(1, 0, 2))], (4096, 4096, 4), f),
         ("(4729, 4729, 3) -> transpose (1, 0, 2) (an image turned; rows that are no whole lines)", "o = a",
          [("a", f, (4729, 4729, 3), T(1, 0, 2))], (4729, 4729, 3), f),
+        ("(9459, 9459, 3) bytes -> transpose (1, 0, 2) (an RGB image turned)", "o = a",
+         [("a", "uint8", (9459, 9459, 3), T(1, 0, 2))], (9459, 9459, 3), "uint8"),
         ("NHWC -> NCHW, (256, 56, 56, 8)", "o = a", [("a", f, (256, 56, 56, 8), T(0, 3, 1, 2))], (256, 8, 56, 56), f),
     ]
 

@@ -840,6 +840,34 @@ def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, n
             assert np.array_equal(read_root(groot, oroot), want), (dtype, f, "result inside a larger buffer")
 
 
+@pytest.mark.parametrize("skew", [1, 2])
+@pytest.mark.parametrize("dtype", ["uint8", "int16", "float16", "float64"])
+def test_matrices_of_short_records_of_other_element_sizes(ctx, knobs, dtype, skew):
+    """The tiles of records with 16, 8 and 2 elements to a 16-byte chunk: byte images
+    turned, records of halves and doubles; with a second operand laid out like the
+    result and a broadcast one, planes, cut tiles; halves computed as floats."""
+    knobs(ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew)
+    rng = np.random.default_rng(977)
+    k = ga.GpuElemwise(ctx, "o = a + b * r", [arg("a", dtype, read=True), arg("b", dtype, read=True),
+                                               arg("r", dtype, read=True), arg("o", dtype, write=True)], convert_f16=True)
+    kc = ga.GpuElemwise(ctx, "o = a", [arg("a", dtype, read=True), arg("o", dtype, write=True)], convert_f16=True)
+    draw = lambda shape: rng.integers(0, 4, size=shape).astype(dtype)
+    for f in (2, 3, 4, 8, 21, 32):
+        for ny, nx in ((64, 64), (100, 257), (65, 1000)):
+            a = draw((nx, ny, f))
+            b = draw((ny, nx, f))
+            r = draw((1, nx, 1))
+            out = gpuarray.empty((ny, nx, f), dtype, context=ctx)
+            k(gpuarray.array(a, context=ctx).transpose(1, 0, 2), gpuarray.array(b, context=ctx),
+              gpuarray.array(r, context=ctx), out, broadcast=True)
+            assert np.array_equal(np.asarray(out), a.transpose(1, 0, 2) + b * r), (f, ny, nx)
+            aroot = draw((2, nx, ny + 2, f))
+            gv, _ = to_gpu_view(aroot[:, :, 1:ny + 1, :], ctx)
+            out2 = gpuarray.empty((2, ny, nx, f), dtype, context=ctx)
+            kc(gv.transpose(0, 2, 1, 3), out2)
+            assert np.array_equal(np.asarray(out2), aroot[:, :, 1:ny + 1, :].transpose(0, 2, 1, 3)), (f, ny, nx, "planes")
+
+
 @pytest.mark.parametrize("loose", [1, 0])
 @pytest.mark.parametrize("dtype", ["float32", "int32"])
 def test_transposed_operands_of_four_byte_elements_on_any_layout(ctx, knobs, dtype, loose):
