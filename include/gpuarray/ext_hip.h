@@ -102,7 +102,8 @@ typedef int (*ga_hip_module_cache_stats_fn)(gpucontext *ctx, size_t out[4]);
  * 15 the same arguments for a short extent of 17 to 64, whole through the LDS;
  * 16 tiles of short records: nd carries the record's elements (plus 256 for
  * four dims), idx64 the width of the offsets in bit 0 and the streaming hint
- * in bit 2 and windows moved onto the last array's 64-byte blocks in bit 3,
+ * in bit 2, windows moved onto the last array's 64-byte blocks in bit 3 and
+ * tiles numbered along Y first in bit 4,
  * tmask bits 0..15 the arrays whose records follow one another
  * along Y, bits 16.. those laid out like the result. */
 typedef char *(*ga_hip_elemwise_source_fn)(const char *preamble, const char *expr,

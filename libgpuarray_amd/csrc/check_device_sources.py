@@ -139,7 +139,8 @@ def main():
     check("elemwise tiles of records of 50, four dims, 64-bit offsets, moved windows",
           gen_e(b"", b"c = a*b + 0.5f", 3, args, 0, 16, 50 | 256, 0b1001, 0b001 | (0b100 << 16)))
     bargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_UBYTE, 2), ElemwiseArg(b"c", GA_UBYTE, 4))
-    check("elemwise tiles of records of 3 bytes, moved windows", gen_e(b"", b"c = a", 2, bargs, 0, 16, 3, 0b1100, 0b01 | (0b10 << 16)))
+    check("elemwise tiles of records of 3 bytes, moved windows, tiles numbered along Y first",
+          gen_e(b"", b"c = a", 2, bargs, 0, 16, 3, 0b11100, 0b01 | (0b10 << 16)))
     dargs2 = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_DOUBLE, 2), ElemwiseArg(b"c", GA_DOUBLE, 4))
     check("elemwise tiles of records of 2 doubles", gen_e(b"", b"c = a", 2, dargs2, 0, 16, 2, 0b0100, 0b01 | (0b10 << 16)))
     iargs = (ElemwiseArg * 2)(ElemwiseArg(b"a", GA_FLOAT, 2), ElemwiseArg(b"c", GA_FLOAT, 6))

@@ -928,7 +928,8 @@ std::string gen_narrow_staged(const GpuElemwise *ge, bool idx64, unsigned F, uns
 // records such a window can reach, and the grid has tiles for 15 more elements
 // (T F must then be a multiple of 16: the windows of neighbouring tiles meet).
 std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, unsigned F, unsigned T, unsigned tmask,
-                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes, int skew = -1, unsigned es = 4) {
+                             unsigned pmask, unsigned ntmask, std::vector<int> &ktypes, int skew = -1, unsigned es = 4,
+                             bool ymajor = false) {
   std::string s;
   const char *I = idx64 ? "ga_ssize" : "ga_int";
   const unsigned R = T * F;          // elements of a run
@@ -975,7 +976,14 @@ std::string gen_record_tiles(const GpuElemwise *ge, unsigned nd, bool idx64, uns
   s += ", const ga_uint ga_gx, const ga_uint ga_ltx) {\n";
   ktypes.push_back(GA_UINT);
   ktypes.push_back(GA_UINT);
-  s += "ga_uint ga_g = GID_0;\nconst ga_uint ga_bx = ga_g % ga_gx; ga_g /= ga_gx;\nconst ga_uint ga_by = ga_g % ga_ltx; ga_g /= ga_ltx;\n";
+  if (ymajor)
+    // tiles that follow one another along Y share the lines in which the transposed arrays' runs
+    // begin and end: they get consecutive numbers, and consecutive numbers one die (group g runs
+    // on die g % 8)
+    s += "ga_uint ga_g = GID_0;\n{ const ga_uint ga_whole = GDIM_0 & ~7u; if (ga_g < ga_whole) ga_g = (ga_g % 8u) * (ga_whole / 8u) + ga_g / 8u; }\n"
+         "const ga_uint ga_by = ga_g % ga_ltx; ga_g /= ga_ltx;\nconst ga_uint ga_bx = ga_g % ga_gx; ga_g /= ga_gx;\n";
+  else
+    s += "ga_uint ga_g = GID_0;\nconst ga_uint ga_bx = ga_g % ga_gx; ga_g /= ga_gx;\nconst ga_uint ga_by = ga_g % ga_ltx; ga_g /= ga_ltx;\n";
   // the tile: elements k0 .. k0 + R - 1 of the result's rows y0 .. y0 + T - 1; the transposed
   // arrays' records from xs on are staged
   appendf(s, "const ga_uint ga_k0 = ga_bx * %uu, ga_y0 = ga_by * %uu, ga_xf = (ga_uint)dim%u * %uu;\n", R, T, dx, F);
@@ -2383,21 +2391,33 @@ class strided_call {
       if ((tm >> k) & 1u) lds += (size_t)(T + extra) * (T * F + V) * es;
     if (lds > 80 * 1024) return false;
     choose_offset_width();
+    // Transposed arrays whose runs are no whole 128-byte lines: the lines in which a tile's runs
+    // begin and end belong to the next tile along Y too, and streamed they were fetched again
+    // ((4729, 4729, 3) floats read 1.58 times the array).  They stay cacheable: records of 3 floats
+    // on such rows 54 -> 66 % of peak, of 5 59 -> 66, of 10 61 -> 69, of 25 63 -> 65; bytes in
+    // records of 2 30 -> 40 %.  Numbering the tiles along Y first, consecutive numbers on one die,
+    // measured 3 to 6 points behind that on floats and 1 to 4 ahead on bytes: a knob, off.
+    bool lines = ((size_t)T * F * es) % 128 == 0;
+    for (unsigned k = 0; k < na && lines; k++)
+      if ((tm >> k) & 1u) lines = offs[k] % 128 == 0 && strs[k][nd - 2] % 128 == 0 && (nd == 3 || strs[k][0] % 128 == 0);
     const unsigned long ntm = TUNE(tn, ELEMWISE_RECORDS_NT, 3);
-    const unsigned nt = ((ntm & 1) ? pm : 0u) | ((ntm & 2) ? tm : 0u);
+    const unsigned nt = ((ntm & 1) ? pm : 0u) | (((ntm & 2) && (lines || (ntm & 4))) ? tm : 0u);
+    const unsigned long ym = TUNE(tn, ELEMWISE_RECORDS_YMAJOR, 0);
+    const bool ymajor = ym == 2 || (ym == 1 && !lines);
     gx = (X * F + (skewed ? B - 1 : 0) + (size_t)T * F - 1) / ((size_t)T * F);
     const size_t gy = (Y + T - 1) / T;
     ltx = (unsigned)gy;
     groups = gx * gy * (nd == 4 ? dims[0] : 1);
     if (groups > 0x7fffffffull) return false;
     char key[64];
-    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x:%d:%zu", nd, F, T, idx64 ? 1 : 0, tm, pm, nt, skewed ? outk : -1, es);
+    snprintf(key, sizeof(key), "r%u:%zu:%u:%d:%x:%x:%x:%d:%zu:%d", nd, F, T, idx64 ? 1 : 0, tm, pm, nt, skewed ? outk : -1, es,
+             ymajor ? 1 : 0);
     auto it = ge->k_strided.find(key);
     if (it != ge->k_strided.end()) {
       kernel = &it->second;
     } else {
       std::vector<int> ktypes;
-      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes, skewed ? outk : -1, (unsigned)es);
+      std::string src = gen_record_tiles(ge, nd, idx64, (unsigned)F, T, tm, pm, nt, ktypes, skewed ? outk : -1, (unsigned)es, ymajor);
       GpuKernel nk = {nullptr, nullptr};
       err = build_kernel(ge, &nk, src, ktypes);
       if (err != GA_NO_ERROR) return true;
@@ -2988,7 +3008,8 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
                                    (idx64 & 32) ? ~(tmask | (tmask >> 16)) & ((1u << ge.narray) - 1u) : 0u).c_str());
   }
   // 16: tiles of short records: nd carries the record's elements (plus 256: planes, four dims), idx64 bit 0 the
-  // offsets' width, bit 2 streaming accesses, bit 3 windows moved onto the last array's 64-byte blocks; tmask the
+  // offsets' width, bit 2 streaming accesses, bit 3 windows moved onto the last array's 64-byte blocks, bit 4 tiles
+  // numbered along Y first; tmask the
   // arrays whose records follow one another along Y, its bits 16.. those laid out like the result
   if (strided == 16) {
     unsigned es = 4;   // the element size of every array: the first one's
@@ -3001,7 +3022,8 @@ GPUARRAY_PUBLIC char *ga_elemwise_gen_source(const char *preamble, const char *e
     unsigned T = fb <= 6 ? 64 : fb <= 28 ? 32 : fb <= 124 ? 16 : 8;
     while ((T * F) % (((idx64 & 8) ? 64 : 16) / es) != 0 && T < 64) T *= 2;
     return strdup(gen_record_tiles(&ge, 3 + (nd >> 8), (idx64 & 1) != 0, F, T, tmask & 0xffffu, tmask >> 16,
-                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 8) ? (int)ge.narray - 1 : -1, es).c_str());
+                                   (idx64 & 4) ? tmask >> 16 : 0u, ktypes, (idx64 & 8) ? (int)ge.narray - 1 : -1, es,
+                                   (idx64 & 16) != 0).c_str());
   }
   // 15: the same arguments for a wider short extent, whole through the LDS
   if (strided == 15)

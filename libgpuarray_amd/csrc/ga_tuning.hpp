@@ -14,7 +14,7 @@
 #define GA_KNOBS(X) \
   X(ALLOW_OTHER_ISA) X(ELEMWISE_BAND) X(ELEMWISE_FLAT_NT_MASK) X(ELEMWISE_GROUPS_PER_CU) \
   X(ELEMWISE_MIXED_ALIGN) X(ELEMWISE_NARROW) X(ELEMWISE_NARROW_CHUNKS) X(ELEMWISE_NARROW_LDS) X(ELEMWISE_NARROW_MIN) X(ELEMWISE_NARROW_MIN_PLANE) X(ELEMWISE_NARROW_NT) X(ELEMWISE_NARROW_QUADS) X(ELEMWISE_NARROW_STAGED) X(ELEMWISE_NARROW_STAGED_WIDE) X(ELEMWISE_NT) X(ELEMWISE_NT_LINES) X(ELEMWISE_NT_MASK) X(ELEMWISE_PAIRS) \
-  X(ELEMWISE_PANEL) X(ELEMWISE_PERIODIC) X(ELEMWISE_PERIODIC_ROWLOAD) X(ELEMWISE_PERIODIC_VEC) X(ELEMWISE_LOOSE) X(ELEMWISE_LOOSE_MIN_BYTES) X(ELEMWISE_QUADS) X(ELEMWISE_RECORDS) X(ELEMWISE_RECORDS_MIN) X(ELEMWISE_RECORDS_NT) X(ELEMWISE_RECORDS_SKEW) X(ELEMWISE_RECORDS_TILE) X(ELEMWISE_SKEW) \
+  X(ELEMWISE_PANEL) X(ELEMWISE_PERIODIC) X(ELEMWISE_PERIODIC_ROWLOAD) X(ELEMWISE_PERIODIC_VEC) X(ELEMWISE_LOOSE) X(ELEMWISE_LOOSE_MIN_BYTES) X(ELEMWISE_QUADS) X(ELEMWISE_RECORDS) X(ELEMWISE_RECORDS_MIN) X(ELEMWISE_RECORDS_NT) X(ELEMWISE_RECORDS_SKEW) X(ELEMWISE_RECORDS_TILE) X(ELEMWISE_RECORDS_YMAJOR) X(ELEMWISE_SKEW) \
   X(ELEMWISE_TILE) X(ELEMWISE_TMIN) X(ELEMWISE_TTILE) X(ELEMWISE_TTILE_FILL) X(ELEMWISE_TTILE_MIN) X(ELEMWISE_UNROLL) X(ELEMWISE_VEC4) \
   X(ELEMWISE_ZMASK) X(FILL_KERNEL_MIN) X(MARK_EVENT_FLAGS) X(MOVE_KERNEL_MIN) X(REDUX_BALANCE) X(REDUX_COLVEC) \
   X(REDUX_COL_BALANCE) X(REDUX_COL_CVMAX) X(REDUX_COL_FAR) X(REDUX_COL_IDLE) X(REDUX_COL_LOOSE) X(REDUX_COL_LOOSE_MIN_BYTES) X(REDUX_COL_ROWS) X(REDUX_COL_U) X(REDUX_FAST8) \

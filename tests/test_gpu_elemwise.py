@@ -794,7 +794,7 @@ def test_very_narrow_planes_between_element_sizes(ctx, knobs):
             assert np.array_equal(np.asarray(out), (b.T + 1).astype(do)), (di, do, n, f, "narrow result")
 
 
-@pytest.mark.parametrize("tile,nt,skew", [(0, 3, 1), (8, 0, 2), (64, 1, 0), (16, 2, 2), (0, 3, 0)])
+@pytest.mark.parametrize("tile,nt,skew", [(0, 3, 1), (8, 0, 2), (64, 1, 0), (16, 6, 2), (0, 7, 0)])
 def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, nt, skew):
     """(X, Y, f) with a short inner dim taken as (Y, X, f): images turned, sequences
     of short feature vectors between batch-major and time-major.  Tiles of records
@@ -802,10 +802,12 @@ def test_matrices_of_short_records_taken_as_their_transposes(ctx, knobs, tile, n
     and cut tiles, a second operand laid out like the result, a broadcast operand,
     planes, and an operand whose records start inside a larger buffer; rectangular
     tiles and windows moved onto the result's 64-byte blocks (ELEMWISE_RECORDS_SKEW:
-    0 never, 1 where the result's rows start off them, 2 always), also with the
+    0 never, 1 where the result's rows start off them, 2 always; the same values
+    for ELEMWISE_RECORDS_YMAJOR, tiles numbered along Y first), also with the
     result inside a larger buffer.  Floats and
     32-bit integers against NumPy, exact."""
-    knobs(ELEMWISE_RECORDS_TILE=tile, ELEMWISE_RECORDS_NT=nt, ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew)
+    knobs(ELEMWISE_RECORDS_TILE=tile, ELEMWISE_RECORDS_NT=nt, ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew,
+          ELEMWISE_RECORDS_YMAJOR=skew)
     rng = np.random.default_rng(950 + tile)
     for dtype in ("float32", "int32"):
         k = ga.GpuElemwise(ctx, "o = a + b * r", [arg("a", dtype, read=True), arg("b", dtype, read=True),
@@ -846,7 +848,7 @@ def test_matrices_of_short_records_of_other_element_sizes(ctx, knobs, dtype, ske
     """The tiles of records with 16, 8 and 2 elements to a 16-byte chunk: byte images
     turned, records of halves and doubles; with a second operand laid out like the
     result and a broadcast one, planes, cut tiles; halves computed as floats."""
-    knobs(ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew)
+    knobs(ELEMWISE_RECORDS_MIN=1, ELEMWISE_RECORDS_SKEW=skew, ELEMWISE_RECORDS_YMAJOR=skew)
     rng = np.random.default_rng(977)
     k = ga.GpuElemwise(ctx, "o = a + b * r", [arg("a", dtype, read=True), arg("b", dtype, read=True),
                                                arg("r", dtype, read=True), arg("o", dtype, write=True)], convert_f16=True)
