@@ -75,6 +75,62 @@ def test_four_elements_per_lane_variants_compile(nd, idx64, tmask, umask):
     assert err == 0, log
 
 
+@pytest.mark.parametrize("f,planes,flags", [(3, 0, 0b00100), (11, 0, 0b01111), (5, 1, 0b11110), (8, 1, 0b101100)])
+def test_narrow_planes_in_registers_compile(f, planes, flags):
+    """Variant 14: (N, f) against its transpose with a lane holding a chunk of
+    positions by the whole short dim; arrays with the short dim innermost direct or
+    through the LDS, the others as chunks, an operand constant along the long dim."""
+    src = take_string(gen_elemwise(b"", b"c = a*b + 0.5f", 3, args_of(F32), 0, 14, f | (planes << 8), flags,
+                                   0b001 | (0b100 << 16)))
+    text = src.decode()
+    assert "union { ga_chunk16 c[%d]; ga_float e[%d]; } a_r;" % (f, 4 * f) in text     # a lane's 4 f elements of a
+    assert ("LOCAL_MEM ga_chunk16 a_s[%d];" % (256 * f) in text) == bool(flags & 8)      # staged or not
+    assert ("ga_float b_z[%d];" % f in text) == bool(flags & 32)                        # fetched once per row
+    assert text.count("c = a*b + 0.5f;") == 4 * f
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
+def test_narrow_planes_of_mixed_element_sizes_compile():
+    """Bytes with the short dim innermost and floats in planes: 16 positions per lane,
+    four chunks of floats per row."""
+    spec = [("a", _lib.GA_UBYTE, R), ("c", _lib.GA_FLOAT, W)]
+    src = take_string(gen_elemwise(b"", b"c = a", 2, args_of(spec), 0, 14, 3, 0b00100, 0b01 | (0b10 << 16)))
+    text = src.decode()
+    assert "union { ga_chunk16 c[3]; ga_ubyte e[48]; } a_r;" in text
+    assert "union { ga_chunk16 c[4]; ga_float e[16]; } c_r[3];" in text
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
+@pytest.mark.parametrize("f,planes,flags", [(17, 0, 0b00100), (33, 1, 0b10111), (64, 0, 0b00000)])
+def test_narrow_planes_through_the_lds_compile(f, planes, flags):
+    """Variant 15: short extents of 17 to 64, a group's piece whole through the LDS."""
+    src = take_string(gen_elemwise(b"", b"c = a*b + 0.5f", 3, args_of(F32), 0, 15, f | (planes << 8), flags,
+                                   0b001 | (0b110 << 16)))
+    assert ("LOCAL_MEM ga_float a_s[%d];" % (260 * (f | 1))).encode() in src
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
+@pytest.mark.parametrize("f,planes,flags,tc", [(3, 0, 0b00100, "GA_FLOAT"), (20, 1, 0b01001, "GA_FLOAT"),
+                                               (3, 0, 0b11100, "GA_UBYTE"), (2, 1, 0b00100, "GA_DOUBLE")])
+def test_tiles_of_records_compile(f, planes, flags, tc):
+    """Variant 16: matrices of short records against their transposes; rectangular
+    tiles and windows moved onto the result's 64-byte blocks, tiles numbered along Y
+    first, element sizes of 1, 4 and 8 bytes."""
+    t = getattr(_lib, tc)
+    spec = [("a", t, R), ("b", t, R), ("c", t, W)]
+    src = take_string(gen_elemwise(b"", b"c = a + b", 3, args_of(spec), 0, 16, f | (planes << 8), flags,
+                                   0b001 | (0b110 << 16)))
+    text = src.decode()
+    assert "LOCAL_MEM" in text and "a_s[" in text and "b_s[" not in text      # only the transposed operand is staged
+    assert ("ga_sh" in text) == bool(flags & 8)
+    assert ("GDIM_0 & ~7u" in text) == bool(flags & 16)
+    err, log = compile_src(src)
+    assert err == 0, log
+
+
 def test_mixed_types_scalars_and_half_compile():
     spec = [("x", _lib.GA_HALF, R), ("k", _lib.GA_DOUBLE, S), ("m", _lib.GA_UBYTE, R),
             ("y", _lib.GA_HALF, R | W), ("z", _lib.GA_LONG, W)]
